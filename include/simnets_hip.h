@@ -1,0 +1,192 @@
+/*
+ * simnets_hip.h - C ABI of the MI355X (gfx950) implementation of the SimNets forward operators.
+ *
+ * This is the boundary an operator layer binds instead of the kernels of HUJI-Deep/simnets-tf:
+ * where that project's TensorFlow OpKernel::Compute methods call im2col_3d + ggemm, an op
+ * layer calls simnets_hip_similarity_fwd / simnets_hip_mex_fwd with device pointers and the
+ * operator attributes.  Citations below name the reference interface each entry point
+ * replaces (paths relative to the reference checkout).
+ *
+ * Conventions
+ *   - All tensors are dense, row-major, fp32, NCHW, resident in device memory; the caller
+ *     owns every buffer.  The library never allocates, frees or keeps device memory: scratch
+ *     comes from the caller's workspace (size from the *_workspace_bytes query).
+ *   - Work is enqueued on the given stream (a hipStream_t passed as void*; NULL = the null
+ *     stream) and the call returns without synchronising.  Calls are re-entrant.
+ *   - Return value: SIMNETS_OK (0) or a negative simnets_status.  Attribute and shape
+ *     validation happens on the host before anything is launched, so the error paths do not
+ *     need a GPU.  simnets_hip_strerror() gives the message; where the reference raises
+ *     InvalidArgument the message is the reference's own text.
+ *   - There is no CPU fallback: on a machine without a usable HIP device the compute entry
+ *     points return SIMNETS_ERR_HIP.
+ */
+#ifndef SIMNETS_HIP_H
+#define SIMNETS_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SIMNETS_HIP_ABI_VERSION 1
+
+typedef enum simnets_status {
+    SIMNETS_OK = 0,
+    SIMNETS_ERR_NULL_POINTER = -1,
+    SIMNETS_ERR_PADDING_LENGTH = -2,        /* similarity_kernel_common.hpp:86 / mex ExpandDimSpec */
+    SIMNETS_ERR_BLOCKS_LENGTH = -3,         /* similarity_kernel_common.hpp:89, mex_kernel_common.cpp:43 */
+    SIMNETS_ERR_STRIDES_LENGTH = -4,        /* similarity_kernel_common.hpp:92, mex_kernel_common.cpp:39 */
+    SIMNETS_ERR_SIMILARITY_FUNCTION = -5,   /* similarity_kernel_common.hpp:95-101 */
+    SIMNETS_ERR_NORMALIZATION_NEEDS_L2 = -6,/* similarity_kernel_common.hpp:106 */
+    SIMNETS_ERR_IGNORE_NAN_NEEDS_NORM = -7, /* similarity_kernel_common.hpp:108 */
+    SIMNETS_ERR_TEMPLATE_CHANNELS = -8,     /* similarity_kernel_common.hpp:160 */
+    SIMNETS_ERR_WEIGHTS_CHANNELS = -9,      /* similarity_kernel_common.hpp:162 */
+    SIMNETS_ERR_STRIDE_NOT_POSITIVE = -10,  /* im2col.hpp:116-118 */
+    SIMNETS_ERR_NUM_INSTANCES = -11,        /* mex_kernel_common.cpp:34 */
+    SIMNETS_ERR_UNSHARED_REGION_LENGTH = -12, /* mex_kernel_common.cpp:54 */
+    SIMNETS_ERR_SHARED_REGION_LENGTH = -13, /* mex_kernel_common.cpp:56 */
+    SIMNETS_ERR_BLOCK_DEPTH = -14,          /* mex_kernel_common.cpp:169 */
+    SIMNETS_ERR_SHAPE = -15,                /* a tensor shape disagrees with the attributes */
+    SIMNETS_ERR_EMPTY_OUTPUT = -16,         /* an output dimension would be <= 0 */
+    SIMNETS_ERR_WORKSPACE = -17,            /* workspace missing, too small or misaligned */
+    SIMNETS_ERR_ALGO = -18,                 /* requested algorithm cannot serve these attributes */
+    SIMNETS_ERR_TOO_LARGE = -19,            /* a dimension product exceeds 32-bit indexing */
+    SIMNETS_ERR_HIP = -20                   /* a HIP call or kernel launch failed */
+} simnets_status;
+
+const char *simnets_hip_strerror(int status);
+int simnets_hip_abi_version(void);
+
+/* ------------------------------------------------------------------------------------------
+ * Similarity:  REGISTER_OP("Similarity")  src/ops/similarity_op.cpp:61-75
+ * ------------------------------------------------------------------------------------------ */
+enum { SIMNETS_SIM_L1 = 0, SIMNETS_SIM_L2 = 1 };
+
+/* How the weighted distance is evaluated.  All choices implement the same operator. */
+enum {
+    SIMNETS_ALGO_AUTO = 0,   /* == DIRECT */
+    SIMNETS_ALGO_DIRECT = 1, /* d = t - x; acc += (-w*d)*d   (L1: acc += -w*|d|), NaN-capable, every mode */
+    SIMNETS_ALGO_SQRTW = 2,  /* plain L2 only: d = sqrt(w)*t - sqrt(w)*x in one fma; acc += -d*d */
+    SIMNETS_ALGO_MFMA = 3    /* plain L2 only, inputs free of NaN/Inf: sum w x^2 - 2 sum (w t) x + sum w t^2
+                                as dense fp32 matrix-core contractions */
+};
+
+typedef struct simnets_similarity_attrs {
+    int similarity_function;         /* attr similarity_function: {'L1','L2'} = 'L2'          */
+    int n_blocks;  int blocks[2];    /* attr blocks  = [3,3]   (README calls it ksize)        */
+    int n_strides; int strides[2];   /* attr strides = [2,2]                                  */
+    int n_padding; int padding[2];   /* attr padding = [0,0]                                  */
+    int normalization_term;          /* attr normalization_term = false                      */
+    float normalization_term_fudge;  /* attr normalization_term_fudge = 0.001                */
+    int ignore_nan_input;            /* attr ignore_nan_input = false                        */
+    float out_of_bounds_value;       /* attr out_of_bounds_value = 0.0 (may be NaN)          */
+    /* -- extensions; zero keeps the documented operator semantics -- */
+    int algo;                        /* SIMNETS_ALGO_*                                       */
+    /* Non-zero reproduces SimilarityKernelCPU::Compute literally for
+     * L2 + normalization_term + !ignore_nan_input: the constant -0.5*K*log(2 pi) is added to the
+     * whole output once per batch iteration (similarity_kernel_cpu.cpp:69,118-120), so image n
+     * carries it (B - n) times.  Zero adds it once per output, which is what SimilarityRef
+     * (similarity_ref_kernel_cpu.cpp:89-93) and the op documentation define. */
+    int norm_const_every_iteration;
+} simnets_similarity_attrs;
+
+/* Fills in the REGISTER_OP defaults (src/ops/similarity_op.cpp:67-74). */
+void simnets_similarity_attrs_default(simnets_similarity_attrs *attrs);
+
+/* Shape function: SimilarityShape (src/ops/similarity_op.cpp:8-53) and
+ * SimilarityKernelCommon::CalculateDimensions (include/kernels/similarity_kernel_common.hpp:113-164).
+ * input_shape = [B,C,H,W], templates_shape = weights_shape = [O,C,bh,bw]; output_shape <- [B,O,oh,ow].
+ * Performs every attribute / shape check of the operator. */
+int simnets_similarity_out_shape(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                 const int templates_shape[4], const int weights_shape[4], int output_shape[4]);
+
+/* Scratch the forward call needs (packed parameters), in bytes. */
+int simnets_hip_similarity_workspace_bytes(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                           const int templates_shape[4], size_t *bytes);
+
+/* Forward: replaces SimilarityKernelGPU<float>::Compute (src/kernels/similarity_kernel_gpu.cu:24-133),
+ * i.e. interlace_gpu + per-image im2col_3d_gpu + ggemm_gpu + the normalization constant.
+ * weights must be non-negative (the reference's Keras layer applies abs, python/simnets/keras.py:65). */
+int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                               const int templates_shape[4], const int weights_shape[4], const float *input,
+                               const float *templates, const float *weights, float *output, void *workspace,
+                               size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * MEX:  REGISTER_OP("Mex")  src/ops/mex_op.cpp:58-74
+ * ------------------------------------------------------------------------------------------ */
+typedef struct simnets_mex_attrs {
+    int num_instances;                   /* attr num_instances (required)                     */
+    int softmax_mode;                    /* attr softmax_mode = false                         */
+    int n_padding; int padding[3];       /* attr padding = [0,0,0]; 2 entries get -1 prepended; -1 -> image dim */
+    int n_strides; int strides[3];       /* attr strides = [1,1,1]; -1 -> image dim           */
+    int n_blocks;  int blocks[3];        /* attr blocks  = [1,1,1]                            */
+    float epsilon;                       /* attr epsilon = 1.0, may be +-inf                  */
+    float blocks_out_of_bounds_value;    /* attr blocks_out_of_bounds_value = 0.0             */
+    int blocks_round_down;               /* attr blocks_round_down = true                     */
+    int use_unshared_regions;            /* attr use_unshared_regions = true                  */
+    int n_shared;   int shared_offset_region[3];    /* attr shared_offset_region = [-1]   (1 or 3) */
+    int n_unshared; int unshared_offset_region[3];  /* attr unshared_offset_region = [-1] (1 or 3) */
+    /* -- extension -- */
+    /* Non-zero: offsets[r,m,:] -= logsumexp(offsets[r,m,:]) before use, what the reference's Keras
+     * layer does in Python for normalize_offsets=True (python/simnets/keras.py:155-160). */
+    int normalize_offsets;
+} simnets_mex_attrs;
+
+/* Fills in the REGISTER_OP defaults (src/ops/mex_op.cpp:62-73); num_instances is set to 1. */
+void simnets_mex_attrs_default(simnets_mex_attrs *attrs);
+
+/* Everything MexDimensionsData::CalculateDimensions derives (src/kernels/mex_kernel_common.cpp:63-158). */
+typedef struct simnets_mex_dims {
+    int pad_c, pad_h, pad_w, stride_c, stride_h, stride_w, block_c, block_h, block_w;
+    int channels_out, height_out, width_out, channels_out_total;
+    int shared_region_c, shared_region_h, shared_region_w;
+    int offsets_c, offsets_h, offsets_w;
+    int num_regions, region_size;
+    int M, K, N;
+    int is_1x1;
+} simnets_mex_dims;
+
+/* MexDimensionsData::CalculateDimensions + the checks of MEXKernelCommon's constructor
+ * (src/kernels/mex_kernel_common.cpp:29-58, :63-158, :169).  image_chw = [C,H,W]. */
+int simnets_mex_calc_dims(const simnets_mex_attrs *attrs, const int image_chw[3], simnets_mex_dims *dims);
+
+/* Shape function: MexShape (src/ops/mex_op.cpp:8-55).  input_shape = [B,C,H,W];
+ * output_shape <- [B, channels_out*num_instances, oh, ow]; offsets_shape <- [R,M,bc,bh,bw]
+ * (either output may be NULL). */
+int simnets_mex_out_shape(const simnets_mex_attrs *attrs, const int input_shape[4], int output_shape[4],
+                          int offsets_shape[5]);
+
+/* Binary-compatible twin of the reference's only C-ABI symbol (src/kernels/mex_dims_helper.cpp:8-44),
+ * so python/simnets/ops/mex.py:17-38 can bind this library unchanged.  Returns num_regions, or -1
+ * when n_blocks != 3. */
+int get_mex_offsets_nregions(int n_input_dim, const int *input_dim, int n_padding, const int *padding,
+                             int n_strides, const int *strides, int num_instances, int blocks_round_down,
+                             int use_unshared_regions, int n_blocks, const int *blocks,
+                             int n_shared_offset_region, const int *shared_offset_region,
+                             int n_unshared_offset_region, const int *unshared_offset_region);
+
+int simnets_hip_mex_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], size_t *bytes);
+
+/* Forward: replaces MEXKernelGPU<float>::Compute (src/kernels/mex_kernel_gpu.cu:60-159), i.e. the
+ * offsets copy + per-image im2col_3d_gpu + split_patches_gpu + ggemm_gpu (max pass) +
+ * ggemm_readc_gpu (exp/sum/log pass) + reverse split_patches_gpu.
+ * offsets_count = number of floats behind `offsets`; must be >= num_regions*num_instances*K. */
+int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                        const float *offsets, size_t offsets_count, float *output, void *workspace,
+                        size_t workspace_bytes, void *stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Glue of the missing-data network between MEX layers: non-overlapping sum pooling, which the
+ * reference example builds from AveragePooling2D * pool area (README.md:108-111,
+ * examples/mnist_ght_model_missing_data.py:60-66).  input [B,C,H,W] -> output [B,C,H/ph,W/pw]
+ * ('valid': a trailing partial window is dropped).
+ * ------------------------------------------------------------------------------------------ */
+int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, const float *input, float *output,
+                             void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SIMNETS_HIP_H */

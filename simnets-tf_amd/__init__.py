@@ -1,0 +1,20 @@
+"""MI355X-native SimNets forward operators (Similarity, MEX) behind the reference's op API.
+
+`similarity(...)` and `mex(...)` take the same arguments as python/simnets/ops/similarity.py:48
+and python/simnets/ops/mex.py:114 of HUJI-Deep/simnets-tf, operate on CUDA(=HIP) torch tensors
+and run hand-written gfx950 kernels through the C ABI of libsimnets_hip.so.  There is no CPU
+fallback: without the compiled library, or without a GPU, the calls raise.
+"""
+from . import _lib  # noqa: F401
+from .ops import (  # noqa: F401
+    SimnetsError,
+    similarity,
+    similarity_output_shape,
+    mex,
+    mex_output_shape,
+    sum_pooling,
+    _mex_dims_helper,
+    _expand_dim_specification,
+)
+
+__all__ = ["similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError"]

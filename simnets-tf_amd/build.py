@@ -1,0 +1,49 @@
+"""Compiles the HIP sources under csrc/ into libsimnets_hip.so next to this file (gfx950 only).
+
+Run as a script (`python simnets-tf_amd/build.py`) or call build().  hipcc cross-compiles, so no
+GPU is needed.  Packed FP32 VALU instructions are switched off for the device pass.
+"""
+import os
+import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "libsimnets_hip.so")
+OBJDIR = os.path.join(HERE, "build")
+
+SOURCES = ["host_logic.cpp", "capi.hip", "similarity_direct.hip", "similarity_mfma.hip", "mex.hip"]
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall",
+          "-Wno-unused-function"]
+DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-fno-fast-math",
+          "-fno-gpu-rdc"]
+
+
+def _compile(src, extra):
+    obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
+    path = os.path.join(CSRC, src)
+    if src.endswith(".hip"):
+        cmd = [HIPCC, "-c", path, "-o", obj] + COMMON + DEVICE + extra
+    else:
+        cmd = [HIPCC, "-x", "c++", "-c", path, "-o", obj] + COMMON + extra
+    subprocess.run(cmd, check=True)
+    return obj
+
+
+def build(extra=(), verbose=False):
+    os.makedirs(OBJDIR, exist_ok=True)
+    extra = list(extra)
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), 6)) as ex:
+        objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
+    subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs, check=True)
+    if verbose:
+        print("built", LIB)
+    return LIB
+
+
+if __name__ == "__main__":
+    build(sys.argv[1:], verbose=True)

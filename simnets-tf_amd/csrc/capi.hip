@@ -1,0 +1,96 @@
+// Compute entry points of the C ABI (include/simnets_hip.h): validate on the host, then enqueue.
+#include <hip/hip_runtime.h>
+
+#include "internal.h"
+
+namespace simnets {
+
+int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                      float *output, void *workspace, size_t workspace_bytes, hipStream_t s);
+size_t sim_mfma_workspace_bytes(const SimPlan &p);
+int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
+                    void *workspace, size_t workspace_bytes, hipStream_t s);
+
+size_t sim_workspace_bytes(const SimPlan &p)
+{
+    if (p.algo == SIMNETS_ALGO_MFMA)
+        return sim_mfma_workspace_bytes(p);
+    return sim_direct_workspace_bytes(p);
+}
+
+int sim_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
+               void *workspace, size_t workspace_bytes, void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (p.algo == SIMNETS_ALGO_MFMA)
+        return sim_mfma_launch(p, input, templates, weights, output, workspace, workspace_bytes, s);
+    return sim_direct_launch(p, input, templates, weights, output, workspace, workspace_bytes, s);
+}
+
+}  // namespace simnets
+
+using namespace simnets;
+
+static bool workspace_ok(const void *workspace, size_t have, size_t need)
+{
+    return need == 0 || (workspace && have >= need && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0);
+}
+
+extern "C" {
+
+int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                               const int templates_shape[4], const int weights_shape[4], const float *input,
+                               const float *templates, const float *weights, float *output, void *workspace,
+                               size_t workspace_bytes, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, weights_shape, &p);
+    if (rc)
+        return rc;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !templates || !weights || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, sim_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_launch(p, input, templates, weights, output, workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                        const float *offsets, size_t offsets_count, float *output, void *workspace,
+                        size_t workspace_bytes, void *stream)
+{
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    if (offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
+        return SIMNETS_ERR_SHAPE;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !offsets || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, mex_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return mex_launch(p, input, offsets, output, workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, const float *input, float *output,
+                             void *stream)
+{
+    if (!input_shape)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (pool_h <= 0 || pool_w <= 0 || input_shape[0] < 0 || input_shape[1] <= 0 || input_shape[2] <= 0 ||
+        input_shape[3] <= 0)
+        return SIMNETS_ERR_SHAPE;
+    if (input_shape[2] / pool_h <= 0 || input_shape[3] / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    if (input_shape[0] == 0)
+        return SIMNETS_OK;
+    if (!input || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    return sum_pool_launch(input_shape[0], input_shape[1], input_shape[2], input_shape[3], pool_h, pool_w, input,
+                           output, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,53 @@
+// Internal declarations shared by the host logic and the kernel launchers of libsimnets_hip.
+#pragma once
+
+#include <cstddef>
+#include <cstdint>
+
+#include "simnets_hip.h"
+
+namespace simnets {
+
+// Which combine the Similarity ggemm applies (the dispatch of
+// src/kernels/similarity_kernel_cpu.cpp:84-116 in the reference).
+enum SimMode { SIM_MODE_L1 = 0, SIM_MODE_L2 = 1, SIM_MODE_L2_NORM = 2, SIM_MODE_L2_NORM_IGNORE_NAN = 3,
+               SIM_MODE_L2_SQRTW = 4 /* internal: plain L2 evaluated as -(sqrt(w) t - sqrt(w) x)^2 */ };
+
+struct SimPlan {
+    int B, C, H, W, O;
+    int bh, bw, sh, sw, ph, pw;
+    int oh, ow, K;
+    int mode;  // SimMode
+    int algo;  // resolved SIMNETS_ALGO_* (never AUTO)
+    float fudge, oob;
+    int norm_const_every_iteration;
+};
+
+// Validates like SimilarityKernelCommon (ctor + CalculateDimensions) and fills the plan.
+int sim_make_plan(const simnets_similarity_attrs *attrs, const int input_shape[4], const int templates_shape[4],
+                  const int weights_shape[4], SimPlan *plan);
+
+size_t sim_workspace_bytes(const SimPlan &p);
+size_t sim_direct_workspace_bytes(const SimPlan &p);
+int sim_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
+               void *workspace, size_t workspace_bytes, void *stream);
+
+struct MexPlan {
+    int B, C, H, W;
+    simnets_mex_dims d;
+    int softmax_mode;
+    float epsilon, oob;
+    int use_unshared;
+    int normalize_offsets;
+};
+
+int mex_make_plan(const simnets_mex_attrs *attrs, const int input_shape[4], MexPlan *plan);
+size_t mex_workspace_bytes(const MexPlan &p);
+int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
+               size_t workspace_bytes, void *stream);
+
+int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *input, float *output, void *stream);
+
+inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace simnets

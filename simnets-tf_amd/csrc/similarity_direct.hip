@@ -1,0 +1,445 @@
+// Similarity forward, direct evaluation on the vector ALU (gfx950).
+//
+// Replaces, for the whole batch in one launch, what the reference does per image with three
+// kernels: interlace_kernel (include/utils/ggemm.cuh:70-87), im2col_3d_gpu_kernel
+// (src/utils/im2col.cu:546-585) and ggemm_kernel (include/utils/ggemm.cuh:108-185) with the
+// combines of include/utils/similarity_utils.hpp:17-80.
+//
+// Shape of the computation
+//   out[b, m, h, w] = sum_k comb(t[m,k], w[m,k], patch[b,h,w][k]),  k = (c*bh + dh)*bw + dw
+// Work split
+//   * a lane owns PT consecutive output columns of one output row ("pixel group") and MT
+//     output channels: PT*MT accumulators in VGPRs, summed over k in the reference's order;
+//   * the MT (template, weight) pairs of a k are the same for all 64 lanes, so they are read
+//     with scalar loads from a packed, k-major copy of the parameters and reach the VALU as
+//     SGPR operands: no LDS or VGPR traffic for the parameters at all;
+//   * a workgroup (4 waves) stages the rows of the input image its pixel groups touch, a few
+//     channels at a time, into LDS with coalesced loads; out-of-image positions are written as
+//     the out_of_bounds_value bit pattern there, so the inner loop has no bounds checks and NaN
+//     padding behaves exactly like NaN data.
+//   The inner loop is VALU bound: per k and lane PT ds_read_b32 against 3*PT*MT VALU ops.
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "internal.h"
+
+namespace simnets {
+
+#define SIMNETS_CONST_AS __attribute__((address_space(4)))
+
+namespace {
+
+constexpr int kWaves = 4;                 // waves per workgroup
+constexpr int kThreads = 64 * kWaves;
+constexpr int kLdsBudgetFloats = 16384;   // 64 KiB of input tile per workgroup
+
+struct SimKernelArgs {
+    const float *in;
+    float *out;
+    const float *pa;   // [mtile][K][MT][2]  (template, scaled negative weight)
+    const float *pc;   // [mtile][K][MT]     per-(m,k) additive constant (normalized modes)
+    int B, C, H, W, O, oh, ow;
+    int bh, bw, sh, sw, ph, pw, K;
+    int G;             // pixel groups per output row = ceil(ow / PT)
+    int gpi;           // pixel groups per image = oh * G
+    int tiles;         // workgroup tiles per image
+    int nws;           // spatial waves per workgroup (1, 2 or 4); kWaves / nws waves split the templates
+    int nws_log2;
+    int n_mtiles;      // ceil(O / MT)
+    int TC;            // LDS tile row pitch (floats)
+    int TRmax;         // LDS rows reserved per channel
+    int CC;            // channels staged per chunk
+    float oob;
+    float norm_const;  // -0.5*K*log(2 pi) for SIM_MODE_L2_NORM, else 0
+    int norm_every_iteration;
+    int vec_store;     // output rows are 16-byte aligned: store float4
+};
+
+// One k step for all MT templates and PT pixels of a lane.
+template <int MODE, int PT, int MT>
+__device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[PT],
+                                         const float SIMNETS_CONST_AS *pa, const float SIMNETS_CONST_AS *pc)
+{
+    if (MODE == SIM_MODE_L2_NORM_IGNORE_NAN) {
+        float keep[PT], xz[PT];
+#pragma unroll
+        for (int p = 0; p < PT; ++p) {
+            const bool ok = x[p] == x[p];
+            keep[p] = ok ? 1.0f : 0.0f;
+            xz[p] = ok ? x[p] : 0.0f;
+        }
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float t = pa[2 * m], nwh = pa[2 * m + 1], c = pc[m];
+#pragma unroll
+            for (int p = 0; p < PT; ++p) {
+                const float d = t - xz[p];
+                const float term = __builtin_fmaf(nwh * d, d, c);
+                acc[m][p] = __builtin_fmaf(keep[p], term, acc[m][p]);
+            }
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float t = pa[2 * m], nw = pa[2 * m + 1];
+            float c = 0.0f;
+            if (MODE == SIM_MODE_L2_NORM)
+                c = pc[m];
+#pragma unroll
+            for (int p = 0; p < PT; ++p) {
+                const float d = t - x[p];
+                if (MODE == SIM_MODE_L2_SQRTW) {
+                    // pa holds (sqrt(w)*t, -sqrt(w)): d = sqrt(w)*(t - x) in one fma, acc -= d*d
+                    const float ds = __builtin_fmaf(nw, x[p], t);
+                    acc[m][p] = __builtin_fmaf(-ds, ds, acc[m][p]);
+                } else if (MODE == SIM_MODE_L1)
+                    acc[m][p] = __builtin_fmaf(nw, __builtin_fabsf(d), acc[m][p]);
+                else if (MODE == SIM_MODE_L2)
+                    acc[m][p] = __builtin_fmaf(nw * d, d, acc[m][p]);
+                else
+                    acc[m][p] += __builtin_fmaf(nw * d, d, c);
+            }
+        }
+    }
+}
+
+template <int MODE, int PT, int MT, int SWT>
+__global__ __launch_bounds__(kThreads, 2) void sim_direct_kernel(const SimKernelArgs a)
+{
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int sw = SWT > 0 ? SWT : a.sw;
+
+    const int b = blockIdx.x / a.tiles;
+    const int tile = blockIdx.x - b * a.tiles;
+    const int ws = wave & (a.nws - 1);            // which 64 pixel groups of the tile
+    const int wm = wave >> a.nws_log2;            // which MT templates
+    const int nwm = kWaves >> a.nws_log2;
+    const int mtile = blockIdx.y * nwm + wm;
+    const bool wave_active = mtile < a.n_mtiles;
+
+    // pixel groups of this workgroup and the input rows they need
+    const int g_first = tile * 64 * a.nws;
+    const int g_last = min(g_first + 64 * a.nws, a.gpi) - 1;
+    const int row_first = g_first / a.G;
+    const int nrows = g_last / a.G - row_first + 1;
+    const int TR = (nrows - 1) * a.sh + a.bh;
+    const int in_row0 = row_first * a.sh - a.ph;
+
+    int g = g_first + ws * 64 + lane;
+    const bool lane_valid = g <= g_last;
+    g = min(g, g_last);
+    const int h = g / a.G;
+    const int gw = g - h * a.G;
+    const int lds_base = (h - row_first) * a.sh * a.TC + gw * PT * sw;
+
+    float acc[MT][PT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            acc[m][p] = 0.0f;
+
+    const float SIMNETS_CONST_AS *pa =
+        (const float SIMNETS_CONST_AS *)(a.pa) + (size_t)(wave_active ? mtile : 0) * a.K * MT * 2;
+    const float SIMNETS_CONST_AS *pc =
+        (const float SIMNETS_CONST_AS *)(a.pc) + (size_t)(wave_active ? mtile : 0) * a.K * MT;
+    const float *img = a.in + (size_t)b * a.C * a.H * a.W;
+    const int chan_lds = TR * a.TC;
+
+    for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
+        const int ccn = min(a.CC, a.C - ch0);
+        __syncthreads();
+        // ---- stage ccn channels x TR rows x TC columns; out-of-image -> oob ----
+        for (int cc = 0; cc < ccn; ++cc) {
+            const float *chan = img + (size_t)(ch0 + cc) * a.H * a.W;
+            for (int r = wave; r < TR; r += kWaves) {
+                const int ih = in_row0 + r;
+                const bool row_ok = ih >= 0 && ih < a.H;
+                const float *rowp = chan + (size_t)(row_ok ? ih : 0) * a.W;
+                float *dst = lds + cc * chan_lds + r * a.TC;
+                for (int col = lane; col < a.TC; col += 64) {
+                    const int iw = col - a.pw;
+                    float v = a.oob;
+                    if (row_ok && iw >= 0 && iw < a.W)
+                        v = rowp[iw];
+                    dst[col] = v;
+                }
+            }
+        }
+        __syncthreads();
+        if (!wave_active)
+            continue;
+        // ---- accumulate over the k of these channels, in k order ----
+        for (int cc = 0; cc < ccn; ++cc) {
+            for (int dh = 0; dh < a.bh; ++dh) {
+                const float *xrow = lds + lds_base + cc * chan_lds + dh * a.TC;
+                for (int dw = 0; dw < a.bw; ++dw) {
+                    float x[PT];
+#pragma unroll
+                    for (int p = 0; p < PT; ++p)
+                        x[p] = xrow[dw + p * sw];
+                    sim_step<MODE, PT, MT>(acc, x, pa, pc);
+                    pa += 2 * MT;
+                    pc += MT;
+                }
+            }
+        }
+    }
+
+    if (!wave_active || !lane_valid)
+        return;
+    // ---- epilogue ----
+    int reps = 0;
+    if (MODE == SIM_MODE_L2_NORM)
+        reps = a.norm_every_iteration ? (a.B - b) : 1;
+    const int w0 = gw * PT;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int mm = mtile * MT + m;
+        if (mm >= a.O)
+            break;
+        float v[PT];
+#pragma unroll
+        for (int p = 0; p < PT; ++p) {
+            v[p] = acc[m][p];
+            for (int r = 0; r < reps; ++r)
+                v[p] += a.norm_const;
+        }
+        float *o = a.out + (((size_t)b * a.O + mm) * a.oh + h) * a.ow + w0;
+        if (a.vec_store && PT % 4 == 0) {
+#pragma unroll
+            for (int q = 0; q < PT / 4; ++q)
+                if (w0 + 4 * q < a.ow)
+                    *reinterpret_cast<float4 *>(o + 4 * q) = make_float4(v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]);
+        } else {
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                if (w0 + p < a.ow)
+                    o[p] = v[p];
+        }
+    }
+}
+
+// Fallback for geometries whose input rows do not fit the LDS budget: one output pixel per
+// lane, patch elements gathered straight from global memory with bounds checks.
+template <int MODE, int MT>
+__global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long pix0 = ((long long)blockIdx.x * kWaves + wave) * 64;
+    const long long npix = (long long)a.B * a.oh * a.ow;
+    if (pix0 >= npix)
+        return;
+    long long pix = pix0 + lane;
+    const bool lane_valid = pix < npix;
+    if (!lane_valid)
+        pix = npix - 1;
+    const int b = (int)(pix / (a.oh * a.ow));
+    const int rem = (int)(pix - (long long)b * a.oh * a.ow);
+    const int h = rem / a.ow, w = rem - h * a.ow;
+    const int mtile = blockIdx.y;
+    const float *img = a.in + (size_t)b * a.C * a.H * a.W;
+    const float SIMNETS_CONST_AS *pa = (const float SIMNETS_CONST_AS *)(a.pa) + (size_t)mtile * a.K * MT * 2;
+    const float SIMNETS_CONST_AS *pc = (const float SIMNETS_CONST_AS *)(a.pc) + (size_t)mtile * a.K * MT;
+    float acc[MT][1];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m][0] = 0.0f;
+    for (int c = 0; c < a.C; ++c)
+        for (int dh = 0; dh < a.bh; ++dh) {
+            const int ih = h * a.sh - a.ph + dh;
+            for (int dw = 0; dw < a.bw; ++dw) {
+                const int iw = w * a.sw - a.pw + dw;
+                float x[1] = {a.oob};
+                if (ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
+                    x[0] = img[((size_t)c * a.H + ih) * a.W + iw];
+                sim_step<MODE, 1, MT>(acc, x, pa, pc);
+                pa += 2 * MT;
+                pc += MT;
+            }
+        }
+    if (!lane_valid)
+        return;
+    int reps = 0;
+    if (MODE == SIM_MODE_L2_NORM)
+        reps = a.norm_every_iteration ? (a.B - b) : 1;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int mm = mtile * MT + m;
+        if (mm >= a.O)
+            break;
+        float v = acc[m][0];
+        for (int r = 0; r < reps; ++r)
+            v += a.norm_const;
+        a.out[(((size_t)b * a.O + mm) * a.oh + h) * a.ow + w] = v;
+    }
+}
+
+// Packs (template, weight) into the k-major, MT-interleaved layout the scalar loads walk, with
+// the sign and the 1/2 of the normalized modes folded into the weight, and precomputes the
+// per-(m,k) logarithm term.  Replaces interlace_kernel (include/utils/ggemm.cuh:70-87).
+__global__ void sim_pack_params_kernel(const float *__restrict__ templates, const float *__restrict__ weights, int O,
+                                       int K, int MT, int n_mtiles, int mode, float fudge, float *__restrict__ pa,
+                                       float *__restrict__ pc)
+{
+    const long long total = (long long)n_mtiles * K * MT;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int mi = (int)(i % MT);
+        const long long r = i / MT;
+        const int k = (int)(r % K);
+        const int mtile = (int)(r / K);
+        const int m = mtile * MT + mi;
+        float t = 0.0f, w = 0.0f, c = 0.0f;
+        if (m < O) {
+            t = templates[(size_t)m * K + k];
+            w = weights[(size_t)m * K + k];
+            if (mode == SIM_MODE_L2_NORM)
+                c = 0.5f * logf(w + fudge);
+            else if (mode == SIM_MODE_L2_NORM_IGNORE_NAN)
+                c = (float)(0.5 * ((double)logf(w + fudge) - 1.8378770664093453 /* log(2 pi) */));
+        }
+        if (mode == SIM_MODE_L2_SQRTW) {
+            const float sq = sqrtf(w);
+            pa[2 * i] = sq * t;
+            pa[2 * i + 1] = -sq;
+        } else {
+            const float scale = (mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? -0.5f : -1.0f;
+            pa[2 * i] = t;
+            pa[2 * i + 1] = scale * w;
+        }
+        pc[i] = c;
+    }
+}
+
+struct Tiling {
+    int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
+    bool lds_ok;
+};
+
+Tiling choose_tiling(const SimPlan &p)
+{
+    Tiling t;
+    // Wide rows and many templates: 8 pixels x 16 templates per lane.  Otherwise 4 x 8, which
+    // keeps narrow images and small template counts from idling lanes and waves.
+    const bool big = p.ow >= 32 && p.O >= 32;
+    t.PT = big ? 8 : 4;
+    t.MT = big ? 16 : 8;
+    t.G = (p.ow + t.PT - 1) / t.PT;
+    t.gpi = p.oh * t.G;
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
+    // spatial waves per workgroup: as many as the template tiles leave free, if the image has the groups
+    t.nws = 1;
+    if (n_mtiles <= 2 && t.gpi >= 128)
+        t.nws = 2;
+    if (n_mtiles <= 1 && t.gpi >= 256)
+        t.nws = 4;
+    t.tiles = (t.gpi + 64 * t.nws - 1) / (64 * t.nws);
+    t.TC = (t.G * t.PT - 1) * p.sw + p.bw;
+    t.TC |= 1;  // odd pitch spreads rows over LDS banks
+    const int max_rows = std::min(p.oh, (64 * t.nws + t.G - 1) / t.G + 1);
+    t.TRmax = (max_rows - 1) * p.sh + p.bh;
+    const long long per_chan = 1LL * t.TRmax * t.TC;
+    t.lds_ok = per_chan <= kLdsBudgetFloats;
+    t.CC = 1;
+    if (t.lds_ok) {
+        const int cc_max = (int)std::min<long long>(p.C, kLdsBudgetFloats / per_chan);
+        const int chunks = (p.C + cc_max - 1) / cc_max;
+        t.CC = (p.C + chunks - 1) / chunks;
+    }
+    return t;
+}
+
+template <int MODE, int PT, int MT>
+hipError_t launch_direct(const SimKernelArgs &a, dim3 grid, size_t lds_bytes, hipStream_t s)
+{
+    if (a.sw == 1)
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1>), grid, dim3(kThreads), lds_bytes, s, a);
+    else if (a.sw == 2)
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 2>), grid, dim3(kThreads), lds_bytes, s, a);
+    else
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 0>), grid, dim3(kThreads), lds_bytes, s, a);
+    return hipGetLastError();
+}
+
+template <int MODE>
+hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
+{
+    if (!t.lds_ok) {
+        const long long npix = (long long)a.B * a.oh * a.ow;
+        dim3 grid((unsigned)((npix + 255) / 256), (unsigned)a.n_mtiles);
+        if (t.MT == 16)
+            hipLaunchKernelGGL((sim_gather_kernel<MODE, 16>), grid, dim3(256), 0, s, a);
+        else
+            hipLaunchKernelGGL((sim_gather_kernel<MODE, 8>), grid, dim3(256), 0, s, a);
+        return hipGetLastError();
+    }
+    const int nwm = kWaves / a.nws;
+    dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
+    const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
+    if (t.PT == 8)
+        return launch_direct<MODE, 8, 16>(a, grid, lds_bytes, s);
+    return launch_direct<MODE, 4, 8>(a, grid, lds_bytes, s);
+}
+
+}  // namespace
+
+size_t sim_direct_workspace_bytes(const SimPlan &p)
+{
+    const Tiling t = choose_tiling(p);
+    const size_t n_mtiles = (p.O + t.MT - 1) / t.MT;
+    // one extra k of slack behind each array: the scalar loads may be issued one step ahead
+    const size_t pa = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
+    const size_t pc = align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
+    return pa + pc;
+}
+
+int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                      float *output, void *workspace, size_t workspace_bytes, hipStream_t s)
+{
+    const Tiling t = choose_tiling(p);
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
+    const size_t pa_bytes = align_up(((size_t)n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
+    if (workspace_bytes < sim_direct_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+    float *pa = reinterpret_cast<float *>(workspace);
+    float *pc = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + pa_bytes);
+
+    const long long total = (long long)n_mtiles * p.K * t.MT;
+    const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
+    const int mode = (p.algo == SIMNETS_ALGO_SQRTW) ? (int)SIM_MODE_L2_SQRTW : p.mode;
+    hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights, p.O, p.K, t.MT,
+                       n_mtiles, mode, p.fudge, pa, pc);
+    if (hipGetLastError() != hipSuccess)
+        return SIMNETS_ERR_HIP;
+
+    SimKernelArgs a;
+    a.in = input; a.out = output; a.pa = pa; a.pc = pc;
+    a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
+    a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.K = p.K;
+    a.G = t.G; a.gpi = t.gpi; a.tiles = t.tiles; a.nws = t.nws; a.n_mtiles = n_mtiles;
+    a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
+    a.vec_store = (p.ow % 4 == 0) && ((reinterpret_cast<uintptr_t>(output) & 15) == 0);
+    a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC;
+    a.oob = p.oob;
+    // Dtype(-0.5) * Dtype(K_) * std::log(2.0 * M_PI), rounded to float by Eigen's constant()
+    a.norm_const = (p.mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)p.K) * std::log(2.0 * M_PI)) : 0.0f;
+    a.norm_every_iteration = p.norm_const_every_iteration;
+
+    hipError_t e;
+    switch (mode) {
+    case SIM_MODE_L1: e = launch_mode<SIM_MODE_L1>(a, t, s); break;
+    case SIM_MODE_L2: e = launch_mode<SIM_MODE_L2>(a, t, s); break;
+    case SIM_MODE_L2_NORM: e = launch_mode<SIM_MODE_L2_NORM>(a, t, s); break;
+    case SIM_MODE_L2_NORM_IGNORE_NAN: e = launch_mode<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, s); break;
+    default: e = launch_mode<SIM_MODE_L2_SQRTW>(a, t, s); break;
+    }
+    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+}  // namespace simnets

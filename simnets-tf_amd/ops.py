@@ -1,0 +1,259 @@
+"""Operator layer: the reference's Python op API (python/simnets/ops/similarity.py,
+python/simnets/ops/mex.py) over the C ABI, with torch tensors as device memory.
+
+Argument names, defaults (None = the registered op default, src/ops/similarity_op.cpp:67-74 and
+src/ops/mex_op.cpp:62-73) and error conditions follow the reference; errors surface as
+SimnetsError carrying the status code and the reference's message.
+"""
+import ctypes as C
+
+import torch
+
+from . import _lib
+from ._lib import MexAttrs, MexDims, SimilarityAttrs
+
+
+class SimnetsError(ValueError):
+    def __init__(self, code):
+        self.code = int(code)
+        super().__init__("simnets_hip status %d: %s" % (self.code, _lib.strerror(self.code)))
+
+
+def _check(code):
+    if code != 0:
+        raise SimnetsError(code)
+
+
+def _fill(dst, values, cap):
+    values = [int(v) for v in values]
+    for i, v in enumerate(values[:cap]):
+        dst[i] = v
+    return len(values)
+
+
+_workspaces = {}
+
+
+def _workspace(device, nbytes):
+    """A per-device scratch tensor, grown on demand and reused across calls (stream-ordered)."""
+    key = (device.type, device.index)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def _require_cuda_f32(name, t):
+    if not isinstance(t, torch.Tensor):
+        raise TypeError("%s must be a torch.Tensor" % name)
+    if t.dtype != torch.float32:
+        raise TypeError("%s must be float32 (the HIP path computes in fp32), got %s" % (name, t.dtype))
+    if not t.is_cuda:
+        raise RuntimeError("%s must live on a HIP device: simnets_tf_amd has no CPU fallback" % name)
+    return t.contiguous()
+
+
+def similarity_attrs(templates_shape=None, similarity_function=None, blocks=None, strides=None, padding=None,
+                     normalization_term=None, normalization_term_fudge=None, ignore_nan_input=None,
+                     out_of_bounds_value=None, algo=None, norm_const_every_iteration=False):
+    a = SimilarityAttrs()
+    _lib.lib().simnets_similarity_attrs_default(C.byref(a))
+    if similarity_function is not None:
+        if isinstance(similarity_function, bytes):
+            similarity_function = similarity_function.decode()
+        a.similarity_function = {"L1": _lib.SIM_L1, "L2": _lib.SIM_L2}.get(similarity_function, -1)
+    if blocks is not None:
+        a.n_blocks = _fill(a.blocks, blocks, 2)
+    if strides is not None:
+        a.n_strides = _fill(a.strides, strides, 2)
+    if padding is not None:
+        a.n_padding = _fill(a.padding, padding, 2)
+    if normalization_term is not None:
+        a.normalization_term = int(bool(normalization_term))
+    if normalization_term_fudge is not None:
+        a.normalization_term_fudge = float(normalization_term_fudge)
+    if ignore_nan_input is not None:
+        a.ignore_nan_input = int(bool(ignore_nan_input))
+    if out_of_bounds_value is not None:
+        a.out_of_bounds_value = float(out_of_bounds_value)
+    a.algo = _lib.ALGOS[algo]
+    a.norm_const_every_iteration = int(bool(norm_const_every_iteration))
+    return a
+
+
+def similarity_output_shape(input_shape, templates_shape, weights_shape=None, **attrs):
+    """Shape function of the op (SimilarityShape); runs every attribute check, needs no GPU."""
+    a = similarity_attrs(**attrs)
+    I4 = C.c_int * 4
+    out = I4()
+    weights_shape = templates_shape if weights_shape is None else weights_shape
+    _check(_lib.lib().simnets_similarity_out_shape(C.byref(a), I4(*input_shape), I4(*templates_shape),
+                                                   I4(*weights_shape), out))
+    return tuple(out)
+
+
+def similarity(input, templates, weights, similarity_function=None, blocks=None, strides=None, padding=None,
+               normalization_term=None, normalization_term_fudge=None, ignore_nan_input=None,
+               out_of_bounds_value=None, name=None, algo=None, norm_const_every_iteration=False, out=None):
+    """Similarity forward; arguments as python/simnets/ops/similarity.py:48-121.
+
+    input [B,C,H,W], templates/weights [O,C,bh,bw] (weights non-negative) -> [B,O,oh,ow].
+    Extensions: `algo` in {None,'direct','sqrtw','mfma'}, `norm_const_every_iteration`, `out`.
+    """
+    x = _require_cuda_f32("input", input)
+    t = _require_cuda_f32("templates", templates)
+    w = _require_cuda_f32("weights", weights)
+    if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
+        raise SimnetsError(-15)
+    a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+                         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+                         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
+                         norm_const_every_iteration=norm_const_every_iteration)
+    l = _lib.lib()
+    I4 = C.c_int * 4
+    xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
+    oshape = I4()
+    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    if out is None:
+        out = torch.empty(tuple(oshape), dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_contiguous() and tuple(out.shape) == tuple(oshape) and out.dtype == torch.float32
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_similarity_fwd(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
+                                            out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return out
+
+
+def mex_attrs(num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
+              blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
+              shared_offset_region=None, unshared_offset_region=None, normalize_offsets=False):
+    a = MexAttrs()
+    _lib.lib().simnets_mex_attrs_default(C.byref(a))
+    a.num_instances = int(num_instances)
+    if softmax_mode is not None:
+        a.softmax_mode = int(bool(softmax_mode))
+    if padding is not None:
+        a.n_padding = _fill(a.padding, padding, 3)
+    if strides is not None:
+        a.n_strides = _fill(a.strides, strides, 3)
+    if blocks is not None:
+        a.n_blocks = _fill(a.blocks, blocks, 3)
+    if epsilon is not None:
+        a.epsilon = float(epsilon)
+    if blocks_out_of_bounds_value is not None:
+        a.blocks_out_of_bounds_value = float(blocks_out_of_bounds_value)
+    if blocks_round_down is not None:
+        a.blocks_round_down = int(bool(blocks_round_down))
+    if use_unshared_regions is not None:
+        a.use_unshared_regions = int(bool(use_unshared_regions))
+    if shared_offset_region is not None:
+        a.n_shared = _fill(a.shared_offset_region, shared_offset_region, 3)
+    if unshared_offset_region is not None:
+        a.n_unshared = _fill(a.unshared_offset_region, unshared_offset_region, 3)
+    a.normalize_offsets = int(bool(normalize_offsets))
+    return a
+
+
+def mex_dims(image_chw, num_instances, **attrs):
+    """MexDimensionsData::CalculateDimensions as a dict; needs no GPU."""
+    a = mex_attrs(num_instances, **attrs)
+    d = MexDims()
+    _check(_lib.lib().simnets_mex_calc_dims(C.byref(a), (C.c_int * 3)(*image_chw), C.byref(d)))
+    return d.asdict()
+
+
+def mex_output_shape(input_shape, num_instances, **attrs):
+    """(output_shape, offsets_shape) of the op (MexShape + the offsets variable of the Keras layer)."""
+    a = mex_attrs(num_instances, **attrs)
+    o, f = (C.c_int * 4)(), (C.c_int * 5)()
+    _check(_lib.lib().simnets_mex_out_shape(C.byref(a), (C.c_int * 4)(*input_shape), C.byref(o), C.byref(f)))
+    return tuple(o), tuple(f)
+
+
+def _mex_dims_helper(input_dim, num_instances, blocks, padding=[0], strides=[1], blocks_round_down=True,
+                     use_unshared_regions=True, shared_offset_region=[-1], unshared_offset_region=[-1]):
+    """Number of offset regions; same signature and C call as python/simnets/ops/mex.py:17-38."""
+    args = []
+
+    def add_array(l):
+        args.extend([C.c_int(len(l)), (C.c_int * len(l))(*[int(v) for v in l])])
+
+    add_array(input_dim)
+    add_array(padding)
+    add_array(strides)
+    args.extend([C.c_int(num_instances), C.c_int(blocks_round_down), C.c_int(use_unshared_regions)])
+    add_array(blocks)
+    add_array(shared_offset_region)
+    add_array(unshared_offset_region)
+    return _lib.lib().get_mex_offsets_nregions(*args)
+
+
+def _expand_dim_specification(image_shape, dim_spec):
+    """python/simnets/ops/mex.py:84-111: prepend -1 to a 2-list, replace -1 by the image dimension."""
+    if len(dim_spec) != 2 and len(dim_spec) != 3:
+        raise ValueError('Bad dimensions specifications, should be a list of two or three, got %s' % dim_spec)
+    image_shape = list(image_shape)
+    if len(image_shape) == 3:
+        image_shape = [None] + image_shape
+    dim_spec = list(dim_spec)
+    if len(dim_spec) == 2:
+        dim_spec = [-1] + dim_spec
+    for i in range(3):
+        if dim_spec[i] == -1:
+            dim_spec[i] = image_shape[i + 1]
+    return dim_spec
+
+
+def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
+        blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
+        shared_offset_region=None, unshared_offset_region=None, name=None, normalize_offsets=False, out=None):
+    """MEX forward; arguments as python/simnets/ops/mex.py:114-195.
+
+    input [B,C,H,W], offsets [num_regions, num_instances, bc, bh, bw] -> [B, channels_out*num_instances, oh, ow].
+    Extension: `normalize_offsets` applies the Keras layer's logsumexp normalisation on the device.
+    """
+    x = _require_cuda_f32("input", input)
+    off = _require_cuda_f32("offsets", offsets)
+    if x.dim() != 4:
+        raise SimnetsError(-15)
+    a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
+                  epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
+                  blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
+                  shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
+                  normalize_offsets=normalize_offsets)
+    l = _lib.lib()
+    xs = (C.c_int * 4)(*x.shape)
+    oshape = (C.c_int * 4)()
+    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    if out is None:
+        out = torch.empty(tuple(oshape), dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_contiguous() and tuple(out.shape) == tuple(oshape) and out.dtype == torch.float32
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
+                                     ws.data_ptr(), ws.numel(), stream))
+    return out
+
+
+def sum_pooling(input, pool_size=(2, 2), out=None):
+    """Non-overlapping 'valid' sum pooling: the AveragePooling2D * area glue of the reference's
+    missing-data example (README.md:108-111)."""
+    x = _require_cuda_f32("input", input)
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    B, Cc, H, W = x.shape
+    if out is None:
+        out = torch.empty((B, Cc, H // max(ph, 1), W // max(pw, 1)), dtype=torch.float32, device=x.device)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),
+                                                   stream))
+    return out

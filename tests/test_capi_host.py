@@ -1,0 +1,186 @@
+"""CPU-only checks of the C ABI: the library loads, exports every declared symbol, and its host-side
+validation / dimension logic agrees with the oracle and with the reference's known answers.  No
+compute entry point is called with data here (that needs a GPU)."""
+import ctypes as C
+import itertools
+import os
+import re
+import subprocess
+
+import pytest
+
+from oracle import oracle as orc
+from conftest import ROOT
+
+
+def test_library_exports_every_declared_symbol(pkg):
+    l = pkg._lib.lib()
+    header = open(os.path.join(ROOT, "include", "simnets_hip.h")).read()
+    declared = set(re.findall(r"\b((?:simnets_[a-z_0-9]+|get_mex_offsets_nregions))\s*\(", header))
+    declared -= {"simnets_status"}
+    assert declared == set(pkg._lib.EXPORTS)
+    for name in declared:
+        assert hasattr(l, name), name
+    assert l.simnets_hip_abi_version() == 1
+    assert pkg._lib.strerror(0) == "ok"
+
+
+def test_struct_layouts_match_the_header(pkg, tmp_path):
+    # sizes as a C compiler sees the header vs the ctypes mirrors
+    src = tmp_path / "sz.c"
+    src.write_text('#include <stdio.h>\n#include "simnets_hip.h"\nint main(void){printf("%zu %zu %zu\\n",'
+                   'sizeof(simnets_similarity_attrs),sizeof(simnets_mex_attrs),sizeof(simnets_mex_dims));return 0;}\n')
+    exe = tmp_path / "sz"
+    subprocess.run(["gcc", "-I" + os.path.join(ROOT, "include"), str(src), "-o", str(exe)], check=True)
+    sizes = [int(v) for v in subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.split()]
+    assert sizes == [C.sizeof(pkg._lib.SimilarityAttrs), C.sizeof(pkg._lib.MexAttrs), C.sizeof(pkg._lib.MexDims)]
+
+
+def test_similarity_defaults_are_the_registered_op_defaults(pkg):
+    a = pkg._lib.SimilarityAttrs()
+    pkg._lib.lib().simnets_similarity_attrs_default(C.byref(a))
+    assert (a.similarity_function, list(a.blocks), list(a.strides), list(a.padding)) == (1, [3, 3], [2, 2], [0, 0])
+    assert (a.normalization_term, a.ignore_nan_input, a.out_of_bounds_value) == (0, 0, 0.0)
+    assert abs(a.normalization_term_fudge - 0.001) < 1e-9
+    m = pkg._lib.MexAttrs()
+    pkg._lib.lib().simnets_mex_attrs_default(C.byref(m))
+    assert (list(m.padding), list(m.strides), list(m.blocks)) == ([0, 0, 0], [1, 1, 1], [1, 1, 1])
+    assert (m.epsilon, m.softmax_mode, m.blocks_round_down, m.use_unshared_regions) == (1.0, 0, 1, 1)
+    assert (m.n_shared, m.shared_offset_region[0], m.n_unshared, m.unshared_offset_region[0]) == (1, -1, 1, -1)
+
+
+@pytest.mark.parametrize("num_instances,padding,strides,blocks,in_shape,out_shape", [
+    (10, [0, 1], [1, 1], [2, 2], (3, 10, 13), (10, 9, 14)),
+    (10, [1, 1], [3, 2], [2, 2], (3, 10, 13), (10, 4, 7)),
+    (2, [1, 1], [3, 2], [2, 2], (1, 10, 13), (2, 4, 7)),
+])
+def test_similarity_known_answer_shapes(pkg, num_instances, padding, strides, blocks, in_shape, out_shape):
+    # python/simnets/test/keras/__init__.py:110-119
+    got = pkg.similarity_output_shape((5,) + in_shape, (num_instances, in_shape[0]) + tuple(blocks),
+                                      similarity_function="L1", blocks=blocks, strides=strides, padding=padding)
+    assert got == (5,) + out_shape
+
+
+@pytest.mark.parametrize("num_instances,padding,strides,blocks,in_shape,out_shape", [
+    (10, [1, 0, 1], [1, 1, 1], [1, 2, 2], (3, 10, 13), (50, 9, 14)),
+    (10, [2, 1, 1], [1, 3, 2], [1, 2, 2], (3, 10, 13), (70, 5, 8)),
+    (2, [1, 1, 1], [1, 3, 2], [1, 2, 2], (1, 10, 13), (6, 5, 8)),
+])
+def test_mex_known_answer_shapes(pkg, num_instances, padding, strides, blocks, in_shape, out_shape):
+    # python/simnets/test/keras/__init__.py:46-55
+    o, f = pkg.mex_output_shape((4,) + in_shape, num_instances, padding=padding, strides=strides, blocks=blocks,
+                                blocks_round_down=False, use_unshared_regions=False, shared_offset_region=[2],
+                                softmax_mode=True, epsilon=2.0)
+    assert o == (4,) + out_shape
+    assert f[1:] == (num_instances,) + tuple(blocks)
+
+
+def test_dims_helper_twin_of_the_reference_symbol(pkg):
+    # python/simnets/test/__init__.py:213
+    assert pkg._mex_dims_helper([1, 90, 90], 3, blocks=[1, 3, 3], padding=[0, 1, 1], strides=[1, 2, 2]) == 2025
+    assert pkg._mex_dims_helper([3, 8, 8], 3, blocks=[1, 3]) == -1
+    assert pkg._expand_dim_specification([5, 3, 10, 12], [2, 2]) == [3, 2, 2]
+    assert pkg._expand_dim_specification([3, 10, 12], [1, -1, 4]) == [1, 10, 4]
+    with pytest.raises(ValueError):
+        pkg._expand_dim_specification([3, 10, 12], [1])
+
+
+@pytest.mark.parametrize("unshared", [True, False])
+@pytest.mark.parametrize("spec", [[2], [3], [1, 5, 4], [-1], [2, 7, 1]])
+@pytest.mark.parametrize("geom", [((3, 41, 40), [1, 3, 3], [0, 1, 0], [1, 4, 1], True),
+                                  ((3, 10, 13), [2, 2, 2], [1, 1, 1], [1, 3, 2], False),
+                                  ((32, 16, 16), [32, 1, 1], [0, 0, 0], [32, 1, 1], True),
+                                  ((4, 9, 9), [4, 3, 3], [0, 0], [-1, 2, 2], True)])
+def test_mex_dims_agree_with_the_oracle(pkg, unshared, spec, geom):
+    image, blocks, padding, strides, rd = geom
+    kw = dict(blocks=blocks, padding=padding, strides=strides, blocks_round_down=rd, use_unshared_regions=unshared,
+              shared_offset_region=spec, unshared_offset_region=spec)
+    got = pkg.ops.mex_dims(image, 5, **kw)
+    want = orc.mex_dims(orc.mex_args((1,) + tuple(image), 5, **kw)).asdict()
+    assert got == want
+
+
+def test_similarity_validation_mirrors_the_reference(pkg):
+    E = pkg.SimnetsError
+    shp = ((2, 3, 10, 10), (4, 3, 3, 3))
+
+    def code(**kw):
+        kw.setdefault("blocks", [3, 3])
+        tshape = kw.pop("tshape", shp[1])
+        wshape = kw.pop("wshape", None)
+        try:
+            pkg.similarity_output_shape(shp[0], tshape, wshape, **kw)
+        except E as e:
+            return e.code
+        return 0
+
+    assert code() == 0
+    assert code(padding=[0]) == -2
+    assert code(blocks=[3]) == -3
+    assert code(strides=[1, 1, 1]) == -4
+    assert code(similarity_function="cosine") == -5
+    assert code(similarity_function="L1", normalization_term=True) == -6
+    assert code(ignore_nan_input=True) == -7
+    assert code(tshape=(4, 2, 3, 3)) == -8
+    assert code(wshape=(4, 2, 3, 3)) == -9
+    assert code(strides=[0, 1]) == -10
+    assert code(blocks=[2, 2]) == -15            # blocks attribute disagrees with the template tensor
+    assert code(blocks=[3, 3], tshape=(4, 3, 3, 3), wshape=(5, 3, 3, 3)) == -15
+    assert code(algo="mfma", normalization_term=True) == -18
+    assert "ignore_nan is relevant only if normalization_term is true" in pkg._lib.strerror(-7)
+    assert "normalization_term is relevant only if similarity_function is L2" in pkg._lib.strerror(-6)
+
+
+def test_mex_validation_mirrors_the_reference(pkg):
+    E = pkg.SimnetsError
+
+    def code(n=2, shape=(1, 3, 8, 8), **kw):
+        try:
+            pkg.mex_output_shape(shape, n, **kw)
+        except E as e:
+            return e.code
+        return 0
+
+    assert code() == 0
+    assert code(n=0) == -11
+    assert code(strides=[1, 1]) == -4
+    assert code(blocks=[1, 1]) == -3
+    assert code(padding=[1]) == -2
+    assert code(unshared_offset_region=[1, 2]) == -12
+    assert code(shared_offset_region=[1, 2]) == -13
+    assert code(blocks=[4, 1, 1]) == -14
+    assert code(strides=[1, 0, 1]) == -10
+    assert code(padding=[0, 0]) == 0              # two entries: -1 (the channel count) is prepended
+    assert "block depth must be smaller than input depth" in pkg._lib.strerror(-14)
+
+
+def test_compute_entry_points_reject_bad_arguments_without_touching_the_device(pkg):
+    l = pkg._lib.lib()
+    a = pkg.ops.similarity_attrs(blocks=[3, 3], ignore_nan_input=True)
+    I4 = C.c_int * 4
+    rc = l.simnets_hip_similarity_fwd(C.byref(a), I4(1, 3, 8, 8), I4(2, 3, 3, 3), I4(2, 3, 3, 3), None, None, None,
+                                      None, None, 0, None)
+    assert rc == -7
+    a = pkg.ops.similarity_attrs(blocks=[3, 3])
+    rc = l.simnets_hip_similarity_fwd(C.byref(a), I4(1, 3, 8, 8), I4(2, 3, 3, 3), I4(2, 3, 3, 3), None, None, None,
+                                      None, None, 0, None)
+    assert rc == -1
+    rc = l.simnets_hip_similarity_fwd(C.byref(a), I4(1, 3, 8, 8), I4(2, 3, 3, 3), I4(2, 3, 3, 3), 256, 256, 256, 256,
+                                      None, 0, None)
+    assert rc == -17
+    m = pkg.ops.mex_attrs(2, blocks=[3, 1, 1])
+    rc = l.simnets_hip_mex_fwd(C.byref(m), I4(1, 3, 8, 8), 256, 256, 5, 256, None, 0, None)
+    assert rc == -15                               # offsets buffer shorter than R*M*K
+    nbytes = C.c_size_t()
+    assert l.simnets_hip_mex_workspace_bytes(C.byref(m), I4(1, 3, 8, 8), C.byref(nbytes)) == 0
+    assert nbytes.value >= 64 * 2 * 3 * 4
+    assert l.simnets_hip_sum_pool_fwd(I4(1, 1, 4, 4), 0, 2, None, None, None) == -15
+
+
+def test_op_layer_refuses_cpu_tensors(pkg):
+    import torch
+    x = torch.zeros(1, 1, 4, 4)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        pkg.similarity(x, x, x, blocks=[4, 4])
+    with pytest.raises(TypeError):
+        pkg.similarity(x.double(), x, x, blocks=[4, 4])

@@ -1,0 +1,255 @@
+"""GPU parity: the HIP library (called through the C ABI via the op layer) against the CPU oracle
+on the same seeded inputs.  Similarity must agree to 1e-5 relative with identical NaN positions,
+MEX to 1e-4 relative (error metric: tests/util.py:rel_err)."""
+import itertools
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from util import config1, config2, config3, rel_err
+
+pytestmark = pytest.mark.gpu
+
+SIM_TOL = 1e-5
+MEX_TOL = 1e-4
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def run_similarity(pkg, x, t, w, **kw):
+    out = pkg.similarity(dev(x), dev(t), dev(w), **kw)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def run_mex(pkg, x, off, n, **kw):
+    out = pkg.mex(dev(x), dev(off), n, **kw)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def sim_inputs(seed, shape, O, blocks, nan_frac=0.0):
+    g = np.random.default_rng(seed)
+    x = g.normal(size=shape).astype(np.float32)
+    t = g.normal(size=(O, shape[1]) + tuple(blocks)).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    if nan_frac:
+        x[g.random(size=x.shape) < nan_frac] = np.nan
+    return x, t, w
+
+
+# ---- the reference's own test matrices (python/simnets/test/__init__.py:106-141) -------------------
+@pytest.mark.parametrize("strides", [[1, 1], [1, 2], [2, 1], [2, 2]])
+@pytest.mark.parametrize("blocks", [[1, 1], [1, 3], [3, 1], [3, 3]])
+@pytest.mark.parametrize("same", [True, False])
+@pytest.mark.parametrize("shape", [(1, 1, 40, 40), (2, 3, 40, 40)])
+def test_similarity_reference_dimensions(pkg, strides, blocks, same, shape):
+    x, t, w = sim_inputs(1, shape, 1, blocks)
+    kw = dict(blocks=blocks, strides=strides, padding=[b // 2 for b in blocks] if same else [0, 0])
+    assert rel_err(run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+
+
+@pytest.mark.parametrize("func,norm,ign", [("L2", False, False), ("L2", True, False), ("L2", True, True),
+                                           ("L1", False, False)])
+@pytest.mark.parametrize("O", [1, 5, 32])
+def test_similarity_reference_params(pkg, func, norm, ign, O):
+    x, t, w = sim_inputs(2, (3, 3, 30, 30), O, (3, 3), nan_frac=0.2 if ign else 0.0)
+    kw = dict(similarity_function=func, blocks=[3, 3], strides=[2, 2], padding=[1, 1], normalization_term=norm,
+              ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else 0.0)
+    assert rel_err(run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+
+
+def test_similarity_l1_on_a_single_pixel(pkg):
+    x, t, w = sim_inputs(3, (1, 1, 1, 1), 1, (1, 1))
+    kw = dict(similarity_function="L1", blocks=[1, 1], strides=[1, 1], padding=[0, 0])
+    assert rel_err(run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+
+
+# ---- geometry edge cases --------------------------------------------------------------------------
+@pytest.mark.parametrize("case", [
+    dict(shape=(2, 3, 50, 31), O=7, blocks=[3, 2], strides=[1, 2], padding=[0, 1]),
+    dict(shape=(1, 2, 9, 70), O=33, blocks=[5, 5], strides=[3, 3], padding=[2, 2]),
+    dict(shape=(2, 1, 28, 28), O=3, blocks=[28, 28], strides=[1, 1], padding=[0, 0]),   # one output pixel
+    dict(shape=(3, 4, 12, 200), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),   # wide rows
+    dict(shape=(1, 130, 6, 6), O=17, blocks=[2, 2], strides=[1, 1], padding=[1, 1]),    # many channels
+    dict(shape=(2, 2, 5, 5), O=2, blocks=[2, 2], strides=[4, 5], padding=[3, 3]),       # padding beyond the block
+    dict(shape=(1, 1, 3, 2100), O=9, blocks=[3, 5], strides=[1, 1], padding=[1, 2]),    # rows too long for the LDS tile
+])
+@pytest.mark.parametrize("func", ["L1", "L2"])
+def test_similarity_geometries(pkg, case, func):
+    x, t, w = sim_inputs(4, case["shape"], case["O"], case["blocks"])
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+              out_of_bounds_value=-0.75)
+    assert rel_err(run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+
+
+def test_similarity_nan_positions_without_ignore_nan(pkg):
+    # NaN padding and NaN pixels must poison exactly the outputs whose patch contains them
+    x, t, w = sim_inputs(5, (2, 2, 12, 12), 6, (3, 3), nan_frac=0.03)
+    for func, norm in (("L1", False), ("L2", False), ("L2", True)):
+        kw = dict(similarity_function=func, blocks=[3, 3], strides=[1, 1], padding=[1, 1],
+                  normalization_term=norm, out_of_bounds_value=float("nan"))
+        got, want = run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)
+        assert np.isnan(want).any() and not np.isnan(want).all()
+        assert rel_err(got, want) <= SIM_TOL
+
+
+def test_similarity_normalization_constant_modes(pkg):
+    x, t, w = sim_inputs(6, (4, 2, 8, 8), 3, (3, 3))
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[0, 0], normalization_term=True)
+    for every in (False, True):
+        got = run_similarity(pkg, x, t, w, norm_const_every_iteration=every, **kw)
+        want = orc.similarity_fwd(x, t, w, norm_const_every_iteration=every, **kw)
+        assert rel_err(got, want) <= SIM_TOL
+
+
+def test_similarity_empty_batch(pkg):
+    x = torch.empty((0, 3, 8, 8), device="cuda")
+    t = torch.zeros((2, 3, 3, 3), device="cuda")
+    out = pkg.similarity(x, t, t.abs(), blocks=[3, 3], strides=[1, 1], padding=[0, 0])
+    assert tuple(out.shape) == (0, 2, 6, 6)
+
+
+def test_similarity_sqrtw_algorithm_matches_direct(pkg):
+    x, t, w = sim_inputs(7, (2, 8, 20, 20), 16, (3, 3))
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    want = orc.similarity_fwd(x, t, w, **kw)
+    assert rel_err(run_similarity(pkg, x, t, w, algo="sqrtw", **kw), want) <= SIM_TOL
+
+
+# ---- BASELINE configurations ------------------------------------------------------------------------
+def test_config1_similarity_missing_data_layer(pkg):
+    x, t, w, kw = config1(batch=64, nan_frac=0.25)
+    got, want = run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)
+    assert got.shape == (64, 32, 16, 16) and not np.isnan(got).any()
+    ring = np.ones((16, 16), bool)
+    ring[1:-1, 1:-1] = False
+    assert np.all(got[:, :, ring] == 0.0) and not np.signbit(got[:, :, ring]).any()
+    assert rel_err(got, want) <= SIM_TOL
+
+
+@pytest.mark.parametrize("func", ["L2", "L1"])
+def test_config3_similarity_conv_scale_sampled(pkg, func):
+    # full-size launch (256 x 64 x 32 x 32, 128 templates); the oracle checks a sample of images
+    x, t, w, kw = config3()
+    got = run_similarity(pkg, x, t, w, similarity_function=func, **kw)
+    assert got.shape == (256, 128, 32, 32)
+    idx = [0, 101, 255]
+    want = orc.similarity_fwd(x[idx], t, w, similarity_function=func, **kw)
+    assert rel_err(got[idx], want) <= SIM_TOL
+    # size-independent property over the whole batch: permuting the images permutes the outputs
+    perm = np.random.default_rng(0).permutation(256)
+    got2 = run_similarity(pkg, x[perm], t, w, similarity_function=func, **kw)
+    assert np.array_equal(got2, got[perm])
+
+
+def test_config2_mex(pkg):
+    x, off, n, kw = config2()
+    offn = orc.normalize_offsets(off)
+    want = orc.mex_fwd(x, offn, n, **kw)
+    assert rel_err(run_mex(pkg, x, off, n, normalize_offsets=True, **kw), want) <= MEX_TOL
+    assert rel_err(run_mex(pkg, x, offn, n, **kw), want) <= MEX_TOL
+
+
+# ---- MEX: the reference's region matrices (python/simnets/test/__init__.py:299-327) and more --------
+def mex_inputs(seed, im_dims, num_instances, **kw):
+    g = np.random.default_rng(seed)
+    d = orc.mex_dims(orc.mex_args(im_dims, num_instances, **kw))
+    x = g.normal(size=im_dims).astype(np.float32)
+    off = g.normal(size=(d.num_regions, num_instances) + tuple(kw["blocks"])).astype(np.float32)
+    return x, off
+
+
+@pytest.mark.parametrize("unshared,spec", [(False, [2]), (False, [3]), (True, [1, 5, 4]), (True, [2])])
+@pytest.mark.parametrize("strides", [[1, 1, 1], [1, 1, 4], [1, 4, 1], [1, 4, 4]])
+@pytest.mark.parametrize("blocks", [[1, 1, 3], [1, 3, 3]])
+@pytest.mark.parametrize("im_dims", [(1, 1, 41, 40), (2, 3, 40, 40), (2, 3, 41, 40)])
+def test_mex_reference_region_matrix(pkg, unshared, spec, strides, blocks, im_dims):
+    kw = dict(softmax_mode=True, padding=[0, 1, 0], strides=strides, blocks=blocks, use_unshared_regions=unshared,
+              shared_offset_region=spec if not unshared else [2], unshared_offset_region=spec if unshared else [1])
+    x, off = mex_inputs(11, im_dims, 2, **kw)
+    assert rel_err(run_mex(pkg, x, off, 2, **kw), orc.mex_fwd(x, off, 2, **kw)) <= MEX_TOL
+
+
+@pytest.mark.parametrize("eps", [1.0, 2.0, -1.5, 0.25, math.inf, -math.inf])
+@pytest.mark.parametrize("softmax", [True, False])
+def test_mex_sanity_geometry_epsilons(pkg, eps, softmax):
+    kw = dict(softmax_mode=softmax, blocks=[1, 3, 3], padding=[0, 1, 1], strides=[1, 2, 2], epsilon=eps)
+    x, off = mex_inputs(12, (5, 1, 90, 90), 3, **kw)
+    assert off.shape[0] == 2025
+    assert rel_err(run_mex(pkg, x, off, 3, **kw), orc.mex_fwd(x, off, 3, **kw)) <= MEX_TOL
+
+
+@pytest.mark.parametrize("round_down", [True, False])
+@pytest.mark.parametrize("unshared", [True, False])
+def test_mex_3d_blocks_channel_padding_round_up(pkg, round_down, unshared):
+    kw = dict(softmax_mode=False, blocks=[2, 2, 2], padding=[1, 1, 1], strides=[1, 3, 2], epsilon=0.7,
+              blocks_out_of_bounds_value=-1.5, blocks_round_down=round_down, use_unshared_regions=unshared,
+              shared_offset_region=[2, 2, 3], unshared_offset_region=[2, 3, 2])
+    x, off = mex_inputs(13, (3, 3, 10, 13), 20, **kw)
+    assert rel_err(run_mex(pkg, x, off, 20, **kw), orc.mex_fwd(x, off, 20, **kw)) <= MEX_TOL
+
+
+@pytest.mark.parametrize("case", [
+    dict(im=(7, 64, 8, 8), n=128), dict(im=(9, 128, 4, 4), n=256), dict(im=(5, 256, 2, 2), n=512),
+    dict(im=(6, 512, 1, 1), n=10, shared=True),
+])
+def test_mex_missing_data_stack_layers(pkg, case):
+    Cc = case["im"][1]
+    kw = dict(softmax_mode=True, blocks=[Cc, 1, 1], strides=[Cc, 1, 1])
+    if case.get("shared"):
+        kw.update(use_unshared_regions=True, shared_offset_region=[1])
+    else:
+        kw.update(use_unshared_regions=True, unshared_offset_region=[2])
+    x, off = mex_inputs(14, case["im"], case["n"], **kw)
+    want = orc.mex_fwd(x, orc.normalize_offsets(off), case["n"], **kw)
+    assert rel_err(run_mex(pkg, x, off, case["n"], normalize_offsets=True, **kw), want) <= MEX_TOL
+
+
+def test_mex_large_dynamic_range(pkg):
+    # log-probability-like inputs spanning hundreds of units must not overflow or lose the max term
+    g = np.random.default_rng(15)
+    x = (g.normal(size=(4, 16, 6, 6)) * 150).astype(np.float32)
+    off = np.log(g.dirichlet([1.0] * 16, size=(4, 8))).astype(np.float32).reshape(4, 8, 16, 1, 1)
+    kw = dict(softmax_mode=True, blocks=[16, 1, 1], strides=[16, 1, 1], unshared_offset_region=[2])
+    assert rel_err(run_mex(pkg, x, off, 8, **kw), orc.mex_fwd(x, off, 8, **kw)) <= MEX_TOL
+
+
+def test_sum_pooling(pkg):
+    g = np.random.default_rng(16)
+    x = g.normal(size=(3, 5, 9, 8)).astype(np.float32)
+    got = pkg.sum_pooling(dev(x), (2, 2)).cpu().numpy()
+    want = x[:, :, :8].reshape(3, 5, 4, 2, 4, 2).sum(axis=(3, 5))
+    assert got.shape == (3, 5, 4, 4)
+    np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
+
+
+def test_missing_data_stack_end_to_end(pkg):
+    # BASELINE configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10)
+    B = 16
+    x, t, w, kw = config1(batch=B, nan_frac=0.25)
+    g = np.random.default_rng(4567)
+    cur_gpu = pkg.similarity(dev(x), dev(t), dev(w), **kw)
+    cur_cpu = orc.similarity_fwd(x, t, w, **kw)
+    ch = 32
+    for layer in range(4):
+        n = ch * 2
+        size = cur_cpu.shape[-1]
+        mkw = dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], unshared_offset_region=[2])
+        off = (g.normal(size=(min(2, size) ** 2, n, ch, 1, 1)) * 0.1).astype(np.float32)
+        cur_gpu = pkg.sum_pooling(pkg.mex(cur_gpu, dev(off), n, normalize_offsets=True, **mkw), (2, 2))
+        m = orc.mex_fwd(cur_cpu, orc.normalize_offsets(off), n, **mkw)
+        cur_cpu = m.reshape(B, n, size // 2, 2, size // 2, 2).sum(axis=(3, 5), dtype=np.float32)
+        ch = n
+        assert rel_err(cur_gpu.cpu().numpy(), cur_cpu) <= MEX_TOL
+    off = (g.normal(size=(1, 10, ch, 1, 1)) * 0.1).astype(np.float32)
+    mkw = dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], shared_offset_region=[1])
+    got = pkg.mex(cur_gpu, dev(off), 10, normalize_offsets=True, **mkw).cpu().numpy()
+    want = orc.mex_fwd(cur_cpu, orc.normalize_offsets(off), 10, **mkw)
+    assert got.shape == (B, 10, 1, 1)
+    assert rel_err(got, want) <= MEX_TOL
