@@ -35,6 +35,9 @@ def main():
                     help="evaluation path of the headline Similarity kernel (default: the library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
+    ap.add_argument("--pmc-calib", action="store_true",
+                    help="also run three 256 MiB device-to-device copies (a plain copy kernel of known size, "
+                         "used to scale the FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-images", type=int, default=2, help="images of configuration 3 the CPU baseline times")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -73,6 +76,14 @@ def main():
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return wall, start.elapsed_time(stop) / steps
+
+    if args.pmc_calib:
+        src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ------------------------------------------------------------------ headline: configuration 3, L2
     x3, t3, w3, kw3 = config3()

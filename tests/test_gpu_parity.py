@@ -151,12 +151,19 @@ def test_config3_similarity_conv_scale_sampled(pkg, func):
 def test_config2_mex(pkg):
     x, off, n, kw = config2()
     offn = orc.normalize_offsets(off)
-    want = orc.mex_fwd(x, offn, n, **kw)
-    assert rel_err(run_mex(pkg, x, off, n, normalize_offsets=True, **kw), want) <= MEX_TOL
-    assert rel_err(run_mex(pkg, x, offn, n, **kw), want) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, off, n, normalize_offsets=True, **kw), x, offn, n, **kw) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, offn, n, **kw), x, offn, n, **kw) <= MEX_TOL
 
 
 # ---- MEX: the reference's region matrices (python/simnets/test/__init__.py:299-327) and more --------
+def mex_err(got, x, off, n, **kw):
+    """MEX parity metric: relative to max(|want|, |m|), m = the max (min for eps < 0) term."""
+    want = orc.mex_fwd(x, off, n, **kw)
+    eps = kw.get("epsilon", 1.0)
+    shift = orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, eps)))
+    return rel_err(got, want, floor=shift)
+
+
 def mex_inputs(seed, im_dims, num_instances, **kw):
     g = np.random.default_rng(seed)
     d = orc.mex_dims(orc.mex_args(im_dims, num_instances, **kw))
@@ -173,7 +180,7 @@ def test_mex_reference_region_matrix(pkg, unshared, spec, strides, blocks, im_di
     kw = dict(softmax_mode=True, padding=[0, 1, 0], strides=strides, blocks=blocks, use_unshared_regions=unshared,
               shared_offset_region=spec if not unshared else [2], unshared_offset_region=spec if unshared else [1])
     x, off = mex_inputs(11, im_dims, 2, **kw)
-    assert rel_err(run_mex(pkg, x, off, 2, **kw), orc.mex_fwd(x, off, 2, **kw)) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, off, 2, **kw), x, off, 2, **kw) <= MEX_TOL
 
 
 @pytest.mark.parametrize("eps", [1.0, 2.0, -1.5, 0.25, math.inf, -math.inf])
@@ -182,7 +189,7 @@ def test_mex_sanity_geometry_epsilons(pkg, eps, softmax):
     kw = dict(softmax_mode=softmax, blocks=[1, 3, 3], padding=[0, 1, 1], strides=[1, 2, 2], epsilon=eps)
     x, off = mex_inputs(12, (5, 1, 90, 90), 3, **kw)
     assert off.shape[0] == 2025
-    assert rel_err(run_mex(pkg, x, off, 3, **kw), orc.mex_fwd(x, off, 3, **kw)) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, off, 3, **kw), x, off, 3, **kw) <= MEX_TOL
 
 
 @pytest.mark.parametrize("round_down", [True, False])
@@ -192,7 +199,7 @@ def test_mex_3d_blocks_channel_padding_round_up(pkg, round_down, unshared):
               blocks_out_of_bounds_value=-1.5, blocks_round_down=round_down, use_unshared_regions=unshared,
               shared_offset_region=[2, 2, 3], unshared_offset_region=[2, 3, 2])
     x, off = mex_inputs(13, (3, 3, 10, 13), 20, **kw)
-    assert rel_err(run_mex(pkg, x, off, 20, **kw), orc.mex_fwd(x, off, 20, **kw)) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, off, 20, **kw), x, off, 20, **kw) <= MEX_TOL
 
 
 @pytest.mark.parametrize("case", [
@@ -207,8 +214,8 @@ def test_mex_missing_data_stack_layers(pkg, case):
     else:
         kw.update(use_unshared_regions=True, unshared_offset_region=[2])
     x, off = mex_inputs(14, case["im"], case["n"], **kw)
-    want = orc.mex_fwd(x, orc.normalize_offsets(off), case["n"], **kw)
-    assert rel_err(run_mex(pkg, x, off, case["n"], normalize_offsets=True, **kw), want) <= MEX_TOL
+    got = run_mex(pkg, x, off, case["n"], normalize_offsets=True, **kw)
+    assert mex_err(got, x, orc.normalize_offsets(off), case["n"], **kw) <= MEX_TOL
 
 
 def test_mex_large_dynamic_range(pkg):
@@ -217,7 +224,7 @@ def test_mex_large_dynamic_range(pkg):
     x = (g.normal(size=(4, 16, 6, 6)) * 150).astype(np.float32)
     off = np.log(g.dirichlet([1.0] * 16, size=(4, 8))).astype(np.float32).reshape(4, 8, 16, 1, 1)
     kw = dict(softmax_mode=True, blocks=[16, 1, 1], strides=[16, 1, 1], unshared_offset_region=[2])
-    assert rel_err(run_mex(pkg, x, off, 8, **kw), orc.mex_fwd(x, off, 8, **kw)) <= MEX_TOL
+    assert mex_err(run_mex(pkg, x, off, 8, **kw), x, off, 8, **kw) <= MEX_TOL
 
 
 def test_sum_pooling(pkg):
@@ -230,26 +237,28 @@ def test_sum_pooling(pkg):
 
 
 def test_missing_data_stack_end_to_end(pkg):
-    # BASELINE configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10)
+    # BASELINE configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10).
+    # Each layer is checked on the GPU's own previous activations, so tolerances do not compound.
     B = 16
     x, t, w, kw = config1(batch=B, nan_frac=0.25)
     g = np.random.default_rng(4567)
-    cur_gpu = pkg.similarity(dev(x), dev(t), dev(w), **kw)
-    cur_cpu = orc.similarity_fwd(x, t, w, **kw)
+    cur = pkg.similarity(dev(x), dev(t), dev(w), **kw)
+    assert rel_err(cur.cpu().numpy(), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
     ch = 32
     for layer in range(4):
-        n = ch * 2
-        size = cur_cpu.shape[-1]
+        n, size = ch * 2, cur.shape[-1]
         mkw = dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], unshared_offset_region=[2])
         off = (g.normal(size=(min(2, size) ** 2, n, ch, 1, 1)) * 0.1).astype(np.float32)
-        cur_gpu = pkg.sum_pooling(pkg.mex(cur_gpu, dev(off), n, normalize_offsets=True, **mkw), (2, 2))
-        m = orc.mex_fwd(cur_cpu, orc.normalize_offsets(off), n, **mkw)
-        cur_cpu = m.reshape(B, n, size // 2, 2, size // 2, 2).sum(axis=(3, 5), dtype=np.float32)
+        inp = cur.cpu().numpy()
+        m = pkg.mex(cur, dev(off), n, normalize_offsets=True, **mkw)
+        assert mex_err(m.cpu().numpy(), inp, orc.normalize_offsets(off), n, **mkw) <= MEX_TOL
+        cur = pkg.sum_pooling(m, (2, 2))
+        pooled = m.cpu().numpy().reshape(B, n, size // 2, 2, size // 2, 2)
+        want = (pooled[:, :, :, 0, :, 0] + pooled[:, :, :, 0, :, 1]) + pooled[:, :, :, 1, :, 0] + pooled[:, :, :, 1, :, 1]
+        assert np.array_equal(cur.cpu().numpy(), want)
         ch = n
-        assert rel_err(cur_gpu.cpu().numpy(), cur_cpu) <= MEX_TOL
     off = (g.normal(size=(1, 10, ch, 1, 1)) * 0.1).astype(np.float32)
     mkw = dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], shared_offset_region=[1])
-    got = pkg.mex(cur_gpu, dev(off), 10, normalize_offsets=True, **mkw).cpu().numpy()
-    want = orc.mex_fwd(cur_cpu, orc.normalize_offsets(off), 10, **mkw)
+    got = pkg.mex(cur, dev(off), 10, normalize_offsets=True, **mkw).cpu().numpy()
     assert got.shape == (B, 10, 1, 1)
-    assert rel_err(got, want) <= MEX_TOL
+    assert mex_err(got, cur.cpu().numpy(), orc.normalize_offsets(off), 10, **mkw) <= MEX_TOL

@@ -2,10 +2,14 @@
 import numpy as np
 
 
-def rel_err(got, want):
-    """max |got - want| / max(|want|, 1e-6 * max|want|) over finite entries of `want`.
+def rel_err(got, want, floor=None):
+    """max |got - want| / max(|want|, floor, 1e-6 * max|want|) over finite entries of `want`.
 
     Outputs may cross zero, so the denominator has an absolute floor tied to the tensor's scale.
+    `floor` (array like `want`, optional) raises it per element: MEX passes |m|, the shift
+    m = max_k(patch_k + offset_k) that every implementation subtracts before exponentiating.
+    The MEX output is m + log(sum exp(eps (v - m))) / eps, so its rounding noise is proportional
+    to |m| even where the two terms cancel and the output itself is near zero.
     NaN / Inf positions must coincide and are excluded from the ratio.
     """
     got = np.asarray(got, dtype=np.float64)
@@ -19,6 +23,8 @@ def rel_err(got, want):
         return 0.0
     scale = np.abs(want[fin]).max()
     den = np.maximum(np.abs(want[fin]), 1e-6 * scale)
+    if floor is not None:
+        den = np.maximum(den, np.abs(np.asarray(floor, dtype=np.float64))[fin])
     den = np.maximum(den, np.finfo(np.float64).tiny)
     return float((np.abs(got[fin] - want[fin]) / den).max())
 
