@@ -23,6 +23,7 @@
 #include <cmath>
 
 #include "internal.h"
+#include "stage.h"
 
 namespace simnets {
 
@@ -154,22 +155,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_direct_kernel(const SimKernel
         const int ccn = min(a.CC, a.C - ch0);
         __syncthreads();
         // ---- stage ccn channels x TR rows x TC columns; out-of-image -> oob ----
-        for (int cc = 0; cc < ccn; ++cc) {
-            const float *chan = img + (size_t)(ch0 + cc) * a.H * a.W;
-            for (int r = wave; r < TR; r += kWaves) {
-                const int ih = in_row0 + r;
-                const bool row_ok = ih >= 0 && ih < a.H;
-                const float *rowp = chan + (size_t)(row_ok ? ih : 0) * a.W;
-                float *dst = lds + cc * chan_lds + r * a.TC;
-                for (int col = lane; col < a.TC; col += 64) {
-                    const int iw = col - a.pw;
-                    float v = a.oob;
-                    if (row_ok && iw >= 0 && iw < a.W)
-                        v = rowp[iw];
-                    dst[col] = v;
-                }
-            }
-        }
+        stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.pw, a.oob,
+                                      nullptr);
         __syncthreads();
         if (!wave_active)
             continue;

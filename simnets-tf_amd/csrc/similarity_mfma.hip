@@ -1,15 +1,350 @@
-// Placeholder for the matrix-core evaluation of plain L2 Similarity (SIMNETS_ALGO_MFMA).
+// Similarity forward, plain L2 only, on the fp32 matrix cores (gfx950 v_mfma_f32_32x32x2_f32).
+//
+// The weighted squared distance is expanded into dense contractions over k:
+//   out[b,m,p] = -sum_k w (t - x)^2
+//              = sum_k (-w[m,k]) * x[p,k]^2  +  sum_k (2 w[m,k] t[m,k]) * x[p,k]  -  sum_k w[m,k] t[m,k]^2
+// i.e. one GEMM with K' = 2K whose left operand is the packed parameter matrix [-w | 2wt] and whose
+// right operand is the implicit im2col matrix [x^2 ; x], plus a per-template bias.  Same operator as
+// the direct kernel (src/kernels/similarity_kernel_gpu.cu:24-133 + sim_l2_forward,
+// include/utils/similarity_utils.hpp:23-36 in the reference) but a different rounding path: the three
+// sums cancel where a patch is close to a template, and NaN / Inf inputs do not marginalise, so this
+// path is opt-in (SIMNETS_ALGO_MFMA) and is checked against the direct path.
+// To keep the cancellation benign, templates and input are shifted per input channel by the mean
+// template value of that channel before squaring ((t - c) - (x - c) = t - x).
+//
+// Work split: a workgroup of 4 waves owns 256 consecutive output pixels of one image and up to 128
+// templates; wave (wm, wp) owns 64 templates x 128 pixels = 2 x 4 MFMA tiles of 32x32 (128
+// accumulator VGPRs).  Templates are the MFMA row index and pixels the column index, so each lane
+// ends up with 16 values of ONE pixel column and stores run along w: coalesced.
+//   * input rows are staged, a few channels at a time, into LDS (out of image -> out_of_bounds_value,
+//     shift applied); a lane reads the pixel operand with one ds_read_b32 per tile and k-pair and
+//     squares it in the VALU, which is otherwise idle;
+//   * the two k of an MFMA k-pair are the same tap (dh, dw) of two adjacent channels, so the
+//     per-lane LDS address is base + uniform offset;
+//   * the parameter operand is read straight from a pre-packed global array in consumption order
+//     (L1/L2 resident: every workgroup walks it in the same order), two steps ahead of its use.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
+
 #include "internal.h"
+#include "stage.h"
 
 namespace simnets {
 
-size_t sim_mfma_workspace_bytes(const SimPlan &) { return 0; }
+namespace {
 
-int sim_mfma_launch(const SimPlan &, const float *, const float *, const float *, float *, void *, size_t, hipStream_t)
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int kThreads = 256;
+constexpr int RM = 2;           // 32-template tiles per wave
+constexpr int RP = 4;           // 32-pixel tiles per wave
+constexpr int WG_PIX = 2 * RP * 32;   // 256 pixels per workgroup (2 pixel waves)
+constexpr int WG_TPL = 2 * RM * 32;   // 128 templates per workgroup (2 template waves)
+constexpr int kLdsBudgetFloats = 12288;  // 48 KiB input tile per workgroup
+
+struct MfmaArgs {
+    const float *in;
+    float *out;
+    const float *pm;    // [step][type][half][Opad]
+    const float *bias;  // [Opad]
+    const float *ctr;   // [C] per-channel shift
+    int B, C, H, W, O, Opad, oh, ow, npix;
+    int bh, bw, sh, sw, ph, pw;
+    int tiles;          // workgroup pixel tiles per image
+    int TC, TRmax, chan_lds, CC;
+    float oob;
+};
+
+__global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
 {
-    return SIMNETS_ERR_ALGO;
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wp = wave >> 1;
+    const int col = lane & 31, half = lane >> 5;
+
+    const int b = blockIdx.x / a.tiles;
+    const int tile = blockIdx.x - b * a.tiles;
+    const int p_first = tile * WG_PIX;
+    const int p_last = min(p_first + WG_PIX, a.npix) - 1;
+    const int h_first = p_first / a.ow;
+    const int nrows = p_last / a.ow - h_first + 1;
+    const int TR = (nrows - 1) * a.sh + a.bh;
+    const int in_row0 = h_first * a.sh - a.ph;
+    const int mbase = blockIdx.y * WG_TPL + wm * (RM * 32);
+
+    // per pixel tile: LDS address of this lane's pixel (k-pair half folded in)
+    int xbase[RP], pix[RP];
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        const int p = p_first + (wp * RP + j) * 32 + col;
+        pix[j] = p;
+        const int pc = min(p, p_last);
+        const int h = pc / a.ow, w = pc - h * a.ow;
+        xbase[j] = (h - h_first) * a.sh * a.TC + w * a.sw + half * a.chan_lds;
+    }
+
+    floatx16 acc[RM][RP];
+#pragma unroll
+    for (int i = 0; i < RM; ++i) {
+        floatx16 init;
+#pragma unroll
+        for (int v = 0; v < 16; ++v)
+            init[v] = a.bias[mbase + i * 32 + 8 * (v / 4) + 4 * half + (v % 4)];
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+            acc[i][j] = init;
+    }
+
+    // parameter operand: this lane's element within a [type][half][Opad] step record
+    const int step_stride = 4 * a.Opad;
+    const float *pm = a.pm + half * a.Opad + mbase + col;
+    const float *img = a.in + (size_t)b * a.C * a.H * a.W;
+
+    float pw_cur[RM], pt_cur[RM], pw_nxt[RM], pt_nxt[RM];
+    auto load_params = [&](const float *p, float (&w_)[RM], float (&t_)[RM]) {
+#pragma unroll
+        for (int i = 0; i < RM; ++i) {
+            w_[i] = p[i * 32];
+            t_[i] = p[2 * a.Opad + i * 32];
+        }
+    };
+    load_params(pm, pw_cur, pt_cur);
+    load_params(pm + step_stride, pw_nxt, pt_nxt);
+    pm += 2 * step_stride;
+
+    for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
+        const int ccn = min(a.CC, a.C - ch0);
+        const int ccp = (ccn + 1) & ~1;
+        __syncthreads();
+        stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccp, ccn, TR, a.TC, a.chan_lds, in_row0, a.pw, a.oob,
+                                      a.ctr);
+        __syncthreads();
+
+        // steps of this chunk in (channel pair, dh, dw) order; the pixel operand of step s+1 and the
+        // parameter operand of step s+2 are requested before the MFMAs of step s are issued
+        const int nsteps = (ccp / 2) * a.bh * a.bw;
+        int dh = 0, dw = 0, row_off = 0, off = 0;
+        float xn[RP];
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+            xn[j] = lds[xbase[j]];
+        for (int st = 0; st < nsteps; ++st) {
+            float x[RP], x2[RP];
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+                x[j] = xn[j];
+            int ndw = dw + 1, ndh = dh, nrow = row_off;
+            if (ndw == a.bw) {
+                ndw = 0;
+                ++ndh;
+                nrow += a.TC;
+                if (ndh == a.bh) {
+                    ndh = 0;
+                    nrow += 2 * a.chan_lds - a.bh * a.TC;
+                }
+            }
+            int noff = nrow + ndw;
+            if (st + 1 == nsteps)
+                noff = off;
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+                xn[j] = lds[xbase[j] + noff];
+            float pw_nn[RM], pt_nn[RM];
+            load_params(pm, pw_nn, pt_nn);
+            pm += step_stride;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int j = 0; j < RP; ++j)
+                x2[j] = x[j] * x[j];
+#pragma unroll
+            for (int i = 0; i < RM; ++i)
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[i], x2[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < RM; ++i)
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[i], x[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+            for (int i = 0; i < RM; ++i) {
+                pw_cur[i] = pw_nxt[i]; pt_cur[i] = pt_nxt[i];
+                pw_nxt[i] = pw_nn[i];  pt_nxt[i] = pt_nn[i];
+            }
+            dw = ndw; dh = ndh; row_off = nrow; off = noff;
+        }
+    }
+
+    // ---- store: lane holds, per tile, 16 templates of one pixel ----
+    const size_t plane = (size_t)a.npix;
+    float *ob = a.out + (size_t)b * a.O * plane;
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+        if (pix[j] > p_last)
+            continue;
+#pragma unroll
+        for (int i = 0; i < RM; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int m = mbase + i * 32 + 8 * (v / 4) + 4 * half + (v % 4);
+                if (m < a.O)
+                    ob[(size_t)m * plane + pix[j]] = acc[i][j][v];
+            }
+    }
+}
+
+// ctr[c] = mean over (m, dh, dw) of templates[m, c, dh, dw]
+__global__ __launch_bounds__(256) void mfma_center_kernel(const float *__restrict__ templates, int O, int C, int bhw,
+                                                          float *__restrict__ ctr)
+{
+    __shared__ float red[256];
+    const int c = blockIdx.x;
+    float s = 0.0f;
+    const int n = O * bhw;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const int m = i / bhw, r = i - m * bhw;
+        s += templates[((size_t)m * C + c) * bhw + r];
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int d = 128; d > 0; d >>= 1) {
+        if (threadIdx.x < d)
+            red[threadIdx.x] += red[threadIdx.x + d];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0)
+        ctr[c] = red[0] / (float)n;
+}
+
+// pm[step][type][half][Opad], step = ((cpair * bh) + dh) * bw + dw, channel = 2 * cpair + half
+__global__ void mfma_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
+                                 const float *__restrict__ ctr, int O, int Opad, int C, int bh, int bw,
+                                 long long total, float *__restrict__ pm)
+{
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int m = (int)(i % Opad);
+        long long r = i / Opad;
+        const int half = (int)(r & 1); r >>= 1;
+        const int type = (int)(r & 1); r >>= 1;
+        const int dw = (int)(r % bw); r /= bw;
+        const int dh = (int)(r % bh);
+        const int cpair = (int)(r / bh);
+        const int c = 2 * cpair + half;
+        float v = 0.0f;
+        if (m < O && c < C) {
+            const size_t idx = (((size_t)m * C + c) * bh + dh) * bw + dw;
+            const float w = weights[idx];
+            const float t = templates[idx] - ctr[c];
+            v = type == 0 ? -w : 2.0f * w * t;
+        }
+        pm[i] = v;
+    }
+}
+
+// bias[m] = -sum_k w (t - ctr)^2
+__global__ __launch_bounds__(256) void mfma_bias_kernel(const float *__restrict__ templates,
+                                                        const float *__restrict__ weights,
+                                                        const float *__restrict__ ctr, int O, int C, int bhw,
+                                                        float *__restrict__ bias)
+{
+    __shared__ float red[256];
+    const int m = blockIdx.x;
+    float s = 0.0f;
+    if (m < O) {
+        const int K = C * bhw;
+        for (int k = threadIdx.x; k < K; k += 256) {
+            const float t = templates[(size_t)m * K + k] - ctr[k / bhw];
+            s += weights[(size_t)m * K + k] * t * t;
+        }
+    }
+    red[threadIdx.x] = s;
+    __syncthreads();
+    for (int d = 128; d > 0; d >>= 1) {
+        if (threadIdx.x < d)
+            red[threadIdx.x] += red[threadIdx.x + d];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0)
+        bias[m] = -red[0];
+}
+
+struct MfmaTiling {
+    int Opad, steps, TC, TRmax, chan_lds, CC;
+    bool ok;
+    size_t pm_floats;
+};
+
+MfmaTiling mfma_tiling(const SimPlan &p)
+{
+    MfmaTiling t;
+    t.Opad = (p.O + WG_TPL - 1) / WG_TPL * WG_TPL;
+    t.steps = (p.C + 1) / 2 * p.bh * p.bw;
+    t.TC = (p.ow - 1) * p.sw + p.bw;
+    const int max_rows = std::min(p.oh, (WG_PIX + p.ow - 1) / p.ow + 1);
+    t.TRmax = (max_rows - 1) * p.sh + p.bh;
+    // channel pitch = 32 mod 64 floats: the two k-pair halves of a wave land in disjoint LDS banks
+    long long pitch = 1LL * t.TRmax * t.TC;
+    pitch = (pitch + 31) / 64 * 64 + 32;
+    if (pitch < 1LL * t.TRmax * t.TC)
+        pitch += 64;
+    t.ok = 2 * pitch <= kLdsBudgetFloats;
+    t.chan_lds = (int)pitch;
+    int cc_max = t.ok ? (int)(kLdsBudgetFloats / pitch) & ~1 : 2;
+    cc_max = std::min(cc_max, (p.C + 1) & ~1);
+    const int chunks = (p.C + cc_max - 1) / cc_max;
+    t.CC = ((p.C + chunks - 1) / chunks + 1) & ~1;
+    // two steps of slack: the parameter loads run two steps ahead
+    t.pm_floats = (size_t)(t.steps + 2) * 4 * t.Opad;
+    return t;
+}
+
+}  // namespace
+
+size_t sim_mfma_workspace_bytes(const SimPlan &p)
+{
+    const MfmaTiling t = mfma_tiling(p);
+    return align_up(t.pm_floats * sizeof(float), 256) + align_up((size_t)t.Opad * sizeof(float), 256) +
+           align_up((size_t)p.C * sizeof(float), 256);
+}
+
+int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
+                    void *workspace, size_t workspace_bytes, hipStream_t s)
+{
+    const MfmaTiling t = mfma_tiling(p);
+    if (!t.ok)
+        return SIMNETS_ERR_ALGO;  // image rows too long for the LDS tile of this path
+    if (workspace_bytes < sim_mfma_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+    char *ws = reinterpret_cast<char *>(workspace);
+    float *pm = reinterpret_cast<float *>(ws);
+    float *bias = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256));
+    float *ctr = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256) +
+                                           align_up((size_t)t.Opad * sizeof(float), 256));
+    const int bhw = p.bh * p.bw;
+    hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, bhw, ctr);
+    const long long total = (long long)t.pm_floats;
+    hipLaunchKernelGGL(mfma_pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 8192)), dim3(256), 0, s,
+                       templates, weights, ctr, p.O, t.Opad, p.C, p.bh, p.bw, total, pm);
+    hipLaunchKernelGGL(mfma_bias_kernel, dim3(t.Opad), dim3(256), 0, s, templates, weights, ctr, p.O, p.C, bhw, bias);
+    if (hipGetLastError() != hipSuccess)
+        return SIMNETS_ERR_HIP;
+
+    MfmaArgs a;
+    a.in = input; a.out = output; a.pm = pm; a.bias = bias; a.ctr = ctr;
+    a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.Opad = t.Opad;
+    a.oh = p.oh; a.ow = p.ow; a.npix = p.oh * p.ow;
+    a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
+    a.tiles = (a.npix + WG_PIX - 1) / WG_PIX;
+    a.TC = t.TC; a.TRmax = t.TRmax; a.chan_lds = t.chan_lds; a.CC = t.CC;
+    a.oob = p.oob;
+    dim3 grid((unsigned)(p.B * a.tiles), (unsigned)(t.Opad / WG_TPL));
+    const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
+    hipLaunchKernelGGL(sim_mfma_kernel, grid, dim3(kThreads), lds_bytes, s, a);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
 }  // namespace simnets

@@ -122,6 +122,31 @@ def test_similarity_sqrtw_algorithm_matches_direct(pkg):
     assert rel_err(run_similarity(pkg, x, t, w, algo="sqrtw", **kw), want) <= SIM_TOL
 
 
+@pytest.mark.parametrize("case", [
+    dict(shape=(2, 8, 20, 20), O=16, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),
+    dict(shape=(3, 5, 17, 13), O=70, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # odd C, ragged pixel tiles
+    dict(shape=(2, 4, 31, 29), O=130, blocks=[2, 3], strides=[2, 1], padding=[0, 2]),    # two template groups
+    dict(shape=(1, 3, 40, 40), O=5, blocks=[5, 5], strides=[2, 2], padding=[2, 2]),
+    dict(shape=(2, 1, 28, 28), O=32, blocks=[2, 2], strides=[2, 2], padding=[2, 2]),     # single channel
+])
+def test_similarity_mfma_algorithm_matches_direct(pkg, case):
+    x, t, w = sim_inputs(8, case["shape"], case["O"], case["blocks"])
+    x += 3.0  # a common offset, which the per-channel shift of the MFMA path must absorb
+    t += 3.0
+    kw = dict(blocks=case["blocks"], strides=case["strides"], padding=case["padding"], out_of_bounds_value=2.5)
+    want = orc.similarity_fwd(x, t, w, **kw)
+    assert rel_err(run_similarity(pkg, x, t, w, algo="mfma", **kw), want) <= SIM_TOL
+
+
+def test_config3_similarity_mfma_sampled(pkg):
+    x, t, w, kw = config3()
+    got = run_similarity(pkg, x, t, w, algo="mfma", **kw)
+    idx = [0, 101, 255]
+    assert rel_err(got[idx], orc.similarity_fwd(x[idx], t, w, **kw)) <= SIM_TOL
+    direct = run_similarity(pkg, x, t, w, algo="direct", **kw)
+    assert rel_err(got, direct) <= SIM_TOL
+
+
 # ---- BASELINE configurations ------------------------------------------------------------------------
 def test_config1_similarity_missing_data_layer(pkg):
     x, t, w, kw = config1(batch=64, nan_frac=0.25)
