@@ -1,0 +1,380 @@
+// Standalone C++ bench harness for libsimnets_hip.so.
+//
+//   simnets_bench --peaks                      machine micro-benchmarks (unpacked FP32 FMA issue rate,
+//                                              fp32 MFMA rate, v_exp_f32 rate, HBM copy bandwidth)
+//   simnets_bench --config N [--algo A] [--steps K] [--warmup W]
+//                                              N in 1..4: times that BASELINE configuration through the
+//                                              C ABI with hipEvents on its own stream
+// Prints one JSON object per measurement.  Inputs are synthetic (fixed-seed counter-based generator),
+// resident in HBM before timing starts.  Parity is not checked here (tests/ does that through the same
+// ABI); this binary links only the product library.
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <string>
+#include <vector>
+
+#include "simnets_hip.h"
+
+#define HIP_OK(x)                                                                                  \
+    do {                                                                                           \
+        hipError_t e_ = (x);                                                                       \
+        if (e_ != hipSuccess) {                                                                    \
+            fprintf(stderr, "HIP error %s at %s:%d\n", hipGetErrorString(e_), __FILE__, __LINE__); \
+            exit(1);                                                                               \
+        }                                                                                          \
+    } while (0)
+#define SN_OK(x)                                                                                 \
+    do {                                                                                         \
+        int r_ = (x);                                                                            \
+        if (r_ != 0) {                                                                           \
+            fprintf(stderr, "simnets error %d (%s) at %s:%d\n", r_, simnets_hip_strerror(r_), __FILE__, __LINE__); \
+            exit(1);                                                                             \
+        }                                                                                        \
+    } while (0)
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+// ---------------------------------------------------------------- micro-benchmarks
+__global__ __launch_bounds__(256) void fma_peak_kernel(float *out, float a, float b, int iters)
+{
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = (float)(threadIdx.x + i);
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 16; ++i)
+                acc[i] = __builtin_fmaf(acc[i], a, b);
+    }
+    float s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        s += acc[i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void mfma_peak_kernel(float *out, float a, float b, int iters)
+{
+    floatx16 acc[4];
+    for (int i = 0; i < 4; ++i)
+        for (int v = 0; v < 16; ++v)
+            acc[i][v] = (float)v;
+    float av = a + threadIdx.x, bv = b;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                acc[i] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc[i], 0, 0, 0);
+    }
+    float s = 0;
+    for (int i = 0; i < 4; ++i)
+        for (int v = 0; v < 16; ++v)
+            s += acc[i][v];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void exp_peak_kernel(float *out, float a, int iters)
+{
+    float acc[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        acc[i] = -(float)(threadIdx.x + i) * a;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i)
+            acc[i] = __builtin_amdgcn_exp2f(acc[i]);
+    }
+    float s = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i)
+        s += acc[i];
+    out[blockIdx.x * blockDim.x + threadIdx.x] = s;
+}
+
+__global__ __launch_bounds__(256) void copy_kernel(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+static float time_ms(hipStream_t s, int reps, const std::function<void()> &fn);
+
+#include <functional>
+static float time_ms(hipStream_t s, int reps, const std::function<void()> &fn)
+{
+    hipEvent_t e0, e1;
+    HIP_OK(hipEventCreate(&e0));
+    HIP_OK(hipEventCreate(&e1));
+    fn();
+    HIP_OK(hipStreamSynchronize(s));
+    HIP_OK(hipEventRecord(e0, s));
+    for (int i = 0; i < reps; ++i)
+        fn();
+    HIP_OK(hipEventRecord(e1, s));
+    HIP_OK(hipEventSynchronize(e1));
+    float ms = 0;
+    HIP_OK(hipEventElapsedTime(&ms, e0, e1));
+    HIP_OK(hipEventDestroy(e0));
+    HIP_OK(hipEventDestroy(e1));
+    return ms / reps;
+}
+
+static void run_peaks(hipStream_t s)
+{
+    hipDeviceProp_t prop;
+    HIP_OK(hipGetDeviceProperties(&prop, 0));
+    const int cus = prop.multiProcessorCount;
+    const int blocks = cus * 8;  // 8 workgroups of 4 waves per CU: 8 waves per SIMD
+    float *out;
+    HIP_OK(hipMalloc(&out, (size_t)blocks * 256 * sizeof(float)));
+    {
+        const int iters = 4096;
+        float ms = time_ms(s, 5, [&] { hipLaunchKernelGGL(fma_peak_kernel, dim3(blocks), dim3(256), 0, s, out, 1.0001f, 0.5f, iters); });
+        const double fma = (double)blocks * 256 * iters * 64.0;
+        printf("{\"peak\": \"valu_fma_f32_unpacked\", \"lane_fma_per_s_T\": %.3f, \"tflops\": %.2f, \"implied_clock_ghz\": %.3f, "
+               "\"cus\": %d, \"ms\": %.4f}\n",
+               fma / (ms * 1e-3) / 1e12, 2 * fma / (ms * 1e-3) / 1e12, fma / (ms * 1e-3) / (cus * 64.0) / 1e9, cus, ms);
+    }
+    {
+        const int iters = 2048;
+        float ms = time_ms(s, 5, [&] { hipLaunchKernelGGL(mfma_peak_kernel, dim3(cus * 2), dim3(256), 0, s, out, 1.0f, 0.5f, iters); });
+        const double mfma = (double)cus * 2 * 4 * iters * 16.0;  // wave-level MFMA instructions
+        const double flop = mfma * 4096.0;
+        printf("{\"peak\": \"mfma_f32_32x32x2\", \"tflops\": %.2f, \"implied_clock_ghz\": %.3f, \"ms\": %.4f}\n",
+               flop / (ms * 1e-3) / 1e12, mfma * 64.0 / (ms * 1e-3) / (cus * 4.0) / 1e9, ms);
+    }
+    {
+        const int iters = 4096;
+        float ms = time_ms(s, 5, [&] { hipLaunchKernelGGL(exp_peak_kernel, dim3(blocks), dim3(256), 0, s, out, 1e-3f, iters); });
+        const double n = (double)blocks * 256 * iters * 16.0;
+        printf("{\"peak\": \"v_exp_f32\", \"exp_per_s_T\": %.3f, \"ms\": %.4f}\n", n / (ms * 1e-3) / 1e12, ms);
+    }
+    {
+        const size_t bytes = (size_t)1 << 30;
+        float4 *a, *b;
+        HIP_OK(hipMalloc(&a, bytes));
+        HIP_OK(hipMalloc(&b, bytes));
+        HIP_OK(hipMemsetAsync(a, 1, bytes, s));
+        float ms = time_ms(s, 5, [&] { hipLaunchKernelGGL(copy_kernel, dim3(cus * 16), dim3(256), 0, s, a, b, bytes / 16); });
+        printf("{\"peak\": \"hbm_copy\", \"GBps_read_plus_write\": %.1f, \"ms\": %.4f}\n", 2.0 * bytes / (ms * 1e-3) / 1e9, ms);
+        HIP_OK(hipFree(a));
+        HIP_OK(hipFree(b));
+    }
+    HIP_OK(hipFree(out));
+}
+
+// ---------------------------------------------------------------- synthetic inputs
+static inline uint64_t mix64(uint64_t z)
+{
+    z += 0x9e3779b97f4a7c15ULL;
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ULL;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebULL;
+    return z ^ (z >> 31);
+}
+static inline float uniform01(uint64_t seed, uint64_t i) { return (float)((mix64(seed * 0x100000001b3ULL + i) >> 40) * (1.0 / 16777216.0)); }
+static void fill_uniform(std::vector<float> &v, uint64_t seed, float lo, float hi)
+{
+    for (size_t i = 0; i < v.size(); ++i)
+        v[i] = lo + (hi - lo) * uniform01(seed, i);
+}
+static void fill_normal(std::vector<float> &v, uint64_t seed, float sigma)
+{
+    for (size_t i = 0; i < v.size(); ++i) {
+        const float u1 = std::max(uniform01(seed, 2 * i), 1e-7f), u2 = uniform01(seed, 2 * i + 1);
+        v[i] = sigma * std::sqrt(-2.0f * std::log(u1)) * std::cos(6.2831853f * u2);
+    }
+}
+static float *upload(const std::vector<float> &v)
+{
+    float *d;
+    HIP_OK(hipMalloc(&d, std::max<size_t>(v.size(), 1) * sizeof(float)));
+    HIP_OK(hipMemcpy(d, v.data(), v.size() * sizeof(float), hipMemcpyHostToDevice));
+    return d;
+}
+
+struct SimCase {
+    simnets_similarity_attrs a;
+    int in[4], tp[4], out[4];
+    float *x, *t, *w, *y;
+    void *ws;
+    size_t ws_bytes;
+};
+
+static SimCase make_similarity(int B, int C, int H, int W, int O, int bh, int bw, int s, int p, bool missing, int algo, int l1)
+{
+    SimCase c;
+    simnets_similarity_attrs_default(&c.a);
+    c.a.blocks[0] = bh; c.a.blocks[1] = bw;
+    c.a.strides[0] = c.a.strides[1] = s;
+    c.a.padding[0] = c.a.padding[1] = p;
+    c.a.algo = algo;
+    c.a.similarity_function = l1 ? SIMNETS_SIM_L1 : SIMNETS_SIM_L2;
+    if (missing) {
+        c.a.normalization_term = 1;
+        c.a.ignore_nan_input = 1;
+        c.a.out_of_bounds_value = NAN;
+    }
+    const int in[4] = {B, C, H, W}, tp[4] = {O, C, bh, bw};
+    memcpy(c.in, in, sizeof(in));
+    memcpy(c.tp, tp, sizeof(tp));
+    SN_OK(simnets_similarity_out_shape(&c.a, c.in, c.tp, c.tp, c.out));
+    std::vector<float> x((size_t)B * C * H * W), t((size_t)O * C * bh * bw), w(t.size());
+    if (missing) {
+        fill_uniform(x, 1234, -0.5f, 0.5f);
+        fill_normal(t, 2345, 0.1f);
+        fill_uniform(w, 3456, 0.5f, 1.5f);
+    } else {
+        fill_normal(x, 1234, 1.0f);
+        fill_normal(t, 2345, 1.0f);
+        fill_uniform(w, 3456, 0.1f, 2.0f);
+    }
+    c.x = upload(x); c.t = upload(t); c.w = upload(w);
+    HIP_OK(hipMalloc(&c.y, (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3] * sizeof(float)));
+    SN_OK(simnets_hip_similarity_workspace_bytes(&c.a, c.in, c.tp, &c.ws_bytes));
+    HIP_OK(hipMalloc(&c.ws, std::max<size_t>(c.ws_bytes, 256)));
+    return c;
+}
+
+struct MexCase {
+    simnets_mex_attrs a;
+    int in[4], out[4], off[5];
+    float *x, *o, *y;
+    void *ws;
+    size_t ws_bytes, off_count;
+};
+
+static MexCase make_mex(int B, int C, int HW, int M, bool shared1, const float *input)
+{
+    MexCase c;
+    simnets_mex_attrs_default(&c.a);
+    c.a.num_instances = M;
+    c.a.softmax_mode = 1;
+    c.a.blocks[0] = C; c.a.strides[0] = C;
+    c.a.normalize_offsets = 1;
+    if (shared1) {
+        c.a.shared_offset_region[0] = 1;
+    } else {
+        c.a.unshared_offset_region[0] = 2;
+    }
+    const int in[4] = {B, C, HW, HW};
+    memcpy(c.in, in, sizeof(in));
+    SN_OK(simnets_mex_out_shape(&c.a, c.in, c.out, c.off));
+    c.off_count = (size_t)c.off[0] * c.off[1] * c.off[2] * c.off[3] * c.off[4];
+    std::vector<float> off(c.off_count);
+    fill_normal(off, 4567 + C, 0.1f);
+    c.o = upload(off);
+    if (input) {
+        c.x = const_cast<float *>(input);
+    } else {
+        std::vector<float> x((size_t)B * C * HW * HW);
+        fill_normal(x, 1234, 1.0f);
+        c.x = upload(x);
+    }
+    HIP_OK(hipMalloc(&c.y, (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3] * sizeof(float)));
+    SN_OK(simnets_hip_mex_workspace_bytes(&c.a, c.in, &c.ws_bytes));
+    HIP_OK(hipMalloc(&c.ws, std::max<size_t>(c.ws_bytes, 256)));
+    return c;
+}
+
+static void run_sim(SimCase &c, hipStream_t s)
+{
+    SN_OK(simnets_hip_similarity_fwd(&c.a, c.in, c.tp, c.tp, c.x, c.t, c.w, c.y, c.ws, c.ws_bytes, s));
+}
+static void run_mex(MexCase &c, hipStream_t s)
+{
+    SN_OK(simnets_hip_mex_fwd(&c.a, c.in, c.x, c.o, c.off_count, c.y, c.ws, c.ws_bytes, s));
+}
+
+static void report(const char *name, double gmac, double bytes, double flop_per_gmac, float ms, int steps)
+{
+    const double gmacs = gmac / (ms * 1e-3);
+    printf("{\"config\": \"%s\", \"ms\": %.4f, \"steps\": %d, \"gmac_per_s_G\": %.1f, \"tflops\": %.2f, "
+           "\"frac_fp32_peak_157.3\": %.4f, \"hbm_frac_8TBs\": %.4f}\n",
+           name, ms, steps, gmacs / 1e9, gmacs * flop_per_gmac / 1e12, gmacs * flop_per_gmac / 157.3e12,
+           bytes / (ms * 1e-3) / 8e12);
+}
+
+int main(int argc, char **argv)
+{
+    int config = 0, steps = 20, warmup = 5, algo = SIMNETS_ALGO_AUTO;
+    bool peaks = false;
+    for (int i = 1; i < argc; ++i) {
+        std::string a = argv[i];
+        if (a == "--peaks") peaks = true;
+        else if (a == "--config" && i + 1 < argc) config = atoi(argv[++i]);
+        else if (a == "--steps" && i + 1 < argc) steps = atoi(argv[++i]);
+        else if (a == "--warmup" && i + 1 < argc) warmup = atoi(argv[++i]);
+        else if (a == "--algo" && i + 1 < argc) {
+            std::string v = argv[++i];
+            algo = v == "direct" ? SIMNETS_ALGO_DIRECT : v == "sqrtw" ? SIMNETS_ALGO_SQRTW : v == "mfma" ? SIMNETS_ALGO_MFMA : SIMNETS_ALGO_AUTO;
+        } else {
+            fprintf(stderr, "usage: %s --peaks | --config N [--algo direct|sqrtw|mfma] [--steps K] [--warmup W]\n", argv[0]);
+            return 2;
+        }
+    }
+    hipStream_t s;
+    HIP_OK(hipStreamCreate(&s));
+    if (peaks)
+        run_peaks(s);
+    if (config == 1) {
+        SimCase c = make_similarity(64, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
+        for (int i = 0; i < warmup; ++i) run_sim(c, s);
+        float ms = time_ms(s, steps, [&] { run_sim(c, s); });
+        report("config1 similarity L2 norm ignore-nan 64x1x28x28 -> 64x32x16x16", 2097152.0, 2298880.0, 6, ms, steps);
+    } else if (config == 2) {
+        MexCase c = make_mex(64, 32, 16, 64, false, nullptr);
+        for (int i = 0; i < warmup; ++i) run_mex(c, s);
+        float ms = time_ms(s, steps, [&] { run_mex(c, s); });
+        report("config2 mex 64x32x16x16 -> 64x64x16x16", 33554432.0, 6324224.0, 5, ms, steps);
+    } else if (config == 3) {
+        for (int l1 = 0; l1 < 2; ++l1) {
+            if (l1 && algo != SIMNETS_ALGO_AUTO && algo != SIMNETS_ALGO_DIRECT)
+                break;
+            SimCase c = make_similarity(256, 64, 32, 32, 128, 3, 3, 1, 1, false, algo, l1);
+            for (int i = 0; i < warmup; ++i) run_sim(c, s);
+            float ms = time_ms(s, steps, [&] { run_sim(c, s); });
+            report(l1 ? "config3 similarity L1 256x64x32x32 x 128 templates 3x3" : "config3 similarity L2 256x64x32x32 x 128 templates 3x3",
+                   19327352832.0, 201916416.0, l1 ? 3 : 4, ms, steps);
+        }
+    } else if (config == 4) {
+        const int B = 512;
+        SimCase sc = make_similarity(B, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
+        std::vector<MexCase> mex;
+        std::vector<float *> pooled;
+        const float *cur = sc.y;
+        int ch = 32, hw = 16;
+        for (int l = 0; l < 4; ++l) {
+            mex.push_back(make_mex(B, ch, hw, 2 * ch, false, cur));
+            float *p;
+            HIP_OK(hipMalloc(&p, (size_t)B * 2 * ch * (hw / 2) * (hw / 2) * sizeof(float)));
+            pooled.push_back(p);
+            cur = p;
+            ch *= 2;
+            hw /= 2;
+        }
+        mex.push_back(make_mex(B, ch, 1, 10, true, cur));
+        auto stack = [&] {
+            run_sim(sc, s);
+            for (int l = 0; l < 4; ++l) {
+                run_mex(mex[l], s);
+                SN_OK(simnets_hip_sum_pool_fwd(mex[l].out, 2, 2, mex[l].y, pooled[l], s));
+            }
+            run_mex(mex[4], s);
+        };
+        for (int i = 0; i < warmup; ++i) stack();
+        float ms = time_ms(s, steps, stack);
+        report("config4 missing-data stack batch 512", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+    }
+    HIP_OK(hipStreamSynchronize(s));
+    HIP_OK(hipStreamDestroy(s));
+    return 0;
+}

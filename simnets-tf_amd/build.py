@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsimnets_hip.so")
+BENCH = os.path.join(HERE, "simnets_bench")
 OBJDIR = os.path.join(HERE, "build")
 
 SOURCES = ["host_logic.cpp", "capi.hip", "similarity_direct.hip", "similarity_mfma.hip", "mex.hip"]
@@ -40,8 +41,12 @@ def build(extra=(), verbose=False):
     with ThreadPoolExecutor(max_workers=min(len(SOURCES), 6)) as ex:
         objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
     subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs, check=True)
+    # standalone C++ harness, linked against the product library only
+    bench_src = os.path.join(HERE, "bench", "simnets_bench.hip")
+    subprocess.run([HIPCC, bench_src, "-o", BENCH] + COMMON + DEVICE + extra +
+                   ["-L" + HERE, "-lsimnets_hip", "-Wl,-rpath,$ORIGIN"], check=True)
     if verbose:
-        print("built", LIB)
+        print("built", LIB, "and", BENCH)
     return LIB
 
 

@@ -57,10 +57,35 @@ struct SimKernelArgs {
     int vec_store;     // output rows are 16-byte aligned: store float4
 };
 
+// Wave-uniform parameter fetch: the address is the same in every lane, so these become scalar loads
+// (s_load_dwordx8/x16) and the values live in SGPRs.
+template <int MODE, int MT>
+__device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT], const float SIMNETS_CONST_AS *ppa,
+                                            const float SIMNETS_CONST_AS *ppc)
+{
+#pragma unroll
+    for (int i = 0; i < 2 * MT; ++i)
+        pa[i] = ppa[i];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+        pc[i] = (MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN) ? ppc[i] : 0.0f;
+}
+
+// Copies a wave-uniform value from its SGPR into a VGPR.  VALU instructions that read an SGPR
+// operand issue at half the rate of all-VGPR ones on this chip (measured: 37 vs 64 T lane-ops/s), so
+// each parameter is moved once per (template, k) and then used from the VGPR by all PT pixels.  The
+// asm keeps the compiler from folding the SGPR back into the arithmetic.
+__device__ __forceinline__ float to_vgpr(float uniform)
+{
+    float v;
+    asm("v_mov_b32 %0, %1" : "=v"(v) : "s"(uniform));
+    return v;
+}
+
 // One k step for all MT templates and PT pixels of a lane.
 template <int MODE, int PT, int MT>
-__device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[PT],
-                                         const float SIMNETS_CONST_AS *pa, const float SIMNETS_CONST_AS *pc)
+__device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[PT], const float (&pa)[2 * MT],
+                                         const float (&pc)[MT])
 {
     if (MODE == SIM_MODE_L2_NORM_IGNORE_NAN) {
         float keep[PT], xz[PT];
@@ -72,7 +97,7 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
         }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const float t = pa[2 * m], nwh = pa[2 * m + 1], c = pc[m];
+            const float t = to_vgpr(pa[2 * m]), nwh = to_vgpr(pa[2 * m + 1]), c = to_vgpr(pc[m]);
 #pragma unroll
             for (int p = 0; p < PT; ++p) {
                 const float d = t - xz[p];
@@ -83,30 +108,61 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
     } else {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const float t = pa[2 * m], nw = pa[2 * m + 1];
+            const float t = to_vgpr(pa[2 * m]), nw = to_vgpr(pa[2 * m + 1]);
             float c = 0.0f;
             if (MODE == SIM_MODE_L2_NORM)
-                c = pc[m];
+                c = to_vgpr(pc[m]);
+            // The combine is a chain of dependent instructions per pixel; a dependent VALU instruction
+            // issued right behind its producer stalls, so the chain is laid out stage by stage across
+            // the PT pixels (PT independent instructions between producer and consumer).
+            float d[PT], q[PT];
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                d[p] = (MODE == SIM_MODE_L2_SQRTW) ? __builtin_fmaf(nw, x[p], t) : t - x[p];
+            __builtin_amdgcn_sched_barrier(0);
+            if (MODE == SIM_MODE_L2 || MODE == SIM_MODE_L2_NORM) {
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    q[p] = nw * d[p];
+                __builtin_amdgcn_sched_barrier(0);
+            }
 #pragma unroll
             for (int p = 0; p < PT; ++p) {
-                const float d = t - x[p];
-                if (MODE == SIM_MODE_L2_SQRTW) {
-                    // pa holds (sqrt(w)*t, -sqrt(w)): d = sqrt(w)*(t - x) in one fma, acc -= d*d
-                    const float ds = __builtin_fmaf(nw, x[p], t);
-                    acc[m][p] = __builtin_fmaf(-ds, ds, acc[m][p]);
-                } else if (MODE == SIM_MODE_L1)
-                    acc[m][p] = __builtin_fmaf(nw, __builtin_fabsf(d), acc[m][p]);
+                if (MODE == SIM_MODE_L2_SQRTW)
+                    acc[m][p] = __builtin_fmaf(-d[p], d[p], acc[m][p]);  // (sqrt(w)*t, -sqrt(w)) in pa
+                else if (MODE == SIM_MODE_L1)
+                    acc[m][p] = __builtin_fmaf(nw, __builtin_fabsf(d[p]), acc[m][p]);
                 else if (MODE == SIM_MODE_L2)
-                    acc[m][p] = __builtin_fmaf(nw * d, d, acc[m][p]);
+                    acc[m][p] = __builtin_fmaf(q[p], d[p], acc[m][p]);
                 else
-                    acc[m][p] += __builtin_fmaf(nw * d, d, c);
+                    q[p] = __builtin_fmaf(q[p], d[p], c);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (MODE == SIM_MODE_L2_NORM) {
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    acc[m][p] += q[p];
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
 }
 
+// Lane tile of the wide-image variant, and of the narrow one.
+#ifndef SIMNETS_BIG_PT
+#define SIMNETS_BIG_PT 16
+#endif
+#ifndef SIMNETS_BIG_MT
+#define SIMNETS_BIG_MT 8
+#endif
+constexpr int kBigPT = SIMNETS_BIG_PT, kBigMT = SIMNETS_BIG_MT;
+constexpr int kSmallPT = 4, kSmallMT = 8;
+// waves per SIMD the register budget is sized for: 64 accumulators leave room for 4, 128 for 2
+constexpr int waves_per_simd(int pt, int mt) { return pt * mt <= 64 ? 4 : 2; }
+constexpr int lds_budget_floats(int pt, int mt) { return pt * mt <= 64 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
+
 template <int MODE, int PT, int MT, int SWT>
-__global__ __launch_bounds__(kThreads, 2) void sim_direct_kernel(const SimKernelArgs a)
+__global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
 {
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
@@ -150,6 +206,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_direct_kernel(const SimKernel
         (const float SIMNETS_CONST_AS *)(a.pc) + (size_t)(wave_active ? mtile : 0) * a.K * MT;
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
     const int chan_lds = TR * a.TC;
+    float pa0[2 * MT], pc0[MT], pa1[2 * MT], pc1[MT];
+    load_params<MODE, MT>(pa0, pc0, pa, pc);
 
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
@@ -160,20 +218,54 @@ __global__ __launch_bounds__(kThreads, 2) void sim_direct_kernel(const SimKernel
         __syncthreads();
         if (!wave_active)
             continue;
-        // ---- accumulate over the k of these channels, in k order ----
-        for (int cc = 0; cc < ccn; ++cc) {
-            for (int dh = 0; dh < a.bh; ++dh) {
-                const float *xrow = lds + lds_base + cc * chan_lds + dh * a.TC;
-                for (int dw = 0; dw < a.bw; ++dw) {
-                    float x[PT];
+        // ---- accumulate over the k of these channels, in k order.  Software pipeline: the pixel
+        //      values and the parameters of step k+1 are requested before the arithmetic of step k,
+        //      ping-ponging between two register sets (no copies) ----
+        const int nk = ccn * a.bh * a.bw;
+        int dh = 0, dw = 0, row_off = 0, off = 0;
+        auto step = [&](const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT], float (&xnx)[PT],
+                        float (&panx)[2 * MT], float (&pcnx)[MT], bool last) {
+            // LDS and scalar loads share one counter and scalar loads return out of order, so a wait
+            // for LDS data after a new scalar load was issued would also wait for that load.  Drain
+            // the counter here, where everything outstanding was issued a whole step ago, and only
+            // then issue the requests for the next step: the arithmetic below needs no further wait.
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+            __builtin_amdgcn_sched_barrier(0);
+            // next tap, branch-free (selects on wave-uniform values keep the step one basic block)
+            const bool wrap_w = dw + 1 == a.bw;
+            const int ndw = wrap_w ? 0 : dw + 1;
+            const bool wrap_h = wrap_w && dh + 1 == a.bh;
+            const int ndh = wrap_h ? 0 : dh + (wrap_w ? 1 : 0);
+            const int nrow = row_off + (wrap_w ? a.TC : 0) + (wrap_h ? chan_lds - a.bh * a.TC : 0);
+            const int noff = last ? off : nrow + ndw;  // nothing is staged beyond this chunk
 #pragma unroll
-                    for (int p = 0; p < PT; ++p)
-                        x[p] = xrow[dw + p * sw];
-                    sim_step<MODE, PT, MT>(acc, x, pa, pc);
-                    pa += 2 * MT;
-                    pc += MT;
-                }
-            }
+            for (int p = 0; p < PT; ++p)
+                xnx[p] = lds[lds_base + noff + p * sw];
+            pa += 2 * MT;
+            pc += MT;
+            load_params<MODE, MT>(panx, pcnx, pa, pc);  // one k of slack exists behind the arrays
+            __builtin_amdgcn_sched_barrier(0);
+            sim_step<MODE, PT, MT>(acc, xc, pac, pcc);
+            __builtin_amdgcn_sched_barrier(0);
+            dw = ndw; dh = ndh; row_off = nrow; off = noff;
+        };
+        float x0[PT], x1[PT];
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            x0[p] = lds[lds_base + p * sw];
+        int kk = 0;
+        for (; kk + 2 <= nk; kk += 2) {
+            step(x0, pa0, pc0, x1, pa1, pc1, false);
+            step(x1, pa1, pc1, x0, pa0, pc0, kk + 2 == nk);
+        }
+        if (kk < nk) {
+            step(x0, pa0, pc0, x1, pa1, pc1, true);
+#pragma unroll
+            for (int i = 0; i < 2 * MT; ++i)
+                pa0[i] = pa1[i];
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                pc0[i] = pc1[i];
         }
     }
 
@@ -245,7 +337,9 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
                 float x[1] = {a.oob};
                 if (ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
                     x[0] = img[((size_t)c * a.H + ih) * a.W + iw];
-                sim_step<MODE, 1, MT>(acc, x, pa, pc);
+                float pav[2 * MT], pcv[MT];
+                load_params<MODE, MT>(pav, pcv, pa, pc);
+                sim_step<MODE, 1, MT>(acc, x, pav, pcv);
                 pa += 2 * MT;
                 pc += MT;
             }
@@ -312,11 +406,13 @@ struct Tiling {
 Tiling choose_tiling(const SimPlan &p)
 {
     Tiling t;
-    // Wide rows and many templates: 8 pixels x 16 templates per lane.  Otherwise 4 x 8, which
+    // Wide rows and many templates: 16 pixels x 8 templates per lane (one s_load_dwordx16 per k, so
+    // two parameter sets fit the SGPR file and the next k can be in flight).  Otherwise 4 x 8, which
     // keeps narrow images and small template counts from idling lanes and waves.
     const bool big = p.ow >= 32 && p.O >= 32;
-    t.PT = big ? 8 : 4;
-    t.MT = big ? 16 : 8;
+    t.PT = big ? kBigPT : kSmallPT;
+    t.MT = big ? kBigMT : kSmallMT;
+    const int budget = lds_budget_floats(t.PT, t.MT);
     t.G = (p.ow + t.PT - 1) / t.PT;
     t.gpi = p.oh * t.G;
     const int n_mtiles = (p.O + t.MT - 1) / t.MT;
@@ -332,10 +428,10 @@ Tiling choose_tiling(const SimPlan &p)
     const int max_rows = std::min(p.oh, (64 * t.nws + t.G - 1) / t.G + 1);
     t.TRmax = (max_rows - 1) * p.sh + p.bh;
     const long long per_chan = 1LL * t.TRmax * t.TC;
-    t.lds_ok = per_chan <= kLdsBudgetFloats;
+    t.lds_ok = per_chan <= budget;
     t.CC = 1;
     if (t.lds_ok) {
-        const int cc_max = (int)std::min<long long>(p.C, kLdsBudgetFloats / per_chan);
+        const int cc_max = (int)std::min<long long>(p.C, budget / per_chan);
         const int chunks = (p.C + cc_max - 1) / cc_max;
         t.CC = (p.C + chunks - 1) / chunks;
     }
@@ -360,7 +456,9 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
     if (!t.lds_ok) {
         const long long npix = (long long)a.B * a.oh * a.ow;
         dim3 grid((unsigned)((npix + 255) / 256), (unsigned)a.n_mtiles);
-        if (t.MT == 16)
+        if (t.MT == 4)
+            hipLaunchKernelGGL((sim_gather_kernel<MODE, 4>), grid, dim3(256), 0, s, a);
+        else if (t.MT == 16)
             hipLaunchKernelGGL((sim_gather_kernel<MODE, 16>), grid, dim3(256), 0, s, a);
         else
             hipLaunchKernelGGL((sim_gather_kernel<MODE, 8>), grid, dim3(256), 0, s, a);
@@ -369,9 +467,9 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
     const int nwm = kWaves / a.nws;
     dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
     const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
-    if (t.PT == 8)
-        return launch_direct<MODE, 8, 16>(a, grid, lds_bytes, s);
-    return launch_direct<MODE, 4, 8>(a, grid, lds_bytes, s);
+    if (t.PT == kBigPT && t.MT == kBigMT)
+        return launch_direct<MODE, kBigPT, kBigMT>(a, grid, lds_bytes, s);
+    return launch_direct<MODE, kSmallPT, kSmallMT>(a, grid, lds_bytes, s);
 }
 
 }  // namespace
