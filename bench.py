@@ -21,9 +21,14 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
-PEAK_FP32_TFLOPS = 157.3   # MI355X published FP32 vector / FP32 matrix peak
+PEAK_FP32_TFLOPS = 157.3   # MI355X published FP32 vector / FP32 matrix peak (256 CU x 128 FMA lanes x 2.4 GHz x 2)
 PEAK_HBM_GBS = 8000.0
-EXP_RATE = 9.83e12         # 256 CU x 16 transcendental lanes x 2.4 GHz
+EXP_RATE = 19.66e12        # v_exp_f32 at a quarter of the 128 lanes/clk/CU VALU rate (17.6e12 measured on the box)
+
+# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
+# same workload scaled by a copy kernel of known size (profiles/sim_direct_l2_config3.md).
+# Keyed by evaluation path; None where no counter run exists for the current kernel.
+MEASURED_TRAFFIC_BYTES = {"direct": 286.8e6}
 
 
 def main():
@@ -112,7 +117,8 @@ def main():
                    "algo": args.algo or "direct", "gmac_per_step": gmac3},
         "roofline": {"bound": "mfma" if args.algo == "mfma" else "valu",
                      "achieved": round(achieved_tflops, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved_tflops / PEAK_FP32_TFLOPS, 4), "traffic": None,
+                     "frac": round(achieved_tflops / PEAK_FP32_TFLOPS, 4),
+                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.algo or "direct"),
                      "kernel_ms": round(ev_ms, 4), "flop_per_gmac": flop_per_gmac,
                      "algorithmic_bytes": bytes3,
                      "hbm_frac": round(bytes3 / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
@@ -127,7 +133,9 @@ def main():
             if flop:
                 e["valu_frac"] = round(gmac / (ms * 1e-3) * flop / 1e12 / PEAK_FP32_TFLOPS, 4)
             if exp_bound:
+                # MEX: 1 exp + 5 flop per gMAC
                 e["exp_frac"] = round(gmac / (ms * 1e-3) / EXP_RATE, 4)
+                e["valu_frac"] = round(gmac / (ms * 1e-3) * 5 / 1e12 / PEAK_FP32_TFLOPS, 4)
             return e
 
         _, ms = timed(sim3("L1", None), args.steps, args.warmup)
@@ -176,7 +184,8 @@ def main():
         _, ms = timed(stack, args.steps, args.warmup)
         gmac4 = 512 * 32 * 256 * 4 + 4 * 268435456 + 512 * 10 * 512
         others["config4_stack"] = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(gmac4 / (ms * 1e-3) / 1e9, 1),
-                                   "batch": 512}
+                                   "exp_frac": round(gmac4 / (ms * 1e-3) / EXP_RATE, 4), "batch": 512,
+                                   "kernels": "similarity + 5 x (offset pack + mex) + 4 x sum pool"}
     result["others"] = others
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)

@@ -9,69 +9,75 @@
 // Work split
 //   * output pixels are enumerated region-major: slot s of region r is image s / region_size,
 //     position s % region_size inside the region (the order split_patches lays them out in,
-//     include/utils/mex_utils.hpp:69-116).  A wave takes 64 consecutive slots of ONE region, so
-//     the offsets it needs, offsets[r, m, k], are the same for all its lanes and are read with
-//     scalar loads into SGPRs; nothing is regrouped in memory, each lane maps its slot straight
-//     to the (c, h, w) it belongs to for either region flavour (contiguous "shared" tiles or
-//     interleaved "unshared" ones).
-//   * a lane gathers its patch element k from the input with the im2col_3d index rule (out of
-//     image -> blocks_out_of_bounds_value) and combines it with MTX instances at once;
-//   * two sweeps over k like the reference (max, then exp-sum relative to the max), with the
-//     2*MTX running values in VGPRs; exp is v_exp_f32 on a pre-scaled argument.
-//   The four waves of a workgroup share the pixels and split the instances, so the second to
-//   fourth gather of an element hit L1.
+//     include/utils/mex_utils.hpp:69-116).  A workgroup takes 64*PX consecutive slots of ONE region,
+//     so the offsets it needs, offsets[r, m, k], do not depend on the pixel; nothing is regrouped in
+//     memory, each thread maps its slot straight to the (c, h, w) it belongs to for either region
+//     flavour (contiguous "shared" tiles or interleaved "unshared" ones).
+//   * K is walked in chunks of KC: the workgroup gathers the patch elements of its pixels with the
+//     im2col_3d index rule (out of image -> blocks_out_of_bounds_value) into LDS, [k][pixel], and
+//     copies the matching offsets, pre-packed [k][instance], next to them.
+//   * a lane owns PX pixels (slots lane, lane+64, ...) and its wave 16 instances: per k it reads its
+//     PX pixel values (lane-distinct) and 16 offsets (one address for the whole wave: an LDS
+//     broadcast, so the operand arrives in VGPRs; VALU instructions with SGPR operands issue at half
+//     rate on this chip) and updates PX*16 running values held in VGPRs.
+//   * the 4 waves of a workgroup split the instances (WM ways) and, when the grid would otherwise
+//     leave SIMDs idle, K (KS ways, WM*KS = 4): each K-split wave keeps its own (max, sum) pair and
+//     the pairs are merged through LDS at the end: sum = sum_i s_i * exp(eps*(m_i - max_i m_i)).
+//   * two sweeps over K like the reference (max, then sum of exp relative to the max); exp is
+//     v_exp_f32 on a pre-scaled argument.  When K fits one chunk the second sweep reuses the LDS tile.
+//   * workgroups that own the different regions of the same pixel chunk are numbered a multiple of
+//     8 apart, so they run on the same XCD and their interleaved partial cache lines meet in one L2.
 #include <hip/hip_runtime.h>
 
+#include <algorithm>
 #include <cmath>
 
 #include "internal.h"
 
 namespace simnets {
 
-#define SIMNETS_CONST_AS __attribute__((address_space(4)))
-
 namespace {
 
-constexpr int MTX = 16;  // instances per wave
+constexpr int MX = 16;        // instances per wave
+constexpr int KC = 32;        // k per LDS chunk
+constexpr int kXcds = 8;
 
 struct MexKernelArgs {
     const float *in;
     float *out;
-    const float *offp;  // [R][mtile][K][MTX]
+    const float *offp;  // [R][mgroup][K][TM]
     int B, C, H, W;
     int Co, Ho, Wo;
     int bc, bh, bw, sc, sh, sw, pc, ph, pw;
     int Cg, Hg, Wg;     // offsets_c/h/w: number of regions along each axis
     int Cs, Hs, Ws;     // shared_region_c/h/w: extent of a region along each axis
     int unshared;
+    int R;              // num_regions
     int RS;             // region_size
     int slots;          // B * RS
-    int cpr;            // 64-slot chunks per region
-    int M, K, n_mtiles;
+    int cpr;            // pixel chunks (64*PX slots) per region
+    int M, K, n_mgroups;
     float c1;           // eps * log2(e)
     float c0;           // (softmax ? 0 : -log K) * log2(e)
-    float eps;
+    float ln2_over_eps; // log(2) / eps
     int finite_eps;
     float oob;
 };
 
-template <bool NEG, bool CHECK>
-__global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
-{
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int mtile = blockIdx.y * 4 + wave;
-    if (mtile >= a.n_mtiles)
-        return;
-    const int r = blockIdx.x / a.cpr;
-    const int chunk = blockIdx.x - r * a.cpr;
+struct PixelRef {
+    const float *base;  // &input[b][c*sc-pc][h*sh-ph][w*sw-pw] (only dereferenced inside the image)
+    int ci0, hi0, wi0;
+    int out_off;        // offset of out[b][c][h][w] within image b's output, -1 if the slot is empty
+    int b;
+};
 
-    // region coordinates: r = (c_g * Hg + h_g) * Wg + w_g
+// slot of region r -> pixel; empty slots (beyond the batch or past a ragged region edge) get
+// out_off = -1 and read pixel (0,0,0) of image 0.
+__device__ __forceinline__ PixelRef locate(const MexKernelArgs &a, int r, int slot)
+{
     const int w_g = r % a.Wg;
     const int h_g = (r / a.Wg) % a.Hg;
     const int c_g = r / (a.Wg * a.Hg);
-
-    const int slot = chunk * 64 + lane;
     bool valid = slot < a.slots;
     const int sl = valid ? slot : 0;
     const int b = sl / a.RS;
@@ -89,102 +95,278 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     if (!valid) {
         c = 0; h = 0; w = 0;
     }
-    const int ci0 = c * a.sc - a.pc, hi0 = h * a.sh - a.ph, wi0 = w * a.sw - a.pw;
-    const float *img = a.in + (size_t)(valid ? b : 0) * a.C * a.H * a.W;
-    const float *base = img + ((ptrdiff_t)ci0 * a.H + hi0) * a.W + wi0;  // only dereferenced in range
+    PixelRef p;
+    p.b = valid ? b : 0;
+    p.ci0 = c * a.sc - a.pc; p.hi0 = h * a.sh - a.ph; p.wi0 = w * a.sw - a.pw;
+    p.base = a.in + (size_t)p.b * a.C * a.H * a.W + ((ptrdiff_t)p.ci0 * a.H + p.hi0) * a.W + p.wi0;
+    p.out_off = valid ? (c * a.Ho + h) * a.Wo + w : -1;
+    return p;
+}
 
-    const float SIMNETS_CONST_AS *offp =
-        (const float SIMNETS_CONST_AS *)(a.offp) + ((size_t)r * a.n_mtiles + mtile) * a.K * MTX;
+constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
-    float mx[MTX];
+template <int PX, int KS, bool NEG, bool CHECK>
+__global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
+{
+    constexpr int WM = 4 / KS;            // instance waves per workgroup
+    constexpr int TM = WM * MX;           // instances per workgroup
+    constexpr int TP = 64 * PX;           // pixels per workgroup
+    constexpr int KSTEP = 256 / TP;       // k handled per staging round (4, 2 or 1)
+    constexpr int KW = KC / KS;           // k of a chunk each K-split wave walks
+    constexpr int kMergeFloats = (KS - 1) * WM * 64 * PX * MX * 2;
+    __shared__ __attribute__((aligned(16))) float smem[cmax(KC * TP + KC * TM, kMergeFloats)];
+    float *xs = smem;                     // [k][pixel]
+    float *os = smem + KC * TP;           // [k][instance]
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave % WM, wk = wave / WM;
+
+    // blockIdx.x -> (pixel chunk, region): the R regions of chunk c get ids that agree mod 8
+    int r, chunk;
+    {
+        const int per_super = kXcds * a.R;
+        const int super = blockIdx.x / per_super;
+        const int within = blockIdx.x - super * per_super;
+        r = within / kXcds;
+        chunk = super * kXcds + (within - r * kXcds);
+    }
+    if (chunk >= a.cpr)
+        return;  // padding of the last super-group (uniform for the whole workgroup)
+    const int mgroup = blockIdx.y;
+    const int m0 = mgroup * TM + wm * MX;            // first instance of this wave
+    const bool wave_active = m0 < a.M;
+
+    // staging role: this thread gathers pixel `sp` for k = sk, sk + KSTEP, ...
+    const int sp = tid % TP, sk = tid / TP;
+    const PixelRef gp = locate(a, r, chunk * TP + sp);
+    const int bhw = a.bh * a.bw;
+    const float *offp = a.offp + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
+
+    auto stage = [&](int k0, int kc) {
+        // patch elements: xs[kk][sp] = patch(sp)[k0 + kk]
+        constexpr int U = KC / KSTEP;  // gathers per thread and chunk: all in flight before the first LDS store
+        for (int kk0 = sk; kk0 < kc; kk0 += KSTEP * U) {
+            float v[U];
 #pragma unroll
-    for (int m = 0; m < MTX; ++m)
-        mx[m] = NEG ? INFINITY : -INFINITY;
-
-    auto gather = [&](int dc, int dh, int dw) -> float {
-        if (CHECK) {
-            const int ci = ci0 + dc, hi = hi0 + dh, wi = wi0 + dw;
-            if (ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W)
-                return base[((ptrdiff_t)dc * a.H + dh) * a.W + dw];
-            return a.oob;
+            for (int u = 0; u < U; ++u) {
+                const int kk = kk0 + u * KSTEP;
+                const int k = k0 + min(kk, kc - 1);
+                int dc = k, dh = 0, dw = 0;
+                if (bhw != 1) {
+                    dc = k / bhw;
+                    const int rem = k - dc * bhw;
+                    dh = rem / a.bw;
+                    dw = rem - dh * a.bw;
+                }
+                const ptrdiff_t o = ((ptrdiff_t)dc * a.H + dh) * a.W + dw;
+                if (CHECK) {
+                    const int ci = gp.ci0 + dc, hi = gp.hi0 + dh, wi = gp.wi0 + dw;
+                    const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                    v[u] = ok ? gp.base[o] : a.oob;
+                } else {
+                    v[u] = gp.base[o];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int kk = kk0 + u * KSTEP;
+                if (kk < kc)
+                    xs[kk * TP + sp] = v[u];
+            }
         }
-        return base[((ptrdiff_t)dc * a.H + dh) * a.W + dw];
+        // offsets: a straight copy of kc * TM floats
+        const float4 *src = reinterpret_cast<const float4 *>(offp + (size_t)k0 * TM);
+        float4 *dst = reinterpret_cast<float4 *>(os);
+        for (int i = tid; i < kc * (TM / 4); i += 256)
+            dst[i] = src[i];
     };
 
-    // ---- sweep 1: running max (min for negative epsilon) of patch + offset ----
-    {
-        const float SIMNETS_CONST_AS *op = offp;
-        for (int dc = 0; dc < a.bc; ++dc)
-            for (int dh = 0; dh < a.bh; ++dh)
-                for (int dw = 0; dw < a.bw; ++dw) {
-                    const float x = gather(dc, dh, dw);
+    float mx[PX][MX];
 #pragma unroll
-                    for (int m = 0; m < MTX; ++m) {
-                        const float v = x + op[m];
-                        mx[m] = NEG ? __builtin_fminf(mx[m], v) : __builtin_fmaxf(mx[m], v);
-                    }
-                    op += MTX;
-                }
+    for (int p = 0; p < PX; ++p)
+#pragma unroll
+        for (int m = 0; m < MX; ++m)
+            mx[p][m] = NEG ? INFINITY : -INFINITY;
+
+    const bool single_chunk = a.K <= KC;
+    const float *xl = xs + lane;                 // this lane's pixels: xl[kk*TP + p*64]
+    const float *ol = os + wm * MX;              // this wave's instances: ol[kk*TM + m]
+
+    // ---- sweep 1: running max (min for negative epsilon) of patch + offset ----
+    for (int k0 = 0; k0 < a.K; k0 += KC) {
+        const int kc = min(KC, a.K - k0);
+        __syncthreads();
+        stage(k0, kc);
+        __syncthreads();
+        if (!wave_active)
+            continue;
+        const int kend = min(kc, (wk + 1) * KW);
+        for (int kk = wk * KW; kk < kend; ++kk) {
+            float x[PX], o[MX];
+#pragma unroll
+            for (int p = 0; p < PX; ++p)
+                x[p] = xl[kk * TP + p * 64];
+#pragma unroll
+            for (int m = 0; m < MX; ++m)
+                o[m] = ol[kk * TM + m];
+            // stage by stage across the 16 instances: a dependent VALU instruction issued right
+            // behind its producer stalls, so producers and consumers are kept 16 instructions apart
+#pragma unroll
+            for (int p = 0; p < PX; ++p) {
+                float v[MX];
+#pragma unroll
+                for (int m = 0; m < MX; ++m)
+                    v[m] = x[p] + o[m];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int m = 0; m < MX; ++m)
+                    mx[p][m] = NEG ? __builtin_fminf(mx[p][m], v[m]) : __builtin_fmaxf(mx[p][m], v[m]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
     }
-    float res[MTX];
+
+    float s[PX][MX];
+#pragma unroll
+    for (int p = 0; p < PX; ++p)
+#pragma unroll
+        for (int m = 0; m < MX; ++m)
+            s[p][m] = 0.0f;
     if (a.finite_eps) {
         // ---- sweep 2: sum of exp(eps * (v - max) + ey), evaluated as exp2 of the scaled argument ----
-        float s[MTX];
+        // the two scale constants are wave-uniform; they are used from VGPRs because VALU instructions
+        // with SGPR operands issue at half rate
+        float c1v, c0v;
+        asm("v_mov_b32 %0, %1" : "=v"(c1v) : "s"(a.c1));
+        asm("v_mov_b32 %0, %1" : "=v"(c0v) : "s"(a.c0));
+        for (int k0 = 0; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            if (!single_chunk) {
+                __syncthreads();
+                stage(k0, kc);
+                __syncthreads();
+            }
+            if (!wave_active)
+                continue;
+            const int kend = min(kc, (wk + 1) * KW);
+            for (int kk = wk * KW; kk < kend; ++kk) {
+                float x[PX], o[MX];
 #pragma unroll
-        for (int m = 0; m < MTX; ++m)
-            s[m] = 0.0f;
-        const float SIMNETS_CONST_AS *op = offp;
-        for (int dc = 0; dc < a.bc; ++dc)
-            for (int dh = 0; dh < a.bh; ++dh)
-                for (int dw = 0; dw < a.bw; ++dw) {
-                    const float x = gather(dc, dh, dw);
+                for (int p = 0; p < PX; ++p)
+                    x[p] = xl[kk * TP + p * 64];
 #pragma unroll
-                    for (int m = 0; m < MTX; ++m) {
-                        const float v = x + op[m];
-                        s[m] += __builtin_amdgcn_exp2f(__builtin_fmaf(v - mx[m], a.c1, a.c0));
-                    }
-                    op += MTX;
+                for (int m = 0; m < MX; ++m)
+                    o[m] = ol[kk * TM + m];
+#pragma unroll
+                for (int p = 0; p < PX; ++p) {
+                    float v[MX];
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        v[m] = x[p] + o[m];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        v[m] = v[m] - mx[p][m];
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        v[m] = __builtin_fmaf(v[m], c1v, c0v);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        v[m] = __builtin_amdgcn_exp2f(v[m]);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        s[p][m] += v[m];
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-#pragma unroll
-        for (int m = 0; m < MTX; ++m)
-            res[m] = mx[m] + logf(s[m]) / a.eps;
-    } else {
-#pragma unroll
-        for (int m = 0; m < MTX; ++m)
-            res[m] = mx[m];
+            }
+        }
     }
-    if (!valid)
-        return;
-    // output channel = instance * channels_out + c  (src/kernels/mex_kernel_cpu.cpp:113-115)
-    const size_t plane = (size_t)a.Ho * a.Wo;
-    float *o = a.out + ((size_t)b * a.M * a.Co + c) * plane + (size_t)h * a.Wo + w;
+
+    if (KS > 1) {
+        // ---- merge the (max, sum) pairs of the K-split waves into wave wk == 0 ----
+        __syncthreads();  // everyone is done with xs / os
+        // layout [split wave][value][lane]: consecutive lanes hit consecutive banks
+        float *mg = smem + (size_t)((wk > 0 ? wk - 1 : 0) * WM + wm) * (PX * MX * 2 * 64) + lane;
+        if (wk > 0 && wave_active) {
 #pragma unroll
-    for (int m = 0; m < MTX; ++m) {
-        const int mm = mtile * MTX + m;
-        if (mm < a.M)
-            o[(size_t)mm * a.Co * plane] = res[m];
+            for (int p = 0; p < PX; ++p)
+#pragma unroll
+                for (int m = 0; m < MX; ++m) {
+                    mg[((p * MX + m) * 2) * 64] = mx[p][m];
+                    mg[((p * MX + m) * 2 + 1) * 64] = s[p][m];
+                }
+        }
+        __syncthreads();
+        if (wk > 0)
+            return;
+        if (wave_active) {
+            for (int j = 1; j < KS; ++j) {
+                const float *src = smem + (size_t)((j - 1) * WM + wm) * (PX * MX * 2 * 64) + lane;
+#pragma unroll
+                for (int p = 0; p < PX; ++p)
+#pragma unroll
+                    for (int m = 0; m < MX; ++m) {
+                        const float m2 = src[((p * MX + m) * 2) * 64], s2 = src[((p * MX + m) * 2 + 1) * 64];
+                        const float m1 = mx[p][m];
+                        const float mm = NEG ? __builtin_fminf(m1, m2) : __builtin_fmaxf(m1, m2);
+                        // a side that saw no finite term keeps sum 0; skip the rescale when its
+                        // max equals the merged one (also avoids inf - inf)
+                        const float f1 = (m1 == mm) ? 1.0f : __builtin_amdgcn_exp2f((m1 - mm) * a.c1);
+                        const float f2 = (m2 == mm) ? 1.0f : __builtin_amdgcn_exp2f((m2 - mm) * a.c1);
+                        s[p][m] = s[p][m] * f1 + s2 * f2;
+                        mx[p][m] = mm;
+                    }
+            }
+        }
+    }
+    if (!wave_active)
+        return;
+
+    // output channel = instance * channels_out + c  (src/kernels/mex_kernel_cpu.cpp:113-115)
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+#pragma unroll
+    for (int p = 0; p < PX; ++p) {
+        const PixelRef cp = locate(a, r, chunk * TP + p * 64 + lane);
+        if (cp.out_off < 0)
+            continue;
+        float *o = a.out + (size_t)cp.b * a.M * plane + cp.out_off;
+#pragma unroll
+        for (int m = 0; m < MX; ++m) {
+            // max + log(sum) / eps, the logarithm taken as log2 (v_log_f32) * log(2)/eps
+            const float res = a.finite_eps ? __builtin_fmaf(__builtin_amdgcn_logf(s[p][m]), a.ln2_over_eps, mx[p][m])
+                                           : mx[p][m];
+            if (m0 + m < a.M)
+                o[(size_t)(m0 + m) * plane] = res;
+        }
     }
 }
 
 // One wave per (region, instance) row of the offsets: optional logsumexp normalisation
-// (python/simnets/keras.py:155-160), then the row is scattered into the k-major packed layout.
+// (python/simnets/keras.py:155-160), then the row is scattered into the k-major packed layout
+// [r][mgroup][k][tm].
 __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__restrict__ offsets, int R, int M, int K,
-                                                              int n_mtiles, int normalize, float *__restrict__ offp)
+                                                              int n_mgroups, int tm, int normalize,
+                                                              float *__restrict__ offp)
 {
     const int lane = threadIdx.x & 63;
     const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const long long rows = (long long)R * n_mtiles * MTX;
+    const long long rows = (long long)R * n_mgroups * tm;
     if (row >= rows)
         return;
-    const int mi = (int)(row % MTX);
-    const long long t = row / MTX;
-    const int mtile = (int)(t % n_mtiles);
-    const int r = (int)(t / n_mtiles);
-    const int m = mtile * MTX + mi;
-    float *dst = offp + ((size_t)r * n_mtiles + mtile) * K * MTX + mi;
+    const int mi = (int)(row % tm);
+    const long long t = row / tm;
+    const int mgroup = (int)(t % n_mgroups);
+    const int r = (int)(t / n_mgroups);
+    const int m = mgroup * tm + mi;
+    float *dst = offp + ((size_t)r * n_mgroups + mgroup) * K * tm + mi;
     if (m >= M) {
         for (int k = lane; k < K; k += 64)
-            dst[(size_t)k * MTX] = 0.0f;
+            dst[(size_t)k * tm] = 0.0f;
         return;
     }
     const float *src = offsets + ((size_t)r * M + m) * K;
@@ -205,15 +387,58 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         lse = logf(sum) + mxv;
     }
     for (int k = lane; k < K; k += 64)
-        dst[(size_t)k * MTX] = src[k] - lse;
+        dst[(size_t)k * tm] = src[k] - lse;
+}
+
+template <int PX, int KS>
+hipError_t launch_variant(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, hipStream_t s)
+{
+    if (neg && inside)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, true, false>), grid, dim3(256), 0, s, a);
+    else if (neg)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, true, true>), grid, dim3(256), 0, s, a);
+    else if (inside)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, false, false>), grid, dim3(256), 0, s, a);
+    else
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, false, true>), grid, dim3(256), 0, s, a);
+    return hipGetLastError();
+}
+
+struct MexTiling {
+    int px, ks, tm, n_mgroups;
+};
+
+// Pixels per lane and K-split: the largest register tile that still gives every SIMD about four
+// waves (a wave issues at most one VALU instruction per 4 cycles, a SIMD retires one per 2, so it
+// takes several resident waves to keep it busy across LDS waits); when even one pixel per lane
+// leaves SIMDs idle and K is long, the waves split K instead.
+MexTiling mex_tiling(const MexPlan &p)
+{
+    const long long slots = (long long)p.B * p.d.region_size;
+    const long long mtiles = (p.d.M + MX - 1) / MX;
+    auto waves = [&](int px) { return p.d.num_regions * ((slots + 64 * px - 1) / (64 * px)) * mtiles; };
+    MexTiling t;
+    t.px = 4;
+    while (t.px > 1 && waves(t.px) < 4096)
+        t.px >>= 1;
+    t.ks = 1;
+    if (t.px == 1) {
+        if (waves(1) < 1024 && p.d.K >= 4 * 16)
+            t.ks = 4;
+        else if (waves(1) < 2048 && p.d.K >= 2 * 16)
+            t.ks = 2;
+    }
+    t.tm = (4 / t.ks) * MX;
+    t.n_mgroups = (p.d.M + t.tm - 1) / t.tm;
+    return t;
 }
 
 }  // namespace
 
 size_t mex_workspace_bytes(const MexPlan &p)
 {
-    const size_t n_mtiles = (p.d.M + MTX - 1) / MTX;
-    return align_up(((size_t)p.d.num_regions * n_mtiles * p.d.K + 1) * MTX * sizeof(float), 256);
+    const MexTiling t = mex_tiling(p);
+    return align_up((size_t)p.d.num_regions * t.n_mgroups * p.d.K * t.tm * sizeof(float), 256);
 }
 
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
@@ -223,12 +448,12 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     const simnets_mex_dims &d = p.d;
     if (workspace_bytes < mex_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
-    const int n_mtiles = (d.M + MTX - 1) / MTX;
+    const MexTiling t = mex_tiling(p);
     float *offp = reinterpret_cast<float *>(workspace);
 
-    const long long rows = (long long)d.num_regions * n_mtiles * MTX;
+    const long long rows = (long long)d.num_regions * t.n_mgroups * t.tm;
     hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, offsets,
-                       d.num_regions, d.M, d.K, n_mtiles, p.normalize_offsets, offp);
+                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, offp);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
 
@@ -242,14 +467,14 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     a.Cg = d.offsets_c; a.Hg = d.offsets_h; a.Wg = d.offsets_w;
     a.Cs = d.shared_region_c; a.Hs = d.shared_region_h; a.Ws = d.shared_region_w;
     a.unshared = p.use_unshared;
+    a.R = d.num_regions;
     a.RS = d.region_size;
     a.slots = p.B * d.region_size;
-    a.cpr = (a.slots + 63) / 64;
-    a.M = d.M; a.K = d.K; a.n_mtiles = n_mtiles;
+    a.M = d.M; a.K = d.K; a.n_mgroups = t.n_mgroups;
     const double log2e = 1.4426950408889634;
     a.finite_eps = std::isfinite(p.epsilon);
-    a.eps = p.epsilon;
     a.c1 = a.finite_eps ? (float)((double)p.epsilon * log2e) : 0.0f;
+    a.ln2_over_eps = a.finite_eps ? (float)(0.6931471805599453 / (double)p.epsilon) : 0.0f;
     // ey = softmax ? 0 : (float)-log(K)   (src/kernels/mex_kernel_cpu.cpp:36)
     const float ey = p.softmax_mode ? 0.0f : (float)-std::log((double)d.K);
     a.c0 = (float)((double)ey * log2e);
@@ -260,20 +485,25 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
                         (d.channels_out - 1) * d.stride_c + d.block_c <= p.C &&
                         (d.height_out - 1) * d.stride_h + d.block_h <= p.H &&
                         (d.width_out - 1) * d.stride_w + d.block_w <= p.W;
-    const long long gx = (long long)d.num_regions * a.cpr;
-    if (gx > 0x7fffffffLL)
+    a.cpr = (a.slots + 64 * t.px - 1) / (64 * t.px);
+    const long long supers = (a.cpr + kXcds - 1) / kXcds;
+    const long long gx = supers * kXcds * d.num_regions;
+    if (gx > 0x7fffffffLL || t.n_mgroups > 65535)
         return SIMNETS_ERR_TOO_LARGE;
-    dim3 grid((unsigned)gx, (unsigned)((n_mtiles + 3) / 4));
+    dim3 grid((unsigned)gx, (unsigned)t.n_mgroups);
     const bool neg = p.epsilon < 0;
-    if (neg && inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<true, false>), grid, dim3(256), 0, s, a);
-    else if (neg)
-        hipLaunchKernelGGL((mex_fwd_kernel<true, true>), grid, dim3(256), 0, s, a);
-    else if (inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<false, false>), grid, dim3(256), 0, s, a);
+    hipError_t e;
+    if (t.px == 4)
+        e = launch_variant<4, 1>(a, grid, neg, inside, s);
+    else if (t.px == 2)
+        e = launch_variant<2, 1>(a, grid, neg, inside, s);
+    else if (t.ks == 1)
+        e = launch_variant<1, 1>(a, grid, neg, inside, s);
+    else if (t.ks == 2)
+        e = launch_variant<1, 2>(a, grid, neg, inside, s);
     else
-        hipLaunchKernelGGL((mex_fwd_kernel<false, true>), grid, dim3(256), 0, s, a);
-    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+        e = launch_variant<1, 4>(a, grid, neg, inside, s);
+    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
 namespace {
