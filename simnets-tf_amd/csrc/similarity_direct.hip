@@ -34,6 +34,9 @@ namespace {
 constexpr int kWaves = 4;                 // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr int kLdsBudgetFloats = 16384;   // 64 KiB of input tile per workgroup
+constexpr int kStagePos = 6;              // tile elements per thread and channel (a channel's tile holds at most
+                                          // kStagePos * kThreads floats; larger geometries use the gather kernel)
+constexpr int kStageChan = 6;             // channels whose loads are in flight at once while staging
 
 struct SimKernelArgs {
     const float *in;
@@ -208,13 +211,14 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     const int chan_lds = TR * a.TC;
     float pa0[2 * MT], pc0[MT], pa1[2 * MT], pc1[MT];
     load_params<MODE, MT>(pa0, pc0, pa, pc);
+    TilePositions<kStagePos> tp;
+    tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
 
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
         __syncthreads();
         // ---- stage ccn channels x TR rows x TC columns; out-of-image -> oob ----
-        stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.pw, a.oob,
-                                      nullptr);
+        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccn, ccn, chan_lds, a.oob, nullptr, tp);
         __syncthreads();
         if (!wave_active)
             continue;
@@ -428,7 +432,7 @@ Tiling choose_tiling(const SimPlan &p)
     const int max_rows = std::min(p.oh, (64 * t.nws + t.G - 1) / t.G + 1);
     t.TRmax = (max_rows - 1) * p.sh + p.bh;
     const long long per_chan = 1LL * t.TRmax * t.TC;
-    t.lds_ok = per_chan <= budget;
+    t.lds_ok = per_chan <= std::min(budget, kStagePos * kThreads);
     t.CC = 1;
     if (t.lds_ok) {
         const int cc_max = (int)std::min<long long>(p.C, budget / per_chan);

@@ -42,6 +42,8 @@ constexpr int RP = 4;           // 32-pixel tiles per wave
 constexpr int WG_PIX = 2 * RP * 32;   // 256 pixels per workgroup (2 pixel waves)
 constexpr int WG_TPL = 2 * RM * 32;   // 128 templates per workgroup (2 template waves)
 constexpr int kLdsBudgetFloats = 12288;  // 48 KiB input tile per workgroup
+constexpr int kStagePos = 8;             // tile elements per thread and channel (at most kStagePos * 256 floats)
+constexpr int kStageChan = 4;            // channels whose loads are in flight at once while staging
 
 struct MfmaArgs {
     const float *in;
@@ -115,12 +117,14 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
     load_params(pm + step_stride, pw_nxt, pt_nxt);
     pm += 2 * step_stride;
 
+    TilePositions<kStagePos> tp;
+    tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
+
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
-        stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccp, ccn, TR, a.TC, a.chan_lds, in_row0, a.pw, a.oob,
-                                      a.ctr);
+        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, a.chan_lds, a.oob, a.ctr, tp);
         __syncthreads();
 
         // steps of this chunk in (channel pair, dh, dw) order; the pixel operand of step s+1 and the
@@ -291,7 +295,7 @@ MfmaTiling mfma_tiling(const SimPlan &p)
     pitch = (pitch + 31) / 64 * 64 + 32;
     if (pitch < 1LL * t.TRmax * t.TC)
         pitch += 64;
-    t.ok = 2 * pitch <= kLdsBudgetFloats;
+    t.ok = 2 * pitch <= kLdsBudgetFloats && 1LL * t.TRmax * t.TC <= kStagePos * kThreads;
     t.chan_lds = (int)pitch;
     int cc_max = t.ok ? (int)(kLdsBudgetFloats / pitch) & ~1 : 2;
     cc_max = std::min(cc_max, (p.C + 1) & ~1);

@@ -46,4 +46,68 @@ __device__ __forceinline__ void stage_input_tile(float *lds, const float *img, i
     }
 }
 
+// Division-free variant for tiles of at most NPOS * NTHREADS elements per channel.  Every channel of a
+// tile has the same (row, column) geometry, so each thread resolves its NPOS positions once per
+// kernel (TilePositions::init) and a chunk is staged with all its loads in flight before the first
+// LDS store: one memory latency per chunk.
+template <int NPOS>
+struct TilePositions {
+    int gofs[NPOS];  // offset inside a channel plane, -1: outside the image, -2: not a tile element
+    int lofs[NPOS];  // offset inside an LDS channel slot
+
+    template <int NTHREADS>
+    __device__ __forceinline__ void init(int H, int W, int TR, int TC, int row0, int pad_w)
+    {
+        const int per_chan = TR * TC;
+#pragma unroll
+        for (int j = 0; j < NPOS; ++j) {
+            const int pos = threadIdx.x + j * NTHREADS;
+            const int r = pos / TC;
+            const int c = pos - r * TC;
+            const int ih = row0 + r, iw = c - pad_w;
+            lofs[j] = pos;  // == r * TC + c
+            if (pos >= per_chan)
+                gofs[j] = -2;
+            else if (ih >= 0 && ih < H && iw >= 0 && iw < W)
+                gofs[j] = ih * W + iw;
+            else
+                gofs[j] = -1;
+        }
+    }
+};
+
+// CCMAX bounds the channels of one chunk (registers: NPOS * CCMAX values in flight).
+template <int NPOS, int CCMAX>
+__device__ __forceinline__ void stage_input_tile_fast(float *lds, const float *img, int H, int W, int ch0, int nchan,
+                                                      int nvalid, int chan_pitch, float oob, const float *shift,
+                                                      const TilePositions<NPOS> &tp)
+{
+    const size_t plane = (size_t)H * W;
+    for (int cc0 = 0; cc0 < nchan; cc0 += CCMAX) {
+        float v[CCMAX][NPOS];
+#pragma unroll
+        for (int i = 0; i < CCMAX; ++i) {
+            const int cc = cc0 + i;
+            const bool chan_ok = cc < nvalid;
+            const float *chan = img + (size_t)(ch0 + (chan_ok ? cc : 0)) * plane;
+            const float sh = (shift != nullptr && chan_ok) ? shift[ch0 + cc] : 0.0f;
+#pragma unroll
+            for (int j = 0; j < NPOS; ++j) {
+                float val = oob;
+                if (chan_ok && cc < nchan && tp.gofs[j] >= 0)
+                    val = chan[tp.gofs[j]];
+                v[i][j] = chan_ok ? val - sh : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < CCMAX; ++i) {
+            const int cc = cc0 + i;
+#pragma unroll
+            for (int j = 0; j < NPOS; ++j)
+                if (cc < nchan && tp.gofs[j] != -2)
+                    lds[cc * chan_pitch + tp.lofs[j]] = v[i][j];
+        }
+    }
+}
+
 }  // namespace simnets
