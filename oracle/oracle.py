@@ -285,4 +285,90 @@ def split_patches(reverse, inp, out, N, Dim, W, H, Cc, W_Gs, H_Gs, C_Gs, W_Step,
        int(bool(use_unshared)))
 
 
+def _sim_grad_common(x, templates, weights, output_grad, kw):
+    x = np.ascontiguousarray(x)
+    templates = np.ascontiguousarray(templates, dtype=x.dtype)
+    weights = np.ascontiguousarray(weights, dtype=x.dtype)
+    output_grad = np.ascontiguousarray(output_grad, dtype=x.dtype)
+    kw.setdefault("blocks", templates.shape[2:])
+    a = similarity_args(x.shape, templates.shape[0], **kw)
+    oh, ow = similarity_out_dims(a)
+    assert output_grad.shape == (x.shape[0], templates.shape[0], oh, ow), output_grad.shape
+    return a, x, templates, weights, output_grad
+
+
+def similarity_input_grad(x, templates, weights, output_grad, **kw):
+    """Restatement of SimilarityInputGradKernelCPU::Compute."""
+    a, x, templates, weights, output_grad = _sim_grad_common(x, templates, weights, output_grad, kw)
+    sfx, _ = _sfx(x.dtype)
+    out = np.empty_like(x)
+    rc = getattr(lib(), "so_similarity_input_grad" + sfx)(C.byref(a), _ptr(x), _ptr(templates), _ptr(weights),
+                                                         _ptr(output_grad), _ptr(out))
+    if rc:
+        raise ValueError("similarity_input_grad oracle failed (%d)" % rc)
+    return out
+
+
+def similarity_params_grad(x, templates, weights, output_grad, **kw):
+    """Restatement of SimilarityParametersGradKernelCPU::Compute -> (templates_grad, weights_grad)."""
+    a, x, templates, weights, output_grad = _sim_grad_common(x, templates, weights, output_grad, kw)
+    sfx, _ = _sfx(x.dtype)
+    gt, gw = np.empty_like(templates), np.empty_like(weights)
+    rc = getattr(lib(), "so_similarity_params_grad" + sfx)(C.byref(a), _ptr(x), _ptr(templates), _ptr(weights),
+                                                          _ptr(output_grad), _ptr(gt), _ptr(gw))
+    if rc:
+        raise ValueError("similarity_params_grad oracle failed (%d)" % rc)
+    return gt, gw
+
+
+def _mex_grad(fn, x, offsets, output, output_grad, num_instances, kw):
+    x = np.ascontiguousarray(x)
+    sfx, _ = _sfx(x.dtype)
+    offsets = np.ascontiguousarray(offsets, dtype=x.dtype)
+    output = np.ascontiguousarray(output, dtype=x.dtype)
+    output_grad = np.ascontiguousarray(output_grad, dtype=x.dtype)
+    a = mex_args(x.shape, num_instances, **kw)
+    d = mex_dims(a)
+    assert output.shape == output_grad.shape == (x.shape[0], d.channels_out_total, d.height_out, d.width_out)
+    assert offsets.size == d.num_regions * d.M * d.K
+    res = np.empty_like(x if fn == "so_mex_input_grad" else offsets)
+    rc = getattr(lib(), fn + sfx)(C.byref(a), _ptr(x), _ptr(offsets), _ptr(output), _ptr(output_grad), _ptr(res))
+    if rc:
+        raise ValueError("%s oracle failed (%d)" % (fn, rc))
+    return res
+
+
+def mex_input_grad(x, offsets, output, output_grad, num_instances, **kw):
+    """Restatement of MEXGradInputKernelCPU::Compute."""
+    return _mex_grad("so_mex_input_grad", x, offsets, output, output_grad, num_instances, kw)
+
+
+def mex_offsets_grad(x, offsets, output, output_grad, num_instances, **kw):
+    """Restatement of MEXGradOffsetsKernelCPU::Compute."""
+    return _mex_grad("so_mex_offsets_grad", x, offsets, output, output_grad, num_instances, kw)
+
+
+def col2im_3d(col, im_shape, patch, pad, stride, round_down=True):
+    col = np.ascontiguousarray(col)
+    sfx, _ = _sfx(col.dtype)
+    Cc, H, W = im_shape
+    im = np.empty(im_shape, dtype=col.dtype)
+    getattr(lib(), "so_col2im_3d" + sfx)(_ptr(col), Cc, H, W, *[int(v) for v in patch], *[int(v) for v in pad],
+                                         *[int(v) for v in stride], _ptr(im), int(bool(round_down)))
+    return im
+
+
+def backward_functor(name, dtype, *args, which="oracle"):
+    """name in {'sim_backward_weights_fn', 'sim_backward_bottom_fn', 'mex_backward_term_fn'}; scalar in, scalar(s) out."""
+    sfx, ct = _sfx(dtype)
+    fn = getattr(lib() if which == "oracle" else ref(), ("so_" if which == "oracle" else "ref_") + name + sfx)
+    cargs = [C.c_int(int(args[0]))] + [ct(float(v)) for v in args[1:]]
+    if name == "sim_backward_weights_fn":
+        out = (ct * 2)()
+        fn(*cargs, out)
+        return np.array([out[0], out[1]], dtype=dtype)
+    fn.restype = ct
+    return np.dtype(dtype).type(fn(*cargs))
+
+
 LOG_2PI = math.log(2.0 * math.pi)

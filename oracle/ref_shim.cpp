@@ -6,7 +6,9 @@
 // reference templates
 //     ggemm_cpu, ggemm_readc_cpu, interlace_cpu            include/utils/ggemm_cpu.hpp
 //     sim_l1_forward, sim_l2_forward, sim_l2_normalized_forward   include/utils/similarity_utils.hpp
-//     mex_forward_exp, mex_forward_out, split_patches_cpu   include/utils/mex_utils.hpp
+//     mex_forward_exp, mex_forward_out, split_patches_cpu,
+//     sim_*_backward_weights, sim_*_backward_bottom (similarity_utils.hpp:82-150),
+//     mex_backward_bottom_finite/infinite (mex_utils.hpp:31-46)   include/utils/mex_utils.hpp
 // with the template arguments their callers use (src/kernels/similarity_kernel_cpu.cpp:84-116,
 // src/kernels/mex_kernel_cpu.cpp:15-37, :134-157) so that the C restatement in
 // simnets_oracle.c can be compared with them bit for bit.
@@ -71,7 +73,51 @@ void mex_forward(int M, int N, int K, bool softmax_mode, T epsilon, const T *off
 
 } // namespace
 
+namespace {
+template <typename T>
+void sim_backward_weights(int mode, T err, T x, T t, T w, T fudge, T *out2)
+{
+    using V2 = typename vec<T>::vec2;
+    V2 p = make_vec2<T>(t, w), r;
+    switch (mode) {
+    case 0: r = sim_l1_backward_weights<T>(err, x, p, 0); break;
+    case 1: r = sim_l2_backward_weights<T, false>(err, x, p, 0); break;
+    case 2: r = sim_l2_normalized_backward_weights<T, false, false>(err, x, p, fudge); break;
+    default: r = sim_l2_normalized_backward_weights<T, false, true>(err, x, p, fudge); break;
+    }
+    out2[0] = r.x;
+    out2[1] = r.y;
+}
+template <typename T>
+T sim_backward_bottom(int mode, T t, T w, T err, T data)
+{
+    using V2 = typename vec<T>::vec2;
+    V2 p = make_vec2<T>(t, w);
+    switch (mode) {
+    case 0: return sim_l1_backward_bottom<T>(p, err, data, 0);
+    case 1: return sim_l2_backward_bottom<T, false>(p, err, data, 0);
+    case 2: return sim_l2_normalized_backward_bottom<T, false, false>(p, err, data, T(0));
+    default: return sim_l2_normalized_backward_bottom<T, false, true>(p, err, data, T(0));
+    }
+}
+template <typename T>
+T mex_backward_term(int finite, T offset, T top_data, T top_diff, T data, T ex, T ey)
+{
+    using V2 = typename vec<T>::vec2;
+    if (finite)
+        return mex_backward_bottom_finite<T>(offset, make_vec2<T>(top_data, top_diff), data, make_vec2<T>(ex, ey));
+    return mex_backward_bottom_infinite<T>(offset, make_vec2<T>(top_data, top_diff), data, 0);
+}
+} // namespace
+
 extern "C" {
+
+void ref_sim_backward_weights_fn_f32(int mode, float err, float x, float t, float w, float fudge, float *o) { sim_backward_weights<float>(mode, err, x, t, w, fudge, o); }
+void ref_sim_backward_weights_fn_f64(int mode, double err, double x, double t, double w, double fudge, double *o) { sim_backward_weights<double>(mode, err, x, t, w, fudge, o); }
+float ref_sim_backward_bottom_fn_f32(int mode, float t, float w, float err, float data) { return sim_backward_bottom<float>(mode, t, w, err, data); }
+double ref_sim_backward_bottom_fn_f64(int mode, double t, double w, double err, double data) { return sim_backward_bottom<double>(mode, t, w, err, data); }
+float ref_mex_backward_term_fn_f32(int finite, float offset, float top_data, float top_diff, float data, float ex, float ey) { return mex_backward_term<float>(finite, offset, top_data, top_diff, data, ex, ey); }
+double ref_mex_backward_term_fn_f64(int finite, double offset, double top_data, double top_diff, double data, double ex, double ey) { return mex_backward_term<double>(finite, offset, top_data, top_diff, data, ex, ey); }
 
 int ref_ggemm_padded_output_size(int M, int N) { return ggemm_padded_output_size(M, N); }
 

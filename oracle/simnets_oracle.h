@@ -142,6 +142,46 @@ void so_mex_forward_f32(int M, int N, int K, int softmax_mode, float epsilon, co
 void so_mex_forward_f64(int M, int N, int K, int softmax_mode, double epsilon, const double *offsets,
                         const double *in, double *out, int batch);
 
+/* ---- backward operators --------------------------------------------------------------------
+ * src/kernels/similarity_grad_kernel_cpu.cpp:158-270 / :23-146, src/kernels/mex_grad_kernel_cpu.cpp:32-208 / :220-369.
+ * Pinned by central differences of the fp64 forward oracle and by torch.autograd on the closed forms
+ * (tests/test_oracle_pins.py); the backward functors are pinned bit-exactly against oracle/_ref. */
+int so_similarity_input_grad_f32(const so_similarity_args *a, const float *input, const float *templates,
+                                 const float *weights, const float *output_grad, float *input_grad);
+int so_similarity_input_grad_f64(const so_similarity_args *a, const double *input, const double *templates,
+                                 const double *weights, const double *output_grad, double *input_grad);
+int so_similarity_params_grad_f32(const so_similarity_args *a, const float *input, const float *templates,
+                                  const float *weights, const float *output_grad, float *templates_grad,
+                                  float *weights_grad);
+int so_similarity_params_grad_f64(const so_similarity_args *a, const double *input, const double *templates,
+                                  const double *weights, const double *output_grad, double *templates_grad,
+                                  double *weights_grad);
+int so_mex_input_grad_f32(const so_mex_args *a, const float *input, const float *offsets, const float *output,
+                          const float *output_grad, float *input_grad);
+int so_mex_input_grad_f64(const so_mex_args *a, const double *input, const double *offsets, const double *output,
+                          const double *output_grad, double *input_grad);
+int so_mex_offsets_grad_f32(const so_mex_args *a, const float *input, const float *offsets, const float *output,
+                            const float *output_grad, float *offsets_grad);
+int so_mex_offsets_grad_f64(const so_mex_args *a, const double *input, const double *offsets, const double *output,
+                            const double *output_grad, double *offsets_grad);
+/* src/utils/im2col.cpp:297-328 */
+void so_col2im_3d_f32(const float *col, int channels, int height, int width, int patch_c, int patch_h, int patch_w,
+                      int pad_c, int pad_h, int pad_w, int stride_c, int stride_h, int stride_w, float *im,
+                      int round_down);
+void so_col2im_3d_f64(const double *col, int channels, int height, int width, int patch_c, int patch_h, int patch_w,
+                      int pad_c, int pad_h, int pad_w, int stride_c, int stride_h, int stride_w, double *im,
+                      int round_down);
+/* the backward combine functors one call at a time (similarity_utils.hpp:82-150, mex_utils.hpp:31-46);
+ * mode as in so_ggemm_similarity, out2 = (d/dtemplate, d/dweight) */
+void so_sim_backward_weights_fn_f32(int mode, float err, float x, float t, float w, float fudge, float *out2);
+void so_sim_backward_weights_fn_f64(int mode, double err, double x, double t, double w, double fudge, double *out2);
+float so_sim_backward_bottom_fn_f32(int mode, float t, float w, float err, float data);
+double so_sim_backward_bottom_fn_f64(int mode, double t, double w, double err, double data);
+float so_mex_backward_term_fn_f32(int finite, float offset, float top_data, float top_diff, float data, float ex,
+                                  float ey);
+double so_mex_backward_term_fn_f64(int finite, double offset, double top_data, double top_diff, double data,
+                                   double ex, double ey);
+
 #ifdef __cplusplus
 }
 #endif

@@ -454,3 +454,215 @@ def test_normalize_offsets_is_logsumexp_normalisation(dtype):
     tol = 1e-12 if dtype == np.float64 else 2e-6
     np.testing.assert_allclose(got, exp, rtol=tol, atol=tol)
     np.testing.assert_allclose(np.exp(got.reshape(24, -1).astype(np.float64)).sum(axis=1), 1.0, rtol=10 * tol)
+
+
+# ---------------------------------------------------------------------------------------------
+# backward operators.  The reference's own tests compare them with numeric differentiation of the
+# forward op (python/simnets/test/__init__.py:60-100, :265-300); the same is done here against the
+# fp64 forward oracle (element by element, central differences), plus torch.autograd on closed
+# forms built from library routines, plus the combine functors bit for bit against oracle/_ref.
+# ---------------------------------------------------------------------------------------------
+def _numeric_grad(f, x, g_out, h=1e-6):
+    """d <f(x), g_out> / dx by central differences; x is modified in place and restored."""
+    grad = np.zeros_like(x)
+    flat, gflat = x.reshape(-1), grad.reshape(-1)
+    for i in range(flat.size):
+        if np.isnan(flat[i]):
+            continue
+        keep = flat[i]
+        flat[i] = keep + h
+        up = f()
+        flat[i] = keep - h
+        dn = f()
+        flat[i] = keep
+        gflat[i] = np.nansum((up - dn) * g_out) / (2 * h)
+    return grad
+
+
+@needs_ref
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_backward_functors_bit_exact_vs_reference(dtype):
+    g = rng(60)
+    vals = g.normal(size=(400, 6)).astype(dtype)
+    vals[::7, 1] = np.nan                       # NaN data: the ignore-NaN variants must return zeros
+    vals[::11, 1] = vals[::11, 2]               # x == t: sign(0) = 0 in the L1 functors
+    for row in vals:
+        err, x, t, w, fudge, extra = [dtype(v) for v in row]
+        w, fudge = abs(w) + dtype(0.1), abs(fudge) * dtype(0.01)
+        for mode in range(4):
+            a = orc.backward_functor("sim_backward_weights_fn", dtype, mode, err, x, t, w, fudge)
+            b = orc.backward_functor("sim_backward_weights_fn", dtype, mode, err, x, t, w, fudge, which="ref")
+            assert a.tobytes() == b.tobytes(), (mode, row)
+            a = orc.backward_functor("sim_backward_bottom_fn", dtype, mode, t, w, err, x)
+            b = orc.backward_functor("sim_backward_bottom_fn", dtype, mode, t, w, err, x, which="ref")
+            assert a.tobytes() == b.tobytes(), (mode, row)
+        if np.isnan(x):
+            continue
+        for finite in (0, 1):
+            top = x + t if (finite == 0 and extra > 0) else extra     # equality branch of the infinite form
+            a = orc.backward_functor("mex_backward_term_fn", dtype, finite, t, top, err, x, w, fudge)
+            b = orc.backward_functor("mex_backward_term_fn", dtype, finite, t, top, err, x, w, fudge, which="ref")
+            assert a.tobytes() == b.tobytes(), (finite, row)
+
+
+@pytest.mark.parametrize("patch,pad,stride", [((1, 3, 3), (0, 1, 1), (1, 1, 1)), ((2, 3, 2), (1, 0, 2), (1, 2, 1)),
+                                              ((3, 1, 1), (0, 0, 0), (3, 1, 1)), ((2, 2, 2), (1, 1, 1), (2, 3, 2))])
+@pytest.mark.parametrize("round_down", [True, False])
+def test_col2im_3d_is_the_adjoint_of_im2col_3d(patch, pad, stride, round_down):
+    g = rng(61)
+    shape = (4, 7, 6)
+    x = g.normal(size=shape)
+    outs = [orc.dimension_out_size(shape[i], pad[i], patch[i], stride[i], round_down) for i in range(3)]
+    col = orc.im2col_3d(x, patch, pad, stride, round_down=round_down, oob=0.0)
+    c = g.normal(size=col.shape)
+    assert col.size == np.prod(patch) * np.prod(outs)
+    back = orc.col2im_3d(c, shape, patch, pad, stride, round_down=round_down)
+    np.testing.assert_allclose(np.sum(col * c), np.sum(x * back), rtol=1e-12)
+    # every basis image: <im2col(e_i), c> = col2im(c)[i]
+    probe = np.zeros(shape)
+    for idx in [(0, 0, 0), (3, 6, 5), (1, 3, 2), (2, 0, 5)]:
+        probe[idx] = 1.0
+        got = np.sum(orc.im2col_3d(probe, patch, pad, stride, round_down=round_down, oob=0.0) * c)
+        probe[idx] = 0.0
+        np.testing.assert_allclose(got, back[idx], rtol=1e-12, atol=1e-14)
+
+
+def test_col2im_2d_matches_torch_fold():
+    g = rng(62)
+    C_, H, W = 3, 9, 8
+    blocks, strides, padding = (3, 2), (2, 1), (1, 1)
+    oh = orc.dimension_out_size(H, padding[0], blocks[0], strides[0])
+    ow = orc.dimension_out_size(W, padding[1], blocks[1], strides[1])
+    col = g.normal(size=(C_ * blocks[0] * blocks[1], oh * ow))
+    want = F.fold(torch.from_numpy(col)[None], (H, W), blocks, padding=padding, stride=strides)[0].numpy()
+    got = orc.col2im_3d(col, (C_, H, W), (C_,) + blocks, (0,) + padding, (C_,) + strides)
+    np.testing.assert_allclose(got, want, rtol=1e-13, atol=1e-13)
+
+
+SIM_GRAD_CASES = [  # func, norm, ignore_nan, blocks, strides, padding
+    ("L2", False, False, (3, 3), (1, 1), (1, 1)),
+    ("L2", False, False, (3, 1), (2, 1), (0, 0)),
+    ("L1", False, False, (3, 3), (2, 2), (1, 1)),
+    ("L1", False, False, (1, 1), (1, 1), (0, 0)),
+    ("L2", True, False, (3, 3), (2, 1), (1, 0)),
+    ("L2", True, True, (3, 3), (1, 1), (1, 1)),
+    ("L2", True, True, (2, 3), (2, 2), (1, 1)),
+]
+
+
+@pytest.mark.parametrize("func,norm,ign,blocks,strides,padding", SIM_GRAD_CASES)
+def test_similarity_grads_match_numeric_differentiation(func, norm, ign, blocks, strides, padding):
+    g = rng(63)
+    x, t, w = _sim_inputs(g, (2, 3, 7, 6), 3, blocks, np.float64)
+    if ign:
+        x[g.random(size=x.shape) < 0.15] = np.nan
+    kw = dict(similarity_function=func, blocks=blocks, strides=strides, padding=padding, normalization_term=norm,
+              ignore_nan_input=ign, out_of_bounds_value=np.nan if ign else 0.3)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    go = g.normal(size=out.shape)
+    f = lambda: orc.similarity_fwd(x, t, w, **kw)
+    gx = orc.similarity_input_grad(x, t, w, go, **kw)
+    gt, gw = orc.similarity_params_grad(x, t, w, go, **kw)
+    assert gx.shape == x.shape and gt.shape == t.shape and gw.shape == w.shape
+    if ign:
+        assert (gx[np.isnan(x)] == 0).all() and not np.isnan(gx).any()
+    np.testing.assert_allclose(gx, _numeric_grad(f, x, go), rtol=2e-7, atol=2e-7)
+    np.testing.assert_allclose(gt, _numeric_grad(f, t, go), rtol=2e-7, atol=2e-7)
+    np.testing.assert_allclose(gw, _numeric_grad(f, w, go), rtol=2e-7, atol=2e-7)
+
+
+@pytest.mark.parametrize("func", ["L1", "L2"])
+def test_similarity_grads_match_torch_autograd_of_unfold_form(func):
+    g = rng(64)
+    blocks, strides, padding = (3, 2), (2, 1), (1, 1)
+    x, t, w = _sim_inputs(g, (3, 4, 9, 8), 5, blocks, np.float64)
+    kw = dict(similarity_function=func, blocks=blocks, strides=strides, padding=padding)
+    tx, tt, tw = [torch.from_numpy(a).requires_grad_() for a in (x, t, w)]
+    cols = F.unfold(tx, blocks, padding=padding, stride=strides)                    # [B, K, P]
+    d = cols[:, None] - tt.reshape(5, -1)[None, :, :, None]                         # [B, O, K, P]
+    d = d.abs() if func == "L1" else d * d
+    out = -(tw.reshape(5, -1)[None, :, :, None] * d).sum(2)
+    go = g.normal(size=tuple(out.shape))
+    out.backward(torch.from_numpy(go))
+    oshape = orc.similarity_fwd(x, t, w, **kw).shape
+    go = go.reshape(oshape)
+    np.testing.assert_allclose(orc.similarity_input_grad(x, t, w, go, **kw), tx.grad.numpy(), rtol=1e-11, atol=1e-12)
+    gt, gw = orc.similarity_params_grad(x, t, w, go, **kw)
+    np.testing.assert_allclose(gt, tt.grad.numpy(), rtol=1e-11, atol=1e-12)
+    np.testing.assert_allclose(gw, tw.grad.numpy(), rtol=1e-11, atol=1e-12)
+
+
+def test_similarity_grads_fp32_follow_fp64():
+    g = rng(65)
+    x, t, w = _sim_inputs(g, (2, 5, 12, 11), 6, (3, 3), np.float32)
+    kw = dict(similarity_function="L2", blocks=(3, 3), strides=(1, 2), padding=(1, 1), normalization_term=True)
+    go = g.normal(size=orc.similarity_fwd(x, t, w, **kw).shape).astype(np.float32)
+    a32 = (orc.similarity_input_grad(x, t, w, go, **kw),) + orc.similarity_params_grad(x, t, w, go, **kw)
+    d = [a.astype(np.float64) for a in (x, t, w, go)]
+    a64 = (orc.similarity_input_grad(*d, **kw),) + orc.similarity_params_grad(*d, **kw)
+    for lo, hi in zip(a32, a64):
+        assert lo.dtype == np.float32
+        np.testing.assert_allclose(lo, hi, rtol=1e-4, atol=1e-4 * np.abs(hi).max())
+
+
+MEX_GRAD_CASES = [  # im_dims, instances, kw
+    ((2, 3, 6, 5), 2, dict(blocks=[1, 3, 3], strides=[1, 1, 1], padding=[0, 1, 1], shared_offset_region=[2])),
+    ((2, 3, 6, 5), 2, dict(blocks=[1, 3, 3], strides=[1, 1, 1], padding=[0, 1, 1], shared_offset_region=[2],
+                           use_unshared_regions=False)),
+    ((1, 4, 7, 6), 3, dict(blocks=[2, 2, 2], strides=[2, 2, 1], padding=[0, 0, 0], shared_offset_region=[1, 2, 3])),
+    ((2, 3, 5, 5), 2, dict(blocks=[3, 1, 1], strides=[3, 1, 1], padding=[0, 0, 0])),
+    ((1, 3, 6, 6), 2, dict(blocks=[2, 3, 2], strides=[1, 2, 2], padding=[1, 1, 0], blocks_round_down=False,
+                           blocks_out_of_bounds_value=-0.7, shared_offset_region=[1, 2, 2])),
+]
+
+
+@pytest.mark.parametrize("eps,softmax", [(1.0, False), (-2.0, False), (0.7, True), (math.inf, False),
+                                         (-math.inf, False)])
+@pytest.mark.parametrize("im_dims,inst,kw", MEX_GRAD_CASES)
+def test_mex_grads_match_numeric_differentiation(im_dims, inst, kw, eps, softmax):
+    g = rng(66)
+    kw = dict(kw, epsilon=eps, softmax_mode=softmax)
+    x, off, d = _mex_case(g, im_dims, inst, np.float64, **kw)
+    out = orc.mex_fwd(x, off, inst, **kw)
+    go = g.normal(size=out.shape)
+    f = lambda: orc.mex_fwd(x, off, inst, **kw)
+    gx = orc.mex_input_grad(x, off, out, go, inst, **kw)
+    goff = orc.mex_offsets_grad(x, off, out, go, inst, **kw)
+    assert gx.shape == x.shape and goff.shape == off.shape
+    np.testing.assert_allclose(gx, _numeric_grad(f, x, go, h=1e-7), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(goff, _numeric_grad(f, off, go, h=1e-7), rtol=1e-6, atol=1e-6)
+
+
+def test_mex_grads_1x1_single_region_match_torch_logsumexp():
+    g = rng(67)
+    B, C_, H, W, M = 2, 6, 4, 5, 3
+    eps = 1.75                                  # exactly representable: the attribute is a C float
+    kw = dict(blocks=[C_, 1, 1], strides=[C_, 1, 1], padding=[0, 0, 0], epsilon=eps, use_unshared_regions=False)
+    x = g.normal(size=(B, C_, H, W))
+    off = g.normal(size=(1, M, C_, 1, 1))
+    tx, to = torch.from_numpy(x).requires_grad_(), torch.from_numpy(off).requires_grad_()
+    z = tx[:, None] + to.reshape(M, C_)[None, :, :, None, None]                 # [B, M, C, H, W]
+    out = (torch.logsumexp(eps * z, dim=2) - math.log(C_)) / eps
+    go = g.normal(size=tuple(out.shape))
+    out.backward(torch.from_numpy(go))
+    fwd = orc.mex_fwd(x, off, M, **kw)
+    np.testing.assert_allclose(fwd, out.detach().numpy(), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(orc.mex_input_grad(x, off, fwd, go, M, **kw), tx.grad.numpy(), rtol=1e-11, atol=1e-13)
+    np.testing.assert_allclose(orc.mex_offsets_grad(x, off, fwd, go, M, **kw), to.grad.numpy(), rtol=1e-11,
+                               atol=1e-13)
+
+
+def test_mex_grads_fp32_follow_fp64():
+    g = rng(68)
+    kw = dict(blocks=[1, 3, 3], strides=[1, 2, 2], padding=[0, 1, 1], shared_offset_region=[3], epsilon=1.0)
+    x, off, d = _mex_case(g, (2, 4, 11, 10), 4, np.float32, **kw)
+    out = orc.mex_fwd(x, off, 4, **kw)
+    go = g.normal(size=out.shape).astype(np.float32)
+    lo = (orc.mex_input_grad(x, off, out, go, 4, **kw), orc.mex_offsets_grad(x, off, out, go, 4, **kw))
+    d64 = [a.astype(np.float64) for a in (x, off)]
+    out64 = orc.mex_fwd(*d64, 4, **kw)
+    hi = (orc.mex_input_grad(*d64, out64, go.astype(np.float64), 4, **kw),
+          orc.mex_offsets_grad(*d64, out64, go.astype(np.float64), 4, **kw))
+    for a, b in zip(lo, hi):
+        assert a.dtype == np.float32
+        np.testing.assert_allclose(a, b, rtol=1e-4, atol=1e-4 * np.abs(b).max())
