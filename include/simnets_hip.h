@@ -113,6 +113,30 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
                                const float *templates, const float *weights, float *output, void *workspace,
                                size_t workspace_bytes, void *stream);
 
+/* Backward.  Scratch sizes of the two gradient calls (either pointer may be NULL). */
+int simnets_hip_similarity_grad_workspace_bytes(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                                const int templates_shape[4], size_t *input_grad_bytes,
+                                                size_t *params_grad_bytes);
+
+/* REGISTER_OP("SimilarityInputGrad") (src/ops/similarity_op.cpp:141-156): replaces
+ * SimilarityInputGradKernelGPU<float>::Compute (src/kernels/similarity_grad_kernel_gpu.cu), i.e. per image
+ * im2col_3d_gpu + ggemm_readc_gpu<TRANSPOSE_A> with sim_*_backward_bottom + col2im_3d_gpu.
+ * output_grad has the forward output's shape, input_grad the input's.  attrs->algo is ignored. */
+int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                      const int templates_shape[4], const int weights_shape[4], const float *input,
+                                      const float *templates, const float *weights, const float *output_grad,
+                                      float *input_grad, void *workspace, size_t workspace_bytes, void *stream);
+
+/* REGISTER_OP("SimilarityParametersGrad") (src/ops/similarity_op.cpp:158-174): replaces
+ * SimilarityParametersGradKernelGPU<float>::Compute, i.e. per image im2col_3d_gpu + ggemm_readc_gpu with
+ * sim_*_backward_weights accumulated over the batch + deinterlace.  templates_grad and weights_grad have
+ * the templates' shape.  The sums over pixels are formed in a fixed order: results are reproducible. */
+int simnets_hip_similarity_params_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                       const int templates_shape[4], const int weights_shape[4], const float *input,
+                                       const float *templates, const float *weights, const float *output_grad,
+                                       float *templates_grad, float *weights_grad, void *workspace,
+                                       size_t workspace_bytes, void *stream);
+
 /* ------------------------------------------------------------------------------------------
  * MEX:  REGISTER_OP("Mex")  src/ops/mex_op.cpp:58-74
  * ------------------------------------------------------------------------------------------ */
@@ -176,6 +200,30 @@ int simnets_hip_mex_workspace_bytes(const simnets_mex_attrs *attrs, const int in
 int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                         const float *offsets, size_t offsets_count, float *output, void *workspace,
                         size_t workspace_bytes, void *stream);
+
+/* Backward.  Scratch sizes of the two gradient calls (either pointer may be NULL). */
+int simnets_hip_mex_grad_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4],
+                                         size_t *input_grad_bytes, size_t *offsets_grad_bytes);
+
+/* REGISTER_OP("MexInputGrad") (src/ops/mex_op.cpp:134-151): replaces MEXGradInputKernelGPU<float>::Compute
+ * (src/kernels/mex_grad_kernel_gpu.cu), i.e. per image im2col_3d_gpu + split_patches + ggemm_readc_gpu with
+ * mex_backward_bottom_finite/_infinite + reverse split_patches + col2im_3d_gpu.
+ * output = the forward result for the same input/offsets/attrs, output_grad has its shape, input_grad the
+ * input's.  When blocks overlap (block > stride) contributions are added with floating-point atomics, so
+ * the summation order, and with it the last bits, may differ between runs. */
+int simnets_hip_mex_input_grad(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                               const float *offsets, size_t offsets_count, const float *output,
+                               const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
+                               void *stream);
+
+/* REGISTER_OP("MexOffsetsGrad") (src/ops/mex_op.cpp:153-170): replaces MEXGradOffsetsKernelGPU<float>::Compute.
+ * offsets_grad has the offsets' shape [R,M,bc,bh,bw]; sums run in a fixed order (reproducible).
+ * With attrs->normalize_offsets the forward op saw o - logsumexp(o); the gradient returned is the one
+ * w.r.t. the raw offsets o (the chain rule through python/simnets/keras.py:155-160 is applied). */
+int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 const float *offsets, size_t offsets_count, const float *output,
+                                 const float *output_grad, float *offsets_grad, void *workspace,
+                                 size_t workspace_bytes, void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Glue of the missing-data network between MEX layers: non-overlapping sum pooling, which the

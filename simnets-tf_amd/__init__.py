@@ -1,4 +1,4 @@
-"""MI355X-native SimNets forward operators (Similarity, MEX) behind the reference's op API.
+"""MI355X-native SimNets operators (Similarity, MEX: forward and gradients) behind the reference's op API.
 
 `similarity(...)` and `mex(...)` take the same arguments as python/simnets/ops/similarity.py:48
 and python/simnets/ops/mex.py:114 of HUJI-Deep/simnets-tf, operate on CUDA(=HIP) torch tensors
@@ -13,8 +13,13 @@ from .ops import (  # noqa: F401
     mex,
     mex_output_shape,
     sum_pooling,
+    similarity_input_grad,
+    similarity_parameters_grad,
+    mex_input_grad,
+    mex_offsets_grad,
     _mex_dims_helper,
     _expand_dim_specification,
 )
 
-__all__ = ["similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError"]
+__all__ = ["similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError",
+           "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad"]

@@ -12,6 +12,9 @@ EXPORTS = [
     "simnets_hip_similarity_workspace_bytes", "simnets_hip_similarity_fwd",
     "simnets_mex_attrs_default", "simnets_mex_calc_dims", "simnets_mex_out_shape", "get_mex_offsets_nregions",
     "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
+    "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
+    "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
+    "simnets_hip_mex_offsets_grad",
 ]
 
 SIM_L1, SIM_L2 = 0, 1
@@ -93,10 +96,26 @@ def lib():
         l.simnets_hip_mex_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
         l.simnets_hip_mex_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, C.c_size_t, P]
         l.simnets_hip_sum_pool_fwd.argtypes = [I4, C.c_int, C.c_int, P, P, P]
+        SZ = C.POINTER(C.c_size_t)
+        l.simnets_hip_similarity_grad_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, SZ, SZ]
+        l.simnets_hip_similarity_input_grad.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P, P,
+                                                        C.c_size_t, P]
+        l.simnets_hip_similarity_params_grad.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P, P, P,
+                                                         C.c_size_t, P]
+        l.simnets_hip_mex_grad_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, SZ, SZ]
+        l.simnets_hip_mex_input_grad.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, C.c_size_t, P]
+        l.simnets_hip_mex_offsets_grad.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, C.c_size_t,
+                                                   P]
         for name in ("simnets_similarity_out_shape", "simnets_hip_similarity_workspace_bytes",
                      "simnets_hip_similarity_fwd", "simnets_mex_calc_dims", "simnets_mex_out_shape",
                      "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
-                     "get_mex_offsets_nregions"):
+    "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
+    "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
+    "simnets_hip_mex_offsets_grad",
+                     "get_mex_offsets_nregions", "simnets_hip_similarity_grad_workspace_bytes",
+                     "simnets_hip_similarity_input_grad", "simnets_hip_similarity_params_grad",
+                     "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
+                     "simnets_hip_mex_offsets_grad"):
             getattr(l, name).restype = C.c_int
         _lib = l
     return _lib

@@ -56,6 +56,87 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
     return sim_launch(p, input, templates, weights, output, workspace, workspace_bytes, stream);
 }
 
+int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                      const int templates_shape[4], const int weights_shape[4], const float *input,
+                                      const float *templates, const float *weights, const float *output_grad,
+                                      float *input_grad, void *workspace, size_t workspace_bytes, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, weights_shape, &p);
+    if (rc)
+        return rc;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !templates || !weights || !output_grad || !input_grad)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, sim_grad_input_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_grad_input(p, input, templates, weights, output_grad, input_grad, workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_similarity_params_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                       const int templates_shape[4], const int weights_shape[4], const float *input,
+                                       const float *templates, const float *weights, const float *output_grad,
+                                       float *templates_grad, float *weights_grad, void *workspace,
+                                       size_t workspace_bytes, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, weights_shape, &p);
+    if (rc)
+        return rc;
+    if (!templates || !weights || !templates_grad || !weights_grad || (p.B > 0 && (!input || !output_grad)))
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, sim_grad_params_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_grad_params(p, input, templates, weights, output_grad, templates_grad, weights_grad, workspace,
+                           workspace_bytes, stream);
+}
+
+static int mex_grad_checks(const simnets_mex_attrs *attrs, const int input_shape[4], size_t offsets_count,
+                           MexPlan *p)
+{
+    const int rc = mex_make_plan(attrs, input_shape, p);
+    if (rc)
+        return rc;
+    if (offsets_count < (size_t)p->d.num_regions * p->d.M * p->d.K)
+        return SIMNETS_ERR_SHAPE;
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_input_grad(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                               const float *offsets, size_t offsets_count, const float *output,
+                               const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
+                               void *stream)
+{
+    MexPlan p;
+    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    if (rc)
+        return rc;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !offsets || !output || !output_grad || !input_grad)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, mex_grad_input_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return mex_grad_input(p, input, offsets, output, output_grad, input_grad, workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 const float *offsets, size_t offsets_count, const float *output,
+                                 const float *output_grad, float *offsets_grad, void *workspace,
+                                 size_t workspace_bytes, void *stream)
+{
+    MexPlan p;
+    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    if (rc)
+        return rc;
+    if (!offsets || !offsets_grad || (p.B > 0 && (!input || !output || !output_grad)))
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, mex_grad_offsets_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return mex_grad_offsets(p, input, offsets, output, output_grad, offsets_grad, workspace, workspace_bytes, stream);
+}
+
 int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                         const float *offsets, size_t offsets_count, float *output, void *workspace,
                         size_t workspace_bytes, void *stream)

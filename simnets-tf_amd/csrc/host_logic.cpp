@@ -308,6 +308,21 @@ int simnets_hip_similarity_workspace_bytes(const simnets_similarity_attrs *attrs
     return SIMNETS_OK;
 }
 
+int simnets_hip_similarity_grad_workspace_bytes(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                                const int templates_shape[4], size_t *input_grad_bytes,
+                                                size_t *params_grad_bytes)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, templates_shape, &p);
+    if (rc)
+        return rc;
+    if (input_grad_bytes)
+        *input_grad_bytes = sim_grad_input_workspace_bytes(p);
+    if (params_grad_bytes)
+        *params_grad_bytes = sim_grad_params_workspace_bytes(p);
+    return SIMNETS_OK;
+}
+
 void simnets_mex_attrs_default(simnets_mex_attrs *a)
 {
     if (!a)
@@ -396,6 +411,20 @@ int simnets_hip_mex_workspace_bytes(const simnets_mex_attrs *attrs, const int in
     if (!bytes)
         return SIMNETS_ERR_NULL_POINTER;
     *bytes = mex_workspace_bytes(p);
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_grad_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4],
+                                         size_t *input_grad_bytes, size_t *offsets_grad_bytes)
+{
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    if (input_grad_bytes)
+        *input_grad_bytes = mex_grad_input_workspace_bytes(p);
+    if (offsets_grad_bytes)
+        *offsets_grad_bytes = mex_grad_offsets_workspace_bytes(p);
     return SIMNETS_OK;
 }
 

@@ -46,6 +46,22 @@ size_t mex_workspace_bytes(const MexPlan &p);
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
                size_t workspace_bytes, void *stream);
 
+// Backward operators (similarity_grad.hip, mex_grad.hip).  `stream` is a hipStream_t.
+size_t sim_grad_input_workspace_bytes(const SimPlan &p);
+size_t sim_grad_params_workspace_bytes(const SimPlan &p);
+int sim_grad_input(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                   const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes, void *stream);
+int sim_grad_params(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                    const float *output_grad, float *templates_grad, float *weights_grad, void *workspace,
+                    size_t workspace_bytes, void *stream);
+size_t mex_grad_input_workspace_bytes(const MexPlan &p);
+size_t mex_grad_offsets_workspace_bytes(const MexPlan &p);
+int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
+                   const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes, void *stream);
+int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,
+                     const float *output_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
+                     void *stream);
+
 int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *input, float *output, void *stream);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }

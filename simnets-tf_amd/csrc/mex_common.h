@@ -1,0 +1,104 @@
+// Argument block and pixel enumeration shared by the MEX forward and backward kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "internal.h"
+
+namespace simnets {
+
+struct MexKernelArgs {
+    const float *in;
+    float *out;
+    const float *offp;  // [R][mgroup][K][TM]
+    int B, C, H, W;
+    int Co, Ho, Wo;
+    int bc, bh, bw, sc, sh, sw, pc, ph, pw;
+    int Cg, Hg, Wg;     // offsets_c/h/w: number of regions along each axis
+    int Cs, Hs, Ws;     // shared_region_c/h/w: extent of a region along each axis
+    int unshared;
+    int R;              // num_regions
+    int RS;             // region_size
+    int slots;          // B * RS
+    int cpr;            // pixel chunks (64*PX slots) per region
+    int M, K, n_mgroups;
+    float c1;           // eps * log2(e)
+    float c0;           // (softmax ? 0 : -log K) * log2(e)
+    float ln2_over_eps; // log(2) / eps
+    int finite_eps;
+    float oob;
+};
+
+struct PixelRef {
+    const float *base;  // &input[b][c*sc-pc][h*sh-ph][w*sw-pw] (only dereferenced inside the image)
+    int ci0, hi0, wi0;
+    int out_off;        // offset of out[b][c][h][w] within image b's output, -1 if the slot is empty
+    int b;
+};
+
+// slot of region r -> pixel; empty slots (beyond the batch or past a ragged region edge) get
+// out_off = -1 and read pixel (0,0,0) of image 0.
+__device__ __forceinline__ PixelRef locate(const MexKernelArgs &a, int r, int slot)
+{
+    const int w_g = r % a.Wg;
+    const int h_g = (r / a.Wg) % a.Hg;
+    const int c_g = r / (a.Wg * a.Hg);
+    bool valid = slot < a.slots;
+    const int sl = valid ? slot : 0;
+    const int b = sl / a.RS;
+    const int q = sl - b * a.RS;
+    const int i = q % a.Ws;
+    const int j = (q / a.Ws) % a.Hs;
+    const int l = q / (a.Ws * a.Hs);
+    int c, h, w;
+    if (a.unshared) {
+        c = c_g + l * a.Cg; h = h_g + j * a.Hg; w = w_g + i * a.Wg;
+    } else {
+        c = c_g * a.Cs + l; h = h_g * a.Hs + j; w = w_g * a.Ws + i;
+    }
+    valid = valid && c < a.Co && h < a.Ho && w < a.Wo;
+    if (!valid) {
+        c = 0; h = 0; w = 0;
+    }
+    PixelRef p;
+    p.b = valid ? b : 0;
+    p.ci0 = c * a.sc - a.pc; p.hi0 = h * a.sh - a.ph; p.wi0 = w * a.sw - a.pw;
+    p.base = a.in + (size_t)p.b * a.C * a.H * a.W + ((ptrdiff_t)p.ci0 * a.H + p.hi0) * a.W + p.wi0;
+    p.out_off = valid ? (c * a.Ho + h) * a.Wo + w : -1;
+    return p;
+}
+
+// Everything of the argument block that follows from the plan alone (pointers and tiling are the
+// caller's).
+inline MexKernelArgs mex_kernel_args(const MexPlan &p)
+{
+    const simnets_mex_dims &d = p.d;
+    MexKernelArgs a;
+    a.in = nullptr; a.out = nullptr; a.offp = nullptr;
+    a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W;
+    a.Co = d.channels_out; a.Ho = d.height_out; a.Wo = d.width_out;
+    a.bc = d.block_c; a.bh = d.block_h; a.bw = d.block_w;
+    a.sc = d.stride_c; a.sh = d.stride_h; a.sw = d.stride_w;
+    a.pc = d.pad_c; a.ph = d.pad_h; a.pw = d.pad_w;
+    a.Cg = d.offsets_c; a.Hg = d.offsets_h; a.Wg = d.offsets_w;
+    a.Cs = d.shared_region_c; a.Hs = d.shared_region_h; a.Ws = d.shared_region_w;
+    a.unshared = p.use_unshared;
+    a.R = d.num_regions;
+    a.RS = d.region_size;
+    a.slots = p.B * d.region_size;
+    a.cpr = 0;
+    a.M = d.M; a.K = d.K; a.n_mgroups = 0;
+    const double log2e = 1.4426950408889634;
+    a.finite_eps = std::isfinite(p.epsilon);
+    a.c1 = a.finite_eps ? (float)((double)p.epsilon * log2e) : 0.0f;
+    a.ln2_over_eps = a.finite_eps ? (float)(0.6931471805599453 / (double)p.epsilon) : 0.0f;
+    // ey = softmax ? 0 : (float)-log(K)   (src/kernels/mex_kernel_cpu.cpp:36)
+    const float ey = p.softmax_mode ? 0.0f : (float)-std::log((double)d.K);
+    a.c0 = (float)((double)ey * log2e);
+    a.oob = p.oob;
+    return a;
+}
+
+}  // namespace simnets

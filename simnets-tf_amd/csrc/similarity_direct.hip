@@ -24,10 +24,9 @@
 
 #include "internal.h"
 #include "stage.h"
+#include "valu_tile.h"
 
 namespace simnets {
-
-#define SIMNETS_CONST_AS __attribute__((address_space(4)))
 
 namespace {
 
@@ -72,17 +71,6 @@ __device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT]
 #pragma unroll
     for (int i = 0; i < MT; ++i)
         pc[i] = (MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN) ? ppc[i] : 0.0f;
-}
-
-// Copies a wave-uniform value from its SGPR into a VGPR.  VALU instructions that read an SGPR
-// operand issue at half the rate of all-VGPR ones on this chip (measured: 37 vs 64 T lane-ops/s), so
-// each parameter is moved once per (template, k) and then used from the VGPR by all PT pixels.  The
-// asm keeps the compiler from folding the SGPR back into the arithmetic.
-__device__ __forceinline__ float to_vgpr(float uniform)
-{
-    float v;
-    asm("v_mov_b32 %0, %1" : "=v"(v) : "s"(uniform));
-    return v;
 }
 
 // One k step for all MT templates and PT pixels of a lane.

@@ -1,0 +1,812 @@
+// Similarity backward on the vector ALU (gfx950): gradient w.r.t. the input, and w.r.t. the
+// templates and weights.
+//
+// Replaces SimilarityInputGradKernelGPU / SimilarityParametersGradKernelGPU
+// (src/kernels/similarity_grad_kernel_gpu.cu), i.e. per image im2col_3d_gpu + ggemm_readc_gpu with
+// the functors of include/utils/similarity_utils.hpp:82-150 (+ col2im_3d_gpu for the input
+// gradient, + deinterlace for the parameters), by one launch over the whole batch each.
+//
+// Input gradient
+//   dX[b,c,y,x] = sum_o sum_{taps (i,j) whose window covers (y,x)} g[b,o,yo,xo] * B(t[o,c,i,j], w[o,c,i,j], X[b,c,y,x])
+//   with yo = (y + ph - i)/sh.  Input pixels are split by phase (ry, rx) = ((y+ph) mod sh, (x+pw) mod sw):
+//   all pixels of a phase see the same tap subset i = ry + sh*ii, j = rx + sw*jj, and in phase
+//   coordinates a = (y+ph)/sh the sum is a stride-1 correlation of g with that tap subset.  Each
+//   phase is one launch of the same register-tile scheme as the forward kernel with the roles
+//   swapped: g rows are staged in LDS (out of range -> 0), a lane owns PT pixels x MT input
+//   channels (accumulators AND the X values they belong to in VGPRs), the packed parameters of a
+//   (o, tap) step are wave-uniform scalar loads.
+// Parameter gradients
+//   dT[o,k], dW[o,k] = sum over all B*oh*ow output pixels of W(g[px,o], patch(px)[k], t[o,k], w[o,k]).
+//   A lane owns 8 templates x 4 patch elements (its t values and the running sums in VGPRs), a wave
+//   64 x 32, a workgroup 128 x 64 (or 64 x 128); pixels stream through LDS in chunks of 64, g as
+//   [o/4][pixel][4] and the gathered patch elements as [k/4][pixel][4], so that every lane reads its
+//   operands with three 16-byte LDS reads per pixel.  The pixel range is split over workgroups; the
+//   partial sums are written out and added up in a fixed order by a second kernel, which also
+//   applies the factors that do not depend on the pixel (2w, -1, 1/(w+fudge)).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cmath>
+
+#include "internal.h"
+#include "stage.h"
+#include "valu_tile.h"
+
+namespace simnets {
+
+namespace {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = 64 * kWaves;
+constexpr int kLdsBudgetFloats = 16384;
+constexpr int kStagePos = 6;
+constexpr int kStageChan = 6;
+
+enum GradMode { GX_L2 = 0, GX_L1 = 1 };
+
+// ------------------------------------------------------------------------------------------------
+// input gradient
+// ------------------------------------------------------------------------------------------------
+struct GradXArgs {
+    const float *g;    // output gradient [B,O,oh,ow]
+    const float *x;    // input [B,C,H,W]
+    float *dx;         // [B,C,H,W]
+    const float *pb;   // this phase's parameters [ctile][K][MT][2], K = O*nI*nJ, taps flipped
+    int B, C, H, W, O, oh, ow;
+    int nI, nJ;        // taps of this phase along h and w
+    int padh, padw;    // padding of g in phase coordinates: phase row h reads g rows h - padh + dh
+    int na, nb;        // extent of the phase grid
+    int y0, x0;        // input pixel of phase position (h, v): (y0 + sh*h, x0 + sw*v)
+    int sh, sw;
+    int K;
+    int G, gpi, tiles, nws, nws_log2, n_ctiles, TC, TRmax, CC;
+    int ignore_nan;
+    int row_limit, col_limit;  // phase rows h <= row_limit (columns v <= col_limit) are covered by a window
+};
+
+template <int MODE, int PT, int MT>
+__device__ __forceinline__ void gx_step(float (&acc)[MT][PT], const float (&xv)[MT][PT], const float (&gv)[PT],
+                                        const float (&pb)[2 * MT])
+{
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const float p0 = to_vgpr(pb[2 * m]), p1 = to_vgpr(pb[2 * m + 1]);
+        float u[PT];
+        if (MODE == GX_L2) {
+            // (s*w*t, -s*w): u = s*w*(t - x)
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                u[p] = __builtin_fmaf(p1, xv[m][p], p0);
+        } else {
+            // (t, w): u = w * sign(t - x), sign(0) = sign(NaN) = 0
+            float d[PT];
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                d[p] = p0 - xv[m][p];
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                u[p] = __builtin_copysignf(p1, d[p]);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                u[p] = __builtin_islessgreater(d[p], 0.0f) ? u[p] : 0.0f;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            acc[m][p] = __builtin_fmaf(gv[p], u[p], acc[m][p]);
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+constexpr int gx_waves_per_simd(int pt, int mt) { return pt * mt <= 32 ? 4 : 2; }
+constexpr int gx_lds_budget(int pt, int mt) { return pt * mt <= 32 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
+
+template <int MODE, int PT, int MT>
+__global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_input_kernel(const GradXArgs a)
+{
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    const int b = blockIdx.x / a.tiles;
+    const int tile = blockIdx.x - b * a.tiles;
+    const int ws = wave & (a.nws - 1);
+    const int wm = wave >> a.nws_log2;
+    const int nwm = kWaves >> a.nws_log2;
+    const int ctile = blockIdx.y * nwm + wm;
+    const bool wave_active = ctile < a.n_ctiles;
+
+    const int g_first = tile * 64 * a.nws;
+    const int g_last = min(g_first + 64 * a.nws, a.gpi) - 1;
+    const int row_first = g_first / a.G;
+    const int nrows = g_last / a.G - row_first + 1;
+    const int TR = nrows - 1 + a.nI;
+    const int in_row0 = row_first - a.padh;
+
+    int grp = g_first + ws * 64 + lane;
+    const bool lane_valid = grp <= g_last;
+    grp = min(grp, g_last);
+    const int h = grp / a.G;
+    const int gw = grp - h * a.G;
+    const int lds_base = (h - row_first) * a.TC + gw * PT;
+    const int v0 = gw * PT;
+
+    // the X values of this lane's tile (NaN -> 0 when NaN inputs are ignored: their gradient is 0)
+    float acc[MT][PT], xv[MT][PT];
+    const size_t plane = (size_t)a.H * a.W;
+    const float *xrow = a.x + (size_t)b * a.C * plane + (size_t)(a.y0 + a.sh * h) * a.W + a.x0;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int c = ctile * MT + m;
+#pragma unroll
+        for (int p = 0; p < PT; ++p) {
+            acc[m][p] = 0.0f;
+            float val = 0.0f;
+            if (wave_active && lane_valid && c < a.C && v0 + p < a.nb)
+                val = xrow[(size_t)c * plane + (size_t)a.sw * (v0 + p)];
+            if (a.ignore_nan && !(val == val))
+                val = 0.0f;
+            xv[m][p] = val;
+        }
+    }
+
+    const float SIMNETS_CONST_AS *pb =
+        (const float SIMNETS_CONST_AS *)(a.pb) + (size_t)(wave_active ? ctile : 0) * (a.K + 1) * MT * 2;
+    const float *img = a.g + (size_t)b * a.O * a.oh * a.ow;
+    const int chan_lds = TR * a.TC;
+    float pb0[2 * MT], pb1[2 * MT];
+    load_uniform<2 * MT>(pb0, pb);
+    TilePositions<kStagePos> tp;
+    tp.template init<kThreads>(a.oh, a.ow, TR, a.TC, in_row0, a.padw);
+
+    for (int ch0 = 0; ch0 < a.O; ch0 += a.CC) {
+        const int ccn = min(a.CC, a.O - ch0);
+        __syncthreads();
+        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.oh, a.ow, ch0, ccn, ccn, chan_lds, 0.0f, nullptr, tp);
+        __syncthreads();
+        if (!wave_active)
+            continue;
+        // software pipeline over the (o, tap) steps of this chunk: the g values and the parameters of
+        // the next step are requested before the arithmetic of the current one
+        const int nk = ccn * a.nI * a.nJ;
+        int dh = 0, dw = 0, row_off = 0, off = 0;
+        auto step = [&](const float (&gc)[PT], const float (&pbc)[2 * MT], float (&gnx)[PT], float (&pbnx)[2 * MT],
+                        bool last) {
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS and scalar loads share the counter
+            __builtin_amdgcn_sched_barrier(0);
+            const bool wrap_w = dw + 1 == a.nJ;
+            const int ndw = wrap_w ? 0 : dw + 1;
+            const bool wrap_h = wrap_w && dh + 1 == a.nI;
+            const int ndh = wrap_h ? 0 : dh + (wrap_w ? 1 : 0);
+            const int nrow = row_off + (wrap_w ? a.TC : 0) + (wrap_h ? chan_lds - a.nI * a.TC : 0);
+            const int noff = last ? off : nrow + ndw;
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                gnx[p] = lds[lds_base + noff + p];
+            pb += 2 * MT;
+            load_uniform<2 * MT>(pbnx, pb);  // one step of slack exists behind each channel tile
+            __builtin_amdgcn_sched_barrier(0);
+            gx_step<MODE, PT, MT>(acc, xv, gc, pbc);
+            __builtin_amdgcn_sched_barrier(0);
+            dw = ndw; dh = ndh; row_off = nrow; off = noff;
+        };
+        float g0[PT], g1[PT];
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            g0[p] = lds[lds_base + p];
+        int kk = 0;
+        for (; kk + 2 <= nk; kk += 2) {
+            step(g0, pb0, g1, pb1, false);
+            step(g1, pb1, g0, pb0, kk + 2 == nk);
+        }
+        if (kk < nk) {
+            step(g0, pb0, g1, pb1, true);
+#pragma unroll
+            for (int i = 0; i < 2 * MT; ++i)
+                pb0[i] = pb1[i];
+        }
+    }
+
+    if (!wave_active || !lane_valid)
+        return;
+    const bool row_covered = h <= a.row_limit;
+    float *drow = a.dx + (size_t)b * a.C * plane + (size_t)(a.y0 + a.sh * h) * a.W + a.x0;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int c = ctile * MT + m;
+        if (c >= a.C)
+            break;
+#pragma unroll
+        for (int p = 0; p < PT; ++p) {
+            if (v0 + p >= a.nb)
+                continue;
+            const size_t o = (size_t)c * plane + (size_t)a.sw * (v0 + p);
+            float val = (row_covered && v0 + p <= a.col_limit) ? acc[m][p] : 0.0f;
+            if (a.ignore_nan) {
+                const float xin = xrow[o];
+                if (!(xin == xin))
+                    val = 0.0f;
+            }
+            drow[o] = val;
+        }
+    }
+}
+
+// Fallback for geometries whose g rows do not fit the LDS budget: one input element per thread.
+__global__ __launch_bounds__(256) void sim_grad_input_gather_kernel(const float *__restrict__ g,
+                                                                    const float *__restrict__ x,
+                                                                    const float *__restrict__ templates,
+                                                                    const float *__restrict__ weights,
+                                                                    float *__restrict__ dx, int B, int C, int H, int W,
+                                                                    int O, int oh, int ow, int bh, int bw, int sh,
+                                                                    int sw, int ph, int pw, int l1, float scale,
+                                                                    int ignore_nan)
+{
+    const long long total = (long long)B * C * H * W;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long long)gridDim.x * blockDim.x) {
+        const int xx = (int)(idx % W);
+        long long r = idx / W;
+        const int yy = (int)(r % H);
+        r /= H;
+        const int c = (int)(r % C);
+        const int b = (int)(r / C);
+        const float xin = x[idx];
+        float acc = 0.0f;
+        if (!(ignore_nan && !(xin == xin))) {
+            for (int o = 0; o < O; ++o)
+                for (int i = 0; i < bh; ++i) {
+                    const int ty = yy + ph - i;
+                    if (ty < 0 || ty % sh != 0 || ty / sh >= oh)
+                        continue;
+                    for (int j = 0; j < bw; ++j) {
+                        const int tx = xx + pw - j;
+                        if (tx < 0 || tx % sw != 0 || tx / sw >= ow)
+                            continue;
+                        const float gv = g[(((size_t)b * O + o) * oh + ty / sh) * ow + tx / sw];
+                        const size_t pi = (((size_t)o * C + c) * bh + i) * bw + j;
+                        const float t = templates[pi], w = weights[pi];
+                        const float d = t - xin;
+                        float u;
+                        if (l1)
+                            u = w * (float)((0.0f < d) - (d < 0.0f));
+                        else
+                            u = scale * w * d;
+                        acc = __builtin_fmaf(gv, u, acc);
+                    }
+                }
+        }
+        dx[idx] = acc;
+    }
+}
+
+__global__ void fill_zero_kernel(float *__restrict__ p, long long n)
+{
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
+        p[i] = 0.0f;
+}
+
+// Packs one phase's (template, weight) pairs as [ctile][k = (o, dh, dw)][MT][2] with the taps flipped
+// (dh = nI-1-ii, original tap i = ry + sh*ii) and the per-mode scaling folded in.
+__global__ void sim_grad_input_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
+                                           int O, int C, int bh, int bw, int sh, int sw, int ry, int rx, int nI,
+                                           int nJ, int MT, int n_ctiles, int l1, float scale, float *__restrict__ pb)
+{
+    const int K = O * nI * nJ;
+    const long long total = (long long)n_ctiles * (K + 1) * MT;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long long)gridDim.x * blockDim.x) {
+        const int mi = (int)(idx % MT);
+        const long long r = idx / MT;
+        const int k = (int)(r % (K + 1));
+        const int ctile = (int)(r / (K + 1));
+        const int c = ctile * MT + mi;
+        float p0 = 0.0f, p1 = 0.0f;
+        if (k < K && c < C) {
+            const int dw = k % nJ;
+            const int dh = (k / nJ) % nI;
+            const int o = k / (nJ * nI);
+            const int i = ry + sh * (nI - 1 - dh), j = rx + sw * (nJ - 1 - dw);
+            const size_t pi = (((size_t)o * C + c) * bh + i) * bw + j;
+            const float t = templates[pi], w = weights[pi];
+            if (l1) {
+                p0 = t;
+                p1 = w;
+            } else {
+                p0 = scale * w * t;
+                p1 = -(scale * w);
+            }
+        }
+        pb[2 * idx] = p0;
+        pb[2 * idx + 1] = p1;
+    }
+}
+
+struct Phase {
+    int ry, rx, nI, nJ, a0, b0, na, nb;
+    bool empty() const { return nI <= 0 || nJ <= 0 || na <= 0 || nb <= 0; }
+};
+
+void phase_axis(int r, int block, int stride, int pad, int size, int *n_taps, int *first, int *count)
+{
+    *n_taps = r < block ? (block - r + stride - 1) / stride : 0;
+    *first = pad > r ? (pad - r + stride - 1) / stride : 0;
+    const int top = size - 1 + pad - r;  // largest y + pad - r
+    *count = top >= 0 ? top / stride - *first + 1 : 0;
+}
+
+Phase make_phase(const SimPlan &p, int ry, int rx)
+{
+    Phase f;
+    f.ry = ry; f.rx = rx;
+    phase_axis(ry, p.bh, p.sh, p.ph, p.H, &f.nI, &f.a0, &f.na);
+    phase_axis(rx, p.bw, p.sw, p.pw, p.W, &f.nJ, &f.b0, &f.nb);
+    return f;
+}
+
+struct GxTiling {
+    int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
+    bool lds_ok;
+};
+
+GxTiling gx_tiling(const SimPlan &p, const Phase &f)
+{
+    GxTiling t;
+    const bool big = f.nb >= 32 && p.C >= 32;
+    t.PT = big ? 8 : 4;
+    t.MT = 8;
+    const int budget = gx_lds_budget(t.PT, t.MT);
+    t.G = (f.nb + t.PT - 1) / t.PT;
+    t.gpi = f.na * t.G;
+    const int n_ctiles = (p.C + t.MT - 1) / t.MT;
+    t.nws = 1;
+    if (n_ctiles <= 2 && t.gpi >= 128)
+        t.nws = 2;
+    if (n_ctiles <= 1 && t.gpi >= 256)
+        t.nws = 4;
+    t.tiles = (t.gpi + 64 * t.nws - 1) / (64 * t.nws);
+    t.TC = (t.G * t.PT - 1) + f.nJ;
+    t.TC |= 1;
+    const int max_rows = std::min(f.na, (64 * t.nws + t.G - 1) / t.G + 1);
+    t.TRmax = max_rows - 1 + f.nI;
+    const long long per_chan = 1LL * t.TRmax * t.TC;
+    t.lds_ok = per_chan <= std::min(budget, kStagePos * kThreads);
+    t.CC = 1;
+    if (t.lds_ok) {
+        const int cc_max = (int)std::min<long long>(p.O, budget / per_chan);
+        const int chunks = (p.O + cc_max - 1) / cc_max;
+        t.CC = (p.O + chunks - 1) / chunks;
+    }
+    return t;
+}
+
+size_t gx_phase_param_bytes(const SimPlan &p, const Phase &f)
+{
+    const size_t n_ctiles = (p.C + 7) / 8;
+    return align_up(n_ctiles * ((size_t)p.O * f.nI * f.nJ + 1) * 8 * 2 * sizeof(float), 256);
+}
+
+bool gx_all_phases_fit(const SimPlan &p)
+{
+    for (int ry = 0; ry < p.sh; ++ry)
+        for (int rx = 0; rx < p.sw; ++rx) {
+            const Phase f = make_phase(p, ry, rx);
+            if (!f.empty() && !gx_tiling(p, f).lds_ok)
+                return false;
+        }
+    return true;
+}
+
+template <int MODE>
+hipError_t gx_launch_phase(const GradXArgs &a, const GxTiling &t, hipStream_t s)
+{
+    const int nwm = kWaves / a.nws;
+    dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_ctiles + nwm - 1) / nwm));
+    const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
+    if (t.PT == 8)
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 8, 8>), grid, dim3(kThreads), lds_bytes, s, a);
+    else
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8>), grid, dim3(kThreads), lds_bytes, s, a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+size_t sim_grad_input_workspace_bytes(const SimPlan &p)
+{
+    if (!gx_all_phases_fit(p))
+        return 0;
+    size_t total = 0;
+    for (int ry = 0; ry < p.sh; ++ry)
+        for (int rx = 0; rx < p.sw; ++rx) {
+            const Phase f = make_phase(p, ry, rx);
+            if (!f.empty())
+                total += gx_phase_param_bytes(p, f);
+        }
+    return total;
+}
+
+int sim_grad_input(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                          const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
+                          void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const bool l1 = p.mode == SIM_MODE_L1;
+    const bool norm = p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+    const float scale = norm ? 1.0f : 2.0f;  // the normalized functor halves the plain L2 one
+    const int ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+    const long long n_in = (long long)p.B * p.C * p.H * p.W;
+
+    if (!gx_all_phases_fit(p)) {
+        const int blocks = (int)std::min<long long>((n_in + 255) / 256, 1 << 20);
+        hipLaunchKernelGGL(sim_grad_input_gather_kernel, dim3(blocks), dim3(256), 0, s, output_grad, input, templates,
+                           weights, input_grad, p.B, p.C, p.H, p.W, p.O, p.oh, p.ow, p.bh, p.bw, p.sh, p.sw, p.ph,
+                           p.pw, (int)l1, scale, ignore_nan);
+        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
+    if (workspace_bytes < sim_grad_input_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+
+    // pixels of a phase without taps (stride larger than the block) are written by no launch
+    if (p.sh > p.bh || p.sw > p.bw) {
+        const int blocks = (int)std::min<long long>((n_in + 255) / 256, 65535);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(blocks), dim3(256), 0, s, input_grad, n_in);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+    }
+
+    char *ws = reinterpret_cast<char *>(workspace);
+    for (int ry = 0; ry < p.sh; ++ry)
+        for (int rx = 0; rx < p.sw; ++rx) {
+            const Phase f = make_phase(p, ry, rx);
+            if (f.empty())
+                continue;
+            const GxTiling t = gx_tiling(p, f);
+            const int n_ctiles = (p.C + t.MT - 1) / t.MT;
+            const int K = p.O * f.nI * f.nJ;
+            float *pb = reinterpret_cast<float *>(ws);
+            ws += gx_phase_param_bytes(p, f);
+
+            const long long total = (long long)n_ctiles * (K + 1) * t.MT;
+            const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
+            hipLaunchKernelGGL(sim_grad_input_pack_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights,
+                               p.O, p.C, p.bh, p.bw, p.sh, p.sw, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, (int)l1, scale,
+                               pb);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+
+            GradXArgs a;
+            a.g = output_grad; a.x = input; a.dx = input_grad; a.pb = pb;
+            a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
+            a.nI = f.nI; a.nJ = f.nJ;
+            a.padh = f.nI - 1 - f.a0; a.padw = f.nJ - 1 - f.b0;
+            a.na = f.na; a.nb = f.nb;
+            a.y0 = p.sh * f.a0 + ry - p.ph; a.x0 = p.sw * f.b0 + rx - p.pw;
+            a.sh = p.sh; a.sw = p.sw;
+            a.K = K;
+            a.G = t.G; a.gpi = t.gpi; a.tiles = t.tiles; a.nws = t.nws;
+            a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
+            a.n_ctiles = n_ctiles; a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC;
+            a.ignore_nan = ignore_nan;
+            // phase row h (a = a0 + h) is covered by some window iff a - (nI-1) <= oh-1
+            a.row_limit = p.oh - 1 + f.nI - 1 - f.a0;
+            a.col_limit = p.ow - 1 + f.nJ - 1 - f.b0;
+            const hipError_t e = l1 ? gx_launch_phase<GX_L1>(a, t, s) : gx_launch_phase<GX_L2>(a, t, s);
+            if (e != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
+    return SIMNETS_OK;
+}
+
+// ------------------------------------------------------------------------------------------------
+// parameter gradients
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr int PC = 64;        // output pixels per LDS chunk
+constexpr int LO = 8, LK = 4; // templates x patch elements per lane
+
+struct GradPArgs {
+    const float *g, *x, *templates;
+    float *partial;    // [nacc][S][Opad][Kpad]
+    int B, C, H, W, O, oh, ow, bh, bw, sh, sw, ph, pw, K;
+    int Opad, Kpad;    // O, K rounded up to the workgroup tile
+    int n_ktiles;
+    long long npix;    // B*oh*ow
+    int nchunks, cps;  // pixel chunks in total, and per split
+    int S;
+    float oob;
+};
+
+// MODE: SimMode of the forward op.  WO: waves along the templates (1 or 2).
+template <int MODE, int WO>
+__global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const GradPArgs a)
+{
+    constexpr int WK = kWaves / WO;
+    constexpr int OWG = WO * 64, KWG = WK * 32;
+    constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
+    constexpr bool IGN = MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
+    constexpr bool L1 = MODE == SIM_MODE_L1;
+    __shared__ __attribute__((aligned(16))) float gs[OWG / 4 * PC * 4];
+    __shared__ __attribute__((aligned(16))) float xs[KWG / 4 * PC * 4];
+    __shared__ int ktab[KWG * 2];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wo = wave % WO, wk = wave / WO;
+    const int lo = lane & 7, lk = lane >> 3;
+    const int ktile = blockIdx.x % a.n_ktiles, otile = blockIdx.x / a.n_ktiles;
+    const int o_wg = otile * OWG, k_wg = ktile * KWG;
+    const int split = blockIdx.y;
+
+    // patch element k -> offset inside an image and tap coordinates
+    const int bhw = a.bh * a.bw;
+    for (int kk = tid; kk < KWG; kk += kThreads) {
+        const int k = k_wg + kk;
+        const int c = k / bhw;
+        const int rem = k - c * bhw;
+        const int i = rem / a.bw, j = rem - i * a.bw;
+        ktab[2 * kk] = k < a.K ? (c * a.H + i) * a.W + j : -1;
+        ktab[2 * kk + 1] = (i << 16) | j;
+    }
+
+    // this lane's templates
+    const int o0 = o_wg + wo * 64 + lo * LO;
+    const int k0 = k_wg + wk * 32 + lk * LK;
+    float t[LO][LK], at[LO][LK], aw[LO][LK], an[NORM ? LO : 1][NORM ? LK : 1];
+#pragma unroll
+    for (int oo = 0; oo < LO; ++oo)
+#pragma unroll
+        for (int kk = 0; kk < LK; ++kk) {
+            const bool ok = o0 + oo < a.O && k0 + kk < a.K;
+            t[oo][kk] = ok ? a.templates[(size_t)(o0 + oo) * a.K + k0 + kk] : 0.0f;
+            at[oo][kk] = 0.0f;
+            aw[oo][kk] = 0.0f;
+            if constexpr (NORM)
+                an[oo][kk] = 0.0f;
+        }
+
+    const int ohow = a.oh * a.ow;
+    const int sp = tid & 63, sg = tid >> 6;   // staging role: pixel sp of the chunk, every 4th group
+    const float4 *g4 = reinterpret_cast<const float4 *>(gs) + (wo * 16 + lo * 2) * PC;
+    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (wk * 8 + lk) * PC;
+
+    const int chunk_end = min((split + 1) * a.cps, a.nchunks);
+    for (int chunk = split * a.cps; chunk < chunk_end; ++chunk) {
+        __syncthreads();  // previous chunk consumed (and ktab written, first time round)
+        {
+            const long long q = (long long)chunk * PC + sp;
+            const bool qok = q < a.npix;
+            const long long qq = qok ? q : 0;
+            const int b = (int)(qq / ohow);
+            const int pix = (int)(qq - (long long)b * ohow);
+            const int yo = pix / a.ow, xo = pix - yo * a.ow;
+            // g: [o/4][pixel][4]
+            const float *gb = a.g + ((size_t)b * a.O) * ohow + pix;
+            float4 gv[OWG / 16];
+#pragma unroll
+            for (int r = 0; r < OWG / 16; ++r) {
+                const int o = o_wg + (sg + 4 * r) * 4;
+                float e[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u)
+                    e[u] = (qok && o + u < a.O) ? gb[(size_t)(o + u) * ohow] : 0.0f;
+                gv[r] = make_float4(e[0], e[1], e[2], e[3]);
+            }
+            // patch elements: [k/4][pixel][4], the im2col_3d rule (outside the image -> oob)
+            const int iy0 = yo * a.sh - a.ph, ix0 = xo * a.sw - a.pw;
+            const float *xb = a.x + (size_t)b * a.C * a.H * a.W + (ptrdiff_t)iy0 * a.W + ix0;
+            float4 xv[KWG / 16];
+#pragma unroll
+            for (int r = 0; r < KWG / 16; ++r) {
+                const int kk = (sg + 4 * r) * 4;
+                float e[4];
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int kofs = ktab[2 * (kk + u)], ij = ktab[2 * (kk + u) + 1];
+                    const int iy = iy0 + (ij >> 16), ix = ix0 + (ij & 0xffff);
+                    float val = 0.0f;
+                    if (qok && kofs >= 0) {
+                        val = a.oob;
+                        if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W)
+                            val = xb[kofs];
+                    }
+                    e[u] = val;
+                }
+                xv[r] = make_float4(e[0], e[1], e[2], e[3]);
+            }
+#pragma unroll
+            for (int r = 0; r < OWG / 16; ++r)
+                reinterpret_cast<float4 *>(gs)[(sg + 4 * r) * PC + sp] = gv[r];
+#pragma unroll
+            for (int r = 0; r < KWG / 16; ++r)
+                reinterpret_cast<float4 *>(xs)[(sg + 4 * r) * PC + sp] = xv[r];
+        }
+        __syncthreads();
+
+        auto compute = [&](const float4 &ga, const float4 &gb2, const float4 &xq) {
+            const float gl[LO] = {ga.x, ga.y, ga.z, ga.w, gb2.x, gb2.y, gb2.z, gb2.w};
+            float xl[LK] = {xq.x, xq.y, xq.z, xq.w};
+            float keep[LK];
+            if (IGN) {
+#pragma unroll
+                for (int kk = 0; kk < LK; ++kk) {
+                    const bool ok = xl[kk] == xl[kk];
+                    keep[kk] = ok ? 1.0f : 0.0f;
+                    xl[kk] = ok ? xl[kk] : 0.0f;
+                }
+            }
+#pragma unroll
+            for (int oo = 0; oo < LO; ++oo) {
+                float d[LK], e[LK], gg[LK];
+#pragma unroll
+                for (int kk = 0; kk < LK; ++kk) {
+                    d[kk] = xl[kk] - t[oo][kk];
+                    gg[kk] = IGN ? gl[oo] * keep[kk] : gl[oo];
+                }
+                if (L1) {
+#pragma unroll
+                    for (int kk = 0; kk < LK; ++kk) {
+                        float sgn = d[kk] < 0.0f ? -gg[kk] : gg[kk];
+                        sgn = __builtin_islessgreater(d[kk], 0.0f) ? sgn : 0.0f;
+                        at[oo][kk] += sgn;
+                        aw[oo][kk] = __builtin_fmaf(gg[kk], __builtin_fabsf(d[kk]), aw[oo][kk]);
+                    }
+                } else {
+#pragma unroll
+                    for (int kk = 0; kk < LK; ++kk)
+                        e[kk] = gg[kk] * d[kk];
+#pragma unroll
+                    for (int kk = 0; kk < LK; ++kk) {
+                        at[oo][kk] += e[kk];
+                        aw[oo][kk] = __builtin_fmaf(e[kk], d[kk], aw[oo][kk]);
+                        if constexpr (NORM)
+                            an[oo][kk] += gg[kk];
+                    }
+                }
+            }
+        };
+        // one pixel ahead: the three reads of pixel p+1 are issued before the arithmetic of pixel p
+        float4 ga = g4[0], gb2 = g4[PC], xq = x4[0];
+        for (int p = 0; p < PC; p += 2) {
+            const float4 ga1 = g4[p + 1], gb1 = g4[PC + p + 1], xq1 = x4[p + 1];
+            compute(ga, gb2, xq);
+            const int pn = p + 2 < PC ? p + 2 : p;
+            ga = g4[pn]; gb2 = g4[PC + pn]; xq = x4[pn];
+            compute(ga1, gb1, xq1);
+        }
+    }
+
+    // partial sums of this split
+    const size_t slab = (size_t)a.Opad * a.Kpad;
+    float *pt = a.partial + (size_t)split * slab;
+    float *pw = a.partial + ((size_t)a.S + split) * slab;
+    float *pn = a.partial + ((size_t)2 * a.S + split) * slab;
+#pragma unroll
+    for (int oo = 0; oo < LO; ++oo) {
+        const size_t o = (size_t)(o0 + oo) * a.Kpad + k0;
+        *reinterpret_cast<float4 *>(pt + o) = make_float4(at[oo][0], at[oo][1], at[oo][2], at[oo][3]);
+        *reinterpret_cast<float4 *>(pw + o) = make_float4(aw[oo][0], aw[oo][1], aw[oo][2], aw[oo][3]);
+        if constexpr (NORM)
+            *reinterpret_cast<float4 *>(pn + o) = make_float4(an[oo][0], an[oo][1], an[oo][2], an[oo][3]);
+    }
+}
+
+// Adds the partial sums in split order and applies the pixel-independent factors.
+__global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial, const float *__restrict__ weights,
+                                              int O, int K, int Opad, int Kpad, int S, int mode, float fudge,
+                                              float *__restrict__ dT, float *__restrict__ dW)
+{
+    const long long total = (long long)O * K;
+    const size_t slab = (size_t)Opad * Kpad;
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long long)gridDim.x * blockDim.x) {
+        const int k = (int)(idx % K);
+        const int o = (int)(idx / K);
+        const size_t src = (size_t)o * Kpad + k;
+        float st = 0.0f, sw = 0.0f, sn = 0.0f;
+        const bool norm = mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+        for (int s = 0; s < S; ++s) {
+            st += partial[(size_t)s * slab + src];
+            sw += partial[((size_t)S + s) * slab + src];
+            if (norm)
+                sn += partial[((size_t)2 * S + s) * slab + src];
+        }
+        const float w = weights[idx];
+        if (mode == SIM_MODE_L1) {
+            dT[idx] = w * st;
+            dW[idx] = -sw;
+        } else if (!norm) {
+            dT[idx] = 2.0f * w * st;
+            dW[idx] = -sw;
+        } else {
+            dT[idx] = w * st;
+            dW[idx] = 0.5f * (sn / (w + fudge) - sw);
+        }
+    }
+}
+
+struct GpTiling {
+    int WO, OWG, KWG, n_otiles, n_ktiles, Opad, Kpad, nchunks, cps, S, nacc;
+};
+
+GpTiling gp_tiling(const SimPlan &p)
+{
+    GpTiling t;
+    t.WO = p.O > 64 ? 2 : 1;
+    t.OWG = t.WO * 64;
+    t.KWG = (kWaves / t.WO) * 32;
+    t.n_otiles = (p.O + t.OWG - 1) / t.OWG;
+    t.n_ktiles = (p.K + t.KWG - 1) / t.KWG;
+    t.Opad = t.n_otiles * t.OWG;
+    t.Kpad = t.n_ktiles * t.KWG;
+    const long long npix = (long long)p.B * p.oh * p.ow;
+    t.nchunks = (int)((npix + PC - 1) / PC);
+    const int tiles = t.n_otiles * t.n_ktiles;
+    int S = std::max(1, 1024 / tiles);
+    S = std::min(S, std::max(1, t.nchunks));
+    t.cps = (t.nchunks + S - 1) / S;
+    t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
+    t.nacc = (p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
+    return t;
+}
+
+template <int MODE>
+hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
+{
+    dim3 grid((unsigned)(t.n_otiles * t.n_ktiles), (unsigned)t.S);
+    if (t.WO == 2)
+        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2>), grid, dim3(kThreads), 0, s, a);
+    else
+        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1>), grid, dim3(kThreads), 0, s, a);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+size_t sim_grad_params_workspace_bytes(const SimPlan &p)
+{
+    const GpTiling t = gp_tiling(p);
+    return align_up((size_t)t.nacc * t.S * t.Opad * t.Kpad * sizeof(float), 256);
+}
+
+int sim_grad_params(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                    const float *output_grad, float *templates_grad, float *weights_grad, void *workspace,
+                    size_t workspace_bytes, void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (workspace_bytes < sim_grad_params_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+    const GpTiling t = gp_tiling(p);
+    if (p.bh > 0xffff || p.bw > 0xffff || t.S > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    GradPArgs a;
+    a.g = output_grad; a.x = input; a.templates = templates;
+    a.partial = reinterpret_cast<float *>(workspace);
+    a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
+    a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.K = p.K;
+    a.Opad = t.Opad; a.Kpad = t.Kpad; a.n_ktiles = t.n_ktiles;
+    a.npix = (long long)p.B * p.oh * p.ow;
+    a.nchunks = t.nchunks; a.cps = t.cps; a.S = t.S;
+    a.oob = p.oob;
+    hipError_t e;
+    switch (p.mode) {
+    case SIM_MODE_L1: e = gp_launch<SIM_MODE_L1>(a, t, s); break;
+    case SIM_MODE_L2: e = gp_launch<SIM_MODE_L2>(a, t, s); break;
+    case SIM_MODE_L2_NORM: e = gp_launch<SIM_MODE_L2_NORM>(a, t, s); break;
+    default: e = gp_launch<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, s); break;
+    }
+    if (e != hipSuccess)
+        return SIMNETS_ERR_HIP;
+    const long long total = (long long)p.O * p.K;
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
+    hipLaunchKernelGGL(sim_grad_params_finish_kernel, dim3(blocks), dim3(256), 0, s, a.partial, weights, p.O, p.K,
+                       t.Opad, t.Kpad, t.S, p.mode, p.fudge, templates_grad, weights_grad);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+}  // namespace simnets

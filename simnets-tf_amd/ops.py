@@ -129,6 +129,65 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
     return out
 
 
+def _similarity_grad_setup(input, templates, weights, output_grad, kw):
+    x = _require_cuda_f32("input", input)
+    t = _require_cuda_f32("templates", templates)
+    w = _require_cuda_f32("weights", weights)
+    g = _require_cuda_f32("output_grad", output_grad)
+    if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
+        raise SimnetsError(-15)
+    a = similarity_attrs(**kw)
+    l = _lib.lib()
+    I4 = C.c_int * 4
+    xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
+    oshape = I4()
+    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
+    if tuple(g.shape) != tuple(oshape):
+        raise SimnetsError(-15)
+    return l, a, x, t, w, g, xs, ts, wsh
+
+
+def similarity_input_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None, strides=None,
+                          padding=None, normalization_term=None, normalization_term_fudge=None,
+                          ignore_nan_input=None, out_of_bounds_value=None, name=None):
+    """Gradient of `similarity` w.r.t. its input: the SimilarityInputGrad op
+    (python/simnets/ops/similarity.py:33-37, src/ops/similarity_op.cpp:141-156)."""
+    l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
+        similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+        normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes), None))
+    ws = _workspace(x.device, nbytes.value)
+    dx = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_similarity_input_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
+                                                   g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return dx
+
+
+def similarity_parameters_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None,
+                               strides=None, padding=None, normalization_term=None, normalization_term_fudge=None,
+                               ignore_nan_input=None, out_of_bounds_value=None, name=None):
+    """Gradients of `similarity` w.r.t. templates and weights: the SimilarityParametersGrad op
+    (python/simnets/ops/similarity.py:38-44, src/ops/similarity_op.cpp:158-174)."""
+    l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
+        similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+        normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, None, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    dt, dw = torch.empty_like(t), torch.empty_like(w)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_similarity_params_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(),
+                                                    w.data_ptr(), g.data_ptr(), dt.data_ptr(), dw.data_ptr(),
+                                                    ws.data_ptr(), ws.numel(), stream))
+    return dt, dw
+
+
 def mex_attrs(num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
               blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
               shared_offset_region=None, unshared_offset_region=None, normalize_offsets=False):
@@ -242,6 +301,67 @@ def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=
         _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
                                      ws.data_ptr(), ws.numel(), stream))
     return out
+
+
+def _mex_grad_setup(input, offsets, output, output_grad, num_instances, kw):
+    x = _require_cuda_f32("input", input)
+    off = _require_cuda_f32("offsets", offsets)
+    y = _require_cuda_f32("output", output)
+    g = _require_cuda_f32("output_grad", output_grad)
+    if x.dim() != 4:
+        raise SimnetsError(-15)
+    a = mex_attrs(num_instances, **kw)
+    l = _lib.lib()
+    xs = (C.c_int * 4)(*x.shape)
+    oshape = (C.c_int * 4)()
+    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+    if tuple(y.shape) != tuple(oshape) or tuple(g.shape) != tuple(oshape):
+        raise SimnetsError(-15)
+    return l, a, x, off, y, g, xs
+
+
+def mex_input_grad(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
+                   blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+                   use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+                   normalize_offsets=False):
+    """Gradient of `mex` w.r.t. its input: the MexInputGrad op (python/simnets/ops/mex.py:63-71,
+    src/ops/mex_op.cpp:134-151).  `output` is the forward result."""
+    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
+        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
+        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
+        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
+        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, C.byref(nbytes), None))
+    ws = _workspace(x.device, nbytes.value)
+    dx = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_mex_input_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
+                                            g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return dx
+
+
+def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None,
+                     strides=None, blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+                     use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+                     normalize_offsets=False):
+    """Gradient of `mex` w.r.t. its offsets: the MexOffsetsGrad op (python/simnets/ops/mex.py:73-80,
+    src/ops/mex_op.cpp:153-170).  With `normalize_offsets` the gradient is w.r.t. the raw offsets."""
+    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
+        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
+        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
+        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
+        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, None, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    doff = torch.empty_like(off)
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_mex_offsets_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
+                                              g.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return doff
 
 
 def sum_pooling(input, pool_size=(2, 2), out=None):

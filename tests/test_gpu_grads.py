@@ -1,0 +1,305 @@
+"""GPU parity of the backward operators: the HIP library (through the C ABI via the op layer) against the
+CPU oracle's restatement of the reference grad kernels on the same seeded inputs, to 1e-4.
+
+Gradients are sums of many signed terms and cross zero, so
+  * the error of an element is taken relative to max(|want|, 1e-2 * max|want|): element-wise for
+    everything above a hundredth of the tensor's scale, relative to that hundredth below it (the
+    rounding noise of an fp32 sum is proportional to the magnitude of its terms, not of its value);
+  * it is measured against the oracle's fp64 instantiation (the exact value of the sum), and the bar
+    is 1e-4 or twice the error the reference's own fp32 arithmetic (the oracle's fp32 instantiation)
+    makes on the same inputs, whichever is larger: where the sum cancels, no fp32 summation order
+    is closer to another than both are to the exact value.
+"""
+import itertools
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from util import config1, config2, config3, rel_err
+
+pytestmark = pytest.mark.gpu
+
+GRAD_TOL = 1e-4
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def grad_err(got, want):
+    want = np.asarray(want)
+    scale = float(np.abs(want[np.isfinite(want)]).max()) if np.isfinite(want).any() else 0.0
+    return rel_err(got, want, floor=np.full(want.shape, 1e-2 * scale))
+
+
+def assert_grad_close(got, want32, want64, what):
+    e_gpu, e_ref = grad_err(got, want64), grad_err(want32, want64)
+    assert e_gpu <= max(GRAD_TOL, 2.0 * e_ref), "%s: gpu %.3g, fp32 reference %.3g" % (what, e_gpu, e_ref)
+
+
+def f64(*arrays):
+    return [np.asarray(a, dtype=np.float64) for a in arrays]
+
+
+def sim_grads_gpu(pkg, x, t, w, g, **kw):
+    dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(g), **kw)
+    dt, dw = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(g), **kw)
+    torch.cuda.synchronize()
+    return dx.cpu().numpy(), dt.cpu().numpy(), dw.cpu().numpy()
+
+
+def check_sim_grads(pkg, x, t, w, seed=99, **kw):
+    out = orc.similarity_fwd(x, t, w, **kw)
+    g = np.random.default_rng(seed).normal(size=out.shape).astype(np.float32)
+    dx, dt, dw = sim_grads_gpu(pkg, x, t, w, g, **kw)
+    want_dx = orc.similarity_input_grad(x, t, w, g, **kw)
+    want_dt, want_dw = orc.similarity_params_grad(x, t, w, g, **kw)
+    d = f64(x, t, w, g)
+    true_dx = orc.similarity_input_grad(*d, **kw)
+    true_dt, true_dw = orc.similarity_params_grad(*d, **kw)
+    assert_grad_close(dx, want_dx, true_dx, "input grad")
+    assert_grad_close(dt, want_dt, true_dt, "templates grad")
+    assert_grad_close(dw, want_dw, true_dw, "weights grad")
+
+
+# ---- the reference's own gradient test matrix (python/simnets/test/__init__.py:55-103, :143-154) ------------
+@pytest.mark.parametrize("strides", [[1, 1], [2, 2]])
+@pytest.mark.parametrize("blocks", [[1, 1], [3, 3]])
+@pytest.mark.parametrize("func,norm,ign", [("L2", True, False), ("L2", True, True), ("L1", False, False),
+                                           ("L2", False, False)])
+@pytest.mark.parametrize("O", [1, 5])
+def test_similarity_grads_reference_matrix(pkg, strides, blocks, func, norm, ign, O):
+    g = np.random.default_rng(167)
+    x = (16.0 + g.normal(size=(1, 3, 10, 10))).astype(np.float32)
+    w = (3.0 + np.abs(g.normal(size=(O, 3) + tuple(blocks)))).astype(np.float32)
+    t = (3.0 + g.normal(size=w.shape)).astype(np.float32)
+    kw = dict(similarity_function=func, blocks=blocks, strides=strides, padding=[0, 0], normalization_term=norm,
+              ignore_nan_input=ign)
+    check_sim_grads(pkg, x, t, w, **kw)
+
+
+def sim_inputs(seed, shape, O, blocks, nan_frac=0.0):
+    g = np.random.default_rng(seed)
+    x = g.normal(size=shape).astype(np.float32)
+    t = g.normal(size=(O, shape[1]) + tuple(blocks)).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    if nan_frac:
+        x[g.random(size=x.shape) < nan_frac] = np.nan
+    return x, t, w
+
+
+@pytest.mark.parametrize("func", ["L2", "L1"])
+@pytest.mark.parametrize("case", [
+    dict(shape=(2, 3, 20, 21), O=7, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),
+    dict(shape=(2, 3, 20, 21), O=7, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),       # phases with 1 and 2 taps
+    dict(shape=(2, 3, 50, 31), O=7, blocks=[3, 2], strides=[1, 2], padding=[0, 1]),
+    dict(shape=(1, 2, 9, 70), O=33, blocks=[5, 5], strides=[3, 3], padding=[2, 2]),
+    dict(shape=(2, 2, 11, 13), O=3, blocks=[2, 2], strides=[3, 4], padding=[0, 1]),       # stride > block: uncovered pixels
+    dict(shape=(2, 1, 28, 28), O=3, blocks=[28, 28], strides=[1, 1], padding=[0, 0]),     # one output pixel
+    dict(shape=(3, 4, 12, 200), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # wide rows
+    dict(shape=(1, 130, 6, 6), O=17, blocks=[2, 2], strides=[1, 1], padding=[1, 1]),      # many channels
+    dict(shape=(2, 40, 34, 34), O=130, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),    # big lane tile, ragged O
+    dict(shape=(2, 2, 5, 5), O=2, blocks=[2, 2], strides=[4, 5], padding=[3, 3]),         # padding beyond the block
+    dict(shape=(1, 1, 7, 7), O=1, blocks=[2, 2], strides=[2, 2], padding=[0, 0]),         # last row/column never covered
+    dict(shape=(1, 2, 6, 700), O=4, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),       # rows too wide for the LDS tile
+])
+def test_similarity_grads_geometries(pkg, case, func):
+    x, t, w = sim_inputs(5, case["shape"], case["O"], case["blocks"])
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+              out_of_bounds_value=0.25)
+    check_sim_grads(pkg, x, t, w, **kw)
+
+
+@pytest.mark.parametrize("nan_frac", [0.0, 0.25, 1.0])
+@pytest.mark.parametrize("blocks,strides,padding", [([2, 2], [2, 2], [2, 2]), ([3, 3], [1, 1], [1, 1]),
+                                                    ([3, 3], [2, 1], [1, 0])])
+def test_similarity_grads_ignore_nan(pkg, nan_frac, blocks, strides, padding):
+    x, t, w = sim_inputs(6, (3, 2, 14, 15), 6, blocks, nan_frac=nan_frac)
+    kw = dict(similarity_function="L2", blocks=blocks, strides=strides, padding=padding, normalization_term=True,
+              ignore_nan_input=True, out_of_bounds_value=float("nan"))
+    check_sim_grads(pkg, x, t, w, **kw)
+
+
+def test_similarity_grads_nan_input_without_ignore_propagates_like_the_reference(pkg):
+    x, t, w = sim_inputs(7, (1, 2, 8, 8), 3, (3, 3))
+    x[0, 1, 4, 4] = np.nan
+    check_sim_grads(pkg, x, t, w, similarity_function="L2", blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+
+
+def test_similarity_grads_first_layer_of_the_missing_data_network(pkg):
+    x, t, w, kw = config1(batch=8, nan_frac=0.25)
+    check_sim_grads(pkg, x, t, w, **kw)
+
+
+@pytest.mark.parametrize("func", ["L2", "L1"])
+def test_similarity_grads_conv_scale_shape_small_batch(pkg, func):
+    x, t, w, kw = config3(batch=3)
+    check_sim_grads(pkg, x, t, w, similarity_function=func, **kw)
+
+
+def test_similarity_grads_conv_scale_full_batch_properties(pkg):
+    """Full config-3 batch: the input gradient of an image depends on that image only (checked against the
+    oracle on two images), and the parameter gradients are additive over the batch (sum of two half-batch
+    calls) and linear in the output gradient."""
+    x, t, w, kw = config3()
+    g = np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32)
+    X, T, W, G = dev(x), dev(t), dev(w), dev(g)
+    dx = pkg.similarity_input_grad(X, T, W, G, **kw)
+    dt, dw = pkg.similarity_parameters_grad(X, T, W, G, **kw)
+    for b in (0, 255):
+        want = orc.similarity_input_grad(x[b:b + 1], t, w, g[b:b + 1], **kw)
+        true = orc.similarity_input_grad(*f64(x[b:b + 1], t, w, g[b:b + 1]), **kw)
+        assert_grad_close(dx[b:b + 1].cpu().numpy(), want, true, "input grad of image %d" % b)
+    dt1, dw1 = pkg.similarity_parameters_grad(X[:128], T, W, G[:128], **kw)
+    dt2, dw2 = pkg.similarity_parameters_grad(X[128:], T, W, G[128:], **kw)
+    assert grad_err((dt1 + dt2).cpu().numpy(), dt.cpu().numpy()) <= GRAD_TOL
+    assert grad_err((dw1 + dw2).cpu().numpy(), dw.cpu().numpy()) <= GRAD_TOL
+    dt3, dw3 = pkg.similarity_parameters_grad(X, T, W, 2.0 * G, **kw)
+    assert torch.equal(dt3, 2.0 * dt) and torch.equal(dw3, 2.0 * dw)      # scaling by 2 is exact in fp32
+    want_dt, want_dw = orc.similarity_params_grad(x[:2], t, w, g[:2], **kw)
+    true_dt, true_dw = orc.similarity_params_grad(*f64(x[:2], t, w, g[:2]), **kw)
+    dt4, dw4 = pkg.similarity_parameters_grad(X[:2], T, W, G[:2], **kw)
+    assert_grad_close(dt4.cpu().numpy(), want_dt, true_dt, "templates grad")
+    assert_grad_close(dw4.cpu().numpy(), want_dw, true_dw, "weights grad")
+
+
+def test_similarity_params_grad_is_reproducible(pkg):
+    x, t, w, kw = config3(batch=16)
+    g = np.random.default_rng(1).normal(size=(16, 128, 32, 32)).astype(np.float32)
+    a = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(g), **kw)
+    b = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(g), **kw)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_similarity_grads_empty_batch(pkg):
+    x, t, w = sim_inputs(8, (0, 3, 9, 9), 4, (3, 3))
+    g = np.zeros((0, 4, 7, 7), np.float32)
+    dx, dt, dw = sim_grads_gpu(pkg, x, t, w, g, blocks=[3, 3], strides=[1, 1], padding=[0, 0])
+    assert dx.shape == x.shape and not dt.any() and not dw.any()
+
+
+def test_similarity_grads_reject_wrong_output_grad_shape(pkg):
+    x, t, w = sim_inputs(9, (1, 3, 9, 9), 4, (3, 3))
+    with pytest.raises(pkg.SimnetsError):
+        pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(np.zeros((1, 4, 9, 9), np.float32)), blocks=[3, 3],
+                                  strides=[1, 1], padding=[0, 0])
+
+
+# ---- MEX ------------------------------------------------------------------------------------------
+def mex_case(seed, im_dims, num_instances, **kw):
+    g = np.random.default_rng(seed)
+    d = orc.mex_dims(orc.mex_args(im_dims, num_instances, **kw))
+    x = g.normal(size=im_dims).astype(np.float32)
+    off = g.normal(size=(d.num_regions, num_instances) + tuple(kw["blocks"])).astype(np.float32)
+    return x, off
+
+
+def check_mex_grads(pkg, x, off, n, seed=77, **kw):
+    out = orc.mex_fwd(x, off, n, **kw)
+    g = np.random.default_rng(seed).normal(size=out.shape).astype(np.float32)
+    X, O, Y, G = dev(x), dev(off), dev(out), dev(g)
+    dx = pkg.mex_input_grad(X, O, Y, G, n, **kw).cpu().numpy()
+    doff = pkg.mex_offsets_grad(X, O, Y, G, n, **kw).cpu().numpy()
+    x64, off64, g64 = f64(x, off, g)
+    out64 = orc.mex_fwd(x64, off64, n, **kw)
+    assert_grad_close(dx, orc.mex_input_grad(x, off, out, g, n, **kw), orc.mex_input_grad(x64, off64, out64, g64, n, **kw),
+                      "input grad")
+    assert_grad_close(doff, orc.mex_offsets_grad(x, off, out, g, n, **kw),
+                      orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "offsets grad")
+
+
+# the reference's gradient tests (python/simnets/test/__init__.py:329-372)
+@pytest.mark.parametrize("unshared", [True, False])
+@pytest.mark.parametrize("shared_spec", [[1, 5, 4], [2], [-1]])
+@pytest.mark.parametrize("unshared_spec", [[1, 5, 4], [2], [-1]])
+def test_mex_grads_reference_matrix(pkg, unshared, shared_spec, unshared_spec):
+    kw = dict(blocks=[3, 3, 1], strides=[1, 1, 2], padding=[0, 1, 0], softmax_mode=True, use_unshared_regions=unshared,
+              shared_offset_region=shared_spec, unshared_offset_region=unshared_spec)
+    x, off = mex_case(11, (2, 3, 12, 13), 2, **kw)
+    check_mex_grads(pkg, x, off, 2, **kw)
+
+
+def test_mex_grads_reference_blocks_bug_case(pkg):
+    kw = dict(blocks=[3, 8, 8], strides=[1, 1, 2], padding=[0, 4, 4], softmax_mode=True, use_unshared_regions=True,
+              shared_offset_region=[3, 3, 3], unshared_offset_region=[2])
+    x, off = mex_case(12, (2, 3, 16, 16), 2, **kw)
+    check_mex_grads(pkg, x, off, 2, **kw)
+
+
+@pytest.mark.parametrize("eps", [1.0, -1.0, 2.5, -0.3, math.inf, -math.inf])
+@pytest.mark.parametrize("softmax", [True, False])
+def test_mex_grads_epsilon(pkg, eps, softmax):
+    kw = dict(blocks=[2, 3, 3], strides=[1, 2, 2], padding=[0, 1, 1], epsilon=eps, softmax_mode=softmax,
+              shared_offset_region=[1, 2, 3], use_unshared_regions=False)
+    x, off = mex_case(13, (3, 5, 11, 10), 5, **kw)
+    check_mex_grads(pkg, x, off, 5, **kw)
+
+
+@pytest.mark.parametrize("case", [
+    dict(im=(2, 6, 9, 9), n=20, kw=dict(blocks=[6, 1, 1], strides=[6, 1, 1], padding=[0, 0, 0], unshared_offset_region=[2])),
+    dict(im=(3, 4, 7, 6), n=3, kw=dict(blocks=[2, 2, 2], strides=[2, 2, 2], padding=[0, 0, 0], use_unshared_regions=False,
+                                      shared_offset_region=[-1])),                       # one region, ragged tiling
+    dict(im=(2, 3, 6, 6), n=2, kw=dict(blocks=[2, 3, 2], strides=[1, 2, 2], padding=[1, 1, 0], blocks_round_down=False,
+                                      blocks_out_of_bounds_value=-0.7, use_unshared_regions=False,
+                                      shared_offset_region=[1, 2, 2])),                  # channel padding, round up
+    dict(im=(2, 3, 5, 5), n=2, kw=dict(blocks=[3, 1, 1], strides=[3, 1, 1], padding=[0, 0, 0])),   # one region per pixel
+    dict(im=(130, 70, 2, 2), n=9, kw=dict(blocks=[70, 1, 1], strides=[70, 1, 1], padding=[0, 0, 0],
+                                        unshared_offset_region=[2])),                   # long K, many images
+    dict(im=(2, 8, 8, 8), n=4, kw=dict(blocks=[1, 2, 2], strides=[1, 3, 3], padding=[0, 0, 0], use_unshared_regions=False,
+                                      shared_offset_region=[2])),                        # stride > block: uncovered input
+])
+def test_mex_grads_geometries(pkg, case):
+    x, off = mex_case(14, case["im"], case["n"], **case["kw"])
+    check_mex_grads(pkg, x, off, case["n"], **case["kw"])
+
+
+def test_mex_grads_config2_shape(pkg):
+    x, off, n, kw = config2(batch=8)
+    off = orc.normalize_offsets(off)
+    check_mex_grads(pkg, x, off, n, **kw)
+
+
+def test_mex_offsets_grad_through_the_offset_normalisation(pkg):
+    """normalize_offsets=True returns d/d(raw offsets): G - softmax(raw) * sum_k G, with G the gradient the
+    reference op would return for the normalised offsets."""
+    x, off, n, kw = config2(batch=4, channels=16, size=6, instances=8)
+    norm = orc.normalize_offsets(off)
+    out = orc.mex_fwd(x, norm, n, **kw)
+    g = np.random.default_rng(3).normal(size=out.shape).astype(np.float32)
+    G = orc.mex_offsets_grad(x.astype(np.float64), norm.astype(np.float64), out.astype(np.float64),
+                             g.astype(np.float64), n, **kw)
+    want = G - np.exp(norm.astype(np.float64)) * G.sum(axis=(2, 3, 4), keepdims=True)
+    got = pkg.mex_offsets_grad(dev(x), dev(off), dev(out), dev(g), n, normalize_offsets=True, **kw).cpu().numpy()
+    assert grad_err(got, want) <= GRAD_TOL
+    got_dx = pkg.mex_input_grad(dev(x), dev(off), dev(out), dev(g), n, normalize_offsets=True, **kw).cpu().numpy()
+    assert grad_err(got_dx, orc.mex_input_grad(x, norm, out, g, n, **kw)) <= GRAD_TOL
+
+
+def test_mex_offsets_grad_is_reproducible_and_additive(pkg):
+    x, off, n, kw = config2(batch=64)
+    off = orc.normalize_offsets(off)
+    X, O = dev(x), dev(off)
+    Y = pkg.mex(X, O, n, **kw)
+    G = dev(np.random.default_rng(4).normal(size=tuple(Y.shape)).astype(np.float32))
+    a = pkg.mex_offsets_grad(X, O, Y, G, n, **kw)
+    b = pkg.mex_offsets_grad(X, O, Y, G, n, **kw)
+    assert torch.equal(a, b)
+    halves = pkg.mex_offsets_grad(X[:32], O, Y[:32], G[:32], n, **kw) + pkg.mex_offsets_grad(X[32:], O, Y[32:], G[32:],
+                                                                                          n, **kw)
+    assert grad_err(halves.cpu().numpy(), a.cpu().numpy()) <= GRAD_TOL
+    # softmax-mode, eps=1: the terms exp(x + off - out) of a pixel sum to 1 over k, so dX summed over the
+    # patch equals the output gradient summed over the instances
+    dx = pkg.mex_input_grad(X, O, Y, G, n, **kw)
+    assert grad_err(dx.sum(dim=1).cpu().numpy(), G.sum(dim=1).cpu().numpy()) <= GRAD_TOL
+
+
+def test_mex_grads_empty_batch(pkg):
+    kw = dict(blocks=[3, 1, 1], strides=[3, 1, 1], padding=[0, 0, 0], use_unshared_regions=False)
+    off = np.zeros((1, 2, 3, 1, 1), np.float32)
+    x = np.zeros((0, 3, 4, 4), np.float32)
+    y = np.zeros((0, 2, 4, 4), np.float32)
+    assert pkg.mex_input_grad(dev(x), dev(off), dev(y), dev(y), 2, **kw).shape == x.shape
+    assert not pkg.mex_offsets_grad(dev(x), dev(off), dev(y), dev(y), 2, **kw).cpu().numpy().any()
