@@ -2,7 +2,7 @@
 //
 //   simnets_bench --peaks                      machine micro-benchmarks (unpacked FP32 FMA issue rate,
 //                                              fp32 MFMA rate, v_exp_f32 rate, HBM copy bandwidth)
-//   simnets_bench --config N [--algo A] [--steps K] [--warmup W]
+//   simnets_bench --config N [--algo A] [--steps K] [--warmup W]     (N = 1..4 forward, 5 backward)
 //                                              N in 1..4: times that BASELINE configuration through the
 //                                              C ABI with hipEvents on its own stream
 // Prints one JSON object per measurement.  Inputs are synthetic (fixed-seed counter-based generator),
@@ -373,6 +373,56 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) stack();
         float ms = time_ms(s, steps, stack);
         report("config4 missing-data stack batch 512", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+    }
+    else if (config == 5) {
+        // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
+        for (int l1 = 0; l1 < 2; ++l1) {
+            SimCase c = make_similarity(256, 64, 32, 32, 128, 3, 3, 1, 1, false, SIMNETS_ALGO_AUTO, l1);
+            const size_t n_out = (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3];
+            std::vector<float> g(n_out);
+            fill_normal(g, 6789, 1.0f);
+            float *dg = upload(g), *dx, *dt, *dw;
+            HIP_OK(hipMalloc(&dx, (size_t)256 * 64 * 32 * 32 * sizeof(float)));
+            HIP_OK(hipMalloc(&dt, (size_t)128 * 64 * 9 * sizeof(float)));
+            HIP_OK(hipMalloc(&dw, (size_t)128 * 64 * 9 * sizeof(float)));
+            size_t wx = 0, wp = 0;
+            SN_OK(simnets_hip_similarity_grad_workspace_bytes(&c.a, c.in, c.tp, &wx, &wp));
+            void *ws;
+            HIP_OK(hipMalloc(&ws, std::max<size_t>(std::max(wx, wp), 256)));
+            auto gx = [&] { SN_OK(simnets_hip_similarity_input_grad(&c.a, c.in, c.tp, c.tp, c.x, c.t, c.w, dg, dx, ws, wx, s)); };
+            auto gp = [&] { SN_OK(simnets_hip_similarity_params_grad(&c.a, c.in, c.tp, c.tp, c.x, c.t, c.w, dg, dt, dw, ws, wp, s)); };
+            for (int i = 0; i < warmup; ++i) { gx(); gp(); }
+            float ms = time_ms(s, steps, gx);
+            // input grad: read g and x, write dx; 2 flop per term for L2 (fma, fma), 5 for L1
+            report(l1 ? "config5 similarity input grad L1 (config-3 shape)" : "config5 similarity input grad L2 (config-3 shape)",
+                   19327352832.0, (n_out + 2.0 * 256 * 64 * 32 * 32) * 4, l1 ? 5 : 4, ms, steps);
+            ms = time_ms(s, steps, gp);
+            report(l1 ? "config5 similarity params grad L1 (config-3 shape)" : "config5 similarity params grad L2 (config-3 shape)",
+                   19327352832.0, (n_out + 256.0 * 64 * 32 * 32) * 4, l1 ? 6 : 5, ms, steps);
+            HIP_OK(hipFree(dg)); HIP_OK(hipFree(dx)); HIP_OK(hipFree(dt)); HIP_OK(hipFree(dw)); HIP_OK(hipFree(ws));
+            HIP_OK(hipFree(c.x)); HIP_OK(hipFree(c.y));
+        }
+        {
+            MexCase c = make_mex(64, 32, 16, 64, false, nullptr);
+            run_mex(c, s);
+            const size_t n_out = (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3];
+            std::vector<float> g(n_out);
+            fill_normal(g, 6789, 1.0f);
+            float *dg = upload(g), *dx, *doff;
+            HIP_OK(hipMalloc(&dx, (size_t)64 * 32 * 16 * 16 * sizeof(float)));
+            HIP_OK(hipMalloc(&doff, c.off_count * sizeof(float)));
+            size_t wx = 0, wo = 0;
+            SN_OK(simnets_hip_mex_grad_workspace_bytes(&c.a, c.in, &wx, &wo));
+            void *ws;
+            HIP_OK(hipMalloc(&ws, std::max<size_t>(std::max(wx, wo), 256)));
+            auto gx = [&] { SN_OK(simnets_hip_mex_input_grad(&c.a, c.in, c.x, c.o, c.off_count, c.y, dg, dx, ws, wx, s)); };
+            auto go = [&] { SN_OK(simnets_hip_mex_offsets_grad(&c.a, c.in, c.x, c.o, c.off_count, c.y, dg, doff, ws, wo, s)); };
+            for (int i = 0; i < warmup; ++i) { gx(); go(); }
+            float ms = time_ms(s, steps, gx);
+            report("config5 mex input grad (config-2 shape)", 33554432.0, (2.0 * n_out + 2.0 * 64 * 32 * 256) * 4, 5, ms, steps);
+            ms = time_ms(s, steps, go);
+            report("config5 mex offsets grad (config-2 shape)", 33554432.0, (2.0 * n_out + 64.0 * 32 * 256) * 4, 5, ms, steps);
+        }
     }
     HIP_OK(hipStreamSynchronize(s));
     HIP_OK(hipStreamDestroy(s));
