@@ -21,5 +21,8 @@ from .ops import (  # noqa: F401
     _expand_dim_specification,
 )
 
-__all__ = ["similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError",
+from . import layers  # noqa: F401,E402
+from .layers import Similarity, Mex, dirichlet_init  # noqa: F401,E402
+
+__all__ = ["layers", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError",
            "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad"]

@@ -1,0 +1,248 @@
+"""Differentiable ops and layer classes on top of the C ABI: the caller-side layer of the reference.
+
+  * `SimilarityFunction` / `MexFunction` wire the backward entry points to torch.autograd the way
+    `_similarity_grad` / `_mex_grad` register them with TensorFlow
+    (python/simnets/ops/similarity.py:18-45, python/simnets/ops/mex.py:47-81).
+  * `Similarity` / `Mex` are torch modules with the constructor arguments, parameter shapes and
+    defaults of the Keras layers in python/simnets/keras.py:19-88 and :113-197, built lazily from
+    the first input like Keras' `build(input_shape)`.
+Everything computes in fp32 on a HIP device through libsimnets_hip.so; there is no CPU path.
+"""
+import math
+
+import numpy as np
+import torch
+
+from . import ops
+
+_SIM_KEYS = ("similarity_function", "blocks", "strides", "padding", "normalization_term",
+             "normalization_term_fudge", "ignore_nan_input", "out_of_bounds_value")
+_MEX_KEYS = ("softmax_mode", "padding", "strides", "blocks", "epsilon", "blocks_out_of_bounds_value",
+             "blocks_round_down", "use_unshared_regions", "shared_offset_region", "unshared_offset_region",
+             "normalize_offsets")
+
+
+class SimilarityFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, templates, weights, attrs):
+        ctx.attrs = attrs
+        ctx.save_for_backward(input, templates, weights)
+        return ops.similarity(input, templates, weights, **attrs)
+
+    @staticmethod
+    def backward(ctx, grad):
+        input, templates, weights = ctx.saved_tensors
+        grad = grad.contiguous()
+        gi = gt = gw = None
+        if ctx.needs_input_grad[0]:
+            gi = ops.similarity_input_grad(input, templates, weights, grad, **ctx.attrs)
+        if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
+            gt, gw = ops.similarity_parameters_grad(input, templates, weights, grad, **ctx.attrs)
+        return gi, gt, gw, None
+
+
+class MexFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input, offsets, num_instances, attrs):
+        ctx.attrs, ctx.num_instances = attrs, num_instances
+        out = ops.mex(input, offsets, num_instances, **attrs)
+        ctx.save_for_backward(input, offsets, out)
+        return out
+
+    @staticmethod
+    def backward(ctx, grad):
+        input, offsets, out = ctx.saved_tensors
+        grad = grad.contiguous()
+        gi = go = None
+        if ctx.needs_input_grad[0]:
+            gi = ops.mex_input_grad(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
+        if ctx.needs_input_grad[1]:
+            go = ops.mex_offsets_grad(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
+        return gi, go, None, None
+
+
+def similarity(input, templates, weights, **attrs):
+    """Differentiable `ops.similarity` (same keyword arguments)."""
+    unknown = set(attrs) - set(_SIM_KEYS)
+    if unknown:
+        raise TypeError("unknown Similarity attributes: %s" % sorted(unknown))
+    return SimilarityFunction.apply(input, templates, weights, attrs)
+
+
+def mex(input, offsets, num_instances, **attrs):
+    """Differentiable `ops.mex` (same keyword arguments)."""
+    unknown = set(attrs) - set(_MEX_KEYS)
+    if unknown:
+        raise TypeError("unknown Mex attributes: %s" % sorted(unknown))
+    return MexFunction.apply(input, offsets, num_instances, attrs)
+
+
+def dirichlet_init(shape, alpha=1.0, generator=None):
+    """log of Dirichlet(alpha) samples over the block volume, one per (region, instance):
+    DirichletInit of python/simnets/keras.py:91-109."""
+    num_regions, num_instances, bc, bh, bw = shape
+    rng = generator if generator is not None else np.random
+    sample = rng.dirichlet([alpha] * (bc * bh * bw), size=(num_regions, num_instances))
+    return torch.from_numpy(np.log(sample).astype(np.float32).reshape(shape))
+
+
+def _resolve_padding(padding, blocks):
+    if isinstance(padding, str):
+        if padding.upper() not in ("SAME", "VALID"):
+            raise ValueError("Padding must be one of SAME, VALID (or a list of ints)")
+        return [0] * len(blocks) if padding.upper() == "VALID" else [e // 2 for e in blocks]
+    return list(padding)
+
+
+class Similarity(torch.nn.Module):
+    """python/simnets/keras.py:19-88.  Parameters: `templates`, `sweights` [num_instances, C, bh, bw];
+    the op sees abs(sweights) (keras.py:65)."""
+
+    def __init__(self, num_instances=None, similarity_function="L2", strides=[1, 1], blocks=[3, 3], padding="SAME",
+                 normalization_term=False, normalization_term_fudge=0.001, ignore_nan_input=False,
+                 out_of_bounds_value=0, templates_initializer="random_normal", weights_initializer="ones",
+                 channels_last=False):
+        super().__init__()
+        assert num_instances is not None
+        self.num_instances = num_instances
+        self.similarity_function = similarity_function
+        self.strides, self.blocks = list(strides), list(blocks)
+        self.padding = _resolve_padding(padding, self.blocks)
+        self.normalization_term = normalization_term
+        self.normalization_term_fudge = normalization_term_fudge
+        self.ignore_nan_input = ignore_nan_input
+        self.out_of_bounds_value = out_of_bounds_value
+        self.templates_initializer, self.weights_initializer = templates_initializer, weights_initializer
+        self.channels_last = channels_last
+        self.templates = torch.nn.UninitializedParameter()
+        self.sweights = torch.nn.UninitializedParameter()
+
+    @staticmethod
+    def _init(param, how):
+        if callable(how):
+            how(param)
+        elif how == "ones":
+            torch.nn.init.ones_(param)
+        elif how == "zeros":
+            torch.nn.init.zeros_(param)
+        elif how == "random_normal":
+            torch.nn.init.normal_(param, 0.0, 0.05)   # Keras' RandomNormal default
+        else:
+            raise ValueError("unknown initializer %r" % (how,))
+
+    def build(self, input_shape):
+        channels = input_shape[3] if self.channels_last else input_shape[1]
+        shape = (self.num_instances, channels, self.blocks[0], self.blocks[1])
+        for p, how in ((self.sweights, self.weights_initializer), (self.templates, self.templates_initializer)):
+            p.materialize(shape, dtype=torch.float32)
+            with torch.no_grad():
+                self._init(p, how)
+
+    def attrs(self):
+        return dict(similarity_function=self.similarity_function, blocks=self.blocks, strides=self.strides,
+                    padding=self.padding, normalization_term=self.normalization_term,
+                    normalization_term_fudge=self.normalization_term_fudge, ignore_nan_input=self.ignore_nan_input,
+                    out_of_bounds_value=self.out_of_bounds_value)
+
+    def forward(self, x):
+        if isinstance(self.templates, torch.nn.UninitializedParameter):
+            self.build(x.shape)
+            self.to(x.device)
+        if self.channels_last:
+            x = x.permute(0, 3, 1, 2).contiguous()
+        out = similarity(x, self.templates, self.sweights.abs(), **self.attrs())
+        return out.permute(0, 2, 3, 1) if self.channels_last else out
+
+    def compute_output_shape(self, input_shape):
+        shape = list(input_shape)
+        if self.channels_last:
+            shape = [shape[0], shape[3], shape[1], shape[2]]
+        out = ops.similarity_output_shape(shape, (self.num_instances, shape[1], self.blocks[0], self.blocks[1]),
+                                          **self.attrs())
+        return (out[0], out[2], out[3], out[1]) if self.channels_last else tuple(out)
+
+    def get_config(self):
+        names = ["num_instances", "similarity_function", "strides", "blocks", "padding", "normalization_term",
+                 "normalization_term_fudge", "ignore_nan_input", "out_of_bounds_value", "templates_initializer",
+                 "weights_initializer", "channels_last"]
+        return {k: getattr(self, k) for k in names}
+
+
+class Mex(torch.nn.Module):
+    """python/simnets/keras.py:113-197.  Parameter: `offsets` [num_regions, num_instances, bc, bh, bw].
+    `normalize_offsets` is applied on the device inside the op (forward and backward)."""
+
+    def __init__(self, num_instances=None, padding=[0, 0, 0], strides=[1, 1, 1], blocks=[1, 1, 1], epsilon=1.0,
+                 use_unshared_regions=True, shared_offset_region=[-1], unshared_offset_region=[-1], softmax_mode=False,
+                 blocks_out_of_bounds_value=0.0, blocks_round_down=True, normalize_offsets=False,
+                 offsets_initializer="dirichlet", channels_last=False):
+        super().__init__()
+        assert num_instances is not None
+        self.num_instances = num_instances
+        self.padding, self.strides, self.blocks = padding, list(strides), list(blocks)
+        self.epsilon = epsilon
+        self.use_unshared_regions = use_unshared_regions
+        self.shared_offset_region = list(shared_offset_region)
+        self.unshared_offset_region = list(unshared_offset_region)
+        self.softmax_mode = softmax_mode
+        self.blocks_out_of_bounds_value = blocks_out_of_bounds_value
+        self.blocks_round_down = blocks_round_down
+        self.normalize_offsets = normalize_offsets
+        self.offsets_initializer = offsets_initializer
+        self.channels_last = channels_last
+        self.offsets = torch.nn.UninitializedParameter()
+
+    def build(self, input_shape):
+        shape = list(input_shape)
+        if self.channels_last:
+            shape = [shape[0], shape[3], shape[1], shape[2]]
+        self.blocks = ops._expand_dim_specification(shape, self.blocks)
+        self.padding = _resolve_padding(self.padding, self.blocks)
+        nregions = ops._mex_dims_helper(shape[1:], self.num_instances, blocks=self.blocks, padding=self.padding,
+                                        strides=self.strides, use_unshared_regions=self.use_unshared_regions,
+                                        shared_offset_region=self.shared_offset_region,
+                                        blocks_round_down=self.blocks_round_down,
+                                        unshared_offset_region=self.unshared_offset_region)
+        oshape = (nregions, self.num_instances) + tuple(self.blocks)
+        self.offsets.materialize(oshape, dtype=torch.float32)
+        with torch.no_grad():
+            how = self.offsets_initializer
+            if callable(how):
+                how(self.offsets)
+            elif how == "dirichlet":
+                self.offsets.copy_(dirichlet_init(oshape))
+            elif how == "zeros":
+                self.offsets.zero_()
+            else:
+                raise ValueError("unknown initializer %r" % (how,))
+
+    def attrs(self):
+        return dict(softmax_mode=self.softmax_mode, padding=self.padding, strides=self.strides, blocks=self.blocks,
+                    epsilon=self.epsilon, blocks_out_of_bounds_value=self.blocks_out_of_bounds_value,
+                    blocks_round_down=self.blocks_round_down, use_unshared_regions=self.use_unshared_regions,
+                    shared_offset_region=self.shared_offset_region,
+                    unshared_offset_region=self.unshared_offset_region, normalize_offsets=self.normalize_offsets)
+
+    def forward(self, x):
+        if isinstance(self.offsets, torch.nn.UninitializedParameter):
+            self.build(x.shape)
+            self.to(x.device)
+        if self.channels_last:
+            x = x.permute(0, 3, 1, 2).contiguous()
+        out = mex(x, self.offsets, self.num_instances, **self.attrs())
+        return out.permute(0, 2, 3, 1) if self.channels_last else out
+
+    def compute_output_shape(self, input_shape):
+        shape = list(input_shape)
+        if self.channels_last:
+            shape = [shape[0], shape[3], shape[1], shape[2]]
+        blocks = ops._expand_dim_specification(shape, self.blocks)
+        attrs = dict(self.attrs(), blocks=blocks, padding=_resolve_padding(self.padding, blocks))
+        out, _ = ops.mex_output_shape(shape, self.num_instances, **attrs)
+        return (out[0], out[2], out[3], out[1]) if self.channels_last else tuple(out)
+
+    def get_config(self):
+        names = ["num_instances", "padding", "strides", "blocks", "epsilon", "use_unshared_regions",
+                 "shared_offset_region", "unshared_offset_region", "softmax_mode", "blocks_out_of_bounds_value",
+                 "blocks_round_down", "normalize_offsets", "offsets_initializer", "channels_last"]
+        return {k: getattr(self, k) for k in names}

@@ -1,0 +1,119 @@
+"""The differentiable op layer and the module classes (python/simnets/keras.py of the reference) on the GPU."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from util import rel_err
+
+pytestmark = pytest.mark.gpu
+
+
+def test_autograd_routes_to_the_grad_entry_points(pkg):
+    g = torch.Generator().manual_seed(1)
+    x = torch.randn(2, 3, 9, 8, generator=g).cuda().requires_grad_()
+    t = torch.randn(4, 3, 3, 3, generator=g).cuda().requires_grad_()
+    w = (torch.rand(4, 3, 3, 3, generator=g) + 0.1).cuda().requires_grad_()
+    kw = dict(blocks=[3, 3], strides=[2, 1], padding=[1, 1])
+    out = pkg.layers.similarity(x, t, w, **kw)
+    go = torch.randn(out.shape, generator=g).cuda()
+    out.backward(go)
+    assert torch.equal(x.grad, pkg.similarity_input_grad(x.detach(), t.detach(), w.detach(), go, **kw))
+    dt, dw = pkg.similarity_parameters_grad(x.detach(), t.detach(), w.detach(), go, **kw)
+    assert torch.equal(t.grad, dt) and torch.equal(w.grad, dw)
+
+    off = torch.randn(4, 5, 3, 1, 1, generator=g).cuda().requires_grad_()
+    x2 = x.detach().clone().requires_grad_()
+    mkw = dict(blocks=[3, 1, 1], strides=[3, 1, 1], unshared_offset_region=[2], softmax_mode=True)
+    y = pkg.layers.mex(x2, off, 5, **mkw)
+    gy = torch.randn(y.shape, generator=g).cuda()
+    y.backward(gy)
+    assert torch.equal(x2.grad, pkg.mex_input_grad(x2.detach(), off.detach(), y.detach(), gy, 5, **mkw))
+    assert torch.equal(off.grad, pkg.mex_offsets_grad(x2.detach(), off.detach(), y.detach(), gy, 5, **mkw))
+
+
+def test_autograd_matches_torch_autograd_of_the_closed_form(pkg):
+    """Similarity L2 written with unfold, MEX 1x1 written with logsumexp: torch's own autograd is the check."""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(2, 3, 10, 9, generator=g).cuda()
+    t = torch.randn(6, 3, 3, 2, generator=g).cuda()
+    w = (torch.rand(6, 3, 3, 2, generator=g) + 0.1).cuda()
+    leaves = [a.clone().requires_grad_() for a in (x, t, w)]
+    out = pkg.layers.similarity(*leaves, blocks=[3, 2], strides=[1, 2], padding=[1, 0])
+    ref_leaves = [a.double().requires_grad_() for a in (x, t, w)]
+    cols = F.unfold(ref_leaves[0], (3, 2), padding=(1, 0), stride=(1, 2))
+    d = cols[:, None] - ref_leaves[1].reshape(6, -1)[None, :, :, None]
+    ref = -(ref_leaves[2].reshape(6, -1)[None, :, :, None] * d * d).sum(2).reshape(out.shape)
+    go = torch.randn(out.shape, generator=g).cuda()
+    out.backward(go)
+    ref.backward(go.double())
+    assert rel_err(out.detach().cpu().numpy(), ref.detach().cpu().numpy()) <= 1e-5
+    for a, b in zip(leaves, ref_leaves):
+        scale = b.grad.abs().max().item()
+        assert rel_err(a.grad.cpu().numpy(), b.grad.cpu().numpy(), floor=np.full(tuple(b.shape), 1e-2 * scale)) <= 1e-4
+
+
+def test_layers_build_lazily_with_the_reference_shapes(pkg):
+    # python/simnets/test/keras/__init__.py:46-55, :110-119
+    for num, padding, strides, blocks, in_shape, out_shape in [
+            (10, [0, 1], [1, 1], [2, 2], (3, 10, 13), (10, 9, 14)),
+            (10, [1, 1], [3, 2], [2, 2], (3, 10, 13), (10, 4, 7)),
+            (2, [1, 1], [3, 2], [2, 2], (1, 10, 13), (2, 4, 7))]:
+        layer = pkg.Similarity(num, padding=padding, strides=strides, blocks=blocks)
+        assert layer.compute_output_shape((5,) + in_shape) == (5,) + out_shape
+        y = layer(torch.zeros((5,) + in_shape).cuda())
+        assert tuple(y.shape) == (5,) + out_shape
+        assert tuple(layer.templates.shape) == (num, in_shape[0]) + tuple(blocks) == tuple(layer.sweights.shape)
+    layer = pkg.Mex(4, blocks=[-1, 2, 2], strides=[3, 2, 2], unshared_offset_region=[2], softmax_mode=True,
+                    normalize_offsets=True)
+    y = layer(torch.randn(2, 3, 8, 8).cuda())
+    assert tuple(y.shape) == (2, 4, 4, 4) == layer.compute_output_shape((2, 3, 8, 8))
+    assert tuple(layer.offsets.shape) == (4, 4, 3, 2, 2)
+    # dirichlet initialisation: rows are log-probabilities
+    np.testing.assert_allclose(layer.offsets.detach().exp().sum(dim=(2, 3, 4)).cpu().numpy(), 1.0, rtol=1e-5)
+
+
+def test_channels_last_is_a_transposition(pkg):
+    torch.manual_seed(3)
+    a = pkg.Similarity(5, blocks=[3, 3], padding="SAME")
+    b = pkg.Similarity(5, blocks=[3, 3], padding="SAME", channels_last=True)
+    x = torch.randn(2, 3, 7, 6).cuda()
+    ya = a(x)
+    b.build((2, 7, 6, 3))
+    b.cuda()
+    with torch.no_grad():
+        b.templates.copy_(a.templates)
+        b.sweights.copy_(a.sweights)
+    yb = b(x.permute(0, 2, 3, 1).contiguous())
+    assert torch.equal(yb.permute(0, 3, 1, 2), ya)
+
+
+def test_a_small_network_trains(pkg):
+    """Similarity -> Mex -> Mex (to 1x1) as in the reference's example network; a few SGD steps on a fixed batch
+    must lower the cross-entropy, with all parameters receiving finite gradients."""
+    torch.manual_seed(4)
+    net = torch.nn.Sequential(
+        pkg.Similarity(8, blocks=[2, 2], strides=[2, 2], padding=[0, 0], normalization_term=True, ignore_nan_input=True,
+                       out_of_bounds_value=float("nan")),
+        pkg.Mex(6, blocks=[-1, 2, 2], strides=[8, 2, 2], softmax_mode=True, normalize_offsets=True,
+                unshared_offset_region=[2]),
+        pkg.Mex(3, blocks=[-1, -1, -1], softmax_mode=True, normalize_offsets=True, use_unshared_regions=False,
+                shared_offset_region=[-1]),
+    )
+    x = torch.rand(16, 1, 8, 8).cuda() - 0.5
+    x[torch.rand(x.shape, device="cuda") < 0.2] = float("nan")
+    labels = (torch.arange(16) % 3).cuda()
+    logits = net(x)
+    assert tuple(logits.shape) == (16, 3, 1, 1)
+    opt = torch.optim.SGD(net.parameters(), lr=0.05)
+    losses = []
+    for _ in range(12):
+        opt.zero_grad()
+        loss = torch.nn.functional.cross_entropy(net(x).flatten(1), labels)
+        loss.backward()
+        for p in net.parameters():
+            assert torch.isfinite(p.grad).all()
+        opt.step()
+        losses.append(loss.item())
+    assert losses[-1] < losses[0]
