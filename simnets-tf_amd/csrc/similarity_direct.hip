@@ -42,6 +42,7 @@ struct SimKernelArgs {
     float *out;
     const float *pa;   // [mtile][K][MT][2]  (template, scaled negative weight)
     const float *pc;   // [mtile][K][MT]     per-(m,k) additive constant (normalized modes)
+    const int *koff;   // [K + 2] LDS offset of patch element k inside the staged chunk: (c % CC) * TRmax*TC + dh*TC + dw
     int B, C, H, W, O, oh, ow;
     int bh, bw, sh, sw, ph, pw, K;
     int G;             // pixel groups per output row = ceil(ow / PT)
@@ -73,11 +74,13 @@ __device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT]
         pc[i] = (MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN) ? ppc[i] : 0.0f;
 }
 
-// One k step for all MT templates and PT pixels of a lane.
-template <int MODE, int PT, int MT>
+// One k step for all MT templates and PT pixels of a lane.  VP: the parameters are already in VGPRs
+// (fetched with vector loads); otherwise they are wave-uniform SGPR values and are moved once.
+template <int MODE, int PT, int MT, bool VP = false>
 __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[PT], const float (&pa)[2 * MT],
                                          const float (&pc)[MT])
 {
+    auto vg = [](float v) { return VP ? v : to_vgpr(v); };
     if (MODE == SIM_MODE_L2_NORM_IGNORE_NAN) {
         float keep[PT], xz[PT];
 #pragma unroll
@@ -88,7 +91,7 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
         }
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const float t = to_vgpr(pa[2 * m]), nwh = to_vgpr(pa[2 * m + 1]), c = to_vgpr(pc[m]);
+            const float t = vg(pa[2 * m]), nwh = vg(pa[2 * m + 1]), c = vg(pc[m]);
 #pragma unroll
             for (int p = 0; p < PT; ++p) {
                 const float d = t - xz[p];
@@ -99,10 +102,10 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
     } else {
 #pragma unroll
         for (int m = 0; m < MT; ++m) {
-            const float t = to_vgpr(pa[2 * m]), nw = to_vgpr(pa[2 * m + 1]);
+            const float t = vg(pa[2 * m]), nw = vg(pa[2 * m + 1]);
             float c = 0.0f;
             if (MODE == SIM_MODE_L2_NORM)
-                c = to_vgpr(pc[m]);
+                c = vg(pc[m]);
             // The combine is a chain of dependent instructions per pixel; a dependent VALU instruction
             // issued right behind its producer stalls, so the chain is laid out stage by stage across
             // the PT pixels (PT independent instructions between producer and consumer).
@@ -191,16 +194,45 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
         for (int p = 0; p < PT; ++p)
             acc[m][p] = 0.0f;
 
-    const float SIMNETS_CONST_AS *pa =
-        (const float SIMNETS_CONST_AS *)(a.pa) + (size_t)(wave_active ? mtile : 0) * a.K * MT * 2;
-    const float SIMNETS_CONST_AS *pc =
-        (const float SIMNETS_CONST_AS *)(a.pc) + (size_t)(wave_active ? mtile : 0) * a.K * MT;
+    // Parameter stream of this wave's templates.  Every lane reads the same address, but through vector
+    // loads (the zero below is opaque to the compiler, so the address counts as lane-dependent): the
+    // values arrive in VGPRs, which is where the arithmetic wants them (VALU instructions with SGPR
+    // operands issue at half rate), at the cost of 4 load instructions per k instead of one scalar load
+    // plus 16 moves; they use the vector-memory counter, so waiting for LDS data never waits for them.
+    unsigned zero_v;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(zero_v));
+    constexpr bool HAS_PC = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
+    const char *pa_base = reinterpret_cast<const char *>(a.pa + (size_t)(wave_active ? mtile : 0) * a.K * MT * 2);
+    const char *pc_base = reinterpret_cast<const char *>(a.pc + (size_t)(wave_active ? mtile : 0) * a.K * MT);
+    unsigned pa_off = zero_v, pc_off = zero_v;  // byte offsets of the NEXT k
+    auto fetch_params = [&](float (&pav)[2 * MT], float (&pcv)[MT]) {
+#pragma unroll
+        for (int i = 0; i < 2 * MT / 4; ++i) {
+            const float4 v = *reinterpret_cast<const float4 *>(pa_base + pa_off + 16 * i);
+            pav[4 * i] = v.x; pav[4 * i + 1] = v.y; pav[4 * i + 2] = v.z; pav[4 * i + 3] = v.w;
+        }
+        pa_off += 2 * MT * sizeof(float);
+        if (HAS_PC) {
+#pragma unroll
+            for (int i = 0; i < MT / 4; ++i) {
+                const float4 v = *reinterpret_cast<const float4 *>(pc_base + pc_off + 16 * i);
+                pcv[4 * i] = v.x; pcv[4 * i + 1] = v.y; pcv[4 * i + 2] = v.z; pcv[4 * i + 3] = v.w;
+            }
+            pc_off += MT * sizeof(float);
+        } else {
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+                pcv[i] = 0.0f;
+        }
+    };
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
-    const int chan_lds = TR * a.TC;
+    const int chan_lds = a.TRmax * a.TC;
     float pa0[2 * MT], pc0[MT], pa1[2 * MT], pc1[MT];
-    load_params<MODE, MT>(pa0, pc0, pa, pc);
+    fetch_params(pa0, pc0);
     TilePositions<kStagePos> tp;
     tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
+    // LDS offsets of the patch elements, one scalar load per k, fetched two steps ahead
+    const int SIMNETS_CONST_AS *kt = (const int SIMNETS_CONST_AS *)(a.koff);
 
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
@@ -214,44 +246,36 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
         //      values and the parameters of step k+1 are requested before the arithmetic of step k,
         //      ping-ponging between two register sets (no copies) ----
         const int nk = ccn * a.bh * a.bw;
-        int dh = 0, dw = 0, row_off = 0, off = 0;
+        int off_next = kt[1];  // offset of step k+1 (the entries behind the last k are 0)
         auto step = [&](const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT], float (&xnx)[PT],
-                        float (&panx)[2 * MT], float (&pcnx)[MT], bool last) {
-            // LDS and scalar loads share one counter and scalar loads return out of order, so a wait
-            // for LDS data after a new scalar load was issued would also wait for that load.  Drain
-            // the counter here, where everything outstanding was issued a whole step ago, and only
-            // then issue the requests for the next step: the arithmetic below needs no further wait.
+                        float (&panx)[2 * MT], float (&pcnx)[MT]) {
+            // everything outstanding on the LDS / scalar counter was issued a whole step ago
             __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
             __builtin_amdgcn_sched_barrier(0);
-            // next tap, branch-free (selects on wave-uniform values keep the step one basic block)
-            const bool wrap_w = dw + 1 == a.bw;
-            const int ndw = wrap_w ? 0 : dw + 1;
-            const bool wrap_h = wrap_w && dh + 1 == a.bh;
-            const int ndh = wrap_h ? 0 : dh + (wrap_w ? 1 : 0);
-            const int nrow = row_off + (wrap_w ? a.TC : 0) + (wrap_h ? chan_lds - a.bh * a.TC : 0);
-            const int noff = last ? off : nrow + ndw;  // nothing is staged beyond this chunk
 #pragma unroll
             for (int p = 0; p < PT; ++p)
-                xnx[p] = lds[lds_base + noff + p * sw];
-            pa += 2 * MT;
-            pc += MT;
-            load_params<MODE, MT>(panx, pcnx, pa, pc);  // one k of slack exists behind the arrays
+                xnx[p] = lds[lds_base + off_next + p * sw];
+            kt += 1;
+            off_next = kt[1];
+            fetch_params(panx, pcnx);  // one k of slack exists behind the arrays
             __builtin_amdgcn_sched_barrier(0);
-            sim_step<MODE, PT, MT>(acc, xc, pac, pcc);
+            sim_step<MODE, PT, MT, true>(acc, xc, pac, pcc);
             __builtin_amdgcn_sched_barrier(0);
-            dw = ndw; dh = ndh; row_off = nrow; off = noff;
         };
         float x0[PT], x1[PT];
+        {
+            const int off0 = kt[0];
 #pragma unroll
-        for (int p = 0; p < PT; ++p)
-            x0[p] = lds[lds_base + p * sw];
+            for (int p = 0; p < PT; ++p)
+                x0[p] = lds[lds_base + off0 + p * sw];
+        }
         int kk = 0;
         for (; kk + 2 <= nk; kk += 2) {
-            step(x0, pa0, pc0, x1, pa1, pc1, false);
-            step(x1, pa1, pc1, x0, pa0, pc0, kk + 2 == nk);
+            step(x0, pa0, pc0, x1, pa1, pc1);
+            step(x1, pa1, pc1, x0, pa0, pc0);
         }
         if (kk < nk) {
-            step(x0, pa0, pc0, x1, pa1, pc1, true);
+            step(x0, pa0, pc0, x1, pa1, pc1);
 #pragma unroll
             for (int i = 0; i < 2 * MT; ++i)
                 pa0[i] = pa1[i];
@@ -358,8 +382,19 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
 // per-(m,k) logarithm term.  Replaces interlace_kernel (include/utils/ggemm.cuh:70-87).
 __global__ void sim_pack_params_kernel(const float *__restrict__ templates, const float *__restrict__ weights, int O,
                                        int K, int MT, int n_mtiles, int mode, float fudge, float *__restrict__ pa,
-                                       float *__restrict__ pc)
+                                       float *__restrict__ pc, int *__restrict__ koff, int taps, int bw, int CC,
+                                       int chan_pitch, int TC)
 {
+    // LDS offset of patch element k inside a staged chunk of CC channels; 0 behind the last k
+    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < K + 2; k += gridDim.x * blockDim.x) {
+        int off = 0;
+        if (k < K) {
+            const int c = k / taps, rem = k - c * taps;
+            const int dh = rem / bw, dw = rem - dh * bw;
+            off = (c % CC) * chan_pitch + dh * TC + dw;
+        }
+        koff[k] = off;
+    }
     const long long total = (long long)n_mtiles * K * MT;
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (long long)gridDim.x * blockDim.x) {
@@ -473,7 +508,8 @@ size_t sim_direct_workspace_bytes(const SimPlan &p)
     // one extra k of slack behind each array: the scalar loads may be issued one step ahead
     const size_t pa = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
     const size_t pc = align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
-    return pa + pc;
+    const size_t koff = align_up(((size_t)p.K + 2) * sizeof(int), 256);
+    return pa + pc + koff;
 }
 
 int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
@@ -485,18 +521,20 @@ int sim_direct_launch(const SimPlan &p, const float *input, const float *templat
     if (workspace_bytes < sim_direct_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     float *pa = reinterpret_cast<float *>(workspace);
+    const size_t pc_bytes = align_up(((size_t)n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
     float *pc = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + pa_bytes);
+    int *koff = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + pa_bytes + pc_bytes);
 
     const long long total = (long long)n_mtiles * p.K * t.MT;
     const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
     const int mode = (p.algo == SIMNETS_ALGO_SQRTW) ? (int)SIM_MODE_L2_SQRTW : p.mode;
     hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights, p.O, p.K, t.MT,
-                       n_mtiles, mode, p.fudge, pa, pc);
+                       n_mtiles, mode, p.fudge, pa, pc, koff, p.bh * p.bw, p.bw, t.CC, t.TRmax * t.TC, t.TC);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
 
     SimKernelArgs a;
-    a.in = input; a.out = output; a.pa = pa; a.pc = pc;
+    a.in = input; a.out = output; a.pa = pa; a.pc = pc; a.koff = koff;
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
     a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.K = p.K;
     a.G = t.G; a.gpi = t.gpi; a.tiles = t.tiles; a.nws = t.nws; a.n_mtiles = n_mtiles;
