@@ -1,11 +1,11 @@
 #!/usr/bin/env python3
-"""Benchmark of the SimNets forward hot path on one MI355X.
+"""Benchmark of the SimNets Similarity / MEX hot path on one MI355X.
 
 One "step" = one Similarity L2 forward over BASELINE configuration 3 (input 256x64x32x32, 128
 templates 64x3x3, stride 1, padding 1 -> 256x128x32x32; 19.33 G generalized MACs), inputs already
 resident in HBM, called through the C ABI exactly as an op layer would.  The other configurations
-(1, 2, 3-L1, 4) and the alternative evaluation paths are timed in the same run and reported under
-"others".  Prints ONE JSON line.
+(1, 2, 3-L1, 4, and the backward operators of configuration 5) and the alternative evaluation paths
+are timed in the same run and reported under "others".  Prints ONE JSON line.
 
 The CPU baseline leg times the CPU oracle (a restatement of the reference's CPU kernels) on a
 bounded sample of the same workload; it is the only place this file touches oracle/.
@@ -115,7 +115,9 @@ def main():
         "config": {"workload": "config3: Similarity L2 fwd 256x64x32x32, 128 templates 64x3x3, s1 p1 "
                                "-> 256x128x32x32 (M=262144 N=128 K=576)",
                    "algo": args.algo or "direct", "gmac_per_step": gmac3},
-        "roofline": {"bound": "mfma" if args.algo == "mfma" else "valu",
+        # compute bound at the FP32 peak, which is the same figure for the vector ALU and the FP32 matrix
+        # cores; "engine" says which of the two the kernel runs on
+        "roofline": {"bound": "mfma", "engine": "mfma" if args.algo == "mfma" else "valu",
                      "achieved": round(achieved_tflops, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tflops / PEAK_FP32_TFLOPS, 4),
                      "traffic": MEASURED_TRAFFIC_BYTES.get(args.algo or "direct"),
@@ -186,6 +188,23 @@ def main():
         others["config4_stack"] = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(gmac4 / (ms * 1e-3) / 1e9, 1),
                                    "exp_frac": round(gmac4 / (ms * 1e-3) / EXP_RATE, 4), "batch": 512,
                                    "kernels": "similarity + 5 x (offset pack + mex) + 4 x sum pool"}
+        # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
+        G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
+        _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,
+                      args.warmup)
+        others["config5_similarity_input_grad_L2"] = entry(ms, gmac3, 2 * 67108864 + 589824 + 134217728, flop=4)
+        _, ms = timed(lambda: pkg.similarity_parameters_grad(X3, T3, W3, G3, similarity_function="L2", **kw3),
+                      args.steps, args.warmup)
+        others["config5_similarity_params_grad_L2"] = entry(ms, gmac3, 67108864 + 3 * 589824 + 134217728, flop=5)
+        del G3
+        Y2 = pkg.mex(X2, O2, n2, normalize_offsets=True, **kw2)
+        G2 = to_dev(np.random.default_rng(6789).normal(size=(64, 64, 16, 16)).astype(np.float32))
+        _, ms = timed(lambda: pkg.mex_input_grad(X2, O2, Y2, G2, n2, normalize_offsets=True, **kw2), args.steps,
+                      args.warmup)
+        others["config5_mex_input_grad"] = entry(ms, 33554432, 2 * 2097152 + 2 * 4194304 + 32768, exp_bound=True)
+        _, ms = timed(lambda: pkg.mex_offsets_grad(X2, O2, Y2, G2, n2, normalize_offsets=True, **kw2), args.steps,
+                      args.warmup)
+        others["config5_mex_offsets_grad"] = entry(ms, 33554432, 2097152 + 2 * 4194304 + 2 * 32768, exp_bound=True)
     result["others"] = others
 
     # ------------------------------------------------------------------ CPU baseline (bounded sample)

@@ -51,7 +51,8 @@ struct GradXArgs {
     const float *g;    // output gradient [B,O,oh,ow]
     const float *x;    // input [B,C,H,W]
     float *dx;         // [B,C,H,W]
-    const float *pb;   // this phase's parameters [ctile][K][MT][2], K = O*nI*nJ, taps flipped
+    const float *pb;   // this phase's parameters [ctile][K + 1][MT][2], K = O*nI*nJ, taps flipped
+    const int *koff;   // [K + 2] LDS offset of step k = (o, dh, dw): (o % CC) * TRmax*TC + dh*TC + dw
     int B, C, H, W, O, oh, ow;
     int nI, nJ;        // taps of this phase along h and w
     int padh, padw;    // padding of g in phase coordinates: phase row h reads g rows h - padh + dh
@@ -70,7 +71,7 @@ __device__ __forceinline__ void gx_step(float (&acc)[MT][PT], const float (&xv)[
 {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
-        const float p0 = to_vgpr(pb[2 * m]), p1 = to_vgpr(pb[2 * m + 1]);
+        const float p0 = pb[2 * m], p1 = pb[2 * m + 1];  // already in VGPRs (vector loads)
         float u[PT];
         if (MODE == GX_L2) {
             // (s*w*t, -s*w): u = s*w*(t - x)
@@ -100,7 +101,7 @@ __device__ __forceinline__ void gx_step(float (&acc)[MT][PT], const float (&xv)[
     }
 }
 
-constexpr int gx_waves_per_simd(int pt, int mt) { return pt * mt <= 32 ? 4 : 2; }
+constexpr int gx_waves_per_simd(int pt, int mt) { return pt * mt <= 32 ? 3 : 2; }
 constexpr int gx_lds_budget(int pt, int mt) { return pt * mt <= 32 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
 
 template <int MODE, int PT, int MT>
@@ -153,14 +154,27 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
         }
     }
 
-    const float SIMNETS_CONST_AS *pb =
-        (const float SIMNETS_CONST_AS *)(a.pb) + (size_t)(wave_active ? ctile : 0) * (a.K + 1) * MT * 2;
+    // parameter stream: same address in every lane, fetched with vector loads so that the values arrive
+    // in VGPRs (the zero is opaque to the compiler, which would otherwise turn them into scalar loads)
+    unsigned zero_v;
+    asm volatile("v_mov_b32 %0, 0" : "=v"(zero_v));
+    const char *pb_base = reinterpret_cast<const char *>(a.pb + (size_t)(wave_active ? ctile : 0) * (a.K + 1) * MT * 2);
+    unsigned pb_off = zero_v;  // byte offset of the NEXT step
+    auto fetch_params = [&](float (&pbv)[2 * MT]) {
+#pragma unroll
+        for (int i = 0; i < 2 * MT / 4; ++i) {
+            const float4 v = *reinterpret_cast<const float4 *>(pb_base + pb_off + 16 * i);
+            pbv[4 * i] = v.x; pbv[4 * i + 1] = v.y; pbv[4 * i + 2] = v.z; pbv[4 * i + 3] = v.w;
+        }
+        pb_off += 2 * MT * sizeof(float);
+    };
     const float *img = a.g + (size_t)b * a.O * a.oh * a.ow;
-    const int chan_lds = TR * a.TC;
+    const int chan_lds = a.TRmax * a.TC;
     float pb0[2 * MT], pb1[2 * MT];
-    load_uniform<2 * MT>(pb0, pb);
+    fetch_params(pb0);
     TilePositions<kStagePos> tp;
     tp.template init<kThreads>(a.oh, a.ow, TR, a.TC, in_row0, a.padw);
+    const int SIMNETS_CONST_AS *kt = (const int SIMNETS_CONST_AS *)(a.koff);
 
     for (int ch0 = 0; ch0 < a.O; ch0 += a.CC) {
         const int ccn = min(a.CC, a.O - ch0);
@@ -172,38 +186,34 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
         // software pipeline over the (o, tap) steps of this chunk: the g values and the parameters of
         // the next step are requested before the arithmetic of the current one
         const int nk = ccn * a.nI * a.nJ;
-        int dh = 0, dw = 0, row_off = 0, off = 0;
-        auto step = [&](const float (&gc)[PT], const float (&pbc)[2 * MT], float (&gnx)[PT], float (&pbnx)[2 * MT],
-                        bool last) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): LDS and scalar loads share the counter
+        int off_next = kt[1];
+        auto step = [&](const float (&gc)[PT], const float (&pbc)[2 * MT], float (&gnx)[PT], float (&pbnx)[2 * MT]) {
+            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): issued a whole step ago
             __builtin_amdgcn_sched_barrier(0);
-            const bool wrap_w = dw + 1 == a.nJ;
-            const int ndw = wrap_w ? 0 : dw + 1;
-            const bool wrap_h = wrap_w && dh + 1 == a.nI;
-            const int ndh = wrap_h ? 0 : dh + (wrap_w ? 1 : 0);
-            const int nrow = row_off + (wrap_w ? a.TC : 0) + (wrap_h ? chan_lds - a.nI * a.TC : 0);
-            const int noff = last ? off : nrow + ndw;
 #pragma unroll
             for (int p = 0; p < PT; ++p)
-                gnx[p] = lds[lds_base + noff + p];
-            pb += 2 * MT;
-            load_uniform<2 * MT>(pbnx, pb);  // one step of slack exists behind each channel tile
+                gnx[p] = lds[lds_base + off_next + p];
+            kt += 1;
+            off_next = kt[1];
+            fetch_params(pbnx);  // one step of slack exists behind each channel tile
             __builtin_amdgcn_sched_barrier(0);
             gx_step<MODE, PT, MT>(acc, xv, gc, pbc);
             __builtin_amdgcn_sched_barrier(0);
-            dw = ndw; dh = ndh; row_off = nrow; off = noff;
         };
         float g0[PT], g1[PT];
+        {
+            const int off0 = kt[0];
 #pragma unroll
-        for (int p = 0; p < PT; ++p)
-            g0[p] = lds[lds_base + p];
+            for (int p = 0; p < PT; ++p)
+                g0[p] = lds[lds_base + off0 + p];
+        }
         int kk = 0;
         for (; kk + 2 <= nk; kk += 2) {
-            step(g0, pb0, g1, pb1, false);
-            step(g1, pb1, g0, pb0, kk + 2 == nk);
+            step(g0, pb0, g1, pb1);
+            step(g1, pb1, g0, pb0);
         }
         if (kk < nk) {
-            step(g0, pb0, g1, pb1, true);
+            step(g0, pb0, g1, pb1);
 #pragma unroll
             for (int i = 0; i < 2 * MT; ++i)
                 pb0[i] = pb1[i];
@@ -293,9 +303,18 @@ __global__ void fill_zero_kernel(float *__restrict__ p, long long n)
 // (dh = nI-1-ii, original tap i = ry + sh*ii) and the per-mode scaling folded in.
 __global__ void sim_grad_input_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
                                            int O, int C, int bh, int bw, int sh, int sw, int ry, int rx, int nI,
-                                           int nJ, int MT, int n_ctiles, int l1, float scale, float *__restrict__ pb)
+                                           int nJ, int MT, int n_ctiles, int l1, float scale, float *__restrict__ pb,
+                                           int *__restrict__ koff, int CC, int chan_pitch, int TC)
 {
     const int K = O * nI * nJ;
+    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < K + 2; k += gridDim.x * blockDim.x) {
+        int off = 0;
+        if (k < K) {
+            const int dw = k % nJ, dh = (k / nJ) % nI, o = k / (nJ * nI);
+            off = (o % CC) * chan_pitch + dh * TC + dw;
+        }
+        koff[k] = off;
+    }
     const long long total = (long long)n_ctiles * (K + 1) * MT;
     for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
          idx += (long long)gridDim.x * blockDim.x) {
@@ -389,6 +408,11 @@ size_t gx_phase_param_bytes(const SimPlan &p, const Phase &f)
     return align_up(n_ctiles * ((size_t)p.O * f.nI * f.nJ + 1) * 8 * 2 * sizeof(float), 256);
 }
 
+size_t gx_phase_table_bytes(const SimPlan &p, const Phase &f)
+{
+    return align_up(((size_t)p.O * f.nI * f.nJ + 2) * sizeof(int), 256);
+}
+
 bool gx_all_phases_fit(const SimPlan &p)
 {
     for (int ry = 0; ry < p.sh; ++ry)
@@ -424,7 +448,7 @@ size_t sim_grad_input_workspace_bytes(const SimPlan &p)
         for (int rx = 0; rx < p.sw; ++rx) {
             const Phase f = make_phase(p, ry, rx);
             if (!f.empty())
-                total += gx_phase_param_bytes(p, f);
+                total += gx_phase_param_bytes(p, f) + gx_phase_table_bytes(p, f);
         }
     return total;
 }
@@ -469,17 +493,19 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             const int K = p.O * f.nI * f.nJ;
             float *pb = reinterpret_cast<float *>(ws);
             ws += gx_phase_param_bytes(p, f);
+            int *koff = reinterpret_cast<int *>(ws);
+            ws += gx_phase_table_bytes(p, f);
 
             const long long total = (long long)n_ctiles * (K + 1) * t.MT;
             const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
             hipLaunchKernelGGL(sim_grad_input_pack_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights,
                                p.O, p.C, p.bh, p.bw, p.sh, p.sw, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, (int)l1, scale,
-                               pb);
+                               pb, koff, t.CC, t.TRmax * t.TC, t.TC);
             if (hipGetLastError() != hipSuccess)
                 return SIMNETS_ERR_HIP;
 
             GradXArgs a;
-            a.g = output_grad; a.x = input; a.dx = input_grad; a.pb = pb;
+            a.g = output_grad; a.x = input; a.dx = input_grad; a.pb = pb; a.koff = koff;
             a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
             a.nI = f.nI; a.nJ = f.nJ;
             a.padh = f.nI - 1 - f.a0; a.padw = f.nJ - 1 - f.b0;
@@ -507,6 +533,8 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
 namespace {
 
 constexpr int PC = 64;        // output pixels per LDS chunk
+constexpr int PCP = PC + 1;   // row pitch of the LDS tiles in float4 units: one more than a multiple of the bank
+                              // period, so the 8 rows a wave reads at once (same pixel) fall into distinct banks
 constexpr int LO = 8, LK = 4; // templates x patch elements per lane
 
 struct GradPArgs {
@@ -514,7 +542,7 @@ struct GradPArgs {
     float *partial;    // [nacc][S][Opad][Kpad]
     int B, C, H, W, O, oh, ow, bh, bw, sh, sw, ph, pw, K;
     int Opad, Kpad;    // O, K rounded up to the workgroup tile
-    int n_ktiles;
+    int n_ktiles, n_tiles;
     long long npix;    // B*oh*ow
     int nchunks, cps;  // pixel chunks in total, and per split
     int S;
@@ -530,8 +558,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool IGN = MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool L1 = MODE == SIM_MODE_L1;
-    __shared__ __attribute__((aligned(16))) float gs[OWG / 4 * PC * 4];
-    __shared__ __attribute__((aligned(16))) float xs[KWG / 4 * PC * 4];
+    __shared__ __attribute__((aligned(16))) float gs[OWG / 4 * PCP * 4];
+    __shared__ __attribute__((aligned(16))) float xs[KWG / 4 * PCP * 4];
     __shared__ int ktab[KWG * 2];
 
     const int tid = threadIdx.x;
@@ -539,9 +567,20 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wo = wave % WO, wk = wave / WO;
     const int lo = lane & 7, lk = lane >> 3;
-    const int ktile = blockIdx.x % a.n_ktiles, otile = blockIdx.x / a.n_ktiles;
+    // blockIdx.x -> (pixel split, tile): the tiles of one split get ids that agree mod 8, so they run on the
+    // same XCD close in time and share the split's g and x chunks through that XCD's L2
+    int split, tile_id;
+    {
+        const int per_super = 8 * a.n_tiles;
+        const int super = blockIdx.x / per_super;
+        const int within = blockIdx.x - super * per_super;
+        tile_id = within >> 3;
+        split = super * 8 + (within & 7);
+    }
+    if (split >= a.S)
+        return;  // padding of the last group of 8 splits (uniform for the workgroup)
+    const int ktile = tile_id % a.n_ktiles, otile = tile_id / a.n_ktiles;
     const int o_wg = otile * OWG, k_wg = ktile * KWG;
-    const int split = blockIdx.y;
 
     // patch element k -> offset inside an image and tap coordinates
     const int bhw = a.bh * a.bw;
@@ -555,15 +594,17 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     }
 
     // this lane's templates
-    const int o0 = o_wg + wo * 64 + lo * LO;
+    // templates of this lane: LDS rows lo and lo + 8 of its wave's 16 (4 templates each).  The 8 lanes that
+    // are served together then read 8 consecutive rows, whose pitch of PCP float4 walks through all banks.
+    auto lane_o = [&](int oo) { return o_wg + wo * 64 + (oo >> 2) * 32 + lo * 4 + (oo & 3); };
     const int k0 = k_wg + wk * 32 + lk * LK;
     float t[LO][LK], at[LO][LK], aw[LO][LK], an[NORM ? LO : 1][NORM ? LK : 1];
 #pragma unroll
     for (int oo = 0; oo < LO; ++oo)
 #pragma unroll
         for (int kk = 0; kk < LK; ++kk) {
-            const bool ok = o0 + oo < a.O && k0 + kk < a.K;
-            t[oo][kk] = ok ? a.templates[(size_t)(o0 + oo) * a.K + k0 + kk] : 0.0f;
+            const bool ok = lane_o(oo) < a.O && k0 + kk < a.K;
+            t[oo][kk] = ok ? a.templates[(size_t)lane_o(oo) * a.K + k0 + kk] : 0.0f;
             at[oo][kk] = 0.0f;
             aw[oo][kk] = 0.0f;
             if constexpr (NORM)
@@ -572,8 +613,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
 
     const int ohow = a.oh * a.ow;
     const int sp = tid & 63, sg = tid >> 6;   // staging role: pixel sp of the chunk, every 4th group
-    const float4 *g4 = reinterpret_cast<const float4 *>(gs) + (wo * 16 + lo * 2) * PC;
-    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (wk * 8 + lk) * PC;
+    const float4 *g4 = reinterpret_cast<const float4 *>(gs) + (wo * 16 + lo) * PCP;
+    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (wk * 8 + lk) * PCP;
 
     const int chunk_end = min((split + 1) * a.cps, a.nchunks);
     for (int chunk = split * a.cps; chunk < chunk_end; ++chunk) {
@@ -621,10 +662,10 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             }
 #pragma unroll
             for (int r = 0; r < OWG / 16; ++r)
-                reinterpret_cast<float4 *>(gs)[(sg + 4 * r) * PC + sp] = gv[r];
+                reinterpret_cast<float4 *>(gs)[(sg + 4 * r) * PCP + sp] = gv[r];
 #pragma unroll
             for (int r = 0; r < KWG / 16; ++r)
-                reinterpret_cast<float4 *>(xs)[(sg + 4 * r) * PC + sp] = xv[r];
+                reinterpret_cast<float4 *>(xs)[(sg + 4 * r) * PCP + sp] = xv[r];
         }
         __syncthreads();
 
@@ -671,12 +712,12 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             }
         };
         // one pixel ahead: the three reads of pixel p+1 are issued before the arithmetic of pixel p
-        float4 ga = g4[0], gb2 = g4[PC], xq = x4[0];
+        float4 ga = g4[0], gb2 = g4[8 * PCP], xq = x4[0];
         for (int p = 0; p < PC; p += 2) {
-            const float4 ga1 = g4[p + 1], gb1 = g4[PC + p + 1], xq1 = x4[p + 1];
+            const float4 ga1 = g4[p + 1], gb1 = g4[8 * PCP + p + 1], xq1 = x4[p + 1];
             compute(ga, gb2, xq);
             const int pn = p + 2 < PC ? p + 2 : p;
-            ga = g4[pn]; gb2 = g4[PC + pn]; xq = x4[pn];
+            ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
             compute(ga1, gb1, xq1);
         }
     }
@@ -688,7 +729,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     float *pn = a.partial + ((size_t)2 * a.S + split) * slab;
 #pragma unroll
     for (int oo = 0; oo < LO; ++oo) {
-        const size_t o = (size_t)(o0 + oo) * a.Kpad + k0;
+        const size_t o = (size_t)lane_o(oo) * a.Kpad + k0;
         *reinterpret_cast<float4 *>(pt + o) = make_float4(at[oo][0], at[oo][1], at[oo][2], at[oo][3]);
         *reinterpret_cast<float4 *>(pw + o) = make_float4(aw[oo][0], aw[oo][1], aw[oo][2], aw[oo][3]);
         if constexpr (NORM)
@@ -758,7 +799,7 @@ GpTiling gp_tiling(const SimPlan &p)
 template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
-    dim3 grid((unsigned)(t.n_otiles * t.n_ktiles), (unsigned)t.S);
+    dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
     if (t.WO == 2)
         hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2>), grid, dim3(kThreads), 0, s, a);
     else
@@ -782,14 +823,14 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
     if (workspace_bytes < sim_grad_params_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     const GpTiling t = gp_tiling(p);
-    if (p.bh > 0xffff || p.bw > 0xffff || t.S > 65535)
+    if (p.bh > 0xffff || p.bw > 0xffff || (long long)(t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
     GradPArgs a;
     a.g = output_grad; a.x = input; a.templates = templates;
     a.partial = reinterpret_cast<float *>(workspace);
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
     a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.K = p.K;
-    a.Opad = t.Opad; a.Kpad = t.Kpad; a.n_ktiles = t.n_ktiles;
+    a.Opad = t.Opad; a.Kpad = t.Kpad; a.n_ktiles = t.n_ktiles; a.n_tiles = t.n_otiles * t.n_ktiles;
     a.npix = (long long)p.B * p.oh * p.ow;
     a.nchunks = t.nchunks; a.cps = t.cps; a.S = t.S;
     a.oob = p.oob;
