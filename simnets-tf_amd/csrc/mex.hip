@@ -13,7 +13,7 @@
 //     so the offsets it needs, offsets[r, m, k], do not depend on the pixel; nothing is regrouped in
 //     memory, each thread maps its slot straight to the (c, h, w) it belongs to for either region
 //     flavour (contiguous "shared" tiles or interleaved "unshared" ones).
-//   * K is walked in chunks of KC: the workgroup gathers the patch elements of its pixels with the
+//   * K is walked in chunks of KC (32, or 64 / 128 for long K at one pixel per lane): the workgroup gathers the patch elements of its pixels with the
 //     im2col_3d index rule (out of image -> blocks_out_of_bounds_value) into LDS, [k][pixel], and
 //     copies the matching offsets, pre-packed [k][instance], next to them.
 //   * a lane owns PX pixels (slots lane, lane+64, ...) and its wave 16 instances: per k it reads its
@@ -40,12 +40,12 @@ namespace simnets {
 namespace {
 
 constexpr int MX = 16;        // instances per wave
-constexpr int KC = 32;        // k per LDS chunk
+constexpr int kChunkMin = 32;  // k per LDS chunk: 32, or 64 / 128 for long K with one pixel per lane
 constexpr int kXcds = 8;
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
-template <int PX, int KS, bool NEG, bool CHECK>
+template <int PX, int KS, int KC, bool NEG, bool CHECK>
 __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 {
     constexpr int WM = 4 / KS;            // instance waves per workgroup
@@ -330,22 +330,152 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         dst[(size_t)k * tm] = src[k] - lse;
 }
 
-template <int PX, int KS>
+template <int PX, int KS, int KC>
 hipError_t launch_variant(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, hipStream_t s)
 {
     if (neg && inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, true, false>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, true, false>), grid, dim3(256), 0, s, a);
     else if (neg)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, true, true>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, true, true>), grid, dim3(256), 0, s, a);
     else if (inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, false, false>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, false, false>), grid, dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, false, true>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, false, true>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
+// one pixel per lane: the LDS chunk grows with K (fewer gather/barrier phases; K <= chunk needs one gather only)
+template <int KS>
+hipError_t launch_px1(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, int kc, hipStream_t s)
+{
+    if (kc == 128)
+        return launch_variant<1, KS, 128>(a, grid, neg, inside, s);
+    if (kc == 64)
+        return launch_variant<1, KS, 64>(a, grid, neg, inside, s);
+    return launch_variant<1, KS, kChunkMin>(a, grid, neg, inside, s);
+}
+
+// Few pixels, long K (the classifier head of a network: a handful of instances over hundreds of channels at 1x1
+// spatial size): the tiling above would launch a few workgroups with long serial instruction streams.  Here one
+// wave owns one output pixel and the lanes split K: KL patch elements per lane stay in registers, and for every
+// instance the wave adds the offsets, reduces max and sum of exponentials with shuffles and lane 0 stores.  The
+// logsumexp normalisation of the offsets (python/simnets/keras.py:155-160) is folded in, so no pack launch is needed.
+constexpr int kSmallMChunk = 16;  // instances per wave
+
+template <int KL, bool NEG>
+__global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, const float *__restrict__ offsets,
+                                                        int normalize)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long gid = (long long)blockIdx.x * 4 + wave;
+    if (gid >= (long long)a.R * a.slots)
+        return;
+    const int r = (int)(gid / a.slots);
+    const int slot = (int)(gid - (long long)r * a.slots);
+    const PixelRef px = locate(a, r, slot);
+    if (px.out_off < 0)
+        return;  // ragged region edge (same for the whole wave)
+
+    const int bhw = a.bh * a.bw;
+    float x[KL];
+    bool kv[KL];
+#pragma unroll
+    for (int j = 0; j < KL; ++j) {
+        const int k = lane + 64 * j;
+        kv[j] = k < a.K;
+        const int kk = kv[j] ? k : 0;
+        const int dc = kk / bhw;
+        const int rem = kk - dc * bhw;
+        const int dh = rem / a.bw, dw = rem - dh * a.bw;
+        const int ci = px.ci0 + dc, hi = px.hi0 + dh, wi = px.wi0 + dw;
+        const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+        x[j] = ok ? px.base[((ptrdiff_t)dc * a.H + dh) * a.W + dw] : a.oob;
+    }
+    auto wave_max = [](float v) {
+        for (int d = 32; d > 0; d >>= 1) {
+            const float o = __shfl_xor(v, d, 64);
+            v = NEG ? __builtin_fminf(v, o) : __builtin_fmaxf(v, o);
+        }
+        return v;
+    };
+    auto wave_sum = [](float v) {
+        for (int d = 32; d > 0; d >>= 1)
+            v += __shfl_xor(v, d, 64);
+        return v;
+    };
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
+    const int m_end = min(a.M, (int)(blockIdx.y + 1) * kSmallMChunk);
+    for (int m = blockIdx.y * kSmallMChunk; m < m_end; ++m) {
+        const float *row = offsets + ((size_t)r * a.M + m) * a.K;
+        float o[KL];
+#pragma unroll
+        for (int j = 0; j < KL; ++j)
+            o[j] = kv[j] ? row[lane + 64 * j] : 0.0f;
+        if (normalize) {
+            float mx = -INFINITY;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                if (kv[j])
+                    mx = fmaxf(mx, o[j]);
+            for (int d = 32; d > 0; d >>= 1)
+                mx = fmaxf(mx, __shfl_xor(mx, d, 64));
+            if (!(fabsf(mx) < INFINITY))
+                mx = 0.0f;
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                if (kv[j])
+                    sum += expf(o[j] - mx);
+            const float lse = logf(wave_sum(sum)) + mx;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                o[j] -= lse;
+        }
+        float v[KL];
+        float best = NEG ? INFINITY : -INFINITY;
+#pragma unroll
+        for (int j = 0; j < KL; ++j) {
+            v[j] = x[j] + o[j];
+            if (kv[j])
+                best = NEG ? __builtin_fminf(best, v[j]) : __builtin_fmaxf(best, v[j]);
+        }
+        best = wave_max(best);
+        float res = best;
+        if (a.finite_eps) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                if (kv[j])
+                    sum += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j] - best, a.c1, a.c0));
+            res = __builtin_fmaf(__builtin_amdgcn_logf(wave_sum(sum)), a.ln2_over_eps, best);
+        }
+        if (lane == 0)
+            out[(size_t)m * plane] = res;
+    }
+}
+
+template <int KL>
+hipError_t launch_small(const MexKernelArgs &a, dim3 grid, bool neg, const float *offsets, int normalize, hipStream_t s)
+{
+    if (neg)
+        hipLaunchKernelGGL((mex_small_kernel<KL, true>), grid, dim3(256), 0, s, a, offsets, normalize);
+    else
+        hipLaunchKernelGGL((mex_small_kernel<KL, false>), grid, dim3(256), 0, s, a, offsets, normalize);
+    return hipGetLastError();
+}
+
+// the wave-per-pixel kernel pays when the tiled one would not even give every CU a workgroup
+bool mex_use_small(const MexPlan &p)
+{
+    const long long slots = (long long)p.B * p.d.region_size;
+    const long long tiled_waves = p.d.num_regions * ((slots + 63) / 64) * ((p.d.M + MX - 1) / MX);
+    return p.d.K >= 64 && p.d.K <= 64 * 16 && tiled_waves < 256 && (long long)p.d.num_regions * slots < (1LL << 31);
+}
+
 struct MexTiling {
-    int px, ks, tm, n_mgroups;
+    int px, ks, kc, tm, n_mgroups;
 };
 
 // Pixels per lane and K-split: the largest register tile that still gives every SIMD about four
@@ -368,6 +498,9 @@ MexTiling mex_tiling(const MexPlan &p)
         else if (waves(1) < 2048 && p.d.K >= 2 * 16)
             t.ks = 2;
     }
+    t.kc = kChunkMin;
+    if (t.px == 1)
+        t.kc = p.d.K >= 128 ? 128 : (p.d.K >= 64 ? 64 : kChunkMin);
     t.tm = (4 / t.ks) * MX;
     t.n_mgroups = (p.d.M + t.tm - 1) / t.tm;
     return t;
@@ -388,6 +521,26 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     const simnets_mex_dims &d = p.d;
     if (workspace_bytes < mex_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
+    if (mex_use_small(p)) {
+        MexKernelArgs a = mex_kernel_args(p);
+        a.in = input; a.out = output;
+        const long long waves = (long long)d.num_regions * a.slots;
+        dim3 grid((unsigned)((waves + 3) / 4), (unsigned)((d.M + kSmallMChunk - 1) / kSmallMChunk));
+        if (grid.y > 65535)
+            return SIMNETS_ERR_TOO_LARGE;
+        const bool neg = p.epsilon < 0;
+        const int kl = (d.K + 63) / 64;
+        hipError_t e;
+        if (kl <= 2)
+            e = launch_small<2>(a, grid, neg, offsets, p.normalize_offsets, s);
+        else if (kl <= 4)
+            e = launch_small<4>(a, grid, neg, offsets, p.normalize_offsets, s);
+        else if (kl <= 8)
+            e = launch_small<8>(a, grid, neg, offsets, p.normalize_offsets, s);
+        else
+            e = launch_small<16>(a, grid, neg, offsets, p.normalize_offsets, s);
+        return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
     const MexTiling t = mex_tiling(p);
     float *offp = reinterpret_cast<float *>(workspace);
 
@@ -415,15 +568,15 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     const bool neg = p.epsilon < 0;
     hipError_t e;
     if (t.px == 4)
-        e = launch_variant<4, 1>(a, grid, neg, inside, s);
+        e = launch_variant<4, 1, kChunkMin>(a, grid, neg, inside, s);
     else if (t.px == 2)
-        e = launch_variant<2, 1>(a, grid, neg, inside, s);
+        e = launch_variant<2, 1, kChunkMin>(a, grid, neg, inside, s);
     else if (t.ks == 1)
-        e = launch_variant<1, 1>(a, grid, neg, inside, s);
+        e = launch_px1<1>(a, grid, neg, inside, t.kc, s);
     else if (t.ks == 2)
-        e = launch_variant<1, 2>(a, grid, neg, inside, s);
+        e = launch_px1<2>(a, grid, neg, inside, t.kc, s);
     else
-        e = launch_variant<1, 4>(a, grid, neg, inside, s);
+        e = launch_px1<4>(a, grid, neg, inside, t.kc, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

@@ -287,3 +287,26 @@ def test_missing_data_stack_end_to_end(pkg):
     got = pkg.mex(cur, dev(off), 10, normalize_offsets=True, **mkw).cpu().numpy()
     assert got.shape == (B, 10, 1, 1)
     assert mex_err(got, cur.cpu().numpy(), orc.normalize_offsets(off), 10, **mkw) <= MEX_TOL
+
+
+# ---- few pixels, long K: the wave-per-pixel kernel ---------------------------------------------------------------
+@pytest.mark.parametrize("eps", [1.0, -2.0, math.inf, -math.inf])
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("case", [
+    dict(im=(20, 64, 1, 1), n=10, kw=dict(blocks=[64, 1, 1], strides=[64, 1, 1], shared_offset_region=[1])),
+    dict(im=(7, 100, 2, 3), n=5, kw=dict(blocks=[100, 1, 1], strides=[100, 1, 1], unshared_offset_region=[2])),
+    dict(im=(3, 300, 3, 2), n=17, kw=dict(blocks=[300, 1, 1], strides=[300, 1, 1], use_unshared_regions=False,
+                                          shared_offset_region=[2])),                          # ragged regions
+    dict(im=(2, 1024, 1, 1), n=3, kw=dict(blocks=[1024, 1, 1], strides=[1024, 1, 1])),
+    dict(im=(2, 9, 6, 6), n=4, kw=dict(blocks=[9, 3, 3], strides=[9, 3, 3], padding=[0, 1, 1],
+                                       blocks_out_of_bounds_value=-0.5, use_unshared_regions=False,
+                                       shared_offset_region=[-1])),                           # K = 81 with padding
+    dict(im=(2, 40, 3, 3), n=2, kw=dict(blocks=[20, 2, 2], strides=[10, 1, 1], padding=[5, 0, 0],
+                                        unshared_offset_region=[1, 2, 2])),                    # 3-D blocks, channel padding
+])
+def test_mex_few_pixels_long_patches(pkg, case, normalize, eps):
+    kw = dict(case["kw"], epsilon=eps, softmax_mode=normalize)
+    x, off = mex_inputs(31, case["im"], case["n"], **kw)
+    ref_off = orc.normalize_offsets(off) if normalize else off
+    got = run_mex(pkg, x, off, case["n"], normalize_offsets=normalize, **kw)
+    assert mex_err(got, x, ref_off, case["n"], **kw) <= MEX_TOL
