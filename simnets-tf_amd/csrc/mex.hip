@@ -42,6 +42,9 @@ namespace {
 constexpr int MX = 16;        // instances per wave
 constexpr int kChunkMin = 32;  // k per LDS chunk: 32, or 64 / 128 for long K with one pixel per lane
 constexpr int kXcds = 8;
+#ifndef SIMNETS_MEX_WAVES
+#define SIMNETS_MEX_WAVES 4096  // pixels per lane shrink until the grid has this many waves
+#endif
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
@@ -489,7 +492,7 @@ MexTiling mex_tiling(const MexPlan &p)
     auto waves = [&](int px) { return p.d.num_regions * ((slots + 64 * px - 1) / (64 * px)) * mtiles; };
     MexTiling t;
     t.px = 4;
-    while (t.px > 1 && waves(t.px) < 4096)
+    while (t.px > 1 && waves(t.px) < SIMNETS_MEX_WAVES)
         t.px >>= 1;
     t.ks = 1;
     if (t.px == 1) {
