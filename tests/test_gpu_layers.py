@@ -117,3 +117,23 @@ def test_a_small_network_trains(pkg):
         opt.step()
         losses.append(loss.item())
     assert losses[-1] < losses[0]
+
+
+def test_layerwise_unsupervised_initialisation(pkg):
+    """perform_unsupervised_init walks the network like python/simnets/keras.py:199-243: each Similarity layer is
+    initialised from what the already initialised layers before it produce."""
+    torch.manual_seed(5)
+    net = torch.nn.Sequential(
+        pkg.Similarity(6, blocks=[2, 2], strides=[2, 2], padding=[0, 0]),
+        pkg.Mex(4, blocks=[-1, 1, 1], strides=[6, 1, 1], softmax_mode=True, normalize_offsets=True),
+        pkg.Similarity(3, blocks=[2, 2], strides=[1, 1], padding=[0, 0]),
+    )
+    data = torch.randn(32, 2, 8, 8).cuda()
+    net(data[:2])    # builds the lazily shaped parameters
+    before = [net[0].templates.detach().clone(), net[2].templates.detach().clone()]
+    pkg.unsupervised.perform_unsupervised_init(net, "kmeans", data=data, batch_size=8)
+    assert not torch.equal(net[0].templates, before[0]) and not torch.equal(net[2].templates, before[1])
+    assert torch.equal(net[0].sweights, torch.ones_like(net[0].sweights))
+    # the first layer's templates are means of input patches: inside the data's range
+    assert net[0].templates.abs().max() <= data.abs().max()
+    assert torch.isfinite(net(data)).all()
