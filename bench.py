@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the SimNets Similarity / MEX hot path on one MI355X.
 
-One "step" = one Similarity L2 forward over BASELINE configuration 3 (input 256x64x32x32, 128
+One "step" = one Similarity L2 forward over benchmark configuration 3 (input 256x64x32x32, 128
 templates 64x3x3, stride 1, padding 1 -> 256x128x32x32; 19.33 G generalized MACs), inputs already
 resident in HBM, called through the C ABI exactly as an op layer would.  The other configurations
 (1, 2, 3-L1, 4, and the backward operators of configuration 5) and the alternative evaluation paths
@@ -48,7 +48,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path is data parallel over the batch; "
-              "see DESIGN.md for how it would shard); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+              "each GPU would take a share of the images); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         sys.exit(2)
 
     import numpy as np

@@ -3,7 +3,7 @@
 //   simnets_bench --peaks                      machine micro-benchmarks (unpacked FP32 FMA issue rate,
 //                                              fp32 MFMA rate, v_exp_f32 rate, HBM copy bandwidth)
 //   simnets_bench --config N [--algo A] [--steps K] [--warmup W]     (N = 1..4 forward, 5 backward)
-//                                              N in 1..4: times that BASELINE configuration through the
+//                                              N in 1..4: times that benchmark configuration through the
 //                                              C ABI with hipEvents on its own stream
 // Prints one JSON object per measurement.  Inputs are synthetic (fixed-seed counter-based generator),
 // resident in HBM before timing starts.  Parity is not checked here (tests/ does that through the same

@@ -79,19 +79,20 @@ __device__ __forceinline__ void gx_step(float (&acc)[MT][PT], const float (&xv)[
             for (int p = 0; p < PT; ++p)
                 u[p] = __builtin_fmaf(p1, xv[m][p], p0);
         } else {
-            // (t, w): u = w * sign(t - x), sign(0) = sign(NaN) = 0
+            // (copysign(2^100, w) * t, w): d = +-2^100 * (t - x) is either 0 or far outside [-|w|, |w|], so its
+            // median with -|w| and |w| is w * sign(t - x) (exactly 0 for t == x).  NaN inputs never get here:
+            // the tile holds 0 in their place and their gradient is stored as 0, which is what sign(NaN) = 0
+            // gives in the reference.
+            const float nbig = -__builtin_copysignf(0x1p100f, p1);
+            const float lim = __builtin_fabsf(p1);
             float d[PT];
 #pragma unroll
             for (int p = 0; p < PT; ++p)
-                d[p] = p0 - xv[m][p];
+                d[p] = __builtin_fmaf(nbig, xv[m][p], p0);
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int p = 0; p < PT; ++p)
-                u[p] = __builtin_copysignf(p1, d[p]);
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int p = 0; p < PT; ++p)
-                u[p] = __builtin_islessgreater(d[p], 0.0f) ? u[p] : 0.0f;
+                u[p] = __builtin_amdgcn_fmed3f(d[p], -lim, lim);
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -148,7 +149,7 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
             float val = 0.0f;
             if (wave_active && lane_valid && c < a.C && v0 + p < a.nb)
                 val = xrow[(size_t)c * plane + (size_t)a.sw * (v0 + p)];
-            if (a.ignore_nan && !(val == val))
+            if ((a.ignore_nan || MODE == GX_L1) && !(val == val))
                 val = 0.0f;
             xv[m][p] = val;
         }
@@ -235,7 +236,7 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
                 continue;
             const size_t o = (size_t)c * plane + (size_t)a.sw * (v0 + p);
             float val = (row_covered && v0 + p <= a.col_limit) ? acc[m][p] : 0.0f;
-            if (a.ignore_nan) {
+            if (a.ignore_nan || MODE == GX_L1) {
                 const float xin = xrow[o];
                 if (!(xin == xin))
                     val = 0.0f;
@@ -332,7 +333,7 @@ __global__ void sim_grad_input_pack_kernel(const float *__restrict__ templates, 
             const size_t pi = (((size_t)o * C + c) * bh + i) * bw + j;
             const float t = templates[pi], w = weights[pi];
             if (l1) {
-                p0 = t;
+                p0 = copysignf(0x1p100f, w) * t;
                 p1 = w;
             } else {
                 p0 = scale * w * t;

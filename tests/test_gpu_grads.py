@@ -303,3 +303,14 @@ def test_mex_grads_empty_batch(pkg):
     y = np.zeros((0, 2, 4, 4), np.float32)
     assert pkg.mex_input_grad(dev(x), dev(off), dev(y), dev(y), 2, **kw).shape == x.shape
     assert not pkg.mex_offsets_grad(dev(x), dev(off), dev(y), dev(y), 2, **kw).cpu().numpy().any()
+
+
+def test_similarity_l1_grads_at_ties_and_nan(pkg):
+    """sign(0) = sign(NaN) = 0 in the reference's L1 functors (similarity_utils.hpp:82-84, :121-125): inputs that
+    equal a template entry exactly, NaN inputs and zero weights."""
+    x, t, w = sim_inputs(21, (2, 2, 9, 9), 3, (3, 3))
+    t[0, 0, 1, 1] = x[0, 0, 4, 4]          # the centre tap of template 0 meets this pixel exactly
+    x[1, 1, :, 3] = t[1, 1, 0, 0]          # a whole column equal to one template entry
+    x[0, 1, 2, 2] = np.nan
+    w[2, 0, 2, 2] = 0.0
+    check_sim_grads(pkg, x, t, w, similarity_function="L1", blocks=[3, 3], strides=[1, 1], padding=[1, 1])

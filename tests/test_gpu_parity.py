@@ -147,7 +147,7 @@ def test_config3_similarity_mfma_sampled(pkg):
     assert rel_err(got, direct) <= SIM_TOL
 
 
-# ---- BASELINE configurations ------------------------------------------------------------------------
+# ---- benchmark configurations ------------------------------------------------------------------------
 def test_config1_similarity_missing_data_layer(pkg):
     x, t, w, kw = config1(batch=64, nan_frac=0.25)
     got, want = run_similarity(pkg, x, t, w, **kw), orc.similarity_fwd(x, t, w, **kw)
@@ -262,7 +262,7 @@ def test_sum_pooling(pkg):
 
 
 def test_missing_data_stack_end_to_end(pkg):
-    # BASELINE configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10).
+    # benchmark configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10).
     # Each layer is checked on the GPU's own previous activations, so tolerances do not compound.
     B = 16
     x, t, w, kw = config1(batch=B, nan_frac=0.25)
