@@ -1,0 +1,110 @@
+"""Seeded random sweep over the attribute space of both operators, forward and backward, against the oracle.
+Every case prints nothing and is small; the point is breadth (block/stride/padding combinations, template
+counts around the tile sizes, region specifications, epsilon signs) beyond the hand-picked cases."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle as orc
+from util import rel_err
+from test_gpu_grads import assert_grad_close, f64
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def random_similarity_case(g):
+    while True:
+        C = int(g.choice([1, 2, 3, 5, 8, 9, 17, 33]))
+        O = int(g.choice([1, 2, 7, 8, 9, 16, 31, 40, 65]))
+        H, W = int(g.integers(3, 40)), int(g.integers(3, 70))
+        bh, bw = int(g.integers(1, min(H, 6) + 1)), int(g.integers(1, min(W, 6) + 1))
+        sh, sw = int(g.integers(1, 5)), int(g.integers(1, 5))
+        ph, pw = int(g.integers(0, bh + 1)), int(g.integers(0, bw + 1))
+        mode = int(g.integers(0, 4))
+        kw = dict(similarity_function="L1" if mode == 0 else "L2", blocks=[bh, bw], strides=[sh, sw], padding=[ph, pw],
+                  normalization_term=mode >= 2, ignore_nan_input=mode == 3,
+                  out_of_bounds_value=float("nan") if mode == 3 else float(g.normal()))
+        B = int(g.integers(1, 4))
+        try:
+            orc.similarity_out_dims(orc.similarity_args((B, C, H, W), O, **{k: v for k, v in kw.items()}))
+        except ValueError:
+            continue
+        x = g.normal(size=(B, C, H, W)).astype(np.float32)
+        if mode == 3:
+            x[g.random(size=x.shape) < 0.2] = np.nan
+        t = g.normal(size=(O, C, bh, bw)).astype(np.float32)
+        w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+        return x, t, w, kw
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_similarity_random_geometry(pkg, seed):
+    g = np.random.default_rng(1000 + seed)
+    x, t, w, kw = random_similarity_case(g)
+    want = orc.similarity_fwd(x, t, w, **kw)
+    got = pkg.similarity(dev(x), dev(t), dev(w), **kw).cpu().numpy()
+    assert rel_err(got, want) <= 1e-5, kw
+    go = g.normal(size=want.shape).astype(np.float32)
+    dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(go), **kw).cpu().numpy()
+    dt, dw = [a.cpu().numpy() for a in pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(go), **kw)]
+    d = f64(x, t, w, go)
+    assert_grad_close(dx, orc.similarity_input_grad(x, t, w, go, **kw), orc.similarity_input_grad(*d, **kw), "dX %s" % kw)
+    w32, w64 = orc.similarity_params_grad(x, t, w, go, **kw), orc.similarity_params_grad(*d, **kw)
+    assert_grad_close(dt, w32[0], w64[0], "dT %s" % kw)
+    assert_grad_close(dw, w32[1], w64[1], "dW %s" % kw)
+
+
+def random_mex_case(g):
+    while True:
+        C, H, W = int(g.choice([1, 2, 3, 6, 16, 70])), int(g.integers(1, 14)), int(g.integers(1, 14))
+        blocks = [int(g.integers(1, C + 1)), int(g.integers(1, min(H, 4) + 1)), int(g.integers(1, min(W, 4) + 1))]
+        strides = [int(g.integers(1, blocks[0] + 2)), int(g.integers(1, 4)), int(g.integers(1, 4))]
+        padding = [int(g.integers(0, blocks[0])), int(g.integers(0, blocks[1])), int(g.integers(0, blocks[2]))]
+        unshared = bool(g.integers(0, 2))
+        spec = [[-1], [1], [2], [3], [1, 2, 3], [2, 1, 2], [-1, 2, -1]][int(g.integers(0, 7))]
+        eps = [1.0, -1.0, 0.5, 3.0, -2.5, math.inf, -math.inf][int(g.integers(0, 7))]
+        kw = dict(blocks=blocks, strides=strides, padding=padding, epsilon=eps, softmax_mode=bool(g.integers(0, 2)),
+                  blocks_round_down=bool(g.integers(0, 2)), blocks_out_of_bounds_value=float(g.normal()),
+                  use_unshared_regions=unshared, shared_offset_region=spec, unshared_offset_region=spec)
+        n = int(g.choice([1, 2, 5, 16, 17, 40]))
+        B = int(g.integers(1, 5))
+        try:
+            d = orc.mex_dims(orc.mex_args((B, C, H, W), n, **kw))
+        except ValueError:
+            continue
+        if d.num_regions * n * d.K > 200000:
+            continue
+        x = g.normal(size=(B, C, H, W)).astype(np.float32)
+        off = g.normal(size=(d.num_regions, n) + tuple(blocks)).astype(np.float32)
+        return x, off, n, kw
+
+
+@pytest.mark.parametrize("seed", range(60))
+def test_mex_random_geometry(pkg, seed):
+    g = np.random.default_rng(2000 + seed)
+    x, off, n, kw = random_mex_case(g)
+    want = orc.mex_fwd(x, off, n, **kw)
+    shift = orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, kw["epsilon"])))
+    got = pkg.mex(dev(x), dev(off), n, **kw)
+    assert rel_err(got.cpu().numpy(), want, floor=shift) <= 1e-4, kw
+    go = g.normal(size=want.shape).astype(np.float32)
+    dx = pkg.mex_input_grad(dev(x), dev(off), dev(want), dev(go), n, **kw).cpu().numpy()
+    doff = pkg.mex_offsets_grad(dev(x), dev(off), dev(want), dev(go), n, **kw).cpu().numpy()
+    x64, off64, g64 = f64(x, off, go)
+    out64 = orc.mex_fwd(x64, off64, n, **kw)
+    if math.isinf(kw["epsilon"]):
+        # the indicator (patch + offset == out) is evaluated on the fp32 data the op saw: compare with the fp32 oracle
+        assert rel_err(dx, orc.mex_input_grad(x, off, want, go, n, **kw), floor=np.full(dx.shape, 1e-2 * np.abs(dx).max())) <= 1e-4, kw
+        assert rel_err(doff, orc.mex_offsets_grad(x, off, want, go, n, **kw),
+                       floor=np.full(doff.shape, 1e-2 * np.abs(doff).max())) <= 1e-4, kw
+    else:
+        assert_grad_close(dx, orc.mex_input_grad(x, off, want, go, n, **kw),
+                          orc.mex_input_grad(x64, off64, out64, g64, n, **kw), "dX %s" % kw)
+        assert_grad_close(doff, orc.mex_offsets_grad(x, off, want, go, n, **kw),
+                          orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "dOff %s" % kw)
