@@ -23,7 +23,8 @@ from .ops import (  # noqa: F401
 
 from . import layers  # noqa: F401,E402
 from . import unsupervised  # noqa: F401,E402
+from . import torch_ops  # noqa: F401,E402  (registers torch.ops.simnets.*)
 from .layers import Similarity, Mex, dirichlet_init  # noqa: F401,E402
 
-__all__ = ["layers", "unsupervised", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError",
+__all__ = ["layers", "unsupervised", "torch_ops", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "similarity_output_shape", "mex_output_shape", "SimnetsError",
            "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad"]
