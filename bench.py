@@ -185,10 +185,24 @@ def main():
                            strides=[ch, 1, 1], shared_offset_region=[1])
 
         _, ms = timed(stack, args.steps, args.warmup)
+        # the same stack captured once into a HIP graph and replayed: 15 launches without per-launch host work
+        stack()
+        torch.cuda.synchronize()
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            stack()
+        torch.cuda.current_stream().wait_stream(side)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            graph_out = stack()
+        _, ms_graph = timed(graph.replay, args.steps, args.warmup)
+        graph_ok = bool(torch.equal(graph_out, stack()))
         gmac4 = 512 * 32 * 256 * 4 + 4 * 268435456 + 512 * 10 * 512
         others["config4_stack"] = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(gmac4 / (ms * 1e-3) / 1e9, 1),
                                    "exp_frac": round(gmac4 / (ms * 1e-3) / EXP_RATE, 4), "batch": 512,
-                                   "kernels": "similarity + 5 x (offset pack + mex) + 4 x sum pool"}
+                                   "kernels": "similarity + 4 x (offset pack + mex + sum pool) + wave-per-pixel mex",
+                                   "hip_graph_replay_ms": round(ms_graph, 4), "hip_graph_matches_eager": graph_ok}
         # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
         _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,

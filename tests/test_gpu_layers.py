@@ -137,3 +137,48 @@ def test_layerwise_unsupervised_initialisation(pkg):
     # the first layer's templates are means of input patches: inside the data's range
     assert net[0].templates.abs().max() <= data.abs().max()
     assert torch.isfinite(net(data)).all()
+
+
+def test_missing_data_stack_replays_from_a_hip_graph(pkg):
+    """The whole stack (Similarity -> 4 x (MEX + sum pool) -> MEX) is kernel launches on the caller's stream and
+    nothing else (no allocation, no memset, no host synchronisation once the workspace exists), so it can be
+    captured once and replayed.  Every replay, with new input contents and eager work in between, must reproduce the
+    eager result bit for bit."""
+    from util import config1
+    x, t, w, kw = config1(batch=32, nan_frac=0.25)
+    T, W = torch.from_numpy(t).cuda(), torch.from_numpy(w).cuda()
+    g = np.random.default_rng(4567)
+    layers, ch, size = [], 32, 16
+    for _ in range(4):
+        n = ch * 2
+        off = torch.from_numpy((g.normal(size=(4 if size > 1 else 1, n, ch, 1, 1)) * 0.1).astype(np.float32)).cuda()
+        layers.append((off, n, dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], unshared_offset_region=[2])))
+        ch, size = n, size // 2
+    offl = torch.from_numpy((g.normal(size=(1, 10, ch, 1, 1)) * 0.1).astype(np.float32)).cuda()
+
+    def stack(inp):
+        cur = pkg.similarity(inp, T, W, **kw)
+        for off, n, lkw in layers:
+            cur = pkg.sum_pooling(pkg.mex(cur, off, n, normalize_offsets=True, **lkw), (2, 2))
+        return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1],
+                       shared_offset_region=[1])
+
+    static_in = torch.from_numpy(x).cuda()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):          # warm-up on the capture stream: workspace and allocator pools exist afterwards
+            stack(static_in)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = stack(static_in)
+    for trial in range(4):
+        fresh, _, _, _ = config1(batch=32, seed=100 + trial, nan_frac=0.25)
+        static_in.copy_(torch.from_numpy(fresh))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = static_out.clone()
+        want = stack(torch.from_numpy(fresh).cuda())     # eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), "replay %d" % trial
