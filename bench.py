@@ -34,8 +34,8 @@ MEASURED_TRAFFIC_BYTES = {"direct": 287.0e6, "mfma": 223.3e6}
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--algo", default=None, choices=[None, "direct", "sqrtw", "mfma"],
                     help="evaluation path of the headline Similarity kernel (default: the library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
