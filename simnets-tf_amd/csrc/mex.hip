@@ -23,8 +23,10 @@
 //   * the 4 waves of a workgroup split the instances (WM ways) and, when the grid would otherwise
 //     leave SIMDs idle, K (KS ways, WM*KS = 4): each K-split wave keeps its own (max, sum) pair and
 //     the pairs are merged through LDS at the end: sum = sum_i s_i * exp(eps*(m_i - max_i m_i)).
-//   * two sweeps over K like the reference (max, then sum of exp relative to the max); exp is
-//     v_exp_f32 on a pre-scaled argument.  When K fits one chunk the second sweep reuses the LDS tile.
+//   * two sweeps over K like the reference (max, then sum of exp relative to the max).  For finite
+//     eps the patch values (when staged) and the offsets (when packed) are multiplied by eps*log2(e)
+//     once, so a term of the second sweep is add, subtract, v_exp_f32, add; a negative eps turns the
+//     reference's minimum into a maximum of the scaled values.  When K fits one chunk the second sweep reuses the LDS tile.
 //   * workgroups that own the different regions of the same pixel chunk are numbered a multiple of
 //     8 apart, so they run on the same XCD and their interleaved partial cache lines meet in one L2.
 #include <hip/hip_runtime.h>
@@ -116,7 +118,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             for (int u = 0; u < U; ++u) {
                 const int kk = kk0 + u * KSTEP;
                 if (kk < kc)
-                    xs[kk * TP + sp] = v[u];
+                    xs[kk * TP + sp] = v[u] * a.scale;
             }
         }
         // offsets: a straight copy of kc * TM floats
@@ -178,12 +180,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
         for (int m = 0; m < MX; ++m)
             s[p][m] = 0.0f;
     if (a.finite_eps) {
-        // ---- sweep 2: sum of exp(eps * (v - max) + ey), evaluated as exp2 of the scaled argument ----
-        // the two scale constants are wave-uniform; they are used from VGPRs because VALU instructions
-        // with SGPR operands issue at half rate
-        float c1v, c0v;
-        asm("v_mov_b32 %0, %1" : "=v"(c1v) : "s"(a.c1));
-        asm("v_mov_b32 %0, %1" : "=v"(c0v) : "s"(a.c0));
+        // ---- sweep 2: sum of exp(eps * (v - max)): patch values and offsets are already multiplied by
+        //      eps*log2(e), so the term is exp2 of a plain difference ----
         for (int k0 = 0; k0 < a.K; k0 += KC) {
             const int kc = min(KC, a.K - k0);
             if (!single_chunk) {
@@ -212,10 +210,6 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 #pragma unroll
                     for (int m = 0; m < MX; ++m)
                         v[m] = v[m] - mx[p][m];
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        v[m] = __builtin_fmaf(v[m], c1v, c0v);
                     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                     for (int m = 0; m < MX; ++m)
@@ -259,8 +253,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                         const float mm = NEG ? __builtin_fminf(m1, m2) : __builtin_fmaxf(m1, m2);
                         // a side that saw no finite term keeps sum 0; skip the rescale when its
                         // max equals the merged one (also avoids inf - inf)
-                        const float f1 = (m1 == mm) ? 1.0f : __builtin_amdgcn_exp2f((m1 - mm) * a.c1);
-                        const float f2 = (m2 == mm) ? 1.0f : __builtin_amdgcn_exp2f((m2 - mm) * a.c1);
+                        const float f1 = (m1 == mm) ? 1.0f : __builtin_amdgcn_exp2f(m1 - mm);
+                        const float f2 = (m2 == mm) ? 1.0f : __builtin_amdgcn_exp2f(m2 - mm);
                         s[p][m] = s[p][m] * f1 + s2 * f2;
                         mx[p][m] = mm;
                     }
@@ -280,8 +274,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
         float *o = a.out + (size_t)cp.b * a.M * plane + cp.out_off;
 #pragma unroll
         for (int m = 0; m < MX; ++m) {
-            // max + log(sum) / eps, the logarithm taken as log2 (v_log_f32) * log(2)/eps
-            const float res = a.finite_eps ? __builtin_fmaf(__builtin_amdgcn_logf(s[p][m]), a.ln2_over_eps, mx[p][m])
+            // (max + ey*log2(e) + log2(sum)) * log(2)/eps in the scaled domain; the plain max for infinite eps
+            const float res = a.finite_eps ? (__builtin_amdgcn_logf(s[p][m]) + (mx[p][m] + a.c0)) * a.ln2_over_eps
                                            : mx[p][m];
             if (m0 + m < a.M)
                 o[(size_t)(m0 + m) * plane] = res;
@@ -293,7 +287,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 // (python/simnets/keras.py:155-160), then the row is scattered into the k-major packed layout
 // [r][mgroup][k][tm].
 __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__restrict__ offsets, int R, int M, int K,
-                                                              int n_mgroups, int tm, int normalize,
+                                                              int n_mgroups, int tm, int normalize, float scale,
                                                               float *__restrict__ offp)
 {
     const int lane = threadIdx.x & 63;
@@ -330,7 +324,7 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         lse = logf(sum) + mxv;
     }
     for (int k = lane; k < K; k += 64)
-        dst[(size_t)k * tm] = src[k] - lse;
+        dst[(size_t)k * tm] = (src[k] - lse) * scale;
 }
 
 template <int PX, int KS, int KC>
@@ -547,13 +541,13 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     const MexTiling t = mex_tiling(p);
     float *offp = reinterpret_cast<float *>(workspace);
 
+    MexKernelArgs a = mex_kernel_args(p);
     const long long rows = (long long)d.num_regions * t.n_mgroups * t.tm;
     hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, offsets,
-                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, offp);
+                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, a.scale, offp);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
 
-    MexKernelArgs a = mex_kernel_args(p);
     a.in = input; a.out = output; a.offp = offp;
     a.n_mgroups = t.n_mgroups;
 
@@ -568,7 +562,8 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     if (gx > 0x7fffffffLL || t.n_mgroups > 65535)
         return SIMNETS_ERR_TOO_LARGE;
     dim3 grid((unsigned)gx, (unsigned)t.n_mgroups);
-    const bool neg = p.epsilon < 0;
+    // finite eps: values are pre-multiplied by eps*log2(e), so the shift is always the maximum
+    const bool neg = !a.finite_eps && p.epsilon < 0;
     hipError_t e;
     if (t.px == 4)
         e = launch_variant<4, 1, kChunkMin>(a, grid, neg, inside, s);

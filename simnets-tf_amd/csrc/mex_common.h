@@ -25,6 +25,7 @@ struct MexKernelArgs {
     int cpr;            // pixel chunks (64*PX slots) per region
     int M, K, n_mgroups;
     float c1;           // eps * log2(e)
+    float scale;        // what the tiled kernel multiplies patch values and offsets by: c1 for finite eps, else 1
     float c0;           // (softmax ? 0 : -log K) * log2(e)
     float ln2_over_eps; // log(2) / eps
     int finite_eps;
@@ -93,6 +94,7 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     const double log2e = 1.4426950408889634;
     a.finite_eps = std::isfinite(p.epsilon);
     a.c1 = a.finite_eps ? (float)((double)p.epsilon * log2e) : 0.0f;
+    a.scale = a.finite_eps ? a.c1 : 1.0f;
     a.ln2_over_eps = a.finite_eps ? (float)(0.6931471805599453 / (double)p.epsilon) : 0.0f;
     // ey = softmax ? 0 : (float)-log(K)   (src/kernels/mex_kernel_cpu.cpp:36)
     const float ey = p.softmax_mode ? 0.0f : (float)-std::log((double)d.K);
