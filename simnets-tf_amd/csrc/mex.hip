@@ -59,9 +59,15 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     constexpr int KSTEP = 256 / TP;       // k handled per staging round (4, 2 or 1)
     constexpr int KW = KC / KS;           // k of a chunk each K-split wave walks
     constexpr int kMergeFloats = (KS - 1) * WM * 64 * PX * MX * 2;
-    __shared__ __attribute__((aligned(16))) float smem[cmax(KC * TP + KC * TM, kMergeFloats)];
-    float *xs = smem;                     // [k][pixel]
-    float *os = smem + KC * TP;           // [k][instance]
+    // The k-oriented gather (below) writes xs with lanes along k: its rows get a pitch of TP + 1 floats so
+    // that those writes spread over the banks.  Only the K-split variants can take it (LDS room).
+    constexpr bool KGATHER = PX == 1 && KS >= 2;
+    constexpr int XP = KGATHER ? TP + 1 : TP;   // KC * XP stays a multiple of 4: the offsets tile behind it is 16-byte aligned
+    __shared__ __attribute__((aligned(16))) float smem[cmax(KC * XP + KC * TM, kMergeFloats)];
+    __shared__ long long pref_off[KGATHER ? 64 : 1];
+    __shared__ int pref_c[KGATHER ? 64 * 3 : 1];
+    float *xs = smem;                     // [k][pixel], row pitch XP
+    float *os = smem + KC * XP;           // [k][instance]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -88,11 +94,47 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     const PixelRef gp = locate(a, r, chunk * TP + sp);
     const int bhw = a.bh * a.bw;
     const float *offp = a.offp + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
+    if (KGATHER && a.kgather && tid < 64) {
+        // pixel table for the k-oriented gather: where each of the 64 pixels' patches starts
+        pref_off[tid] = gp.base - a.in;
+        pref_c[3 * tid] = gp.ci0; pref_c[3 * tid + 1] = gp.hi0; pref_c[3 * tid + 2] = gp.wi0;
+    }
 
     auto stage = [&](int k0, int kc) {
+        if (KGATHER && a.kgather) {
+            // Consecutive pixel slots are different images here (one pixel per image and region), a whole image
+            // apart in memory, while consecutive patch elements are one channel plane apart: lanes run along k.
+            // Thread (kq, pq) gathers elements kq, kq + 64, ... of pixels pq, pq + 4, ...
+            const int kq = tid & 63, pq = tid >> 6;   // (the pixel table was written before the barrier in front of this call)
+            for (int kk = kq; kk < kc; kk += 64) {
+                const int k = k0 + kk;
+                int dc = k, dh = 0, dw = 0;
+                if (bhw != 1) {
+                    dc = k / bhw;
+                    const int rem = k - dc * bhw;
+                    dh = rem / a.bw;
+                    dw = rem - dh * a.bw;
+                }
+                const ptrdiff_t o = ((ptrdiff_t)dc * a.H + dh) * a.W + dw;
+                float v[16];
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    const int p = pq + 4 * i;
+                    bool ok = true;
+                    if (CHECK) {
+                        const int ci = pref_c[3 * p] + dc, hi = pref_c[3 * p + 1] + dh, wi = pref_c[3 * p + 2] + dw;
+                        ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                    }
+                    v[i] = ok ? a.in[pref_off[p] + o] : a.oob;
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i)
+                    xs[kk * XP + pq + 4 * i] = v[i] * a.scale;
+            }
+        } else
         // patch elements: xs[kk][sp] = patch(sp)[k0 + kk]
-        constexpr int U = KC / KSTEP;  // gathers per thread and chunk: all in flight before the first LDS store
-        for (int kk0 = sk; kk0 < kc; kk0 += KSTEP * U) {
+        for (int kk0 = sk; kk0 < kc; kk0 += KSTEP * (KC / KSTEP)) {
+            constexpr int U = KC / KSTEP;  // gathers per thread and chunk: all in flight before the first LDS store
             float v[U];
 #pragma unroll
             for (int u = 0; u < U; ++u) {
@@ -118,7 +160,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             for (int u = 0; u < U; ++u) {
                 const int kk = kk0 + u * KSTEP;
                 if (kk < kc)
-                    xs[kk * TP + sp] = v[u] * a.scale;
+                    xs[kk * XP + sp] = v[u] * a.scale;
             }
         }
         // offsets: a straight copy of kc * TM floats
@@ -152,7 +194,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             float x[PX], o[MX];
 #pragma unroll
             for (int p = 0; p < PX; ++p)
-                x[p] = xl[kk * TP + p * 64];
+                x[p] = xl[kk * XP + p * 64];
 #pragma unroll
             for (int m = 0; m < MX; ++m)
                 o[m] = ol[kk * TM + m];
@@ -196,7 +238,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                 float x[PX], o[MX];
 #pragma unroll
                 for (int p = 0; p < PX; ++p)
-                    x[p] = xl[kk * TP + p * 64];
+                    x[p] = xl[kk * XP + p * 64];
 #pragma unroll
                 for (int m = 0; m < MX; ++m)
                     o[m] = ol[kk * TM + m];
@@ -389,67 +431,101 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, c
         const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
         x[j] = ok ? px.base[((ptrdiff_t)dc * a.H + dh) * a.W + dw] : a.oob;
     }
-    auto wave_max = [](float v) {
-        for (int d = 32; d > 0; d >>= 1) {
-            const float o = __shfl_xor(v, d, 64);
-            v = NEG ? __builtin_fminf(v, o) : __builtin_fmaxf(v, o);
-        }
-        return v;
-    };
-    auto wave_sum = [](float v) {
+    // four instances at a time: their shuffle reductions are independent, so the latencies overlap
+    constexpr int MG = 4;
+    auto wave_sum = [](float (&v)[MG]) {
         for (int d = 32; d > 0; d >>= 1)
-            v += __shfl_xor(v, d, 64);
-        return v;
+#pragma unroll
+            for (int g = 0; g < MG; ++g)
+                v[g] += __shfl_xor(v[g], d, 64);
+    };
+    auto wave_best = [](float (&v)[MG], bool neg) {
+        for (int d = 32; d > 0; d >>= 1)
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                const float o = __shfl_xor(v[g], d, 64);
+                v[g] = neg ? __builtin_fminf(v[g], o) : __builtin_fmaxf(v[g], o);
+            }
     };
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
     const int m_end = min(a.M, (int)(blockIdx.y + 1) * kSmallMChunk);
-    for (int m = blockIdx.y * kSmallMChunk; m < m_end; ++m) {
-        const float *row = offsets + ((size_t)r * a.M + m) * a.K;
-        float o[KL];
+    for (int m0 = blockIdx.y * kSmallMChunk; m0 < m_end; m0 += MG) {
+        float o[MG][KL];
 #pragma unroll
-        for (int j = 0; j < KL; ++j)
-            o[j] = kv[j] ? row[lane + 64 * j] : 0.0f;
+        for (int g = 0; g < MG; ++g) {
+            const float *row = offsets + ((size_t)r * a.M + min(m0 + g, a.M - 1)) * a.K;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                o[g][j] = kv[j] ? row[lane + 64 * j] : 0.0f;
+        }
         if (normalize) {
-            float mx = -INFINITY;
+            float mx[MG], sum[MG];
 #pragma unroll
-            for (int j = 0; j < KL; ++j)
-                if (kv[j])
-                    mx = fmaxf(mx, o[j]);
-            for (int d = 32; d > 0; d >>= 1)
-                mx = fmaxf(mx, __shfl_xor(mx, d, 64));
-            if (!(fabsf(mx) < INFINITY))
-                mx = 0.0f;
-            float sum = 0.0f;
+            for (int g = 0; g < MG; ++g) {
+                mx[g] = -INFINITY;
 #pragma unroll
-            for (int j = 0; j < KL; ++j)
-                if (kv[j])
-                    sum += expf(o[j] - mx);
-            const float lse = logf(wave_sum(sum)) + mx;
+                for (int j = 0; j < KL; ++j)
+                    if (kv[j])
+                        mx[g] = fmaxf(mx[g], o[g][j]);
+            }
+            wave_best(mx, false);
 #pragma unroll
-            for (int j = 0; j < KL; ++j)
-                o[j] -= lse;
+            for (int g = 0; g < MG; ++g) {
+                if (!(fabsf(mx[g]) < INFINITY))
+                    mx[g] = 0.0f;
+                sum[g] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < KL; ++j)
+                    if (kv[j])
+                        sum[g] += expf(o[g][j] - mx[g]);
+            }
+            wave_sum(sum);
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                const float lse = logf(sum[g]) + mx[g];
+#pragma unroll
+                for (int j = 0; j < KL; ++j)
+                    o[g][j] -= lse;
+            }
         }
-        float v[KL];
-        float best = NEG ? INFINITY : -INFINITY;
+        float best[MG];
 #pragma unroll
-        for (int j = 0; j < KL; ++j) {
-            v[j] = x[j] + o[j];
-            if (kv[j])
-                best = NEG ? __builtin_fminf(best, v[j]) : __builtin_fmaxf(best, v[j]);
+        for (int g = 0; g < MG; ++g) {
+            best[g] = NEG ? INFINITY : -INFINITY;
+#pragma unroll
+            for (int j = 0; j < KL; ++j) {
+                o[g][j] += x[j];   // patch + offset
+                if (kv[j])
+                    best[g] = NEG ? __builtin_fminf(best[g], o[g][j]) : __builtin_fmaxf(best[g], o[g][j]);
+            }
         }
-        best = wave_max(best);
-        float res = best;
+        wave_best(best, NEG);
+        float res[MG];
+#pragma unroll
+        for (int g = 0; g < MG; ++g)
+            res[g] = best[g];
         if (a.finite_eps) {
-            float sum = 0.0f;
+            float sum[MG];
 #pragma unroll
-            for (int j = 0; j < KL; ++j)
-                if (kv[j])
-                    sum += __builtin_amdgcn_exp2f(__builtin_fmaf(v[j] - best, a.c1, a.c0));
-            res = __builtin_fmaf(__builtin_amdgcn_logf(wave_sum(sum)), a.ln2_over_eps, best);
+            for (int g = 0; g < MG; ++g) {
+                sum[g] = 0.0f;
+#pragma unroll
+                for (int j = 0; j < KL; ++j)
+                    if (kv[j])
+                        sum[g] += __builtin_amdgcn_exp2f(__builtin_fmaf(o[g][j] - best[g], a.c1, a.c0));
+            }
+            wave_sum(sum);
+#pragma unroll
+            for (int g = 0; g < MG; ++g)
+                res[g] = __builtin_fmaf(__builtin_amdgcn_logf(sum[g]), a.ln2_over_eps, best[g]);
         }
-        if (lane == 0)
-            out[(size_t)m * plane] = res;
+        if (lane == 0) {
+#pragma unroll
+            for (int g = 0; g < MG; ++g)
+                if (m0 + g < m_end)
+                    out[(size_t)(m0 + g) * plane] = res[g];
+        }
     }
 }
 
@@ -550,6 +626,7 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
 
     a.in = input; a.out = output; a.offp = offp;
     a.n_mgroups = t.n_mgroups;
+    a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;
 
     // bounds checks are needed unless every patch lies inside the image
     const bool inside = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 &&

@@ -29,6 +29,7 @@ struct MexKernelArgs {
     float c0;           // (softmax ? 0 : -log K) * log2(e)
     float ln2_over_eps; // log(2) / eps
     int finite_eps;
+    int kgather;        // tiled kernel: gather patch elements with lanes along k (pixels of a chunk lie an image apart)
     float oob;
 };
 
@@ -100,6 +101,7 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     const float ey = p.softmax_mode ? 0.0f : (float)-std::log((double)d.K);
     a.c0 = (float)((double)ey * log2e);
     a.oob = p.oob;
+    a.kgather = 0;
     return a;
 }
 

@@ -310,3 +310,20 @@ def test_mex_few_pixels_long_patches(pkg, case, normalize, eps):
     ref_off = orc.normalize_offsets(off) if normalize else off
     got = run_mex(pkg, x, off, case["n"], normalize_offsets=normalize, **kw)
     assert mex_err(got, x, ref_off, case["n"], **kw) <= MEX_TOL
+
+
+# ---- one pixel per image and region, long K: the tiled kernel gathers with lanes along k ------------------------------
+@pytest.mark.parametrize("eps", [1.0, -1.5, math.inf])
+@pytest.mark.parametrize("case", [
+    dict(im=(100, 256, 2, 2), n=64, kw=dict(blocks=[256, 1, 1], strides=[256, 1, 1], unshared_offset_region=[2])),
+    dict(im=(130, 96, 1, 1), n=200, kw=dict(blocks=[96, 1, 1], strides=[96, 1, 1], shared_offset_region=[1],
+                                           use_unshared_regions=False)),
+    dict(im=(70, 40, 2, 2), n=48, kw=dict(blocks=[30, 2, 2], strides=[10, 1, 1], padding=[5, 1, 1],
+                                         blocks_out_of_bounds_value=0.3)),                  # bounds checks, per-pixel regions
+    dict(im=(65, 33, 3, 2), n=17, kw=dict(blocks=[33, 1, 1], strides=[33, 1, 1])),           # ragged K and M
+])
+def test_mex_one_pixel_per_region_long_patches(pkg, case, eps):
+    kw = dict(case["kw"], epsilon=eps, softmax_mode=True)
+    x, off = mex_inputs(41, case["im"], case["n"], **kw)
+    got = run_mex(pkg, x, off, case["n"], **kw)
+    assert mex_err(got, x, off, case["n"], **kw) <= MEX_TOL
