@@ -10,14 +10,16 @@
 // Work split
 //   * a lane owns PT consecutive output columns of one output row ("pixel group") and MT
 //     output channels: PT*MT accumulators in VGPRs, summed over k in the reference's order;
-//   * the MT (template, weight) pairs of a k are the same for all 64 lanes, so they are read
-//     with scalar loads from a packed, k-major copy of the parameters and reach the VALU as
-//     SGPR operands: no LDS or VGPR traffic for the parameters at all;
+//   * the MT (template, weight) pairs of a k are the same for all 64 lanes; they come from a packed,
+//     k-major copy of the parameters through vector loads with a lane-uniform address, one step
+//     ahead, so that the arithmetic reads VGPRs only (SGPR operands halve the VALU issue rate here);
+//     the gather fallback fetches them with scalar loads and moves each to a VGPR once;
 //   * a workgroup (4 waves) stages the rows of the input image its pixel groups touch, a few
 //     channels at a time, into LDS with coalesced loads; out-of-image positions are written as
 //     the out_of_bounds_value bit pattern there, so the inner loop has no bounds checks and NaN
 //     padding behaves exactly like NaN data.
-//   The inner loop is VALU bound: per k and lane PT ds_read_b32 against 3*PT*MT VALU ops.
+//   The inner loop is VALU bound: per k and lane PT/2 ds_read2_b32 and 4 global_load_dwordx4 against
+//   3*PT*MT VALU ops (L2).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -60,8 +62,8 @@ struct SimKernelArgs {
     int vec_store;     // output rows are 16-byte aligned: store float4
 };
 
-// Wave-uniform parameter fetch: the address is the same in every lane, so these become scalar loads
-// (s_load_dwordx8/x16) and the values live in SGPRs.
+// Wave-uniform parameter fetch of the gather fallback: the address is the same in every lane, so these
+// become scalar loads (s_load_dwordx8/x16) and the values live in SGPRs.
 template <int MODE, int MT>
 __device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT], const float SIMNETS_CONST_AS *ppa,
                                             const float SIMNETS_CONST_AS *ppc)
@@ -377,7 +379,7 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
     }
 }
 
-// Packs (template, weight) into the k-major, MT-interleaved layout the scalar loads walk, with
+// Packs (template, weight) into the k-major, MT-interleaved layout the parameter loads walk, with
 // the sign and the 1/2 of the normalized modes folded into the weight, and precomputes the
 // per-(m,k) logarithm term.  Replaces interlace_kernel (include/utils/ggemm.cuh:70-87).
 __global__ void sim_pack_params_kernel(const float *__restrict__ templates, const float *__restrict__ weights, int O,
@@ -433,8 +435,8 @@ struct Tiling {
 Tiling choose_tiling(const SimPlan &p)
 {
     Tiling t;
-    // Wide rows and many templates: 16 pixels x 8 templates per lane (one s_load_dwordx16 per k, so
-    // two parameter sets fit the SGPR file and the next k can be in flight).  Otherwise 4 x 8, which
+    // Wide rows and many templates: 16 pixels x 8 templates per lane (128 accumulators, two waves per
+    // SIMD; 8x8 and 16x4 tiles measured slower on the 256x64x32x32 / 128-template case).  Otherwise 4 x 8, which
     // keeps narrow images and small template counts from idling lanes and waves.
     const bool big = p.ow >= 32 && p.O >= 32;
     t.PT = big ? kBigPT : kSmallPT;
@@ -505,7 +507,7 @@ size_t sim_direct_workspace_bytes(const SimPlan &p)
 {
     const Tiling t = choose_tiling(p);
     const size_t n_mtiles = (p.O + t.MT - 1) / t.MT;
-    // one extra k of slack behind each array: the scalar loads may be issued one step ahead
+    // one extra k of slack behind each array: the parameter loads are issued one step ahead
     const size_t pa = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
     const size_t pc = align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
     const size_t koff = align_up(((size_t)p.K + 2) * sizeof(int), 256);

@@ -14,7 +14,7 @@
 //   phase is one launch of the same register-tile scheme as the forward kernel with the roles
 //   swapped: g rows are staged in LDS (out of range -> 0), a lane owns PT pixels x MT input
 //   channels (accumulators AND the X values they belong to in VGPRs), the packed parameters of a
-//   (o, tap) step are wave-uniform scalar loads.
+//   (o, tap) step arrive through vector loads with a lane-uniform address, one step ahead.
 // Parameter gradients
 //   dT[o,k], dW[o,k] = sum over all B*oh*ow output pixels of W(g[px,o], patch(px)[k], t[o,k], w[o,k]).
 //   A lane owns 8 templates x 4 patch elements (its t values and the running sums in VGPRs), a wave
