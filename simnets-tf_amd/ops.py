@@ -35,8 +35,10 @@ _workspaces = {}
 
 
 def _workspace(device, nbytes):
-    """A per-device scratch tensor, grown on demand and reused across calls (stream-ordered)."""
-    key = (device.type, device.index)
+    """A scratch tensor per (device, current stream), grown on demand and reused across calls: the kernels that
+    use it are ordered on that stream, and calls on different streams never share one."""
+    with torch.cuda.device(device):
+        key = (device.index, torch.cuda.current_stream().cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)

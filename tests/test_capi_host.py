@@ -184,3 +184,33 @@ def test_op_layer_refuses_cpu_tensors(pkg):
         pkg.similarity(x, x, x, blocks=[4, 4])
     with pytest.raises(TypeError):
         pkg.similarity(x.double(), x, x, blocks=[4, 4])
+
+
+def test_gradient_entry_points_reject_bad_arguments_without_touching_the_device(pkg):
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    shapes = (I4(2, 3, 8, 8), I4(4, 3, 3, 3), I4(4, 3, 3, 3))
+    a = pkg.ops.similarity_attrs(blocks=[3, 3], ignore_nan_input=True)     # ignore_nan_input needs normalization_term
+    assert l.simnets_hip_similarity_input_grad(C.byref(a), *shapes, 256, 256, 256, 256, 256, None, 0, None) == -7
+    a = pkg.ops.similarity_attrs(blocks=[3, 3])
+    assert l.simnets_hip_similarity_input_grad(C.byref(a), *shapes, None, 256, 256, 256, 256, None, 0, None) == -1
+    assert l.simnets_hip_similarity_params_grad(C.byref(a), *shapes, 256, 256, 256, None, 256, 256, None, 0, None) == -1
+    wx, wp = C.c_size_t(), C.c_size_t()
+    assert l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), shapes[0], shapes[1], C.byref(wx), C.byref(wp)) == 0
+    assert wx.value > 0 and wp.value >= 2 * 4 * 27 * 4          # packed parameters; partial sums for both gradients
+    assert l.simnets_hip_similarity_input_grad(C.byref(a), *shapes, 256, 256, 256, 256, 256, None, 0, None) == -17
+    assert l.simnets_hip_similarity_params_grad(C.byref(a), *shapes, 256, 256, 256, 256, 256, 256, 256, 16, None) == -17
+    assert l.simnets_hip_similarity_input_grad(C.byref(a), *shapes, 256, 256, 256, 256, 256, 257, 1 << 30, None) == -17  # misaligned
+
+    m = pkg.ops.mex_attrs(2, blocks=[3, 1, 1], normalize_offsets=True)
+    xs = I4(2, 3, 8, 8)
+    assert l.simnets_hip_mex_input_grad(C.byref(m), xs, 256, 256, 5, 256, 256, 256, None, 0, None) == -15   # short offsets
+    n_off = 64 * 2 * 3
+    assert l.simnets_hip_mex_input_grad(C.byref(m), xs, 256, 256, n_off, None, 256, 256, None, 0, None) == -1
+    assert l.simnets_hip_mex_offsets_grad(C.byref(m), xs, 256, 256, n_off, 256, 256, None, None, 0, None) == -1
+    wi, wo = C.c_size_t(), C.c_size_t()
+    assert l.simnets_hip_mex_grad_workspace_bytes(C.byref(m), xs, C.byref(wi), C.byref(wo)) == 0
+    assert wi.value >= n_off * 4 and wo.value >= 2 * n_off * 4    # normalised copy; + partial sums
+    assert l.simnets_hip_mex_input_grad(C.byref(m), xs, 256, 256, n_off, 256, 256, 256, None, 0, None) == -17
+    bad = pkg.ops.mex_attrs(2, blocks=[4, 1, 1])                  # block deeper than the image
+    assert l.simnets_hip_mex_offsets_grad(C.byref(bad), xs, 256, 256, n_off, 256, 256, 256, None, 0, None) < 0
