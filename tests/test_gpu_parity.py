@@ -327,3 +327,32 @@ def test_mex_one_pixel_per_region_long_patches(pkg, case, eps):
     x, off = mex_inputs(41, case["im"], case["n"], **kw)
     got = run_mex(pkg, x, off, case["n"], **kw)
     assert mex_err(got, x, off, case["n"], **kw) <= MEX_TOL
+
+
+# ---- larger, network-like geometries (oracle on one image; the batch must not matter) -----------------------------------
+def test_similarity_stem_like_geometry(pkg):
+    """7x7 templates, stride 2, padding 3 on 224x224 images: rows wider than the LDS tile of the big lane tile."""
+    x, t, w = sim_inputs(51, (3, 3, 224, 224), 64, (7, 7))
+    kw = dict(blocks=[7, 7], strides=[2, 2], padding=[3, 3])
+    got = run_similarity(pkg, x, t, w, **kw)
+    assert got.shape == (3, 64, 112, 112)
+    for b in (0, 2):
+        assert rel_err(got[b:b + 1], orc.similarity_fwd(x[b:b + 1], t, w, **kw)) <= SIM_TOL
+
+
+def test_similarity_many_templates_small_images(pkg):
+    x, t, w = sim_inputs(52, (64, 96, 8, 8), 384, (3, 3))
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1], similarity_function="L1")
+    got = run_similarity(pkg, x, t, w, **kw)
+    for b in (0, 63):
+        assert rel_err(got[b:b + 1], orc.similarity_fwd(x[b:b + 1], t, w, **kw)) <= SIM_TOL
+
+
+def test_mex_overlapping_3d_blocks_network_like(pkg):
+    kw = dict(blocks=[64, 3, 3], strides=[64, 1, 1], padding=[0, 1, 1], softmax_mode=True, epsilon=1.0,
+              use_unshared_regions=False, shared_offset_region=[4])
+    x, off = mex_inputs(53, (6, 64, 28, 28), 32, **kw)
+    got = run_mex(pkg, x, off, 32, **kw)
+    assert got.shape == (6, 32, 28, 28)
+    for b in (0, 5):
+        assert mex_err(got[b:b + 1], x[b:b + 1], off, 32, **kw) <= MEX_TOL
