@@ -60,6 +60,7 @@ struct SimKernelArgs {
     float norm_const;  // -0.5*K*log(2 pi) for SIM_MODE_L2_NORM, else 0
     int norm_every_iteration;
     int vec_store;     // output rows are 16-byte aligned: store float4
+    int fast_stage;    // the channel tile has at most kStagePos * kThreads elements: division-free staging
 };
 
 // Wave-uniform parameter fetch of the gather fallback: the address is the same in every lane, so these
@@ -240,7 +241,11 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
         const int ccn = min(a.CC, a.C - ch0);
         __syncthreads();
         // ---- stage ccn channels x TR rows x TC columns; out-of-image -> oob ----
-        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccn, ccn, chan_lds, a.oob, nullptr, tp);
+        if (a.fast_stage)
+            stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccn, ccn, chan_lds, a.oob, nullptr, tp);
+        else  // tiles with more elements per channel than the precomputed positions cover
+            stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.pw, a.oob,
+                                          nullptr);
         __syncthreads();
         if (!wave_active)
             continue;
@@ -429,35 +434,26 @@ __global__ void sim_pack_params_kernel(const float *__restrict__ templates, cons
 
 struct Tiling {
     int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
-    bool lds_ok;
+    bool lds_ok;       // the rows of a workgroup's pixel groups fit the LDS tile (else: gather kernel)
+    bool fast_stage;   // ... and the division-free staging (at most kStagePos elements per thread and channel)
 };
 
-Tiling choose_tiling(const SimPlan &p)
+// One candidate: lane tile (PT, MT) with `nws` spatial waves per workgroup.
+Tiling try_tiling(const SimPlan &p, int PT, int MT, int nws)
 {
     Tiling t;
-    // Wide rows and many templates: 16 pixels x 8 templates per lane (128 accumulators, two waves per
-    // SIMD; 8x8 and 16x4 tiles measured slower on the 256x64x32x32 / 128-template case).  Otherwise 4 x 8, which
-    // keeps narrow images and small template counts from idling lanes and waves.
-    const bool big = p.ow >= 32 && p.O >= 32;
-    t.PT = big ? kBigPT : kSmallPT;
-    t.MT = big ? kBigMT : kSmallMT;
-    const int budget = lds_budget_floats(t.PT, t.MT);
-    t.G = (p.ow + t.PT - 1) / t.PT;
+    t.PT = PT; t.MT = MT; t.nws = nws;
+    const int budget = lds_budget_floats(PT, MT);
+    t.G = (p.ow + PT - 1) / PT;
     t.gpi = p.oh * t.G;
-    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
-    // spatial waves per workgroup: as many as the template tiles leave free, if the image has the groups
-    t.nws = 1;
-    if (n_mtiles <= 2 && t.gpi >= 128)
-        t.nws = 2;
-    if (n_mtiles <= 1 && t.gpi >= 256)
-        t.nws = 4;
-    t.tiles = (t.gpi + 64 * t.nws - 1) / (64 * t.nws);
-    t.TC = (t.G * t.PT - 1) * p.sw + p.bw;
+    t.tiles = (t.gpi + 64 * nws - 1) / (64 * nws);
+    t.TC = (t.G * PT - 1) * p.sw + p.bw;
     t.TC |= 1;  // odd pitch spreads rows over LDS banks
-    const int max_rows = std::min(p.oh, (64 * t.nws + t.G - 1) / t.G + 1);
+    const int max_rows = std::min(p.oh, (64 * nws + t.G - 1) / t.G + 1);
     t.TRmax = (max_rows - 1) * p.sh + p.bh;
     const long long per_chan = 1LL * t.TRmax * t.TC;
-    t.lds_ok = per_chan <= std::min(budget, kStagePos * kThreads);
+    t.lds_ok = per_chan <= budget;
+    t.fast_stage = per_chan <= kStagePos * kThreads;
     t.CC = 1;
     if (t.lds_ok) {
         const int cc_max = (int)std::min<long long>(p.C, budget / per_chan);
@@ -465,6 +461,42 @@ Tiling choose_tiling(const SimPlan &p)
         t.CC = (p.C + chunks - 1) / chunks;
     }
     return t;
+}
+
+// Lane tile and workgroup shape for a problem.
+Tiling choose_tiling(const SimPlan &p)
+{
+    auto pick = [&](int PT, int MT) {
+        const int n_mtiles = (p.O + MT - 1) / MT;
+        const int G = (p.ow + PT - 1) / PT, gpi = p.oh * G;
+        // spatial waves per workgroup: as many as the template tiles leave free, if the image has the groups;
+        // fewer if the rows of that many groups do not fit the LDS tile (or its fast staging)
+        int nws = 1;
+        if (n_mtiles <= 2 && gpi >= 128)
+            nws = 2;
+        if (n_mtiles <= 1 && gpi >= 256)
+            nws = 4;
+        Tiling t = try_tiling(p, PT, MT, nws);
+        while (nws > 1 && !(t.lds_ok && t.fast_stage)) {
+            nws >>= 1;
+            t = try_tiling(p, PT, MT, nws);
+        }
+        return t;
+    };
+    auto waves = [&](const Tiling &t) {
+        const int n_mtiles = (p.O + t.MT - 1) / t.MT, nwm = kWaves / t.nws;
+        return (long long)p.B * t.tiles * ((n_mtiles + nwm - 1) / nwm) * kWaves;
+    };
+    // Wide rows and many templates: 16 pixels x 8 templates per lane (128 accumulators, two waves per SIMD; 8x8
+    // and 16x4 tiles measured slower on the 256x64x32x32 / 128-template case) - provided the grid then still
+    // gives the SIMDs about two waves each (1.5 on average): a SIMD with a single wave issues at half rate.  Otherwise 4 x 8, which
+    // keeps narrow images, small template counts and small batches from idling lanes, waves and CUs.
+    if (p.ow >= 32 && p.O >= 32) {
+        const Tiling big = pick(kBigPT, kBigMT);
+        if (big.lds_ok && waves(big) >= 1536)
+            return big;
+    }
+    return pick(kSmallPT, kSmallMT);
 }
 
 template <int MODE, int PT, int MT>
@@ -542,7 +574,7 @@ int sim_direct_launch(const SimPlan &p, const float *input, const float *templat
     a.G = t.G; a.gpi = t.gpi; a.tiles = t.tiles; a.nws = t.nws; a.n_mtiles = n_mtiles;
     a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
     a.vec_store = (p.ow % 4 == 0) && ((reinterpret_cast<uintptr_t>(output) & 15) == 0);
-    a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC;
+    a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC; a.fast_stage = t.fast_stage;
     a.oob = p.oob;
     // Dtype(-0.5) * Dtype(K_) * std::log(2.0 * M_PI), rounded to float by Eigen's constant()
     a.norm_const = (p.mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)p.K) * std::log(2.0 * M_PI)) : 0.0f;

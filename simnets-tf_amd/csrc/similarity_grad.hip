@@ -62,6 +62,7 @@ struct GradXArgs {
     int K;
     int G, gpi, tiles, nws, nws_log2, n_ctiles, TC, TRmax, CC;
     int ignore_nan;
+    int fast_stage;    // the g tile of a channel has at most kStagePos * kThreads elements: division-free staging
     int row_limit, col_limit;  // phase rows h <= row_limit (columns v <= col_limit) are covered by a window
 };
 
@@ -180,7 +181,11 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
     for (int ch0 = 0; ch0 < a.O; ch0 += a.CC) {
         const int ccn = min(a.CC, a.O - ch0);
         __syncthreads();
-        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.oh, a.ow, ch0, ccn, ccn, chan_lds, 0.0f, nullptr, tp);
+        if (a.fast_stage)
+            stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.oh, a.ow, ch0, ccn, ccn, chan_lds, 0.0f, nullptr, tp);
+        else
+            stage_input_tile<kThreads, 8>(lds, img, a.oh, a.ow, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.padw, 0.0f,
+                                          nullptr);
         __syncthreads();
         if (!wave_active)
             continue;
@@ -369,31 +374,24 @@ Phase make_phase(const SimPlan &p, int ry, int rx)
 
 struct GxTiling {
     int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
-    bool lds_ok;
+    bool lds_ok, fast_stage;
 };
 
-GxTiling gx_tiling(const SimPlan &p, const Phase &f)
+GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws)
 {
     GxTiling t;
-    const bool big = f.nb >= 32 && p.C >= 32;
-    t.PT = big ? 8 : 4;
-    t.MT = 8;
+    t.PT = PT; t.MT = 8; t.nws = nws;
     const int budget = gx_lds_budget(t.PT, t.MT);
     t.G = (f.nb + t.PT - 1) / t.PT;
     t.gpi = f.na * t.G;
-    const int n_ctiles = (p.C + t.MT - 1) / t.MT;
-    t.nws = 1;
-    if (n_ctiles <= 2 && t.gpi >= 128)
-        t.nws = 2;
-    if (n_ctiles <= 1 && t.gpi >= 256)
-        t.nws = 4;
-    t.tiles = (t.gpi + 64 * t.nws - 1) / (64 * t.nws);
+    t.tiles = (t.gpi + 64 * nws - 1) / (64 * nws);
     t.TC = (t.G * t.PT - 1) + f.nJ;
     t.TC |= 1;
-    const int max_rows = std::min(f.na, (64 * t.nws + t.G - 1) / t.G + 1);
+    const int max_rows = std::min(f.na, (64 * nws + t.G - 1) / t.G + 1);
     t.TRmax = max_rows - 1 + f.nI;
     const long long per_chan = 1LL * t.TRmax * t.TC;
-    t.lds_ok = per_chan <= std::min(budget, kStagePos * kThreads);
+    t.lds_ok = per_chan <= budget;
+    t.fast_stage = per_chan <= kStagePos * kThreads;
     t.CC = 1;
     if (t.lds_ok) {
         const int cc_max = (int)std::min<long long>(p.O, budget / per_chan);
@@ -401,6 +399,34 @@ GxTiling gx_tiling(const SimPlan &p, const Phase &f)
         t.CC = (p.O + chunks - 1) / chunks;
     }
     return t;
+}
+
+GxTiling gx_tiling(const SimPlan &p, const Phase &f)
+{
+    auto pick = [&](int PT) {
+        const int n_ctiles = (p.C + 7) / 8;
+        const int gpi = f.na * ((f.nb + PT - 1) / PT);
+        int nws = 1;
+        if (n_ctiles <= 2 && gpi >= 128)
+            nws = 2;
+        if (n_ctiles <= 1 && gpi >= 256)
+            nws = 4;
+        GxTiling t = gx_try(p, f, PT, nws);
+        while (nws > 1 && !(t.lds_ok && t.fast_stage)) {   // fewer spatial waves: fewer g rows per workgroup
+            nws >>= 1;
+            t = gx_try(p, f, PT, nws);
+        }
+        return t;
+    };
+    // 8 x 8 lane tile for wide phase grids with many channels, if the grid then still gives every SIMD two waves
+    if (f.nb >= 32 && p.C >= 32) {
+        const GxTiling big = pick(8);
+        const int n_ctiles = (p.C + 7) / 8, nwm = kWaves / big.nws;
+        const long long waves = (long long)p.B * big.tiles * ((n_ctiles + nwm - 1) / nwm) * kWaves;
+        if (big.lds_ok && waves >= 1536)
+            return big;
+    }
+    return pick(4);
 }
 
 size_t gx_phase_param_bytes(const SimPlan &p, const Phase &f)
@@ -518,6 +544,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
             a.n_ctiles = n_ctiles; a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC;
             a.ignore_nan = ignore_nan;
+            a.fast_stage = t.fast_stage;
             // phase row h (a = a0 + h) is covered by some window iff a - (nI-1) <= oh-1
             a.row_limit = p.oh - 1 + f.nI - 1 - f.a0;
             a.col_limit = p.ow - 1 + f.nJ - 1 - f.b0;
