@@ -44,6 +44,7 @@ namespace {
 constexpr int MX = 16;        // instances per wave
 constexpr int kChunkMin = 32;  // k per LDS chunk: 32, or 64 / 128 for long K with one pixel per lane
 constexpr int kXcds = 8;
+constexpr float kProductRange = 90.0f;  // widest row range of the scaled offsets (a power of two) the product form takes
 #ifndef SIMNETS_MEX_WAVES
 #define SIMNETS_MEX_WAVES 4096  // pixels per lane shrink until the grid has this many waves
 #endif
@@ -66,6 +67,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     __shared__ __attribute__((aligned(16))) float smem[cmax(KC * XP + KC * TM, kMergeFloats)];
     __shared__ long long pref_off[KGATHER ? 64 : 1];
     __shared__ int pref_c[KGATHER ? 64 * 3 : 1];
+    __shared__ float pmx[256];            // product form: partial pixel maxima [k phase][pixel]
+    __shared__ float fsh[TP], msh[TP];    // product form: per pixel, the rescale factor of this chunk and the running maximum
     float *xs = smem;                     // [k][pixel], row pitch XP
     float *os = smem + KC * XP;           // [k][instance]
 
@@ -93,7 +96,20 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     const int sp = tid % TP, sk = tid / TP;
     const PixelRef gp = locate(a, r, chunk * TP + sp);
     const int bhw = a.bh * a.bw;
-    const float *offp = a.offp + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
+    // Product form (finite epsilon): with bounds mp >= patch values of the pixel and mo >= offsets of the instance,
+    // sum_k exp2(x_k + o_k - mp - mo) = sum_k exp2(x_k - mp) * exp2(o_k - mo): one exponential per staged patch
+    // element (shared by all instances), the offsets' exponentials packed once, and one fused multiply-add per
+    // term.  The largest term is at least exp2(-(row range of the offsets)), so the form is used when the ranges
+    // of all instances of the workgroup are small enough for that to stay far inside the normal range; otherwise
+    // the workgroup runs the two sweeps.
+    bool prod = false;
+    if (a.finite_eps) {
+        const float *rng = a.orng + ((size_t)r * a.n_mgroups + mgroup) * TM;
+        const int wide = tid < TM ? !(rng[tid] <= kProductRange) : 0;
+        prod = !__syncthreads_or(wide);
+    }
+    const float *offp = (prod ? a.offe : a.offp) + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
+    float m_run = -INFINITY;  // running maximum of this thread's staging pixel (product form)
     if (KGATHER && a.kgather && tid < 64) {
         // pixel table for the k-oriented gather: where each of the 64 pixels' patches starts
         pref_off[tid] = gp.base - a.in;
@@ -101,6 +117,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     }
 
     auto stage = [&](int k0, int kc) {
+        constexpr int U = KC / KSTEP;  // patch elements per thread and chunk
+        float v[U];
         if (KGATHER && a.kgather) {
             // Consecutive pixel slots are different images here (one pixel per image and region), a whole image
             // apart in memory, while consecutive patch elements are one channel plane apart: lanes run along k.
@@ -116,7 +134,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                     dw = rem - dh * a.bw;
                 }
                 const ptrdiff_t o = ((ptrdiff_t)dc * a.H + dh) * a.W + dw;
-                float v[16];
+                float g[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int p = pq + 4 * i;
@@ -125,20 +143,24 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                         const int ci = pref_c[3 * p] + dc, hi = pref_c[3 * p + 1] + dh, wi = pref_c[3 * p + 2] + dw;
                         ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
                     }
-                    v[i] = ok ? a.in[pref_off[p] + o] : a.oob;
+                    g[i] = ok ? a.in[pref_off[p] + o] : a.oob;
                 }
 #pragma unroll
                 for (int i = 0; i < 16; ++i)
-                    xs[kk * XP + pq + 4 * i] = v[i] * a.scale;
+                    xs[kk * XP + pq + 4 * i] = g[i] * a.scale;
             }
-        } else
-        // patch elements: xs[kk][sp] = patch(sp)[k0 + kk]
-        for (int kk0 = sk; kk0 < kc; kk0 += KSTEP * (KC / KSTEP)) {
-            constexpr int U = KC / KSTEP;  // gathers per thread and chunk: all in flight before the first LDS store
-            float v[U];
+            if (prod) {
+                __syncthreads();
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    v[u] = xs[min(sk + u * KSTEP, kc - 1) * XP + sp];
+            }
+        } else {
+            // patch elements: xs[kk][sp] = patch(sp)[k0 + kk], kk = sk, sk + KSTEP, ...: all gathers of the chunk
+            // in flight before the first LDS store
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int kk = kk0 + u * KSTEP;
+                const int kk = sk + u * KSTEP;
                 const int k = k0 + min(kk, kc - 1);
                 int dc = k, dh = 0, dw = 0;
                 if (bhw != 1) {
@@ -157,11 +179,44 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                 }
             }
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int kk = kk0 + u * KSTEP;
-                if (kk < kc)
-                    xs[kk * XP + sp] = v[u] * a.scale;
+            for (int u = 0; u < U; ++u)
+                v[u] *= a.scale;
+            if (!prod) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int kk = sk + u * KSTEP;
+                    if (kk < kc)
+                        xs[kk * XP + sp] = v[u];
+                }
             }
+        }
+        if (prod) {
+            // pixel maximum over the chunk -> running maximum; the staged values become exp2(x - maximum)
+            float pm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (sk + u * KSTEP < kc)
+                    pm = fmaxf(pm, v[u]);
+            if (KSTEP > 1) {
+                pmx[sk * TP + sp] = pm;
+                __syncthreads();
+#pragma unroll
+                for (int j = 0; j < KSTEP; ++j)
+                    pm = fmaxf(pm, pmx[j * TP + sp]);
+            }
+            const float m_new = fmaxf(m_run, pm);
+            const float m_sub = m_new == -INFINITY ? 0.0f : m_new;  // nothing finite yet: the terms are exp2(-inf) = 0
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int kk = sk + u * KSTEP;
+                if (kk < kc)
+                    xs[kk * XP + sp] = __builtin_amdgcn_exp2f(v[u] - m_sub);
+            }
+            if (sk == 0) {
+                fsh[sp] = m_run == m_new ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                msh[sp] = m_new;
+            }
+            m_run = m_new;
         }
         // offsets: a straight copy of kc * TM floats
         const float4 *src = reinterpret_cast<const float4 *>(offp + (size_t)k0 * TM);
@@ -181,6 +236,57 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     const float *xl = xs + lane;                 // this lane's pixels: xl[kk*TP + p*64]
     const float *ol = os + wm * MX;              // this wave's instances: ol[kk*TM + m]
 
+    float s[PX][MX];
+#pragma unroll
+    for (int p = 0; p < PX; ++p)
+#pragma unroll
+        for (int m = 0; m < MX; ++m)
+            s[p][m] = 0.0f;
+
+    if (prod) {
+        // ---- one sweep: s = sum_k exp2(x_k - mp) * exp2(o_k - mo), rescaled when a chunk raises mp ----
+        for (int k0 = 0; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            __syncthreads();
+            stage(k0, kc);
+            __syncthreads();
+            if (!wave_active)
+                continue;
+            if (k0 > 0) {
+#pragma unroll
+                for (int p = 0; p < PX; ++p) {
+                    const float f = fsh[p * 64 + lane];
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        s[p][m] *= f;
+                }
+            }
+            const int kend = min(kc, (wk + 1) * KW);
+            for (int kk = wk * KW; kk < kend; ++kk) {
+                float x[PX], o[MX];
+#pragma unroll
+                for (int p = 0; p < PX; ++p)
+                    x[p] = xl[kk * XP + p * 64];
+#pragma unroll
+                for (int m = 0; m < MX; ++m)
+                    o[m] = ol[kk * TM + m];
+#pragma unroll
+                for (int p = 0; p < PX; ++p)
+#pragma unroll
+                    for (int m = 0; m < MX; ++m)
+                        s[p][m] = __builtin_fmaf(x[p], o[m], s[p][m]);
+            }
+        }
+        // the shift of every instance: the pixel bound (an infinite one makes the result NaN, as the reference's
+        // exp(inf - inf) does); the instance bound is added in the epilogue
+#pragma unroll
+        for (int p = 0; p < PX; ++p) {
+            const float mp = msh[p * 64 + lane];
+#pragma unroll
+            for (int m = 0; m < MX; ++m)
+                mx[p][m] = mp;
+        }
+    } else {
     // ---- sweep 1: running max (min for negative epsilon) of patch + offset ----
     for (int k0 = 0; k0 < a.K; k0 += KC) {
         const int kc = min(KC, a.K - k0);
@@ -215,12 +321,6 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
         }
     }
 
-    float s[PX][MX];
-#pragma unroll
-    for (int p = 0; p < PX; ++p)
-#pragma unroll
-        for (int m = 0; m < MX; ++m)
-            s[p][m] = 0.0f;
     if (a.finite_eps) {
         // ---- sweep 2: sum of exp(eps * (v - max)): patch values and offsets are already multiplied by
         //      eps*log2(e), so the term is exp2 of a plain difference ----
@@ -265,6 +365,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             }
         }
     }
+    }
 
     if (KS > 1) {
         // ---- merge the (max, sum) pairs of the K-split waves into wave wk == 0 ----
@@ -308,6 +409,14 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 
     // output channel = instance * channels_out + c  (src/kernels/mex_kernel_cpu.cpp:113-115)
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    if (prod) {
+        const float *omax = a.omax + ((size_t)r * a.n_mgroups + mgroup) * TM + wm * MX;
+#pragma unroll
+        for (int p = 0; p < PX; ++p)
+#pragma unroll
+            for (int m = 0; m < MX; ++m)
+                mx[p][m] = (mx[p][m] - mx[p][m]) + mx[p][m] + omax[m];
+    }
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
         const PixelRef cp = locate(a, r, chunk * TP + p * 64 + lane);
@@ -326,11 +435,14 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 }
 
 // One wave per (region, instance) row of the offsets: optional logsumexp normalisation
-// (python/simnets/keras.py:155-160), then the row is scattered into the k-major packed layout
-// [r][mgroup][k][tm].
+// (python/simnets/keras.py:155-160) and the scaling, then the row is scattered into the k-major packed layout
+// [r][mgroup][k][tm]; for finite epsilon also its exponentials relative to the row maximum, the maximum and the
+// row's range (what the product form of the forward kernel reads).
 __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__restrict__ offsets, int R, int M, int K,
                                                               int n_mgroups, int tm, int normalize, float scale,
-                                                              float *__restrict__ offp)
+                                                              int finite_eps, float *__restrict__ offp,
+                                                              float *__restrict__ offe, float *__restrict__ omax,
+                                                              float *__restrict__ orng)
 {
     const int lane = threadIdx.x & 63;
     const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -342,10 +454,19 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
     const int mgroup = (int)(t % n_mgroups);
     const int r = (int)(t / n_mgroups);
     const int m = mgroup * tm + mi;
-    float *dst = offp + ((size_t)r * n_mgroups + mgroup) * K * tm + mi;
+    const size_t at = ((size_t)r * n_mgroups + mgroup) * K * tm + mi;
+    float *dst = offp + at;
+    float *dste = offe + at;
     if (m >= M) {
-        for (int k = lane; k < K; k += 64)
+        for (int k = lane; k < K; k += 64) {
             dst[(size_t)k * tm] = 0.0f;
+            if (finite_eps)
+                dste[(size_t)k * tm] = 0.0f;
+        }
+        if (finite_eps && lane == 0) {
+            omax[row] = 0.0f;
+            orng[row] = 0.0f;
+        }
         return;
     }
     const float *src = offsets + ((size_t)r * M + m) * K;
@@ -365,8 +486,30 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
             sum += __shfl_xor(sum, d, 64);
         lse = logf(sum) + mxv;
     }
-    for (int k = lane; k < K; k += 64)
-        dst[(size_t)k * tm] = (src[k] - lse) * scale;
+    if (!finite_eps) {
+        for (int k = lane; k < K; k += 64)
+            dst[(size_t)k * tm] = (src[k] - lse) * scale;
+        return;
+    }
+    float hi = -INFINITY, lo = INFINITY;
+    for (int k = lane; k < K; k += 64) {
+        const float v = (src[k] - lse) * scale;
+        hi = fmaxf(hi, v);
+        lo = fminf(lo, v);
+    }
+    for (int d = 32; d > 0; d >>= 1) {
+        hi = fmaxf(hi, __shfl_xor(hi, d, 64));
+        lo = fminf(lo, __shfl_xor(lo, d, 64));
+    }
+    for (int k = lane; k < K; k += 64) {
+        const float v = (src[k] - lse) * scale;
+        dst[(size_t)k * tm] = v;
+        dste[(size_t)k * tm] = __builtin_amdgcn_exp2f(v - hi);
+    }
+    if (lane == 0) {
+        omax[row] = hi;
+        orng[row] = hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
+    }
 }
 
 template <int PX, int KS, int KC>
@@ -584,7 +727,9 @@ MexTiling mex_tiling(const MexPlan &p)
 size_t mex_workspace_bytes(const MexPlan &p)
 {
     const MexTiling t = mex_tiling(p);
-    return align_up((size_t)p.d.num_regions * t.n_mgroups * p.d.K * t.tm * sizeof(float), 256);
+    const size_t packed = align_up((size_t)p.d.num_regions * t.n_mgroups * p.d.K * t.tm * sizeof(float), 256);
+    const size_t rows = align_up((size_t)p.d.num_regions * t.n_mgroups * t.tm * sizeof(float), 256);
+    return 2 * packed + 2 * rows;  // scaled offsets, their exponentials; row maxima, row ranges
 }
 
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
@@ -615,16 +760,23 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
         return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
     }
     const MexTiling t = mex_tiling(p);
-    float *offp = reinterpret_cast<float *>(workspace);
+    const long long rows = (long long)d.num_regions * t.n_mgroups * t.tm;
+    const size_t packed = align_up((size_t)rows * d.K * sizeof(float), 256);
+    const size_t row_bytes = align_up((size_t)rows * sizeof(float), 256);
+    char *ws = reinterpret_cast<char *>(workspace);
+    float *offp = reinterpret_cast<float *>(ws);
+    float *offe = reinterpret_cast<float *>(ws + packed);
+    float *omax = reinterpret_cast<float *>(ws + 2 * packed);
+    float *orng = reinterpret_cast<float *>(ws + 2 * packed + row_bytes);
 
     MexKernelArgs a = mex_kernel_args(p);
-    const long long rows = (long long)d.num_regions * t.n_mgroups * t.tm;
     hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, offsets,
-                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, a.scale, offp);
+                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, a.scale, a.finite_eps, offp,
+                       offe, omax, orng);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
 
-    a.in = input; a.out = output; a.offp = offp;
+    a.in = input; a.out = output; a.offp = offp; a.offe = offe; a.omax = omax; a.orng = orng;
     a.n_mgroups = t.n_mgroups;
     a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;
 

@@ -12,7 +12,10 @@ namespace simnets {
 struct MexKernelArgs {
     const float *in;
     float *out;
-    const float *offp;  // [R][mgroup][K][TM]
+    const float *offp;  // [R][mgroup][K][TM]  offsets * scale
+    const float *offe;  // [R][mgroup][K][TM]  exp2(offsets * scale - row maximum)   (finite epsilon only)
+    const float *omax;  // [R][mgroup][TM]     row maximum of offsets * scale
+    const float *orng;  // [R][mgroup][TM]     row maximum - row minimum of offsets * scale
     int B, C, H, W;
     int Co, Ho, Wo;
     int bc, bh, bw, sc, sh, sw, pc, ph, pw;
@@ -78,7 +81,7 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
 {
     const simnets_mex_dims &d = p.d;
     MexKernelArgs a;
-    a.in = nullptr; a.out = nullptr; a.offp = nullptr;
+    a.in = nullptr; a.out = nullptr; a.offp = nullptr; a.offe = nullptr; a.omax = nullptr; a.orng = nullptr;
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W;
     a.Co = d.channels_out; a.Ho = d.height_out; a.Wo = d.width_out;
     a.bc = d.block_c; a.bh = d.block_h; a.bw = d.block_w;

@@ -252,6 +252,37 @@ def test_mex_large_dynamic_range(pkg):
     assert mex_err(run_mex(pkg, x, off, 8, **kw), x, off, 8, **kw) <= MEX_TOL
 
 
+@pytest.mark.parametrize("geom", [
+    dict(im=(6, 8, 40, 40), n=130, blocks=[8, 3, 3], strides=[8, 1, 1], padding=[0, 1, 1]),    # several pixels per lane, K = 72
+    dict(im=(5, 200, 4, 4), n=70, blocks=[200, 1, 1], strides=[200, 1, 1], padding=[0, 0, 0]),  # K split over the waves
+    dict(im=(40, 96, 2, 2), n=64, blocks=[96, 1, 1], strides=[96, 1, 1], padding=[0, 0, 0]),    # one pixel per image and region
+])
+@pytest.mark.parametrize("spread", ["narrow", "wide", "mixed", "masked"])
+@pytest.mark.parametrize("eps", [1.0, -2.0, 30.0])
+def test_mex_offset_ranges_product_and_two_sweep_forms(pkg, geom, spread, eps):
+    # Finite epsilon: instances whose offsets span a small range take the product form
+    # (sum_k exp(x_k - max x) * exp(o_k - max o)), wide or infinite ranges the two sweeps; groups of instances of
+    # one launch may differ.  Patch values grow along k so that later chunks raise the running pixel maximum.
+    g = np.random.default_rng(17)
+    kw = dict(softmax_mode=False, blocks=geom["blocks"], strides=geom["strides"], padding=geom["padding"], epsilon=eps,
+              unshared_offset_region=[2], blocks_out_of_bounds_value=-3.0)
+    n = geom["n"]
+    d = orc.mex_dims(orc.mex_args(geom["im"], n, **kw))
+    x = (g.normal(size=geom["im"]) * 20).astype(np.float32)
+    x += (np.arange(geom["im"][1], dtype=np.float32) * 0.5 * np.sign(eps))[None, :, None, None]
+    off = (g.normal(size=(d.num_regions, n) + tuple(geom["blocks"])) * 0.3).astype(np.float32)
+    if spread == "wide":
+        off *= 400
+    elif spread == "mixed":
+        off[:, n // 2:] *= 400
+        off[:, 3] *= 400
+    elif spread == "masked":
+        off[g.random(size=off.shape) < 0.2] = -math.inf if eps > 0 else math.inf
+    got = run_mex(pkg, x, off, n, **kw)
+    assert np.isfinite(got).all()
+    assert mex_err(got, x, off, n, **kw) <= MEX_TOL
+
+
 def test_sum_pooling(pkg):
     g = np.random.default_rng(16)
     x = g.normal(size=(3, 5, 9, 8)).astype(np.float32)
