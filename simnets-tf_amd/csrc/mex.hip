@@ -51,6 +51,8 @@ constexpr float kProductRange = 90.0f;  // widest row range of the scaled offset
 
 constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
 template <int PX, int KS, int KC, bool NEG, bool CHECK>
 __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 {
@@ -69,6 +71,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     __shared__ int pref_c[KGATHER ? 64 * 3 : 1];
     __shared__ float pmx[256];            // product form: partial pixel maxima [k phase][pixel]
     __shared__ float fsh[TP], msh[TP];    // product form: per pixel, the rescale factor of this chunk and the running maximum
+    __shared__ long long pout[TP];        // product form: where instance 0 of the pixel goes in the output, -1 for an empty slot
     float *xs = smem;                     // [k][pixel], row pitch XP
     float *os = smem + KC * XP;           // [k][instance]
 
@@ -81,7 +84,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     int r, chunk;
     {
         const int per_super = kXcds * a.R;
-        const int super = blockIdx.x / per_super;
+        const int super = (int)fast_div(blockIdx.x, a.dSuper);
         const int within = blockIdx.x - super * per_super;
         r = within / kXcds;
         chunk = super * kXcds + (within - r * kXcds);
@@ -94,8 +97,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 
     // staging role: this thread gathers pixel `sp` for k = sk, sk + KSTEP, ...
     const int sp = tid % TP, sk = tid / TP;
+    const int sk_u = __builtin_amdgcn_readfirstlane(sk);
     const PixelRef gp = locate(a, r, chunk * TP + sp);
-    const int bhw = a.bh * a.bw;
     // Product form (finite epsilon): with bounds mp >= patch values of the pixel and mo >= offsets of the instance,
     // sum_k exp2(x_k + o_k - mp - mo) = sum_k exp2(x_k - mp) * exp2(o_k - mo): one exponential per staged patch
     // element (shared by all instances), the offsets' exponentials packed once, and one fused multiply-add per
@@ -110,6 +113,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     }
     const float *offp = (prod ? a.offe : a.offp) + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
     float m_run = -INFINITY;  // running maximum of this thread's staging pixel (product form)
+    if (prod && sk == 0)
+        pout[sp] = gp.out_off < 0 ? -1 : (long long)gp.b * a.M * ((long long)a.Co * a.Ho * a.Wo) + gp.out_off;
     if (KGATHER && a.kgather && tid < 64) {
         // pixel table for the k-oriented gather: where each of the 64 pixels' patches starts
         pref_off[tid] = gp.base - a.in;
@@ -117,7 +122,12 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
     }
 
     auto stage = [&](int k0, int kc) {
-        constexpr int U = KC / KSTEP;  // patch elements per thread and chunk
+        constexpr int U = KC / KSTEP;                    // patch elements per thread and chunk
+        const bool full = kc == KC;                      // all but the last chunk: no per-element guards
+        // offsets: a straight copy of kc * TM floats, after the gather's loads have been issued
+        const float4 *src = reinterpret_cast<const float4 *>(offp + (size_t)k0 * TM);
+        float4 *dst = reinterpret_cast<float4 *>(os);
+        const int on = kc * (TM / 4);
         float v[U];
         if (KGATHER && a.kgather) {
             // Consecutive pixel slots are different images here (one pixel per image and region), a whole image
@@ -125,15 +135,8 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             // Thread (kq, pq) gathers elements kq, kq + 64, ... of pixels pq, pq + 4, ...
             const int kq = tid & 63, pq = tid >> 6;   // (the pixel table was written before the barrier in front of this call)
             for (int kk = kq; kk < kc; kk += 64) {
-                const int k = k0 + kk;
-                int dc = k, dh = 0, dw = 0;
-                if (bhw != 1) {
-                    dc = k / bhw;
-                    const int rem = k - dc * bhw;
-                    dh = rem / a.bw;
-                    dw = rem - dh * a.bw;
-                }
-                const ptrdiff_t o = ((ptrdiff_t)dc * a.H + dh) * a.W + dw;
+                const int4 ke = a.ktab[k0 + kk];
+                const int o = ke.x, dc = ke.y, dh = ke.z, dw = ke.w;
                 float g[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -160,17 +163,12 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             // in flight before the first LDS store
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                const int kk = sk + u * KSTEP;
-                const int k = k0 + min(kk, kc - 1);
-                int dc = k, dh = 0, dw = 0;
-                if (bhw != 1) {
-                    dc = k / bhw;
-                    const int rem = k - dc * bhw;
-                    dh = rem / a.bw;
-                    dw = rem - dh * a.bw;
-                }
-                const ptrdiff_t o = ((ptrdiff_t)dc * a.H + dh) * a.W + dw;
+                // sk is the same for a whole wave (TP is a multiple of 64): the table entry comes through a scalar load
+                const int kk = sk_u + u * KSTEP;
+                const int4 ke = a.ktab[k0 + (full ? kk : min(kk, kc - 1))];
+                const int o = ke.x;
                 if (CHECK) {
+                    const int dc = ke.y, dh = ke.z, dw = ke.w;
                     const int ci = gp.ci0 + dc, hi = gp.hi0 + dh, wi = gp.wi0 + dw;
                     const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
                     v[u] = ok ? gp.base[o] : a.oob;
@@ -178,16 +176,18 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                     v[u] = gp.base[o];
                 }
             }
+        }
+        for (int i = tid; i < on; i += 256)
+            dst[i] = src[i];
+        if (!(KGATHER && a.kgather)) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
                 v[u] *= a.scale;
             if (!prod) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int kk = sk + u * KSTEP;
-                    if (kk < kc)
-                        xs[kk * XP + sp] = v[u];
-                }
+                for (int u = 0; u < U; ++u)
+                    if (full || sk_u + u * KSTEP < kc)
+                        xs[(sk + u * KSTEP) * XP + sp] = v[u];
             }
         }
         if (prod) {
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             float pm = -INFINITY;
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (sk + u * KSTEP < kc)
+                if (full || sk_u + u * KSTEP < kc)
                     pm = fmaxf(pm, v[u]);
             if (KSTEP > 1) {
                 pmx[sk * TP + sp] = pm;
@@ -207,22 +207,23 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             const float m_new = fmaxf(m_run, pm);
             const float m_sub = m_new == -INFINITY ? 0.0f : m_new;  // nothing finite yet: the terms are exp2(-inf) = 0
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                const int kk = sk + u * KSTEP;
-                if (kk < kc)
-                    xs[kk * XP + sp] = __builtin_amdgcn_exp2f(v[u] - m_sub);
-            }
+            for (int u = 0; u < U; ++u)
+                if (full || sk_u + u * KSTEP < kc)
+                    xs[(sk + u * KSTEP) * XP + sp] = __builtin_amdgcn_exp2f(v[u] - m_sub);
             if (sk == 0) {
                 fsh[sp] = m_run == m_new ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
                 msh[sp] = m_new;
             }
             m_run = m_new;
+            if (!full) {
+                // the matrix instruction takes 4 k at a time: rows kc .. next multiple of 4 are zeros
+                const int kc4 = (kc + 3) & ~3;
+                for (int i = tid; i < (kc4 - kc) * TP; i += 256)
+                    xs[(kc + i / TP) * XP + i % TP] = 0.0f;
+                for (int i = tid; i < (kc4 - kc) * TM; i += 256)
+                    os[kc * TM + i] = 0.0f;
+            }
         }
-        // offsets: a straight copy of kc * TM floats
-        const float4 *src = reinterpret_cast<const float4 *>(offp + (size_t)k0 * TM);
-        float4 *dst = reinterpret_cast<float4 *>(os);
-        for (int i = tid; i < kc * (TM / 4); i += 256)
-            dst[i] = src[i];
     };
 
     float mx[PX][MX];
@@ -244,7 +245,18 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
             s[p][m] = 0.0f;
 
     if (prod) {
-        // ---- one sweep: s = sum_k exp2(x_k - mp) * exp2(o_k - mo), rescaled when a chunk raises mp ----
+        // ---- one sweep on the fp32 matrix cores: S[instance][pixel] = sum_k exp2(o_k - mo) * exp2(x_k - mp), in
+        //      tiles of 16 instances x 16 pixels x 4 k (v_mfma_f32_16x16x4_f32: lane (lr, lq) supplies
+        //      A[instance lr][k lq] and B[k lq][pixel lr] and holds D[instance 4*lq + v][pixel lr]); the sums are
+        //      rescaled when a chunk raises mp ----
+        constexpr int NT = 4 * PX;  // 16-pixel tiles across the workgroup's pixels
+        const int lr = lane & 15, lq = lane >> 4;
+        floatx4 acc[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        const float *xa = xs + lq * XP + lr;
+        const float *oa = os + lq * TM + wm * MX + lr;
         for (int k0 = 0; k0 < a.K; k0 += KC) {
             const int kc = min(KC, a.K - k0);
             __syncthreads();
@@ -254,39 +266,79 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                 continue;
             if (k0 > 0) {
 #pragma unroll
-                for (int p = 0; p < PX; ++p) {
-                    const float f = fsh[p * 64 + lane];
+                for (int t = 0; t < NT; ++t)
+                    acc[t] *= fsh[t * 16 + lr];
+            }
+            const int kend = min((kc + 3) & ~3, (wk + 1) * KW);  // rows kc .. kend - 1 hold zeros
+#pragma unroll 2
+            for (int kq = wk * KW; kq < kend; kq += 4) {
+                const float av = oa[kq * TM];
+                float bv[NT];
 #pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        s[p][m] *= f;
+                for (int t = 0; t < NT; ++t)
+                    bv[t] = xa[kq * XP + t * 16];
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv[t], acc[t], 0, 0, 0);
+            }
+        }
+        float mp[NT];
+#pragma unroll
+        for (int t = 0; t < NT; ++t)
+            mp[t] = msh[t * 16 + lr];
+        if (KS > 1) {
+            // the K-split waves saw the same pixel maxima: their sums add up in wave wk == 0
+            __syncthreads();  // everyone is done with xs / os
+            if (wk > 0 && wave_active) {
+                float *mg = smem + (size_t)((wk - 1) * WM + wm) * (NT * 4 * 64) + lane;
+#pragma unroll
+                for (int t = 0; t < NT; ++t)
+#pragma unroll
+                    for (int v = 0; v < 4; ++v)
+                        mg[(t * 4 + v) * 64] = acc[t][v];
+            }
+            __syncthreads();
+            if (wk > 0)
+                return;
+            if (wave_active) {
+                for (int j = 1; j < KS; ++j) {
+                    const float *src = smem + (size_t)((j - 1) * WM + wm) * (NT * 4 * 64) + lane;
+#pragma unroll
+                    for (int t = 0; t < NT; ++t)
+#pragma unroll
+                        for (int v = 0; v < 4; ++v)
+                            acc[t][v] += src[(t * 4 + v) * 64];
                 }
             }
-            const int kend = min(kc, (wk + 1) * KW);
-            for (int kk = wk * KW; kk < kend; ++kk) {
-                float x[PX], o[MX];
+        }
+        if (!wave_active)
+            return;
+        const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+        const float *omax = a.omax + ((size_t)r * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
+        float shift[4];
 #pragma unroll
-                for (int p = 0; p < PX; ++p)
-                    x[p] = xl[kk * XP + p * 64];
+        for (int v = 0; v < 4; ++v)
+            shift[v] = omax[v] + a.c0;
+        const size_t row0 = (size_t)(m0 + 4 * lq) * plane;  // this lane's first instance row
+        const bool all_rows = m0 + MX <= a.M;               // same for the whole wave
 #pragma unroll
-                for (int m = 0; m < MX; ++m)
-                    o[m] = ol[kk * TM + m];
+        for (int t = 0; t < NT; ++t) {
+            const long long po = pout[t * 16 + lr];  // written before the first barrier
+            if (po < 0)
+                continue;
+            float *o = a.out + po + row0;
+            // an infinite pixel bound makes the result NaN, as the reference's exp(inf - inf) does
+            const float mpt = (mp[t] - mp[t]) + mp[t];
 #pragma unroll
-                for (int p = 0; p < PX; ++p)
-#pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        s[p][m] = __builtin_fmaf(x[p], o[m], s[p][m]);
+            for (int v = 0; v < 4; ++v) {
+                const float res = (__builtin_amdgcn_logf(acc[t][v]) + (mpt + shift[v])) * a.ln2_over_eps;
+                if (all_rows || m0 + 4 * lq + v < a.M)
+                    o[v * plane] = res;
             }
         }
-        // the shift of every instance: the pixel bound (an infinite one makes the result NaN, as the reference's
-        // exp(inf - inf) does); the instance bound is added in the epilogue
-#pragma unroll
-        for (int p = 0; p < PX; ++p) {
-            const float mp = msh[p * 64 + lane];
-#pragma unroll
-            for (int m = 0; m < MX; ++m)
-                mx[p][m] = mp;
-        }
-    } else {
+        return;
+    }
+    {
     // ---- sweep 1: running max (min for negative epsilon) of patch + offset ----
     for (int k0 = 0; k0 < a.K; k0 += KC) {
         const int kc = min(KC, a.K - k0);
@@ -409,14 +461,6 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 
     // output channel = instance * channels_out + c  (src/kernels/mex_kernel_cpu.cpp:113-115)
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
-    if (prod) {
-        const float *omax = a.omax + ((size_t)r * a.n_mgroups + mgroup) * TM + wm * MX;
-#pragma unroll
-        for (int p = 0; p < PX; ++p)
-#pragma unroll
-            for (int m = 0; m < MX; ++m)
-                mx[p][m] = (mx[p][m] - mx[p][m]) + mx[p][m] + omax[m];
-    }
 #pragma unroll
     for (int p = 0; p < PX; ++p) {
         const PixelRef cp = locate(a, r, chunk * TP + p * 64 + lane);
@@ -442,8 +486,18 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                                                               int n_mgroups, int tm, int normalize, float scale,
                                                               int finite_eps, float *__restrict__ offp,
                                                               float *__restrict__ offe, float *__restrict__ omax,
-                                                              float *__restrict__ orng)
+                                                              float *__restrict__ orng, int4 *__restrict__ ktab, int H,
+                                                              int W, int bh, int bw)
 {
+    if (blockIdx.x == 0) {
+        // patch element k = (dc*bh + dh)*bw + dw -> where it lies relative to the patch origin
+        for (int k = threadIdx.x; k < K; k += 256) {
+            const int dc = k / (bh * bw);
+            const int rem = k - dc * bh * bw;
+            const int dh = rem / bw, dw = rem - dh * bw;
+            ktab[k] = make_int4((dc * H + dh) * W + dw, dc, dh, dw);
+        }
+    }
     const int lane = threadIdx.x & 63;
     const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
     const long long rows = (long long)R * n_mgroups * tm;
@@ -729,7 +783,8 @@ size_t mex_workspace_bytes(const MexPlan &p)
     const MexTiling t = mex_tiling(p);
     const size_t packed = align_up((size_t)p.d.num_regions * t.n_mgroups * p.d.K * t.tm * sizeof(float), 256);
     const size_t rows = align_up((size_t)p.d.num_regions * t.n_mgroups * t.tm * sizeof(float), 256);
-    return 2 * packed + 2 * rows;  // scaled offsets, their exponentials; row maxima, row ranges
+    // scaled offsets, their exponentials; row maxima, row ranges; patch element table
+    return 2 * packed + 2 * rows + align_up((size_t)p.d.K * sizeof(int4), 256);
 }
 
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
@@ -768,15 +823,16 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     float *offe = reinterpret_cast<float *>(ws + packed);
     float *omax = reinterpret_cast<float *>(ws + 2 * packed);
     float *orng = reinterpret_cast<float *>(ws + 2 * packed + row_bytes);
+    int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
 
     MexKernelArgs a = mex_kernel_args(p);
     hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, offsets,
                        d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, a.scale, a.finite_eps, offp,
-                       offe, omax, orng);
+                       offe, omax, orng, ktab, p.H, p.W, d.block_h, d.block_w);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
 
-    a.in = input; a.out = output; a.offp = offp; a.offe = offe; a.omax = omax; a.orng = orng;
+    a.in = input; a.out = output; a.offp = offp; a.offe = offe; a.omax = omax; a.orng = orng; a.ktab = ktab;
     a.n_mgroups = t.n_mgroups;
     a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;
 
@@ -788,7 +844,7 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     a.cpr = (a.slots + 64 * t.px - 1) / (64 * t.px);
     const long long supers = (a.cpr + kXcds - 1) / kXcds;
     const long long gx = supers * kXcds * d.num_regions;
-    if (gx > 0x7fffffffLL || t.n_mgroups > 65535)
+    if (gx > 0x7fffffffLL || t.n_mgroups > 65535 || (long long)d.block_c * p.H * p.W > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
     dim3 grid((unsigned)gx, (unsigned)t.n_mgroups);
     // finite eps: values are pre-multiplied by eps*log2(e), so the shift is always the maximum

@@ -9,6 +9,36 @@
 
 namespace simnets {
 
+// Division of a 32-bit unsigned number by a divisor fixed at launch time: one multiply-high and a few shifts
+// (Granlund & Montgomery, "Division by invariant integers using multiplication", figure 4.1, N = 32); exact for
+// every n < 2^32 and d >= 1.
+struct FastDiv {
+    unsigned mul, sh1, sh2, d;
+};
+
+inline FastDiv make_fast_div(unsigned d)
+{
+    FastDiv f;
+    unsigned l = 0;
+    while (l < 32 && (1ull << l) < d)
+        ++l;  // ceil(log2 d)
+    f.mul = (unsigned)(((1ull << 32) * ((1ull << l) - d)) / d + 1);
+    f.sh1 = l < 1 ? l : 1;
+    f.sh2 = l > 0 ? l - 1 : 0;
+    f.d = d;
+    return f;
+}
+
+__host__ __device__ __forceinline__ unsigned fast_div(unsigned n, const FastDiv &f)
+{
+#if defined(__HIP_DEVICE_COMPILE__)
+    const unsigned t = __umulhi(f.mul, n);
+#else
+    const unsigned t = (unsigned)(((unsigned long long)f.mul * n) >> 32);
+#endif
+    return (t + ((n - t) >> f.sh1)) >> f.sh2;
+}
+
 struct MexKernelArgs {
     const float *in;
     float *out;
@@ -16,6 +46,7 @@ struct MexKernelArgs {
     const float *offe;  // [R][mgroup][K][TM]  exp2(offsets * scale - row maximum)   (finite epsilon only)
     const float *omax;  // [R][mgroup][TM]     row maximum of offsets * scale
     const float *orng;  // [R][mgroup][TM]     row maximum - row minimum of offsets * scale
+    const int4 *ktab;   // [K] patch element k -> {offset (dc*H + dh)*W + dw inside an image, dc, dh, dw}
     int B, C, H, W;
     int Co, Ho, Wo;
     int bc, bh, bw, sc, sh, sw, pc, ph, pw;
@@ -24,6 +55,8 @@ struct MexKernelArgs {
     int unshared;
     int R;              // num_regions
     int RS;             // region_size
+    FastDiv dRS, dWs, dWsHs, dWg, dWgHg;  // divisions of locate()
+    FastDiv dSuper;     // by 8 * R: workgroup numbering of the forward kernel
     int slots;          // B * RS
     int cpr;            // pixel chunks (64*PX slots) per region
     int M, K, n_mgroups;
@@ -47,16 +80,18 @@ struct PixelRef {
 // out_off = -1 and read pixel (0,0,0) of image 0.
 __device__ __forceinline__ PixelRef locate(const MexKernelArgs &a, int r, int slot)
 {
-    const int w_g = r % a.Wg;
-    const int h_g = (r / a.Wg) % a.Hg;
-    const int c_g = r / (a.Wg * a.Hg);
+    const int rw = (int)fast_div((unsigned)r, a.dWg);
+    const int w_g = r - rw * a.Wg;
+    const int c_g = (int)fast_div((unsigned)r, a.dWgHg);
+    const int h_g = rw - c_g * a.Hg;
     bool valid = slot < a.slots;
     const int sl = valid ? slot : 0;
-    const int b = sl / a.RS;
+    const int b = (int)fast_div((unsigned)sl, a.dRS);
     const int q = sl - b * a.RS;
-    const int i = q % a.Ws;
-    const int j = (q / a.Ws) % a.Hs;
-    const int l = q / (a.Ws * a.Hs);
+    const int qw = (int)fast_div((unsigned)q, a.dWs);
+    const int i = q - qw * a.Ws;
+    const int l = (int)fast_div((unsigned)q, a.dWsHs);
+    const int j = qw - l * a.Hs;
     int c, h, w;
     if (a.unshared) {
         c = c_g + l * a.Cg; h = h_g + j * a.Hg; w = w_g + i * a.Wg;
@@ -81,7 +116,7 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
 {
     const simnets_mex_dims &d = p.d;
     MexKernelArgs a;
-    a.in = nullptr; a.out = nullptr; a.offp = nullptr; a.offe = nullptr; a.omax = nullptr; a.orng = nullptr;
+    a.in = nullptr; a.out = nullptr; a.offp = nullptr; a.offe = nullptr; a.omax = nullptr; a.orng = nullptr; a.ktab = nullptr;
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W;
     a.Co = d.channels_out; a.Ho = d.height_out; a.Wo = d.width_out;
     a.bc = d.block_c; a.bh = d.block_h; a.bw = d.block_w;
@@ -93,6 +128,10 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     a.R = d.num_regions;
     a.RS = d.region_size;
     a.slots = p.B * d.region_size;
+    a.dRS = make_fast_div((unsigned)a.RS); a.dWs = make_fast_div((unsigned)a.Ws);
+    a.dWsHs = make_fast_div((unsigned)(a.Ws * a.Hs));
+    a.dWg = make_fast_div((unsigned)a.Wg); a.dWgHg = make_fast_div((unsigned)(a.Wg * a.Hg));
+    a.dSuper = make_fast_div(8u * (unsigned)a.R);
     a.cpr = 0;
     a.M = d.M; a.K = d.K; a.n_mgroups = 0;
     const double log2e = 1.4426950408889634;
