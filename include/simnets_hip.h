@@ -234,6 +234,19 @@ int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input
 int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, const float *input, float *output,
                              void *stream);
 
+/* MEX followed by that sum pooling, as one call: output [B, M*channels_out, height_out/pool_h, width_out/pool_w]
+ * = simnets_hip_sum_pool_fwd(simnets_hip_mex_fwd(...)).  The pair the reference's networks run back to back
+ * (README.md:108-129: MEX with unshared_offset_region = the pooling window, then pooling).  When the offsets are
+ * unshared with regions [1, pool_h, pool_w] (a pooling window is then one pixel of every region), epsilon is finite
+ * and the window has 2 or 4 pixels, one kernel computes the MEX values of a window in one lane, adds them in the
+ * window's row-major order and writes only the pooled tensor; any other geometry runs the two kernels through
+ * scratch memory.  No gradient entry point takes the pooled tensor: training keeps the two separate calls. */
+int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
+                                             int pool_w, size_t *bytes);
+int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
+                                 void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -15,6 +15,7 @@ EXPORTS = [
     "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
     "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
     "simnets_hip_mex_offsets_grad",
+    "simnets_hip_mex_sum_pool_workspace_bytes", "simnets_hip_mex_sum_pool_fwd",
 ]
 
 SIM_L1, SIM_L2 = 0, 1
@@ -96,6 +97,10 @@ def lib():
         l.simnets_hip_mex_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
         l.simnets_hip_mex_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, C.c_size_t, P]
         l.simnets_hip_sum_pool_fwd.argtypes = [I4, C.c_int, C.c_int, P, P, P]
+        l.simnets_hip_mex_sum_pool_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.c_int, C.c_int,
+                                                               C.POINTER(C.c_size_t)]
+        l.simnets_hip_mex_sum_pool_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int, P, P,
+                                                   C.c_size_t, P]
         SZ = C.POINTER(C.c_size_t)
         l.simnets_hip_similarity_grad_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, SZ, SZ]
         l.simnets_hip_similarity_input_grad.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P, P,
@@ -115,7 +120,8 @@ def lib():
                      "get_mex_offsets_nregions", "simnets_hip_similarity_grad_workspace_bytes",
                      "simnets_hip_similarity_input_grad", "simnets_hip_similarity_params_grad",
                      "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
-                     "simnets_hip_mex_offsets_grad"):
+                     "simnets_hip_mex_offsets_grad", "simnets_hip_mex_sum_pool_workspace_bytes",
+                     "simnets_hip_mex_sum_pool_fwd"):
             getattr(l, name).restype = C.c_int
         _lib = l
     return _lib

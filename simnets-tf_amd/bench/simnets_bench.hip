@@ -373,6 +373,23 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) stack();
         float ms = time_ms(s, steps, stack);
         report("config4 missing-data stack batch 512", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        // the same stack with each MEX + pooling pair as one call (simnets_hip_mex_sum_pool_fwd)
+        std::vector<void *> fws(4);
+        std::vector<size_t> fbytes(4);
+        for (int l = 0; l < 4; ++l) {
+            SN_OK(simnets_hip_mex_sum_pool_workspace_bytes(&mex[l].a, mex[l].in, 2, 2, &fbytes[l]));
+            HIP_OK(hipMalloc(&fws[l], std::max<size_t>(fbytes[l], 256)));
+        }
+        auto fused = [&] {
+            run_sim(sc, s);
+            for (int l = 0; l < 4; ++l)
+                SN_OK(simnets_hip_mex_sum_pool_fwd(&mex[l].a, mex[l].in, mex[l].x, mex[l].o, mex[l].off_count, 2, 2,
+                                                   pooled[l], fws[l], fbytes[l], s));
+            run_mex(mex[4], s);
+        };
+        for (int i = 0; i < warmup; ++i) fused();
+        ms = time_ms(s, steps, fused);
+        report("config4 missing-data stack batch 512, MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
     }
     else if (config == 5) {
         // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)

@@ -16,7 +16,7 @@ BENCH = os.path.join(HERE, "simnets_bench")
 OBJDIR = os.path.join(HERE, "build")
 
 SOURCES = ["host_logic.cpp", "capi.hip", "similarity_direct.hip", "similarity_mfma.hip", "mex.hip",
-           "similarity_grad.hip", "mex_grad.hip"]
+           "similarity_grad.hip", "mex_grad.hip", "mex_pool.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 COMMON = ["-O3", "-std=c++17", "-fPIC", "-I" + os.path.join(ROOT, "include"), "-I" + CSRC, "-Wall",
@@ -39,7 +39,7 @@ def _compile(src, extra):
 def build(extra=(), verbose=False):
     os.makedirs(OBJDIR, exist_ok=True)
     extra = list(extra)
-    with ThreadPoolExecutor(max_workers=min(len(SOURCES), 7)) as ex:
+    with ThreadPoolExecutor(max_workers=min(len(SOURCES), 8)) as ex:
         objs = list(ex.map(lambda s: _compile(s, extra), SOURCES))
     subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs, check=True)
     # standalone C++ harness, linked against the product library only

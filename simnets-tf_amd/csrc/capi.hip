@@ -174,4 +174,42 @@ int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, c
                            output, stream);
 }
 
+int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
+                                             int pool_w, size_t *bytes)
+{
+    if (!bytes)
+        return SIMNETS_ERR_NULL_POINTER;
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    if (pool_h <= 0 || pool_w <= 0)
+        return SIMNETS_ERR_SHAPE;
+    if (p.d.height_out / pool_h <= 0 || p.d.width_out / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    *bytes = mex_pool_workspace_bytes(p, pool_h, pool_w);
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
+                                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    if (pool_h <= 0 || pool_w <= 0 || offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
+        return SIMNETS_ERR_SHAPE;
+    if (p.d.height_out / pool_h <= 0 || p.d.width_out / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !offsets || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, mex_pool_workspace_bytes(p, pool_h, pool_w)))
+        return SIMNETS_ERR_WORKSPACE;
+    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream);
+}
+
 }  // extern "C"

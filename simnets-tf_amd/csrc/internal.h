@@ -63,6 +63,11 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
                      void *stream);
 
 int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *input, float *output, void *stream);
+// MEX followed by non-overlapping sum pooling: one fused kernel when a pooling window is one pixel of every
+// offsets region, else MEX into scratch + pooling
+size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw);
+int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
+                    void *workspace, size_t workspace_bytes, void *stream);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

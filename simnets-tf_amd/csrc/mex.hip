@@ -44,7 +44,6 @@ namespace {
 constexpr int MX = 16;        // instances per wave
 constexpr int kChunkMin = 32;  // k per LDS chunk: 32, or 64 / 128 for long K with one pixel per lane
 constexpr int kXcds = 8;
-constexpr float kProductRange = 90.0f;  // widest row range of the scaled offsets (a power of two) the product form takes
 #ifndef SIMNETS_MEX_WAVES
 #define SIMNETS_MEX_WAVES 4096  // pixels per lane shrink until the grid has this many waves
 #endif
@@ -778,13 +777,44 @@ MexTiling mex_tiling(const MexPlan &p)
 
 }  // namespace
 
+size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups)
+{
+    const size_t packed = align_up((size_t)p.d.num_regions * n_mgroups * p.d.K * tm * sizeof(float), 256);
+    const size_t rows = align_up((size_t)p.d.num_regions * n_mgroups * tm * sizeof(float), 256);
+    // scaled offsets, their exponentials; row maxima, row ranges; patch element table
+    return 2 * packed + 2 * rows + align_up((size_t)p.d.K * sizeof(int4), 256);
+}
+
+int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
+                     void *stream)
+{
+    const simnets_mex_dims &d = p.d;
+    const long long rows = (long long)d.num_regions * n_mgroups * tm;
+    const size_t packed = align_up((size_t)rows * d.K * sizeof(float), 256);
+    const size_t row_bytes = align_up((size_t)rows * sizeof(float), 256);
+    char *ws = reinterpret_cast<char *>(workspace);
+    float *offp = reinterpret_cast<float *>(ws);
+    float *offe = reinterpret_cast<float *>(ws + packed);
+    float *omax = reinterpret_cast<float *>(ws + 2 * packed);
+    float *orng = reinterpret_cast<float *>(ws + 2 * packed + row_bytes);
+    int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
+    if ((long long)d.block_c * p.H * p.W > 0x7fffffffLL)
+        return SIMNETS_ERR_TOO_LARGE;  // the table holds 32-bit offsets
+    hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       reinterpret_cast<hipStream_t>(stream), offsets, d.num_regions, d.M, d.K, n_mgroups, tm,
+                       p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W, d.block_h,
+                       d.block_w);
+    if (hipGetLastError() != hipSuccess)
+        return SIMNETS_ERR_HIP;
+    a->offp = offp; a->offe = offe; a->omax = omax; a->orng = orng; a->ktab = ktab;
+    a->n_mgroups = n_mgroups;
+    return SIMNETS_OK;
+}
+
 size_t mex_workspace_bytes(const MexPlan &p)
 {
     const MexTiling t = mex_tiling(p);
-    const size_t packed = align_up((size_t)p.d.num_regions * t.n_mgroups * p.d.K * t.tm * sizeof(float), 256);
-    const size_t rows = align_up((size_t)p.d.num_regions * t.n_mgroups * t.tm * sizeof(float), 256);
-    // scaled offsets, their exponentials; row maxima, row ranges; patch element table
-    return 2 * packed + 2 * rows + align_up((size_t)p.d.K * sizeof(int4), 256);
+    return mex_packed_bytes(p, t.tm, t.n_mgroups);
 }
 
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
@@ -815,25 +845,11 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
         return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
     }
     const MexTiling t = mex_tiling(p);
-    const long long rows = (long long)d.num_regions * t.n_mgroups * t.tm;
-    const size_t packed = align_up((size_t)rows * d.K * sizeof(float), 256);
-    const size_t row_bytes = align_up((size_t)rows * sizeof(float), 256);
-    char *ws = reinterpret_cast<char *>(workspace);
-    float *offp = reinterpret_cast<float *>(ws);
-    float *offe = reinterpret_cast<float *>(ws + packed);
-    float *omax = reinterpret_cast<float *>(ws + 2 * packed);
-    float *orng = reinterpret_cast<float *>(ws + 2 * packed + row_bytes);
-    int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
-
     MexKernelArgs a = mex_kernel_args(p);
-    hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, offsets,
-                       d.num_regions, d.M, d.K, t.n_mgroups, t.tm, p.normalize_offsets, a.scale, a.finite_eps, offp,
-                       offe, omax, orng, ktab, p.H, p.W, d.block_h, d.block_w);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
-
-    a.in = input; a.out = output; a.offp = offp; a.offe = offe; a.omax = omax; a.orng = orng; a.ktab = ktab;
-    a.n_mgroups = t.n_mgroups;
+    const int rc = mex_pack_offsets(p, offsets, t.tm, t.n_mgroups, workspace, &a, stream);
+    if (rc)
+        return rc;
+    a.in = input; a.out = output;
     a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;
 
     // bounds checks are needed unless every patch lies inside the image
@@ -844,7 +860,7 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     a.cpr = (a.slots + 64 * t.px - 1) / (64 * t.px);
     const long long supers = (a.cpr + kXcds - 1) / kXcds;
     const long long gx = supers * kXcds * d.num_regions;
-    if (gx > 0x7fffffffLL || t.n_mgroups > 65535 || (long long)d.block_c * p.H * p.W > 0x7fffffffLL)
+    if (gx > 0x7fffffffLL || t.n_mgroups > 65535)
         return SIMNETS_ERR_TOO_LARGE;
     dim3 grid((unsigned)gx, (unsigned)t.n_mgroups);
     // finite eps: values are pre-multiplied by eps*log2(e), so the shift is always the maximum

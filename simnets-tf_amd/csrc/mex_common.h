@@ -69,6 +69,10 @@ struct MexKernelArgs {
     float oob;
 };
 
+// widest row range of the scaled offsets (an exponent of two) for which the forward kernels use the product form
+// sum_k exp2(x_k - max x) * exp2(o_k - max o): the largest term is at least exp2(-range)
+constexpr float kProductRange = 90.0f;
+
 struct PixelRef {
     const float *base;  // &input[b][c*sc-pc][h*sh-ph][w*sw-pw] (only dereferenced inside the image)
     int ci0, hi0, wi0;
@@ -146,5 +150,12 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     a.kgather = 0;
     return a;
 }
+
+// Packs the offsets for the forward kernels (k-major tiles of tm instances per group: scaled values, their
+// exponentials relative to the row maximum, row maxima and ranges) and the patch element table into `workspace`
+// (mex_packed_bytes), and points the argument block at them.
+size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
+int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
+                     void *stream);
 
 }  // namespace simnets

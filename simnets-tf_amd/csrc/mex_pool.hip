@@ -1,0 +1,339 @@
+// MEX forward fused with the non-overlapping sum pooling that follows it in the reference's networks
+// (README.md:108-129, examples/mnist_ght_model_missing_data.py:60-66: MEX with unshared offset regions of the
+// pooling window's size, then AveragePooling2D * window area).
+//
+// With unshared regions [1, ph, pw] the pixels of one pooling window are one pixel of each of the ph*pw regions,
+// and they carry the same slot number inside their regions (include/utils/mex_utils.hpp:69-116).  A workgroup
+// therefore takes 16 (or 32) slots of ALL regions and 64 instances: the MEX values of a window end up in one
+// lane and are added there, in the window's row-major order (the order sum pooling uses), and only the pooled
+// tensor is written: a quarter of the MEX output, and no pooling launch.
+//
+// Arithmetic as in the tiled forward kernel (finite epsilon): product form on the fp32 matrix cores,
+//   S[instance][pixel] = sum_k exp2(o_k - max o) * exp2(x_k - max x)   (v_mfma_f32_16x16x4_f32),
+// per 16-pixel tile with the offsets tile of that tile's region; workgroups whose offsets span too wide a range
+// for the product form evaluate the logsumexp term by term instead (slow, rare).
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+
+#include "internal.h"
+#include "mex_common.h"
+
+namespace simnets {
+
+namespace {
+
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+constexpr int KC = 32;             // k per LDS chunk
+constexpr int TM = 64, MX = 16;    // instances per workgroup / per wave
+constexpr int KSTEP = 4, U = KC / KSTEP;
+constexpr int XP = 64;             // pixel columns of a workgroup: 4 tiles of 16
+
+struct PoolArgs {
+    float *pooled;
+    int Hp, Wp;   // pooled height and width
+    int spw;      // slots per workgroup: 64 / R
+};
+
+template <int R, bool CHECK>
+__global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, const PoolArgs q)
+{
+    constexpr int G = 4 / R;       // slot groups of 16 per workgroup
+    __shared__ __attribute__((aligned(16))) float xs[KC * XP];       // [k][column]
+    __shared__ __attribute__((aligned(16))) float os[R * KC * TM];   // [region][k][instance]
+    __shared__ float pmx[KSTEP * XP];   // partial column maxima
+    __shared__ float fsh[XP], msh[XP];  // per column: rescale factor of this chunk, running maximum
+    __shared__ long long ppos[16 * G];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // instance wave; also the k phase when staging
+    const int chunk = blockIdx.x, mgroup = blockIdx.y;
+    const int m0 = mgroup * TM + wm * MX;
+    const bool wave_active = m0 < a.M;
+
+    // staging role: column of tile (slot group, region), consecutive threads = neighbouring pixels of a window row
+    const int sreg = lane % R, ssl = lane / R;
+    const int col = ((ssl >> 4) * R + sreg) * 16 + (ssl & 15);
+    const PixelRef gp = locate(a, sreg, chunk * (16 * G) + ssl);
+
+    if (tid < 16 * G) {
+        const int slot = chunk * (16 * G) + tid;
+        long long pos = -1;
+        if (slot < a.slots) {
+            const int b = (int)fast_div((unsigned)slot, a.dRS);
+            const int sq = slot - b * a.RS;
+            const int qw = (int)fast_div((unsigned)sq, a.dWs);
+            const int i = sq - qw * a.Ws;
+            const int l = (int)fast_div((unsigned)sq, a.dWsHs);
+            const int j = qw - l * a.Hs;
+            if (l < a.Co && j < q.Hp && i < q.Wp)
+                pos = ((long long)b * a.M * a.Co + l) * ((long long)q.Hp * q.Wp) + (long long)j * q.Wp + i;
+        }
+        ppos[tid] = pos;
+    }
+
+    bool prod;
+    {
+        int wide = 0;
+        if (tid < TM) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+                wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
+        }
+        prod = !__syncthreads_or(wide);
+    }
+    float m_run = -INFINITY;  // running maximum of this thread's staging column
+
+    auto stage = [&](int k0, int kc) {
+        const bool full = kc == KC;
+        float v[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int kk = wm + u * KSTEP;
+            const int4 ke = a.ktab[k0 + (full ? kk : min(kk, kc - 1))];  // same for the whole wave: scalar load
+            if (CHECK) {
+                const int ci = gp.ci0 + ke.y, hi = gp.hi0 + ke.z, wi = gp.wi0 + ke.w;
+                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                v[u] = ok ? gp.base[ke.x] : a.oob;
+            } else {
+                v[u] = gp.base[ke.x];
+            }
+        }
+        // offsets tiles of the R regions: straight copies of kc * TM floats each
+        const int on = kc * (TM / 4);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float4 *src = reinterpret_cast<const float4 *>(
+                (prod ? a.offe : a.offp) + (((size_t)r * a.n_mgroups + mgroup) * a.K + k0) * TM);
+            float4 *dst = reinterpret_cast<float4 *>(os + r * KC * TM);
+            for (int i = tid; i < on; i += 256)
+                dst[i] = src[i];
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            v[u] *= a.scale;
+        if (!prod) {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (full || wm + u * KSTEP < kc)
+                    xs[(wm + u * KSTEP) * XP + col] = v[u];
+            return;
+        }
+        // column maximum over the chunk -> running maximum; the staged values become exp2(x - maximum)
+        float pm = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (full || wm + u * KSTEP < kc)
+                pm = fmaxf(pm, v[u]);
+        pmx[wm * XP + col] = pm;
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < KSTEP; ++j)
+            pm = fmaxf(pm, pmx[j * XP + col]);
+        const float m_new = fmaxf(m_run, pm);
+        const float m_sub = m_new == -INFINITY ? 0.0f : m_new;  // nothing finite yet: the terms are exp2(-inf) = 0
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (full || wm + u * KSTEP < kc)
+                xs[(wm + u * KSTEP) * XP + col] = __builtin_amdgcn_exp2f(v[u] - m_sub);
+        if (wm == 0) {
+            fsh[col] = m_run == m_new ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+            msh[col] = m_new;
+        }
+        m_run = m_new;
+        if (!full) {
+            // the matrix instruction takes 4 k at a time: rows kc .. next multiple of 4 are zeros
+            const int kc4 = (kc + 3) & ~3;
+            for (int i = tid; i < (kc4 - kc) * XP; i += 256)
+                xs[kc * XP + i] = 0.0f;
+            for (int i = tid; i < (kc4 - kc) * TM * R; i += 256)
+                os[(i / ((kc4 - kc) * TM)) * KC * TM + kc * TM + i % ((kc4 - kc) * TM)] = 0.0f;
+        }
+    };
+
+    const int lr = lane & 15, lq = lane >> 4;
+    const size_t plane_p = (size_t)a.Co * q.Hp * q.Wp;
+    const size_t row0 = (size_t)(m0 + 4 * lq) * plane_p;  // this lane's first instance row
+    const bool all_rows = m0 + MX <= a.M;                 // same for the whole wave
+    float res[4][4];  // [tile][v]: MEX value of (pixel lr of the tile, instance m0 + 4*lq + v)
+
+    if (prod) {
+        floatx4 acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        const float *xa = xs + lq * XP + lr;
+        const float *oa = os + lq * TM + wm * MX + lr;
+        for (int k0 = 0; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            __syncthreads();
+            stage(k0, kc);
+            __syncthreads();
+            if (!wave_active)
+                continue;
+            if (k0 > 0) {
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[t] *= fsh[t * 16 + lr];
+            }
+            const int kend = (kc + 3) & ~3;
+            for (int kq = 0; kq < kend; kq += 4) {
+                float av[R], bv[4];
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+                    av[r] = oa[r * KC * TM + kq * TM];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    bv[t] = xa[kq * XP + t * 16];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t % R], bv[t], acc[t], 0, 0, 0);
+            }
+        }
+        if (!wave_active)
+            return;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float *omax = a.omax + ((size_t)(t % R) * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
+            const float mp = msh[t * 16 + lr];
+            // an infinite column bound makes the result NaN, as the reference's exp(inf - inf) does
+            const float mpt = (mp - mp) + mp + a.c0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                res[t][v] = (__builtin_amdgcn_logf(acc[t][v]) + (mpt + omax[v])) * a.ln2_over_eps;
+        }
+    } else {
+        // term by term: running (maximum, sum) per output, rescaled when a chunk raises the maximum
+        float best[4][4], sum[4][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                best[t][v] = -INFINITY;
+                sum[t][v] = 0.0f;
+            }
+        for (int k0 = 0; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            __syncthreads();
+            stage(k0, kc);
+            __syncthreads();
+            if (!wave_active)
+                continue;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const float *xc = xs + t * 16 + lr;
+                    const float *oc = os + (t % R) * KC * TM + wm * MX + 4 * lq + v;
+                    float cb = -INFINITY;
+                    for (int kk = 0; kk < kc; ++kk)
+                        cb = fmaxf(cb, xc[kk * XP] + oc[kk * TM]);
+                    const float nb = fmaxf(best[t][v], cb);
+                    const float nsub = nb == -INFINITY ? 0.0f : nb;
+                    float sacc = sum[t][v] * (best[t][v] == nb ? 1.0f : __builtin_amdgcn_exp2f(best[t][v] - nb));
+                    for (int kk = 0; kk < kc; ++kk)
+                        sacc += __builtin_amdgcn_exp2f(xc[kk * XP] + oc[kk * TM] - nsub);
+                    sum[t][v] = sacc;
+                    best[t][v] = nb;
+                }
+        }
+        if (!wave_active)
+            return;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float b = best[t][v];
+                res[t][v] = (__builtin_amdgcn_logf(sum[t][v]) + ((b - b) + b + a.c0)) * a.ln2_over_eps;
+            }
+    }
+
+    // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+        const long long pos = ppos[g * 16 + lr];  // written before the first barrier
+        if (pos < 0)
+            continue;
+        float *o = q.pooled + pos + row0;
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            float w = res[g * R][v];
+#pragma unroll
+            for (int r = 1; r < R; ++r)
+                w += res[g * R + r][v];
+            if (all_rows || m0 + 4 * lq + v < a.M)
+                o[v * plane_p] = w;
+        }
+    }
+}
+
+template <int R>
+hipError_t launch_pool(const MexKernelArgs &a, const PoolArgs &q, dim3 grid, bool inside, hipStream_t s)
+{
+    if (inside)
+        hipLaunchKernelGGL((mex_pool_kernel<R, false>), grid, dim3(256), 0, s, a, q);
+    else
+        hipLaunchKernelGGL((mex_pool_kernel<R, true>), grid, dim3(256), 0, s, a, q);
+    return hipGetLastError();
+}
+
+// The fused kernel applies when a pooling window is exactly one pixel of every offsets region.
+bool fusable(const MexPlan &p, int ph, int pw)
+{
+    const simnets_mex_dims &d = p.d;
+    const int r = ph * pw;
+    return p.use_unshared && std::isfinite(p.epsilon) && d.offsets_c == 1 && d.offsets_h == ph && d.offsets_w == pw &&
+           (r == 2 || r == 4) && d.num_regions == r;
+}
+
+}  // namespace
+
+size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw)
+{
+    if (fusable(p, ph, pw))
+        return mex_packed_bytes(p, TM, (p.d.M + TM - 1) / TM);
+    // otherwise: MEX into a scratch tensor, then the pooling kernel
+    const size_t out = (size_t)p.B * p.d.M * p.d.channels_out * p.d.height_out * p.d.width_out * sizeof(float);
+    return mex_workspace_bytes(p) + align_up(out, 256);
+}
+
+int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
+                    void *workspace, size_t workspace_bytes, void *stream)
+{
+    const simnets_mex_dims &d = p.d;
+    if (workspace_bytes < mex_pool_workspace_bytes(p, ph, pw))
+        return SIMNETS_ERR_WORKSPACE;
+    if (!fusable(p, ph, pw)) {
+        float *full = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_workspace_bytes(p));
+        const int rc = mex_launch(p, input, offsets, full, workspace, mex_workspace_bytes(p), stream);
+        if (rc)
+            return rc;
+        return sum_pool_launch(p.B, d.M * d.channels_out, d.height_out, d.width_out, ph, pw, full, pooled, stream);
+    }
+    const int n_mgroups = (d.M + TM - 1) / TM;
+    MexKernelArgs a = mex_kernel_args(p);
+    const int rc = mex_pack_offsets(p, offsets, TM, n_mgroups, workspace, &a, stream);
+    if (rc)
+        return rc;
+    a.in = input;
+    PoolArgs q;
+    q.pooled = pooled;
+    q.Hp = d.height_out / ph;
+    q.Wp = d.width_out / pw;
+    q.spw = 64 / (ph * pw);
+    const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
+    if (gx > 0x7fffffffLL || n_mgroups > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    const bool inside = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 &&
+                        (d.channels_out - 1) * d.stride_c + d.block_c <= p.C &&
+                        (d.height_out - 1) * d.stride_h + d.block_h <= p.H &&
+                        (d.width_out - 1) * d.stride_w + d.block_w <= p.W;
+    dim3 grid((unsigned)gx, (unsigned)n_mgroups);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const hipError_t e = ph * pw == 4 ? launch_pool<4>(a, q, grid, inside, s) : launch_pool<2>(a, q, grid, inside, s);
+    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+}  // namespace simnets

@@ -366,6 +366,42 @@ def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax
     return doff
 
 
+def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
+                 blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+                 use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+                 normalize_offsets=False, out=None):
+    """`sum_pooling(mex(...), pool_size)` as one call (forward only): the MEX layer + pooling pair of the reference's
+    networks (README.md:108-129).  With unshared offset regions equal to the pooling window and a finite epsilon a
+    single kernel writes only the pooled tensor; other geometries run the two kernels through scratch memory."""
+    x = _require_cuda_f32("input", input)
+    off = _require_cuda_f32("offsets", offsets)
+    if x.dim() != 4:
+        raise SimnetsError(-15)
+    a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
+                  epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
+                  blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
+                  shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
+                  normalize_offsets=normalize_offsets)
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    l = _lib.lib()
+    xs = (C.c_int * 4)(*x.shape)
+    oshape = (C.c_int * 4)()
+    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    pshape = (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw)
+    if out is None:
+        out = torch.empty(pshape, dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_mex_sum_pool_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), ph, pw,
+                                              out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return out
+
+
 def sum_pooling(input, pool_size=(2, 2), out=None):
     """Non-overlapping 'valid' sum pooling: the AveragePooling2D * area glue of the reference's
     missing-data example (README.md:108-111)."""

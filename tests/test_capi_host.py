@@ -177,6 +177,28 @@ def test_compute_entry_points_reject_bad_arguments_without_touching_the_device(p
     assert l.simnets_hip_sum_pool_fwd(I4(1, 1, 4, 4), 0, 2, None, None, None) == -15
 
 
+def test_fused_mex_sum_pool_entry_validates_without_touching_the_device(pkg):
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    m = pkg.ops.mex_attrs(8, blocks=[3, 1, 1], unshared_offset_region=[2])
+    fused, plain, split = C.c_size_t(), C.c_size_t(), C.c_size_t()
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), 2, 2, C.byref(fused)) == 0
+    assert l.simnets_hip_mex_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), C.byref(plain)) == 0
+    # a 3x3 window is not one pixel of each 2x2 region: MEX into scratch (the full output) + pooling
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), 3, 3, C.byref(split)) == 0
+    assert split.value >= plain.value + 2 * 8 * 8 * 8 * 4 > fused.value > 0
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), 0, 2, C.byref(fused)) == -15
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), 9, 2, C.byref(fused)) == -16
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), I4(2, 3, 8, 8), 2, 2, None) == -1
+    assert l.simnets_hip_mex_sum_pool_fwd(C.byref(m), I4(2, 3, 8, 8), 256, 256, 5, 2, 2, 256, None, 0, None) == -15
+    assert l.simnets_hip_mex_sum_pool_fwd(C.byref(m), I4(2, 3, 8, 8), None, 256, 4 * 8 * 3, 2, 2, 256, None, 0,
+                                          None) == -1
+    assert l.simnets_hip_mex_sum_pool_fwd(C.byref(m), I4(2, 3, 8, 8), 256, 256, 4 * 8 * 3, 2, 2, 256, None, 0,
+                                          None) == -17
+    assert l.simnets_hip_mex_sum_pool_fwd(C.byref(m), I4(0, 3, 8, 8), None, None, 4 * 8 * 3, 2, 2, None, None, 0,
+                                          None) == 0
+
+
 def test_op_layer_refuses_cpu_tensors(pkg):
     import torch
     x = torch.zeros(1, 1, 4, 4)

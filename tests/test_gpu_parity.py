@@ -283,6 +283,69 @@ def test_mex_offset_ranges_product_and_two_sweep_forms(pkg, geom, spread, eps):
     assert mex_err(got, x, off, n, **kw) <= MEX_TOL
 
 
+def pooled(y, ph, pw):
+    B, Cc, H, W = y.shape
+    return y[:, :, :H // ph * ph, :W // pw * pw].reshape(B, Cc, H // ph, ph, W // pw, pw).sum(axis=(3, 5))
+
+
+@pytest.mark.parametrize("case", [
+    dict(im=(9, 32, 16, 16), n=64, pool=(2, 2)),                       # the missing-data stack's first MEX layer
+    dict(im=(7, 100, 4, 4), n=70, pool=(2, 2)),                        # several K chunks, a partial instance group
+    dict(im=(5, 40, 2, 2), n=130, pool=(2, 2)),                        # one window per image
+    dict(im=(3, 6, 9, 11), n=20, pool=(2, 2)),                         # odd sizes: trailing row and column dropped
+    dict(im=(4, 8, 6, 10), n=33, pool=(1, 2)),                         # two-pixel windows
+    dict(im=(4, 8, 10, 6), n=33, pool=(2, 1)),
+    dict(im=(3, 5, 12, 12), n=24, pool=(2, 2), blocks=[5, 3, 3], padding=[0, 1, 1]),   # spatial blocks, padding
+    dict(im=(3, 6, 12, 12), n=24, pool=(2, 2), blocks=[2, 1, 1], strides=[2, 1, 1]),   # several output channels
+])
+@pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("wide", 1.0), ("mixed", 3.0)])
+def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
+    # unshared regions = the pooling window: one kernel computes a window's MEX values in one lane and adds them
+    g = np.random.default_rng(18)
+    Cc = case["im"][1]
+    ph, pw = case["pool"]
+    kw = dict(softmax_mode=False, blocks=case.get("blocks", [Cc, 1, 1]), strides=case.get("strides", [Cc, 1, 1]),
+              padding=case.get("padding", [0, 0, 0]), epsilon=eps, use_unshared_regions=True,
+              unshared_offset_region=[1, ph, pw], blocks_out_of_bounds_value=-2.0)
+    n = case["n"]
+    d = orc.mex_dims(orc.mex_args(case["im"], n, **kw))
+    assert d.num_regions == ph * pw
+    x = (g.normal(size=case["im"]) * 5).astype(np.float32)
+    off = (g.normal(size=(d.num_regions, n) + tuple(kw["blocks"])) * 0.3).astype(np.float32)
+    if spread == "wide":
+        off *= 400
+    elif spread == "mixed":
+        off[:, n // 2:] *= 400
+    got = pkg.mex_sum_pool(dev(x), dev(off), n, (ph, pw), **kw).cpu().numpy()
+    want = pooled(orc.mex_fwd(x, off, n, **kw), ph, pw)
+    shift = pooled(np.abs(orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, eps)))), ph, pw)
+    assert got.shape == want.shape
+    assert rel_err(got, want, floor=shift) <= MEX_TOL
+    # and it is the two separate calls, up to the rounding of the MEX values
+    two = pkg.sum_pooling(pkg.mex(dev(x), dev(off), n, **kw), (ph, pw)).cpu().numpy()
+    assert rel_err(got, two, floor=shift) <= 1e-5
+
+
+@pytest.mark.parametrize("kw,pool", [
+    (dict(use_unshared_regions=True, unshared_offset_region=[1, 2, 2], epsilon=math.inf), (2, 2)),   # max: no product form
+    (dict(use_unshared_regions=True, unshared_offset_region=[1, 2, 2]), (4, 4)),                     # window != regions
+    (dict(use_unshared_regions=False, shared_offset_region=[2]), (2, 2)),                            # shared regions
+    (dict(use_unshared_regions=True, unshared_offset_region=[2, 2, 2]), (2, 2)),                     # regions over channels
+])
+def test_mex_sum_pool_other_geometries_run_the_two_kernels(pkg, kw, pool):
+    g = np.random.default_rng(19)
+    kw = dict(dict(softmax_mode=True, blocks=[3, 1, 1], strides=[3, 1, 1]), **kw)
+    im, n = (4, 12, 8, 8), 10
+    d = orc.mex_dims(orc.mex_args(im, n, **kw))
+    x = g.normal(size=im).astype(np.float32)
+    off = g.normal(size=(d.num_regions, n, 3, 1, 1)).astype(np.float32)
+    got = pkg.mex_sum_pool(dev(x), dev(off), n, pool, **kw).cpu().numpy()
+    two = pkg.sum_pooling(pkg.mex(dev(x), dev(off), n, **kw), pool).cpu().numpy()
+    assert np.array_equal(got, two)
+    want = pooled(orc.mex_fwd(x, off, n, **kw), *pool)
+    assert rel_err(got, want, floor=np.ones_like(want)) <= MEX_TOL
+
+
 def test_sum_pooling(pkg):
     g = np.random.default_rng(16)
     x = g.normal(size=(3, 5, 9, 8)).astype(np.float32)
