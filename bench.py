@@ -203,6 +203,19 @@ def main():
                                    "exp_frac": round(gmac4 / (ms * 1e-3) / EXP_RATE, 4), "batch": 512,
                                    "kernels": "similarity + 4 x (offset pack + mex + sum pool) + wave-per-pixel mex",
                                    "hip_graph_replay_ms": round(ms_graph, 4), "hip_graph_matches_eager": graph_ok}
+        # the same stack with every MEX + pooling pair as one call (a fused kernel for this geometry)
+        def fused_stack():
+            cur = pkg.similarity(X4, T4, W4, **kw4)
+            for off, n, kw in layers:
+                cur = pkg.mex_sum_pool(cur, off, n, (2, 2), normalize_offsets=True, **kw)
+            return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
+                           strides=[ch, 1, 1], shared_offset_region=[1])
+
+        _, ms_fused = timed(fused_stack, args.steps, args.warmup)
+        ref4 = stack()
+        dev4 = float((fused_stack() - ref4).abs().max() / ref4.abs().max())
+        others["config4_stack"].update({"fused_pool_kernel_ms": round(ms_fused, 4),
+                                        "fused_pool_max_dev_of_scale": dev4})
         # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
         _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,

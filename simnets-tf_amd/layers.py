@@ -77,6 +77,21 @@ def mex(input, offsets, num_instances, **attrs):
     return MexFunction.apply(input, offsets, num_instances, attrs)
 
 
+def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), **attrs):
+    """`mex` followed by non-overlapping sum pooling (the MEX layer + pooling pair of the reference's networks,
+    README.md:108-129).  Without gradients the pair is one call of the library (a fused kernel when the offsets are
+    unshared over exactly the pooling window); when a gradient is needed the two steps stay separate, because the
+    MEX gradients take the unpooled output."""
+    unknown = set(attrs) - set(_MEX_KEYS)
+    if unknown:
+        raise TypeError("unknown Mex attributes: %s" % sorted(unknown))
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    if torch.is_grad_enabled() and (input.requires_grad or offsets.requires_grad):
+        y = MexFunction.apply(input, offsets, num_instances, attrs)
+        return torch.nn.functional.avg_pool2d(y, (ph, pw)) * float(ph * pw)
+    return ops.mex_sum_pool(input, offsets, num_instances, (ph, pw), **attrs)
+
+
 def dirichlet_init(shape, alpha=1.0, generator=None):
     """log of Dirichlet(alpha) samples over the block volume, one per (region, instance):
     DirichletInit of python/simnets/keras.py:91-109."""

@@ -182,3 +182,20 @@ def test_missing_data_stack_replays_from_a_hip_graph(pkg):
         want = stack(torch.from_numpy(fresh).cuda())     # eager work between the replays
         torch.cuda.synchronize()
         assert torch.equal(got, want), "replay %d" % trial
+
+
+def test_mex_sum_pool_functional_fused_without_gradients_split_with(pkg):
+    g = np.random.default_rng(31)
+    x = torch.from_numpy(g.normal(size=(3, 16, 8, 8)).astype(np.float32)).cuda()
+    off = torch.from_numpy((g.normal(size=(4, 12, 16, 1, 1)) * 0.2).astype(np.float32)).cuda()
+    kw = dict(blocks=[16, 1, 1], strides=[16, 1, 1], unshared_offset_region=[1, 2, 2], softmax_mode=True)
+    with torch.no_grad():
+        fused = pkg.layers.mex_sum_pool(x, off, 12, (2, 2), **kw)
+    off.requires_grad_()
+    split = pkg.layers.mex_sum_pool(x, off, 12, (2, 2), **kw)
+    assert split.requires_grad and fused.shape == split.shape == (3, 12, 4, 4)
+    assert float((fused - split).abs().max()) <= 1e-5 * float(split.abs().max())
+    split.sum().backward()
+    y = pkg.mex(x, off.detach(), 12, **kw)
+    want = pkg.mex_offsets_grad(x, off.detach(), y, torch.ones_like(y), 12, **kw)
+    assert torch.allclose(off.grad, want, rtol=1e-5, atol=1e-6)
