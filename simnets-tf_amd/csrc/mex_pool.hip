@@ -28,38 +28,44 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 constexpr int KC = 32;             // k per LDS chunk
 constexpr int TM = 64, MX = 16;    // instances per workgroup / per wave
 constexpr int KSTEP = 4, U = KC / KSTEP;
-constexpr int XP = 64;             // pixel columns of a workgroup: 4 tiles of 16
 
 struct PoolArgs {
     float *pooled;
     int Hp, Wp;   // pooled height and width
-    int spw;      // slots per workgroup: 64 / R
+    int spw;      // slots per workgroup: NH * 64 / R
 };
 
-template <int R, bool CHECK>
-__global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, const PoolArgs q)
+// NH = column halves of a workgroup (64 pixel columns = 4 tiles of 16 each), 4 instance waves per half: two halves
+// share the offsets tiles and double the waves per SIMD the LDS budget allows, which is what hides the latencies of
+// the short dependent phases; one half only when there are no slots for a second one.
+template <int R, int NH, bool CHECK>
+__global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs a, const PoolArgs q)
 {
-    constexpr int G = 4 / R;       // slot groups of 16 per workgroup
+    constexpr int XP = 64 * NH;         // pixel columns of a workgroup
+    constexpr int kThreads = 256 * NH;
+    constexpr int G = 4 / R;       // slot groups of 16 per column half
     __shared__ __attribute__((aligned(16))) float xs[KC * XP];       // [k][column]
     __shared__ __attribute__((aligned(16))) float os[R * KC * TM];   // [region][k][instance]
     __shared__ float pmx[KSTEP * XP];   // partial column maxima
     __shared__ float fsh[XP], msh[XP];  // per column: rescale factor of this chunk, running maximum
-    __shared__ long long ppos[16 * G];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
+    __shared__ long long ppos[16 * G * NH];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wm = __builtin_amdgcn_readfirstlane(tid >> 6);  // instance wave; also the k phase when staging
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 3, wh = wave >> 2;      // computing: instance group and column half of this wave
+    const int sk = wave / NH, sh = wave % NH;     // staging: k phase and column half of this wave
     const int chunk = blockIdx.x, mgroup = blockIdx.y;
     const int m0 = mgroup * TM + wm * MX;
     const bool wave_active = m0 < a.M;
 
     // staging role: column of tile (slot group, region), consecutive threads = neighbouring pixels of a window row
     const int sreg = lane % R, ssl = lane / R;
-    const int col = ((ssl >> 4) * R + sreg) * 16 + (ssl & 15);
-    const PixelRef gp = locate(a, sreg, chunk * (16 * G) + ssl);
+    const int col = sh * 64 + ((ssl >> 4) * R + sreg) * 16 + (ssl & 15);
+    const PixelRef gp = locate(a, sreg, (chunk * NH + sh) * (16 * G) + ssl);
 
-    if (tid < 16 * G) {
-        const int slot = chunk * (16 * G) + tid;
+    if (tid < 16 * G * NH) {
+        const int slot = chunk * (16 * G * NH) + tid;
         long long pos = -1;
         if (slot < a.slots) {
             const int b = (int)fast_div((unsigned)slot, a.dRS);
@@ -91,7 +97,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
         float v[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int kk = wm + u * KSTEP;
+            const int kk = sk + u * KSTEP;
             const int4 ke = a.ktab[k0 + (full ? kk : min(kk, kc - 1))];  // same for the whole wave: scalar load
             if (CHECK) {
                 const int ci = gp.ci0 + ke.y, hi = gp.hi0 + ke.z, wi = gp.wi0 + ke.w;
@@ -108,7 +114,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
             const float4 *src = reinterpret_cast<const float4 *>(
                 (prod ? a.offe : a.offp) + (((size_t)r * a.n_mgroups + mgroup) * a.K + k0) * TM);
             float4 *dst = reinterpret_cast<float4 *>(os + r * KC * TM);
-            for (int i = tid; i < on; i += 256)
+            for (int i = tid; i < on; i += kThreads)
                 dst[i] = src[i];
         }
 #pragma unroll
@@ -117,17 +123,17 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
         if (!prod) {
 #pragma unroll
             for (int u = 0; u < U; ++u)
-                if (full || wm + u * KSTEP < kc)
-                    xs[(wm + u * KSTEP) * XP + col] = v[u];
+                if (full || sk + u * KSTEP < kc)
+                    xs[(sk + u * KSTEP) * XP + col] = v[u];
             return;
         }
         // column maximum over the chunk -> running maximum; the staged values become exp2(x - maximum)
         float pm = -INFINITY;
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (full || wm + u * KSTEP < kc)
+            if (full || sk + u * KSTEP < kc)
                 pm = fmaxf(pm, v[u]);
-        pmx[wm * XP + col] = pm;
+        pmx[sk * XP + col] = pm;
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < KSTEP; ++j)
@@ -136,9 +142,9 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
         const float m_sub = m_new == -INFINITY ? 0.0f : m_new;  // nothing finite yet: the terms are exp2(-inf) = 0
 #pragma unroll
         for (int u = 0; u < U; ++u)
-            if (full || wm + u * KSTEP < kc)
-                xs[(wm + u * KSTEP) * XP + col] = __builtin_amdgcn_exp2f(v[u] - m_sub);
-        if (wm == 0) {
+            if (full || sk + u * KSTEP < kc)
+                xs[(sk + u * KSTEP) * XP + col] = __builtin_amdgcn_exp2f(v[u] - m_sub);
+        if (sk == 0) {
             fsh[col] = m_run == m_new ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
             msh[col] = m_new;
         }
@@ -146,9 +152,9 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
         if (!full) {
             // the matrix instruction takes 4 k at a time: rows kc .. next multiple of 4 are zeros
             const int kc4 = (kc + 3) & ~3;
-            for (int i = tid; i < (kc4 - kc) * XP; i += 256)
+            for (int i = tid; i < (kc4 - kc) * XP; i += kThreads)
                 xs[kc * XP + i] = 0.0f;
-            for (int i = tid; i < (kc4 - kc) * TM * R; i += 256)
+            for (int i = tid; i < (kc4 - kc) * TM * R; i += kThreads)
                 os[(i / ((kc4 - kc) * TM)) * KC * TM + kc * TM + i % ((kc4 - kc) * TM)] = 0.0f;
         }
     };
@@ -164,7 +170,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
 #pragma unroll
         for (int t = 0; t < 4; ++t)
             acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-        const float *xa = xs + lq * XP + lr;
+        const float *xa = xs + lq * XP + wh * 64 + lr;
         const float *oa = os + lq * TM + wm * MX + lr;
         for (int k0 = 0; k0 < a.K; k0 += KC) {
             const int kc = min(KC, a.K - k0);
@@ -176,7 +182,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
             if (k0 > 0) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t)
-                    acc[t] *= fsh[t * 16 + lr];
+                    acc[t] *= fsh[wh * 64 + t * 16 + lr];
             }
             const int kend = (kc + 3) & ~3;
             for (int kq = 0; kq < kend; kq += 4) {
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const float *omax = a.omax + ((size_t)(t % R) * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
-            const float mp = msh[t * 16 + lr];
+            const float mp = msh[wh * 64 + t * 16 + lr];
             // an infinite column bound makes the result NaN, as the reference's exp(inf - inf) does
             const float mpt = (mp - mp) + mp + a.c0;
 #pragma unroll
@@ -225,7 +231,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
             for (int t = 0; t < 4; ++t)
 #pragma unroll
                 for (int v = 0; v < 4; ++v) {
-                    const float *xc = xs + t * 16 + lr;
+                    const float *xc = xs + wh * 64 + t * 16 + lr;
                     const float *oc = os + (t % R) * KC * TM + wm * MX + 4 * lq + v;
                     float cb = -INFINITY;
                     for (int kk = 0; kk < kc; ++kk)
@@ -253,7 +259,7 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
     // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
 #pragma unroll
     for (int g = 0; g < G; ++g) {
-        const long long pos = ppos[g * 16 + lr];  // written before the first barrier
+        const long long pos = ppos[(wh * G + g) * 16 + lr];  // written before the first barrier
         if (pos < 0)
             continue;
         float *o = q.pooled + pos + row0;
@@ -269,13 +275,13 @@ __global__ __launch_bounds__(256) void mex_pool_kernel(const MexKernelArgs a, co
     }
 }
 
-template <int R>
+template <int R, int NH>
 hipError_t launch_pool(const MexKernelArgs &a, const PoolArgs &q, dim3 grid, bool inside, hipStream_t s)
 {
     if (inside)
-        hipLaunchKernelGGL((mex_pool_kernel<R, false>), grid, dim3(256), 0, s, a, q);
+        hipLaunchKernelGGL((mex_pool_kernel<R, NH, false>), grid, dim3(256 * NH), 0, s, a, q);
     else
-        hipLaunchKernelGGL((mex_pool_kernel<R, true>), grid, dim3(256), 0, s, a, q);
+        hipLaunchKernelGGL((mex_pool_kernel<R, NH, true>), grid, dim3(256 * NH), 0, s, a, q);
     return hipGetLastError();
 }
 
@@ -322,7 +328,10 @@ int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const 
     q.pooled = pooled;
     q.Hp = d.height_out / ph;
     q.Wp = d.width_out / pw;
-    q.spw = 64 / (ph * pw);
+    // two column halves per workgroup whenever there are slots for both: the extra waves per compute unit pay even
+    // when the launch then has fewer workgroups than compute units (measured on 512 images of 2x2 pixels)
+    const int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
+    q.spw = nh * 64 / (ph * pw);
     const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
     if (gx > 0x7fffffffLL || n_mgroups > 65535)
         return SIMNETS_ERR_TOO_LARGE;
@@ -332,7 +341,11 @@ int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const 
                         (d.width_out - 1) * d.stride_w + d.block_w <= p.W;
     dim3 grid((unsigned)gx, (unsigned)n_mgroups);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const hipError_t e = ph * pw == 4 ? launch_pool<4>(a, q, grid, inside, s) : launch_pool<2>(a, q, grid, inside, s);
+    hipError_t e;
+    if (ph * pw == 4)
+        e = nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s);
+    else
+        e = nh == 2 ? launch_pool<2, 2>(a, q, grid, inside, s) : launch_pool<2, 1>(a, q, grid, inside, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

@@ -296,6 +296,9 @@ def pooled(y, ph, pw):
     dict(im=(4, 8, 6, 10), n=33, pool=(1, 2)),                         # two-pixel windows
     dict(im=(4, 8, 10, 6), n=33, pool=(2, 1)),
     dict(im=(3, 5, 12, 12), n=24, pool=(2, 2), blocks=[5, 3, 3], padding=[0, 1, 1]),   # spatial blocks, padding
+    dict(im=(40, 16, 32, 32), n=20, pool=(2, 2)),                      # enough windows for the two-half workgroups
+    dict(im=(36, 8, 16, 32), n=70, pool=(1, 2)),
+    dict(im=(33, 7, 31, 33), n=20, pool=(2, 2), blocks=[7, 3, 3], padding=[0, 1, 1]),  # the same with ragged edges
     dict(im=(3, 6, 12, 12), n=24, pool=(2, 2), blocks=[2, 1, 1], strides=[2, 1, 1]),   # several output channels
 ])
 @pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("wide", 1.0), ("mixed", 3.0)])
