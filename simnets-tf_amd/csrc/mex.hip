@@ -480,7 +480,9 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
 // One wave per (region, instance) row of the offsets: optional logsumexp normalisation
 // (python/simnets/keras.py:155-160) and the scaling, then the row is scattered into the k-major packed layout
 // [r][mgroup][k][tm]; for finite epsilon also its exponentials relative to the row maximum, the maximum and the
-// row's range (what the product form of the forward kernel reads).
+// row's range (what the product form of the forward kernel reads).  KL > 0: the row (K <= 64 * KL) is read once and
+// kept in registers for the three reductions and the scatter; KL = 0: every pass reads it again.
+template <int KL>
 __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__restrict__ offsets, int R, int M, int K,
                                                               int n_mgroups, int tm, int normalize, float scale,
                                                               int finite_eps, float *__restrict__ offp,
@@ -523,42 +525,56 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         return;
     }
     const float *src = offsets + ((size_t)r * M + m) * K;
+    float rv[KL > 0 ? KL : 1];
+    if (KL > 0) {
+#pragma unroll
+        for (int j = 0; j < KL; ++j)
+            rv[j] = src[min(lane + 64 * j, K - 1)];
+    }
+    auto each = [&](auto &&f) __attribute__((always_inline)) {
+        if constexpr (KL > 0) {
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                if (lane + 64 * j < K)
+                    f(lane + 64 * j, rv[j]);
+        } else {
+            for (int k = lane; k < K; k += 64)
+                f(k, src[k]);
+        }
+    };
     float lse = 0.0f;
     if (normalize) {
         float mxv = -INFINITY;
-        for (int k = lane; k < K; k += 64)
-            mxv = fmaxf(mxv, src[k]);
+        each([&](int, float x) { mxv = fmaxf(mxv, x); });
         for (int d = 32; d > 0; d >>= 1)
             mxv = fmaxf(mxv, __shfl_xor(mxv, d, 64));
         if (!(fabsf(mxv) < INFINITY))
             mxv = 0.0f;
         float sum = 0.0f;
-        for (int k = lane; k < K; k += 64)
-            sum += expf(src[k] - mxv);
+        each([&](int, float x) { sum += expf(x - mxv); });
         for (int d = 32; d > 0; d >>= 1)
             sum += __shfl_xor(sum, d, 64);
         lse = logf(sum) + mxv;
     }
     if (!finite_eps) {
-        for (int k = lane; k < K; k += 64)
-            dst[(size_t)k * tm] = (src[k] - lse) * scale;
+        each([&](int k, float x) { dst[(size_t)k * tm] = (x - lse) * scale; });
         return;
     }
     float hi = -INFINITY, lo = INFINITY;
-    for (int k = lane; k < K; k += 64) {
-        const float v = (src[k] - lse) * scale;
+    each([&](int, float x) {
+        const float v = (x - lse) * scale;
         hi = fmaxf(hi, v);
         lo = fminf(lo, v);
-    }
+    });
     for (int d = 32; d > 0; d >>= 1) {
         hi = fmaxf(hi, __shfl_xor(hi, d, 64));
         lo = fminf(lo, __shfl_xor(lo, d, 64));
     }
-    for (int k = lane; k < K; k += 64) {
-        const float v = (src[k] - lse) * scale;
+    each([&](int k, float x) {
+        const float v = (x - lse) * scale;
         dst[(size_t)k * tm] = v;
         dste[(size_t)k * tm] = __builtin_amdgcn_exp2f(v - hi);
-    }
+    });
     if (lane == 0) {
         omax[row] = hi;
         orng[row] = hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
@@ -646,15 +662,27 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, c
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
     const int m_end = min(a.M, (int)(blockIdx.y + 1) * kSmallMChunk);
-    for (int m0 = blockIdx.y * kSmallMChunk; m0 < m_end; m0 += MG) {
-        float o[MG][KL];
+    // the offsets rows of the next four instances are requested while the current four are reduced
+    float on[MG][KL];
+    auto fetch_rows = [&](int m0) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < MG; ++g) {
             const float *row = offsets + ((size_t)r * a.M + min(m0 + g, a.M - 1)) * a.K;
 #pragma unroll
             for (int j = 0; j < KL; ++j)
-                o[g][j] = kv[j] ? row[lane + 64 * j] : 0.0f;
+                on[g][j] = row[kv[j] ? lane + 64 * j : 0];
         }
+    };
+    fetch_rows(blockIdx.y * kSmallMChunk);
+    for (int m0 = blockIdx.y * kSmallMChunk; m0 < m_end; m0 += MG) {
+        float o[MG][KL];
+#pragma unroll
+        for (int g = 0; g < MG; ++g)
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                o[g][j] = kv[j] ? on[g][j] : 0.0f;
+        if (m0 + MG < m_end)
+            fetch_rows(m0 + MG);
         if (normalize) {
             float mx[MG], sum[MG];
 #pragma unroll
@@ -800,10 +828,21 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
     int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
     if ((long long)d.block_c * p.H * p.W > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;  // the table holds 32-bit offsets
-    hipLaunchKernelGGL(mex_pack_offsets_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       reinterpret_cast<hipStream_t>(stream), offsets, d.num_regions, d.M, d.K, n_mgroups, tm,
-                       p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W, d.block_h,
-                       d.block_w);
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
+#define SIMNETS_PACK_LAUNCH(KL)                                                                                        \
+    hipLaunchKernelGGL(mex_pack_offsets_kernel<KL>, grid, dim3(256), 0, hs, offsets, d.num_regions, d.M, d.K, n_mgroups, \
+                       tm, p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W,         \
+                       d.block_h, d.block_w)
+    if (d.K <= 64)
+        SIMNETS_PACK_LAUNCH(1);
+    else if (d.K <= 256)
+        SIMNETS_PACK_LAUNCH(4);
+    else if (d.K <= 1024)
+        SIMNETS_PACK_LAUNCH(16);
+    else
+        SIMNETS_PACK_LAUNCH(0);
+#undef SIMNETS_PACK_LAUNCH
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
     a->offp = offp; a->offe = offe; a->omax = omax; a->orng = orng; a->ktab = ktab;
