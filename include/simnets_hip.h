@@ -65,9 +65,12 @@ enum { SIMNETS_SIM_L1 = 0, SIMNETS_SIM_L2 = 1 };
 
 /* How the weighted distance is evaluated.  All choices implement the same operator. */
 enum {
-    SIMNETS_ALGO_AUTO = 0,   /* == DIRECT */
+    SIMNETS_ALGO_AUTO = 0,   /* SQRTW for plain L2 (no normalization term), DIRECT for every other mode */
     SIMNETS_ALGO_DIRECT = 1, /* d = t - x; acc += (-w*d)*d   (L1: acc += -w*|d|), NaN-capable, every mode */
-    SIMNETS_ALGO_SQRTW = 2,  /* plain L2 only: d = sqrt(w)*t - sqrt(w)*x in one fma; acc += -d*d */
+    SIMNETS_ALGO_SQRTW = 2,  /* plain L2 only: d = sqrt(w)*t - sqrt(w)*x in one fma; acc += -d*d.  Outputs closer to
+                                zero than sum_k w t^2 / 1024 (where the different rounding of d could exceed 4e-6
+                                relative), and all outputs of a template with a negative or NaN weight, are then
+                                recomputed with DIRECT's arithmetic, so the result stays within the tolerance */
     SIMNETS_ALGO_MFMA = 3    /* plain L2 only, inputs free of NaN/Inf: sum w x^2 - 2 sum (w t) x + sum w t^2
                                 as dense fp32 matrix-core contractions */
 };

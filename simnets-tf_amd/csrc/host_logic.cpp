@@ -87,6 +87,9 @@ int sim_make_plan(const simnets_similarity_attrs *a, const int in[4], const int 
     p->norm_const_every_iteration = a->norm_const_every_iteration != 0;
     switch (a->algo) {
     case SIMNETS_ALGO_AUTO:
+        // plain L2: the two-instruction sqrt-weight form, with its small outputs recomputed exactly
+        p->algo = p->mode == SIM_MODE_L2 ? SIMNETS_ALGO_SQRTW : SIMNETS_ALGO_DIRECT;
+        break;
     case SIMNETS_ALGO_DIRECT:
         p->algo = SIMNETS_ALGO_DIRECT;
         break;

@@ -61,7 +61,40 @@ struct SimKernelArgs {
     int norm_every_iteration;
     int vec_store;     // output rows are 16-byte aligned: store float4
     int fast_stage;    // the channel tile has at most kStagePos * kThreads elements: division-free staging
+    // sqrt-weight form only (see sim_guard_fix_kernel)
+    const float *templates, *weights;  // the caller's arrays [O][K]
+    const float *thr;  // [O] outputs of template m above -thr[m] are recomputed exactly
+    int *flags;        // [workgroups * kWaves] set by a wave that wrote such an output
 };
+
+// Output positions of a lane: the mapping shared by sim_direct_kernel and sim_guard_fix_kernel.
+struct LanePos {
+    int b, tile, ws, mtile;
+    int g_first, g_last, row_first;
+    int h, gw;
+    bool wave_active, lane_valid;
+};
+
+__device__ __forceinline__ LanePos lane_pos(const SimKernelArgs &a, int wave, int lane)
+{
+    LanePos q;
+    q.b = blockIdx.x / a.tiles;
+    q.tile = blockIdx.x - q.b * a.tiles;
+    q.ws = wave & (a.nws - 1);                   // which 64 pixel groups of the tile
+    const int wm = wave >> a.nws_log2;           // which MT templates
+    const int nwm = kWaves >> a.nws_log2;
+    q.mtile = blockIdx.y * nwm + wm;
+    q.wave_active = q.mtile < a.n_mtiles;
+    q.g_first = q.tile * 64 * a.nws;
+    q.g_last = min(q.g_first + 64 * a.nws, a.gpi) - 1;
+    q.row_first = q.g_first / a.G;
+    int g = q.g_first + q.ws * 64 + lane;
+    q.lane_valid = g <= q.g_last;
+    g = min(g, q.g_last);
+    q.h = g / a.G;
+    q.gw = g - q.h * a.G;
+    return q;
+}
 
 // Wave-uniform parameter fetch of the gather fallback: the address is the same in every lane, so these
 // become scalar loads (s_load_dwordx8/x16) and the values live in SGPRs.
@@ -167,27 +200,15 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int sw = SWT > 0 ? SWT : a.sw;
 
-    const int b = blockIdx.x / a.tiles;
-    const int tile = blockIdx.x - b * a.tiles;
-    const int ws = wave & (a.nws - 1);            // which 64 pixel groups of the tile
-    const int wm = wave >> a.nws_log2;            // which MT templates
-    const int nwm = kWaves >> a.nws_log2;
-    const int mtile = blockIdx.y * nwm + wm;
-    const bool wave_active = mtile < a.n_mtiles;
+    const LanePos lp = lane_pos(a, wave, lane);
+    const int b = lp.b, mtile = lp.mtile, h = lp.h, gw = lp.gw;
+    const bool wave_active = lp.wave_active, lane_valid = lp.lane_valid;
 
     // pixel groups of this workgroup and the input rows they need
-    const int g_first = tile * 64 * a.nws;
-    const int g_last = min(g_first + 64 * a.nws, a.gpi) - 1;
-    const int row_first = g_first / a.G;
-    const int nrows = g_last / a.G - row_first + 1;
+    const int row_first = lp.row_first;
+    const int nrows = lp.g_last / a.G - row_first + 1;
     const int TR = (nrows - 1) * a.sh + a.bh;
     const int in_row0 = row_first * a.sh - a.ph;
-
-    int g = g_first + ws * 64 + lane;
-    const bool lane_valid = g <= g_last;
-    g = min(g, g_last);
-    const int h = g / a.G;
-    const int gw = g - h * a.G;
     const int lds_base = (h - row_first) * a.sh * a.TC + gw * PT * sw;
 
     float acc[MT][PT];
@@ -299,6 +320,7 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     if (MODE == SIM_MODE_L2_NORM)
         reps = a.norm_every_iteration ? (a.B - b) : 1;
     const int w0 = gw * PT;
+    bool suspect = false;  // sqrt-weight form: an output so close to zero that its rounding error may show
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int mm = mtile * MT + m;
@@ -310,6 +332,12 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
             v[p] = acc[m][p];
             for (int r = 0; r < reps; ++r)
                 v[p] += a.norm_const;
+        }
+        if (MODE == SIM_MODE_L2_SQRTW) {
+            const float thr = a.thr[mm];
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                suspect |= w0 + p < a.ow && !(-v[p] >= thr);  // (also catches NaN)
         }
         float *o = a.out + (((size_t)b * a.O + mm) * a.oh + h) * a.ow + w0;
         if (a.vec_store && PT % 4 == 0) {
@@ -323,6 +351,79 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
                 if (w0 + p < a.ow)
                     o[p] = v[p];
         }
+    }
+    if (MODE == SIM_MODE_L2_SQRTW && suspect)
+        a.flags[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + wave] = 1;
+}
+
+// Second pass of the sqrt-weight form (plain L2 evaluated as -(sqrt(w) t - sqrt(w) x)^2: 2 instead of 3 VALU
+// instructions per term).  Its rounding differs from the reference's w (t - x)^2 only inside d = sqrt(w)(t - x):
+// |err(d)| <= eps (|sqrt(w) t| + |d|), so by Cauchy-Schwarz the relative error of an output `out` of template m is
+// at most 2 eps sqrt(T_m / out) + O(eps) with T_m = sum_k w t^2: below 4e-6 unless out < T_m / 1024.  The main
+// kernel flags the waves that wrote such an output (exact matches of a patch and a template, in practice); this
+// kernel, launched with the same grid, returns at once for the others and recomputes the flagged waves' small
+// outputs with the reference's arithmetic (d = t - x; acc = fma(-w d, d, acc), k ascending: bit-identical to the
+// direct kernel).  thr[m] = T_m / 1024, or +inf for a template with a negative or NaN weight (sqrt undefined):
+// all outputs of such a template are recomputed.
+template <int PT, int MT>
+__global__ __launch_bounds__(kThreads) void sim_guard_fix_kernel(const SimKernelArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    if (a.flags[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + wave] == 0)
+        return;
+    const LanePos lp = lane_pos(a, wave, lane);
+    if (!lp.wave_active || !lp.lane_valid)
+        return;
+    const int w0 = lp.gw * PT, bhw = a.bh * a.bw;
+    const float *img = a.in + (size_t)lp.b * a.C * a.H * a.W;
+    for (int m = 0; m < MT; ++m) {
+        const int mm = lp.mtile * MT + m;
+        if (mm >= a.O)
+            break;
+        const float thr = a.thr[mm];
+        const float *tp = a.templates + (size_t)mm * a.K, *wp = a.weights + (size_t)mm * a.K;
+        float *o = a.out + (((size_t)lp.b * a.O + mm) * a.oh + lp.h) * a.ow + w0;
+        for (int p = 0; p < PT && w0 + p < a.ow; ++p) {
+            if (-o[p] >= thr)
+                continue;
+            const int hi0 = lp.h * a.sh - a.ph, wi0 = (w0 + p) * a.sw - a.pw;
+            float acc = 0.0f;
+            for (int k = 0; k < a.K; ++k) {
+                const int c = k / bhw, rem = k - c * bhw;
+                const int hi = hi0 + rem / a.bw, wi = wi0 + rem % a.bw;
+                const bool inside = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                const float x = inside ? img[((size_t)c * a.H + hi) * a.W + wi] : a.oob;
+                const float d = tp[k] - x;
+                acc = __builtin_fmaf(-wp[k] * d, d, acc);
+            }
+            o[p] = acc;
+        }
+    }
+}
+
+// Thresholds of the sqrt-weight form (one wave per template) and the cleared flags.
+__global__ __launch_bounds__(256) void sim_guard_prep_kernel(const float *__restrict__ templates,
+                                                            const float *__restrict__ weights, int O, int K,
+                                                            float *__restrict__ thr, int *__restrict__ flags,
+                                                            long long n_flags)
+{
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n_flags; i += (long long)gridDim.x * 256)
+        flags[i] = 0;
+    const int lane = threadIdx.x & 63;
+    for (int m = blockIdx.x * 4 + (threadIdx.x >> 6); m < O; m += gridDim.x * 4) {
+        float t2 = 0.0f;
+        bool bad = false;
+        for (int k = lane; k < K; k += 64) {
+            const float t = templates[(size_t)m * K + k], w = weights[(size_t)m * K + k];
+            t2 = __builtin_fmaf(w * t, t, t2);
+            bad |= !(w >= 0.0f);
+        }
+        for (int d = 32; d > 0; d >>= 1)
+            t2 += __shfl_xor(t2, d, 64);
+        const bool any_bad = __any(bad);
+        if (lane == 0)
+            thr[m] = (any_bad || !(t2 >= 0.0f)) ? INFINITY : t2 * (1.0f / 1024.0f);
     }
 }
 
@@ -533,6 +634,22 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
     return launch_direct<MODE, kSmallPT, kSmallMT>(a, grid, lds_bytes, s);
 }
 
+// the sqrt-weight form runs on the tiled kernel only; its thresholds [O] and wave flags
+bool use_sqrtw(const SimPlan &p, const Tiling &t) { return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok; }
+
+long long guard_flags(const SimPlan &p, const Tiling &t)
+{
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT, nwm = kWaves / t.nws;
+    return (long long)p.B * t.tiles * ((n_mtiles + nwm - 1) / nwm) * kWaves;
+}
+
+size_t guard_bytes(const SimPlan &p, const Tiling &t)
+{
+    if (!use_sqrtw(p, t))
+        return 0;
+    return align_up((size_t)p.O * sizeof(float), 256) + align_up((size_t)guard_flags(p, t) * sizeof(int), 256);
+}
+
 }  // namespace
 
 size_t sim_direct_workspace_bytes(const SimPlan &p)
@@ -543,7 +660,7 @@ size_t sim_direct_workspace_bytes(const SimPlan &p)
     const size_t pa = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
     const size_t pc = align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
     const size_t koff = align_up(((size_t)p.K + 2) * sizeof(int), 256);
-    return pa + pc + koff;
+    return pa + pc + koff + guard_bytes(p, t);
 }
 
 int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
@@ -561,7 +678,19 @@ int sim_direct_launch(const SimPlan &p, const float *input, const float *templat
 
     const long long total = (long long)n_mtiles * p.K * t.MT;
     const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
-    const int mode = (p.algo == SIMNETS_ALGO_SQRTW) ? (int)SIM_MODE_L2_SQRTW : p.mode;
+    const bool sqrtw = use_sqrtw(p, t);
+    const int mode = sqrtw ? (int)SIM_MODE_L2_SQRTW : p.mode;
+    const size_t koff_bytes = align_up(((size_t)p.K + 2) * sizeof(int), 256);
+    float *thr = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + pa_bytes + pc_bytes + koff_bytes);
+    int *flags = reinterpret_cast<int *>(reinterpret_cast<char *>(thr) + align_up((size_t)p.O * sizeof(float), 256));
+    if (sqrtw) {
+        const long long n_flags = guard_flags(p, t);
+        const int blocks = (int)std::min<long long>(std::max<long long>((p.O + 3) / 4, (n_flags + 255) / 256), 1024);
+        hipLaunchKernelGGL(sim_guard_prep_kernel, dim3(blocks), dim3(256), 0, s, templates, weights, p.O, p.K, thr,
+                           flags, n_flags);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+    }
     hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights, p.O, p.K, t.MT,
                        n_mtiles, mode, p.fudge, pa, pc, koff, p.bh * p.bw, p.bw, t.CC, t.TRmax * t.TC, t.TC);
     if (hipGetLastError() != hipSuccess)
@@ -579,6 +708,7 @@ int sim_direct_launch(const SimPlan &p, const float *input, const float *templat
     // Dtype(-0.5) * Dtype(K_) * std::log(2.0 * M_PI), rounded to float by Eigen's constant()
     a.norm_const = (p.mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)p.K) * std::log(2.0 * M_PI)) : 0.0f;
     a.norm_every_iteration = p.norm_const_every_iteration;
+    a.templates = templates; a.weights = weights; a.thr = thr; a.flags = flags;
 
     hipError_t e;
     switch (mode) {
@@ -587,6 +717,16 @@ int sim_direct_launch(const SimPlan &p, const float *input, const float *templat
     case SIM_MODE_L2_NORM: e = launch_mode<SIM_MODE_L2_NORM>(a, t, s); break;
     case SIM_MODE_L2_NORM_IGNORE_NAN: e = launch_mode<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, s); break;
     default: e = launch_mode<SIM_MODE_L2_SQRTW>(a, t, s); break;
+    }
+    if (e == hipSuccess && sqrtw) {
+        // same grid as the main kernel: a wave looks at its flag and, almost always, returns
+        const int nwm = kWaves / a.nws;
+        dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
+        if (t.PT == kBigPT && t.MT == kBigMT)
+            hipLaunchKernelGGL((sim_guard_fix_kernel<kBigPT, kBigMT>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((sim_guard_fix_kernel<kSmallPT, kSmallMT>), grid, dim3(kThreads), 0, s, a);
+        e = hipGetLastError();
     }
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }

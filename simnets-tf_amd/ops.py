@@ -101,7 +101,7 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
     """Similarity forward; arguments as python/simnets/ops/similarity.py:48-121.
 
     input [B,C,H,W], templates/weights [O,C,bh,bw] (weights non-negative) -> [B,O,oh,ow].
-    Extensions: `algo` in {None,'direct','sqrtw','mfma'}, `norm_const_every_iteration`, `out`.
+    Extensions: `algo` in {None,'direct','sqrtw','mfma'} (None: 'sqrtw' for plain L2, else 'direct'), `norm_const_every_iteration`, `out`.
     """
     x = _require_cuda_f32("input", input)
     t = _require_cuda_f32("templates", templates)

@@ -122,6 +122,60 @@ def test_similarity_sqrtw_algorithm_matches_direct(pkg):
     assert rel_err(run_similarity(pkg, x, t, w, algo="sqrtw", **kw), want) <= SIM_TOL
 
 
+# Plain L2 runs the sqrt-weight form by default: -(sqrt(w) t - sqrt(w) x)^2 rounds differently from the reference's
+# -w (t - x)^2 where a patch (nearly) equals a template, so outputs near zero are recomputed with the reference's
+# arithmetic.  These cases put outputs exactly at, and close to, zero.
+@pytest.mark.parametrize("geom", [
+    dict(shape=(3, 6, 40, 40), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # 16 x 8 lane tiles
+    dict(shape=(2, 5, 17, 13), O=19, blocks=[3, 2], strides=[2, 1], padding=[0, 1]),     # 4 x 8 lane tiles, ragged
+    dict(shape=(2, 3, 9, 50), O=9, blocks=[2, 2], strides=[1, 2], padding=[1, 0], out_of_bounds_value=0.75),
+])
+@pytest.mark.parametrize("kind", ["exact", "near", "negative_weights", "nan_input", "all_zero"])
+def test_similarity_l2_default_form_recomputes_outputs_near_zero(pkg, geom, kind):
+    g = np.random.default_rng(41)
+    shape, O, blocks = geom["shape"], geom["O"], geom["blocks"]
+    kw = {k: v for k, v in geom.items() if k not in ("shape", "O")}
+    x = (g.normal(size=shape) * 3 + 50).astype(np.float32)          # |t| >> |t - x|: the rounding of d matters
+    t = (g.normal(size=(O, shape[1]) + tuple(blocks)) * 3 + 50).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    hits = []
+    if kind in ("exact", "near"):
+        # templates cut out of the (padded) input: their outputs at those positions are exactly 0
+        ph, pw = geom["padding"]
+        xp = np.full((shape[0], shape[1], shape[2] + 2 * ph, shape[3] + 2 * pw), geom.get("out_of_bounds_value", 0.0),
+                     np.float32)
+        xp[:, :, ph:ph + shape[2], pw:pw + shape[3]] = x
+        oh = (shape[2] + 2 * ph - blocks[0]) // geom["strides"][0] + 1
+        ow = (shape[3] + 2 * pw - blocks[1]) // geom["strides"][1] + 1
+        for m in range(0, O, 2):
+            b, i, j = int(g.integers(shape[0])), int(g.integers(oh)), int(g.integers(ow))
+            i0, j0 = i * geom["strides"][0], j * geom["strides"][1]
+            t[m] = xp[b, :, i0:i0 + blocks[0], j0:j0 + blocks[1]]
+            hits.append((b, m, i, j))
+        if kind == "near":
+            t += (g.normal(size=t.shape) * 1e-4).astype(np.float32)
+    elif kind == "negative_weights":
+        w[1::3] *= -1.0
+        w[2, 0, 0, 0] = -0.5
+    elif kind == "nan_input":
+        x[g.random(size=x.shape) < 0.02] = np.nan
+    elif kind == "all_zero":
+        x[:], t[:] = 0.0, 0.0
+    want = orc.similarity_fwd(x, t, w, **kw)
+    got = run_similarity(pkg, x, t, w, **kw)
+    assert rel_err(got, want) <= SIM_TOL
+    if kind == "exact":
+        for b, m, i, j in hits:
+            assert got[b, m, i, j] == 0.0
+    # the recomputed outputs are the three-instruction form's, bit for bit; the others agree to rounding
+    exact_form = run_similarity(pkg, x, t, w, algo="direct", **kw)
+    assert rel_err(got, exact_form) <= SIM_TOL
+    if kind == "negative_weights":   # every output of a template with a negative weight is recomputed
+        assert np.array_equal(got[:, 1::3], exact_form[:, 1::3], equal_nan=True)
+    if kind == "all_zero":
+        assert np.array_equal(got[exact_form == 0.0], exact_form[exact_form == 0.0])
+
+
 @pytest.mark.parametrize("case", [
     dict(shape=(2, 8, 20, 20), O=16, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),
     dict(shape=(3, 5, 17, 13), O=70, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # odd C, ragged pixel tiles
