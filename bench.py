@@ -28,7 +28,7 @@ EXP_RATE = 19.66e12        # v_exp_f32 at a quarter of the 128 lanes/clk/CU VALU
 # HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
 # same workload scaled by a copy kernel of known size (profiles/sim_direct_l2_config3.md).
 # Keyed by evaluation path; None where no counter run exists for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"direct": 287.0e6, "mfma": 223.3e6}
+MEASURED_TRAFFIC_BYTES = {"sqrtw": 311.3e6, "direct": 287.0e6, "mfma": 223.3e6}
 
 
 def main():
