@@ -236,3 +236,43 @@ def test_gradient_entry_points_reject_bad_arguments_without_touching_the_device(
     assert l.simnets_hip_mex_input_grad(C.byref(m), xs, 256, 256, n_off, 256, 256, 256, None, 0, None) == -17
     bad = pkg.ops.mex_attrs(2, blocks=[4, 1, 1])                  # block deeper than the image
     assert l.simnets_hip_mex_offsets_grad(C.byref(bad), xs, 256, 256, n_off, 256, 256, 256, None, 0, None) < 0
+
+
+def test_launch_time_division_constants_divide_exactly(tmp_path):
+    # csrc/fast_div.h (the pixel enumeration of the MEX kernels divides by region sizes fixed per launch):
+    # host restatement checked against `/` around multiples of d, at the ends of the range and on random values
+    src = tmp_path / "fd.cpp"
+    src.write_text(r"""
+#include <cstdio>
+#include <cstdlib>
+#include "fast_div.h"
+using namespace simnets;
+int main() {
+    const unsigned ds[] = {1, 2, 3, 4, 5, 6, 7, 9, 10, 15, 16, 17, 31, 32, 33, 63, 64, 65, 100, 255, 256, 257, 1000, 4096,
+                           65535, 65536, 65537, 1000003, 1u << 30, (1u << 31) - 1, 1u << 31, 0xffffffffu};
+    long bad = 0;
+    srand(1);
+    for (unsigned d : ds) {
+        const FastDiv f = make_fast_div(d);
+        for (long i = 0; i < 300000; ++i) {
+            const unsigned n = i < 1000 ? (unsigned)i : i < 2000 ? 0xffffffffu - (unsigned)(i - 1000)
+                                                                 : ((unsigned)rand() << 16) ^ ((unsigned)rand() * 2654435761u);
+            for (int dd = -1; dd <= 1; ++dd) {
+                const unsigned nn = n - n % d + dd;
+                bad += fast_div(nn, f) != nn / d;
+            }
+        }
+    }
+    for (unsigned d = 1; d < 2000; ++d) {
+        const FastDiv f = make_fast_div(d);
+        for (unsigned n = 0; n < 100000; ++n)
+            bad += fast_div(n, f) != n / d;
+    }
+    printf("%ld\n", bad);
+    return 0;
+}
+""")
+    exe = tmp_path / "fd"
+    subprocess.run(["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "simnets-tf_amd", "csrc"), str(src), "-o",
+                    str(exe)], check=True)
+    assert subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.strip() == "0"
