@@ -217,6 +217,22 @@ def main():
         dev4 = float((fused_stack() - ref4).abs().max() / ref4.abs().max())
         others["config4_stack"].update({"fused_pool_kernel_ms": round(ms_fused, 4),
                                         "fused_pool_max_dev_of_scale": dev4})
+
+        # ... and with the Similarity layer evaluated inside the first of those kernels
+        off0, n0, kwm0 = layers[0]
+
+        def fused_stack3():
+            cur = pkg.similarity_mex_sum_pool(X4, T4, W4, off0, n0, (2, 2), similarity=kw4,
+                                              mex=dict(kwm0, normalize_offsets=True))
+            for off, n, kw in layers[1:]:
+                cur = pkg.mex_sum_pool(cur, off, n, (2, 2), normalize_offsets=True, **kw)
+            return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
+                           strides=[ch, 1, 1], shared_offset_region=[1])
+
+        _, ms_fused3 = timed(fused_stack3, args.steps, args.warmup)
+        dev43 = float((fused_stack3() - ref4).abs().max() / ref4.abs().max())
+        others["config4_stack"].update({"fused_similarity_mex_pool_kernel_ms": round(ms_fused3, 4),
+                                        "fused_similarity_mex_pool_max_dev_of_scale": dev43})
         # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
         _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,

@@ -250,6 +250,24 @@ int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input
                                  const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* Similarity, MEX over its output, sum pooling, as one call: the first layers of the reference's networks
+ * (README.md:108-129: Similarity on the image, MEX over all of its channels per pixel, pooling).  output =
+ * simnets_hip_sum_pool_fwd(simnets_hip_mex_fwd(simnets_hip_similarity_fwd(...))); mex_attrs describe the MEX layer
+ * over the Similarity output [B, O, oh, ow]; weights have the templates' shape.  When the MEX + pooling pair is
+ * fusable (above), the MEX blocks are [O, 1, 1] without padding and a Similarity patch has at most 16 elements, one
+ * kernel evaluates the Similarity channels inside its staging (same arithmetic and order as the Similarity kernel,
+ * term by term as SIMNETS_ALGO_DIRECT) and neither intermediate tensor exists; any other combination runs the
+ * separate kernels through scratch memory.  Forward only. */
+int simnets_hip_similarity_mex_sum_pool_workspace_bytes(const simnets_similarity_attrs *sim_attrs,
+                                                        const int input_shape[4], const int templates_shape[4],
+                                                        const simnets_mex_attrs *mex_attrs, int pool_h, int pool_w,
+                                                        size_t *bytes);
+int simnets_hip_similarity_mex_sum_pool_fwd(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                                            const int templates_shape[4], const float *input, const float *templates,
+                                            const float *weights, const simnets_mex_attrs *mex_attrs,
+                                            const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                            float *output, void *workspace, size_t workspace_bytes, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -16,6 +16,7 @@ EXPORTS = [
     "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
     "simnets_hip_mex_offsets_grad",
     "simnets_hip_mex_sum_pool_workspace_bytes", "simnets_hip_mex_sum_pool_fwd",
+    "simnets_hip_similarity_mex_sum_pool_workspace_bytes", "simnets_hip_similarity_mex_sum_pool_fwd",
 ]
 
 SIM_L1, SIM_L2 = 0, 1
@@ -102,6 +103,11 @@ def lib():
         l.simnets_hip_mex_sum_pool_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int, P, P,
                                                    C.c_size_t, P]
         SZ = C.POINTER(C.c_size_t)
+        l.simnets_hip_similarity_mex_sum_pool_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4,
+                                                                          C.POINTER(MexAttrs), C.c_int, C.c_int, SZ]
+        l.simnets_hip_similarity_mex_sum_pool_fwd.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, P, P, P,
+                                                              C.POINTER(MexAttrs), P, C.c_size_t, C.c_int, C.c_int, P,
+                                                              P, C.c_size_t, P]
         l.simnets_hip_similarity_grad_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, SZ, SZ]
         l.simnets_hip_similarity_input_grad.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P, P,
                                                         C.c_size_t, P]
@@ -121,7 +127,8 @@ def lib():
                      "simnets_hip_similarity_input_grad", "simnets_hip_similarity_params_grad",
                      "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
                      "simnets_hip_mex_offsets_grad", "simnets_hip_mex_sum_pool_workspace_bytes",
-                     "simnets_hip_mex_sum_pool_fwd"):
+                     "simnets_hip_mex_sum_pool_fwd", "simnets_hip_similarity_mex_sum_pool_workspace_bytes",
+                     "simnets_hip_similarity_mex_sum_pool_fwd"):
             getattr(l, name).restype = C.c_int
         _lib = l
     return _lib

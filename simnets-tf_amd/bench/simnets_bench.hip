@@ -390,6 +390,22 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) fused();
         ms = time_ms(s, steps, fused);
         report("config4 missing-data stack batch 512, MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        // ... and with the Similarity layer evaluated inside the first of those kernels
+        size_t f0bytes = 0;
+        SN_OK(simnets_hip_similarity_mex_sum_pool_workspace_bytes(&sc.a, sc.in, sc.tp, &mex[0].a, 2, 2, &f0bytes));
+        void *f0ws;
+        HIP_OK(hipMalloc(&f0ws, std::max<size_t>(f0bytes, 256)));
+        auto fused3 = [&] {
+            SN_OK(simnets_hip_similarity_mex_sum_pool_fwd(&sc.a, sc.in, sc.tp, sc.x, sc.t, sc.w, &mex[0].a, mex[0].o,
+                                                          mex[0].off_count, 2, 2, pooled[0], f0ws, f0bytes, s));
+            for (int l = 1; l < 4; ++l)
+                SN_OK(simnets_hip_mex_sum_pool_fwd(&mex[l].a, mex[l].in, mex[l].x, mex[l].o, mex[l].off_count, 2, 2,
+                                                   pooled[l], fws[l], fbytes[l], s));
+            run_mex(mex[4], s);
+        };
+        for (int i = 0; i < warmup; ++i) fused3();
+        ms = time_ms(s, steps, fused3);
+        report("config4 missing-data stack batch 512, Similarity + MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
     }
     else if (config == 5) {
         // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)

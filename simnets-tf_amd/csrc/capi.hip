@@ -212,4 +212,61 @@ int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input
     return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream);
 }
 
+static int sim_mex_pool_plans(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                              const int templates_shape[4], const simnets_mex_attrs *mex_attrs, int pool_h, int pool_w,
+                              SimPlan *sp, MexPlan *mp)
+{
+    int rc = sim_make_plan(sim_attrs, input_shape, templates_shape, templates_shape, sp);
+    if (rc)
+        return rc;
+    const int mid[4] = {sp->B, sp->O, sp->oh, sp->ow};
+    rc = mex_make_plan(mex_attrs, mid, mp);
+    if (rc)
+        return rc;
+    if (pool_h <= 0 || pool_w <= 0)
+        return SIMNETS_ERR_SHAPE;
+    if (mp->d.height_out / pool_h <= 0 || mp->d.width_out / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    return SIMNETS_OK;
+}
+
+int simnets_hip_similarity_mex_sum_pool_workspace_bytes(const simnets_similarity_attrs *sim_attrs,
+                                                        const int input_shape[4], const int templates_shape[4],
+                                                        const simnets_mex_attrs *mex_attrs, int pool_h, int pool_w,
+                                                        size_t *bytes)
+{
+    if (!bytes)
+        return SIMNETS_ERR_NULL_POINTER;
+    SimPlan sp;
+    MexPlan mp;
+    const int rc = sim_mex_pool_plans(sim_attrs, input_shape, templates_shape, mex_attrs, pool_h, pool_w, &sp, &mp);
+    if (rc)
+        return rc;
+    *bytes = sim_mex_pool_workspace_bytes(sp, mp, pool_h, pool_w);
+    return SIMNETS_OK;
+}
+
+int simnets_hip_similarity_mex_sum_pool_fwd(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                                            const int templates_shape[4], const float *input, const float *templates,
+                                            const float *weights, const simnets_mex_attrs *mex_attrs,
+                                            const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                            float *output, void *workspace, size_t workspace_bytes, void *stream)
+{
+    SimPlan sp;
+    MexPlan mp;
+    const int rc = sim_mex_pool_plans(sim_attrs, input_shape, templates_shape, mex_attrs, pool_h, pool_w, &sp, &mp);
+    if (rc)
+        return rc;
+    if (offsets_count < (size_t)mp.d.num_regions * mp.d.M * mp.d.K)
+        return SIMNETS_ERR_SHAPE;
+    if (sp.B == 0)
+        return SIMNETS_OK;
+    if (!input || !templates || !weights || !offsets || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, sim_mex_pool_workspace_bytes(sp, mp, pool_h, pool_w)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_mex_pool_launch(sp, mp, pool_h, pool_w, input, templates, weights, offsets, output, workspace,
+                               workspace_bytes, stream);
+}
+
 }  // extern "C"

@@ -68,6 +68,13 @@ int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *inp
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw);
 int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
                     void *workspace, size_t workspace_bytes, void *stream);
+// Similarity, then MEX over its output, then sum pooling; `mp` is the MEX plan for the Similarity output's shape.
+// One kernel when the MEX patch of a pixel is exactly the Similarity channels of that pixel (and the MEX + pooling
+// pair is fusable), else the separate kernels through scratch memory.
+size_t sim_mex_pool_workspace_bytes(const SimPlan &sp, const MexPlan &mp, int ph, int pw);
+int sim_mex_pool_launch(const SimPlan &sp, const MexPlan &mp, int ph, int pw, const float *input,
+                        const float *templates, const float *weights, const float *offsets, float *pooled,
+                        void *workspace, size_t workspace_bytes, void *stream);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

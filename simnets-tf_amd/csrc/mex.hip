@@ -36,6 +36,7 @@
 
 #include "internal.h"
 #include "mex_common.h"
+#include "sim_step.h"
 
 namespace simnets {
 
@@ -488,8 +489,25 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                                                               int finite_eps, float *__restrict__ offp,
                                                               float *__restrict__ offe, float *__restrict__ omax,
                                                               float *__restrict__ orng, int4 *__restrict__ ktab, int H,
-                                                              int W, int bh, int bw)
+                                                              int W, int bh, int bw, int row_blocks, SimPackJob job)
 {
+    if ((int)blockIdx.x >= row_blocks) {
+        // extra workgroups: the parameters of a Similarity layer evaluated inside the MEX staging
+        // layout: channels in chunks of 32, inside a chunk by staging phase (k % 4) and then k / 4, so that the 8
+        // channels one staging thread evaluates for a tap are 16 (pa) / 8 (pc) consecutive floats
+        const int Opad = (job.O + 31) & ~31;
+        const long long total = (long long)Opad * job.K;
+        for (long long i = (long long)(blockIdx.x - row_blocks) * 256 + threadIdx.x; i < total;
+             i += (long long)(gridDim.x - row_blocks) * 256) {
+            const int k = (int)(i / job.K), j = (int)(i - (long long)k * job.K);
+            const size_t src = (size_t)min(k, job.O - 1) * job.K + j;   // past the last channel: a copy (never used)
+            const int r32 = k & 31;
+            const size_t pos = ((((size_t)(k >> 5) * 4 + (r32 & 3)) * job.K + j) * 8) + (r32 >> 2);
+            sim_pack_element(job.mode, true, job.templates[src], job.weights[src], job.fudge, job.pa[2 * pos],
+                             job.pa[2 * pos + 1], job.pc[pos]);
+        }
+        return;
+    }
     if (blockIdx.x == 0) {
         // patch element k = (dc*bh + dh)*bw + dw -> where it lies relative to the patch origin
         for (int k = threadIdx.x; k < K; k += 256) {
@@ -814,7 +832,7 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups)
 }
 
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream)
+                     void *stream, const SimPackJob *job)
 {
     const simnets_mex_dims &d = p.d;
     const long long rows = (long long)d.num_regions * n_mgroups * tm;
@@ -828,12 +846,19 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
     int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
     if ((long long)d.block_c * p.H * p.W > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;  // the table holds 32-bit offsets
-    const dim3 grid((unsigned)((rows + 3) / 4));
+    const int row_blocks = (int)((rows + 3) / 4);
+    SimPackJob pj = {nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0.0f};
+    int extra = 0;
+    if (job) {
+        pj = *job;
+        extra = (int)std::min<long long>(((long long)((pj.O + 31) & ~31) * pj.K + 255) / 256, 64);
+    }
+    const dim3 grid((unsigned)(row_blocks + extra));
     hipStream_t hs = reinterpret_cast<hipStream_t>(stream);
 #define SIMNETS_PACK_LAUNCH(KL)                                                                                        \
     hipLaunchKernelGGL(mex_pack_offsets_kernel<KL>, grid, dim3(256), 0, hs, offsets, d.num_regions, d.M, d.K, n_mgroups, \
                        tm, p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W,         \
-                       d.block_h, d.block_w)
+                       d.block_h, d.block_w, row_blocks, pj)
     if (d.K <= 64)
         SIMNETS_PACK_LAUNCH(1);
     else if (d.K <= 256)

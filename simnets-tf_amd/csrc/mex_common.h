@@ -125,8 +125,17 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
 // Packs the offsets for the forward kernels (k-major tiles of tm instances per group: scaled values, their
 // exponentials relative to the row maximum, row maxima and ranges) and the patch element table into `workspace`
 // (mex_packed_bytes), and points the argument block at them.
+// `job` (optional): the parameters of a Similarity layer, packed by extra workgroups of the same launch
+// (sim_pack_element) for the kernel that evaluates that layer inside the MEX staging: channels in chunks of 32,
+// pa[chunk][k % 4][tap][k / 4 % 8] = (template, scaled negative weight), pc likewise.
+struct SimPackJob {
+    const float *templates, *weights;  // [O][K]
+    float *pa, *pc;                    // (O rounded up to 32) * K pairs / values
+    int O, K, mode;
+    float fudge;
+};
 size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream);
+                     void *stream, const SimPackJob *job = nullptr);
 
 }  // namespace simnets

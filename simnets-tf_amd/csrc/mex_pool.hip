@@ -18,6 +18,7 @@
 
 #include "internal.h"
 #include "mex_common.h"
+#include "sim_step.h"
 
 namespace simnets {
 
@@ -29,16 +30,29 @@ constexpr int KC = 32;             // k per LDS chunk
 constexpr int TM = 64, MX = 16;    // instances per workgroup / per wave
 constexpr int KSTEP = 4, U = KC / KSTEP;
 
+constexpr int kSimTaps = 16;       // longest Similarity patch the kernel evaluates inside its staging
+
 struct PoolArgs {
     float *pooled;
     int Hp, Wp;   // pooled height and width
     int spw;      // slots per workgroup: NH * 64 / R
+    // SIMF: the MEX input is the output of a Similarity layer that is evaluated on the fly
+    const float *sx;        // its input [B][sC][sH][sW]
+    const float *spa, *spc; // packed parameters [O][sK] (pairs) and [O][sK] (sim_pack_element)
+    int sC, sH, sW, sbh, sbw, ssh, ssw, sph, spw_, sK, smode;
+    float soob, snorm;      // out-of-bounds value; -0.5 K log(2 pi) of the normalized mode
+    int snorm_every, sB;    // reproduce the reference's per-iteration addition of that constant
 };
 
 // NH = column halves of a workgroup (64 pixel columns = 4 tiles of 16 each), 4 instance waves per half: two halves
 // share the offsets tiles and double the waves per SIMD the LDS budget allows, which is what hides the latencies of
 // the short dependent phases; one half only when there are no slots for a second one.
-template <int R, int NH, bool CHECK>
+// SIMF: the input of the MEX layer is a Similarity layer's output whose channels are exactly the MEX patch (blocks
+// [O, 1, 1], no padding): the staging evaluates Similarity channel k of its pixel from the layer's input (the patch
+// taps of the pixel sit in LDS, the packed parameters of channel k come through scalar loads) with the Similarity
+// kernel's own combine step in the same order, so the value is the one that kernel would have stored, and neither
+// that tensor nor its launches exist.
+template <int R, int NH, bool CHECK, bool SIMF>
 __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs a, const PoolArgs q)
 {
     constexpr int XP = 64 * NH;         // pixel columns of a workgroup
@@ -49,6 +63,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     __shared__ float pmx[KSTEP * XP];   // partial column maxima
     __shared__ float fsh[XP], msh[XP];  // per column: rescale factor of this chunk, running maximum
     __shared__ long long ppos[16 * G * NH];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
+    __shared__ float xt[SIMF ? kSimTaps * XP : 1];  // SIMF: Similarity patch taps of the columns, [tap][column]
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -95,6 +110,54 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     auto stage = [&](int k0, int kc) {
         const bool full = kc == KC;
         float v[U];
+        if (SIMF) {
+            if (k0 == 0) {
+                // taps of this column's Similarity patch (im2col_3d rule of that layer), once per workgroup
+                const int sbhw = q.sbh * q.sbw;
+                for (int j = sk; j < q.sK; j += KSTEP) {
+                    const int c = j / sbhw, rem = j - c * sbhw;
+                    const int hi = gp.hi0 * q.ssh - q.sph + rem / q.sbw, wi = gp.wi0 * q.ssw - q.spw_ + rem % q.sbw;
+                    const bool ok = hi >= 0 && hi < q.sH && wi >= 0 && wi < q.sW;
+                    xt[j * XP + col] = ok ? q.sx[(((size_t)gp.b * q.sC + c) * q.sH + hi) * q.sW + wi] : q.soob;
+                }
+                __syncthreads();
+            }
+            int reps = 0;
+            if (q.smode == SIM_MODE_L2_NORM)
+                reps = q.snorm_every ? q.sB - gp.b : 1;
+            // this thread's 8 channels of the chunk (k0 + sk + 4u) are 8 "templates" of one pixel for the combine
+            // step; their parameters for a tap are consecutive (one scalar load each for pa and pc)
+            static_assert(U == 8 && KC == 32 && KSTEP == 4, "parameter layout of the Similarity evaluation");
+            float acc[U][1];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                acc[u][0] = 0.0f;
+            const float *pa = q.spa + ((size_t)(k0 / KC) * KSTEP + sk) * q.sK * (2 * U);
+            const float *pc = q.spc + ((size_t)(k0 / KC) * KSTEP + sk) * q.sK * U;
+            for (int j = 0; j < q.sK; ++j) {
+                const float x1[1] = {xt[j * XP + col]};
+                float p2[2 * U], c1[U];
+#pragma unroll
+                for (int i = 0; i < 2 * U; ++i)
+                    p2[i] = pa[j * 2 * U + i];
+#pragma unroll
+                for (int i = 0; i < U; ++i)
+                    c1[i] = pc[j * U + i];
+                switch (q.smode) {
+                case SIM_MODE_L1: sim_step<SIM_MODE_L1, 1, U, true>(acc, x1, p2, c1); break;
+                case SIM_MODE_L2: sim_step<SIM_MODE_L2, 1, U, true>(acc, x1, p2, c1); break;
+                case SIM_MODE_L2_NORM: sim_step<SIM_MODE_L2_NORM, 1, U, true>(acc, x1, p2, c1); break;
+                default: sim_step<SIM_MODE_L2_NORM_IGNORE_NAN, 1, U, true>(acc, x1, p2, c1); break;
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                float val = acc[u][0];
+                for (int rr = 0; rr < reps; ++rr)
+                    val += q.snorm;
+                v[u] = val;
+            }
+        } else
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int kk = sk + u * KSTEP;
@@ -278,10 +341,12 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
 template <int R, int NH>
 hipError_t launch_pool(const MexKernelArgs &a, const PoolArgs &q, dim3 grid, bool inside, hipStream_t s)
 {
-    if (inside)
-        hipLaunchKernelGGL((mex_pool_kernel<R, NH, false>), grid, dim3(256 * NH), 0, s, a, q);
+    if (q.sx)
+        hipLaunchKernelGGL((mex_pool_kernel<R, NH, false, true>), grid, dim3(256 * NH), 0, s, a, q);
+    else if (inside)
+        hipLaunchKernelGGL((mex_pool_kernel<R, NH, false, false>), grid, dim3(256 * NH), 0, s, a, q);
     else
-        hipLaunchKernelGGL((mex_pool_kernel<R, NH, true>), grid, dim3(256 * NH), 0, s, a, q);
+        hipLaunchKernelGGL((mex_pool_kernel<R, NH, true, false>), grid, dim3(256 * NH), 0, s, a, q);
     return hipGetLastError();
 }
 
@@ -292,6 +357,65 @@ bool fusable(const MexPlan &p, int ph, int pw)
     const int r = ph * pw;
     return p.use_unshared && std::isfinite(p.epsilon) && d.offsets_c == 1 && d.offsets_h == ph && d.offsets_w == pw &&
            (r == 2 || r == 4) && d.num_regions == r;
+}
+
+// ... and the Similarity layer in front can be evaluated inside the staging when its channels are exactly the MEX
+// patch of a pixel and its own patches are short
+bool sim_fusable(const SimPlan &sp, const MexPlan &p, int ph, int pw)
+{
+    const simnets_mex_dims &d = p.d;
+    return fusable(p, ph, pw) && sp.K <= kSimTaps && sp.algo != SIMNETS_ALGO_MFMA && d.block_c == sp.O &&
+           d.block_h == 1 && d.block_w == 1 && d.stride_h == 1 && d.stride_w == 1 && d.pad_c == 0 && d.pad_h == 0 &&
+           d.pad_w == 0 && d.channels_out == 1;
+}
+
+size_t sim_packed_bytes(const SimPlan &sp) { return align_up((size_t)((sp.O + 31) & ~31) * sp.K * 3 * sizeof(float), 256); }
+
+int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
+                void *workspace, const SimPlan *sp, const float *templates, const float *weights, void *stream)
+{
+    const simnets_mex_dims &d = p.d;
+    const int n_mgroups = (d.M + TM - 1) / TM;
+    MexKernelArgs a = mex_kernel_args(p);
+    PoolArgs q;
+    q.sx = nullptr;
+    SimPackJob job;
+    if (sp) {
+        float *pa = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_packed_bytes(p, TM, n_mgroups));
+        job.templates = templates; job.weights = weights; job.pa = pa; job.pc = pa + (size_t)((sp->O + 31) & ~31) * sp->K * 2;
+        job.O = sp->O; job.K = sp->K; job.mode = sp->mode; job.fudge = sp->fudge;
+        q.sx = input; q.spa = job.pa; q.spc = job.pc;
+        q.sC = sp->C; q.sH = sp->H; q.sW = sp->W; q.sbh = sp->bh; q.sbw = sp->bw; q.ssh = sp->sh; q.ssw = sp->sw;
+        q.sph = sp->ph; q.spw_ = sp->pw; q.sK = sp->K; q.smode = sp->mode; q.soob = sp->oob;
+        q.snorm = (sp->mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)sp->K) * std::log(2.0 * M_PI)) : 0.0f;
+        q.snorm_every = sp->norm_const_every_iteration; q.sB = sp->B;
+    }
+    const int rc = mex_pack_offsets(p, offsets, TM, n_mgroups, workspace, &a, stream, sp ? &job : nullptr);
+    if (rc)
+        return rc;
+    a.in = sp ? nullptr : input;
+    q.pooled = pooled;
+    q.Hp = d.height_out / ph;
+    q.Wp = d.width_out / pw;
+    // two column halves per workgroup whenever there are slots for both: the extra waves per compute unit pay even
+    // when the launch then has fewer workgroups than compute units (measured on 512 images of 2x2 pixels)
+    const int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
+    q.spw = nh * 64 / (ph * pw);
+    const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
+    if (gx > 0x7fffffffLL || n_mgroups > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    const bool inside = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 &&
+                        (d.channels_out - 1) * d.stride_c + d.block_c <= p.C &&
+                        (d.height_out - 1) * d.stride_h + d.block_h <= p.H &&
+                        (d.width_out - 1) * d.stride_w + d.block_w <= p.W;
+    dim3 grid((unsigned)gx, (unsigned)n_mgroups);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    hipError_t e;
+    if (ph * pw == 4)
+        e = nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s);
+    else
+        e = nh == 2 ? launch_pool<2, 2>(a, q, grid, inside, s) : launch_pool<2, 1>(a, q, grid, inside, s);
+    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
 }  // namespace
@@ -318,35 +442,34 @@ int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const 
             return rc;
         return sum_pool_launch(p.B, d.M * d.channels_out, d.height_out, d.width_out, ph, pw, full, pooled, stream);
     }
-    const int n_mgroups = (d.M + TM - 1) / TM;
-    MexKernelArgs a = mex_kernel_args(p);
-    const int rc = mex_pack_offsets(p, offsets, TM, n_mgroups, workspace, &a, stream);
+    return pool_launch(p, ph, pw, input, offsets, pooled, workspace, nullptr, nullptr, nullptr, stream);
+}
+
+// Similarity -> MEX -> sum pooling.  `mp` is the MEX plan over the Similarity output's shape.
+size_t sim_mex_pool_workspace_bytes(const SimPlan &sp, const MexPlan &mp, int ph, int pw)
+{
+    if (sim_fusable(sp, mp, ph, pw))
+        return mex_packed_bytes(mp, TM, (mp.d.M + TM - 1) / TM) + sim_packed_bytes(sp);
+    // otherwise: the Similarity output in scratch memory, then the two (or three) kernels
+    const size_t mid = align_up((size_t)sp.B * sp.O * sp.oh * sp.ow * sizeof(float), 256);
+    return mid + std::max(sim_workspace_bytes(sp), mex_pool_workspace_bytes(mp, ph, pw));
+}
+
+int sim_mex_pool_launch(const SimPlan &sp, const MexPlan &mp, int ph, int pw, const float *input,
+                        const float *templates, const float *weights, const float *offsets, float *pooled,
+                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (workspace_bytes < sim_mex_pool_workspace_bytes(sp, mp, ph, pw))
+        return SIMNETS_ERR_WORKSPACE;
+    if (sim_fusable(sp, mp, ph, pw))
+        return pool_launch(mp, ph, pw, input, offsets, pooled, workspace, &sp, templates, weights, stream);
+    const size_t mid_bytes = align_up((size_t)sp.B * sp.O * sp.oh * sp.ow * sizeof(float), 256);
+    float *mid = reinterpret_cast<float *>(workspace);
+    char *rest = reinterpret_cast<char *>(workspace) + mid_bytes;
+    int rc = sim_launch(sp, input, templates, weights, mid, rest, workspace_bytes - mid_bytes, stream);
     if (rc)
         return rc;
-    a.in = input;
-    PoolArgs q;
-    q.pooled = pooled;
-    q.Hp = d.height_out / ph;
-    q.Wp = d.width_out / pw;
-    // two column halves per workgroup whenever there are slots for both: the extra waves per compute unit pay even
-    // when the launch then has fewer workgroups than compute units (measured on 512 images of 2x2 pixels)
-    const int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
-    q.spw = nh * 64 / (ph * pw);
-    const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
-    if (gx > 0x7fffffffLL || n_mgroups > 65535)
-        return SIMNETS_ERR_TOO_LARGE;
-    const bool inside = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 &&
-                        (d.channels_out - 1) * d.stride_c + d.block_c <= p.C &&
-                        (d.height_out - 1) * d.stride_h + d.block_h <= p.H &&
-                        (d.width_out - 1) * d.stride_w + d.block_w <= p.W;
-    dim3 grid((unsigned)gx, (unsigned)n_mgroups);
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    hipError_t e;
-    if (ph * pw == 4)
-        e = nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s);
-    else
-        e = nh == 2 ? launch_pool<2, 2>(a, q, grid, inside, s) : launch_pool<2, 1>(a, q, grid, inside, s);
-    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    return mex_pool_launch(mp, ph, pw, mid, offsets, pooled, rest, workspace_bytes - mid_bytes, stream);
 }
 
 }  // namespace simnets

@@ -402,6 +402,45 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
     return out
 
 
+def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, pool_size=(2, 2), similarity=None,
+                            mex=None, out=None):
+    """`sum_pooling(mex(similarity(input, templates, weights, **similarity), offsets, num_instances, **mex), pool_size)`
+    as one call (forward only): the first layers of the reference's networks (README.md:108-129).  `similarity` and
+    `mex` are dicts of the keyword arguments of those two functions.  One kernel when the MEX blocks are
+    [templates, 1, 1], the offsets are unshared over exactly the pooling window and a Similarity patch has at most 16
+    elements; the separate kernels through scratch memory otherwise."""
+    x = _require_cuda_f32("input", input)
+    t = _require_cuda_f32("templates", templates)
+    w = _require_cuda_f32("weights", weights)
+    off = _require_cuda_f32("offsets", offsets)
+    if x.dim() != 4 or t.dim() != 4 or tuple(w.shape) != tuple(t.shape):
+        raise SimnetsError(-15)
+    sa = similarity_attrs(**(similarity or {}))
+    ma = mex_attrs(num_instances, **(mex or {}))
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    l = _lib.lib()
+    I4 = C.c_int * 4
+    xs, ts = I4(*x.shape), I4(*t.shape)
+    mid, oshape = I4(), I4()
+    _check(l.simnets_similarity_out_shape(C.byref(sa), xs, ts, ts, mid))
+    _check(l.simnets_mex_out_shape(C.byref(ma), mid, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), xs, ts, C.byref(ma), ph, pw,
+                                                                 C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    pshape = (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw)
+    if out is None:
+        out = torch.empty(pshape, dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
+    with torch.cuda.device(x.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _check(l.simnets_hip_similarity_mex_sum_pool_fwd(C.byref(sa), xs, ts, x.data_ptr(), t.data_ptr(), w.data_ptr(),
+                                                         C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
+                                                         out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
+    return out
+
+
 def sum_pooling(input, pool_size=(2, 2), out=None):
     """Non-overlapping 'valid' sum pooling: the AveragePooling2D * area glue of the reference's
     missing-data example (README.md:108-111)."""

@@ -199,6 +199,29 @@ def test_fused_mex_sum_pool_entry_validates_without_touching_the_device(pkg):
                                           None) == 0
 
 
+def test_similarity_mex_sum_pool_entry_validates_without_touching_the_device(pkg):
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    sa = pkg.ops.similarity_attrs(blocks=[2, 2], strides=[2, 2], padding=[2, 2])
+    ma = pkg.ops.mex_attrs(8, blocks=[4, 1, 1], strides=[4, 1, 1], unshared_offset_region=[2])
+    x, t = I4(2, 1, 28, 28), I4(4, 1, 2, 2)
+    one, split = C.c_size_t(), C.c_size_t()
+    f = l.simnets_hip_similarity_mex_sum_pool_workspace_bytes
+    assert f(C.byref(sa), x, t, C.byref(ma), 2, 2, C.byref(one)) == 0 and one.value > 0
+    # a 4x4 window is not the 2x2 region grid: the Similarity output (2 x 4 x 16 x 16 floats) lives in scratch memory
+    assert f(C.byref(sa), x, t, C.byref(ma), 4, 4, C.byref(split)) == 0
+    assert split.value >= 2 * 4 * 16 * 16 * 4 + one.value - 4 * 4 * 3 * 4
+    assert f(C.byref(sa), x, t, C.byref(ma), 0, 2, C.byref(one)) == -15
+    assert f(C.byref(sa), x, t, C.byref(ma), 2, 2, None) == -1
+    assert f(C.byref(sa), x, I4(4, 2, 2, 2), C.byref(ma), 2, 2, C.byref(one)) != 0      # template channels != input's
+    g = l.simnets_hip_similarity_mex_sum_pool_fwd
+    assert g(C.byref(sa), x, t, 256, 256, 256, C.byref(ma), 256, 5, 2, 2, 256, None, 0, None) == -15
+    assert g(C.byref(sa), x, t, None, 256, 256, C.byref(ma), 256, 4 * 8 * 4, 2, 2, 256, None, 0, None) == -1
+    assert g(C.byref(sa), x, t, 256, 256, 256, C.byref(ma), 256, 4 * 8 * 4, 2, 2, 256, None, 0, None) == -17
+    assert g(C.byref(sa), I4(0, 1, 28, 28), t, None, None, None, C.byref(ma), None, 4 * 8 * 4, 2, 2, None, None, 0,
+             None) == 0
+
+
 def test_op_layer_refuses_cpu_tensors(pkg):
     import torch
     x = torch.zeros(1, 1, 4, 4)

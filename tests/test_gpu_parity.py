@@ -403,6 +403,62 @@ def test_mex_sum_pool_other_geometries_run_the_two_kernels(pkg, kw, pool):
     assert rel_err(got, want, floor=np.ones_like(want)) <= MEX_TOL
 
 
+@pytest.mark.parametrize("sim", [
+    dict(blocks=[2, 2], strides=[2, 2], padding=[2, 2], normalization_term=True, ignore_nan_input=True,
+         out_of_bounds_value=float("nan")),                                                   # the missing-data layer
+    dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1], normalization_term=True),             # normalized, 9 taps
+    dict(blocks=[2, 2], strides=[1, 1], padding=[0, 0]),                                      # plain L2
+    dict(blocks=[3, 2], strides=[2, 1], padding=[1, 0], similarity_function="L1", out_of_bounds_value=0.5),
+])
+@pytest.mark.parametrize("case", [
+    dict(im=(9, 1, 28, 28), O=32, n=64), dict(im=(40, 1, 30, 34), O=40, n=70), dict(im=(3, 2, 13, 16), O=8, n=5),
+])
+def test_similarity_mex_sum_pool_one_kernel(pkg, sim, case):
+    # Similarity channels = the MEX patch of a pixel, offsets unshared over the pooling window: a single kernel
+    g = np.random.default_rng(23)
+    im, O, n = case["im"], case["O"], case["n"]
+    if im[1] * sim["blocks"][0] * sim["blocks"][1] > 16:
+        pytest.skip("patch longer than the fused kernel takes (covered by the split path test)")
+    x = g.uniform(-0.5, 0.5, size=im).astype(np.float32)
+    if sim.get("ignore_nan_input"):
+        x[g.random(size=x.shape) < 0.25] = np.nan
+    t = (g.normal(size=(O, im[1]) + tuple(sim["blocks"])) * 0.3).astype(np.float32)
+    w = g.uniform(0.5, 1.5, size=t.shape).astype(np.float32)
+    s_ref = orc.similarity_fwd(x, t, w, **sim)
+    mkw = dict(softmax_mode=True, blocks=[O, 1, 1], strides=[O, 1, 1], use_unshared_regions=True,
+               unshared_offset_region=[1, 2, 2])
+    d = orc.mex_dims(orc.mex_args(s_ref.shape, n, **mkw))
+    off = (g.normal(size=(d.num_regions, n, O, 1, 1)) * 0.2).astype(np.float32)
+    got = pkg.similarity_mex_sum_pool(dev(x), dev(t), dev(w), dev(off), n, (2, 2), similarity=sim,
+                                      mex=dict(mkw, normalize_offsets=True)).cpu().numpy()
+    offn = orc.normalize_offsets(off)
+    want = pooled(orc.mex_fwd(s_ref, offn, n, **mkw), 2, 2)
+    shift = pooled(np.abs(orc.mex_fwd(s_ref, offn, n, **dict(mkw, epsilon=math.inf))), 2, 2)
+    assert got.shape == want.shape
+    assert rel_err(got, want, floor=shift) <= MEX_TOL
+    # the Similarity values inside the kernel are the Similarity kernel's own (term-by-term form), so the result is
+    # the separate calls' to the last bit
+    s_dev = pkg.similarity(dev(x), dev(t), dev(w), algo="direct", **sim)
+    two = pkg.mex_sum_pool(s_dev, dev(off), n, (2, 2), normalize_offsets=True, **mkw).cpu().numpy()
+    assert np.array_equal(got, two, equal_nan=True)
+
+
+def test_similarity_mex_sum_pool_other_geometries_run_the_separate_kernels(pkg):
+    g = np.random.default_rng(24)
+    x = g.normal(size=(3, 3, 12, 12)).astype(np.float32)
+    t = g.normal(size=(6, 3, 3, 3)).astype(np.float32)          # 27 taps: too long for the fused kernel
+    w = g.uniform(0.5, 1.5, size=t.shape).astype(np.float32)
+    sim = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    mkw = dict(softmax_mode=True, blocks=[3, 1, 1], strides=[3, 1, 1], unshared_offset_region=[1, 2, 2])
+    off = g.normal(size=(4, 5, 3, 1, 1)).astype(np.float32)
+    got = pkg.similarity_mex_sum_pool(dev(x), dev(t), dev(w), dev(off), 5, (2, 2), similarity=sim, mex=mkw)
+    two = pkg.mex_sum_pool(pkg.similarity(dev(x), dev(t), dev(w), **sim), dev(off), 5, (2, 2), **mkw)
+    assert torch.equal(got, two)
+    s_ref = orc.similarity_fwd(x, t, w, **sim)
+    want = pooled(orc.mex_fwd(s_ref, off, 5, **mkw), 2, 2)
+    assert rel_err(got.cpu().numpy(), want, floor=np.ones_like(want) * np.abs(s_ref).max()) <= MEX_TOL
+
+
 def test_sum_pooling(pkg):
     g = np.random.default_rng(16)
     x = g.normal(size=(3, 5, 9, 8)).astype(np.float32)
