@@ -46,6 +46,32 @@ def _workspace(device, nbytes):
     return ws
 
 
+_plans = {}
+
+
+def _plan_key(*parts):
+    """Hashable key of shapes and attribute values (floats by repr: NaN out-of-bounds values must compare equal)."""
+    def freeze(v):
+        if isinstance(v, (list, tuple)):
+            return tuple(freeze(e) for e in v)
+        if isinstance(v, dict):
+            return tuple(sorted((k, freeze(e)) for k, e in v.items()))
+        return repr(v) if isinstance(v, float) else v
+    return freeze(parts)
+
+
+def _cached_plan(key, make):
+    """Attribute struct, shapes and workspace size of a call: the host-side queries are pure functions of the
+    shapes and attributes, and repeated calls of a layer would otherwise spend more time in them than the GPU
+    spends in a small kernel."""
+    plan = _plans.get(key)
+    if plan is None:
+        if len(_plans) >= 512:
+            _plans.clear()
+        plan = _plans[key] = make()
+    return plan
+
+
 def _require_cuda_f32(name, t):
     if not isinstance(t, torch.Tensor):
         raise TypeError("%s must be a torch.Tensor" % name)
@@ -108,22 +134,30 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
     w = _require_cuda_f32("weights", weights)
     if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
         raise SimnetsError(-15)
-    a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
-                         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-                         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
-                         norm_const_every_iteration=norm_const_every_iteration)
     l = _lib.lib()
-    I4 = C.c_int * 4
-    xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
-    oshape = I4()
-    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+
+    def make():
+        a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+                             normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+                             ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
+                             norm_const_every_iteration=norm_const_every_iteration)
+        I4 = C.c_int * 4
+        xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
+        oshape = I4()
+        _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
+        nbytes = C.c_size_t()
+        _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
+        return a, xs, ts, wsh, tuple(oshape), nbytes.value
+
+    a, xs, ts, wsh, oshape, nbytes = _cached_plan(
+        _plan_key("similarity", x.shape, t.shape, w.shape, similarity_function, blocks, strides, padding,
+                  normalization_term, normalization_term_fudge, ignore_nan_input, out_of_bounds_value, algo,
+                  norm_const_every_iteration), make)
+    ws = _workspace(x.device, nbytes)
     if out is None:
-        out = torch.empty(tuple(oshape), dtype=torch.float32, device=x.device)
+        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
-        assert out.is_contiguous() and tuple(out.shape) == tuple(oshape) and out.dtype == torch.float32
+        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream().cuda_stream
         _check(l.simnets_hip_similarity_fwd(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
@@ -282,22 +316,30 @@ def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=
     off = _require_cuda_f32("offsets", offsets)
     if x.dim() != 4:
         raise SimnetsError(-15)
-    a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
-                  epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
-                  blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
-                  shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
-                  normalize_offsets=normalize_offsets)
     l = _lib.lib()
-    xs = (C.c_int * 4)(*x.shape)
-    oshape = (C.c_int * 4)()
-    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+
+    def make():
+        a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
+                      epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
+                      blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
+                      shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
+                      normalize_offsets=normalize_offsets)
+        xs = (C.c_int * 4)(*x.shape)
+        oshape = (C.c_int * 4)()
+        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+        nbytes = C.c_size_t()
+        _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
+        return a, xs, tuple(oshape), nbytes.value
+
+    a, xs, oshape, nbytes = _cached_plan(
+        _plan_key("mex", x.shape, num_instances, softmax_mode, padding, strides, blocks, epsilon,
+                  blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                  unshared_offset_region, normalize_offsets), make)
+    ws = _workspace(x.device, nbytes)
     if out is None:
-        out = torch.empty(tuple(oshape), dtype=torch.float32, device=x.device)
+        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
-        assert out.is_contiguous() and tuple(out.shape) == tuple(oshape) and out.dtype == torch.float32
+        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
     with torch.cuda.device(x.device):
         stream = torch.cuda.current_stream().cuda_stream
         _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
@@ -377,20 +419,27 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
     off = _require_cuda_f32("offsets", offsets)
     if x.dim() != 4:
         raise SimnetsError(-15)
-    a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
-                  epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
-                  blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
-                  shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
-                  normalize_offsets=normalize_offsets)
     ph, pw = int(pool_size[0]), int(pool_size[1])
     l = _lib.lib()
-    xs = (C.c_int * 4)(*x.shape)
-    oshape = (C.c_int * 4)()
-    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
-    pshape = (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw)
+
+    def make():
+        a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
+                      epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
+                      blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
+                      shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
+                      normalize_offsets=normalize_offsets)
+        xs = (C.c_int * 4)(*x.shape)
+        oshape = (C.c_int * 4)()
+        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+        nbytes = C.c_size_t()
+        _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
+        return a, xs, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), nbytes.value
+
+    a, xs, pshape, nbytes = _cached_plan(
+        _plan_key("mex_sum_pool", x.shape, num_instances, ph, pw, softmax_mode, padding, strides, blocks, epsilon,
+                  blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                  unshared_offset_region, normalize_offsets), make)
+    ws = _workspace(x.device, nbytes)
     if out is None:
         out = torch.empty(pshape, dtype=torch.float32, device=x.device)
     else:
