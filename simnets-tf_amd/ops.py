@@ -37,8 +37,7 @@ _workspaces = {}
 def _workspace(device, nbytes):
     """A scratch tensor per (device, current stream), grown on demand and reused across calls: the kernels that
     use it are ordered on that stream, and calls on different streams never share one."""
-    with torch.cuda.device(device):
-        key = (device.index, torch.cuda.current_stream().cuda_stream)
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
@@ -70,6 +69,22 @@ def _cached_plan(key, make):
             _plans.clear()
         plan = _plans[key] = make()
     return plan
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device(device):
+    """Context that makes `device` current for a launch; free when it already is (the usual case)."""
+    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
 
 
 def _require_cuda_f32(name, t):
@@ -158,8 +173,8 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
         out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_fwd(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                             out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out
@@ -196,8 +211,8 @@ def similarity_input_grad(input, templates, weights, output_grad, similarity_fun
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes), None))
     ws = _workspace(x.device, nbytes.value)
     dx = torch.empty_like(x)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_input_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                                    g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return dx
@@ -216,8 +231,8 @@ def similarity_parameters_grad(input, templates, weights, output_grad, similarit
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, None, C.byref(nbytes)))
     ws = _workspace(x.device, nbytes.value)
     dt, dw = torch.empty_like(t), torch.empty_like(w)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_params_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(),
                                                     w.data_ptr(), g.data_ptr(), dt.data_ptr(), dw.data_ptr(),
                                                     ws.data_ptr(), ws.numel(), stream))
@@ -340,8 +355,8 @@ def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=
         out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
                                      ws.data_ptr(), ws.numel(), stream))
     return out
@@ -379,8 +394,8 @@ def mex_input_grad(input, offsets, output, output_grad, num_instances, softmax_m
     _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, C.byref(nbytes), None))
     ws = _workspace(x.device, nbytes.value)
     dx = torch.empty_like(x)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_input_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
                                             g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return dx
@@ -401,8 +416,8 @@ def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax
     _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, None, C.byref(nbytes)))
     ws = _workspace(x.device, nbytes.value)
     doff = torch.empty_like(off)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_offsets_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
                                               g.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return doff
@@ -444,8 +459,8 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
         out = torch.empty(pshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_sum_pool_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), ph, pw,
                                               out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out
@@ -482,8 +497,8 @@ def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, p
         out = torch.empty(pshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_mex_sum_pool_fwd(C.byref(sa), xs, ts, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                                          C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
                                                          out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
@@ -498,8 +513,8 @@ def sum_pooling(input, pool_size=(2, 2), out=None):
     B, Cc, H, W = x.shape
     if out is None:
         out = torch.empty((B, Cc, H // max(ph, 1), W // max(pw, 1)), dtype=torch.float32, device=x.device)
-    with torch.cuda.device(x.device):
-        stream = torch.cuda.current_stream().cuda_stream
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),
                                                    stream))
     return out
