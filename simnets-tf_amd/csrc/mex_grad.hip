@@ -62,17 +62,10 @@ __device__ __forceinline__ float mex_term(float x_plus_off, float out, float g, 
 
 constexpr int GX_KT = 8;   // patch elements per lane (input gradient)
 
-// grid.x: (region, pixel chunk of 64 slots); grid.y: tile of 4*GX_KT patch elements (one GX_KT per wave)
-__global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs ga)
+// One wave: the 64 pixel slots of (region r, chunk) x GX_KT patch elements from k0, term by term.
+__device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r, int chunk, int k0, int lane)
 {
     const MexKernelArgs &a = ga.k;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int r = blockIdx.x / ga.cpr;
-    const int chunk = blockIdx.x - r * ga.cpr;
-    const int k0 = (blockIdx.y * 4 + wave) * GX_KT;
-    if (k0 >= a.K)
-        return;
     const PixelRef px = locate(a, r, chunk * 64 + lane);
     const bool valid = px.out_off >= 0;
 
@@ -114,21 +107,152 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
     }
 }
 
-constexpr int GO_MT = 4, GO_KT = 8;  // instances x patch elements per lane (offsets gradient)
-
-// grid.x: (region, pixel chunk of 64*pxl slots); grid.y: tile of 4*GO_MT instances (one GO_MT per wave);
-// grid.z: tile of GO_KT patch elements
-__global__ __launch_bounds__(256) void mex_grad_offsets_kernel(const MexGradArgs ga)
+// grid.x: (region, pixel chunk of 64 slots); grid.y: tile of 4*GX_KT patch elements (one GX_KT per wave)
+__global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs ga)
 {
-    const MexKernelArgs &a = ga.k;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int r = blockIdx.x / ga.cpr;
     const int chunk = blockIdx.x - r * ga.cpr;
-    const int m0 = (blockIdx.y * 4 + wave) * GO_MT;
-    const int k0 = blockIdx.z * GO_KT;
-    if (m0 >= a.M)
-        return;
+    const int k0 = (blockIdx.y * 4 + wave) * GX_KT;
+    if (k0 < ga.k.K)
+        mex_grad_input_wave(ga, r, chunk, k0, lane);
+}
+
+// Finite epsilon, product form on the fp32 matrix cores.  In the scaled domain (xs = c1 x, os = c1 off, outs = c1 out,
+// c1 = eps log2 e) a term is g 2^(xs_k + os_mk - outs_m + c0), and outs_m - c0 = log2 sum_k 2^(xs_k + os_mk) bounds every
+// xs_k + os_mk from above.  With lo_m = min_k os_mk and a = min_m (outs_m - c0 - lo_m) >= every xs_k of the pixel:
+//   term = 2^(xs_k - a) * 2^(os_mk - mo_m) * [ g_m 2^(a + mo_m - outs_m + c0) ],
+// all three factors at most 2^(range of the instance's offsets), and for the terms that matter (near 1) at least
+// 2^-range: d patch_k = 2^(xs_k - a) * sum_m W_m EO_mk is a GEMM over the instances (v_mfma_f32_16x16x4_f32 tiles:
+// 16 patch elements x 16 pixels x 4 instances) of the pixel factors W (computed from g and out, which the kernel
+// reads anyway: no pass over the patches is needed for the bound) with the packed offset exponentials EO of the
+// forward pass.  Used when every instance of the region has an offsets range of at most kProductRange; otherwise the
+// workgroup falls back to the term-by-term waves.
+// grid.x: (region, pixel chunk of 64 slots); grid.y: tile of GM_KT patch elements (16 per wave)
+constexpr int GM_TM = 32;   // instances per packed group = contraction chunk
+constexpr int GM_KT = 64;
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+__global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradArgs ga)
+{
+    const MexKernelArgs &a = ga.k;
+    __shared__ float eo[GM_KT * (GM_TM + 1)];   // [k][instance], padded rows
+    __shared__ float wt[GM_TM * 65];            // [instance][pixel], padded rows
+    __shared__ float pmn[4 * 64], ap[64];
+    __shared__ int pb[64], pc0[64], ph0[64], pw0[64];   // pixel table: image (-1: empty slot), patch origin
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = blockIdx.x / ga.cpr;
+    const int chunk = blockIdx.x - r * ga.cpr;
+    const int k0 = blockIdx.y * GM_KT;
+    const int n_mg = a.n_mgroups;
+    const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
+    {
+        int wide = 0;
+        for (int m = tid; m < a.M; m += 256)
+            wide |= !(orng_r[m] <= kProductRange);
+        if (__syncthreads_or(wide)) {
+#pragma unroll
+            for (int h = 0; h < GM_KT / (4 * GX_KT); ++h) {
+                const int kk0 = k0 + (wave * (GM_KT / (4 * GX_KT)) + h) * GX_KT;
+                if (kk0 < a.K)
+                    mex_grad_input_wave(ga, r, chunk, kk0, lane);
+            }
+            return;
+        }
+    }
+    const PixelRef px = locate(a, r, chunk * 64 + lane);
+    const bool valid = px.out_off >= 0;
+    if (wave == 0) {
+        pb[lane] = valid ? px.b : -1;
+        pc0[lane] = px.ci0; ph0[lane] = px.hi0; pw0[lane] = px.wi0;
+    }
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    // the pixel's bound a = min_m (outs_m - c0 - lo_m)
+    float amin = INFINITY;
+    for (int m = wave; m < a.M; m += 4)
+        amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
+    pmn[wave * 64 + lane] = amin;
+    __syncthreads();
+    if (wave == 0)
+        ap[lane] = valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
+    __syncthreads();
+    const float a_p = ap[lane];
+
+    const int lr = lane & 15, lq = lane >> 4;
+    floatx4 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (int mg = 0; mg < n_mg; ++mg) {
+        __syncthreads();  // the previous chunk's matrix instructions are done with eo / wt
+        const float4 *src = reinterpret_cast<const float4 *>(a.offe + (((size_t)r * n_mg + mg) * a.K + k0) * GM_TM);
+        for (int i = tid; i < GM_KT * (GM_TM / 4); i += 256) {
+            const int row = i / (GM_TM / 4), c4 = i % (GM_TM / 4);
+            const float4 v = k0 + row < a.K ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            float *d = eo + row * (GM_TM + 1) + 4 * c4;
+            d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
+        }
+#pragma unroll
+        for (int i = 0; i < GM_TM / 4; ++i) {
+            const int mm = wave + 4 * i, m = mg * GM_TM + mm;
+            float w = 0.0f;
+            if (valid && m < a.M) {
+                // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
+                const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
+                w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+            }
+            wt[mm * 65 + lane] = w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ms = 0; ms < GM_TM; ms += 4) {
+            const float av = eo[(wave * 16 + lr) * (GM_TM + 1) + ms + lq];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, wt[(ms + lq) * 65 + t * 16 + lr], acc[t], 0, 0, 0);
+        }
+    }
+    // ---- d patch_k = 2^(xs_k - a) * acc, scattered to the input element the patch element is ----
+    const int bhw = a.bh * a.bw;
+    const size_t chw = (size_t)a.C * a.H * a.W;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int k = k0 + wave * 16 + 4 * lq + v;
+        if (k >= a.K)
+            continue;
+        const int dc = k / bhw, rem = k - dc * bhw;
+        const int dh = rem / a.bw, dw = rem - dh * a.bw;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int p = t * 16 + lr;
+            const int b = pb[p];
+            if (b < 0)
+                continue;
+            const int ci = pc0[p] + dc, hi = ph0[p] + dh, wi = pw0[p] + dw;
+            if (!(ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W))
+                continue;
+            const size_t at = (size_t)b * chw + ((size_t)ci * a.H + hi) * a.W + wi;
+            const float val = acc[t][v] * __builtin_amdgcn_exp2f(__builtin_fmaf(a.in[at], a.c1, -ap[p]));
+            if (ga.overlap)
+                unsafeAtomicAdd(ga.dx + at, val);
+            else
+                ga.dx[at] = val;
+        }
+    }
+}
+
+constexpr int GO_MT = 4, GO_KT = 8;  // instances x patch elements per lane (offsets gradient)
+
+// One wave: GO_MT instances from m0 x GO_KT patch elements from k0 over the 64*pxl pixel slots of (region r,
+// chunk), term by term; writes its partial sums.
+__device__ __forceinline__ void mex_grad_offsets_wave(const MexGradArgs &ga, int r, int chunk, int m0, int k0, int lane)
+{
+    const MexKernelArgs &a = ga.k;
 
     float acc[GO_MT][GO_KT];
 #pragma unroll
@@ -191,15 +315,158 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_kernel(const MexGradArgs
     }
 }
 
-// dOff[r,m,k] = sum over pixel chunks, in chunk order
-__global__ void mex_grad_offsets_finish_kernel(const float *__restrict__ partial, long long n, int chunks,
-                                               float *__restrict__ doff)
+// grid.x: (region, pixel chunk of 64*pxl slots); grid.y: tile of 4*GO_MT instances (one GO_MT per wave);
+// grid.z: tile of GO_KT patch elements
+__global__ __launch_bounds__(256) void mex_grad_offsets_kernel(const MexGradArgs ga)
 {
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int r = blockIdx.x / ga.cpr;
+    const int chunk = blockIdx.x - r * ga.cpr;
+    const int m0 = (blockIdx.y * 4 + wave) * GO_MT;
+    if (m0 < ga.k.M)
+        mex_grad_offsets_wave(ga, r, chunk, m0, blockIdx.z * GO_KT, lane);
+}
+
+// Finite epsilon, product form (see mex_grad_input_mfma_kernel): d off_mk = 2^(os_mk - mo_m) * sum_px W_px,m 2^(xs_px,k - a_px)
+// is a GEMM over the pixels.  The bound a of a pixel only has to hold for the instances of the workgroup's tile, so
+// it is the minimum over those.  A workgroup owns 64 instances x 64 patch elements (wave: 16 x 64, four 16 x 16
+// tiles) and walks its pxl groups of 64 pixel slots: pixel factors W [pixel][instance] and patch exponentials
+// [pixel][k] go to LDS, 16 matrix steps of 4 pixels each.
+// grid.x: (region, pixel chunk of 64*pxl slots); grid.y: tile of 64 instances; grid.z: tile of 64 patch elements
+constexpr int GOM_MT = 64, GOM_KT = 64;
+
+__global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGradArgs ga)
+{
+    const MexKernelArgs &a = ga.k;
+    __shared__ float wt[64 * 65];   // [pixel][instance], padded rows
+    __shared__ float ex[64 * 65];   // [pixel][k], padded rows
+    __shared__ float pmn[4 * 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = blockIdx.x / ga.cpr;
+    const int chunk = blockIdx.x - r * ga.cpr;
+    const int m0 = blockIdx.y * GOM_MT, k0 = blockIdx.z * GOM_KT;
+    const int n_mg = a.n_mgroups;
+    const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
+    {
+        int wide = 0;
+        for (int m = tid; m < a.M; m += 256)
+            wide |= !(orng_r[m] <= kProductRange);
+        if (__syncthreads_or(wide)) {
+            // term by term: this workgroup's tile as GO_MT x GO_KT wave tiles
+            for (int i = wave; i < (GOM_MT / GO_MT) * (GOM_KT / GO_KT); i += 4) {
+                const int mm0 = m0 + (i / (GOM_KT / GO_KT)) * GO_MT, kk0 = k0 + (i % (GOM_KT / GO_KT)) * GO_KT;
+                if (mm0 < a.M && kk0 < a.K)
+                    mex_grad_offsets_wave(ga, r, chunk, mm0, kk0, lane);
+            }
+            return;
+        }
+    }
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    const int lr = lane & 15, lq = lane >> 4;
+    const int bhw = a.bh * a.bw;
+    floatx4 acc[4];
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    // this thread's instances when staging (16 of the tile, the same for the whole wave) and their constants
+    const int ms0 = m0 + wave * 16;
+    for (int s = 0; s < ga.pxl; ++s) {
+        const PixelRef px = locate(a, r, (chunk * ga.pxl + s) * 64 + lane);
+        const bool valid = px.out_off >= 0;
+        const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+        const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+        float ov[16], gv[16];
+        float amin = INFINITY;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = ms0 + i;
+            ov[i] = 0.0f;
+            gv[i] = 0.0f;
+            if (m < a.M) {
+                ov[i] = op[(size_t)m * plane];
+                gv[i] = valid ? gp[(size_t)m * plane] : 0.0f;
+                amin = fminf(amin, __builtin_fmaf(ov[i], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
+            }
+        }
+        __syncthreads();  // the previous group's matrix instructions are done with wt / ex / ap
+        pmn[wave * 64 + lane] = amin;
+        __syncthreads();
+        const float a_p = valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = ms0 + i;
+            float w = 0.0f;
+            if (m < a.M)
+                w = gv[i] * __builtin_amdgcn_exp2f(__builtin_fmaf(-ov[i], a.c1, a_p) + (omax_r[m] + a.c0));
+            wt[lane * 65 + wave * 16 + i] = w;
+        }
+        // patch exponentials: this thread's pixel, 16 of the tile's patch elements
+        const size_t img = (size_t)px.b * a.C * a.H * a.W;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int kk = wave * 16 + i, k = k0 + kk;
+            float e = 0.0f;
+            if (valid && k < a.K) {
+                const int dc = k / bhw, rem = k - dc * bhw;
+                const int ci = px.ci0 + dc, hi = px.hi0 + rem / a.bw, wi = px.wi0 + rem % a.bw;
+                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                const float x = ok ? a.in[img + ((size_t)ci * a.H + hi) * a.W + wi] : a.oob;
+                e = __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.c1, -a_p));
+            }
+            ex[lane * 65 + kk] = e;
+        }
+        __syncthreads();
+#pragma unroll 4
+        for (int ps = 0; ps < 64; ps += 4) {
+            const float av = wt[(ps + lq) * 65 + wave * 16 + lr];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, ex[(ps + lq) * 65 + t * 16 + lr], acc[t], 0, 0, 0);
+        }
+    }
+    // ---- partial sums of this pixel chunk: acc * 2^(os_mk - mo_m) ----
+    float *dst = ga.partial + ((size_t)chunk * a.R + r) * a.M * a.K;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int m = m0 + wave * 16 + 4 * lq + v;
+        if (m >= a.M)
+            continue;
+        const float *eo = a.offe + (((size_t)r * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int k = k0 + t * 16 + lr;
+            if (k < a.K)
+                dst[(size_t)m * a.K + k] = acc[t][v] * eo[(size_t)k * GM_TM];
+        }
+    }
+}
+
+// dOff[r,m,k] = sum over pixel chunks, in a fixed order (reproducible): a workgroup takes 32 consecutive elements,
+// its 8 groups of 32 threads each sum every 8th chunk in chunk order, and the 8 sums are added in group order.
+__global__ __launch_bounds__(256) void mex_grad_offsets_finish_kernel(const float *__restrict__ partial, long long n,
+                                                                     int chunks, float *__restrict__ doff)
+{
+    __shared__ float sm[8][32];
+    const int e = threadIdx.x & 31, sub = threadIdx.x >> 5;
+    for (long long i0 = (long long)blockIdx.x * 32; i0 < n; i0 += (long long)gridDim.x * 32) {
+        const long long i = i0 + e;
         float s = 0.0f;
-        for (int c = 0; c < chunks; ++c)
-            s += partial[(size_t)c * n + i];
-        doff[i] = s;
+        if (i < n)
+            for (int c = sub; c < chunks; c += 8)
+                s += partial[(size_t)c * n + i];
+        sm[sub][e] = s;
+        __syncthreads();
+        if (sub == 0 && i < n) {
+            float t = sm[0][e];
+#pragma unroll
+            for (int j = 1; j < 8; ++j)
+                t += sm[j][e];
+            doff[i] = t;
+        }
+        __syncthreads();
     }
 }
 
@@ -256,7 +523,8 @@ __global__ void mex_fill_zero_kernel(float *__restrict__ p, long long n)
 
 struct MexGradTiling {
     int pxl, cpr_offsets;
-    size_t norm_bytes, partial_bytes;
+    bool mfma;           // finite epsilon: the matrix-core kernels, fed by the forward pass's packed offsets
+    size_t norm_bytes, partial_bytes, packed_bytes;
 };
 
 MexGradTiling mex_grad_tiling(const MexPlan &p)
@@ -264,15 +532,18 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
     const simnets_mex_dims &d = p.d;
     MexGradTiling t;
     const long long slots = (long long)p.B * d.region_size;
-    const long long mk = (long long)((d.M + GO_MT - 1) / GO_MT) * ((d.K + GO_KT - 1) / GO_KT);
+    t.mfma = std::isfinite(p.epsilon);
+    const long long mk = t.mfma ? 4LL * ((d.M + GOM_MT - 1) / GOM_MT) * ((d.K + GOM_KT - 1) / GOM_KT)
+                                : (long long)((d.M + GO_MT - 1) / GO_MT) * ((d.K + GO_KT - 1) / GO_KT);
     auto waves = [&](int pxl) { return d.num_regions * ((slots + 64LL * pxl - 1) / (64LL * pxl)) * mk; };
     t.pxl = 16;
-    while (t.pxl > 1 && waves(t.pxl) < 4096)
+    while (t.pxl > 1 && waves(t.pxl) < (t.mfma ? 2048 : 4096))
         t.pxl >>= 1;
     t.cpr_offsets = (int)((slots + 64LL * t.pxl - 1) / (64LL * t.pxl));
     const size_t rmk = (size_t)d.num_regions * d.M * d.K * sizeof(float);
     t.norm_bytes = p.normalize_offsets ? align_up(rmk, 256) : 0;
     t.partial_bytes = align_up(rmk * t.cpr_offsets, 256);
+    t.packed_bytes = t.mfma ? mex_packed_bytes(p, GM_TM, (d.M + GM_TM - 1) / GM_TM) : 0;
     return t;
 }
 
@@ -292,12 +563,17 @@ int prepare_offsets(const MexPlan &p, const float *offsets, void *workspace, hip
 
 }  // namespace
 
-size_t mex_grad_input_workspace_bytes(const MexPlan &p) { return mex_grad_tiling(p).norm_bytes; }
+// finite epsilon: the matrix-core kernels read the forward pass's packed offsets (groups of GM_TM instances)
+size_t mex_grad_input_workspace_bytes(const MexPlan &p)
+{
+    const MexGradTiling t = mex_grad_tiling(p);
+    return t.norm_bytes + t.packed_bytes;
+}
 
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p)
 {
     const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.partial_bytes;
+    return t.norm_bytes + t.partial_bytes + t.packed_bytes;
 }
 
 int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
@@ -327,6 +603,17 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
     const long long gx = (long long)d.num_regions * ga.cpr;
+    if (std::isfinite(p.epsilon)) {
+        void *packed = reinterpret_cast<char *>(workspace) + mex_grad_tiling(p).norm_bytes;
+        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed, &ga.k, stream);
+        if (rc)
+            return rc;
+        const int gy = (d.K + GM_KT - 1) / GM_KT;
+        if (gx > 0x7fffffffLL || gy > 65535)
+            return SIMNETS_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
+        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
     const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
     if (gx > 0x7fffffffLL || gy > 65535)
         return SIMNETS_ERR_TOO_LARGE;
@@ -362,15 +649,28 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
     ga.cpr = t.cpr_offsets;
 
     const long long gx = (long long)d.num_regions * ga.cpr;
-    const int gy = (d.M + 4 * GO_MT - 1) / (4 * GO_MT);
-    const int gz = (d.K + GO_KT - 1) / GO_KT;
-    if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
-        return SIMNETS_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(mex_grad_offsets_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s, ga);
+    if (t.mfma) {
+        void *packed = reinterpret_cast<char *>(workspace) + t.norm_bytes + t.partial_bytes;
+        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed, &ga.k, stream);
+        if (rc)
+            return rc;
+        const int gy = (d.M + GOM_MT - 1) / GOM_MT, gz = (d.K + GOM_KT - 1) / GOM_KT;
+        if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
+            return SIMNETS_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(mex_grad_offsets_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
+                           ga);
+    } else {
+        const int gy = (d.M + 4 * GO_MT - 1) / (4 * GO_MT);
+        const int gz = (d.K + GO_KT - 1) / GO_KT;
+        if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
+            return SIMNETS_ERR_TOO_LARGE;
+        hipLaunchKernelGGL(mex_grad_offsets_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
+                           ga);
+    }
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
     const long long n = (long long)d.num_regions * d.M * d.K;
-    hipLaunchKernelGGL(mex_grad_offsets_finish_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 65535)),
+    hipLaunchKernelGGL(mex_grad_offsets_finish_kernel, dim3((unsigned)std::min<long long>((n + 31) / 32, 65535)),
                        dim3(256), 0, s, ga.partial, n, ga.cpr, offsets_grad);
     if (hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;

@@ -257,6 +257,29 @@ def test_mex_grads_geometries(pkg, case):
     check_mex_grads(pkg, x, off, case["n"], **case["kw"])
 
 
+@pytest.mark.parametrize("spread", ["narrow", "wide", "mixed"])
+@pytest.mark.parametrize("eps", [1.0, -2.0, 5.0, 12.0])
+@pytest.mark.parametrize("geom", [
+    dict(im=(5, 40, 6, 6), n=70, kw=dict(blocks=[40, 1, 1], strides=[40, 1, 1], padding=[0, 0, 0],
+                                         unshared_offset_region=[2])),                  # several instance groups
+    dict(im=(3, 6, 12, 12), n=10, kw=dict(blocks=[3, 3, 3], strides=[2, 1, 1], padding=[1, 1, 1],
+                                          use_unshared_regions=False, shared_offset_region=[2])),   # overlapping patches
+])
+def test_mex_grads_offset_ranges_product_and_term_by_term_forms(pkg, geom, spread, eps):
+    # finite epsilon: regions whose offsets span a small range run the product form on the matrix cores, wide ranges
+    # the term-by-term waves; regions of one launch may differ
+    g = np.random.default_rng(81)
+    kw = dict(geom["kw"], epsilon=eps, softmax_mode=False)
+    x, off = mex_case(15, geom["im"], geom["n"], **kw)
+    x = x * 4
+    off = off * 0.3
+    if spread == "wide":
+        off *= 300
+    elif spread == "mixed":
+        off[::2] *= 300
+    check_mex_grads(pkg, x, off, geom["n"], **kw)
+
+
 def test_mex_grads_config2_shape(pkg):
     x, off, n, kw = config2(batch=8)
     off = orc.normalize_offsets(off)
