@@ -85,6 +85,7 @@ int sim_make_plan(const simnets_similarity_attrs *a, const int in[4], const int 
     p->fudge = a->normalization_term_fudge;
     p->oob = a->out_of_bounds_value;
     p->norm_const_every_iteration = a->norm_const_every_iteration != 0;
+    p->exact_terms = a->algo == SIMNETS_ALGO_DIRECT;
     switch (a->algo) {
     case SIMNETS_ALGO_AUTO:
         // plain L2: the two-instruction sqrt-weight form, with its small outputs recomputed exactly

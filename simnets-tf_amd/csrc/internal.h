@@ -19,6 +19,7 @@ struct SimPlan {
     int oh, ow, K;
     int mode;  // SimMode
     int algo;  // resolved SIMNETS_ALGO_* (never AUTO)
+    int exact_terms;  // the caller named SIMNETS_ALGO_DIRECT: gradients, too, sum the reference's terms one by one
     float fudge, oob;
     int norm_const_every_iteration;
 };

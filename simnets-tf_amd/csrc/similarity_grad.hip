@@ -567,7 +567,7 @@ constexpr int LO = 8, LK = 4; // templates x patch elements per lane
 
 struct GradPArgs {
     const float *g, *x, *templates;
-    float *partial;    // [nacc][S][Opad][Kpad]
+    float *partial;    // [nacc][S][Opad][Kpad], then one [Opad][Kpad] slab of centres (moment form)
     int B, C, H, W, O, oh, ow, bh, bw, sh, sw, ph, pw, K;
     int Opad, Kpad;    // O, K rounded up to the workgroup tile
     int n_ktiles, n_tiles;
@@ -578,9 +578,18 @@ struct GradPArgs {
 };
 
 // MODE: SimMode of the forward op.  WO: waves along the templates (1 or 2).
-template <int MODE, int WO>
+// MOM (L2 modes): moment form.  With a centre c per (lane, patch element) - the mean of the lane's 8 templates -
+// and xc = x - c, tc = t - c, the sums over the pixels are
+//     sum g (x - t)   = S1 - tc G            S1 = sum g xc,  S2 = sum g xc^2,  G = sum g
+//     sum g (x - t)^2 = S2 - 2 tc S1 + tc^2 G
+// so a term costs two fused multiply-adds (xc and xc^2 are shared by the lane's 8 templates) instead of four
+// instructions; the finish kernel combines the moments in double precision.  The centre keeps tc of the order
+// of the spread of the templates, which bounds the cancellation: the error is eps sqrt(N) |g| (xc^2 + tc^2),
+// the same order as that of the term-by-term sums unless every template and every patch sit in one point.
+template <int MODE, int WO, bool MOM>
 __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const GradPArgs a)
 {
+    static_assert(!MOM || MODE != SIM_MODE_L1, "the moment form is for the L2 modes");
     constexpr int WK = kWaves / WO;
     constexpr int OWG = WO * 64, KWG = WK * 32;
     constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
@@ -638,6 +647,25 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             if constexpr (NORM)
                 an[oo][kk] = 0.0f;
         }
+    // moment form: centre per patch element of this lane, the sum of g of one template per lane (template lk of
+    // the lane's 8: the 8 lanes that share the templates cover them all)
+    float ctr[LK] = {0.0f, 0.0f, 0.0f, 0.0f}, gsum = 0.0f;
+    if constexpr (MOM) {
+        int nvalid = 0;
+#pragma unroll
+        for (int oo = 0; oo < LO; ++oo)
+            nvalid += lane_o(oo) < a.O ? 1 : 0;
+        const float inv = 1.0f / (float)max(nvalid, 1);
+#pragma unroll
+        for (int kk = 0; kk < LK; ++kk) {
+            float m = 0.0f;
+#pragma unroll
+            for (int oo = 0; oo < LO; ++oo)
+                m += t[oo][kk];  // 0 for the templates past the last one
+            m *= inv;
+            ctr[kk] = __builtin_fabsf(m) < __builtin_inff() ? m : 0.0f;  // a NaN/inf template stays its own affair
+        }
+    }
 
     const int ohow = a.oh * a.ow;
     constexpr int NSG = kThreads / PC;        // staging groups: thread (sp, sg) handles pixel sp, every NSG-th row
@@ -716,6 +744,26 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             const float gl[LO] = {ga.x, ga.y, ga.z, ga.w, gb2.x, gb2.y, gb2.z, gb2.w};
             float xl[LK] = {xq.x, xq.y, xq.z, xq.w};
             float keep[LK];
+            if constexpr (MOM) {
+                float xc[LK], x2[LK];
+#pragma unroll
+                for (int kk = 0; kk < LK; ++kk) {
+                    const bool ok = !IGN || xl[kk] == xl[kk];
+                    keep[kk] = ok ? 1.0f : 0.0f;
+                    xc[kk] = ok ? xl[kk] - ctr[kk] : 0.0f;
+                    x2[kk] = xc[kk] * xc[kk];
+                }
+#pragma unroll
+                for (int oo = 0; oo < LO; ++oo)
+#pragma unroll
+                    for (int kk = 0; kk < LK; ++kk) {
+                        at[oo][kk] = __builtin_fmaf(gl[oo], xc[kk], at[oo][kk]);
+                        aw[oo][kk] = __builtin_fmaf(gl[oo], x2[kk], aw[oo][kk]);
+                        if constexpr (IGN)
+                            an[oo][kk] = __builtin_fmaf(gl[oo], keep[kk], an[oo][kk]);
+                    }
+                return;
+            }
             if (IGN) {
 #pragma unroll
                 for (int kk = 0; kk < LK; ++kk) {
@@ -763,6 +811,13 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
             compute(ga1, gb1, xq1);
         }
+        if constexpr (MOM && !IGN) {
+            // sum of g of template lk of this lane (pixel order)
+            const float *g1 = gs[buf] + ((size_t)(g_row + (lk >> 2) * 8 * PCP)) * 4 + (lk & 3);
+#pragma unroll 8
+            for (int p = 0; p < PC; ++p)
+                gsum += g1[p * 4];
+        }
         if (more)
             store_chunk(buf ^ 1, gv, xv);
         __syncthreads();  // the other buffer is complete; nobody reads this one any more
@@ -778,30 +833,49 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         const size_t o = (size_t)lane_o(oo) * a.Kpad + k0;
         *reinterpret_cast<float4 *>(pt + o) = make_float4(at[oo][0], at[oo][1], at[oo][2], at[oo][3]);
         *reinterpret_cast<float4 *>(pw + o) = make_float4(aw[oo][0], aw[oo][1], aw[oo][2], aw[oo][3]);
-        if constexpr (NORM)
+        if constexpr (IGN || (NORM && !MOM))
             *reinterpret_cast<float4 *>(pn + o) = make_float4(an[oo][0], an[oo][1], an[oo][2], an[oo][3]);
+        if constexpr (MOM) {
+            if (split == 0)
+                *reinterpret_cast<float4 *>(a.partial + (size_t)3 * a.S * slab + o) =
+                    make_float4(ctr[0], ctr[1], ctr[2], ctr[3]);
+        }
     }
+    if constexpr (MOM && !IGN)
+        pn[(size_t)lane_o(lk) * a.Kpad + k0] = gsum;  // read back from patch-element tile 0: [o][4 * (o's slot)]
 }
 
 // Adds the partial sums in split order and applies the pixel-independent factors.
-__global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial, const float *__restrict__ weights,
-                                              int O, int K, int Opad, int Kpad, int S, int mode, float fudge,
-                                              float *__restrict__ dT, float *__restrict__ dW)
+// moment != 0: the partial sums are the moments S1, S2, G of sim_grad_params_kernel<.., MOM = true>.
+__global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial, const float *__restrict__ templates,
+                                              const float *__restrict__ weights, int O, int K, int Opad, int Kpad,
+                                              int S, int mode, int moment, float fudge, float *__restrict__ dT,
+                                              float *__restrict__ dW)
 {
     const long long total = (long long)O * K;
     const size_t slab = (size_t)Opad * Kpad;
+    const bool norm = mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+    const bool ign = mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
          idx += (long long)gridDim.x * blockDim.x) {
         const int k = (int)(idx % K);
         const int o = (int)(idx / K);
         const size_t src = (size_t)o * Kpad + k;
+        // where the sum of g lives: per (o, k) with ignore-NaN, else once per template (see the kernel's epilogue)
+        const int r = o & 63;
+        const size_t gsrc = moment && !ign ? (size_t)o * Kpad + 4 * (((r >> 5) << 2) | (r & 3)) : src;
         float st = 0.0f, sw = 0.0f, sn = 0.0f;
-        const bool norm = mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN;
         for (int s = 0; s < S; ++s) {
             st += partial[(size_t)s * slab + src];
             sw += partial[((size_t)S + s) * slab + src];
-            if (norm)
-                sn += partial[((size_t)2 * S + s) * slab + src];
+            if (norm || moment)
+                sn += partial[((size_t)2 * S + s) * slab + gsrc];
+        }
+        if (moment) {
+            const double tc = (double)templates[idx] - (double)partial[(size_t)3 * S * slab + src];
+            const double s1 = st, s2 = sw, g = sn;
+            st = (float)(s1 - tc * g);
+            sw = (float)(s2 + tc * (tc * g - 2.0 * s1));
         }
         const float w = weights[idx];
         if (mode == SIM_MODE_L1) {
@@ -819,6 +893,7 @@ __global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial,
 
 struct GpTiling {
     int WO, OWG, KWG, n_otiles, n_ktiles, Opad, Kpad, nchunks, cps, S, nacc;
+    bool moment;  // L2 modes unless the caller asked for the term-by-term arithmetic (algo DIRECT)
 };
 
 GpTiling gp_tiling(const SimPlan &p)
@@ -838,7 +913,8 @@ GpTiling gp_tiling(const SimPlan &p)
     S = std::min(S, std::max(1, t.nchunks));
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
-    t.nacc = (p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
+    t.moment = p.mode != SIM_MODE_L1 && !p.exact_terms;
+    t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
     return t;
 }
 
@@ -846,10 +922,17 @@ template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
     dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
-    if (t.WO == 2)
-        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2>), grid, dim3(kThreads), 0, s, a);
-    else
-        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1>), grid, dim3(kThreads), 0, s, a);
+    constexpr bool CAN = MODE != SIM_MODE_L1;
+    if (t.moment && CAN) {
+        if (t.WO == 2)
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, CAN>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, CAN>), grid, dim3(kThreads), 0, s, a);
+    } else if (t.WO == 2) {
+        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, false>), grid, dim3(kThreads), 0, s, a);
+    } else {
+        hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, false>), grid, dim3(kThreads), 0, s, a);
+    }
     return hipGetLastError();
 }
 
@@ -858,7 +941,7 @@ hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 size_t sim_grad_params_workspace_bytes(const SimPlan &p)
 {
     const GpTiling t = gp_tiling(p);
-    return align_up((size_t)t.nacc * t.S * t.Opad * t.Kpad * sizeof(float), 256);
+    return align_up(((size_t)t.nacc * t.S + (t.moment ? 1 : 0)) * t.Opad * t.Kpad * sizeof(float), 256);
 }
 
 int sim_grad_params(const SimPlan &p, const float *input, const float *templates, const float *weights,
@@ -891,8 +974,8 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
         return SIMNETS_ERR_HIP;
     const long long total = (long long)p.O * p.K;
     const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
-    hipLaunchKernelGGL(sim_grad_params_finish_kernel, dim3(blocks), dim3(256), 0, s, a.partial, weights, p.O, p.K,
-                       t.Opad, t.Kpad, t.S, p.mode, p.fudge, templates_grad, weights_grad);
+    hipLaunchKernelGGL(sim_grad_params_finish_kernel, dim3(blocks), dim3(256), 0, s, a.partial, templates, weights,
+                       p.O, p.K, t.Opad, t.Kpad, t.S, p.mode, t.moment ? 1 : 0, p.fudge, templates_grad, weights_grad);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

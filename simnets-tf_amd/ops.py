@@ -200,13 +200,13 @@ def _similarity_grad_setup(input, templates, weights, output_grad, kw):
 
 def similarity_input_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None, strides=None,
                           padding=None, normalization_term=None, normalization_term_fudge=None,
-                          ignore_nan_input=None, out_of_bounds_value=None, name=None):
+                          ignore_nan_input=None, out_of_bounds_value=None, name=None, algo=None):
     """Gradient of `similarity` w.r.t. its input: the SimilarityInputGrad op
     (python/simnets/ops/similarity.py:33-37, src/ops/similarity_op.cpp:141-156)."""
     l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
         similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value))
+        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes), None))
     ws = _workspace(x.device, nbytes.value)
@@ -220,13 +220,16 @@ def similarity_input_grad(input, templates, weights, output_grad, similarity_fun
 
 def similarity_parameters_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None,
                                strides=None, padding=None, normalization_term=None, normalization_term_fudge=None,
-                               ignore_nan_input=None, out_of_bounds_value=None, name=None):
+                               ignore_nan_input=None, out_of_bounds_value=None, name=None, algo=None):
     """Gradients of `similarity` w.r.t. templates and weights: the SimilarityParametersGrad op
-    (python/simnets/ops/similarity.py:38-44, src/ops/similarity_op.cpp:158-174)."""
+    (python/simnets/ops/similarity.py:38-44, src/ops/similarity_op.cpp:158-174).
+
+    Extension: `algo='direct'` sums the reference's terms one by one; by default the L2 modes accumulate the
+    moments sum g xc, sum g xc^2, sum g about a centre near the templates and combine them at the end."""
     l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
         similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value))
+        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, None, C.byref(nbytes)))
     ws = _workspace(x.device, nbytes.value)

@@ -123,6 +123,45 @@ def test_similarity_grads_ignore_nan(pkg, nan_frac, blocks, strides, padding):
     check_sim_grads(pkg, x, t, w, **kw)
 
 
+@pytest.mark.parametrize("algo", [None, "direct"])
+@pytest.mark.parametrize("func,norm,ign", [("L2", False, False), ("L2", True, False), ("L2", True, True)])
+@pytest.mark.parametrize("offset,spread", [(0.0, 1.0), (40.0, 1.0), (-7.0, 0.01), (3.0, 30.0)])
+def test_similarity_params_grad_moment_and_term_by_term_forms(pkg, algo, func, norm, ign, offset, spread):
+    """The L2 modes' parameter gradients by default combine moments about a centre near the templates; with
+    algo='direct' they sum the reference's terms.  Both forms stay within the bar when the data sit far from zero
+    (offset), when patches and templates nearly coincide (tiny spread) and when the templates lie far apart."""
+    g = np.random.default_rng(31)
+    x = (offset + g.normal(size=(3, 5, 14, 15))).astype(np.float32)
+    t = (offset + spread * g.normal(size=(11, 5, 3, 3))).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    if ign:
+        x[g.random(size=x.shape) < 0.2] = np.nan
+    kw = dict(similarity_function=func, blocks=[3, 3], strides=[1, 1], padding=[1, 1], normalization_term=norm,
+              ignore_nan_input=ign, out_of_bounds_value=offset)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = g.normal(size=out.shape).astype(np.float32)
+    dt, dw = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(og), algo=algo, **kw)
+    want_dt, want_dw = orc.similarity_params_grad(x, t, w, og, **kw)
+    true_dt, true_dw = orc.similarity_params_grad(*f64(x, t, w, og), **kw)
+    assert_grad_close(dt.cpu().numpy(), want_dt, true_dt, "templates grad")
+    assert_grad_close(dw.cpu().numpy(), want_dw, true_dw, "weights grad")
+
+
+def test_similarity_params_grad_nan_template_stays_in_its_own_row(pkg):
+    """A non-finite template poisons its own gradients only (the centre of the moment form ignores it)."""
+    x, t, w = sim_inputs(8, (2, 3, 9, 9), 5, (2, 2))
+    t[2, 1, 0, 1] = np.nan
+    kw = dict(similarity_function="L2", blocks=[2, 2], strides=[1, 1], padding=[0, 0])
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = np.random.default_rng(3).normal(size=out.shape).astype(np.float32)
+    dt, dw = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(og), **kw)
+    want_dt, want_dw = orc.similarity_params_grad(x, t, w, og, **kw)
+    for got, want in ((dt.cpu().numpy(), want_dt), (dw.cpu().numpy(), want_dw)):
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        ok = ~np.isnan(want)
+        assert rel_err(got[ok], want[ok], floor=np.full(want[ok].shape, 1e-2 * np.abs(want[ok]).max())) <= GRAD_TOL
+
+
 def test_similarity_grads_nan_input_without_ignore_propagates_like_the_reference(pkg):
     x, t, w = sim_inputs(7, (1, 2, 8, 8), 3, (3, 3))
     x[0, 1, 4, 4] = np.nan
