@@ -647,9 +647,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             if constexpr (NORM)
                 an[oo][kk] = 0.0f;
         }
-    // moment form: centre per patch element of this lane, the sum of g of one template per lane (template lk of
-    // the lane's 8: the 8 lanes that share the templates cover them all)
-    float ctr[LK] = {0.0f, 0.0f, 0.0f, 0.0f}, gsum = 0.0f;
+    // moment form: centre per patch element of this lane
+    float ctr[LK] = {0.0f, 0.0f, 0.0f, 0.0f};
     if constexpr (MOM) {
         int nvalid = 0;
 #pragma unroll
@@ -714,10 +713,20 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         }
     };
     // registers -> LDS buffer `buf`: g as [o/4][pixel][4], patch elements as [k/4][pixel][4]
+    // moment form without ignore-NaN: sum of g per template.  Every chunk passes through store_chunk once, so the
+    // staging thread adds up what it stores (its pixel sp of every chunk); the 32 pixel slots are added at the end.
+    float4 gacc[GR];
+#pragma unroll
+    for (int r = 0; r < GR; ++r)
+        gacc[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     auto store_chunk = [&](int buf, const float4 (&gv)[GR], const float4 (&xv)[XR]) {
 #pragma unroll
-        for (int r = 0; r < GR; ++r)
+        for (int r = 0; r < GR; ++r) {
             reinterpret_cast<float4 *>(gs[buf])[(sg + NSG * r) * PCP + sp] = gv[r];
+            if constexpr (MOM && !IGN) {
+                gacc[r].x += gv[r].x; gacc[r].y += gv[r].y; gacc[r].z += gv[r].z; gacc[r].w += gv[r].w;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < XR; ++r)
             reinterpret_cast<float4 *>(xs[buf])[(sg + NSG * r) * PCP + sp] = xv[r];
@@ -811,13 +820,6 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
             compute(ga1, gb1, xq1);
         }
-        if constexpr (MOM && !IGN) {
-            // sum of g of template lk of this lane (pixel order)
-            const float *g1 = gs[buf] + ((size_t)(g_row + (lk >> 2) * 8 * PCP)) * 4 + (lk & 3);
-#pragma unroll 8
-            for (int p = 0; p < PC; ++p)
-                gsum += g1[p * 4];
-        }
         if (more)
             store_chunk(buf ^ 1, gv, xv);
         __syncthreads();  // the other buffer is complete; nobody reads this one any more
@@ -841,8 +843,21 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
                     make_float4(ctr[0], ctr[1], ctr[2], ctr[3]);
         }
     }
-    if constexpr (MOM && !IGN)
-        pn[(size_t)lane_o(lk) * a.Kpad + k0] = gsum;  // read back from patch-element tile 0: [o][4 * (o's slot)]
+    if constexpr (MOM && !IGN) {
+        // pixel slots -> one sum per template, in slot order; the finish kernel reads patch-element tile 0's copy
+        // (the loop's last barrier has passed: nobody reads gs any more)
+#pragma unroll
+        for (int r = 0; r < GR; ++r)
+            reinterpret_cast<float4 *>(gs[0])[(sg + NSG * r) * PCP + sp] = gacc[r];
+        __syncthreads();
+        if (tid < OWG) {
+            const float *row = gs[0] + (size_t)(tid >> 2) * PCP * 4 + (tid & 3);
+            float sum = 0.0f;
+            for (int q = 0; q < PC; ++q)
+                sum += row[q * 4];
+            pn[(size_t)(o_wg + tid) * a.Kpad + k_wg] = sum;
+        }
+    }
 }
 
 // Adds the partial sums in split order and applies the pixel-independent factors.
@@ -862,8 +877,7 @@ __global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial,
         const int o = (int)(idx / K);
         const size_t src = (size_t)o * Kpad + k;
         // where the sum of g lives: per (o, k) with ignore-NaN, else once per template (see the kernel's epilogue)
-        const int r = o & 63;
-        const size_t gsrc = moment && !ign ? (size_t)o * Kpad + 4 * (((r >> 5) << 2) | (r & 3)) : src;
+        const size_t gsrc = moment && !ign ? (size_t)o * Kpad : src;
         float st = 0.0f, sw = 0.0f, sn = 0.0f;
         for (int s = 0; s < S; ++s) {
             st += partial[(size_t)s * slab + src];
