@@ -860,48 +860,60 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     }
 }
 
-// Adds the partial sums in split order and applies the pixel-independent factors.
+// Adds the partial sums in a fixed order and applies the pixel-independent factors.  256 threads = 32 elements x 8
+// groups: group j adds the splits j, j + 8, ..., the 8 group sums are added in group order through LDS.
 // moment != 0: the partial sums are the moments S1, S2, G of sim_grad_params_kernel<.., MOM = true>.
-__global__ void sim_grad_params_finish_kernel(const float *__restrict__ partial, const float *__restrict__ templates,
-                                              const float *__restrict__ weights, int O, int K, int Opad, int Kpad,
-                                              int S, int mode, int moment, float fudge, float *__restrict__ dT,
-                                              float *__restrict__ dW)
+__global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
+    const float *__restrict__ partial, const float *__restrict__ templates, const float *__restrict__ weights, int O,
+    int K, int Opad, int Kpad, int S, int mode, int moment, float fudge, float *__restrict__ dT,
+    float *__restrict__ dW)
 {
+    __shared__ float sm[3][8][32];
     const long long total = (long long)O * K;
     const size_t slab = (size_t)Opad * Kpad;
     const bool norm = mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     const bool ign = mode == SIM_MODE_L2_NORM_IGNORE_NAN;
-    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (long long)gridDim.x * blockDim.x) {
-        const int k = (int)(idx % K);
-        const int o = (int)(idx / K);
-        const size_t src = (size_t)o * Kpad + k;
-        // where the sum of g lives: per (o, k) with ignore-NaN, else once per template (see the kernel's epilogue)
-        const size_t gsrc = moment && !ign ? (size_t)o * Kpad : src;
-        float st = 0.0f, sw = 0.0f, sn = 0.0f;
-        for (int s = 0; s < S; ++s) {
+    const int e = threadIdx.x & 31, grp = threadIdx.x >> 5;
+    const long long idx = (long long)blockIdx.x * 32 + e;
+    const bool live = idx < total;
+    const int k = live ? (int)(idx % K) : 0;
+    const int o = live ? (int)(idx / K) : 0;
+    const size_t src = (size_t)o * Kpad + k;
+    // where the sum of g lives: per (o, k) with ignore-NaN, else once per template (see the kernel's epilogue)
+    const size_t gsrc = moment && !ign ? (size_t)o * Kpad : src;
+    float st = 0.0f, sw = 0.0f, sn = 0.0f;
+    if (live)
+        for (int s = grp; s < S; s += 8) {
             st += partial[(size_t)s * slab + src];
             sw += partial[((size_t)S + s) * slab + src];
             if (norm || moment)
                 sn += partial[((size_t)2 * S + s) * slab + gsrc];
         }
-        if (moment) {
-            const double tc = (double)templates[idx] - (double)partial[(size_t)3 * S * slab + src];
-            const double s1 = st, s2 = sw, g = sn;
-            st = (float)(s1 - tc * g);
-            sw = (float)(s2 + tc * (tc * g - 2.0 * s1));
-        }
-        const float w = weights[idx];
-        if (mode == SIM_MODE_L1) {
-            dT[idx] = w * st;
-            dW[idx] = -sw;
-        } else if (!norm) {
-            dT[idx] = 2.0f * w * st;
-            dW[idx] = -sw;
-        } else {
-            dT[idx] = w * st;
-            dW[idx] = 0.5f * (sn / (w + fudge) - sw);
-        }
+    sm[0][grp][e] = st; sm[1][grp][e] = sw; sm[2][grp][e] = sn;
+    __syncthreads();
+    if (grp != 0 || !live)
+        return;
+    st = sw = sn = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        st += sm[0][j][e]; sw += sm[1][j][e]; sn += sm[2][j][e];
+    }
+    if (moment) {
+        const double tc = (double)templates[idx] - (double)partial[(size_t)3 * S * slab + src];
+        const double s1 = st, s2 = sw, g = sn;
+        st = (float)(s1 - tc * g);
+        sw = (float)(s2 + tc * (tc * g - 2.0 * s1));
+    }
+    const float w = weights[idx];
+    if (mode == SIM_MODE_L1) {
+        dT[idx] = w * st;
+        dW[idx] = -sw;
+    } else if (!norm) {
+        dT[idx] = 2.0f * w * st;
+        dW[idx] = -sw;
+    } else {
+        dT[idx] = w * st;
+        dW[idx] = 0.5f * (sn / (w + fudge) - sw);
     }
 }
 
@@ -987,7 +999,11 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
     if (e != hipSuccess)
         return SIMNETS_ERR_HIP;
     const long long total = (long long)p.O * p.K;
-    const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
+    if (total == 0)
+        return SIMNETS_OK;
+    if ((total + 31) / 32 > 0x7fffffffLL)
+        return SIMNETS_ERR_TOO_LARGE;
+    const unsigned blocks = (unsigned)((total + 31) / 32);
     hipLaunchKernelGGL(sim_grad_params_finish_kernel, dim3(blocks), dim3(256), 0, s, a.partial, templates, weights,
                        p.O, p.K, t.Opad, t.Kpad, t.S, p.mode, t.moment ? 1 : 0, p.fudge, templates_grad, weights_grad);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
