@@ -8,7 +8,8 @@
 // Both gradients are sums of the same term
 //   e(px, m, k) = g[px,m] * exp(eps * (patch(px)[k] + off[r(px),m,k] - out[px,m]) + ey)        finite eps
 //               = g[px,m] * (patch(px)[k] + off[r(px),m,k] == out[px,m])                        eps = +-inf
-//   d patch(px)[k]  = sum_m e(px, m, k)          (then scattered to the input element the patch element is)
+//   d patch(px)[k]  = sum_m e(px, m, k)          (then stored to the input element the patch element is; patches
+//                                                 that overlap are added per element by mex_col2im_kernel)
 //   d off[r, m, k]  = sum_{px in region r} e(px, m, k)
 // Output pixels are enumerated region-major exactly like the forward kernel does, a lane owns
 // pixel slots, so the offsets a wave needs are the same for all its lanes (scalar loads).
@@ -32,7 +33,8 @@ struct MexGradArgs {
     const float *g;        // output gradient
     float *dx;             // input gradient
     float *partial;        // offsets gradient partial sums [chunk][R][M][K]
-    int overlap;           // patches overlap: the scatter must add atomically
+    int overlap;           // patches overlap: the per-patch gradients go to `col`, mex_col2im_kernel adds them up
+    float *col;            // [B][Co*Ho*Wo][K] gradient of every patch element (overlapping patches only)
     int cpr;               // pixel chunks per region
     int pxl;               // pixel slots per lane (offsets gradient)
 };
@@ -96,12 +98,13 @@ __device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r
     if (!valid)
         return;
     float *dimg = ga.dx + (size_t)px.b * a.C * a.H * a.W;
+    float *dcol = ga.col + ((size_t)px.b * plane + px.out_off) * a.K + k0;
 #pragma unroll
     for (int j = 0; j < GX_KT; ++j) {
         if (io[j] < 0)
             continue;
         if (ga.overlap)
-            unsafeAtomicAdd(dimg + io[j], acc[j]);
+            dcol[j] = acc[j];
         else
             dimg[io[j]] = acc[j];
     }
@@ -141,6 +144,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     __shared__ float wt[GM_TM * 65];            // [instance][pixel], padded rows
     __shared__ float pmn[4 * 64], ap[64];
     __shared__ int pb[64], pc0[64], ph0[64], pw0[64];   // pixel table: image (-1: empty slot), patch origin
+    __shared__ int pout[64];                            // ... and the pixel's offset within the image's output
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -168,6 +172,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     if (wave == 0) {
         pb[lane] = valid ? px.b : -1;
         pc0[lane] = px.ci0; ph0[lane] = px.hi0; pw0[lane] = px.wi0;
+        pout[lane] = px.out_off;
     }
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
@@ -239,11 +244,48 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             const size_t at = (size_t)b * chw + ((size_t)ci * a.H + hi) * a.W + wi;
             const float val = acc[t][v] * __builtin_amdgcn_exp2f(__builtin_fmaf(a.in[at], a.c1, -ap[p]));
             if (ga.overlap)
-                unsafeAtomicAdd(ga.dx + at, val);
+                ga.col[((size_t)b * plane + pout[p]) * a.K + k] = val;
             else
                 ga.dx[at] = val;
         }
     }
+}
+
+// Overlapping patches: input gradient = sum, over the patches that cover the element, of the patch-element
+// gradients in `col` (the reference's col2im_3d, src/utils/im2col.cpp:297-328), patches in ascending (c, h, w)
+// order.  One thread per input element; elements no patch covers get 0.
+__global__ __launch_bounds__(256) void mex_col2im_kernel(const MexKernelArgs a, const float *__restrict__ col,
+                                                         float *__restrict__ dx, long long n)
+{
+    const long long idx = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n)
+        return;
+    const int w = (int)(idx % a.W);
+    long long q = idx / a.W;
+    const int h = (int)(q % a.H); q /= a.H;
+    const int c = (int)(q % a.C);
+    const long long b = q / a.C;
+    // patches o along an axis that cover coordinate x: 0 <= x + pad - o * stride < block
+    auto first = [](int x, int pad, int block, int stride) {
+        const int lo = x + pad - block + 1;
+        return lo <= 0 ? 0 : (lo + stride - 1) / stride;
+    };
+    const int co_lo = first(c, a.pc, a.bc, a.sc), co_hi = min(a.Co - 1, (c + a.pc) / a.sc);
+    const int ho_lo = first(h, a.ph, a.bh, a.sh), ho_hi = min(a.Ho - 1, (h + a.ph) / a.sh);
+    const int wo_lo = first(w, a.pw, a.bw, a.sw), wo_hi = min(a.Wo - 1, (w + a.pw) / a.sw);
+    const float *cb = col + (size_t)b * a.Co * a.Ho * a.Wo * a.K;
+    float acc = 0.0f;
+    for (int co = co_lo; co <= co_hi; ++co) {
+        const int dc = c + a.pc - co * a.sc;
+        for (int ho = ho_lo; ho <= ho_hi; ++ho) {
+            const int dh = h + a.ph - ho * a.sh;
+            for (int wo = wo_lo; wo <= wo_hi; ++wo) {
+                const int dw = w + a.pw - wo * a.sw;
+                acc += cb[(((size_t)co * a.Ho + ho) * a.Wo + wo) * a.K + (dc * a.bh + dh) * a.bw + dw];
+            }
+        }
+    }
+    dx[idx] = acc;
 }
 
 constexpr int GO_MT = 4, GO_KT = 8;  // instances x patch elements per lane (offsets gradient)
@@ -525,6 +567,8 @@ struct MexGradTiling {
     int pxl, cpr_offsets;
     bool mfma;           // finite epsilon: the matrix-core kernels, fed by the forward pass's packed offsets
     size_t norm_bytes, partial_bytes, packed_bytes;
+    bool overlap;        // input gradient: patches overlap
+    size_t col_bytes;    // ... and their per-patch gradients pass through a [B][Co*Ho*Wo][K] buffer
 };
 
 MexGradTiling mex_grad_tiling(const MexPlan &p)
@@ -544,6 +588,10 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
     t.norm_bytes = p.normalize_offsets ? align_up(rmk, 256) : 0;
     t.partial_bytes = align_up(rmk * t.cpr_offsets, 256);
     t.packed_bytes = t.mfma ? mex_packed_bytes(p, GM_TM, (d.M + GM_TM - 1) / GM_TM) : 0;
+    t.overlap = (d.block_c > d.stride_c && d.channels_out > 1) || (d.block_h > d.stride_h && d.height_out > 1) ||
+                (d.block_w > d.stride_w && d.width_out > 1);
+    t.col_bytes = t.overlap ? align_up((size_t)p.B * d.channels_out * d.height_out * d.width_out * d.K * sizeof(float),
+                                       256) : 0;
     return t;
 }
 
@@ -567,7 +615,7 @@ int prepare_offsets(const MexPlan &p, const float *offsets, void *workspace, hip
 size_t mex_grad_input_workspace_bytes(const MexPlan &p)
 {
     const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.packed_bytes;
+    return t.norm_bytes + t.packed_bytes + t.col_bytes;
 }
 
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p)
@@ -591,34 +639,51 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
     if (rc)
         return rc;
     ga.out = output; ga.g = output_grad; ga.dx = input_grad; ga.partial = nullptr;
-    ga.overlap = (d.block_c > d.stride_c && d.channels_out > 1) || (d.block_h > d.stride_h && d.height_out > 1) ||
-                 (d.block_w > d.stride_w && d.width_out > 1);
+    const MexGradTiling t = mex_grad_tiling(p);
+    ga.overlap = t.overlap ? 1 : 0;
+    ga.col = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes);
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
 
-    // elements no patch covers keep gradient 0; overlapping patches add into it
     const long long n_in = (long long)p.B * p.C * p.H * p.W;
-    hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)), dim3(256),
-                       0, s, input_grad, n_in);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
+    if (n_in == 0)
+        return SIMNETS_OK;
+    if ((n_in + 255) / 256 > 0x7fffffffLL)
+        return SIMNETS_ERR_TOO_LARGE;
+    if (!t.overlap) {
+        // every element belongs to at most one patch, which stores its gradient; the others keep 0
+        hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
+                           dim3(256), 0, s, input_grad, n_in);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+    }
     const long long gx = (long long)d.num_regions * ga.cpr;
-    if (std::isfinite(p.epsilon)) {
-        void *packed = reinterpret_cast<char *>(workspace) + mex_grad_tiling(p).norm_bytes;
+    if (t.mfma) {
+        void *packed = reinterpret_cast<char *>(workspace) + t.norm_bytes;
         rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed, &ga.k, stream);
         if (rc)
             return rc;
         const int gy = (d.K + GM_KT - 1) / GM_KT;
         if (gx > 0x7fffffffLL || gy > 65535)
             return SIMNETS_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
-        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+        if (gx > 0)
+            hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
+    } else {
+        const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
+        if (gx > 0x7fffffffLL || gy > 65535)
+            return SIMNETS_ERR_TOO_LARGE;
+        if (gx > 0)
+            hipLaunchKernelGGL(mex_grad_input_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
     }
-    const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
-    if (gx > 0x7fffffffLL || gy > 65535)
-        return SIMNETS_ERR_TOO_LARGE;
-    hipLaunchKernelGGL(mex_grad_input_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
-    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    if (hipGetLastError() != hipSuccess)
+        return SIMNETS_ERR_HIP;
+    if (t.overlap) {
+        hipLaunchKernelGGL(mex_col2im_kernel, dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, s, ga.k, ga.col,
+                           input_grad, n_in);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+    }
+    return SIMNETS_OK;
 }
 
 int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,
@@ -644,7 +709,7 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
         return rc;
     ga.out = output; ga.g = output_grad; ga.dx = nullptr;
     ga.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes);
-    ga.overlap = 0;
+    ga.overlap = 0; ga.col = nullptr;
     ga.pxl = t.pxl;
     ga.cpr = t.cpr_offsets;
 

@@ -319,6 +319,21 @@ def test_mex_grads_offset_ranges_product_and_term_by_term_forms(pkg, geom, sprea
     check_mex_grads(pkg, x, off, geom["n"], **kw)
 
 
+@pytest.mark.parametrize("eps", [2.0, -math.inf])
+def test_mex_input_grad_of_overlapping_patches_is_reproducible(pkg, eps):
+    """Overlapping patches: the per-patch gradients are added per input element in a fixed order (no atomics), so
+    two calls agree bit for bit; the sum over patches matches the oracle's col2im."""
+    kw = dict(blocks=[3, 3, 3], strides=[1, 2, 1], padding=[1, 0, 2], epsilon=eps, softmax_mode=True,
+              use_unshared_regions=False, shared_offset_region=[2, 3, 1], blocks_out_of_bounds_value=0.5)
+    x, off = mex_case(23, (4, 7, 11, 9), 9, **kw)
+    out = orc.mex_fwd(x, off, 9, **kw)
+    go = np.random.default_rng(5).normal(size=out.shape).astype(np.float32)
+    runs = [pkg.mex_input_grad(dev(x), dev(off), dev(out), dev(go), 9, **kw).cpu().numpy() for _ in range(3)]
+    assert np.array_equal(runs[0], runs[1]) and np.array_equal(runs[0], runs[2])
+    want = orc.mex_input_grad(x, off, out, go, 9, **kw)
+    assert rel_err(runs[0], want, floor=np.full(want.shape, 1e-2 * np.abs(want).max())) <= GRAD_TOL
+
+
 def test_mex_grads_config2_shape(pkg):
     x, off, n, kw = config2(batch=8)
     off = orc.normalize_offsets(off)
