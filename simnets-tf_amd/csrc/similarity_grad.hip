@@ -902,7 +902,9 @@ __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
         const double tc = (double)templates[idx] - (double)partial[(size_t)3 * S * slab + src];
         const double s1 = st, s2 = sw, g = sn;
         st = (float)(s1 - tc * g);
-        sw = (float)(s2 + tc * (tc * g - 2.0 * s1));
+        // an infinite second moment (infinite inputs, overflow) is the answer as it stands; the correction would
+        // turn it into inf - inf
+        sw = __builtin_isfinite(s2) ? (float)(s2 + tc * (tc * g - 2.0 * s1)) : sw;
     }
     const float w = weights[idx];
     if (mode == SIM_MODE_L1) {

@@ -162,6 +162,26 @@ def test_similarity_params_grad_nan_template_stays_in_its_own_row(pkg):
         assert rel_err(got[ok], want[ok], floor=np.full(want[ok].shape, 1e-2 * np.abs(want[ok]).max())) <= GRAD_TOL
 
 
+@pytest.mark.parametrize("algo", [None, "direct"])
+def test_similarity_params_grad_infinite_input_like_the_reference(pkg, algo):
+    """An infinite input element gives the parameter gradients of its patch element the reference's infinities and
+    NaNs (g (x - t) = +-inf, sums of both signs = NaN), in both forms of the sums."""
+    x, t, w = sim_inputs(9, (2, 2, 6, 6), 4, (2, 2))
+    x[1, 0, 2, 3] = np.inf
+    kw = dict(similarity_function="L2", blocks=[2, 2], strides=[2, 2], padding=[0, 0])
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = np.abs(np.random.default_rng(4).normal(size=out.shape)).astype(np.float32)   # one sign: the sums stay +-inf
+    dt, dw = pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(og), algo=algo, **kw)
+    with np.errstate(invalid="ignore", over="ignore"):
+        want_dt, want_dw = orc.similarity_params_grad(x, t, w, og, **kw)
+    for got, want in ((dt.cpu().numpy(), want_dt), (dw.cpu().numpy(), want_dw)):
+        assert np.isinf(want).any()
+        assert np.array_equal(np.isnan(got), np.isnan(want))
+        assert np.array_equal(got[np.isinf(want)], want[np.isinf(want)])
+        ok = np.isfinite(want)
+        assert rel_err(got[ok], want[ok], floor=np.full(want[ok].shape, 1e-2 * np.abs(want[ok]).max())) <= GRAD_TOL
+
+
 def test_similarity_grads_nan_input_without_ignore_propagates_like_the_reference(pkg):
     x, t, w = sim_inputs(7, (1, 2, 8, 8), 3, (3, 3))
     x[0, 1, 4, 4] = np.nan
