@@ -586,10 +586,16 @@ struct GradPArgs {
 // instructions; the finish kernel combines the moments in double precision.  The centre keeps tc of the order
 // of the spread of the templates, which bounds the cancellation: the error is eps sqrt(N) |g| (xc^2 + tc^2),
 // the same order as that of the term-by-term sums unless every template and every patch sit in one point.
+// MOM (L1): scaled-sign form.  With dB = 2^64 (x - t) (one fma against the pre-scaled template; exact scaling),
+// sign(x - t) = med3(dB, -1, 1) and |x - t| = 2^-64 |dB|: four instructions per term (fma, med3, fma, fma against
+// g and 2^-64 g) instead of seven with compares and selects, bit-identical to them unless 0 < |x - t| < 2^-64,
+// |g| < 2^-62 or a value beyond 2^63.  A pixel chunk with a NaN input (found while staging, uniform for the
+// workgroup) takes the compare-and-select arithmetic, which has the reference's NaN rules.
 template <int MODE, int WO, bool MOM>
 __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const GradPArgs a)
 {
-    static_assert(!MOM || MODE != SIM_MODE_L1, "the moment form is for the L2 modes");
+    constexpr bool MOM2 = MOM && MODE != SIM_MODE_L1;   // moment form of the L2 modes
+    constexpr bool SGN = MOM && MODE == SIM_MODE_L1;    // scaled-sign form of L1
     constexpr int WK = kWaves / WO;
     constexpr int OWG = WO * 64, KWG = WK * 32;
     constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
@@ -642,6 +648,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         for (int kk = 0; kk < LK; ++kk) {
             const bool ok = lane_o(oo) < a.O && k0 + kk < a.K;
             t[oo][kk] = ok ? a.templates[(size_t)lane_o(oo) * a.K + k0 + kk] : 0.0f;
+            if constexpr (SGN)
+                t[oo][kk] *= 0x1p64f;
             at[oo][kk] = 0.0f;
             aw[oo][kk] = 0.0f;
             if constexpr (NORM)
@@ -649,7 +657,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         }
     // moment form: centre per patch element of this lane
     float ctr[LK] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if constexpr (MOM) {
+    if constexpr (MOM2) {
         int nvalid = 0;
 #pragma unroll
         for (int oo = 0; oo < LO; ++oo)
@@ -723,7 +731,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
 #pragma unroll
         for (int r = 0; r < GR; ++r) {
             reinterpret_cast<float4 *>(gs[buf])[(sg + NSG * r) * PCP + sp] = gv[r];
-            if constexpr (MOM && !IGN) {
+            if constexpr (MOM2 && !IGN) {
                 gacc[r].x += gv[r].x; gacc[r].y += gv[r].y; gacc[r].z += gv[r].z; gacc[r].w += gv[r].w;
             }
         }
@@ -736,11 +744,24 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     const int chunk_end = min((split + 1) * a.cps, a.nchunks);
     float4 gv[GR], xv[XR];
     __syncthreads();  // ktab written
+    auto has_nan = [](const float4 (&xv)[XR]) {
+        bool any = false;
+#pragma unroll
+        for (int r = 0; r < XR; ++r)
+            any |= xv[r].x != xv[r].x || xv[r].y != xv[r].y || xv[r].z != xv[r].z || xv[r].w != xv[r].w;
+        return any;
+    };
+    bool nan_chunk = false;  // scaled-sign form: the chunk in use holds a NaN input (uniform for the workgroup)
     if (chunk_begin < chunk_end) {
         load_chunk(chunk_begin, gv, xv);
         store_chunk(0, gv, xv);
+        if constexpr (SGN)
+            nan_chunk = has_nan(xv);
     }
-    __syncthreads();
+    if constexpr (SGN)
+        nan_chunk = __syncthreads_or(nan_chunk);
+    else
+        __syncthreads();
     for (int chunk = chunk_begin; chunk < chunk_end; ++chunk) {
         const int buf = (chunk - chunk_begin) & 1;
         const bool more = chunk + 1 < chunk_end;
@@ -749,11 +770,35 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         const float4 *g4 = reinterpret_cast<const float4 *>(gs[buf]) + g_row;
         const float4 *x4 = reinterpret_cast<const float4 *>(xs[buf]) + x_row;
 
+        // scaled-sign form of a pixel (chunks without NaN inputs)
+        auto compute_sgn = [&](const float4 &ga, const float4 &gb2, const float4 &xq) {
+            const float gl[LO] = {ga.x, ga.y, ga.z, ga.w, gb2.x, gb2.y, gb2.z, gb2.w};
+            const float xl[LK] = {xq.x, xq.y, xq.z, xq.w};
+            float gsc[LO];
+#pragma unroll
+            for (int oo = 0; oo < LO; ++oo)
+                gsc[oo] = gl[oo] * 0x1p-64f;
+#pragma unroll
+            for (int oo = 0; oo < LO; ++oo)
+#pragma unroll
+                for (int kk = 0; kk < LK; ++kk) {
+                    const float db = __builtin_fmaf(xl[kk], 0x1p64f, -t[oo][kk]);
+                    const float sg = __builtin_amdgcn_fmed3f(db, -1.0f, 1.0f);
+                    at[oo][kk] = __builtin_fmaf(sg, gl[oo], at[oo][kk]);
+                    aw[oo][kk] = __builtin_fmaf(gsc[oo], __builtin_fabsf(db), aw[oo][kk]);
+                }
+        };
+        // scaled-sign form, chunk with a NaN input: the compare-and-select arithmetic below on the templates scaled
+        // back.  The factor is opaque to the compiler (set per pixel) so that the 32 products are formed where they
+        // are used and not kept in registers.
         auto compute = [&](const float4 &ga, const float4 &gb2, const float4 &xq) {
             const float gl[LO] = {ga.x, ga.y, ga.z, ga.w, gb2.x, gb2.y, gb2.z, gb2.w};
             float xl[LK] = {xq.x, xq.y, xq.z, xq.w};
             float keep[LK];
-            if constexpr (MOM) {
+            float unscale = 1.0f;
+            if constexpr (SGN)
+                asm volatile("v_mov_b32 %0, 0x1f800000" : "=v"(unscale));  // 2^-64
+            if constexpr (MOM2) {
                 float xc[LK], x2[LK];
 #pragma unroll
                 for (int kk = 0; kk < LK; ++kk) {
@@ -786,7 +831,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
                 float d[LK], e[LK], gg[LK];
 #pragma unroll
                 for (int kk = 0; kk < LK; ++kk) {
-                    d[kk] = xl[kk] - t[oo][kk];
+                    d[kk] = xl[kk] - (SGN ? t[oo][kk] * unscale : t[oo][kk]);
                     gg[kk] = IGN ? gl[oo] * keep[kk] : gl[oo];
                 }
                 if (L1) {
@@ -812,17 +857,33 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             }
         };
         // one pixel ahead: the three reads of pixel p+1 are issued before the arithmetic of pixel p
-        float4 ga = g4[0], gb2 = g4[8 * PCP], xq = x4[0];
-        for (int p = 0; p < PC; p += 2) {
-            const float4 ga1 = g4[p + 1], gb1 = g4[8 * PCP + p + 1], xq1 = x4[p + 1];
-            compute(ga, gb2, xq);
-            const int pn = p + 2 < PC ? p + 2 : p;
-            ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
-            compute(ga1, gb1, xq1);
+        auto pixels = [&](auto &&fn) {
+            float4 ga = g4[0], gb2 = g4[8 * PCP], xq = x4[0];
+            for (int p = 0; p < PC; p += 2) {
+                const float4 ga1 = g4[p + 1], gb1 = g4[8 * PCP + p + 1], xq1 = x4[p + 1];
+                fn(ga, gb2, xq);
+                const int pn = p + 2 < PC ? p + 2 : p;
+                ga = g4[pn]; gb2 = g4[8 * PCP + pn]; xq = x4[pn];
+                fn(ga1, gb1, xq1);
+            }
+        };
+        if (SGN && !nan_chunk) {
+            pixels(compute_sgn);
+        } else if (SGN) {
+            // rare: one pixel at a time, no read-ahead (keeps this loop out of the register budget of the other)
+#pragma unroll 1
+            for (int p = 0; p < PC; ++p)
+                compute(g4[p], g4[8 * PCP + p], x4[p]);
+        } else {
+            pixels(compute);
         }
         if (more)
             store_chunk(buf ^ 1, gv, xv);
-        __syncthreads();  // the other buffer is complete; nobody reads this one any more
+        // the other buffer is complete; nobody reads this one any more
+        if constexpr (SGN)
+            nan_chunk = __syncthreads_or(more && has_nan(xv));
+        else
+            __syncthreads();
     }
 
     // partial sums of this split
@@ -837,13 +898,13 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         *reinterpret_cast<float4 *>(pw + o) = make_float4(aw[oo][0], aw[oo][1], aw[oo][2], aw[oo][3]);
         if constexpr (IGN || (NORM && !MOM))
             *reinterpret_cast<float4 *>(pn + o) = make_float4(an[oo][0], an[oo][1], an[oo][2], an[oo][3]);
-        if constexpr (MOM) {
+        if constexpr (MOM2) {
             if (split == 0)
                 *reinterpret_cast<float4 *>(a.partial + (size_t)3 * a.S * slab + o) =
                     make_float4(ctr[0], ctr[1], ctr[2], ctr[3]);
         }
     }
-    if constexpr (MOM && !IGN) {
+    if constexpr (MOM2 && !IGN) {
         // pixel slots -> one sum per template, in slot order; the finish kernel reads patch-element tile 0's copy
         // (the loop's last barrier has passed: nobody reads gs any more)
 #pragma unroll
@@ -921,7 +982,9 @@ __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
 
 struct GpTiling {
     int WO, OWG, KWG, n_otiles, n_ktiles, Opad, Kpad, nchunks, cps, S, nacc;
-    bool moment;  // L2 modes unless the caller asked for the term-by-term arithmetic (algo DIRECT)
+    bool fast;    // unless the caller asked for the term-by-term arithmetic (algo DIRECT): moment form (L2 modes),
+                  // scaled-sign form (L1)
+    bool moment;  // fast and an L2 mode
 };
 
 GpTiling gp_tiling(const SimPlan &p)
@@ -941,7 +1004,8 @@ GpTiling gp_tiling(const SimPlan &p)
     S = std::min(S, std::max(1, t.nchunks));
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
-    t.moment = p.mode != SIM_MODE_L1 && !p.exact_terms;
+    t.fast = !p.exact_terms;
+    t.moment = t.fast && p.mode != SIM_MODE_L1;
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
     return t;
 }
@@ -950,12 +1014,11 @@ template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
     dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
-    constexpr bool CAN = MODE != SIM_MODE_L1;
-    if (t.moment && CAN) {
+    if (t.fast) {
         if (t.WO == 2)
-            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, CAN>), grid, dim3(kThreads), 0, s, a);
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true>), grid, dim3(kThreads), 0, s, a);
         else
-            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, CAN>), grid, dim3(kThreads), 0, s, a);
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, true>), grid, dim3(kThreads), 0, s, a);
     } else if (t.WO == 2) {
         hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, false>), grid, dim3(kThreads), 0, s, a);
     } else {

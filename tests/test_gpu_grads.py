@@ -412,3 +412,31 @@ def test_similarity_l1_grads_at_ties_and_nan(pkg):
     x[0, 1, 2, 2] = np.nan
     w[2, 0, 2, 2] = 0.0
     check_sim_grads(pkg, x, t, w, similarity_function="L1", blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+
+
+@pytest.mark.parametrize("nan", [False, True])
+def test_similarity_l1_params_grad_scaled_sign_form_equals_the_term_by_term_form(pkg, nan):
+    """L1 parameter gradients by default take sign and magnitude from 2^64 (x - t) (fma, med3); with algo='direct'
+    they use compares and selects.  Same sums in the same order: bit-identical, ties and zero weights included;
+    pixel chunks with a NaN input run the compare-and-select arithmetic in both."""
+    x, t, w = sim_inputs(22, (3, 5, 17, 19), 37, (3, 3))
+    t[0, 0, 1, 1] = x[0, 0, 4, 4]
+    x[1, 1, :, 3] = t[1, 1, 0, 0]
+    x[2, 3, 5:9, 2:11] = 0.0
+    w[2, 0, 2, 2] = 0.0
+    if nan:
+        x[0, 1, 2, 2] = np.nan
+        x[2, 4, 16, 18] = np.nan
+    kw = dict(similarity_function="L1", blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = np.random.default_rng(8).normal(size=out.shape).astype(np.float32)
+    fast = [a.cpu().numpy() for a in pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(og), **kw)]
+    exact = [a.cpu().numpy() for a in pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(og), algo="direct", **kw)]
+    assert np.array_equal(fast[0], exact[0], equal_nan=True)
+    assert np.array_equal(fast[1], exact[1], equal_nan=True)
+    want_dt, want_dw = orc.similarity_params_grad(x, t, w, og, **kw)
+    assert np.array_equal(np.isnan(fast[0]), np.isnan(want_dt)) and np.array_equal(np.isnan(fast[1]), np.isnan(want_dw))
+    true_dt, true_dw = orc.similarity_params_grad(*f64(x, t, w, og), **kw)
+    ok = ~np.isnan(want_dw)
+    assert_grad_close(fast[0], want_dt, true_dt, "templates grad")
+    assert_grad_close(np.where(ok, fast[1], 0), np.where(ok, want_dw, 0), np.where(ok, true_dw, 0), "weights grad")
