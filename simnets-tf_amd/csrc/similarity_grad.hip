@@ -36,6 +36,8 @@ namespace simnets {
 
 namespace {
 
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
 constexpr int kWaves = 4;
 constexpr int kThreads = 64 * kWaves;
 constexpr int kLdsBudgetFloats = 16384;
@@ -591,9 +593,15 @@ struct GradPArgs {
 // g and 2^-64 g) instead of seven with compares and selects, bit-identical to them unless 0 < |x - t| < 2^-64,
 // |g| < 2^-62 or a value beyond 2^63.  A pixel chunk with a NaN input (found while staging, uniform for the
 // workgroup) takes the compare-and-select arithmetic, which has the reference's NaN rules.
-template <int MODE, int WO, bool MOM>
+// MF (with MOM, L2 modes): the moments on the fp32 matrix cores.  S1 = g^T xc, S2 = g^T xc^2 (and, with ignore-NaN,
+// G = g^T keep) are contractions over the pixels: a wave's 64 templates x 32 patch elements are two
+// v_mfma_f32_32x32x2_f32 tiles per moment, templates = rows, patch elements = columns, two pixels per instruction;
+// the operands come from the same LDS chunks (one ds_read_b32 each: lane = (row or column, pixel parity)).  The
+// centre is then per (wave, patch element): the mean over the wave's 64 templates.
+template <int MODE, int WO, bool MOM, bool MF = false>
 __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const GradPArgs a)
 {
+    static_assert(!MF || (MOM && MODE != SIM_MODE_L1), "the matrix-core form computes the moments of the L2 modes");
     constexpr bool MOM2 = MOM && MODE != SIM_MODE_L1;   // moment form of the L2 modes
     constexpr bool SGN = MOM && MODE == SIM_MODE_L1;    // scaled-sign form of L1
     constexpr int WK = kWaves / WO;
@@ -646,7 +654,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     for (int oo = 0; oo < LO; ++oo)
 #pragma unroll
         for (int kk = 0; kk < LK; ++kk) {
-            const bool ok = lane_o(oo) < a.O && k0 + kk < a.K;
+            const bool ok = !MF && lane_o(oo) < a.O && k0 + kk < a.K;
             t[oo][kk] = ok ? a.templates[(size_t)lane_o(oo) * a.K + k0 + kk] : 0.0f;
             if constexpr (SGN)
                 t[oo][kk] *= 0x1p64f;
@@ -657,7 +665,31 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         }
     // moment form: centre per patch element of this lane
     float ctr[LK] = {0.0f, 0.0f, 0.0f, 0.0f};
-    if constexpr (MOM2) {
+    // matrix-core form: this lane's column (patch element) and pixel parity, the centre of the column, accumulators
+    const int mcol = lane & 31, mhalf = lane >> 5;
+    const int mk = k_wg + wk * 32 + mcol;
+    float mctr = 0.0f;
+    floatx16 ms1[2], ms2[2], msn[2];
+    if constexpr (MF) {
+        float m = 0.0f;
+        int nvalid = 0;
+        for (int r = 0; r < 64; ++r) {
+            const int o = o_wg + wo * 64 + r;
+            if (o < a.O && mk < a.K) {
+                m += a.templates[(size_t)o * a.K + mk];
+                ++nvalid;
+            }
+        }
+        m *= 1.0f / (float)max(nvalid, 1);
+        mctr = __builtin_fabsf(m) < __builtin_inff() ? m : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                ms1[i][v] = 0.0f; ms2[i][v] = 0.0f; msn[i][v] = 0.0f;
+            }
+    }
+    if constexpr (MOM2 && !MF) {
         int nvalid = 0;
 #pragma unroll
         for (int oo = 0; oo < LO; ++oo)
@@ -867,7 +899,31 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
                 fn(ga1, gb1, xq1);
             }
         };
-        if (SGN && !nan_chunk) {
+        if constexpr (MF) {
+            // two pixels per step: rows = templates (g), columns = patch elements (xc, xc^2, keep); the reads of
+            // the next step are issued before this step's matrix instructions
+            const float *ga_ = gs[buf] + ((size_t)(wo * 16 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3);
+            const float *xb_ = xs[buf] + ((size_t)(wk * 8 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3);
+            float a0 = ga_[0], a1 = ga_[8 * PCP * 4], xv_ = xb_[0];
+#pragma unroll 4
+            for (int p = 0; p < PC; p += 2) {
+                const int pn = p + 2 < PC ? p + 2 : p;
+                const float na0 = ga_[pn * 4], na1 = ga_[8 * PCP * 4 + pn * 4], nx = xb_[pn * 4];
+                const bool ok = !IGN || xv_ == xv_;
+                const float xc = ok ? xv_ - mctr : 0.0f;
+                const float x2 = xc * xc;
+                ms1[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, xc, ms1[0], 0, 0, 0);
+                ms1[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, xc, ms1[1], 0, 0, 0);
+                ms2[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, x2, ms2[0], 0, 0, 0);
+                ms2[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, x2, ms2[1], 0, 0, 0);
+                if constexpr (IGN) {
+                    const float keep1 = ok ? 1.0f : 0.0f;
+                    msn[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, keep1, msn[0], 0, 0, 0);
+                    msn[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, keep1, msn[1], 0, 0, 0);
+                }
+                a0 = na0; a1 = na1; xv_ = nx;
+            }
+        } else if (SGN && !nan_chunk) {
             pixels(compute_sgn);
         } else if (SGN) {
             // rare: one pixel at a time, no read-ahead (keeps this loop out of the register budget of the other)
@@ -891,8 +947,23 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     float *pt = a.partial + (size_t)split * slab;
     float *pw = a.partial + ((size_t)a.S + split) * slab;
     float *pn = a.partial + ((size_t)2 * a.S + split) * slab;
+    if constexpr (MF) {
+        // tile i, register v: template row 8 (v / 4) + 4 * parity + v % 4, column mcol
 #pragma unroll
-    for (int oo = 0; oo < LO; ++oo) {
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const size_t o = (size_t)(o_wg + wo * 64 + i * 32 + 8 * (v / 4) + 4 * mhalf + (v % 4)) * a.Kpad + mk;
+                pt[o] = ms1[i][v];
+                pw[o] = ms2[i][v];
+                if constexpr (IGN)
+                    pn[o] = msn[i][v];
+                if (split == 0)
+                    a.partial[(size_t)3 * a.S * slab + o] = mctr;
+            }
+    }
+#pragma unroll
+    for (int oo = 0; oo < LO && !MF; ++oo) {
         const size_t o = (size_t)lane_o(oo) * a.Kpad + k0;
         *reinterpret_cast<float4 *>(pt + o) = make_float4(at[oo][0], at[oo][1], at[oo][2], at[oo][3]);
         *reinterpret_cast<float4 *>(pw + o) = make_float4(aw[oo][0], aw[oo][1], aw[oo][2], aw[oo][3]);
@@ -1014,7 +1085,13 @@ template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
     dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
-    if (t.fast) {
+    constexpr bool L2M = MODE != SIM_MODE_L1;
+    if (t.fast && L2M) {
+        if (t.WO == 2)
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true, L2M>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, true, L2M>), grid, dim3(kThreads), 0, s, a);
+    } else if (t.fast) {
         if (t.WO == 2)
             hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true>), grid, dim3(kThreads), 0, s, a);
         else
