@@ -598,10 +598,15 @@ struct GradPArgs {
 // v_mfma_f32_32x32x2_f32 tiles per moment, templates = rows, patch elements = columns, two pixels per instruction;
 // the operands come from the same LDS chunks (one ds_read_b32 each: lane = (row or column, pixel parity)).  The
 // centre is then per (wave, patch element): the mean over the wave's 64 templates.
-template <int MODE, int WO, bool MOM, bool MF = false>
+// ROW (with MF; output width a multiple of the chunk of 32 pixels, so a chunk is a piece of one output row): g and
+// the patch elements are staged row by row - a thread loads four consecutive pixels of a template row (one 16-byte
+// load) or of a patch-element row (bounds per element, constants per row) - into [row][pixel] LDS tiles of pitch
+// 34, instead of element by element with the im2col arithmetic per element.
+template <int MODE, int WO, bool MOM, bool MF = false, bool ROW = false>
 __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const GradPArgs a)
 {
     static_assert(!MF || (MOM && MODE != SIM_MODE_L1), "the matrix-core form computes the moments of the L2 modes");
+    static_assert(!ROW || MF, "row staging feeds the matrix-core form");
     constexpr bool MOM2 = MOM && MODE != SIM_MODE_L1;   // moment form of the L2 modes
     constexpr bool SGN = MOM && MODE == SIM_MODE_L1;    // scaled-sign form of L1
     constexpr int WK = kWaves / WO;
@@ -609,8 +614,9 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     constexpr bool NORM = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool IGN = MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
     constexpr bool L1 = MODE == SIM_MODE_L1;
-    __shared__ __attribute__((aligned(16))) float gs[2][OWG / 4 * PCP * 4];
-    __shared__ __attribute__((aligned(16))) float xs[2][KWG / 4 * PCP * 4];
+    constexpr int PR = 34;  // row pitch of the [row][pixel] tiles: rows r and r + 1 start two banks apart
+    __shared__ __attribute__((aligned(16))) float gs[2][ROW ? OWG * PR : OWG / 4 * PCP * 4];
+    __shared__ __attribute__((aligned(16))) float xs[2][ROW ? KWG * PR : KWG / 4 * PCP * 4];
     __shared__ int ktab[KWG * 2];
 
     const int tid = threadIdx.x;
@@ -774,6 +780,121 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
 
     const int chunk_begin = split * a.cps;
     const int chunk_end = min((split + 1) * a.cps, a.nchunks);
+    // matrix-core form, one chunk: two pixels per step, rows = templates (g at ga, second tile a1_off further),
+    // columns = patch elements (xc, xc^2, keep from xb); `ps` floats from pixel to pixel; the reads of the next step
+    // are issued before this step's matrix instructions
+    auto mfma_steps = [&](const float *ga_, int a1_off, const float *xb_, int ps) {
+        float a0 = ga_[0], a1 = ga_[a1_off], xv_ = xb_[0];
+#pragma unroll 4
+        for (int p = 0; p < PC; p += 2) {
+            const int pn = p + 2 < PC ? p + 2 : p;
+            const float na0 = ga_[pn * ps], na1 = ga_[a1_off + pn * ps], nx = xb_[pn * ps];
+            const bool ok = !IGN || xv_ == xv_;
+            const float xc = ok ? xv_ - mctr : 0.0f;
+            const float x2 = xc * xc;
+            ms1[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, xc, ms1[0], 0, 0, 0);
+            ms1[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, xc, ms1[1], 0, 0, 0);
+            ms2[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, x2, ms2[0], 0, 0, 0);
+            ms2[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, x2, ms2[1], 0, 0, 0);
+            if constexpr (IGN) {
+                const float keep1 = ok ? 1.0f : 0.0f;
+                msn[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, keep1, msn[0], 0, 0, 0);
+                msn[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, keep1, msn[1], 0, 0, 0);
+            }
+            a0 = na0; a1 = na1; xv_ = nx;
+        }
+    };
+    if constexpr (ROW) {
+        constexpr int RG = OWG / 32, RX = KWG / 32;
+        const int rrow = tid >> 3, jq = tid & 7;   // rows rrow + 32 r; pixels 4 jq .. 4 jq + 3 of the chunk
+        int kch[RX], kdh[RX], kdw[RX];             // this thread's patch-element rows: channel (-1: past K), tap
+#pragma unroll
+        for (int r = 0; r < RX; ++r) {
+            const int k = k_wg + rrow + 32 * r;
+            const int c = k / bhw, rem = k - c * bhw;
+            kch[r] = k < a.K ? c : -1;
+            kdh[r] = rem / a.bw;
+            kdw[r] = rem - kdh[r] * a.bw;
+        }
+        float4 rg[RG];
+        float rx[RX][4], gsum[RG];
+#pragma unroll
+        for (int r = 0; r < RG; ++r)
+            gsum[r] = 0.0f;
+        auto row_load = [&](int chunk) {
+            // the chunk's first pixel (uniform): image, output row, first output column
+            const long long q0 = (long long)chunk * PC;
+            const int b = (int)(q0 / ohow);
+            const int pix0 = (int)(q0 - (long long)b * ohow);
+            const int yo = pix0 / a.ow, xo0 = pix0 - yo * a.ow;
+#pragma unroll
+            for (int r = 0; r < RG; ++r) {
+                const int o = o_wg + rrow + 32 * r;
+                rg[r] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                if (o < a.O)
+                    rg[r] = *reinterpret_cast<const float4 *>(a.g + ((size_t)b * a.O + o) * ohow + pix0 + 4 * jq);
+            }
+#pragma unroll
+            for (int r = 0; r < RX; ++r) {
+                const int iy = yo * a.sh - a.ph + kdh[r];
+                const bool row_ok = kch[r] >= 0 && iy >= 0 && iy < a.H;
+                const float fill = kch[r] >= 0 ? a.oob : 0.0f;
+                const float *row = a.x + (((size_t)b * a.C + max(kch[r], 0)) * a.H + (row_ok ? iy : 0)) * a.W;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int ix = (xo0 + 4 * jq + e) * a.sw - a.pw + kdw[r];
+                    rx[r][e] = fill;
+                    if (row_ok && ix >= 0 && ix < a.W)
+                        rx[r][e] = row[ix];
+                }
+            }
+        };
+        auto row_store = [&](int buf) {
+#pragma unroll
+            for (int r = 0; r < RG; ++r) {
+                float2 *d = reinterpret_cast<float2 *>(gs[buf] + (rrow + 32 * r) * PR + 4 * jq);
+                d[0] = make_float2(rg[r].x, rg[r].y);
+                d[1] = make_float2(rg[r].z, rg[r].w);
+                if constexpr (!IGN)
+                    gsum[r] += (rg[r].x + rg[r].y) + (rg[r].z + rg[r].w);
+            }
+#pragma unroll
+            for (int r = 0; r < RX; ++r) {
+                float2 *d = reinterpret_cast<float2 *>(xs[buf] + (rrow + 32 * r) * PR + 4 * jq);
+                d[0] = make_float2(rx[r][0], rx[r][1]);
+                d[1] = make_float2(rx[r][2], rx[r][3]);
+            }
+        };
+        if (chunk_begin < chunk_end) {
+            row_load(chunk_begin);
+            row_store(0);
+        }
+        __syncthreads();
+        for (int chunk = chunk_begin; chunk < chunk_end; ++chunk) {
+            const int buf = (chunk - chunk_begin) & 1;
+            const bool more = chunk + 1 < chunk_end;
+            if (more)
+                row_load(chunk + 1);   // in flight while this chunk is used
+            mfma_steps(gs[buf] + (wo * 64 + mcol) * PR + mhalf, 32 * PR, xs[buf] + (wk * 32 + mcol) * PR + mhalf, 1);
+            if (more)
+                row_store(buf ^ 1);
+            __syncthreads();  // the other buffer is complete; nobody reads this one any more
+        }
+        if constexpr (!IGN) {
+            // sum of g per template: the 8 pixel groups of a row, in group order; the finish kernel reads
+            // patch-element tile 0's copy
+#pragma unroll
+            for (int r = 0; r < RG; ++r)
+                gs[0][(rrow + 32 * r) * PR + jq] = gsum[r];
+            __syncthreads();
+            if (tid < OWG) {
+                float sum = 0.0f;
+                for (int q = 0; q < 8; ++q)
+                    sum += gs[0][tid * PR + q];
+                a.partial[((size_t)2 * a.S + split) * (size_t)a.Opad * a.Kpad + (size_t)(o_wg + tid) * a.Kpad + k_wg] = sum;
+            }
+        }
+    }
     float4 gv[GR], xv[XR];
     __syncthreads();  // ktab written
     auto has_nan = [](const float4 (&xv)[XR]) {
@@ -784,7 +905,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         return any;
     };
     bool nan_chunk = false;  // scaled-sign form: the chunk in use holds a NaN input (uniform for the workgroup)
-    if (chunk_begin < chunk_end) {
+    if (chunk_begin < chunk_end && !ROW) {
         load_chunk(chunk_begin, gv, xv);
         store_chunk(0, gv, xv);
         if constexpr (SGN)
@@ -794,7 +915,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         nan_chunk = __syncthreads_or(nan_chunk);
     else
         __syncthreads();
-    for (int chunk = chunk_begin; chunk < chunk_end; ++chunk) {
+    for (int chunk = chunk_begin; chunk < chunk_end && !ROW; ++chunk) {
         const int buf = (chunk - chunk_begin) & 1;
         const bool more = chunk + 1 < chunk_end;
         if (more)
@@ -900,29 +1021,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             }
         };
         if constexpr (MF) {
-            // two pixels per step: rows = templates (g), columns = patch elements (xc, xc^2, keep); the reads of
-            // the next step are issued before this step's matrix instructions
-            const float *ga_ = gs[buf] + ((size_t)(wo * 16 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3);
-            const float *xb_ = xs[buf] + ((size_t)(wk * 8 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3);
-            float a0 = ga_[0], a1 = ga_[8 * PCP * 4], xv_ = xb_[0];
-#pragma unroll 4
-            for (int p = 0; p < PC; p += 2) {
-                const int pn = p + 2 < PC ? p + 2 : p;
-                const float na0 = ga_[pn * 4], na1 = ga_[8 * PCP * 4 + pn * 4], nx = xb_[pn * 4];
-                const bool ok = !IGN || xv_ == xv_;
-                const float xc = ok ? xv_ - mctr : 0.0f;
-                const float x2 = xc * xc;
-                ms1[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, xc, ms1[0], 0, 0, 0);
-                ms1[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, xc, ms1[1], 0, 0, 0);
-                ms2[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, x2, ms2[0], 0, 0, 0);
-                ms2[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, x2, ms2[1], 0, 0, 0);
-                if constexpr (IGN) {
-                    const float keep1 = ok ? 1.0f : 0.0f;
-                    msn[0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, keep1, msn[0], 0, 0, 0);
-                    msn[1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, keep1, msn[1], 0, 0, 0);
-                }
-                a0 = na0; a1 = na1; xv_ = nx;
-            }
+            mfma_steps(gs[buf] + ((size_t)(wo * 16 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 8 * PCP * 4,
+                       xs[buf] + ((size_t)(wk * 8 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 4);
         } else if (SGN && !nan_chunk) {
             pixels(compute_sgn);
         } else if (SGN) {
@@ -975,7 +1075,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
                     make_float4(ctr[0], ctr[1], ctr[2], ctr[3]);
         }
     }
-    if constexpr (MOM2 && !IGN) {
+    if constexpr (MOM2 && !IGN && !ROW) {
         // pixel slots -> one sum per template, in slot order; the finish kernel reads patch-element tile 0's copy
         // (the loop's last barrier has passed: nobody reads gs any more)
 #pragma unroll
@@ -1071,12 +1171,15 @@ GpTiling gp_tiling(const SimPlan &p)
     const long long npix = (long long)p.B * p.oh * p.ow;
     t.nchunks = (int)((npix + PC - 1) / PC);
     const int tiles = t.n_otiles * t.n_ktiles;
-    int S = std::max(1, 1024 / tiles);
+    t.fast = !p.exact_terms;
+    t.moment = t.fast && p.mode != SIM_MODE_L1;
+    // workgroups per launch: two rounds of 2 per compute unit for the vector forms, more and shorter ones for the
+    // matrix-core form (measured on 256x64x32x32, 128 templates 3x3: 0.85 / 0.86 / 0.80 / 0.83 ms for 512 / 1024 /
+    // 1536 / 2048)
+    int S = std::max(1, (t.moment ? 1536 : 1024) / tiles);
     S = std::min(S, std::max(1, t.nchunks));
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
-    t.fast = !p.exact_terms;
-    t.moment = t.fast && p.mode != SIM_MODE_L1;
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
     return t;
 }
@@ -1086,7 +1189,12 @@ hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
     dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
     constexpr bool L2M = MODE != SIM_MODE_L1;
-    if (t.fast && L2M) {
+    if (t.fast && L2M && a.ow % PC == 0) {
+        if (t.WO == 2)
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true, L2M, L2M>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 1, true, L2M, L2M>), grid, dim3(kThreads), 0, s, a);
+    } else if (t.fast && L2M) {
         if (t.WO == 2)
             hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true, L2M>), grid, dim3(kThreads), 0, s, a);
         else

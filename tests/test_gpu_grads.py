@@ -440,3 +440,21 @@ def test_similarity_l1_params_grad_scaled_sign_form_equals_the_term_by_term_form
     ok = ~np.isnan(want_dw)
     assert_grad_close(fast[0], want_dt, true_dt, "templates grad")
     assert_grad_close(np.where(ok, fast[1], 0), np.where(ok, want_dw, 0), np.where(ok, true_dw, 0), "weights grad")
+
+
+@pytest.mark.parametrize("func,norm,ign", [("L2", False, False), ("L2", True, False), ("L2", True, True)])
+@pytest.mark.parametrize("case", [
+    dict(shape=(3, 5, 9, 32), O=70, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # ow = 32, ragged O and K
+    dict(shape=(2, 3, 12, 64), O=9, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),     # ow = 32 through stride 2
+    dict(shape=(1, 16, 6, 66), O=130, blocks=[2, 3], strides=[1, 1], padding=[0, 0]),   # ow = 64, two chunks per row
+    dict(shape=(2, 2, 5, 30), O=4, blocks=[1, 5], strides=[1, 1], padding=[0, 3]),      # ow = 32 with padding beyond the image
+])
+def test_similarity_params_grad_row_staged_matrix_form(pkg, case, func, norm, ign):
+    """Output widths that are multiples of 32: the L2 parameter gradients stage g and the patch elements row by
+    row for the matrix-core moments."""
+    x, t, w = sim_inputs(41, case["shape"], case["O"], case["blocks"], nan_frac=0.15 if ign else 0.0)
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+              normalization_term=norm, ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else -0.75)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    assert out.shape[3] % 32 == 0
+    check_sim_grads(pkg, x, t, w, **kw)
