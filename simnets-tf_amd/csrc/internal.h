@@ -48,6 +48,12 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
                size_t workspace_bytes, void *stream);
 
 // Backward operators (similarity_grad.hip, mex_grad.hip).  `stream` is a hipStream_t.
+// Input gradient of the L2 modes at stride 1 on the matrix cores (similarity_mfma.hip)
+bool sim_mfma_grad_input_supported(const SimPlan &p);
+size_t sim_mfma_grad_input_workspace_bytes(const SimPlan &p);
+int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                               const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
+                               void *stream);
 size_t sim_grad_input_workspace_bytes(const SimPlan &p);
 size_t sim_grad_params_workspace_bytes(const SimPlan &p);
 int sim_grad_input(const SimPlan &p, const float *input, const float *templates, const float *weights,

@@ -470,6 +470,8 @@ hipError_t gx_launch_phase(const GradXArgs &a, const GxTiling &t, hipStream_t s)
 
 size_t sim_grad_input_workspace_bytes(const SimPlan &p)
 {
+    if (sim_mfma_grad_input_supported(p))
+        return sim_mfma_grad_input_workspace_bytes(p);
     if (!gx_all_phases_fit(p))
         return 0;
     size_t total = 0;
@@ -493,6 +495,9 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
     const int ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     const long long n_in = (long long)p.B * p.C * p.H * p.W;
 
+    if (sim_mfma_grad_input_supported(p))
+        return sim_mfma_grad_input_launch(p, input, templates, weights, output_grad, input_grad, workspace,
+                                          workspace_bytes, stream);
     if (!gx_all_phases_fit(p)) {
         const int blocks = (int)std::min<long long>((n_in + 255) / 256, 1 << 20);
         hipLaunchKernelGGL(sim_grad_input_gather_kernel, dim3(blocks), dim3(256), 0, s, output_grad, input, templates,

@@ -51,6 +51,9 @@ struct MfmaArgs {
     const float *pm;    // [step][type][half][Opad]
     const float *bias;  // [Opad]
     const float *ctr;   // [C] per-channel shift
+    const float *x;     // input-gradient variant: the forward op's input (one value per output element)
+    int x_channels;     // ... and its channel count (rows of the product that exist)
+    int ignore_nan;     // ... NaN inputs get gradient 0
     int B, C, H, W, O, Opad, oh, ow, npix;
     int bh, bw, sh, sw, ph, pw;
     int tiles;          // workgroup pixel tiles per image
@@ -58,6 +61,15 @@ struct MfmaArgs {
     float oob;
 };
 
+// GRAD: the same contraction machinery computes the input gradient of the L2 modes at stride 1.  With
+// P0 = s w (t - c), P1 = s w (s = 2, or 1 with the normalization term; c = the channel's centre),
+//   dX[b,ch,y,x] = sum_{m,dh,dw} g[b,m,y+ph-dh,x+pw-dw] (P0 - (X - c) P1)[m,ch,dh,dw] = A - (X[b,ch,y,x] - c) B,
+// two products over (m, dh, dw) whose right operand is the output gradient read like an input image padded by
+// (bh-1-ph, bw-1-pw) with zeros, taps flipped (src/kernels/similarity_grad_kernel_cpu.cpp:148-270 computes the
+// same sums term by term).  Here the "image" is g (its channels are the templates), the rows are input channels:
+// row tile 0 of a wave accumulates A and row tile 1 accumulates B for the same 32 channels, so a lane ends up
+// with both values of an element and combines them with X at the store.
+template <bool GRAD>
 __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
 {
     extern __shared__ float lds[];
@@ -75,7 +87,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
     const int nrows = p_last / a.ow - h_first + 1;
     const int TR = (nrows - 1) * a.sh + a.bh;
     const int in_row0 = h_first * a.sh - a.ph;
-    const int mbase = blockIdx.y * WG_TPL + wm * (RM * 32);
+    const int mbase = GRAD ? blockIdx.y * (WG_TPL / 2) + wm * 32 : blockIdx.y * WG_TPL + wm * (RM * 32);
 
     // per pixel tile: LDS address of this lane's pixel (k-pair half folded in)
     int xbase[RP], pix[RP];
@@ -94,7 +106,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
         floatx16 init;
 #pragma unroll
         for (int v = 0; v < 16; ++v)
-            init[v] = a.bias[mbase + i * 32 + 8 * (v / 4) + 4 * half + (v % 4)];
+            init[v] = GRAD ? 0.0f : a.bias[mbase + i * 32 + 8 * (v / 4) + 4 * half + (v % 4)];
 #pragma unroll
         for (int j = 0; j < RP; ++j)
             acc[i][j] = init;
@@ -109,6 +121,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
     auto load_params = [&](const float *p, float (&w_)[RM], float (&t_)[RM]) {
 #pragma unroll
         for (int i = 0; i < RM; ++i) {
+            if (GRAD && i > 0)
+                break;  // one row tile of parameters: type 0 feeds accumulator tile 0, type 1 tile 1
             w_[i] = p[i * 32];
             t_[i] = p[2 * a.Opad + i * 32];
         }
@@ -124,7 +138,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
         const int ccn = min(a.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
-        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, a.chan_lds, a.oob, a.ctr, tp);
+        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, a.chan_lds, a.oob,
+                                                     GRAD ? nullptr : a.ctr, tp);
         __syncthreads();
 
         // steps of this chunk in (channel pair, dh, dw) order; the pixel operand of step s+1 and the
@@ -160,21 +175,32 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
             load_params(pm, pw_nn, pt_nn);
             pm += step_stride;
             __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int j = 0; j < RP; ++j)
-                x2[j] = x[j] * x[j];
-#pragma unroll
-            for (int i = 0; i < RM; ++i)
+            if constexpr (GRAD) {
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[i], x2[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-            for (int i = 0; i < RM; ++i)
+                    acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[0], x[j], acc[0][j], 0, 0, 0);
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[i], x[j], acc[i][j], 0, 0, 0);
+                    acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[0], x[j], acc[1][j], 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int j = 0; j < RP; ++j)
+                    x2[j] = x[j] * x[j];
+#pragma unroll
+                for (int i = 0; i < RM; ++i)
+#pragma unroll
+                    for (int j = 0; j < RP; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[i], x2[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+                for (int i = 0; i < RM; ++i)
+#pragma unroll
+                    for (int j = 0; j < RP; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[i], x[j], acc[i][j], 0, 0, 0);
+            }
 #pragma unroll
             for (int i = 0; i < RM; ++i) {
+                if (GRAD && i > 0)
+                    break;
                 pw_cur[i] = pw_nxt[i]; pt_cur[i] = pt_nxt[i];
                 pw_nxt[i] = pw_nn[i];  pt_nxt[i] = pt_nn[i];
             }
@@ -182,8 +208,30 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
         }
     }
 
-    // ---- store: lane holds, per tile, 16 templates of one pixel ----
     const size_t plane = (size_t)a.npix;
+    if constexpr (GRAD) {
+        // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel ----
+        float *ob = a.out + (size_t)b * a.x_channels * plane;
+        const float *xb = a.x + (size_t)b * a.x_channels * plane;
+#pragma unroll
+        for (int j = 0; j < RP; ++j) {
+            if (pix[j] > p_last)
+                continue;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int ch = mbase + 8 * (v / 4) + 4 * half + (v % 4);
+                if (ch >= a.x_channels)
+                    continue;
+                const float xin = xb[(size_t)ch * plane + pix[j]];
+                float d = __builtin_fmaf(-(xin - a.ctr[ch]), acc[1][j][v], acc[0][j][v]);
+                if (a.ignore_nan && xin != xin)
+                    d = 0.0f;
+                ob[(size_t)ch * plane + pix[j]] = d;
+            }
+        }
+        return;
+    }
+    // ---- store: lane holds, per tile, 16 templates of one pixel ----
     float *ob = a.out + (size_t)b * a.O * plane;
 #pragma unroll
     for (int j = 0; j < RP; ++j) {
@@ -276,6 +324,32 @@ __global__ __launch_bounds__(256) void mfma_bias_kernel(const float *__restrict_
         bias[m] = -red[0];
 }
 
+// Input-gradient variant: pm[step][type][half][Cpad], step = ((mpair * bh) + dh) * bw + dw over the flipped taps,
+// template m = 2 * mpair + half, row = input channel: type 0 = s w (t - ctr), type 1 = s w.
+__global__ void mfma_grad_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
+                                      const float *__restrict__ ctr, int O, int C, int Cpad, int bh, int bw,
+                                      float scale, long long total, float *__restrict__ pm)
+{
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int c = (int)(i % Cpad);
+        long long r = i / Cpad;
+        const int half = (int)(r & 1); r >>= 1;
+        const int type = (int)(r & 1); r >>= 1;
+        const int dw = (int)(r % bw); r /= bw;
+        const int dh = (int)(r % bh);
+        const int mpair = (int)(r / bh);
+        const int m = 2 * mpair + half;
+        float v = 0.0f;
+        if (m < O && c < C) {
+            const size_t idx = (((size_t)m * C + c) * bh + (bh - 1 - dh)) * bw + (bw - 1 - dw);
+            const float w = scale * weights[idx];
+            v = type == 0 ? w * (templates[idx] - ctr[c]) : w;
+        }
+        pm[i] = v;
+    }
+}
+
 struct MfmaTiling {
     int Opad, steps, TC, TRmax, chan_lds, CC;
     bool ok;
@@ -347,7 +421,85 @@ int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates
     a.oob = p.oob;
     dim3 grid((unsigned)(p.B * a.tiles), (unsigned)(t.Opad / WG_TPL));
     const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
-    hipLaunchKernelGGL(sim_mfma_kernel, grid, dim3(kThreads), lds_bytes, s, a);
+    hipLaunchKernelGGL(sim_mfma_kernel<false>, grid, dim3(kThreads), lds_bytes, s, a);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+namespace {
+
+// The product the input gradient needs, in the forward kernel's terms: the output gradient is the image (its
+// channels are the templates), the input grid is the output grid, padding (bh-1-ph, bw-1-pw), stride 1.
+MfmaTiling mfma_grad_tiling(const SimPlan &q)
+{
+    MfmaTiling t = mfma_tiling(q);
+    // a workgroup covers 64 rows (channels) here: 2 waves x one 32-row tile for each of the two products
+    t.Opad = (q.O + WG_TPL / 2 - 1) / (WG_TPL / 2) * (WG_TPL / 2);
+    t.pm_floats = (size_t)(t.steps + 2) * 4 * t.Opad;
+    return t;
+}
+
+SimPlan grad_as_forward(const SimPlan &p)
+{
+    SimPlan q = p;
+    q.C = p.O; q.H = p.oh; q.W = p.ow;
+    q.O = p.C; q.oh = p.H; q.ow = p.W;
+    q.ph = p.bh - 1 - p.ph; q.pw = p.bw - 1 - p.pw;
+    q.K = p.O * p.bh * p.bw;
+    return q;
+}
+
+}  // namespace
+
+bool sim_mfma_grad_input_supported(const SimPlan &p)
+{
+    if (p.mode == SIM_MODE_L1 || p.exact_terms || p.sh != 1 || p.sw != 1 || p.ph > p.bh - 1 || p.pw > p.bw - 1)
+        return false;
+    // 32 channels per row tile, two templates per step: smaller problems leave the tiles mostly empty
+    if (p.C < 24 || p.O < 8 || p.B == 0)
+        return false;
+    return mfma_grad_tiling(grad_as_forward(p)).ok;
+}
+
+size_t sim_mfma_grad_input_workspace_bytes(const SimPlan &p)
+{
+    const MfmaTiling t = mfma_grad_tiling(grad_as_forward(p));
+    return align_up(t.pm_floats * sizeof(float), 256) + align_up((size_t)p.C * sizeof(float), 256);
+}
+
+int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                               const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
+                               void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const SimPlan q = grad_as_forward(p);
+    const MfmaTiling t = mfma_grad_tiling(q);
+    if (!t.ok)
+        return SIMNETS_ERR_ALGO;
+    if (workspace_bytes < sim_mfma_grad_input_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+    char *ws = reinterpret_cast<char *>(workspace);
+    float *pm = reinterpret_cast<float *>(ws);
+    float *ctr = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256));
+    const bool norm = p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+    hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, p.bh * p.bw, ctr);
+    const long long total = (long long)t.pm_floats;
+    hipLaunchKernelGGL(mfma_grad_pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 8192)), dim3(256),
+                       0, s, templates, weights, ctr, p.O, p.C, t.Opad, p.bh, p.bw, norm ? 1.0f : 2.0f, total, pm);
+    if (hipGetLastError() != hipSuccess)
+        return SIMNETS_ERR_HIP;
+
+    MfmaArgs a;
+    a.in = output_grad; a.out = input_grad; a.pm = pm; a.bias = nullptr; a.ctr = ctr;
+    a.x = input; a.x_channels = p.C; a.ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+    a.B = q.B; a.C = q.C; a.H = q.H; a.W = q.W; a.O = q.O; a.Opad = t.Opad;
+    a.oh = q.oh; a.ow = q.ow; a.npix = q.oh * q.ow;
+    a.bh = q.bh; a.bw = q.bw; a.sh = 1; a.sw = 1; a.ph = q.ph; a.pw = q.pw;
+    a.tiles = (a.npix + WG_PIX - 1) / WG_PIX;
+    a.TC = t.TC; a.TRmax = t.TRmax; a.chan_lds = t.chan_lds; a.CC = t.CC;
+    a.oob = 0.0f;
+    dim3 grid((unsigned)(q.B * a.tiles), (unsigned)(t.Opad / (WG_TPL / 2)));
+    const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
+    hipLaunchKernelGGL(sim_mfma_kernel<true>, grid, dim3(kThreads), lds_bytes, s, a);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
