@@ -458,3 +458,31 @@ def test_similarity_params_grad_row_staged_matrix_form(pkg, case, func, norm, ig
     out = orc.similarity_fwd(x, t, w, **kw)
     assert out.shape[3] % 32 == 0
     check_sim_grads(pkg, x, t, w, **kw)
+
+
+@pytest.mark.parametrize("func,norm,ign", [("L2", False, False), ("L2", True, False), ("L2", True, True)])
+@pytest.mark.parametrize("case", [
+    dict(shape=(2, 40, 13, 17), O=9, blocks=[3, 3], padding=[1, 1]),       # ragged channel tile, odd template count
+    dict(shape=(1, 70, 9, 40), O=33, blocks=[2, 4], padding=[0, 3]),       # two channel tiles, asymmetric block
+    dict(shape=(3, 24, 20, 20), O=16, blocks=[5, 5], padding=[4, 0]),      # padding = block - 1
+    dict(shape=(2, 32, 6, 300), O=12, blocks=[1, 3], padding=[0, 1]),      # several pixel tiles per row
+])
+def test_similarity_input_grad_matrix_form(pkg, case, func, norm, ign):
+    """Stride 1, at least 24 channels: the L2 modes' input gradient is A - (x - c) B with both products on the
+    matrix cores.  Data sit away from zero (the centre c matters); algo='direct' takes the term-by-term kernel."""
+    g = np.random.default_rng(52)
+    x = (3.0 + g.normal(size=case["shape"])).astype(np.float32)
+    t = (3.0 + g.normal(size=(case["O"], case["shape"][1]) + tuple(case["blocks"]))).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    if ign:
+        x[g.random(size=x.shape) < 0.15] = np.nan
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=[1, 1], padding=case["padding"],
+              normalization_term=norm, ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else 1.5)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = g.normal(size=out.shape).astype(np.float32)
+    want = orc.similarity_input_grad(x, t, w, og, **kw)
+    true = orc.similarity_input_grad(*f64(x, t, w, og), **kw)
+    for algo in (None, "direct"):
+        dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), algo=algo, **kw).cpu().numpy()
+        assert np.array_equal(np.isnan(dx), np.isnan(want))
+        assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad (%s)" % algo)
