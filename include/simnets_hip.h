@@ -124,7 +124,10 @@ int simnets_hip_similarity_grad_workspace_bytes(const simnets_similarity_attrs *
 /* REGISTER_OP("SimilarityInputGrad") (src/ops/similarity_op.cpp:141-156): replaces
  * SimilarityInputGradKernelGPU<float>::Compute (src/kernels/similarity_grad_kernel_gpu.cu), i.e. per image
  * im2col_3d_gpu + ggemm_readc_gpu<TRANSPOSE_A> with sim_*_backward_bottom + col2im_3d_gpu.
- * output_grad has the forward output's shape, input_grad the input's.  attrs->algo is ignored. */
+ * output_grad has the forward output's shape, input_grad the input's.  attrs->algo: SIMNETS_ALGO_DIRECT sums
+ * the reference's terms one by one in every case; otherwise the L2 modes at stride 1 with 24 channels or more
+ * evaluate A - (x - c) B with A = sum g s w (t - c), B = sum g s w on the fp32 matrix cores (same sum, other
+ * rounding; c = the channel's mean template value). */
 int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
                                       const int templates_shape[4], const int weights_shape[4], const float *input,
                                       const float *templates, const float *weights, const float *output_grad,
@@ -133,7 +136,11 @@ int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, con
 /* REGISTER_OP("SimilarityParametersGrad") (src/ops/similarity_op.cpp:158-174): replaces
  * SimilarityParametersGradKernelGPU<float>::Compute, i.e. per image im2col_3d_gpu + ggemm_readc_gpu with
  * sim_*_backward_weights accumulated over the batch + deinterlace.  templates_grad and weights_grad have
- * the templates' shape.  The sums over pixels are formed in a fixed order: results are reproducible. */
+ * the templates' shape.  The sums over pixels are formed in a fixed order: results are reproducible.
+ * attrs->algo: SIMNETS_ALGO_DIRECT sums the reference's terms one by one; otherwise the L2 modes accumulate the
+ * moments sum g (x - c), sum g (x - c)^2, sum g about a centre c near the templates on the fp32 matrix cores and
+ * combine them in double precision, and L1 takes sign and magnitude from 2^64 (x - t) (bit-identical to the
+ * term-by-term sums unless 0 < |x - t| < 2^-64). */
 int simnets_hip_similarity_params_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
                                        const int templates_shape[4], const int weights_shape[4], const float *input,
                                        const float *templates, const float *weights, const float *output_grad,
