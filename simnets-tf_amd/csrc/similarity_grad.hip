@@ -253,7 +253,10 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
     }
 }
 
-// Fallback for geometries whose g rows do not fit the LDS budget: one input element per thread.
+// One input element per thread: the taps whose window covers the element outside, the templates inside (no
+// divisions in the inner loop; the threads of a wave read neighbouring g values).  Used for geometries whose g
+// rows do not fit the LDS budget and for inputs of one or two channels (the first layer of the reference's
+// networks), where the channel lanes of the tiled kernel would idle and each stride phase costs two launches.
 __global__ __launch_bounds__(256) void sim_grad_input_gather_kernel(const float *__restrict__ g,
                                                                     const float *__restrict__ x,
                                                                     const float *__restrict__ templates,
@@ -264,6 +267,7 @@ __global__ __launch_bounds__(256) void sim_grad_input_gather_kernel(const float 
                                                                     int ignore_nan)
 {
     const long long total = (long long)B * C * H * W;
+    const size_t oplane = (size_t)oh * ow, tplane = (size_t)C * bh * bw;
     for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
          idx += (long long)gridDim.x * blockDim.x) {
         const int xx = (int)(idx % W);
@@ -275,18 +279,19 @@ __global__ __launch_bounds__(256) void sim_grad_input_gather_kernel(const float 
         const float xin = x[idx];
         float acc = 0.0f;
         if (!(ignore_nan && !(xin == xin))) {
-            for (int o = 0; o < O; ++o)
-                for (int i = 0; i < bh; ++i) {
-                    const int ty = yy + ph - i;
-                    if (ty < 0 || ty % sh != 0 || ty / sh >= oh)
+            for (int i = 0; i < bh; ++i) {
+                const int ty = yy + ph - i;
+                if (ty < 0 || ty % sh != 0 || ty / sh >= oh)
+                    continue;
+                for (int j = 0; j < bw; ++j) {
+                    const int tx = xx + pw - j;
+                    if (tx < 0 || tx % sw != 0 || tx / sw >= ow)
                         continue;
-                    for (int j = 0; j < bw; ++j) {
-                        const int tx = xx + pw - j;
-                        if (tx < 0 || tx % sw != 0 || tx / sw >= ow)
-                            continue;
-                        const float gv = g[(((size_t)b * O + o) * oh + ty / sh) * ow + tx / sw];
-                        const size_t pi = (((size_t)o * C + c) * bh + i) * bw + j;
-                        const float t = templates[pi], w = weights[pi];
+                    const float *gp = g + (size_t)b * O * oplane + (size_t)(ty / sh) * ow + tx / sw;
+                    const size_t pi = ((size_t)c * bh + i) * bw + j;
+                    for (int o = 0; o < O; ++o) {
+                        const float gv = gp[(size_t)o * oplane];
+                        const float t = templates[(size_t)o * tplane + pi], w = weights[(size_t)o * tplane + pi];
                         const float d = t - xin;
                         float u;
                         if (l1)
@@ -296,6 +301,7 @@ __global__ __launch_bounds__(256) void sim_grad_input_gather_kernel(const float 
                         acc = __builtin_fmaf(gv, u, acc);
                     }
                 }
+            }
         }
         dx[idx] = acc;
     }
@@ -468,11 +474,14 @@ hipError_t gx_launch_phase(const GradXArgs &a, const GxTiling &t, hipStream_t s)
 
 }  // namespace
 
+// the one-element-per-thread kernel: rows too long for the LDS tile, or one or two input channels
+static bool gx_gather(const SimPlan &p) { return !gx_all_phases_fit(p) || p.C <= 2; }
+
 size_t sim_grad_input_workspace_bytes(const SimPlan &p)
 {
     if (sim_mfma_grad_input_supported(p))
         return sim_mfma_grad_input_workspace_bytes(p);
-    if (!gx_all_phases_fit(p))
+    if (gx_gather(p))
         return 0;
     size_t total = 0;
     for (int ry = 0; ry < p.sh; ++ry)
@@ -498,7 +507,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
     if (sim_mfma_grad_input_supported(p))
         return sim_mfma_grad_input_launch(p, input, templates, weights, output_grad, input_grad, workspace,
                                           workspace_bytes, stream);
-    if (!gx_all_phases_fit(p)) {
+    if (gx_gather(p)) {
         const int blocks = (int)std::min<long long>((n_in + 255) / 256, 1 << 20);
         hipLaunchKernelGGL(sim_grad_input_gather_kernel, dim3(blocks), dim3(256), 0, s, output_grad, input, templates,
                            weights, input_grad, p.B, p.C, p.H, p.W, p.O, p.oh, p.ow, p.bh, p.bw, p.sh, p.sw, p.ph,
@@ -1058,7 +1067,10 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
         for (int i = 0; i < 2; ++i)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                const size_t o = (size_t)(o_wg + wo * 64 + i * 32 + 8 * (v / 4) + 4 * mhalf + (v % 4)) * a.Kpad + mk;
+                const int orow = o_wg + wo * 64 + i * 32 + 8 * (v / 4) + 4 * mhalf + (v % 4);
+                if (orow >= a.O || mk >= a.K)
+                    continue;  // nobody reads the padding of the tile
+                const size_t o = (size_t)orow * a.Kpad + mk;
                 pt[o] = ms1[i][v];
                 pw[o] = ms2[i][v];
                 if constexpr (IGN)
@@ -1097,21 +1109,23 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     }
 }
 
-// Adds the partial sums in a fixed order and applies the pixel-independent factors.  256 threads = 32 elements x 8
-// groups: group j adds the splits j, j + 8, ..., the 8 group sums are added in group order through LDS.
+// Adds the partial sums in a fixed order and applies the pixel-independent factors.  256 threads = E elements x
+// 256 / E groups (E = 32, or 8 when there are few elements): group j adds the splits j, j + G, ..., the group sums
+// are added in group order through LDS.
 // moment != 0: the partial sums are the moments S1, S2, G of sim_grad_params_kernel<.., MOM = true>.
 __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
     const float *__restrict__ partial, const float *__restrict__ templates, const float *__restrict__ weights, int O,
-    int K, int Opad, int Kpad, int S, int mode, int moment, float fudge, float *__restrict__ dT,
+    int K, int Opad, int Kpad, int S, int mode, int moment, float fudge, int E, float *__restrict__ dT,
     float *__restrict__ dW)
 {
-    __shared__ float sm[3][8][32];
+    __shared__ float sm[3][256];
     const long long total = (long long)O * K;
     const size_t slab = (size_t)Opad * Kpad;
     const bool norm = mode == SIM_MODE_L2_NORM || mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     const bool ign = mode == SIM_MODE_L2_NORM_IGNORE_NAN;
-    const int e = threadIdx.x & 31, grp = threadIdx.x >> 5;
-    const long long idx = (long long)blockIdx.x * 32 + e;
+    const int G = 256 / E;
+    const int e = threadIdx.x % E, grp = threadIdx.x / E;
+    const long long idx = (long long)blockIdx.x * E + e;
     const bool live = idx < total;
     const int k = live ? (int)(idx % K) : 0;
     const int o = live ? (int)(idx / K) : 0;
@@ -1120,20 +1134,19 @@ __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
     const size_t gsrc = moment && !ign ? (size_t)o * Kpad : src;
     float st = 0.0f, sw = 0.0f, sn = 0.0f;
     if (live)
-        for (int s = grp; s < S; s += 8) {
+        for (int s = grp; s < S; s += G) {
             st += partial[(size_t)s * slab + src];
             sw += partial[((size_t)S + s) * slab + src];
             if (norm || moment)
                 sn += partial[((size_t)2 * S + s) * slab + gsrc];
         }
-    sm[0][grp][e] = st; sm[1][grp][e] = sw; sm[2][grp][e] = sn;
+    sm[0][threadIdx.x] = st; sm[1][threadIdx.x] = sw; sm[2][threadIdx.x] = sn;
     __syncthreads();
     if (grp != 0 || !live)
         return;
     st = sw = sn = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        st += sm[0][j][e]; sw += sm[1][j][e]; sn += sm[2][j][e];
+    for (int j = 0; j < G; ++j) {
+        st += sm[0][j * E + e]; sw += sm[1][j * E + e]; sn += sm[2][j * E + e];
     }
     if (moment) {
         const double tc = (double)templates[idx] - (double)partial[(size_t)3 * S * slab + src];
@@ -1183,6 +1196,10 @@ GpTiling gp_tiling(const SimPlan &p)
     // 1536 / 2048)
     int S = std::max(1, (t.moment ? 1536 : 1024) / tiles);
     S = std::min(S, std::max(1, t.nchunks));
+    // every split costs a prologue, an epilogue and a slab of partial sums: at least 8 chunks (256 pixels) per
+    // split as long as that still leaves two workgroups per compute unit
+    if (t.nchunks / 8 >= 512 / tiles)
+        S = std::min(S, t.nchunks / 8);
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
@@ -1256,11 +1273,12 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
     const long long total = (long long)p.O * p.K;
     if (total == 0)
         return SIMNETS_OK;
-    if ((total + 31) / 32 > 0x7fffffffLL)
+    const int E = total <= 4096 ? 8 : 32;  // few elements: more threads per element
+    if ((total + E - 1) / E > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
-    const unsigned blocks = (unsigned)((total + 31) / 32);
+    const unsigned blocks = (unsigned)((total + E - 1) / E);
     hipLaunchKernelGGL(sim_grad_params_finish_kernel, dim3(blocks), dim3(256), 0, s, a.partial, templates, weights,
-                       p.O, p.K, t.Opad, t.Kpad, t.S, p.mode, t.moment ? 1 : 0, p.fudge, templates_grad, weights_grad);
+                       p.O, p.K, t.Opad, t.Kpad, t.S, p.mode, t.moment ? 1 : 0, p.fudge, E, templates_grad, weights_grad);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

@@ -263,7 +263,7 @@ __global__ __launch_bounds__(256) void mfma_center_kernel(const float *__restric
     red[threadIdx.x] = s;
     __syncthreads();
     for (int d = 128; d > 0; d >>= 1) {
-        if (threadIdx.x < d)
+        if ((int)threadIdx.x < d)
             red[threadIdx.x] += red[threadIdx.x + d];
         __syncthreads();
     }
@@ -316,7 +316,7 @@ __global__ __launch_bounds__(256) void mfma_bias_kernel(const float *__restrict_
     red[threadIdx.x] = s;
     __syncthreads();
     for (int d = 128; d > 0; d >>= 1) {
-        if (threadIdx.x < d)
+        if ((int)threadIdx.x < d)
             red[threadIdx.x] += red[threadIdx.x + d];
         __syncthreads();
     }
