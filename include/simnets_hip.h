@@ -244,6 +244,12 @@ int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input
 int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, const float *input, float *output,
                              void *stream);
 
+/* Its gradient (what the framework's AveragePooling2D gradient times the pool area gives in the reference example,
+ * examples/mnist_ght_model_missing_data.py:60-66): input_grad [B,C,H,W] <- output_grad [B,C,H/ph,W/pw] of the
+ * element's window; elements of a dropped trailing row or column get 0. */
+int simnets_hip_sum_pool_input_grad(const int input_shape[4], int pool_h, int pool_w, const float *output_grad,
+                                    float *input_grad, void *stream);
+
 /* MEX followed by that sum pooling, as one call: output [B, M*channels_out, height_out/pool_h, width_out/pool_w]
  * = simnets_hip_sum_pool_fwd(simnets_hip_mex_fwd(...)).  The pair the reference's networks run back to back
  * (README.md:108-129: MEX with unshared_offset_region = the pooling window, then pooling).  When the offsets are

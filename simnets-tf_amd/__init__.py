@@ -13,6 +13,7 @@ from .ops import (  # noqa: F401
     mex,
     mex_output_shape,
     sum_pooling,
+    sum_pooling_input_grad,
     mex_sum_pool,
     similarity_mex_sum_pool,
     similarity_input_grad,
@@ -29,4 +30,5 @@ from . import torch_ops  # noqa: F401,E402  (registers torch.ops.simnets.*)
 from .layers import Similarity, Mex, dirichlet_init  # noqa: F401,E402
 
 __all__ = ["layers", "unsupervised", "torch_ops", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "mex_sum_pool", "similarity_mex_sum_pool", "similarity_output_shape", "mex_output_shape", "SimnetsError",
-           "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad"]
+           "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad",
+           "sum_pooling_input_grad"]

@@ -12,6 +12,7 @@ EXPORTS = [
     "simnets_hip_similarity_workspace_bytes", "simnets_hip_similarity_fwd",
     "simnets_mex_attrs_default", "simnets_mex_calc_dims", "simnets_mex_out_shape", "get_mex_offsets_nregions",
     "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
+    "simnets_hip_sum_pool_input_grad",
     "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
     "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
     "simnets_hip_mex_offsets_grad",
@@ -98,6 +99,7 @@ def lib():
         l.simnets_hip_mex_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
         l.simnets_hip_mex_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, C.c_size_t, P]
         l.simnets_hip_sum_pool_fwd.argtypes = [I4, C.c_int, C.c_int, P, P, P]
+        l.simnets_hip_sum_pool_input_grad.argtypes = [I4, C.c_int, C.c_int, P, P, P]
         l.simnets_hip_mex_sum_pool_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.c_int, C.c_int,
                                                                C.POINTER(C.c_size_t)]
         l.simnets_hip_mex_sum_pool_fwd.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int, P, P,
@@ -120,6 +122,7 @@ def lib():
         for name in ("simnets_similarity_out_shape", "simnets_hip_similarity_workspace_bytes",
                      "simnets_hip_similarity_fwd", "simnets_mex_calc_dims", "simnets_mex_out_shape",
                      "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
+                     "simnets_hip_sum_pool_input_grad",
     "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
     "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
     "simnets_hip_mex_offsets_grad",

@@ -174,6 +174,24 @@ int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, c
                            output, stream);
 }
 
+int simnets_hip_sum_pool_input_grad(const int input_shape[4], int pool_h, int pool_w, const float *output_grad,
+                                    float *input_grad, void *stream)
+{
+    if (!input_shape)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (pool_h <= 0 || pool_w <= 0 || input_shape[0] < 0 || input_shape[1] <= 0 || input_shape[2] <= 0 ||
+        input_shape[3] <= 0)
+        return SIMNETS_ERR_SHAPE;
+    if (input_shape[2] / pool_h <= 0 || input_shape[3] / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    if (input_shape[0] == 0)
+        return SIMNETS_OK;
+    if (!output_grad || !input_grad)
+        return SIMNETS_ERR_NULL_POINTER;
+    return sum_pool_grad_launch(input_shape[0], input_shape[1], input_shape[2], input_shape[3], pool_h, pool_w,
+                                output_grad, input_grad, stream);
+}
+
 int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
                                              int pool_w, size_t *bytes)
 {

@@ -70,6 +70,8 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
                      void *stream);
 
 int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *input, float *output, void *stream);
+int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float *output_grad, float *input_grad,
+                         void *stream);
 // MEX followed by non-overlapping sum pooling: one fused kernel when a pooling window is one pixel of every
 // offsets region, else MEX into scratch + pooling
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw);

@@ -963,6 +963,36 @@ __global__ void sum_pool_kernel(const float *__restrict__ in, float *__restrict_
 }
 }  // namespace
 
+namespace {
+// gradient of the sum pooling: every input element of a window receives the window's gradient, the elements
+// of a dropped trailing row or column receive 0
+__global__ void sum_pool_grad_kernel(const float *__restrict__ gout, float *__restrict__ gin, long long total, int H,
+                                     int W, int Ho, int Wo, int ph, int pw)
+{
+    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (long long)gridDim.x * blockDim.x) {
+        const int w = (int)(idx % W);
+        const long long t = idx / W;
+        const int h = (int)(t % H);
+        const long long bc = t / H;
+        const int ho = h / ph, wo = w / pw;
+        gin[idx] = (ho < Ho && wo < Wo) ? gout[(bc * Ho + ho) * Wo + wo] : 0.0f;
+    }
+}
+}  // namespace
+
+int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float *output_grad, float *input_grad,
+                         void *stream)
+{
+    const long long total = (long long)B * C * H * W;
+    if (total == 0)
+        return SIMNETS_OK;
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
+    hipLaunchKernelGGL(sum_pool_grad_kernel, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       output_grad, input_grad, total, H, W, H / ph, W / pw, ph, pw);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
 int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *input, float *output, void *stream)
 {
     const int Ho = H / ph, Wo = W / pw;

@@ -650,7 +650,12 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
         return SIMNETS_OK;
     if ((n_in + 255) / 256 > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
-    if (!t.overlap) {
+    // patches that tile the input exactly (no padding, stride = block, nothing left over) write every element
+    const bool tiles_input = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 && d.stride_c == d.block_c &&
+                             d.stride_h == d.block_h && d.stride_w == d.block_w &&
+                             d.channels_out * d.block_c == p.C && d.height_out * d.block_h == p.H &&
+                             d.width_out * d.block_w == p.W;
+    if (!t.overlap && !tiles_input) {
         // every element belongs to at most one patch, which stores its gradient; the others keep 0
         hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
                            dim3(256), 0, s, input_grad, n_in);

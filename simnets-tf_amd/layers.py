@@ -61,6 +61,24 @@ class MexFunction(torch.autograd.Function):
         return gi, go, None, None
 
 
+class SumPoolFunction(torch.autograd.Function):
+    """Non-overlapping 'valid' sum pooling (`ops.sum_pooling`) with its gradient."""
+
+    @staticmethod
+    def forward(ctx, input, ph, pw):
+        ctx.shape, ctx.pool = tuple(input.shape), (ph, pw)
+        return ops.sum_pooling(input.contiguous(), (ph, pw))
+
+    @staticmethod
+    def backward(ctx, grad):
+        return ops.sum_pooling_input_grad(grad.contiguous(), ctx.shape, ctx.pool), None, None
+
+
+def sum_pooling(input, pool_size=(2, 2)):
+    """Differentiable `ops.sum_pooling`."""
+    return SumPoolFunction.apply(input, int(pool_size[0]), int(pool_size[1]))
+
+
 def similarity(input, templates, weights, **attrs):
     """Differentiable `ops.similarity` (same keyword arguments)."""
     unknown = set(attrs) - set(_SIM_KEYS)
@@ -88,7 +106,7 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), **attrs):
     ph, pw = int(pool_size[0]), int(pool_size[1])
     if torch.is_grad_enabled() and (input.requires_grad or offsets.requires_grad):
         y = MexFunction.apply(input, offsets, num_instances, attrs)
-        return torch.nn.functional.avg_pool2d(y, (ph, pw)) * float(ph * pw)
+        return SumPoolFunction.apply(y, ph, pw)
     return ops.mex_sum_pool(input, offsets, num_instances, (ph, pw), **attrs)
 
 

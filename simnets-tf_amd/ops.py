@@ -521,3 +521,19 @@ def sum_pooling(input, pool_size=(2, 2), out=None):
         _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),
                                                    stream))
     return out
+
+
+def sum_pooling_input_grad(output_grad, input_shape, pool_size=(2, 2)):
+    """Gradient of `sum_pooling` w.r.t. its input: each element receives its window's gradient, elements of a
+    dropped trailing row or column receive 0."""
+    g = _require_cuda_f32("output_grad", output_grad)
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    B, Cc, H, W = [int(v) for v in input_shape]
+    if tuple(g.shape) != (B, Cc, H // max(ph, 1), W // max(pw, 1)):
+        raise SimnetsError(-15)
+    dx = torch.empty((B, Cc, H, W), dtype=torch.float32, device=g.device)
+    with _on_device(g.device):
+        stream = torch.cuda.current_stream(g.device).cuda_stream
+        _check(_lib.lib().simnets_hip_sum_pool_input_grad((C.c_int * 4)(B, Cc, H, W), ph, pw, g.data_ptr(),
+                                                          dx.data_ptr(), stream))
+    return dx

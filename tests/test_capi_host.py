@@ -299,3 +299,12 @@ int main() {
     subprocess.run(["g++", "-O2", "-std=c++17", "-I" + os.path.join(ROOT, "simnets-tf_amd", "csrc"), str(src), "-o",
                     str(exe)], check=True)
     assert subprocess.run([str(exe)], check=True, capture_output=True, text=True).stdout.strip() == "0"
+
+
+def test_sum_pool_input_grad_validates_like_the_forward_call(pkg):
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    assert l.simnets_hip_sum_pool_input_grad(I4(2, 3, 8, 8), 0, 2, None, None, None) < 0      # pool size
+    assert l.simnets_hip_sum_pool_input_grad(I4(2, 3, 1, 8), 2, 2, None, None, None) < 0      # empty output
+    assert l.simnets_hip_sum_pool_input_grad(I4(0, 3, 8, 8), 2, 2, None, None, None) == 0     # empty batch: nothing to do
+    assert l.simnets_hip_sum_pool_input_grad(I4(2, 3, 8, 8), 2, 2, None, None, None) < 0      # null pointers

@@ -199,3 +199,20 @@ def test_mex_sum_pool_functional_fused_without_gradients_split_with(pkg):
     y = pkg.mex(x, off.detach(), 12, **kw)
     want = pkg.mex_offsets_grad(x, off.detach(), y, torch.ones_like(y), 12, **kw)
     assert torch.allclose(off.grad, want, rtol=1e-5, atol=1e-6)
+
+
+@pytest.mark.parametrize("shape,pool", [((3, 5, 8, 10), (2, 2)), ((2, 3, 7, 9), (2, 3)), ((1, 4, 5, 5), (5, 1))])
+def test_sum_pooling_gradient(pkg, shape, pool):
+    """layers.sum_pooling: forward = avg_pool2d * area ('valid': trailing rows/columns dropped), the gradient spreads
+    each window's gradient over its elements and gives the dropped ones 0 - checked against torch's own autograd."""
+    x = torch.randn(*shape, device="cuda", requires_grad=True)
+    y = pkg.layers.sum_pooling(x, pool)
+    g = torch.randn_like(y)
+    y.backward(g)
+    xr = x.detach().clone().requires_grad_()
+    yr = torch.nn.functional.avg_pool2d(xr, pool) * float(pool[0] * pool[1])
+    yr.backward(g)
+    assert torch.allclose(y, yr, rtol=1e-6, atol=1e-6)
+    assert torch.equal(x.grad, xr.grad * 0 + x.grad) and torch.allclose(x.grad, xr.grad, rtol=1e-6, atol=1e-7)
+    with pytest.raises(pkg.SimnetsError):
+        pkg.sum_pooling_input_grad(g[:, :, :-1] if g.shape[2] > 1 else g[:, :-1], shape, pool)
