@@ -243,6 +243,25 @@ def main():
         dev43 = float((fused_stack3() - ref4).abs().max() / ref4.abs().max())
         others["config4_stack"].update({"fused_similarity_mex_pool_kernel_ms": round(ms_fused3, 4),
                                         "fused_similarity_mex_pool_max_dev_of_scale": dev43})
+        # a training step of the same stack through the differentiable layer functions: forward with the unfused
+        # MEX calls (their gradients take the unpooled outputs), then every operator's gradient calls
+        L = pkg.layers
+        train_params = [T4.clone().requires_grad_(), W4.clone().requires_grad_()] + \
+                       [off.clone().requires_grad_() for off, _, _ in layers] + [offl.clone().requires_grad_()]
+
+        def train_step():
+            for q in train_params:
+                q.grad = None
+            cur = L.similarity(X4, train_params[0], train_params[1], **kw4)
+            for i, (_, n, kw) in enumerate(layers):
+                cur = L.mex_sum_pool(cur, train_params[2 + i], n, (2, 2), normalize_offsets=True, **kw)
+            out = L.mex(cur, train_params[-1], 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
+                        strides=[ch, 1, 1], shared_offset_region=[1])
+            out.sum().backward()
+
+        _, ms_train = timed(train_step, args.steps, args.warmup)
+        others["config4_stack"]["train_step_ms"] = round(ms_train, 4)
+        del train_params
         # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
         _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,
