@@ -91,8 +91,14 @@ def test_mex_random_geometry(pkg, seed):
     x, off, n, kw = random_mex_case(g)
     want = orc.mex_fwd(x, off, n, **kw)
     shift = orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, kw["epsilon"])))
-    got = pkg.mex(dev(x), dev(off), n, **kw)
-    assert rel_err(got.cpu().numpy(), want, floor=shift) <= 1e-4, kw
+    got = pkg.mex(dev(x), dev(off), n, **kw).cpu().numpy()
+    # against the fp32 oracle, or - where a log-sum-exp lands near zero and the fp32 oracle's own rounding shows -
+    # against the float64 oracle with twice the fp32 oracle's error as the bar
+    e32 = rel_err(got, want, floor=shift)
+    if e32 > 1e-4:
+        x64, off64 = f64(x, off)
+        true = orc.mex_fwd(x64, off64, n, **kw)
+        assert rel_err(got, true, floor=np.abs(shift)) <= max(1e-4, 2.0 * rel_err(want, true, floor=np.abs(shift))), kw
     go = g.normal(size=want.shape).astype(np.float32)
     dx = pkg.mex_input_grad(dev(x), dev(off), dev(want), dev(go), n, **kw).cpu().numpy()
     doff = pkg.mex_offsets_grad(dev(x), dev(off), dev(want), dev(go), n, **kw).cpu().numpy()
