@@ -223,15 +223,14 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
         }
     }
     // ---- d patch_k = 2^(xs_k - a) * acc, scattered to the input element the patch element is ----
-    const int bhw = a.bh * a.bw;
     const size_t chw = (size_t)a.C * a.H * a.W;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int k = k0 + wave * 16 + 4 * lq + v;
         if (k >= a.K)
             continue;
-        const int dc = k / bhw, rem = k - dc * bhw;
-        const int dh = rem / a.bw, dw = rem - dh * a.bw;
+        const int4 ke = a.ktab[k];
+        const int dc = ke.y, dh = ke.z, dw = ke.w;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int p = t * 16 + lr;
@@ -408,7 +407,6 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     }
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     const int lr = lane & 15, lq = lane >> 4;
-    const int bhw = a.bh * a.bw;
     floatx4 acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
@@ -446,16 +444,15 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             wt[lane * 65 + wave * 16 + i] = w;
         }
         // patch exponentials: this thread's pixel, 16 of the tile's patch elements
-        const size_t img = (size_t)px.b * a.C * a.H * a.W;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int kk = wave * 16 + i, k = k0 + kk;
             float e = 0.0f;
             if (valid && k < a.K) {
-                const int dc = k / bhw, rem = k - dc * bhw;
-                const int ci = px.ci0 + dc, hi = px.hi0 + rem / a.bw, wi = px.wi0 + rem % a.bw;
+                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
+                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
                 const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-                const float x = ok ? a.in[img + ((size_t)ci * a.H + hi) * a.W + wi] : a.oob;
+                const float x = ok ? px.base[ke.x] : a.oob;
                 e = __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.c1, -a_p));
             }
             ex[lane * 65 + kk] = e;
