@@ -300,6 +300,24 @@ def main():
         got = out3.cpu().numpy() if False else pkg.similarity(X3[:n_img], T3, W3, similarity_function="L2",
                                                                algo=args.algo, **kw3).cpu().numpy()
         err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-6 * np.abs(ref).max())))
+        # the reference's own ggemm_cpu (its header, compiled as it lies; include/utils/ggemm_cpu.hpp:462-511) on the
+        # im2col matrices of a few of the same images: the loop the reference's CPU kernel spends its time in
+        ref_ggemm = None
+        if oracle.ref() is not None:
+            A = np.ascontiguousarray(np.stack([t3.reshape(128, 576), w3.reshape(128, 576)], axis=-1))
+            n_ref = min(n_img, 4)
+            cols = []
+            for i in range(n_ref):
+                xp = np.pad(x3[i], ((0, 0), (1, 1), (1, 1)))
+                cols.append(np.ascontiguousarray(np.stack([xp[:, dh:dh + 32, dw:dw + 32] for dh in range(3)
+                                                           for dw in range(3)], axis=1).reshape(576, 1024)))
+            t0 = time.perf_counter()
+            outs = [oracle.ggemm_similarity(1, A, col, 128, 1024, 576, 0.001, "ref") for col in cols]
+            dtr = time.perf_counter() - t0
+            same = all(np.array_equal(o.reshape(128, 32, 32), ref[i]) for i, o in enumerate(outs))
+            ref_ggemm = {"value": round(n_ref * 128 * 1024 * 576 / dtr / 1e9, 4), "unit": "GMAC/s", "images": n_ref,
+                         "bit_identical_to_port": bool(same),
+                         "what": "reference ggemm_cpu<sim_l2_forward> from its own header, im2col and interlace not timed"}
         result["cpu_baseline"] = {
             "value": round(gm / dt / 1e9, 4), "unit": "GMAC/s", "cores": 1, "kind": "port",
             "sample": "%d of 256 images of config 3 (L2), single thread like the reference; -O2, no fast-math" % n_img,
@@ -308,6 +326,8 @@ def main():
             "host_cpus": cores,
             "max_rel_err_gpu_vs_cpu": err,
         }
+        if ref_ggemm is not None:
+            result["cpu_baseline"]["reference_ggemm"] = ref_ggemm
     print(json.dumps(result))
 
 
