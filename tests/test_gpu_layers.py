@@ -216,3 +216,59 @@ def test_sum_pooling_gradient(pkg, shape, pool):
     assert torch.equal(x.grad, xr.grad * 0 + x.grad) and torch.allclose(x.grad, xr.grad, rtol=1e-6, atol=1e-7)
     with pytest.raises(pkg.SimnetsError):
         pkg.sum_pooling_input_grad(g[:, :, :-1] if g.shape[2] > 1 else g[:, :-1], shape, pool)
+
+
+def test_gradient_calls_replay_from_a_hip_graph(pkg):
+    """The gradient calls, too, are kernel launches on the caller's stream and nothing else: their scratch (partial
+    sums, centres, packed parameters, flags, the patch-gradient buffer of overlapping MEX patches) is rewritten by
+    every call.  Captured once, every replay on new data - with eager calls in between - reproduces the eager
+    results bit for bit (the sums run in a fixed order)."""
+    g = np.random.default_rng(77)
+    skw = dict(similarity_function="L2", blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    mkw = dict(blocks=[3, 2, 2], strides=[2, 1, 1], padding=[1, 0, 0], epsilon=2.0, softmax_mode=True,
+               use_unshared_regions=False, shared_offset_region=[2])
+    T = torch.from_numpy(g.normal(size=(12, 32, 3, 3)).astype(np.float32)).cuda()
+    W = torch.from_numpy((np.abs(g.normal(size=(12, 32, 3, 3))) + 0.05).astype(np.float32)).cuda()
+
+    def fresh(seed):
+        q = np.random.default_rng(seed)
+        x = torch.from_numpy(q.normal(size=(3, 32, 12, 32)).astype(np.float32)).cuda()
+        gs = torch.from_numpy(q.normal(size=(3, 12, 12, 32)).astype(np.float32)).cuda()
+        return x, gs
+
+    sx, sg = fresh(0)
+    n_inst = 5
+    y0 = pkg.similarity(sx, T, W, **skw)
+    dshape, oshape = pkg.mex_output_shape(tuple(y0.shape), n_inst, **mkw)
+    off = torch.from_numpy((g.normal(size=oshape) * 0.3).astype(np.float32)).cuda()
+    gm = torch.from_numpy(g.normal(size=dshape).astype(np.float32)).cuda()
+
+    def work(x, gs):
+        y = pkg.similarity(x, T, W, **skw)
+        dx = pkg.similarity_input_grad(x, T, W, gs, **skw)
+        dt, dw = pkg.similarity_parameters_grad(x, T, W, gs, **skw)
+        z = pkg.mex(y, off, n_inst, **mkw)
+        dy = pkg.mex_input_grad(y, off, z, gm, n_inst, **mkw)
+        do = pkg.mex_offsets_grad(y, off, z, gm, n_inst, **mkw)
+        return dx, dt, dw, dy, do
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            work(sx, sg)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        static_out = work(sx, sg)
+    for trial in range(3):
+        x, gs = fresh(10 + trial)
+        sx.copy_(x)
+        sg.copy_(gs)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in static_out]
+        want = work(x, gs)
+        torch.cuda.synchronize()
+        for a, b, name in zip(got, want, ("dX", "dT", "dW", "mex dX", "mex dOff")):
+            assert torch.equal(a, b), "replay %d: %s" % (trial, name)
