@@ -36,6 +36,9 @@ struct MexGradArgs {
     int overlap;           // patches overlap: the per-patch gradients go to `col`, mex_col2im_kernel adds them up
     float *col;            // [B][Co*Ho*Wo][K] gradient of every patch element (overlapping patches only)
     int cpr;               // pixel chunks per region
+    int msplit;            // input gradient: the instances are split over gridDim.z workgroups (1: no split) ...
+    int mg_per_split;      // ... of this many packed groups (GM_TM instances) each, which write their partial
+    float *dx_splits;      // gradients to [split][input] for mex_sum_splits_kernel
     int pxl;               // pixel slots per lane (offsets gradient)
 };
 
@@ -65,7 +68,8 @@ __device__ __forceinline__ float mex_term(float x_plus_off, float out, float g, 
 constexpr int GX_KT = 8;   // patch elements per lane (input gradient)
 
 // One wave: the 64 pixel slots of (region r, chunk) x GX_KT patch elements from k0, term by term.
-__device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r, int chunk, int k0, int lane)
+__device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r, int chunk, int k0, int lane,
+                                                    int m_begin, int m_end, float *dx)
 {
     const MexKernelArgs &a = ga.k;
     const PixelRef px = locate(a, r, chunk * 64 + lane);
@@ -86,7 +90,7 @@ __device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float SIMNETS_CONST_AS *off = (const float SIMNETS_CONST_AS *)(ga.off) + (size_t)r * a.M * a.K + k0;
     const bool finite = a.finite_eps != 0;
-    for (int m = 0; m < a.M; ++m) {
+    for (int m = m_begin; m < m_end; ++m) {
         const float g = valid ? gp[(size_t)m * plane] : 0.0f;
         const float o = op[(size_t)m * plane];
 #pragma unroll
@@ -97,7 +101,7 @@ __device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r
     }
     if (!valid)
         return;
-    float *dimg = ga.dx + (size_t)px.b * a.C * a.H * a.W;
+    float *dimg = dx + (size_t)px.b * a.C * a.H * a.W;
     float *dcol = ga.col + ((size_t)px.b * plane + px.out_off) * a.K + k0;
 #pragma unroll
     for (int j = 0; j < GX_KT; ++j) {
@@ -119,7 +123,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
     const int chunk = blockIdx.x - r * ga.cpr;
     const int k0 = (blockIdx.y * 4 + wave) * GX_KT;
     if (k0 < ga.k.K)
-        mex_grad_input_wave(ga, r, chunk, k0, lane);
+        mex_grad_input_wave(ga, r, chunk, k0, lane, 0, ga.k.M, ga.dx);
 }
 
 // Finite epsilon, product form on the fp32 matrix cores.  In the scaled domain (xs = c1 x, os = c1 off, outs = c1 out,
@@ -134,6 +138,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
 // workgroup falls back to the term-by-term waves.
 // grid.x: (region, pixel chunk of 64 slots); grid.y: tile of GM_KT patch elements (16 per wave)
 constexpr int GM_TM = 32;   // instances per packed group = contraction chunk
+constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) up to which a few instances give the bound
 constexpr int GM_KT = 64;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
@@ -152,17 +157,26 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     const int chunk = blockIdx.x - r * ga.cpr;
     const int k0 = blockIdx.y * GM_KT;
     const int n_mg = a.n_mgroups;
+    // this workgroup's share of the instances (all of them unless the launch splits them over gridDim.z) and where
+    // its gradients go
+    const int mg_begin = blockIdx.z * ga.mg_per_split, mg_end = min(n_mg, mg_begin + ga.mg_per_split);
+    float *dxo = ga.msplit > 1 ? ga.dx_splits + (size_t)blockIdx.z * a.B * a.C * a.H * a.W : ga.dx;
     const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
+    int roomy;  // some instance's offsets range is large enough for the choice of the bound to matter (below)
     {
-        int wide = 0;
-        for (int m = tid; m < a.M; m += 256)
+        int wide = 0, big = 0;
+        for (int m = tid; m < a.M; m += 256) {
             wide |= !(orng_r[m] <= kProductRange);
+            big |= !(orng_r[m] <= kLooseBoundRange);
+        }
+        roomy = __syncthreads_or(big);
         if (__syncthreads_or(wide)) {
 #pragma unroll
             for (int h = 0; h < GM_KT / (4 * GX_KT); ++h) {
                 const int kk0 = k0 + (wave * (GM_KT / (4 * GX_KT)) + h) * GX_KT;
                 if (kk0 < a.K)
-                    mex_grad_input_wave(ga, r, chunk, kk0, lane);
+                    mex_grad_input_wave(ga, r, chunk, kk0, lane, min(a.M, mg_begin * GM_TM), min(a.M, mg_end * GM_TM),
+                                        dxo);
             }
             return;
         }
@@ -177,9 +191,14 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
-    // the pixel's bound a = min_m (outs_m - c0 - lo_m)
+    // the pixel's bound a = min_m (outs_m - c0 - lo_m).  Every single term of the minimum is a valid bound
+    // (>= every xs_k); with the minimum over all instances the exponent of W_m stays below the instance's own
+    // offsets range, with the minimum over a few it stays below that range + the range of those few + log2 K.
+    // While no range exceeds kLooseBoundRange that is far from overflow, and the first four instances (one
+    // strided load per thread instead of M / 4) do.
+    const int m_scan = roomy ? a.M : min(a.M, 4);
     float amin = INFINITY;
-    for (int m = wave; m < a.M; m += 4)
+    for (int m = wave; m < m_scan; m += 4)
         amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
     pmn[wave * 64 + lane] = amin;
     __syncthreads();
@@ -193,7 +212,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
 #pragma unroll
     for (int t = 0; t < 4; ++t)
         acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
-    for (int mg = 0; mg < n_mg; ++mg) {
+    for (int mg = mg_begin; mg < mg_end; ++mg) {
         __syncthreads();  // the previous chunk's matrix instructions are done with eo / wt
         const float4 *src = reinterpret_cast<const float4 *>(a.offe + (((size_t)r * n_mg + mg) * a.K + k0) * GM_TM);
         for (int i = tid; i < GM_KT * (GM_TM / 4); i += 256) {
@@ -245,8 +264,20 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             if (ga.overlap)
                 ga.col[((size_t)b * plane + pout[p]) * a.K + k] = val;
             else
-                ga.dx[at] = val;
+                dxo[at] = val;
         }
+    }
+}
+
+// Instances split over several workgroups: input gradient = sum of their partial gradients, in split order.
+__global__ __launch_bounds__(256) void mex_sum_splits_kernel(const float *__restrict__ parts, long long n, int splits,
+                                                            float *__restrict__ dx)
+{
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long long)gridDim.x * 256) {
+        float s = parts[i];
+        for (int z = 1; z < splits; ++z)
+            s += parts[(size_t)z * n + i];
+        dx[i] = s;
     }
 }
 
@@ -566,6 +597,9 @@ struct MexGradTiling {
     size_t norm_bytes, partial_bytes, packed_bytes;
     bool overlap;        // input gradient: patches overlap
     size_t col_bytes;    // ... and their per-patch gradients pass through a [B][Co*Ho*Wo][K] buffer
+    bool tiles_input;    // patches tile the input exactly: every element is written by exactly one patch
+    int msplit, mg_per_split;  // input gradient, matrix form: instance groups split over gridDim.z workgroups
+    size_t split_bytes;  // ... whose partial gradients [split][input] are added by mex_sum_splits_kernel
 };
 
 MexGradTiling mex_grad_tiling(const MexPlan &p)
@@ -589,6 +623,20 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
                 (d.block_w > d.stride_w && d.width_out > 1);
     t.col_bytes = t.overlap ? align_up((size_t)p.B * d.channels_out * d.height_out * d.width_out * d.K * sizeof(float),
                                        256) : 0;
+    t.tiles_input = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 && d.stride_c == d.block_c &&
+                    d.stride_h == d.block_h && d.stride_w == d.block_w && d.channels_out * d.block_c == p.C &&
+                    d.height_out * d.block_h == p.H && d.width_out * d.block_w == p.W;
+    // Few pixels and many instances (deep layers on small maps): a workgroup would walk all instance groups alone
+    // while most of the chip idles.  Then the groups are split over up to 8 workgroups (two groups each at least)
+    // until the launch has about two workgroups per compute unit.
+    t.msplit = 1;
+    const int n_mg = (d.M + GM_TM - 1) / GM_TM;
+    const long long wgs = (long long)d.num_regions * ((slots + 63) / 64) * ((d.K + GM_KT - 1) / GM_KT);
+    if (t.mfma && t.tiles_input && wgs <= 256 && n_mg >= 4)
+        t.msplit = (int)std::max<long long>(1, std::min<long long>(std::min(8, n_mg / 2), 512 / std::max<long long>(wgs, 1)));
+    t.mg_per_split = (n_mg + t.msplit - 1) / t.msplit;
+    t.msplit = (n_mg + t.mg_per_split - 1) / t.mg_per_split;
+    t.split_bytes = t.msplit > 1 ? align_up((size_t)t.msplit * p.B * p.C * p.H * p.W * sizeof(float), 256) : 0;
     return t;
 }
 
@@ -612,7 +660,7 @@ int prepare_offsets(const MexPlan &p, const float *offsets, void *workspace, hip
 size_t mex_grad_input_workspace_bytes(const MexPlan &p)
 {
     const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.packed_bytes + t.col_bytes;
+    return t.norm_bytes + t.packed_bytes + t.col_bytes + t.split_bytes;
 }
 
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p)
@@ -639,6 +687,9 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
     const MexGradTiling t = mex_grad_tiling(p);
     ga.overlap = t.overlap ? 1 : 0;
     ga.col = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes);
+    ga.msplit = t.msplit; ga.mg_per_split = t.mg_per_split;
+    ga.dx_splits = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes +
+                                             t.col_bytes);
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
 
@@ -647,11 +698,7 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
         return SIMNETS_OK;
     if ((n_in + 255) / 256 > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
-    // patches that tile the input exactly (no padding, stride = block, nothing left over) write every element
-    const bool tiles_input = d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 && d.stride_c == d.block_c &&
-                             d.stride_h == d.block_h && d.stride_w == d.block_w &&
-                             d.channels_out * d.block_c == p.C && d.height_out * d.block_h == p.H &&
-                             d.width_out * d.block_w == p.W;
+    const bool tiles_input = t.tiles_input;
     if (!t.overlap && !tiles_input) {
         // every element belongs to at most one patch, which stores its gradient; the others keep 0
         hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
@@ -669,7 +716,14 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
         if (gx > 0x7fffffffLL || gy > 65535)
             return SIMNETS_ERR_TOO_LARGE;
         if (gx > 0)
-            hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
+            hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)t.msplit),
+                               dim3(256), 0, s, ga);
+        if (gx > 0 && t.msplit > 1) {
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+            hipLaunchKernelGGL(mex_sum_splits_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
+                               dim3(256), 0, s, ga.dx_splits, n_in, t.msplit, input_grad);
+        }
     } else {
         const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
         if (gx > 0x7fffffffLL || gy > 65535)
@@ -712,6 +766,7 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
     ga.out = output; ga.g = output_grad; ga.dx = nullptr;
     ga.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes);
     ga.overlap = 0; ga.col = nullptr;
+    ga.msplit = 1; ga.mg_per_split = ga.k.n_mgroups; ga.dx_splits = nullptr;
     ga.pxl = t.pxl;
     ga.cpr = t.cpr_offsets;
 
