@@ -39,6 +39,11 @@ struct MexGradArgs {
     int msplit;            // input gradient: the instances are split over gridDim.z workgroups (1: no split) ...
     int mg_per_split;      // ... of this many packed groups (GM_TM instances) each, which write their partial
     float *dx_splits;      // gradients to [split][input] for mex_sum_splits_kernel
+    // Factor buffers (finite epsilon, optional): the pixel factors W [R][slots_pad][Mp] and the patch exponentials
+    // EX [R][slots_pad][Kp] of mex_grad_factors_kernel, which the matrix kernels then load instead of forming them
+    // (again and again: once per tile of the other dimension).  nullptr: the kernels form them themselves.
+    float *wbuf, *exbuf;
+    int slots_pad, Mp, Kp;
     int pxl;               // pixel slots per lane (offsets gradient)
 };
 
@@ -142,6 +147,86 @@ constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) 
 constexpr int GM_KT = 64;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
+// Pixel factors and patch exponentials of the product form, once per pixel: for the 64 pixel slots of
+// (region, chunk) the bound a, W_m = g_m 2^(a + mo_m - outs_m + c0) for every instance and 2^(xs_k - a) for every
+// patch element, written as rows [slot][Mp] and [slot][Kp] (through LDS, so that the stores run along the rows);
+// a workgroup forms one block of 32 instances or 32 patch elements (grid.y), each from the same bound.
+// Regions with an offsets range beyond kProductRange are left alone: the matrix kernels fall back to the
+// term-by-term waves there and never look at the buffers.
+__global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs ga)
+{
+    const MexKernelArgs &a = ga.k;
+    __shared__ float tile[32 * 65];   // [instance or patch element][pixel], padded rows
+    __shared__ float pmn[4 * 64];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = blockIdx.x / ga.cpr;
+    const int chunk = blockIdx.x - r * ga.cpr;
+    const int n_mg = a.n_mgroups;
+    const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
+    int wide = 0, big = 0;
+    for (int m = tid; m < a.M; m += 256) {
+        wide |= !(orng_r[m] <= kProductRange);
+        big |= !(orng_r[m] <= kLooseBoundRange);
+    }
+    const int roomy = __syncthreads_or(big);
+    if (__syncthreads_or(wide))
+        return;
+    const PixelRef px = locate(a, r, chunk * 64 + lane);
+    const bool valid = px.out_off >= 0;
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const int m_scan = roomy ? a.M : min(a.M, 4);   // see mex_grad_input_mfma_kernel
+    float amin = INFINITY;
+    for (int m = wave; m < m_scan; m += 4)
+        amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
+    pmn[wave * 64 + lane] = amin;
+    __syncthreads();
+    const float a_p = valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
+    // rows of this chunk; thread (column c, pixels pr, pr + 8, ...) writes the tile out
+    const size_t row0 = (size_t)r * ga.slots_pad + (size_t)chunk * 64;
+    const int c = tid & 31, pr = tid >> 5;
+    // grid.y: one block of 32 columns per workgroup - the instance groups first, then the patch-element blocks
+    if ((int)blockIdx.y < n_mg) {
+        const int mg = blockIdx.y;
+#pragma unroll
+        for (int i = 0; i < GM_TM / 4; ++i) {
+            const int mm = wave + 4 * i, m = mg * GM_TM + mm;
+            float w = 0.0f;
+            if (valid && m < a.M) {
+                const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
+                w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+            }
+            tile[mm * 65 + lane] = w;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            ga.wbuf[(row0 + pr + 8 * j) * ga.Mp + mg * GM_TM + c] = tile[c * 65 + pr + 8 * j];
+    } else {
+        const int kb = ((int)blockIdx.y - n_mg) * 32;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int kk = wave + 4 * i, k = kb + kk;
+            float e = 0.0f;
+            if (valid && k < a.K) {
+                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
+                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
+                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                const float x = ok ? px.base[ke.x] : a.oob;
+                e = __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.c1, -a_p));
+            }
+            tile[kk * 65 + lane] = e;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            ga.exbuf[(row0 + pr + 8 * j) * ga.Kp + kb + c] = tile[c * 65 + pr + 8 * j];
+    }
+}
+
 __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradArgs ga)
 {
     const MexKernelArgs &a = ga.k;
@@ -191,12 +276,14 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const bool buffered = ga.wbuf != nullptr;   // W and 2^(xs - a) come from mex_grad_factors_kernel
+    const size_t row0 = (size_t)r * ga.slots_pad + (size_t)chunk * 64;
     // the pixel's bound a = min_m (outs_m - c0 - lo_m).  Every single term of the minimum is a valid bound
     // (>= every xs_k); with the minimum over all instances the exponent of W_m stays below the instance's own
     // offsets range, with the minimum over a few it stays below that range + the range of those few + log2 K.
     // While no range exceeds kLooseBoundRange that is far from overflow, and the first four instances (one
     // strided load per thread instead of M / 4) do.
-    const int m_scan = roomy ? a.M : min(a.M, 4);
+    const int m_scan = buffered ? 0 : (roomy ? a.M : min(a.M, 4));
     float amin = INFINITY;
     for (int m = wave; m < m_scan; m += 4)
         amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
@@ -221,16 +308,24 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             float *d = eo + row * (GM_TM + 1) + 4 * c4;
             d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
         }
+        if (buffered) {
+            // rows of 32 instances: thread (instance c, pixels pr, pr + 8, ...)
+            const int c = tid & 31, pr = tid >> 5;
 #pragma unroll
-        for (int i = 0; i < GM_TM / 4; ++i) {
-            const int mm = wave + 4 * i, m = mg * GM_TM + mm;
-            float w = 0.0f;
-            if (valid && m < a.M) {
-                // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
-                const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
-                w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+            for (int j = 0; j < 8; ++j)
+                wt[c * 65 + pr + 8 * j] = ga.wbuf[(row0 + pr + 8 * j) * ga.Mp + mg * GM_TM + c];
+        } else {
+#pragma unroll
+            for (int i = 0; i < GM_TM / 4; ++i) {
+                const int mm = wave + 4 * i, m = mg * GM_TM + mm;
+                float w = 0.0f;
+                if (valid && m < a.M) {
+                    // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
+                    const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
+                    w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+                }
+                wt[mm * 65 + lane] = w;
             }
-            wt[mm * 65 + lane] = w;
         }
         __syncthreads();
 #pragma unroll
@@ -260,7 +355,8 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             if (!(ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W))
                 continue;
             const size_t at = (size_t)b * chw + ((size_t)ci * a.H + hi) * a.W + wi;
-            const float val = acc[t][v] * __builtin_amdgcn_exp2f(__builtin_fmaf(a.in[at], a.c1, -ap[p]));
+            const float val = acc[t][v] * (buffered ? ga.exbuf[(row0 + p) * ga.Kp + k]
+                                                    : __builtin_amdgcn_exp2f(__builtin_fmaf(a.in[at], a.c1, -ap[p])));
             if (ga.overlap)
                 ga.col[((size_t)b * plane + pout[p]) * a.K + k] = val;
             else
@@ -444,7 +540,32 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
         acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // this thread's instances when staging (16 of the tile, the same for the whole wave) and their constants
     const int ms0 = m0 + wave * 16;
+    const bool buffered = ga.wbuf != nullptr;   // W and 2^(xs - a) come from mex_grad_factors_kernel
     for (int s = 0; s < ga.pxl; ++s) {
+        if (buffered) {
+            // rows of the group's 64 pixel slots: thread (column cc of the tile, pixels pq, pq + 4, ...)
+            const int grp = chunk * ga.pxl + s;
+            if (grp * 64 >= ga.slots_pad)
+                break;  // no slots left in the region (uniform)
+            const size_t row0 = (size_t)r * ga.slots_pad + (size_t)grp * 64;
+            const int cc = tid & 63, pq = tid >> 6;
+            __syncthreads();  // the previous group's matrix instructions are done with wt / ex
+#pragma unroll
+            for (int j = 0; j < 16; ++j) {
+                const int pp = pq + 4 * j;
+                wt[pp * 65 + cc] = m0 + cc < ga.Mp ? ga.wbuf[(row0 + pp) * ga.Mp + m0 + cc] : 0.0f;
+                ex[pp * 65 + cc] = k0 + cc < ga.Kp ? ga.exbuf[(row0 + pp) * ga.Kp + k0 + cc] : 0.0f;
+            }
+            __syncthreads();
+#pragma unroll 4
+            for (int ps = 0; ps < 64; ps += 4) {
+                const float av = wt[(ps + lq) * 65 + wave * 16 + lr];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, ex[(ps + lq) * 65 + t * 16 + lr], acc[t], 0, 0, 0);
+            }
+            continue;
+        }
         const PixelRef px = locate(a, r, (chunk * ga.pxl + s) * 64 + lane);
         const bool valid = px.out_off >= 0;
         const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
@@ -600,6 +721,11 @@ struct MexGradTiling {
     bool tiles_input;    // patches tile the input exactly: every element is written by exactly one patch
     int msplit, mg_per_split;  // input gradient, matrix form: instance groups split over gridDim.z workgroups
     size_t split_bytes;  // ... whose partial gradients [split][input] are added by mex_sum_splits_kernel
+    // factor buffers of mex_grad_factors_kernel: used when a matrix kernel would otherwise form the same factors
+    // in several workgroups (more than one tile along the dimension it does not contract)
+    bool factors_input, factors_offsets;
+    int slots_pad, Mp, Kp;
+    size_t factor_bytes;
 };
 
 MexGradTiling mex_grad_tiling(const MexPlan &p)
@@ -637,6 +763,15 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
     t.mg_per_split = (n_mg + t.msplit - 1) / t.msplit;
     t.msplit = (n_mg + t.mg_per_split - 1) / t.mg_per_split;
     t.split_bytes = t.msplit > 1 ? align_up((size_t)t.msplit * p.B * p.C * p.H * p.W * sizeof(float), 256) : 0;
+    t.slots_pad = (int)((slots + 63) / 64 * 64);
+    t.Mp = n_mg * GM_TM;
+    t.Kp = (d.K + 31) / 32 * 32;
+    const int k_tiles = (d.K + GM_KT - 1) / GM_KT, m_tiles = (d.M + GOM_MT - 1) / GOM_MT;
+    // (the extra launch and the round trip through memory cost about 10 us: measured to pay from 4 tiles of patch
+    // elements and 128 instances on for the input gradient and from 16 tiles on for the offsets gradient)
+    t.factors_input = t.mfma && k_tiles >= 4 && d.M >= 128;
+    t.factors_offsets = t.mfma && m_tiles * ((d.K + GOM_KT - 1) / GOM_KT) >= 16;
+    t.factor_bytes = align_up((size_t)d.num_regions * t.slots_pad * ((size_t)t.Mp + t.Kp) * sizeof(float), 256);
     return t;
 }
 
@@ -654,19 +789,38 @@ int prepare_offsets(const MexPlan &p, const float *offsets, void *workspace, hip
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
+// Launches mex_grad_factors_kernel into `buffers` and points ga at them (ga.k must hold the packed offsets).
+int launch_factors(const MexPlan &p, const MexGradTiling &t, MexGradArgs &ga, void *buffers, hipStream_t s)
+{
+    ga.slots_pad = t.slots_pad; ga.Mp = t.Mp; ga.Kp = t.Kp;
+    ga.wbuf = reinterpret_cast<float *>(buffers);
+    ga.exbuf = ga.wbuf + (size_t)p.d.num_regions * t.slots_pad * t.Mp;
+    MexGradArgs fa = ga;
+    fa.cpr = t.slots_pad / 64;
+    const long long gx = (long long)p.d.num_regions * fa.cpr;
+    if (gx > 0x7fffffffLL)
+        return SIMNETS_ERR_TOO_LARGE;
+    const int gy = t.Mp / GM_TM + t.Kp / 32;
+    if (gy > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    if (gx > 0)
+        hipLaunchKernelGGL(mex_grad_factors_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, fa);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
 }  // namespace
 
 // finite epsilon: the matrix-core kernels read the forward pass's packed offsets (groups of GM_TM instances)
 size_t mex_grad_input_workspace_bytes(const MexPlan &p)
 {
     const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.packed_bytes + t.col_bytes + t.split_bytes;
+    return t.norm_bytes + t.packed_bytes + t.col_bytes + t.split_bytes + (t.factors_input ? t.factor_bytes : 0);
 }
 
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p)
 {
     const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.partial_bytes + t.packed_bytes;
+    return t.norm_bytes + t.partial_bytes + t.packed_bytes + (t.factors_offsets ? t.factor_bytes : 0);
 }
 
 int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
@@ -690,6 +844,7 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
     ga.msplit = t.msplit; ga.mg_per_split = t.mg_per_split;
     ga.dx_splits = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes +
                                              t.col_bytes);
+    ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
 
@@ -715,6 +870,12 @@ int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, c
         const int gy = (d.K + GM_KT - 1) / GM_KT;
         if (gx > 0x7fffffffLL || gy > 65535)
             return SIMNETS_ERR_TOO_LARGE;
+        if (t.factors_input) {
+            rc = launch_factors(p, t, ga, reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes +
+                                              t.col_bytes + t.split_bytes, s);
+            if (rc)
+                return rc;
+        }
         if (gx > 0)
             hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)t.msplit),
                                dim3(256), 0, s, ga);
@@ -767,6 +928,7 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
     ga.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes);
     ga.overlap = 0; ga.col = nullptr;
     ga.msplit = 1; ga.mg_per_split = ga.k.n_mgroups; ga.dx_splits = nullptr;
+    ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
     ga.pxl = t.pxl;
     ga.cpr = t.cpr_offsets;
 
@@ -779,6 +941,12 @@ int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets,
         const int gy = (d.M + GOM_MT - 1) / GOM_MT, gz = (d.K + GOM_KT - 1) / GOM_KT;
         if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
             return SIMNETS_ERR_TOO_LARGE;
+        if (t.factors_offsets) {
+            rc = launch_factors(p, t, ga, reinterpret_cast<char *>(workspace) + t.norm_bytes + t.partial_bytes +
+                                              t.packed_bytes, s);
+            if (rc)
+                return rc;
+        }
         hipLaunchKernelGGL(mex_grad_offsets_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
                            ga);
     } else {

@@ -486,3 +486,19 @@ def test_similarity_input_grad_matrix_form(pkg, case, func, norm, ign):
         dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), algo=algo, **kw).cpu().numpy()
         assert np.array_equal(np.isnan(dx), np.isnan(want))
         assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad (%s)" % algo)
+
+
+@pytest.mark.parametrize("spread", ["narrow", "mixed"])
+@pytest.mark.parametrize("eps", [1.0, -2.0])
+def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, spread):
+    """200 instances x 200 patch elements on 4x4 maps: the matrix kernels take the pixel factors and patch
+    exponentials from the buffers of the factors kernel (formed once per pixel instead of once per tile of the other
+    dimension), the input gradient splits the instance groups over workgroups; slot, instance and element counts are
+    no multiples of the tile sizes.  'mixed': every other region has a wide offsets range and runs term by term."""
+    kw = dict(blocks=[200, 1, 1], strides=[200, 1, 1], padding=[0, 0, 0], unshared_offset_region=[2], epsilon=eps,
+              softmax_mode=True)
+    x, off = mex_case(61, (6, 200, 4, 4), 200, **kw)
+    off = off * 0.3
+    if spread == "mixed":
+        off[::2] *= 300
+    check_mex_grads(pkg, x, off, 200, **kw)
