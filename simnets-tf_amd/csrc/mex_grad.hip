@@ -541,6 +541,40 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     // this thread's instances when staging (16 of the tile, the same for the whole wave) and their constants
     const int ms0 = m0 + wave * 16;
     const bool buffered = ga.wbuf != nullptr;   // W and 2^(xs - a) come from mex_grad_factors_kernel
+    // global loads of a group of 64 pixel slots: this thread's pixel, its 16 instances' output and gradient values
+    // and 16 of the tile's patch elements; the loads of group s + 1 are issued before group s is processed
+    struct Group {
+        bool valid;
+        float ov[16], gv[16], xr[16];
+    };
+    auto load_group = [&](int s, Group &q) {
+        const PixelRef px = locate(a, r, (chunk * ga.pxl + s) * 64 + lane);
+        q.valid = px.out_off >= 0;
+        const float *gp = ga.g + (size_t)px.b * a.M * plane + (q.valid ? px.out_off : 0);
+        const float *op = ga.out + (size_t)px.b * a.M * plane + (q.valid ? px.out_off : 0);
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = ms0 + i;
+            q.ov[i] = 0.0f;
+            q.gv[i] = 0.0f;
+            if (m < a.M) {
+                q.ov[i] = op[(size_t)m * plane];
+                q.gv[i] = q.valid ? gp[(size_t)m * plane] : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int k = k0 + wave * 16 + i;
+            q.xr[i] = 0.0f;
+            if (q.valid && k < a.K) {
+                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
+                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
+                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                q.xr[i] = ok ? px.base[ke.x] : a.oob;
+            }
+        }
+    };
+    Group cur;
     for (int s = 0; s < ga.pxl; ++s) {
         if (buffered) {
             // rows of the group's 64 pixel slots: thread (column cc of the tile, pixels pq, pq + 4, ...)
@@ -566,33 +600,28 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             }
             continue;
         }
-        const PixelRef px = locate(a, r, (chunk * ga.pxl + s) * 64 + lane);
-        const bool valid = px.out_off >= 0;
-        const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
-        const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
-        float ov[16], gv[16];
+        if (s == 0)
+            load_group(0, cur);
+        Group nxt;
+        if (s + 1 < ga.pxl)
+            load_group(s + 1, nxt);   // in flight while this group is processed
         float amin = INFINITY;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int m = ms0 + i;
-            ov[i] = 0.0f;
-            gv[i] = 0.0f;
-            if (m < a.M) {
-                ov[i] = op[(size_t)m * plane];
-                gv[i] = valid ? gp[(size_t)m * plane] : 0.0f;
-                amin = fminf(amin, __builtin_fmaf(ov[i], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
-            }
+            if (m < a.M)
+                amin = fminf(amin, __builtin_fmaf(cur.ov[i], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
         }
         __syncthreads();  // the previous group's matrix instructions are done with wt / ex / ap
         pmn[wave * 64 + lane] = amin;
         __syncthreads();
-        const float a_p = valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
+        const float a_p = cur.valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int m = ms0 + i;
             float w = 0.0f;
             if (m < a.M)
-                w = gv[i] * __builtin_amdgcn_exp2f(__builtin_fmaf(-ov[i], a.c1, a_p) + (omax_r[m] + a.c0));
+                w = cur.gv[i] * __builtin_amdgcn_exp2f(__builtin_fmaf(-cur.ov[i], a.c1, a_p) + (omax_r[m] + a.c0));
             wt[lane * 65 + wave * 16 + i] = w;
         }
         // patch exponentials: this thread's pixel, 16 of the tile's patch elements
@@ -600,13 +629,8 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
         for (int i = 0; i < 16; ++i) {
             const int kk = wave * 16 + i, k = k0 + kk;
             float e = 0.0f;
-            if (valid && k < a.K) {
-                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
-                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
-                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-                const float x = ok ? px.base[ke.x] : a.oob;
-                e = __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.c1, -a_p));
-            }
+            if (cur.valid && k < a.K)
+                e = __builtin_amdgcn_exp2f(__builtin_fmaf(cur.xr[i], a.c1, -a_p));
             ex[lane * 65 + kk] = e;
         }
         __syncthreads();
@@ -617,6 +641,8 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             for (int t = 0; t < 4; ++t)
                 acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, ex[(ps + lq) * 65 + t * 16 + lr], acc[t], 0, 0, 0);
         }
+        if (s + 1 < ga.pxl)
+            cur = nxt;
     }
     // ---- partial sums of this pixel chunk: acc * 2^(os_mk - mo_m) ----
     float *dst = ga.partial + ((size_t)chunk * a.R + r) * a.M * a.K;
