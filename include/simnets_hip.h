@@ -219,8 +219,8 @@ int simnets_hip_mex_grad_workspace_bytes(const simnets_mex_attrs *attrs, const i
  * (src/kernels/mex_grad_kernel_gpu.cu), i.e. per image im2col_3d_gpu + split_patches + ggemm_readc_gpu with
  * mex_backward_bottom_finite/_infinite + reverse split_patches + col2im_3d_gpu.
  * output = the forward result for the same input/offsets/attrs, output_grad has its shape, input_grad the
- * input's.  When blocks overlap (block > stride) contributions are added with floating-point atomics, so
- * the summation order, and with it the last bits, may differ between runs. */
+ * input's.  When blocks overlap (block > stride) the patches' contributions to an element are added in
+ * ascending (c, h, w) order of the patches, like col2im_3d does: results are reproducible. */
 int simnets_hip_mex_input_grad(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                                const float *offsets, size_t offsets_count, const float *output,
                                const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
@@ -234,6 +234,16 @@ int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input
                                  const float *offsets, size_t offsets_count, const float *output,
                                  const float *output_grad, float *offsets_grad, void *workspace,
                                  size_t workspace_bytes, void *stream);
+
+/* Both gradients of one MEX layer in one call, as the gradient registered for the Mex op needs them
+ * (python/simnets/ops/mex.py:47-81 calls MexInputGrad and MexOffsetsGrad on the same tensors): the results are those
+ * of simnets_hip_mex_input_grad and simnets_hip_mex_offsets_grad, bit for bit; the offsets as the forward op used
+ * them, their packed form and the per-pixel factors are prepared once for both. */
+int simnets_hip_mex_grads_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], size_t *bytes);
+int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                          const float *offsets, size_t offsets_count, const float *output, const float *output_grad,
+                          float *input_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
+                          void *stream);
 
 /* ------------------------------------------------------------------------------------------
  * Glue of the missing-data network between MEX layers: non-overlapping sum pooling, which the

@@ -20,6 +20,7 @@ from .ops import (  # noqa: F401
     similarity_parameters_grad,
     mex_input_grad,
     mex_offsets_grad,
+    mex_grads,
     _mex_dims_helper,
     _expand_dim_specification,
 )
@@ -31,4 +32,4 @@ from .layers import Similarity, Mex, dirichlet_init  # noqa: F401,E402
 
 __all__ = ["layers", "unsupervised", "torch_ops", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "mex_sum_pool", "similarity_mex_sum_pool", "similarity_output_shape", "mex_output_shape", "SimnetsError",
            "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad",
-           "sum_pooling_input_grad"]
+           "sum_pooling_input_grad", "mex_grads"]

@@ -15,7 +15,7 @@ EXPORTS = [
     "simnets_hip_sum_pool_input_grad",
     "simnets_hip_similarity_grad_workspace_bytes", "simnets_hip_similarity_input_grad",
     "simnets_hip_similarity_params_grad", "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
-    "simnets_hip_mex_offsets_grad",
+    "simnets_hip_mex_offsets_grad", "simnets_hip_mex_grads_workspace_bytes", "simnets_hip_mex_grads",
     "simnets_hip_mex_sum_pool_workspace_bytes", "simnets_hip_mex_sum_pool_fwd",
     "simnets_hip_similarity_mex_sum_pool_workspace_bytes", "simnets_hip_similarity_mex_sum_pool_fwd",
 ]
@@ -119,6 +119,8 @@ def lib():
         l.simnets_hip_mex_input_grad.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, C.c_size_t, P]
         l.simnets_hip_mex_offsets_grad.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, C.c_size_t,
                                                    P]
+        l.simnets_hip_mex_grads_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
+        l.simnets_hip_mex_grads.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, P, C.c_size_t, P]
         for name in ("simnets_similarity_out_shape", "simnets_hip_similarity_workspace_bytes",
                      "simnets_hip_similarity_fwd", "simnets_mex_calc_dims", "simnets_mex_out_shape",
                      "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
@@ -129,7 +131,8 @@ def lib():
                      "get_mex_offsets_nregions", "simnets_hip_similarity_grad_workspace_bytes",
                      "simnets_hip_similarity_input_grad", "simnets_hip_similarity_params_grad",
                      "simnets_hip_mex_grad_workspace_bytes", "simnets_hip_mex_input_grad",
-                     "simnets_hip_mex_offsets_grad", "simnets_hip_mex_sum_pool_workspace_bytes",
+                     "simnets_hip_mex_offsets_grad", "simnets_hip_mex_grads_workspace_bytes",
+                     "simnets_hip_mex_grads", "simnets_hip_mex_sum_pool_workspace_bytes",
                      "simnets_hip_mex_sum_pool_fwd", "simnets_hip_similarity_mex_sum_pool_workspace_bytes",
                      "simnets_hip_similarity_mex_sum_pool_fwd"):
             getattr(l, name).restype = C.c_int

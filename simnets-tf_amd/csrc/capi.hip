@@ -137,6 +137,35 @@ int simnets_hip_mex_offsets_grad(const simnets_mex_attrs *attrs, const int input
     return mex_grad_offsets(p, input, offsets, output, output_grad, offsets_grad, workspace, workspace_bytes, stream);
 }
 
+int simnets_hip_mex_grads_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], size_t *bytes)
+{
+    if (!bytes)
+        return SIMNETS_ERR_NULL_POINTER;
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    *bytes = mex_grads_workspace_bytes(p, true, true);
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                          const float *offsets, size_t offsets_count, const float *output, const float *output_grad,
+                          float *input_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
+                          void *stream)
+{
+    MexPlan p;
+    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    if (rc)
+        return rc;
+    if (!offsets || !offsets_grad || (p.B > 0 && (!input || !output || !output_grad || !input_grad)))
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(workspace, workspace_bytes, mex_grads_workspace_bytes(p, true, true)))
+        return SIMNETS_ERR_WORKSPACE;
+    return mex_grads(p, input, offsets, output, output_grad, input_grad, offsets_grad, workspace, workspace_bytes,
+                     stream);
+}
+
 int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                         const float *offsets, size_t offsets_count, float *output, void *workspace,
                         size_t workspace_bytes, void *stream)

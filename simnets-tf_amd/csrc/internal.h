@@ -63,6 +63,11 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
                     size_t workspace_bytes, void *stream);
 size_t mex_grad_input_workspace_bytes(const MexPlan &p);
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p);
+size_t mex_grads_workspace_bytes(const MexPlan &p, bool want_input, bool want_offsets);
+// either gradient or both: a null gradient pointer skips one
+int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
+              const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
+              size_t workspace_bytes, void *stream);
 int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
                    const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes, void *stream);
 int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,

@@ -836,168 +836,196 @@ int launch_factors(const MexPlan &p, const MexGradTiling &t, MexGradArgs &ga, vo
 
 }  // namespace
 
-// finite epsilon: the matrix-core kernels read the forward pass's packed offsets (groups of GM_TM instances)
-size_t mex_grad_input_workspace_bytes(const MexPlan &p)
+namespace {
+
+// Scratch of a gradient call, in this order: normalised offsets | packed offsets | offsets-gradient partial sums |
+// patch gradients of overlapping patches | partial input gradients of the instance split | factor buffers.
+struct MexGradScratch {
+    size_t norm, packed, partial, col, split, factors, total;
+    bool use_factors;
+};
+
+MexGradScratch mex_grad_scratch(const MexGradTiling &t, bool want_input, bool want_offsets)
 {
-    const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.packed_bytes + t.col_bytes + t.split_bytes + (t.factors_input ? t.factor_bytes : 0);
+    MexGradScratch w;
+    // both gradients in one call: the factors are formed once for the kernels that want them
+    w.use_factors = (want_input && t.factors_input) || (want_offsets && t.factors_offsets);
+    size_t at = 0;
+    w.norm = at;    at += t.norm_bytes;
+    w.packed = at;  at += t.packed_bytes;
+    w.partial = at; at += want_offsets ? t.partial_bytes : 0;
+    w.col = at;     at += want_input ? t.col_bytes : 0;
+    w.split = at;   at += want_input ? t.split_bytes : 0;
+    w.factors = at; at += w.use_factors ? t.factor_bytes : 0;
+    w.total = at;
+    return w;
 }
 
-size_t mex_grad_offsets_workspace_bytes(const MexPlan &p)
+}  // namespace
+
+size_t mex_grads_workspace_bytes(const MexPlan &p, bool want_input, bool want_offsets)
 {
-    const MexGradTiling t = mex_grad_tiling(p);
-    return t.norm_bytes + t.partial_bytes + t.packed_bytes + (t.factors_offsets ? t.factor_bytes : 0);
+    return mex_grad_scratch(mex_grad_tiling(p), want_input, want_offsets).total;
 }
 
-int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
-                          const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes,
-                          void *stream)
+size_t mex_grad_input_workspace_bytes(const MexPlan &p) { return mex_grads_workspace_bytes(p, true, false); }
+
+size_t mex_grad_offsets_workspace_bytes(const MexPlan &p) { return mex_grads_workspace_bytes(p, false, true); }
+
+// Either gradient or both (a null pointer skips one).  The offsets as the forward op used them, their packed form
+// and, where used, the factor buffers are prepared once and shared.
+int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
+              const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
+              size_t workspace_bytes, void *stream)
 {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (workspace_bytes < mex_grad_input_workspace_bytes(p))
+    const bool want_input = input_grad != nullptr, want_offsets = offsets_grad != nullptr;
+    const MexGradTiling t = mex_grad_tiling(p);
+    const MexGradScratch w = mex_grad_scratch(t, want_input, want_offsets);
+    if (workspace_bytes < w.total)
         return SIMNETS_ERR_WORKSPACE;
     const simnets_mex_dims &d = p.d;
+    const long long n_in = (long long)p.B * p.C * p.H * p.W;
+    const long long n_off = (long long)d.num_regions * d.M * d.K;
+    if (p.B == 0) {  // an empty batch has an empty input gradient and a zero offsets gradient
+        if (want_offsets) {
+            hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_off + 255) / 256, 65535)),
+                               dim3(256), 0, s, offsets_grad, n_off);
+            return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+        }
+        return SIMNETS_OK;
+    }
+    if ((n_in + 255) / 256 > 0x7fffffffLL)
+        return SIMNETS_ERR_TOO_LARGE;
+    char *ws = reinterpret_cast<char *>(workspace);
+
     MexGradArgs ga;
     ga.k = mex_kernel_args(p);
     ga.k.in = input;
-    int rc = prepare_offsets(p, offsets, workspace, s, &ga.off);
+    int rc = prepare_offsets(p, offsets, ws + w.norm, s, &ga.off);
     if (rc)
         return rc;
-    ga.out = output; ga.g = output_grad; ga.dx = input_grad; ga.partial = nullptr;
-    const MexGradTiling t = mex_grad_tiling(p);
-    ga.overlap = t.overlap ? 1 : 0;
-    ga.col = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes);
-    ga.msplit = t.msplit; ga.mg_per_split = t.mg_per_split;
-    ga.dx_splits = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes +
-                                             t.col_bytes);
+    ga.out = output; ga.g = output_grad;
+    ga.dx = input_grad;
+    ga.partial = reinterpret_cast<float *>(ws + w.partial);
+    ga.overlap = 0;
+    ga.col = reinterpret_cast<float *>(ws + w.col);
+    ga.msplit = 1; ga.mg_per_split = (d.M + GM_TM - 1) / GM_TM;
+    ga.dx_splits = reinterpret_cast<float *>(ws + w.split);
     ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
-
-    const long long n_in = (long long)p.B * p.C * p.H * p.W;
-    if (n_in == 0)
-        return SIMNETS_OK;
-    if ((n_in + 255) / 256 > 0x7fffffffLL)
-        return SIMNETS_ERR_TOO_LARGE;
-    const bool tiles_input = t.tiles_input;
-    if (!t.overlap && !tiles_input) {
-        // every element belongs to at most one patch, which stores its gradient; the others keep 0
-        hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
-                           dim3(256), 0, s, input_grad, n_in);
-        if (hipGetLastError() != hipSuccess)
-            return SIMNETS_ERR_HIP;
-    }
-    const long long gx = (long long)d.num_regions * ga.cpr;
     if (t.mfma) {
-        void *packed = reinterpret_cast<char *>(workspace) + t.norm_bytes;
-        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed, &ga.k, stream);
+        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream);
         if (rc)
             return rc;
-        const int gy = (d.K + GM_KT - 1) / GM_KT;
-        if (gx > 0x7fffffffLL || gy > 65535)
-            return SIMNETS_ERR_TOO_LARGE;
-        if (t.factors_input) {
-            rc = launch_factors(p, t, ga, reinterpret_cast<char *>(workspace) + t.norm_bytes + t.packed_bytes +
-                                              t.col_bytes + t.split_bytes, s);
+        if (w.use_factors) {
+            rc = launch_factors(p, t, ga, ws + w.factors, s);
             if (rc)
                 return rc;
         }
-        if (gx > 0)
-            hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)t.msplit),
-                               dim3(256), 0, s, ga);
-        if (gx > 0 && t.msplit > 1) {
+    }
+
+    if (want_input) {
+        MexGradArgs gi = ga;
+        gi.overlap = t.overlap ? 1 : 0;
+        gi.msplit = t.msplit; gi.mg_per_split = t.mg_per_split;
+        gi.pxl = 1;
+        gi.cpr = (ga.k.slots + 63) / 64;
+        if (!t.factors_input)
+            gi.wbuf = gi.exbuf = nullptr;  // (each gradient forms its factors as it does in a call of its own)
+        if (!t.overlap && !t.tiles_input) {
+            // every element belongs to at most one patch, which stores its gradient; the others keep 0 (patches
+            // that tile the input exactly write every element; overlapping ones go through mex_col2im_kernel)
+            hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
+                               dim3(256), 0, s, input_grad, n_in);
             if (hipGetLastError() != hipSuccess)
                 return SIMNETS_ERR_HIP;
-            hipLaunchKernelGGL(mex_sum_splits_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
-                               dim3(256), 0, s, ga.dx_splits, n_in, t.msplit, input_grad);
         }
-    } else {
-        const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
-        if (gx > 0x7fffffffLL || gy > 65535)
-            return SIMNETS_ERR_TOO_LARGE;
-        if (gx > 0)
-            hipLaunchKernelGGL(mex_grad_input_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, ga);
-    }
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
-    if (t.overlap) {
-        hipLaunchKernelGGL(mex_col2im_kernel, dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, s, ga.k, ga.col,
-                           input_grad, n_in);
+        const long long gx = (long long)d.num_regions * gi.cpr;
+        if (t.mfma) {
+            const int gy = (d.K + GM_KT - 1) / GM_KT;
+            if (gx > 0x7fffffffLL || gy > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            if (gx > 0)
+                hipLaunchKernelGGL(mex_grad_input_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)t.msplit),
+                                   dim3(256), 0, s, gi);
+            if (gx > 0 && t.msplit > 1) {
+                if (hipGetLastError() != hipSuccess)
+                    return SIMNETS_ERR_HIP;
+                hipLaunchKernelGGL(mex_sum_splits_kernel,
+                                   dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)), dim3(256), 0, s,
+                                   gi.dx_splits, n_in, t.msplit, input_grad);
+            }
+        } else {
+            const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);
+            if (gx > 0x7fffffffLL || gy > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            if (gx > 0)
+                hipLaunchKernelGGL(mex_grad_input_kernel, dim3((unsigned)gx, (unsigned)gy), dim3(256), 0, s, gi);
+        }
         if (hipGetLastError() != hipSuccess)
             return SIMNETS_ERR_HIP;
+        if (t.overlap) {
+            hipLaunchKernelGGL(mex_col2im_kernel, dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, s, gi.k, gi.col,
+                               input_grad, n_in);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
+    }
+
+    if (want_offsets) {
+        MexGradArgs go = ga;
+        go.dx = nullptr; go.col = nullptr; go.dx_splits = nullptr;
+        go.overlap = 0; go.msplit = 1;
+        go.pxl = t.pxl;
+        go.cpr = t.cpr_offsets;
+        if (!t.factors_offsets)
+            go.wbuf = go.exbuf = nullptr;
+        const long long gx = (long long)d.num_regions * go.cpr;
+        if (t.mfma) {
+            const int gy = (d.M + GOM_MT - 1) / GOM_MT, gz = (d.K + GOM_KT - 1) / GOM_KT;
+            if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            hipLaunchKernelGGL(mex_grad_offsets_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256),
+                               0, s, go);
+        } else {
+            const int gy = (d.M + 4 * GO_MT - 1) / (4 * GO_MT);
+            const int gz = (d.K + GO_KT - 1) / GO_KT;
+            if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            hipLaunchKernelGGL(mex_grad_offsets_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
+                               go);
+        }
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+        hipLaunchKernelGGL(mex_grad_offsets_finish_kernel,
+                           dim3((unsigned)std::min<long long>((n_off + 31) / 32, 65535)), dim3(256), 0, s, go.partial,
+                           n_off, go.cpr, offsets_grad);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+        if (p.normalize_offsets) {
+            const long long rows = (long long)d.num_regions * d.M;
+            hipLaunchKernelGGL(mex_normalize_rows_backward_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s,
+                               go.off, rows, d.K, offsets_grad);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
     }
     return SIMNETS_OK;
 }
 
-int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,
-                            const float *output_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
-                            void *stream)
+int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
+                   const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes, void *stream)
 {
-    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    if (workspace_bytes < mex_grad_offsets_workspace_bytes(p))
-        return SIMNETS_ERR_WORKSPACE;
-    const simnets_mex_dims &d = p.d;
-    if (p.B == 0) {  // an empty batch has a zero gradient
-        const long long n = (long long)d.num_regions * d.M * d.K;
-        hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 65535)), dim3(256),
-                           0, s, offsets_grad, n);
-        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
-    }
-    const MexGradTiling t = mex_grad_tiling(p);
-    MexGradArgs ga;
-    ga.k = mex_kernel_args(p);
-    ga.k.in = input;
-    int rc = prepare_offsets(p, offsets, workspace, s, &ga.off);
-    if (rc)
-        return rc;
-    ga.out = output; ga.g = output_grad; ga.dx = nullptr;
-    ga.partial = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + t.norm_bytes);
-    ga.overlap = 0; ga.col = nullptr;
-    ga.msplit = 1; ga.mg_per_split = ga.k.n_mgroups; ga.dx_splits = nullptr;
-    ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
-    ga.pxl = t.pxl;
-    ga.cpr = t.cpr_offsets;
+    return mex_grads(p, input, offsets, output, output_grad, input_grad, nullptr, workspace, workspace_bytes, stream);
+}
 
-    const long long gx = (long long)d.num_regions * ga.cpr;
-    if (t.mfma) {
-        void *packed = reinterpret_cast<char *>(workspace) + t.norm_bytes + t.partial_bytes;
-        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed, &ga.k, stream);
-        if (rc)
-            return rc;
-        const int gy = (d.M + GOM_MT - 1) / GOM_MT, gz = (d.K + GOM_KT - 1) / GOM_KT;
-        if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
-            return SIMNETS_ERR_TOO_LARGE;
-        if (t.factors_offsets) {
-            rc = launch_factors(p, t, ga, reinterpret_cast<char *>(workspace) + t.norm_bytes + t.partial_bytes +
-                                              t.packed_bytes, s);
-            if (rc)
-                return rc;
-        }
-        hipLaunchKernelGGL(mex_grad_offsets_mfma_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
-                           ga);
-    } else {
-        const int gy = (d.M + 4 * GO_MT - 1) / (4 * GO_MT);
-        const int gz = (d.K + GO_KT - 1) / GO_KT;
-        if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
-            return SIMNETS_ERR_TOO_LARGE;
-        hipLaunchKernelGGL(mex_grad_offsets_kernel, dim3((unsigned)gx, (unsigned)gy, (unsigned)gz), dim3(256), 0, s,
-                           ga);
-    }
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
-    const long long n = (long long)d.num_regions * d.M * d.K;
-    hipLaunchKernelGGL(mex_grad_offsets_finish_kernel, dim3((unsigned)std::min<long long>((n + 31) / 32, 65535)),
-                       dim3(256), 0, s, ga.partial, n, ga.cpr, offsets_grad);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
-    if (p.normalize_offsets) {
-        const long long rows = (long long)d.num_regions * d.M;
-        hipLaunchKernelGGL(mex_normalize_rows_backward_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s, ga.off,
-                           rows, d.K, offsets_grad);
-        if (hipGetLastError() != hipSuccess)
-            return SIMNETS_ERR_HIP;
-    }
-    return SIMNETS_OK;
+int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,
+                     const float *output_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
+                     void *stream)
+{
+    return mex_grads(p, input, offsets, output, output_grad, nullptr, offsets_grad, workspace, workspace_bytes, stream);
 }
 
 }  // namespace simnets

@@ -54,9 +54,11 @@ class MexFunction(torch.autograd.Function):
         input, offsets, out = ctx.saved_tensors
         grad = grad.contiguous()
         gi = go = None
-        if ctx.needs_input_grad[0]:
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
+            gi, go = ops.mex_grads(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
+        elif ctx.needs_input_grad[0]:
             gi = ops.mex_input_grad(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
-        if ctx.needs_input_grad[1]:
+        elif ctx.needs_input_grad[1]:
             go = ops.mex_offsets_grad(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
         return gi, go, None, None
 

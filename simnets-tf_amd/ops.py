@@ -426,6 +426,30 @@ def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax
     return doff
 
 
+def mex_grads(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
+              blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+              use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+              normalize_offsets=False):
+    """`(mex_input_grad(...), mex_offsets_grad(...))` as one call of the library: the same results bit for bit, with
+    the work both share (offsets normalisation and packing, per-pixel factors) done once.  What the gradient
+    registered for the Mex op (python/simnets/ops/mex.py:47-81) computes."""
+    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
+        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
+        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
+        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
+        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_grads_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
+    ws = _workspace(x.device, nbytes.value)
+    dx, doff = torch.empty_like(x), torch.empty_like(off)
+    with _on_device(x.device):
+        stream = torch.cuda.current_stream(x.device).cuda_stream
+        _check(l.simnets_hip_mex_grads(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
+                                       g.data_ptr(), dx.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(),
+                                       stream))
+    return dx, doff
+
+
 def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
                  blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
                  use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,

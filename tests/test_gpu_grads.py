@@ -502,3 +502,29 @@ def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, sp
     if spread == "mixed":
         off[::2] *= 300
     check_mex_grads(pkg, x, off, 200, **kw)
+
+
+@pytest.mark.parametrize("case", [
+    dict(im=(5, 40, 6, 6), n=70, kw=dict(blocks=[40, 1, 1], strides=[40, 1, 1], padding=[0, 0, 0],
+                                         unshared_offset_region=[2], epsilon=2.0, softmax_mode=True)),
+    dict(im=(3, 6, 12, 12), n=10, kw=dict(blocks=[3, 3, 3], strides=[2, 1, 1], padding=[1, 1, 1], epsilon=-1.5,
+                                          use_unshared_regions=False, shared_offset_region=[2])),   # overlapping patches
+    dict(im=(4, 9, 7, 5), n=6, kw=dict(blocks=[3, 2, 2], strides=[3, 2, 2], padding=[0, 1, 0],
+                                       epsilon=-math.inf, softmax_mode=False)),                     # infinite epsilon
+    dict(im=(6, 200, 4, 4), n=200, kw=dict(blocks=[200, 1, 1], strides=[200, 1, 1], padding=[0, 0, 0],
+                                           unshared_offset_region=[2], epsilon=1.0, softmax_mode=True)),  # factor buffers
+])
+@pytest.mark.parametrize("normalize", [False, True])
+def test_mex_grads_in_one_call_equal_the_two_calls(pkg, case, normalize):
+    """mex_grads = (mex_input_grad, mex_offsets_grad) bit for bit, with the shared preparation done once."""
+    kw = dict(case["kw"], normalize_offsets=normalize)
+    x, off = mex_case(33, case["im"], case["n"], **case["kw"])
+    off = off * 0.5
+    X, O = dev(x), dev(off)
+    Y = pkg.mex(X, O, case["n"], **kw)
+    G = torch.randn_like(Y)
+    dx, doff = pkg.mex_grads(X, O, Y, G, case["n"], **kw)
+    dx1 = pkg.mex_input_grad(X, O, Y, G, case["n"], **kw)
+    do1 = pkg.mex_offsets_grad(X, O, Y, G, case["n"], **kw)
+    assert torch.equal(do1, doff)
+    assert torch.equal(dx1, dx)
