@@ -944,20 +944,21 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
 }
 
 namespace {
-__global__ void sum_pool_kernel(const float *__restrict__ in, float *__restrict__ out, long long total, int H, int W,
-                                int Ho, int Wo, int ph, int pw)
+// I: index type (int while the element count fits: 64-bit divisions cost several times the rest of the kernel)
+template <typename I>
+__global__ void sum_pool_kernel(const float *__restrict__ in, float *__restrict__ out, I total, int H, int W, int Ho,
+                                int Wo, int ph, int pw)
 {
-    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (long long)gridDim.x * blockDim.x) {
-        const int wo = (int)(idx % Wo);
-        const long long t = idx / Wo;
-        const int ho = (int)(t % Ho);
-        const long long bc = t / Ho;
-        const float *src = in + (bc * H + (long long)ho * ph) * W + (long long)wo * pw;
+    for (I idx = (I)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (I)gridDim.x * blockDim.x) {
+        const I wo = idx % Wo;
+        const I t = idx / Wo;
+        const I ho = t % Ho;
+        const I bc = t / Ho;
+        const float *src = in + ((size_t)bc * H + (size_t)ho * ph) * W + (size_t)wo * pw;
         float acc = 0.0f;
         for (int i = 0; i < ph; ++i)
             for (int j = 0; j < pw; ++j)
-                acc += src[(long long)i * W + j];
+                acc += src[(size_t)i * W + j];
         out[idx] = acc;
     }
 }
@@ -966,17 +967,17 @@ __global__ void sum_pool_kernel(const float *__restrict__ in, float *__restrict_
 namespace {
 // gradient of the sum pooling: every input element of a window receives the window's gradient, the elements
 // of a dropped trailing row or column receive 0
-__global__ void sum_pool_grad_kernel(const float *__restrict__ gout, float *__restrict__ gin, long long total, int H,
-                                     int W, int Ho, int Wo, int ph, int pw)
+template <typename I>
+__global__ void sum_pool_grad_kernel(const float *__restrict__ gout, float *__restrict__ gin, I total, int H, int W,
+                                     int Ho, int Wo, int ph, int pw)
 {
-    for (long long idx = (long long)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-         idx += (long long)gridDim.x * blockDim.x) {
-        const int w = (int)(idx % W);
-        const long long t = idx / W;
-        const int h = (int)(t % H);
-        const long long bc = t / H;
-        const int ho = h / ph, wo = w / pw;
-        gin[idx] = (ho < Ho && wo < Wo) ? gout[(bc * Ho + ho) * Wo + wo] : 0.0f;
+    for (I idx = (I)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (I)gridDim.x * blockDim.x) {
+        const I w = idx % W;
+        const I t = idx / W;
+        const I h = t % H;
+        const I bc = t / H;
+        const I ho = h / ph, wo = w / pw;
+        gin[idx] = (ho < Ho && wo < Wo) ? gout[((size_t)bc * Ho + ho) * Wo + wo] : 0.0f;
     }
 }
 }  // namespace
@@ -987,9 +988,14 @@ int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float
     const long long total = (long long)B * C * H * W;
     if (total == 0)
         return SIMNETS_OK;
-    const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
-    hipLaunchKernelGGL(sum_pool_grad_kernel, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
-                       output_grad, input_grad, total, H, W, H / ph, W / pw, ph, pw);
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (total + 256LL * blocks < 0x7fffffffLL)
+        hipLaunchKernelGGL(sum_pool_grad_kernel<int>, dim3(blocks), dim3(256), 0, s, output_grad, input_grad, (int)total,
+                           H, W, H / ph, W / pw, ph, pw);
+    else
+        hipLaunchKernelGGL(sum_pool_grad_kernel<long long>, dim3(blocks), dim3(256), 0, s, output_grad, input_grad,
+                           total, H, W, H / ph, W / pw, ph, pw);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
@@ -999,9 +1005,14 @@ int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *inp
     const long long total = (long long)B * C * Ho * Wo;
     if (total == 0)
         return SIMNETS_OK;
-    const int blocks = (int)std::min<long long>((total + 255) / 256, 65535);
-    hipLaunchKernelGGL(sum_pool_kernel, dim3(blocks), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), input,
-                       output, total, H, W, Ho, Wo, ph, pw);
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (total + 256LL * blocks < 0x7fffffffLL)
+        hipLaunchKernelGGL(sum_pool_kernel<int>, dim3(blocks), dim3(256), 0, s, input, output, (int)total, H, W, Ho, Wo,
+                           ph, pw);
+    else
+        hipLaunchKernelGGL(sum_pool_kernel<long long>, dim3(blocks), dim3(256), 0, s, input, output, total, H, W, Ho,
+                           Wo, ph, pw);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
