@@ -797,6 +797,9 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     // matrix-core form, one chunk: two pixels per step, rows = templates (g at ga, second tile a1_off further),
     // columns = patch elements (xc, xc^2, keep from xb); `ps` floats from pixel to pixel; the reads of the next step
     // are issued before this step's matrix instructions
+    // a wave whose 64 templates or 32 patch elements all lie past the last one only takes part in the staging
+    // (few templates or patch elements: the first layer of a network)
+    const bool wave_has_work = o_wg + wo * 64 < a.O && k_wg + wk * 32 < a.K;
     auto mfma_steps = [&](const float *ga_, int a1_off, const float *xb_, int ps) {
         float a0 = ga_[0], a1 = ga_[a1_off], xv_ = xb_[0];
 #pragma unroll 4
@@ -889,7 +892,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             const bool more = chunk + 1 < chunk_end;
             if (more)
                 row_load(chunk + 1);   // in flight while this chunk is used
-            mfma_steps(gs[buf] + (wo * 64 + mcol) * PR + mhalf, 32 * PR, xs[buf] + (wk * 32 + mcol) * PR + mhalf, 1);
+            if (wave_has_work)
+                mfma_steps(gs[buf] + (wo * 64 + mcol) * PR + mhalf, 32 * PR, xs[buf] + (wk * 32 + mcol) * PR + mhalf, 1);
             if (more)
                 row_store(buf ^ 1);
             __syncthreads();  // the other buffer is complete; nobody reads this one any more
@@ -1035,8 +1039,9 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
             }
         };
         if constexpr (MF) {
-            mfma_steps(gs[buf] + ((size_t)(wo * 16 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 8 * PCP * 4,
-                       xs[buf] + ((size_t)(wk * 8 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 4);
+            if (wave_has_work)
+                mfma_steps(gs[buf] + ((size_t)(wo * 16 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 8 * PCP * 4,
+                           xs[buf] + ((size_t)(wk * 8 + (mcol >> 2)) * PCP + mhalf) * 4 + (mcol & 3), 4);
         } else if (SGN && !nan_chunk) {
             pixels(compute_sgn);
         } else if (SGN) {
