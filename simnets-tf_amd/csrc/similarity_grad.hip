@@ -1203,8 +1203,10 @@ GpTiling gp_tiling(const SimPlan &p)
     S = std::min(S, std::max(1, t.nchunks));
     // every split costs a prologue, an epilogue and a slab of partial sums: at least 8 chunks (256 pixels) per
     // split as long as that still leaves two workgroups per compute unit
-    if (t.nchunks / 8 >= 512 / tiles)
+    // (fewer than 8 chunks in all: one split, decided above; with more than 512 tiles the right-hand side is 0)
+    if (t.nchunks >= 8 && t.nchunks / 8 >= 512 / tiles)
         S = std::min(S, t.nchunks / 8);
+    S = std::max(S, 1);
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;

@@ -37,7 +37,9 @@ _workspaces = {}
 def _workspace(device, nbytes):
     """A scratch tensor per (device, current stream), grown on demand and reused across calls: the kernels that
     use it are ordered on that stream, and calls on different streams never share one."""
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    # a buffer first allocated during stream capture lives in that graph's private pool: kept apart from the
+    # eager calls' buffer, which a later replay of the graph must not share
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream, torch.cuda.is_current_stream_capturing())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
@@ -536,10 +538,16 @@ def sum_pooling(input, pool_size=(2, 2), out=None):
     """Non-overlapping 'valid' sum pooling: the AveragePooling2D * area glue of the reference's
     missing-data example (README.md:108-111)."""
     x = _require_cuda_f32("input", input)
+    if x.dim() != 4:
+        raise SimnetsError(-15)
     ph, pw = int(pool_size[0]), int(pool_size[1])
     B, Cc, H, W = x.shape
+    oshape = (B, Cc, H // max(ph, 1), W // max(pw, 1))
     if out is None:
-        out = torch.empty((B, Cc, H // max(ph, 1), W // max(pw, 1)), dtype=torch.float32, device=x.device)
+        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
+    else:
+        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32 \
+            and out.device == x.device
     with _on_device(x.device):
         stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),

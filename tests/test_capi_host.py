@@ -308,3 +308,21 @@ def test_sum_pool_input_grad_validates_like_the_forward_call(pkg):
     assert l.simnets_hip_sum_pool_input_grad(I4(2, 3, 1, 8), 2, 2, None, None, None) < 0      # empty output
     assert l.simnets_hip_sum_pool_input_grad(I4(0, 3, 8, 8), 2, 2, None, None, None) == 0     # empty batch: nothing to do
     assert l.simnets_hip_sum_pool_input_grad(I4(2, 3, 8, 8), 2, 2, None, None, None) < 0      # null pointers
+
+
+def test_parameter_gradient_tiling_with_many_tiles_and_few_pixels(pkg):
+    # dense-layer-like Similarity (1x1 output): more than 512 template x patch-element tiles, fewer than 256 output
+    # pixels, and the empty batch: the pixel-split arithmetic must not divide by zero (host only, no launch)
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    a = pkg.ops.similarity_attrs(blocks=[8, 8], strides=[1, 1], padding=[0, 0])
+    for batch in (4, 1, 0):
+        wp = C.c_size_t()
+        assert l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), I4(batch, 64, 8, 8), I4(1100, 64, 8, 8), None,
+                                                             C.byref(wp)) == 0
+        assert wp.value >= 2 * 1100 * 64 * 8 * 8 * 4
+    a = pkg.ops.similarity_attrs(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    wp = C.c_size_t()
+    assert l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), I4(0, 64, 32, 32), I4(128, 64, 3, 3), None,
+                                                         C.byref(wp)) == 0
+
