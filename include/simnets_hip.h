@@ -52,7 +52,8 @@ typedef enum simnets_status {
     SIMNETS_ERR_WORKSPACE = -17,            /* workspace missing, too small or misaligned */
     SIMNETS_ERR_ALGO = -18,                 /* requested algorithm cannot serve these attributes */
     SIMNETS_ERR_TOO_LARGE = -19,            /* a dimension product exceeds 32-bit indexing */
-    SIMNETS_ERR_HIP = -20                   /* a HIP call or kernel launch failed */
+    SIMNETS_ERR_HIP = -20,                  /* a HIP call or kernel launch failed */
+    SIMNETS_ERR_STATIC_SCRATCH = -21        /* the call needs more scratch than SIMNETS_HIP_STATIC_SCRATCH_BYTES */
 } simnets_status;
 
 const char *simnets_hip_strerror(int status);
@@ -115,6 +116,19 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
                                const int templates_shape[4], const int weights_shape[4], const float *input,
                                const float *templates, const float *weights, float *output, void *workspace,
                                size_t workspace_bytes, void *stream);
+
+/* simnets_hip_similarity_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc) and so have no workspace to pass.  It has no counterpart in the
+ * reference.  Same arguments minus the workspace, same kernels, same results bit for bit; the scratch is a fixed
+ * device array of SIMNETS_HIP_STATIC_SCRATCH_BYTES inside the library (one copy per GPU, held until the process
+ * ends) and the call allocates nothing.  Calls whose simnets_hip_similarity_workspace_bytes exceeds that size
+ * return SIMNETS_ERR_STATIC_SCRATCH before anything is launched.  All calls on one GPU share that GPU's array:
+ * calls that may overlap on one GPU (different streams, different threads) race; order them on one stream.  The
+ * first call on a device looks up the array's address (hipGetSymbolAddress): make it outside graph capture. */
+#define SIMNETS_HIP_STATIC_SCRATCH_BYTES (4u << 20)
+int simnets_hip_similarity_fwd_static(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                      const int templates_shape[4], const int weights_shape[4], const float *input,
+                                      const float *templates, const float *weights, float *output, void *stream);
 
 /* Backward.  Scratch sizes of the two gradient calls (either pointer may be NULL). */
 int simnets_hip_similarity_grad_workspace_bytes(const simnets_similarity_attrs *attrs, const int input_shape[4],

@@ -9,7 +9,7 @@ LIB_PATH = os.path.join(HERE, "libsimnets_hip.so")
 EXPORTS = [
     "simnets_hip_strerror", "simnets_hip_abi_version",
     "simnets_similarity_attrs_default", "simnets_similarity_out_shape",
-    "simnets_hip_similarity_workspace_bytes", "simnets_hip_similarity_fwd",
+    "simnets_hip_similarity_workspace_bytes", "simnets_hip_similarity_fwd", "simnets_hip_similarity_fwd_static",
     "simnets_mex_attrs_default", "simnets_mex_calc_dims", "simnets_mex_out_shape", "get_mex_offsets_nregions",
     "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",
     "simnets_hip_sum_pool_input_grad",
@@ -21,6 +21,7 @@ EXPORTS = [
 ]
 
 SIM_L1, SIM_L2 = 0, 1
+STATIC_SCRATCH_BYTES = 4 << 20  # SIMNETS_HIP_STATIC_SCRATCH_BYTES
 ALGO_AUTO, ALGO_DIRECT, ALGO_SQRTW, ALGO_MFMA = 0, 1, 2, 3
 ALGOS = {None: ALGO_AUTO, "auto": ALGO_AUTO, "direct": ALGO_DIRECT, "sqrtw": ALGO_SQRTW, "mfma": ALGO_MFMA}
 
@@ -92,6 +93,8 @@ def lib():
         l.simnets_hip_similarity_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4,
                                                              C.POINTER(C.c_size_t)]
         l.simnets_hip_similarity_fwd.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P, C.c_size_t, P]
+        l.simnets_hip_similarity_fwd_static.argtypes = [C.POINTER(SimilarityAttrs), I4, I4, I4, P, P, P, P, P]
+        l.simnets_hip_similarity_fwd_static.restype = C.c_int
         l.simnets_mex_attrs_default.argtypes = [C.POINTER(MexAttrs)]
         l.simnets_mex_attrs_default.restype = None
         l.simnets_mex_calc_dims.argtypes = [C.POINTER(MexAttrs), I3, C.POINTER(MexDims)]

@@ -1,6 +1,8 @@
 // Compute entry points of the C ABI (include/simnets_hip.h): validate on the host, then enqueue.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "internal.h"
 
 namespace simnets {
@@ -36,7 +38,57 @@ static bool workspace_ok(const void *workspace, size_t have, size_t need)
     return need == 0 || (workspace && have >= need && (reinterpret_cast<uintptr_t>(workspace) & 255) == 0);
 }
 
+// Scratch of simnets_hip_similarity_fwd_static: a fixed device array instead of a caller workspace.  Every GPU the
+// library runs on holds its own copy, at its own address, until the process ends.  In host code the array's name
+// is only a handle for hipGetSymbolAddress: the device address it yields (per device) is what kernels receive.
+static __device__ __align__(256) unsigned char scratch[SIMNETS_HIP_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxDevices = 64;
+std::atomic<void *> g_scratch_ptr[kMaxDevices];
+
+// Device address of `scratch` on the current device, looked up once per device.
+int static_scratch(void **ptr)
+{
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices)
+        return SIMNETS_ERR_HIP;
+    void *p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p)
+            return SIMNETS_ERR_HIP;
+        g_scratch_ptr[dev].store(p, std::memory_order_release);  // racing threads store the same address
+    }
+    *ptr = p;
+    return SIMNETS_OK;
+}
+}  // namespace
+
 extern "C" {
+
+int simnets_hip_similarity_fwd_static(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                      const int templates_shape[4], const int weights_shape[4], const float *input,
+                                      const float *templates, const float *weights, float *output, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, weights_shape, &p);
+    if (rc)
+        return rc;
+    const size_t need = sim_workspace_bytes(p);
+    if (need > SIMNETS_HIP_STATIC_SCRATCH_BYTES)
+        return SIMNETS_ERR_STATIC_SCRATCH;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !templates || !weights || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    void *ws = nullptr;
+    const int rs = static_scratch(&ws);
+    if (rs)
+        return rs;
+    // the pack and guard-prep kernels rewrite every part of the scratch the main kernel reads (parameters,
+    // tables, thresholds, cleared flags), so nothing of an earlier call survives into this one
+    return sim_launch(p, input, templates, weights, output, ws, SIMNETS_HIP_STATIC_SCRATCH_BYTES, stream);
+}
 
 int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int input_shape[4],
                                const int templates_shape[4], const int weights_shape[4], const float *input,

@@ -267,6 +267,7 @@ const char *simnets_hip_strerror(int status)
     case SIMNETS_ERR_ALGO: return "the requested algorithm does not support these attributes";
     case SIMNETS_ERR_TOO_LARGE: return "a per-image dimension product exceeds 32-bit indexing";
     case SIMNETS_ERR_HIP: return "a HIP runtime call or kernel launch failed (no usable gfx950 device?)";
+    case SIMNETS_ERR_STATIC_SCRATCH: return "the call needs more scratch than the library's static device buffer holds (SIMNETS_HIP_STATIC_SCRATCH_BYTES); use the entry point that takes a workspace";
     default: return "unknown simnets status";
     }
 }

@@ -326,3 +326,23 @@ def test_parameter_gradient_tiling_with_many_tiles_and_few_pixels(pkg):
     assert l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), I4(0, 64, 32, 32), I4(128, 64, 3, 3), None,
                                                          C.byref(wp)) == 0
 
+
+def test_static_scratch_entry_point_validates_and_bounds_its_scratch(pkg):
+    # simnets_hip_similarity_fwd_static: same validation as the workspace entry point, plus the size limit of the
+    # library's fixed device array; all decided on the host before anything touches a device
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    a = pkg.ops.similarity_attrs(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    f = l.simnets_hip_similarity_fwd_static
+    big = I4(1024, 64, 3, 3)
+    need = C.c_size_t()
+    assert l.simnets_hip_similarity_workspace_bytes(C.byref(a), I4(1, 64, 8, 8), big, C.byref(need)) == 0
+    assert need.value > pkg._lib.STATIC_SCRATCH_BYTES
+    assert f(C.byref(a), I4(1, 64, 8, 8), big, big, 256, 256, 256, 256, None) == -21
+    assert "scratch" in pkg._lib.strerror(-21)
+    small = I4(8, 64, 3, 3)
+    assert f(C.byref(a), I4(0, 64, 8, 8), small, small, None, None, None, None, None) == 0     # empty batch
+    assert f(C.byref(a), I4(1, 64, 8, 8), small, small, None, 256, 256, 256, None) == -1       # null input
+    assert f(C.byref(a), I4(1, 63, 8, 8), small, small, 256, 256, 256, 256, None) == -8        # channel mismatch
+    bad = pkg.ops.similarity_attrs(blocks=[3, 3], ignore_nan_input=True)
+    assert f(C.byref(bad), I4(1, 64, 8, 8), small, small, 256, 256, 256, 256, None) == -7
