@@ -56,3 +56,22 @@ def config3(batch=256, seed=1234, channels=64, size=32, templates=128):
     w = np.random.default_rng(3456).uniform(0.1, 2.0, size=t.shape).astype(np.float32)
     kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
     return x, t, w, kw
+
+
+def config4_stack(batch=512):
+    """The missing-data network (examples/mnist_ght_model_missing_data.py:81-112 of the reference): Similarity on
+    1x28x28 images with 25 % NaN pixels, four MEX layers (64, 128, 256, 512 instances over all channels of a pixel,
+    offsets unshared over 2x2) each followed by 2x2 sum pooling, and a MEX layer to 10 classes.
+    Returns (x, templates, weights, similarity kwargs, [(offsets, num_instances, mex kwargs)] x 4, (offsets, 10, kwargs))."""
+    x, t, w, skw = config1(batch=batch, nan_frac=0.25)
+    g = np.random.default_rng(4567)
+    layers, ch, size = [], 32, 16
+    for _ in range(4):
+        n = ch * 2
+        off = (g.normal(size=(4 if size > 1 else 1, n, ch, 1, 1)) * 0.1).astype(np.float32)
+        layers.append((off, n, dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1],
+                                    unshared_offset_region=[2])))
+        ch, size = n, size // 2
+    offl = (g.normal(size=(1, 10, ch, 1, 1)) * 0.1).astype(np.float32)
+    last = (offl, 10, dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1], shared_offset_region=[1]))
+    return x, t, w, skw, layers, last
