@@ -37,6 +37,7 @@ def grad_err(got, want):
 
 def assert_grad_close(got, want32, want64, what):
     e_gpu, e_ref = grad_err(got, want64), grad_err(want32, want64)
+    print("%s: gpu %.3g, fp32 reference %.3g (of max(|want|, 1%% of the scale), against fp64)" % (what, e_gpu, e_ref))
     assert e_gpu <= max(GRAD_TOL, 2.0 * e_ref), "%s: gpu %.3g, fp32 reference %.3g" % (what, e_gpu, e_ref)
 
 
@@ -199,31 +200,54 @@ def test_similarity_grads_conv_scale_shape_small_batch(pkg, func):
     check_sim_grads(pkg, x, t, w, similarity_function=func, **kw)
 
 
-def test_similarity_grads_conv_scale_full_batch_properties(pkg):
-    """Full config-3 batch: the input gradient of an image depends on that image only (checked against the
-    oracle on two images), and the parameter gradients are additive over the batch (sum of two half-batch
-    calls) and linear in the output gradient."""
+def oracle_params_grad_over_batch(x, t, w, g, kw, dtype, threads=8):
+    """Parameter gradients of the oracle summed over a large batch.  fp32: one call, images accumulated one after
+    the other like the reference's batch loop.  fp64 (the exact value, for which the order does not matter at the
+    tolerances used here): the batch split over threads, partial sums added at the end."""
+    from concurrent.futures import ThreadPoolExecutor
+    if dtype == np.float32:
+        return orc.similarity_params_grad(x, t, w, g, **kw)
+    t64, w64 = f64(t, w)
+    chunks = np.array_split(np.arange(len(x)), threads)
+    with ThreadPoolExecutor(threads) as ex:
+        parts = list(ex.map(lambda c: orc.similarity_params_grad(x[c].astype(np.float64), t64, w64,
+                                                                 g[c].astype(np.float64), **kw), chunks))
+    return sum(p[0] for p in parts), sum(p[1] for p in parts)
+
+
+@pytest.mark.parametrize("func", ["L2", "L1"])
+def test_similarity_grads_conv_scale_full_batch_against_the_oracle(pkg, func, record_property):
+    """Full config-3 batch (256 images).  Input gradient: per-image oracle on a sample of images.  Parameter gradients:
+    a template's gradient depends on that template's parameters and output-gradient channel only, so the oracle over
+    all 256 images for a subset of the 128 templates pins those rows of the full call - for the default forms
+    (moments on the matrix cores / scaled sign) and for algo='direct' (the reference's terms one by one), which must
+    meet the plain 1e-4 bar.  Properties over everything: linearity in the output gradient (exact for a factor 2)."""
     x, t, w, kw = config3()
+    kw = dict(kw, similarity_function=func)
     g = np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32)
     X, T, W, G = dev(x), dev(t), dev(w), dev(g)
     dx = pkg.similarity_input_grad(X, T, W, G, **kw)
-    dt, dw = pkg.similarity_parameters_grad(X, T, W, G, **kw)
-    for b in (0, 255):
+    for b in (0, 131, 255):
         want = orc.similarity_input_grad(x[b:b + 1], t, w, g[b:b + 1], **kw)
         true = orc.similarity_input_grad(*f64(x[b:b + 1], t, w, g[b:b + 1]), **kw)
         assert_grad_close(dx[b:b + 1].cpu().numpy(), want, true, "input grad of image %d" % b)
-    dt1, dw1 = pkg.similarity_parameters_grad(X[:128], T, W, G[:128], **kw)
-    dt2, dw2 = pkg.similarity_parameters_grad(X[128:], T, W, G[128:], **kw)
-    # two fp32 summation orders of 262144-term sums against each other: a few 1e-4 of rounding noise
-    assert grad_err((dt1 + dt2).cpu().numpy(), dt.cpu().numpy()) <= 5 * GRAD_TOL
-    assert grad_err((dw1 + dw2).cpu().numpy(), dw.cpu().numpy()) <= 5 * GRAD_TOL
-    dt3, dw3 = pkg.similarity_parameters_grad(X, T, W, 2.0 * G, **kw)
-    assert torch.equal(dt3, 2.0 * dt) and torch.equal(dw3, 2.0 * dw)      # scaling by 2 is exact in fp32
-    want_dt, want_dw = orc.similarity_params_grad(x[:2], t, w, g[:2], **kw)
-    true_dt, true_dw = orc.similarity_params_grad(*f64(x[:2], t, w, g[:2]), **kw)
-    dt4, dw4 = pkg.similarity_parameters_grad(X[:2], T, W, G[:2], **kw)
-    assert_grad_close(dt4.cpu().numpy(), want_dt, true_dt, "templates grad")
-    assert_grad_close(dw4.cpu().numpy(), want_dw, true_dw, "weights grad")
+    idx = [0, 1, 37, 63, 64, 100, 126, 127]
+    gs = np.ascontiguousarray(g[:, idx])
+    ref_dt, ref_dw = oracle_params_grad_over_batch(x, t[idx], w[idx], gs, kw, np.float32)
+    true_dt, true_dw = oracle_params_grad_over_batch(x, t[idx], w[idx], gs, kw, np.float64)
+    e_ref = (grad_err(ref_dt, true_dt), grad_err(ref_dw, true_dw))
+    for algo in (None, "direct"):
+        dt, dw = pkg.similarity_parameters_grad(X, T, W, G, algo=algo, **kw)
+        e = (grad_err(dt.cpu().numpy()[idx], true_dt), grad_err(dw.cpu().numpy()[idx], true_dw))
+        print("config-3 %s parameter gradients, 256 images, algo=%s: templates %.3g, weights %.3g of the scale "
+              "(fp32 oracle: %.3g, %.3g)" % (func, algo, e[0], e[1], e_ref[0], e_ref[1]))
+        record_property("params_grad_err_%s_%s" % (func, algo), e)
+        if algo == "direct":
+            assert max(e) <= GRAD_TOL, e
+        else:
+            assert e[0] <= max(GRAD_TOL, 2 * e_ref[0]) and e[1] <= max(GRAD_TOL, 2 * e_ref[1]), (e, e_ref)
+        dt3, dw3 = pkg.similarity_parameters_grad(X, T, W, 2.0 * G, algo=algo, **kw)
+        assert torch.equal(dt3, 2.0 * dt) and torch.equal(dw3, 2.0 * dw)      # scaling by 2 is exact in fp32
 
 
 def test_similarity_params_grad_is_reproducible(pkg):
@@ -355,7 +379,7 @@ def test_mex_input_grad_of_overlapping_patches_is_reproducible(pkg, eps):
 
 
 def test_mex_grads_config2_shape(pkg):
-    x, off, n, kw = config2(batch=8)
+    x, off, n, kw = config2(batch=64)
     off = orc.normalize_offsets(off)
     check_mex_grads(pkg, x, off, n, **kw)
 
