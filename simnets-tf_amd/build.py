@@ -25,6 +25,20 @@ DEVICE = ["--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang", "-pa
           "-fno-gpu-rdc"]
 
 
+# hipcc hands the -target-feature switch to its host pass as well, which does not know an AMDGPU feature and says so
+# once per file; the switch only matters to (and is honoured by) the device pass, so that one line is dropped.
+_HOST_PASS_NOTE = "'-packed-fp32-ops' is not a recognized feature for this target"
+
+
+def _run(cmd):
+    r = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    noise = [ln for ln in r.stderr.splitlines() if _HOST_PASS_NOTE not in ln]
+    if noise:
+        print("\n".join(noise), file=sys.stderr)
+    if r.returncode != 0:
+        raise subprocess.CalledProcessError(r.returncode, cmd)
+
+
 def _compile(src, extra):
     obj = os.path.join(OBJDIR, os.path.splitext(src)[0] + ".o")
     path = os.path.join(CSRC, src)
@@ -32,7 +46,7 @@ def _compile(src, extra):
         cmd = [HIPCC, "-c", path, "-o", obj] + COMMON + DEVICE + extra
     else:
         cmd = [HIPCC, "-x", "c++", "-c", path, "-o", obj] + COMMON + extra
-    subprocess.run(cmd, check=True)
+    _run(cmd)
     return obj
 
 
@@ -44,8 +58,8 @@ def build(extra=(), verbose=False):
     subprocess.run([HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB] + objs, check=True)
     # standalone C++ harness, linked against the product library only
     bench_src = os.path.join(HERE, "bench", "simnets_bench.hip")
-    subprocess.run([HIPCC, bench_src, "-o", BENCH] + COMMON + DEVICE + extra +
-                   ["-L" + HERE, "-lsimnets_hip", "-Wl,-rpath,$ORIGIN"], check=True)
+    _run([HIPCC, bench_src, "-o", BENCH] + COMMON + DEVICE + extra +
+         ["-L" + HERE, "-lsimnets_hip", "-Wl,-rpath,$ORIGIN"])
     if verbose:
         print("built", LIB, "and", BENCH)
     return LIB

@@ -292,36 +292,34 @@ def mex_output_shape(input_shape, num_instances, **attrs):
 
 def _mex_dims_helper(input_dim, num_instances, blocks, padding=[0], strides=[1], blocks_round_down=True,
                      use_unshared_regions=True, shared_offset_region=[-1], unshared_offset_region=[-1]):
-    """Number of offset regions; same signature and C call as python/simnets/ops/mex.py:17-38."""
-    args = []
+    """Number of offset regions of a MEX layer over an image of `input_dim` = (C, H, W).
 
-    def add_array(l):
-        args.extend([C.c_int(len(l)), (C.c_int * len(l))(*[int(v) for v in l])])
+    Same name, argument meaning and C call (`get_mex_offsets_nregions`, every list passed as a length followed by
+    an int array) as the reference's helper, python/simnets/ops/mex.py:17-38.
+    """
+    def counted(values):
+        ints = [int(v) for v in values]
+        return C.c_int(len(ints)), (C.c_int * len(ints))(*ints)
 
-    add_array(input_dim)
-    add_array(padding)
-    add_array(strides)
-    args.extend([C.c_int(num_instances), C.c_int(blocks_round_down), C.c_int(use_unshared_regions)])
-    add_array(blocks)
-    add_array(shared_offset_region)
-    add_array(unshared_offset_region)
-    return _lib.lib().get_mex_offsets_nregions(*args)
+    flags = (C.c_int(int(num_instances)), C.c_int(int(bool(blocks_round_down))),
+             C.c_int(int(bool(use_unshared_regions))))
+    call = counted(input_dim) + counted(padding) + counted(strides) + flags + counted(blocks) + \
+        counted(shared_offset_region) + counted(unshared_offset_region)
+    return _lib.lib().get_mex_offsets_nregions(*call)
 
 
 def _expand_dim_specification(image_shape, dim_spec):
-    """python/simnets/ops/mex.py:84-111: prepend -1 to a 2-list, replace -1 by the image dimension."""
-    if len(dim_spec) != 2 and len(dim_spec) != 3:
+    """A (channels, rows, columns) triple from a 2- or 3-entry specification: a 2-entry one covers all channels,
+    and an entry of -1 stands for the whole extent of the image (NCHW, or CHW without the batch) along that axis.
+    Behaviour of python/simnets/ops/mex.py:84-111.
+    """
+    spec = list(dim_spec)
+    if len(spec) not in (2, 3):
         raise ValueError('Bad dimensions specifications, should be a list of two or three, got %s' % dim_spec)
-    image_shape = list(image_shape)
-    if len(image_shape) == 3:
-        image_shape = [None] + image_shape
-    dim_spec = list(dim_spec)
-    if len(dim_spec) == 2:
-        dim_spec = [-1] + dim_spec
-    for i in range(3):
-        if dim_spec[i] == -1:
-            dim_spec[i] = image_shape[i + 1]
-    return dim_spec
+    chw = list(image_shape)[-3:]
+    if len(spec) == 2:
+        spec.insert(0, -1)
+    return [extent if want == -1 else want for want, extent in zip(spec, chw)]
 
 
 def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
