@@ -68,10 +68,13 @@ enum { SIMNETS_SIM_L1 = 0, SIMNETS_SIM_L2 = 1 };
 enum {
     SIMNETS_ALGO_AUTO = 0,   /* SQRTW for plain L2 (no normalization term), DIRECT for every other mode */
     SIMNETS_ALGO_DIRECT = 1, /* d = t - x; acc += (-w*d)*d   (L1: acc += -w*|d|), NaN-capable, every mode */
-    SIMNETS_ALGO_SQRTW = 2,  /* plain L2 only: d = sqrt(w)*t - sqrt(w)*x in one fma; acc += -d*d.  Outputs closer to
-                                zero than sum_k w t^2 / 1024 (where the different rounding of d could exceed 4e-6
-                                relative), and all outputs of a template with a negative or NaN weight, are then
-                                recomputed with DIRECT's arithmetic, so the result stays within the tolerance */
+    SIMNETS_ALGO_SQRTW = 2,  /* plain L2 only: d = sqrt(w)*t - sqrt(w)*x in one fma; acc += -d*d.  The rounding of d
+                                could exceed 4e-6 relative only for outputs closer to zero than sum_k w t^2 / 1024.
+                                The terms all have one sign, so a wave (64 pixel groups x 8 templates) whose partial
+                                sums after the first channel chunk all lie beyond that bound is safe; a wave with one
+                                that does not (or with a template of negative or NaN weight) stops there and a second,
+                                flag-gated pass recomputes all its outputs with DIRECT's arithmetic, bit-identical
+                                to SIMNETS_ALGO_DIRECT */
     SIMNETS_ALGO_MFMA = 3    /* plain L2 only, inputs free of NaN/Inf: sum w x^2 - 2 sum (w t) x + sum w t^2
                                 as dense fp32 matrix-core contractions */
 };
@@ -116,6 +119,22 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
                                const int templates_shape[4], const int weights_shape[4], const float *input,
                                const float *templates, const float *weights, float *output, void *workspace,
                                size_t workspace_bytes, void *stream);
+
+/* The same forward with the parameter-only work taken out of the steady-state call, for callers whose templates and
+ * weights stay fixed across calls (inference): where SimilarityKernelGPU::Compute interlaces the parameters on
+ * every call (src/kernels/similarity_kernel_gpu.cu:70), simnets_hip_similarity_prepare does the packing once
+ * (packed parameters, tables, and for the sqrt-weight form the second packed copy and the thresholds) into a
+ * caller-owned buffer of simnets_hip_similarity_workspace_bytes bytes (256-byte aligned), and
+ * simnets_hip_similarity_fwd_prepared runs only the forward kernels on it.  attrs, input_shape (batch size
+ * included: the tiling depends on it) and templates_shape must be the ones the buffer was prepared with; results
+ * are those of simnets_hip_similarity_fwd bit for bit.  The buffer also holds a few bytes of per-call scratch (the
+ * wave flags of the sqrt-weight form), so calls that share one prepared buffer must not overlap. */
+int simnets_hip_similarity_prepare(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                   const int templates_shape[4], const int weights_shape[4], const float *templates,
+                                   const float *weights, void *prepared, size_t prepared_bytes, void *stream);
+int simnets_hip_similarity_fwd_prepared(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                        const int templates_shape[4], const float *input, void *prepared,
+                                        size_t prepared_bytes, float *output, void *stream);
 
 /* simnets_hip_similarity_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight
  * serving loops, harnesses that forbid hipMalloc) and so have no workspace to pass.  It has no counterpart in the
@@ -225,6 +244,18 @@ int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4]
                         const float *offsets, size_t offsets_count, float *output, void *workspace,
                         size_t workspace_bytes, void *stream);
 
+/* The same forward with the offsets-only work taken out of the steady-state call (fixed offsets, inference): where
+ * MEXKernelGPU::Compute copies the offsets on every call (src/kernels/mex_kernel_gpu.cu:98-112),
+ * simnets_hip_mex_prepare packs them once (normalised if attrs say so, scaled, k-major per instance group, with their
+ * exponentials, row maxima and ranges, and the patch element table) into a caller-owned buffer of
+ * simnets_hip_mex_workspace_bytes bytes (256-byte aligned) and simnets_hip_mex_fwd_prepared runs only the forward
+ * kernel on it.  attrs and input_shape (batch size included) must be the ones the buffer was prepared with; results
+ * are those of simnets_hip_mex_fwd bit for bit. */
+int simnets_hip_mex_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
+                            size_t offsets_count, void *prepared, size_t prepared_bytes, void *stream);
+int simnets_hip_mex_fwd_prepared(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 void *prepared, size_t prepared_bytes, float *output, void *stream);
+
 /* Backward.  Scratch sizes of the two gradient calls (either pointer may be NULL). */
 int simnets_hip_mex_grad_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4],
                                          size_t *input_grad_bytes, size_t *offsets_grad_bytes);
@@ -287,6 +318,16 @@ int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input
                                  const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
                                  void *workspace, size_t workspace_bytes, void *stream);
 
+/* ... in two halves, like simnets_hip_mex_prepare / simnets_hip_mex_fwd_prepared: the buffer has
+ * simnets_hip_mex_sum_pool_workspace_bytes bytes; when the geometry runs the two kernels through scratch memory the
+ * buffer holds that scratch as well, so calls that share one prepared buffer must not overlap. */
+int simnets_hip_mex_sum_pool_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
+                                     size_t offsets_count, int pool_h, int pool_w, void *prepared,
+                                     size_t prepared_bytes, void *stream);
+int simnets_hip_mex_sum_pool_fwd_prepared(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                          int pool_h, int pool_w, void *prepared, size_t prepared_bytes, float *output,
+                                          void *stream);
+
 /* Similarity, MEX over its output, sum pooling, as one call: the first layers of the reference's networks
  * (README.md:108-129: Similarity on the image, MEX over all of its channels per pixel, pooling).  output =
  * simnets_hip_sum_pool_fwd(simnets_hip_mex_fwd(simnets_hip_similarity_fwd(...))); mex_attrs describe the MEX layer
@@ -304,6 +345,20 @@ int simnets_hip_similarity_mex_sum_pool_fwd(const simnets_similarity_attrs *sim_
                                             const float *weights, const simnets_mex_attrs *mex_attrs,
                                             const float *offsets, size_t offsets_count, int pool_h, int pool_w,
                                             float *output, void *workspace, size_t workspace_bytes, void *stream);
+
+/* ... in two halves: templates, weights and offsets are packed once into a buffer of
+ * simnets_hip_similarity_mex_sum_pool_workspace_bytes bytes; the steady-state call takes the input only.  Same
+ * conditions as the other prepared calls (same attrs and shapes; no overlapping calls on one buffer). */
+int simnets_hip_similarity_mex_sum_pool_prepare(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                                                const int templates_shape[4], const float *templates,
+                                                const float *weights, const simnets_mex_attrs *mex_attrs,
+                                                const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                                void *prepared, size_t prepared_bytes, void *stream);
+int simnets_hip_similarity_mex_sum_pool_fwd_prepared(const simnets_similarity_attrs *sim_attrs,
+                                                     const int input_shape[4], const int templates_shape[4],
+                                                     const float *input, const simnets_mex_attrs *mex_attrs, int pool_h,
+                                                     int pool_w, void *prepared, size_t prepared_bytes, float *output,
+                                                     void *stream);
 
 #ifdef __cplusplus
 }

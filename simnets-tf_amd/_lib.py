@@ -18,6 +18,10 @@ EXPORTS = [
     "simnets_hip_mex_offsets_grad", "simnets_hip_mex_grads_workspace_bytes", "simnets_hip_mex_grads",
     "simnets_hip_mex_sum_pool_workspace_bytes", "simnets_hip_mex_sum_pool_fwd",
     "simnets_hip_similarity_mex_sum_pool_workspace_bytes", "simnets_hip_similarity_mex_sum_pool_fwd",
+    "simnets_hip_similarity_prepare", "simnets_hip_similarity_fwd_prepared",
+    "simnets_hip_mex_prepare", "simnets_hip_mex_fwd_prepared",
+    "simnets_hip_mex_sum_pool_prepare", "simnets_hip_mex_sum_pool_fwd_prepared",
+    "simnets_hip_similarity_mex_sum_pool_prepare", "simnets_hip_similarity_mex_sum_pool_fwd_prepared",
 ]
 
 SIM_L1, SIM_L2 = 0, 1
@@ -124,6 +128,22 @@ def lib():
                                                    P]
         l.simnets_hip_mex_grads_workspace_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
         l.simnets_hip_mex_grads.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, P, P, C.c_size_t, P]
+        SA, MA = C.POINTER(SimilarityAttrs), C.POINTER(MexAttrs)
+        l.simnets_hip_similarity_prepare.argtypes = [SA, I4, I4, I4, P, P, P, C.c_size_t, P]
+        l.simnets_hip_similarity_fwd_prepared.argtypes = [SA, I4, I4, P, P, C.c_size_t, P, P]
+        l.simnets_hip_mex_prepare.argtypes = [MA, I4, P, C.c_size_t, P, C.c_size_t, P]
+        l.simnets_hip_mex_fwd_prepared.argtypes = [MA, I4, P, P, C.c_size_t, P, P]
+        l.simnets_hip_mex_sum_pool_prepare.argtypes = [MA, I4, P, C.c_size_t, C.c_int, C.c_int, P, C.c_size_t, P]
+        l.simnets_hip_mex_sum_pool_fwd_prepared.argtypes = [MA, I4, P, C.c_int, C.c_int, P, C.c_size_t, P, P]
+        l.simnets_hip_similarity_mex_sum_pool_prepare.argtypes = [SA, I4, I4, P, P, MA, P, C.c_size_t, C.c_int, C.c_int,
+                                                                  P, C.c_size_t, P]
+        l.simnets_hip_similarity_mex_sum_pool_fwd_prepared.argtypes = [SA, I4, I4, P, MA, C.c_int, C.c_int, P,
+                                                                       C.c_size_t, P, P]
+        for name in ("simnets_hip_similarity_prepare", "simnets_hip_similarity_fwd_prepared",
+                     "simnets_hip_mex_prepare", "simnets_hip_mex_fwd_prepared", "simnets_hip_mex_sum_pool_prepare",
+                     "simnets_hip_mex_sum_pool_fwd_prepared", "simnets_hip_similarity_mex_sum_pool_prepare",
+                     "simnets_hip_similarity_mex_sum_pool_fwd_prepared"):
+            getattr(l, name).restype = C.c_int
         for name in ("simnets_similarity_out_shape", "simnets_hip_similarity_workspace_bytes",
                      "simnets_hip_similarity_fwd", "simnets_mex_calc_dims", "simnets_mex_out_shape",
                      "simnets_hip_mex_workspace_bytes", "simnets_hip_mex_fwd", "simnets_hip_sum_pool_fwd",

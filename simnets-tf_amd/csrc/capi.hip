@@ -13,6 +13,15 @@ size_t sim_mfma_workspace_bytes(const SimPlan &p);
 int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
                     void *workspace, size_t workspace_bytes, hipStream_t s);
 
+int sim_direct_prepare(const SimPlan &p, const float *templates, const float *weights, void *workspace,
+                       size_t workspace_bytes, hipStream_t s);
+int sim_direct_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
+                   hipStream_t s);
+int sim_mfma_prepare(const SimPlan &p, const float *templates, const float *weights, void *workspace,
+                     size_t workspace_bytes, hipStream_t s);
+int sim_mfma_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
+                 hipStream_t s);
+
 size_t sim_workspace_bytes(const SimPlan &p)
 {
     if (p.algo == SIMNETS_ALGO_MFMA)
@@ -27,6 +36,23 @@ int sim_launch(const SimPlan &p, const float *input, const float *templates, con
     if (p.algo == SIMNETS_ALGO_MFMA)
         return sim_mfma_launch(p, input, templates, weights, output, workspace, workspace_bytes, s);
     return sim_direct_launch(p, input, templates, weights, output, workspace, workspace_bytes, s);
+}
+
+int sim_prepare(const SimPlan &p, const float *templates, const float *weights, void *prepared, size_t prepared_bytes,
+                void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (p.algo == SIMNETS_ALGO_MFMA)
+        return sim_mfma_prepare(p, templates, weights, prepared, prepared_bytes, s);
+    return sim_direct_prepare(p, templates, weights, prepared, prepared_bytes, s);
+}
+
+int sim_run(const SimPlan &p, const float *input, float *output, void *prepared, size_t prepared_bytes, void *stream)
+{
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (p.algo == SIMNETS_ALGO_MFMA)
+        return sim_mfma_run(p, input, output, prepared, prepared_bytes, s);
+    return sim_direct_run(p, input, output, prepared, prepared_bytes, s);
 }
 
 }  // namespace simnets
@@ -85,8 +111,8 @@ int simnets_hip_similarity_fwd_static(const simnets_similarity_attrs *attrs, con
     const int rs = static_scratch(&ws);
     if (rs)
         return rs;
-    // the pack and guard-prep kernels rewrite every part of the scratch the main kernel reads (parameters,
-    // tables, thresholds, cleared flags), so nothing of an earlier call survives into this one
+    // the pack kernel rewrites every part of the scratch the main kernel reads (parameters, tables, thresholds)
+    // and the main kernel writes every flag the recomputing pass reads, so nothing of an earlier call survives
     return sim_launch(p, input, templates, weights, output, ws, SIMNETS_HIP_STATIC_SCRATCH_BYTES, stream);
 }
 
@@ -106,6 +132,38 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
     if (!workspace_ok(workspace, workspace_bytes, sim_workspace_bytes(p)))
         return SIMNETS_ERR_WORKSPACE;
     return sim_launch(p, input, templates, weights, output, workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_similarity_prepare(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                   const int templates_shape[4], const int weights_shape[4], const float *templates,
+                                   const float *weights, void *prepared, size_t prepared_bytes, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, weights_shape, &p);
+    if (rc)
+        return rc;
+    if (!templates || !weights)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(prepared, prepared_bytes, sim_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_prepare(p, templates, weights, prepared, prepared_bytes, stream);
+}
+
+int simnets_hip_similarity_fwd_prepared(const simnets_similarity_attrs *attrs, const int input_shape[4],
+                                        const int templates_shape[4], const float *input, void *prepared,
+                                        size_t prepared_bytes, float *output, void *stream)
+{
+    SimPlan p;
+    const int rc = sim_make_plan(attrs, input_shape, templates_shape, templates_shape, &p);
+    if (rc)
+        return rc;
+    if (p.B == 0)
+        return SIMNETS_OK;
+    if (!input || !output)
+        return SIMNETS_ERR_NULL_POINTER;
+    if (!workspace_ok(prepared, prepared_bytes, sim_workspace_bytes(p)))
+        return SIMNETS_ERR_WORKSPACE;
+    return sim_run(p, input, output, prepared, prepared_bytes, stream);
 }
 
 int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
@@ -218,23 +276,44 @@ int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[
                      stream);
 }
 
-int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
-                        const float *offsets, size_t offsets_count, float *output, void *workspace,
-                        size_t workspace_bytes, void *stream)
+static int mex_fwd_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                         const float *offsets, size_t offsets_count, float *output, void *workspace,
+                         size_t workspace_bytes, void *stream, int phase)
 {
     MexPlan p;
     const int rc = mex_make_plan(attrs, input_shape, &p);
     if (rc)
         return rc;
-    if (offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
+    if ((phase & kMexPrepare) && offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
         return SIMNETS_ERR_SHAPE;
-    if (p.B == 0)
+    if (p.B == 0 && phase != kMexPrepare)
         return SIMNETS_OK;
-    if (!input || !offsets || !output)
+    if (((phase & kMexRun) && (!input || !output)) || ((phase & kMexPrepare) && !offsets))
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_workspace_bytes(p)))
         return SIMNETS_ERR_WORKSPACE;
-    return mex_launch(p, input, offsets, output, workspace, workspace_bytes, stream);
+    return mex_launch(p, input, offsets, output, workspace, workspace_bytes, stream, phase);
+}
+
+int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                        const float *offsets, size_t offsets_count, float *output, void *workspace,
+                        size_t workspace_bytes, void *stream)
+{
+    return mex_fwd_phase(attrs, input_shape, input, offsets, offsets_count, output, workspace, workspace_bytes, stream,
+                         kMexWhole);
+}
+
+int simnets_hip_mex_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
+                            size_t offsets_count, void *prepared, size_t prepared_bytes, void *stream)
+{
+    return mex_fwd_phase(attrs, input_shape, nullptr, offsets, offsets_count, nullptr, prepared, prepared_bytes, stream,
+                         kMexPrepare);
+}
+
+int simnets_hip_mex_fwd_prepared(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 void *prepared, size_t prepared_bytes, float *output, void *stream)
+{
+    return mex_fwd_phase(attrs, input_shape, input, nullptr, 0, output, prepared, prepared_bytes, stream, kMexRun);
 }
 
 int simnets_hip_sum_pool_fwd(const int input_shape[4], int pool_h, int pool_w, const float *input, float *output,
@@ -290,25 +369,50 @@ int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, con
     return SIMNETS_OK;
 }
 
-int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
-                                 const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
-                                 void *workspace, size_t workspace_bytes, void *stream)
+static int mex_sum_pool_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                              const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
+                              void *workspace, size_t workspace_bytes, void *stream, int phase)
 {
     MexPlan p;
     const int rc = mex_make_plan(attrs, input_shape, &p);
     if (rc)
         return rc;
-    if (pool_h <= 0 || pool_w <= 0 || offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
+    if (pool_h <= 0 || pool_w <= 0 ||
+        ((phase & kMexPrepare) && offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K))
         return SIMNETS_ERR_SHAPE;
     if (p.d.height_out / pool_h <= 0 || p.d.width_out / pool_w <= 0)
         return SIMNETS_ERR_EMPTY_OUTPUT;
-    if (p.B == 0)
+    if (p.B == 0 && phase != kMexPrepare)
         return SIMNETS_OK;
-    if (!input || !offsets || !output)
+    if (((phase & kMexRun) && (!input || !output)) || ((phase & kMexPrepare) && !offsets))
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_pool_workspace_bytes(p, pool_h, pool_w)))
         return SIMNETS_ERR_WORKSPACE;
-    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream);
+    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream, phase);
+}
+
+int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                 const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
+                                 void *workspace, size_t workspace_bytes, void *stream)
+{
+    return mex_sum_pool_phase(attrs, input_shape, input, offsets, offsets_count, pool_h, pool_w, output, workspace,
+                              workspace_bytes, stream, kMexWhole);
+}
+
+int simnets_hip_mex_sum_pool_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
+                                     size_t offsets_count, int pool_h, int pool_w, void *prepared,
+                                     size_t prepared_bytes, void *stream)
+{
+    return mex_sum_pool_phase(attrs, input_shape, nullptr, offsets, offsets_count, pool_h, pool_w, nullptr, prepared,
+                              prepared_bytes, stream, kMexPrepare);
+}
+
+int simnets_hip_mex_sum_pool_fwd_prepared(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                          int pool_h, int pool_w, void *prepared, size_t prepared_bytes, float *output,
+                                          void *stream)
+{
+    return mex_sum_pool_phase(attrs, input_shape, input, nullptr, 0, pool_h, pool_w, output, prepared, prepared_bytes,
+                              stream, kMexRun);
 }
 
 static int sim_mex_pool_plans(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
@@ -345,27 +449,57 @@ int simnets_hip_similarity_mex_sum_pool_workspace_bytes(const simnets_similarity
     return SIMNETS_OK;
 }
 
-int simnets_hip_similarity_mex_sum_pool_fwd(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
-                                            const int templates_shape[4], const float *input, const float *templates,
-                                            const float *weights, const simnets_mex_attrs *mex_attrs,
-                                            const float *offsets, size_t offsets_count, int pool_h, int pool_w,
-                                            float *output, void *workspace, size_t workspace_bytes, void *stream)
+static int sim_mex_pool_phase(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                              const int templates_shape[4], const float *input, const float *templates,
+                              const float *weights, const simnets_mex_attrs *mex_attrs, const float *offsets,
+                              size_t offsets_count, int pool_h, int pool_w, float *output, void *workspace,
+                              size_t workspace_bytes, void *stream, int phase)
 {
     SimPlan sp;
     MexPlan mp;
     const int rc = sim_mex_pool_plans(sim_attrs, input_shape, templates_shape, mex_attrs, pool_h, pool_w, &sp, &mp);
     if (rc)
         return rc;
-    if (offsets_count < (size_t)mp.d.num_regions * mp.d.M * mp.d.K)
+    if ((phase & kMexPrepare) && offsets_count < (size_t)mp.d.num_regions * mp.d.M * mp.d.K)
         return SIMNETS_ERR_SHAPE;
-    if (sp.B == 0)
+    if (sp.B == 0 && phase != kMexPrepare)
         return SIMNETS_OK;
-    if (!input || !templates || !weights || !offsets || !output)
+    if (((phase & kMexRun) && (!input || !output)) || ((phase & kMexPrepare) && (!templates || !weights || !offsets)))
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, sim_mex_pool_workspace_bytes(sp, mp, pool_h, pool_w)))
         return SIMNETS_ERR_WORKSPACE;
     return sim_mex_pool_launch(sp, mp, pool_h, pool_w, input, templates, weights, offsets, output, workspace,
-                               workspace_bytes, stream);
+                               workspace_bytes, stream, phase);
+}
+
+int simnets_hip_similarity_mex_sum_pool_fwd(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                                            const int templates_shape[4], const float *input, const float *templates,
+                                            const float *weights, const simnets_mex_attrs *mex_attrs,
+                                            const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                            float *output, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return sim_mex_pool_phase(sim_attrs, input_shape, templates_shape, input, templates, weights, mex_attrs, offsets,
+                              offsets_count, pool_h, pool_w, output, workspace, workspace_bytes, stream, kMexWhole);
+}
+
+int simnets_hip_similarity_mex_sum_pool_prepare(const simnets_similarity_attrs *sim_attrs, const int input_shape[4],
+                                                const int templates_shape[4], const float *templates,
+                                                const float *weights, const simnets_mex_attrs *mex_attrs,
+                                                const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                                void *prepared, size_t prepared_bytes, void *stream)
+{
+    return sim_mex_pool_phase(sim_attrs, input_shape, templates_shape, nullptr, templates, weights, mex_attrs, offsets,
+                              offsets_count, pool_h, pool_w, nullptr, prepared, prepared_bytes, stream, kMexPrepare);
+}
+
+int simnets_hip_similarity_mex_sum_pool_fwd_prepared(const simnets_similarity_attrs *sim_attrs,
+                                                     const int input_shape[4], const int templates_shape[4],
+                                                     const float *input, const simnets_mex_attrs *mex_attrs, int pool_h,
+                                                     int pool_w, void *prepared, size_t prepared_bytes, float *output,
+                                                     void *stream)
+{
+    return sim_mex_pool_phase(sim_attrs, input_shape, templates_shape, input, nullptr, nullptr, mex_attrs, nullptr, 0,
+                              pool_h, pool_w, output, prepared, prepared_bytes, stream, kMexRun);
 }
 
 }  // extern "C"

@@ -33,6 +33,11 @@ size_t sim_direct_workspace_bytes(const SimPlan &p);
 int sim_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
                void *workspace, size_t workspace_bytes, void *stream);
 
+// The forward call in two halves: everything that depends on the parameters only, and the launches that read it.
+int sim_prepare(const SimPlan &p, const float *templates, const float *weights, void *prepared, size_t prepared_bytes,
+                void *stream);
+int sim_run(const SimPlan &p, const float *input, float *output, void *prepared, size_t prepared_bytes, void *stream);
+
 struct MexPlan {
     int B, C, H, W;
     simnets_mex_dims d;
@@ -44,8 +49,11 @@ struct MexPlan {
 
 int mex_make_plan(const simnets_mex_attrs *attrs, const int input_shape[4], MexPlan *plan);
 size_t mex_workspace_bytes(const MexPlan &p);
+// The forward calls in two halves (`phase`): the launch that depends on the parameters alone, and the launches that
+// read what it wrote; the default is the whole call.
+enum { kMexPrepare = 1, kMexRun = 2, kMexWhole = 3 };
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
-               size_t workspace_bytes, void *stream);
+               size_t workspace_bytes, void *stream, int phase = kMexWhole);
 
 // Backward operators (similarity_grad.hip, mex_grad.hip).  `stream` is a hipStream_t.
 // Input gradient of the L2 modes at stride 1 on the matrix cores (similarity_mfma.hip)
@@ -81,14 +89,14 @@ int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float
 // offsets region, else MEX into scratch + pooling
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw);
 int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
-                    void *workspace, size_t workspace_bytes, void *stream);
+                    void *workspace, size_t workspace_bytes, void *stream, int phase = kMexWhole);
 // Similarity, then MEX over its output, then sum pooling; `mp` is the MEX plan for the Similarity output's shape.
 // One kernel when the MEX patch of a pixel is exactly the Similarity channels of that pixel (and the MEX + pooling
 // pair is fusable), else the separate kernels through scratch memory.
 size_t sim_mex_pool_workspace_bytes(const SimPlan &sp, const MexPlan &mp, int ph, int pw);
 int sim_mex_pool_launch(const SimPlan &sp, const MexPlan &mp, int ph, int pw, const float *input,
                         const float *templates, const float *weights, const float *offsets, float *pooled,
-                        void *workspace, size_t workspace_bytes, void *stream);
+                        void *workspace, size_t workspace_bytes, void *stream, int phase = kMexWhole);
 
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 

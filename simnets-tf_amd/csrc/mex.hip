@@ -626,14 +626,16 @@ hipError_t launch_px1(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, 
 
 // Few pixels, long K (the classifier head of a network: a handful of instances over hundreds of channels at 1x1
 // spatial size): the tiling above would launch a few workgroups with long serial instruction streams.  Here one
-// wave owns one output pixel and the lanes split K: KL patch elements per lane stay in registers, and for every
-// instance the wave adds the offsets, reduces max and sum of exponentials with shuffles and lane 0 stores.  The
-// logsumexp normalisation of the offsets (python/simnets/keras.py:155-160) is folded in, so no pack launch is needed.
+// wave owns one output pixel and the lanes split K: KL patch elements per lane stay in registers.  Finite epsilon:
+// the product form of the tiled kernel, per wave - the pixel's maximum mp (one shuffle reduction), exp2(x_k - mp)
+// once per element, then per instance a dot product with the packed exp2(o_k - mo) row and one shuffle reduction.
+// Instances whose offsets range is too wide for that, and infinite epsilon, take patch + offset term by term
+// (maximum, then the sum of exponentials relative to it).  The offsets come packed with one instance per group:
+// rows [r][m][k].
 constexpr int kSmallMChunk = 16;  // instances per wave
 
 template <int KL, bool NEG>
-__global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, const float *__restrict__ offsets,
-                                                        int normalize)
+__global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
 {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -679,88 +681,102 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, c
     };
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
-    const int m_end = min(a.M, (int)(blockIdx.y + 1) * kSmallMChunk);
+    const int m_first = blockIdx.y * kSmallMChunk;
+    const int m_end = min(a.M, m_first + kSmallMChunk);
+    const size_t row0 = (size_t)r * a.M;
+    // which form each instance of this wave takes (wave-uniform): bit g of `wide` set -> term by term
+    unsigned wide = a.finite_eps ? 0u : 0xffffu;
+    if (a.finite_eps) {
+        for (int m = m_first; m < m_end; ++m)
+            if (!(a.orng[row0 + m] <= kProductRange))
+                wide |= 1u << (m - m_first);
+    }
     // the offsets rows of the next four instances are requested while the current four are reduced
     float on[MG][KL];
     auto fetch_rows = [&](int m0) __attribute__((always_inline)) {
 #pragma unroll
         for (int g = 0; g < MG; ++g) {
-            const float *row = offsets + ((size_t)r * a.M + min(m0 + g, a.M - 1)) * a.K;
+            const int m = min(m0 + g, a.M - 1);
+            const float *row = (((wide >> (m - m_first)) & 1u) ? a.offp : a.offe) + (row0 + m) * a.K;
 #pragma unroll
             for (int j = 0; j < KL; ++j)
                 on[g][j] = row[kv[j] ? lane + 64 * j : 0];
         }
     };
-    fetch_rows(blockIdx.y * kSmallMChunk);
-    for (int m0 = blockIdx.y * kSmallMChunk; m0 < m_end; m0 += MG) {
+    fetch_rows(m_first);
+    // scaled patch values, their maximum and exponentials (finite epsilon)
+    float ex[KL];
+    float mp = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < KL; ++j) {
+        x[j] *= a.scale;
+        if (kv[j])
+            mp = fmaxf(mp, x[j]);
+    }
+    if (a.finite_eps) {
+        for (int d = 32; d > 0; d >>= 1)
+            mp = fmaxf(mp, __shfl_xor(mp, d, 64));
+        const float m_sub = mp == -INFINITY ? 0.0f : mp;
+#pragma unroll
+        for (int j = 0; j < KL; ++j)
+            ex[j] = kv[j] ? __builtin_amdgcn_exp2f(x[j] - m_sub) : 0.0f;
+    }
+    const float mpt = (mp - mp) + mp;  // an infinite pixel bound makes the result NaN, as the reference's exp(inf - inf) does
+    for (int m0 = m_first; m0 < m_end; m0 += MG) {
         float o[MG][KL];
 #pragma unroll
         for (int g = 0; g < MG; ++g)
 #pragma unroll
             for (int j = 0; j < KL; ++j)
-                o[g][j] = kv[j] ? on[g][j] : 0.0f;
+                o[g][j] = on[g][j];
         if (m0 + MG < m_end)
             fetch_rows(m0 + MG);
-        if (normalize) {
-            float mx[MG], sum[MG];
-#pragma unroll
-            for (int g = 0; g < MG; ++g) {
-                mx[g] = -INFINITY;
-#pragma unroll
-                for (int j = 0; j < KL; ++j)
-                    if (kv[j])
-                        mx[g] = fmaxf(mx[g], o[g][j]);
-            }
-            wave_best(mx, false);
-#pragma unroll
-            for (int g = 0; g < MG; ++g) {
-                if (!(fabsf(mx[g]) < INFINITY))
-                    mx[g] = 0.0f;
-                sum[g] = 0.0f;
-#pragma unroll
-                for (int j = 0; j < KL; ++j)
-                    if (kv[j])
-                        sum[g] += expf(o[g][j] - mx[g]);
-            }
-            wave_sum(sum);
-#pragma unroll
-            for (int g = 0; g < MG; ++g) {
-                const float lse = logf(sum[g]) + mx[g];
-#pragma unroll
-                for (int j = 0; j < KL; ++j)
-                    o[g][j] -= lse;
-            }
-        }
-        float best[MG];
-#pragma unroll
-        for (int g = 0; g < MG; ++g) {
-            best[g] = NEG ? INFINITY : -INFINITY;
-#pragma unroll
-            for (int j = 0; j < KL; ++j) {
-                o[g][j] += x[j];   // patch + offset
-                if (kv[j])
-                    best[g] = NEG ? __builtin_fminf(best[g], o[g][j]) : __builtin_fmaxf(best[g], o[g][j]);
-            }
-        }
-        wave_best(best, NEG);
+        const unsigned wide4 = (wide >> (m0 - m_first)) & 0xfu;
         float res[MG];
-#pragma unroll
-        for (int g = 0; g < MG; ++g)
-            res[g] = best[g];
-        if (a.finite_eps) {
+        if (wide4 != 0xfu) {
             float sum[MG];
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
                 sum[g] = 0.0f;
 #pragma unroll
                 for (int j = 0; j < KL; ++j)
-                    if (kv[j])
-                        sum[g] += __builtin_amdgcn_exp2f(__builtin_fmaf(o[g][j] - best[g], a.c1, a.c0));
+                    sum[g] = __builtin_fmaf(ex[j], kv[j] ? o[g][j] : 0.0f, sum[g]);
             }
             wave_sum(sum);
 #pragma unroll
             for (int g = 0; g < MG; ++g)
-                res[g] = __builtin_fmaf(__builtin_amdgcn_logf(sum[g]), a.ln2_over_eps, best[g]);
+                res[g] = (__builtin_amdgcn_logf(sum[g]) + (mpt + (a.omax[row0 + min(m0 + g, a.M - 1)] + a.c0))) *
+                         a.ln2_over_eps;
+        }
+        if (wide4 != 0) {
+            float best[MG], v[MG][KL];
+#pragma unroll
+            for (int g = 0; g < MG; ++g) {
+                best[g] = NEG ? INFINITY : -INFINITY;
+#pragma unroll
+                for (int j = 0; j < KL; ++j) {
+                    v[g][j] = x[j] + o[g][j];   // patch + offset
+                    if (kv[j])
+                        best[g] = NEG ? __builtin_fminf(best[g], v[g][j]) : __builtin_fmaxf(best[g], v[g][j]);
+                }
+            }
+            wave_best(best, NEG);
+            float sum[MG];
+            if (a.finite_eps) {
+#pragma unroll
+                for (int g = 0; g < MG; ++g) {
+                    sum[g] = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < KL; ++j)
+                        if (kv[j])
+                            sum[g] += __builtin_amdgcn_exp2f(v[g][j] - best[g]);
+                }
+                wave_sum(sum);
+            }
+#pragma unroll
+            for (int g = 0; g < MG; ++g)
+                if ((wide4 >> g) & 1u)
+                    res[g] = a.finite_eps ? (__builtin_amdgcn_logf(sum[g]) + (best[g] + a.c0)) * a.ln2_over_eps : best[g];
         }
         if (lane == 0) {
 #pragma unroll
@@ -772,12 +788,12 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a, c
 }
 
 template <int KL>
-hipError_t launch_small(const MexKernelArgs &a, dim3 grid, bool neg, const float *offsets, int normalize, hipStream_t s)
+hipError_t launch_small(const MexKernelArgs &a, dim3 grid, bool neg, hipStream_t s)
 {
     if (neg)
-        hipLaunchKernelGGL((mex_small_kernel<KL, true>), grid, dim3(256), 0, s, a, offsets, normalize);
+        hipLaunchKernelGGL((mex_small_kernel<KL, true>), grid, dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL((mex_small_kernel<KL, false>), grid, dim3(256), 0, s, a, offsets, normalize);
+        hipLaunchKernelGGL((mex_small_kernel<KL, false>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
@@ -832,7 +848,7 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups)
 }
 
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream, const SimPackJob *job)
+                     void *stream, const SimPackJob *job, bool launch)
 {
     const simnets_mex_dims &d = p.d;
     const long long rows = (long long)d.num_regions * n_mgroups * tm;
@@ -846,6 +862,10 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
     int4 *ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
     if ((long long)d.block_c * p.H * p.W > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;  // the table holds 32-bit offsets
+    a->offp = offp; a->offe = offe; a->omax = omax; a->orng = orng; a->ktab = ktab;
+    a->n_mgroups = n_mgroups;
+    if (!launch)
+        return SIMNETS_OK;  // the arrays are in place already: only the pointers were wanted
     const int row_blocks = (int)((rows + 3) / 4);
     SimPackJob pj = {nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0.0f};
     int extra = 0;
@@ -868,50 +888,56 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
     else
         SIMNETS_PACK_LAUNCH(0);
 #undef SIMNETS_PACK_LAUNCH
-    if (hipGetLastError() != hipSuccess)
+    if (launch && hipGetLastError() != hipSuccess)
         return SIMNETS_ERR_HIP;
-    a->offp = offp; a->offe = offe; a->omax = omax; a->orng = orng; a->ktab = ktab;
-    a->n_mgroups = n_mgroups;
     return SIMNETS_OK;
 }
 
 size_t mex_workspace_bytes(const MexPlan &p)
 {
+    if (mex_use_small(p))
+        return mex_packed_bytes(p, 1, p.d.M);
     const MexTiling t = mex_tiling(p);
     return mex_packed_bytes(p, t.tm, t.n_mgroups);
 }
 
+// phase: kMexPrepare = only the launch that depends on the offsets alone (packing), kMexRun = only the launches
+// that read the packed workspace, both = the whole call.
 int mex_launch(const MexPlan &p, const float *input, const float *offsets, float *output, void *workspace,
-               size_t workspace_bytes, void *stream)
+               size_t workspace_bytes, void *stream, int phase)
 {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const simnets_mex_dims &d = p.d;
     if (workspace_bytes < mex_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
+    const bool pack = (phase & kMexPrepare) != 0;
     if (mex_use_small(p)) {
         MexKernelArgs a = mex_kernel_args(p);
+        const int rc = mex_pack_offsets(p, offsets, 1, d.M, workspace, &a, stream, nullptr, pack);
+        if (rc || !(phase & kMexRun))
+            return rc;
         a.in = input; a.out = output;
         const long long waves = (long long)d.num_regions * a.slots;
         dim3 grid((unsigned)((waves + 3) / 4), (unsigned)((d.M + kSmallMChunk - 1) / kSmallMChunk));
         if (grid.y > 65535)
             return SIMNETS_ERR_TOO_LARGE;
-        const bool neg = p.epsilon < 0;
+        const bool neg = !a.finite_eps && p.epsilon < 0;
         const int kl = (d.K + 63) / 64;
         hipError_t e;
         if (kl <= 2)
-            e = launch_small<2>(a, grid, neg, offsets, p.normalize_offsets, s);
+            e = launch_small<2>(a, grid, neg, s);
         else if (kl <= 4)
-            e = launch_small<4>(a, grid, neg, offsets, p.normalize_offsets, s);
+            e = launch_small<4>(a, grid, neg, s);
         else if (kl <= 8)
-            e = launch_small<8>(a, grid, neg, offsets, p.normalize_offsets, s);
+            e = launch_small<8>(a, grid, neg, s);
         else
-            e = launch_small<16>(a, grid, neg, offsets, p.normalize_offsets, s);
+            e = launch_small<16>(a, grid, neg, s);
         return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
     }
     const MexTiling t = mex_tiling(p);
     MexKernelArgs a = mex_kernel_args(p);
-    const int rc = mex_pack_offsets(p, offsets, t.tm, t.n_mgroups, workspace, &a, stream);
-    if (rc)
+    const int rc = mex_pack_offsets(p, offsets, t.tm, t.n_mgroups, workspace, &a, stream, nullptr, pack);
+    if (rc || !(phase & kMexRun))
         return rc;
     a.in = input; a.out = output;
     a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;

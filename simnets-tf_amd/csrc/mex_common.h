@@ -135,7 +135,8 @@ struct SimPackJob {
     float fudge;
 };
 size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
+// launch = false: the arrays were packed by an earlier call with the same arguments; only the pointers are set.
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream, const SimPackJob *job = nullptr);
+                     void *stream, const SimPackJob *job = nullptr, bool launch = true);
 
 }  // namespace simnets

@@ -372,7 +372,8 @@ bool sim_fusable(const SimPlan &sp, const MexPlan &p, int ph, int pw)
 size_t sim_packed_bytes(const SimPlan &sp) { return align_up((size_t)((sp.O + 31) & ~31) * sp.K * 3 * sizeof(float), 256); }
 
 int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
-                void *workspace, const SimPlan *sp, const float *templates, const float *weights, void *stream)
+                void *workspace, const SimPlan *sp, const float *templates, const float *weights, void *stream,
+                int phase)
 {
     const simnets_mex_dims &d = p.d;
     const int n_mgroups = (d.M + TM - 1) / TM;
@@ -390,8 +391,9 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
         q.snorm = (sp->mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)sp->K) * std::log(2.0 * M_PI)) : 0.0f;
         q.snorm_every = sp->norm_const_every_iteration; q.sB = sp->B;
     }
-    const int rc = mex_pack_offsets(p, offsets, TM, n_mgroups, workspace, &a, stream, sp ? &job : nullptr);
-    if (rc)
+    const int rc = mex_pack_offsets(p, offsets, TM, n_mgroups, workspace, &a, stream, sp ? &job : nullptr,
+                                    (phase & kMexPrepare) != 0);
+    if (rc || !(phase & kMexRun))
         return rc;
     a.in = sp ? nullptr : input;
     q.pooled = pooled;
@@ -430,19 +432,19 @@ size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw)
 }
 
 int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
-                    void *workspace, size_t workspace_bytes, void *stream)
+                    void *workspace, size_t workspace_bytes, void *stream, int phase)
 {
     const simnets_mex_dims &d = p.d;
     if (workspace_bytes < mex_pool_workspace_bytes(p, ph, pw))
         return SIMNETS_ERR_WORKSPACE;
     if (!fusable(p, ph, pw)) {
         float *full = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_workspace_bytes(p));
-        const int rc = mex_launch(p, input, offsets, full, workspace, mex_workspace_bytes(p), stream);
-        if (rc)
+        const int rc = mex_launch(p, input, offsets, full, workspace, mex_workspace_bytes(p), stream, phase);
+        if (rc || !(phase & kMexRun))
             return rc;
         return sum_pool_launch(p.B, d.M * d.channels_out, d.height_out, d.width_out, ph, pw, full, pooled, stream);
     }
-    return pool_launch(p, ph, pw, input, offsets, pooled, workspace, nullptr, nullptr, nullptr, stream);
+    return pool_launch(p, ph, pw, input, offsets, pooled, workspace, nullptr, nullptr, nullptr, stream, phase);
 }
 
 // Similarity -> MEX -> sum pooling.  `mp` is the MEX plan over the Similarity output's shape.
@@ -452,24 +454,32 @@ size_t sim_mex_pool_workspace_bytes(const SimPlan &sp, const MexPlan &mp, int ph
         return mex_packed_bytes(mp, TM, (mp.d.M + TM - 1) / TM) + sim_packed_bytes(sp);
     // otherwise: the Similarity output in scratch memory, then the two (or three) kernels
     const size_t mid = align_up((size_t)sp.B * sp.O * sp.oh * sp.ow * sizeof(float), 256);
-    return mid + std::max(sim_workspace_bytes(sp), mex_pool_workspace_bytes(mp, ph, pw));
+    return mid + align_up(sim_workspace_bytes(sp), 256) + mex_pool_workspace_bytes(mp, ph, pw);
 }
 
 int sim_mex_pool_launch(const SimPlan &sp, const MexPlan &mp, int ph, int pw, const float *input,
                         const float *templates, const float *weights, const float *offsets, float *pooled,
-                        void *workspace, size_t workspace_bytes, void *stream)
+                        void *workspace, size_t workspace_bytes, void *stream, int phase)
 {
     if (workspace_bytes < sim_mex_pool_workspace_bytes(sp, mp, ph, pw))
         return SIMNETS_ERR_WORKSPACE;
     if (sim_fusable(sp, mp, ph, pw))
-        return pool_launch(mp, ph, pw, input, offsets, pooled, workspace, &sp, templates, weights, stream);
+        return pool_launch(mp, ph, pw, input, offsets, pooled, workspace, &sp, templates, weights, stream, phase);
+    // separate kernels: [Similarity output | Similarity workspace | MEX + pooling workspace] (the two workspaces side
+    // by side, so that both can stay prepared)
     const size_t mid_bytes = align_up((size_t)sp.B * sp.O * sp.oh * sp.ow * sizeof(float), 256);
+    const size_t sim_bytes = align_up(sim_workspace_bytes(sp), 256);
     float *mid = reinterpret_cast<float *>(workspace);
-    char *rest = reinterpret_cast<char *>(workspace) + mid_bytes;
-    int rc = sim_launch(sp, input, templates, weights, mid, rest, workspace_bytes - mid_bytes, stream);
+    char *sim_ws = reinterpret_cast<char *>(workspace) + mid_bytes;
+    char *rest = sim_ws + sim_bytes;
+    int rc = SIMNETS_OK;
+    if (phase & kMexPrepare)
+        rc = sim_prepare(sp, templates, weights, sim_ws, sim_bytes, stream);
+    if (!rc && (phase & kMexRun))
+        rc = sim_run(sp, input, mid, sim_ws, sim_bytes, stream);
     if (rc)
         return rc;
-    return mex_pool_launch(mp, ph, pw, mid, offsets, pooled, rest, workspace_bytes - mid_bytes, stream);
+    return mex_pool_launch(mp, ph, pw, mid, offsets, pooled, rest, workspace_bytes - mid_bytes - sim_bytes, stream, phase);
 }
 
 }  // namespace simnets

@@ -62,13 +62,14 @@ struct SimKernelArgs {
     int norm_every_iteration;
     int vec_store;     // output rows are 16-byte aligned: store float4
     int fast_stage;    // the channel tile has at most kStagePos * kThreads elements: division-free staging
-    // sqrt-weight form only (see sim_guard_fix_kernel)
-    const float *templates, *weights;  // the caller's arrays [O][K]
-    const float *thr;  // [O] outputs of template m above -thr[m] are recomputed exactly
-    int *flags;        // [workgroups * kWaves] set by a wave that wrote such an output
+    int plds_off;      // PLDS variants: where the workgroup's parameter copy starts in LDS (floats, multiple of 4)
+    // sqrt-weight form only (see the guard in sim_direct_kernel)
+    const float *pa2;  // [mtile][K][MT][2]  (template, negative weight): what the recomputing pass reads
+    const float *thr;  // [O] a partial sum of template m above -thr[m] sends its wave to the recomputing pass
+    int *flags;        // [workgroups * kWaves] 1: the wave left its outputs to the recomputing pass
 };
 
-// Output positions of a lane: the mapping shared by sim_direct_kernel and sim_guard_fix_kernel.
+// Output positions of a lane.
 struct LanePos {
     int b, tile, ws, mtile;
     int g_first, g_last, row_first;
@@ -124,7 +125,12 @@ constexpr int kSmallPT = 4, kSmallMT = 8;
 constexpr int waves_per_simd(int pt, int mt) { return pt * mt <= 64 ? 4 : 2; }
 constexpr int lds_budget_floats(int pt, int mt) { return pt * mt <= 64 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
 
-template <int MODE, int PT, int MT, int SWT>
+// GATED: the recomputing pass of the sqrt-weight form - same grid as the main launch, a workgroup none of whose
+//        waves raised its flag returns at once, the others recompute the flagged waves' outputs (MODE = SIM_MODE_L2
+//        on the second packed copy, bit-identical to SIMNETS_ALGO_DIRECT).
+// PLDS:  the workgroup's packed parameters (all K) are copied to LDS once and read from there by broadcast:
+//        for short K the step-ahead global loads would cost one memory latency per k.
+template <int MODE, int PT, int MT, int SWT, bool GATED = false, bool PLDS = false>
 __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
 {
     extern __shared__ float lds[];
@@ -135,7 +141,15 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
 
     const LanePos lp = lane_pos(a, wave, lane);
     const int b = lp.b, mtile = lp.mtile, h = lp.h, gw = lp.gw;
-    const bool wave_active = lp.wave_active, lane_valid = lp.lane_valid;
+    const bool lane_valid = lp.lane_valid;
+    bool wave_active = lp.wave_active;
+    const size_t flag0 = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves;
+    if (GATED) {
+        const int SIMNETS_CONST_AS *f = (const int SIMNETS_CONST_AS *)(a.flags) + flag0;
+        if ((f[0] | f[1] | f[2] | f[3]) == 0)
+            return;
+        wave_active = wave_active && f[wave] != 0;  // the other waves only help staging
+    }
 
     // pixel groups of this workgroup and the input rows they need
     const int row_first = lp.row_first;
@@ -156,11 +170,33 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     // values arrive in VGPRs, which is where the arithmetic wants them (VALU instructions with SGPR
     // operands issue at half rate), at the cost of 4 load instructions per k instead of one scalar load
     // plus 16 moves; they use the vector-memory counter, so waiting for LDS data never waits for them.
+    // PLDS: the same stream out of the LDS copy (every lane one address: a broadcast read).
     unsigned zero_v;
     asm volatile("v_mov_b32 %0, 0" : "=v"(zero_v));
     constexpr bool HAS_PC = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
-    const char *pa_base = reinterpret_cast<const char *>(a.pa + (size_t)(wave_active ? mtile : 0) * a.K * MT * 2);
-    const char *pc_base = reinterpret_cast<const char *>(a.pc + (size_t)(wave_active ? mtile : 0) * a.K * MT);
+    const int mtile_c = lp.wave_active ? mtile : 0;
+    const int wm = wave >> a.nws_log2;
+    const int pk = (a.K + 1) * MT;  // floats of one wave's pc block in LDS (its pa block: twice that), one k of slack
+    const char *pa_base = PLDS ? reinterpret_cast<const char *>(lds + a.plds_off + wm * 3 * pk)
+                               : reinterpret_cast<const char *>((GATED ? a.pa2 : a.pa) + (size_t)mtile_c * a.K * MT * 2);
+    const char *pc_base = PLDS ? reinterpret_cast<const char *>(lds + a.plds_off + wm * 3 * pk + 2 * pk)
+                               : reinterpret_cast<const char *>(a.pc + (size_t)mtile_c * a.K * MT);
+    if (PLDS) {
+        // copy the parameters of the workgroup's template tiles: [wm][pa: K*MT*2 | slack | pc: K*MT | slack]
+        const int nwm = kWaves >> a.nws_log2;
+        for (int j = 0; j < nwm; ++j) {
+            const int mt = min((int)blockIdx.y * nwm + j, a.n_mtiles - 1);
+            const float *ga = a.pa + (size_t)mt * a.K * MT * 2;
+            float *la = lds + a.plds_off + j * 3 * pk;
+            for (int i = tid; i < a.K * MT * 2; i += kThreads)
+                la[i] = ga[i];
+            if (HAS_PC) {
+                const float *gc = a.pc + (size_t)mt * a.K * MT;
+                for (int i = tid; i < a.K * MT; i += kThreads)
+                    la[2 * pk + i] = gc[i];
+            }
+        }
+    }
     unsigned pa_off = zero_v, pc_off = zero_v;  // byte offsets of the NEXT k
     auto fetch_params = [&](float (&pav)[2 * MT], float (&pcv)[MT]) {
 #pragma unroll
@@ -185,7 +221,8 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
     const int chan_lds = a.TRmax * a.TC;
     float pa0[2 * MT], pc0[MT], pa1[2 * MT], pc1[MT];
-    fetch_params(pa0, pc0);
+    if (!PLDS)
+        fetch_params(pa0, pc0);
     TilePositions<kStagePos> tp;
     tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
     // LDS offsets of the patch elements, one scalar load per k, fetched two steps ahead
@@ -201,48 +238,73 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
             stage_input_tile<kThreads, 8>(lds, img, a.H, a.W, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.pw, a.oob,
                                           nullptr);
         __syncthreads();
-        if (!wave_active)
-            continue;
-        // ---- accumulate over the k of these channels, in k order.  Software pipeline: the pixel
-        //      values and the parameters of step k+1 are requested before the arithmetic of step k,
-        //      ping-ponging between two register sets (no copies) ----
-        const int nk = ccn * a.bh * a.bw;
-        int off_next = kt[1];  // offset of step k+1 (the entries behind the last k are 0)
-        auto step = [&](const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT], float (&xnx)[PT],
-                        float (&panx)[2 * MT], float (&pcnx)[MT]) {
-            // everything outstanding on the LDS / scalar counter was issued a whole step ago
-            __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
-            __builtin_amdgcn_sched_barrier(0);
+        if (PLDS && ch0 == 0)
+            fetch_params(pa0, pc0);  // the parameter copy is in place behind the same barrier
+        if (wave_active) {
+            // ---- accumulate over the k of these channels, in k order.  Software pipeline: the pixel
+            //      values and the parameters of step k+1 are requested before the arithmetic of step k,
+            //      ping-ponging between two register sets (no copies) ----
+            const int nk = ccn * a.bh * a.bw;
+            int off_next = kt[1];  // offset of step k+1 (the entries behind the last k are 0)
+            auto step = [&](const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT], float (&xnx)[PT],
+                            float (&panx)[2 * MT], float (&pcnx)[MT]) {
+                // everything outstanding on the LDS / scalar counter was issued a whole step ago
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0)
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int p = 0; p < PT; ++p)
-                xnx[p] = lds[lds_base + off_next + p * sw];
-            kt += 1;
-            off_next = kt[1];
-            fetch_params(panx, pcnx);  // one k of slack exists behind the arrays
-            __builtin_amdgcn_sched_barrier(0);
-            sim_step<MODE, PT, MT, true>(acc, xc, pac, pcc);
-            __builtin_amdgcn_sched_barrier(0);
-        };
-        float x0[PT], x1[PT];
-        {
-            const int off0 = kt[0];
+                for (int p = 0; p < PT; ++p)
+                    xnx[p] = lds[lds_base + off_next + p * sw];
+                kt += 1;
+                off_next = kt[1];
+                fetch_params(panx, pcnx);  // one k of slack exists behind the arrays
+                __builtin_amdgcn_sched_barrier(0);
+                sim_step<MODE, PT, MT, true>(acc, xc, pac, pcc);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            float x0[PT], x1[PT];
+            {
+                const int off0 = kt[0];
 #pragma unroll
-            for (int p = 0; p < PT; ++p)
-                x0[p] = lds[lds_base + off0 + p * sw];
+                for (int p = 0; p < PT; ++p)
+                    x0[p] = lds[lds_base + off0 + p * sw];
+            }
+            int kk = 0;
+            for (; kk + 2 <= nk; kk += 2) {
+                step(x0, pa0, pc0, x1, pa1, pc1);
+                step(x1, pa1, pc1, x0, pa0, pc0);
+            }
+            if (kk < nk) {
+                step(x0, pa0, pc0, x1, pa1, pc1);
+#pragma unroll
+                for (int i = 0; i < 2 * MT; ++i)
+                    pa0[i] = pa1[i];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    pc0[i] = pc1[i];
+            }
         }
-        int kk = 0;
-        for (; kk + 2 <= nk; kk += 2) {
-            step(x0, pa0, pc0, x1, pa1, pc1);
-            step(x1, pa1, pc1, x0, pa0, pc0);
-        }
-        if (kk < nk) {
-            step(x0, pa0, pc0, x1, pa1, pc1);
+        if (MODE == SIM_MODE_L2_SQRTW && ch0 == 0) {
+            // Guard of the sqrt-weight form.  The terms are all <= 0, so -acc only grows from here on: a partial sum
+            // that already lies beyond the template's threshold proves the final output does; a wave with a partial
+            // sum that does not (or is NaN) stops here and leaves its outputs to the recomputing pass.
+            bool suspect = false;
+            if (wave_active && lane_valid) {
 #pragma unroll
-            for (int i = 0; i < 2 * MT; ++i)
-                pa0[i] = pa1[i];
+                for (int m = 0; m < MT; ++m) {
+                    const int mm = mtile * MT + m;
+                    if (mm >= a.O)
+                        break;
+                    const float thr = a.thr[mm];
 #pragma unroll
-            for (int i = 0; i < MT; ++i)
-                pc0[i] = pc1[i];
+                    for (int p = 0; p < PT; ++p)
+                        suspect |= gw * PT + p < a.ow && !(-acc[m][p] >= thr);
+                }
+            }
+            const bool bail = __any(suspect);
+            if (lane == 0)
+                a.flags[flag0 + wave] = bail ? 1 : 0;
+            if (bail)
+                wave_active = false;
         }
     }
 
@@ -253,7 +315,6 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     if (MODE == SIM_MODE_L2_NORM)
         reps = a.norm_every_iteration ? (a.B - b) : 1;
     const int w0 = gw * PT;
-    bool suspect = false;  // sqrt-weight form: an output so close to zero that its rounding error may show
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int mm = mtile * MT + m;
@@ -265,12 +326,6 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
             v[p] = acc[m][p];
             for (int r = 0; r < reps; ++r)
                 v[p] += a.norm_const;
-        }
-        if (MODE == SIM_MODE_L2_SQRTW) {
-            const float thr = a.thr[mm];
-#pragma unroll
-            for (int p = 0; p < PT; ++p)
-                suspect |= w0 + p < a.ow && !(-v[p] >= thr);  // (also catches NaN)
         }
         float *o = a.out + (((size_t)b * a.O + mm) * a.oh + h) * a.ow + w0;
         if (a.vec_store && PT % 4 == 0) {
@@ -284,79 +339,6 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
                 if (w0 + p < a.ow)
                     o[p] = v[p];
         }
-    }
-    if (MODE == SIM_MODE_L2_SQRTW && suspect)
-        a.flags[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + wave] = 1;
-}
-
-// Second pass of the sqrt-weight form (plain L2 evaluated as -(sqrt(w) t - sqrt(w) x)^2: 2 instead of 3 VALU
-// instructions per term).  Its rounding differs from the reference's w (t - x)^2 only inside d = sqrt(w)(t - x):
-// |err(d)| <= eps (|sqrt(w) t| + |d|), so by Cauchy-Schwarz the relative error of an output `out` of template m is
-// at most 2 eps sqrt(T_m / out) + O(eps) with T_m = sum_k w t^2: below 4e-6 unless out < T_m / 1024.  The main
-// kernel flags the waves that wrote such an output (exact matches of a patch and a template, in practice); this
-// kernel, launched with the same grid, returns at once for the others and recomputes the flagged waves' small
-// outputs with the reference's arithmetic (d = t - x; acc = fma(-w d, d, acc), k ascending: bit-identical to the
-// direct kernel).  thr[m] = T_m / 1024, or +inf for a template with a negative or NaN weight (sqrt undefined):
-// all outputs of such a template are recomputed.
-template <int PT, int MT>
-__global__ __launch_bounds__(kThreads) void sim_guard_fix_kernel(const SimKernelArgs a)
-{
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    if (a.flags[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves + wave] == 0)
-        return;
-    const LanePos lp = lane_pos(a, wave, lane);
-    if (!lp.wave_active || !lp.lane_valid)
-        return;
-    const int w0 = lp.gw * PT, bhw = a.bh * a.bw;
-    const float *img = a.in + (size_t)lp.b * a.C * a.H * a.W;
-    for (int m = 0; m < MT; ++m) {
-        const int mm = lp.mtile * MT + m;
-        if (mm >= a.O)
-            break;
-        const float thr = a.thr[mm];
-        const float *tp = a.templates + (size_t)mm * a.K, *wp = a.weights + (size_t)mm * a.K;
-        float *o = a.out + (((size_t)lp.b * a.O + mm) * a.oh + lp.h) * a.ow + w0;
-        for (int p = 0; p < PT && w0 + p < a.ow; ++p) {
-            if (-o[p] >= thr)
-                continue;
-            const int hi0 = lp.h * a.sh - a.ph, wi0 = (w0 + p) * a.sw - a.pw;
-            float acc = 0.0f;
-            for (int k = 0; k < a.K; ++k) {
-                const int c = k / bhw, rem = k - c * bhw;
-                const int hi = hi0 + rem / a.bw, wi = wi0 + rem % a.bw;
-                const bool inside = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-                const float x = inside ? img[((size_t)c * a.H + hi) * a.W + wi] : a.oob;
-                const float d = tp[k] - x;
-                acc = __builtin_fmaf(-wp[k] * d, d, acc);
-            }
-            o[p] = acc;
-        }
-    }
-}
-
-// Thresholds of the sqrt-weight form (one wave per template) and the cleared flags.
-__global__ __launch_bounds__(256) void sim_guard_prep_kernel(const float *__restrict__ templates,
-                                                            const float *__restrict__ weights, int O, int K,
-                                                            float *__restrict__ thr, int *__restrict__ flags,
-                                                            long long n_flags)
-{
-    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < n_flags; i += (long long)gridDim.x * 256)
-        flags[i] = 0;
-    const int lane = threadIdx.x & 63;
-    for (int m = blockIdx.x * 4 + (threadIdx.x >> 6); m < O; m += gridDim.x * 4) {
-        float t2 = 0.0f;
-        bool bad = false;
-        for (int k = lane; k < K; k += 64) {
-            const float t = templates[(size_t)m * K + k], w = weights[(size_t)m * K + k];
-            t2 = __builtin_fmaf(w * t, t, t2);
-            bad |= !(w >= 0.0f);
-        }
-        for (int d = 32; d > 0; d >>= 1)
-            t2 += __shfl_xor(t2, d, 64);
-        const bool any_bad = __any(bad);
-        if (lane == 0)
-            thr[m] = (any_bad || !(t2 >= 0.0f)) ? INFINITY : t2 * (1.0f / 1024.0f);
     }
 }
 
@@ -421,13 +403,39 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
 // Packs (template, weight) into the k-major, MT-interleaved layout the parameter loads walk, with
 // the sign and the 1/2 of the normalized modes folded into the weight, and precomputes the
 // per-(m,k) logarithm term.  Replaces interlace_kernel (include/utils/ggemm.cuh:70-87).
-__global__ void sim_pack_params_kernel(const float *__restrict__ templates, const float *__restrict__ weights, int O,
-                                       int K, int MT, int n_mtiles, int mode, float fudge, float *__restrict__ pa,
-                                       float *__restrict__ pc, int *__restrict__ koff, int taps, int bw, int CC,
-                                       int chan_pitch, int TC)
+// Sqrt-weight form (pa2 != nullptr): pa holds (sqrt(w) t, -sqrt(w)), pa2 the plain (t, -w) pairs of the recomputing
+// pass, and the workgroups from `pack_blocks` on write the thresholds, one wave per template:
+// thr[m] = sum_k w t^2 / 1024, or +inf for a template with a negative or NaN weight (sqrt undefined).
+__global__ __launch_bounds__(256) void sim_pack_params_kernel(const float *__restrict__ templates,
+                                                             const float *__restrict__ weights, int O, int K, int MT,
+                                                             int n_mtiles, int mode, float fudge, float *__restrict__ pa,
+                                                             float *__restrict__ pc, int *__restrict__ koff, int taps,
+                                                             int bw, int CC, int chan_pitch, int TC,
+                                                             float *__restrict__ pa2, float *__restrict__ thr,
+                                                             int pack_blocks)
 {
+    if ((int)blockIdx.x >= pack_blocks) {
+        const int lane = threadIdx.x & 63;
+        const int nb = gridDim.x - pack_blocks;
+        for (int m = (blockIdx.x - pack_blocks) * 4 + (threadIdx.x >> 6); m < O; m += nb * 4) {
+            float t2 = 0.0f;
+            bool bad = false;
+            for (int k = lane; k < K; k += 64) {
+                const float t = templates[(size_t)m * K + k], w = weights[(size_t)m * K + k];
+                t2 = __builtin_fmaf(w * t, t, t2);
+                bad |= !(w >= 0.0f);
+            }
+            for (int d = 32; d > 0; d >>= 1)
+                t2 += __shfl_xor(t2, d, 64);
+            const bool any_bad = __any(bad);
+            if (lane == 0)
+                thr[m] = (any_bad || !(t2 >= 0.0f)) ? INFINITY : t2 * (1.0f / 1024.0f);
+        }
+        return;
+    }
+    const int nthreads = pack_blocks * 256;
     // LDS offset of patch element k inside a staged chunk of CC channels; 0 behind the last k
-    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < K + 2; k += gridDim.x * blockDim.x) {
+    for (int k = blockIdx.x * 256 + threadIdx.x; k < K + 2; k += nthreads) {
         int off = 0;
         if (k < K) {
             const int c = k / taps, rem = k - c * taps;
@@ -437,8 +445,7 @@ __global__ void sim_pack_params_kernel(const float *__restrict__ templates, cons
         koff[k] = off;
     }
     const long long total = (long long)n_mtiles * K * MT;
-    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
-         i += (long long)gridDim.x * blockDim.x) {
+    for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < total; i += nthreads) {
         const int mi = (int)(i % MT);
         const long long r = i / MT;
         const int k = (int)(r % K);
@@ -450,6 +457,10 @@ __global__ void sim_pack_params_kernel(const float *__restrict__ templates, cons
             w = weights[(size_t)m * K + k];
         }
         sim_pack_element(mode, m < O, t, w, fudge, pa[2 * i], pa[2 * i + 1], pc[i]);
+        if (pa2 != nullptr) {
+            float unused;
+            sim_pack_element(SIM_MODE_L2, m < O, t, w, fudge, pa2[2 * i], pa2[2 * i + 1], unused);
+        }
     }
 }
 
@@ -520,20 +531,29 @@ Tiling choose_tiling(const SimPlan &p)
     return pick(kSmallPT, kSmallMT);
 }
 
-template <int MODE, int PT, int MT>
+template <int MODE, int PT, int MT, bool GATED, bool PLDS>
 hipError_t launch_direct(const SimKernelArgs &a, dim3 grid, size_t lds_bytes, hipStream_t s)
 {
     if (a.sw == 1)
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     else if (a.sw == 2)
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 2>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 2, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     else
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 0>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 0, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     return hipGetLastError();
 }
 
-template <int MODE>
-hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
+// Floats of the workgroup's parameter copy in LDS (PLDS variants): per template wave (K + 1) * MT * 3.
+size_t plds_floats(const SimPlan &p, const Tiling &t) { return (size_t)(kWaves / t.nws) * (p.K + 1) * t.MT * 3; }
+
+// Short K on the small lane tile: the parameters go through LDS (one memory latency instead of one per k).
+bool use_plds(const SimPlan &p, const Tiling &t)
+{
+    return t.lds_ok && t.PT == kSmallPT && t.MT == kSmallMT && plds_floats(p, t) * sizeof(float) <= 16384;
+}
+
+template <int MODE, bool GATED = false>
+hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipStream_t s)
 {
     if (!t.lds_ok) {
         const long long npix = (long long)a.B * a.oh * a.ow;
@@ -548,13 +568,17 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, hipStream_t s)
     }
     const int nwm = kWaves / a.nws;
     dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
-    const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
+    size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
     if (t.PT == kBigPT && t.MT == kBigMT)
-        return launch_direct<MODE, kBigPT, kBigMT>(a, grid, lds_bytes, s);
-    return launch_direct<MODE, kSmallPT, kSmallMT>(a, grid, lds_bytes, s);
+        return launch_direct<MODE, kBigPT, kBigMT, GATED, false>(a, grid, lds_bytes, s);
+    if (plds && !GATED) {
+        lds_bytes = ((size_t)a.plds_off + (size_t)nwm * (a.K + 1) * kSmallMT * 3) * sizeof(float);
+        return launch_direct<MODE, kSmallPT, kSmallMT, false, true>(a, grid, lds_bytes, s);
+    }
+    return launch_direct<MODE, kSmallPT, kSmallMT, GATED, false>(a, grid, lds_bytes, s);
 }
 
-// the sqrt-weight form runs on the tiled kernel only; its thresholds [O] and wave flags
+// the sqrt-weight form runs on the tiled kernel only
 bool use_sqrtw(const SimPlan &p, const Tiling &t) { return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok; }
 
 long long guard_flags(const SimPlan &p, const Tiling &t)
@@ -563,92 +587,112 @@ long long guard_flags(const SimPlan &p, const Tiling &t)
     return (long long)p.B * t.tiles * ((n_mtiles + nwm - 1) / nwm) * kWaves;
 }
 
-size_t guard_bytes(const SimPlan &p, const Tiling &t)
+// Where the pieces of the workspace lie.  The first three are what every mode reads; the sqrt-weight form adds
+// the second packed copy, the thresholds (all written by the pack kernel) and the wave flags (written by every
+// main launch, read by the recomputing launch behind it).
+struct Layout {
+    size_t pa, pc, koff, pa2, thr, flags, total;
+};
+
+Layout layout(const SimPlan &p, const Tiling &t)
 {
-    if (!use_sqrtw(p, t))
-        return 0;
-    return align_up((size_t)p.O * sizeof(float), 256) + align_up((size_t)guard_flags(p, t) * sizeof(int), 256);
+    const size_t n_mtiles = (p.O + t.MT - 1) / t.MT;
+    // one extra k of slack behind each array: the parameter loads are issued one step ahead
+    const size_t pa_bytes = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
+    Layout l;
+    l.pa = 0;
+    l.pc = l.pa + pa_bytes;
+    l.koff = l.pc + align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
+    l.pa2 = l.koff + align_up(((size_t)p.K + 2) * sizeof(int), 256);
+    l.thr = l.pa2;
+    l.flags = l.pa2;
+    l.total = l.pa2;
+    if (use_sqrtw(p, t)) {
+        l.thr = l.pa2 + pa_bytes;
+        l.flags = l.thr + align_up((size_t)p.O * sizeof(float), 256);
+        l.total = l.flags + align_up((size_t)guard_flags(p, t) * sizeof(int), 256);
+    }
+    return l;
 }
 
 }  // namespace
 
-size_t sim_direct_workspace_bytes(const SimPlan &p)
-{
-    const Tiling t = choose_tiling(p);
-    const size_t n_mtiles = (p.O + t.MT - 1) / t.MT;
-    // one extra k of slack behind each array: the parameter loads are issued one step ahead
-    const size_t pa = align_up((n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
-    const size_t pc = align_up((n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
-    const size_t koff = align_up(((size_t)p.K + 2) * sizeof(int), 256);
-    return pa + pc + koff + guard_bytes(p, t);
-}
+size_t sim_direct_workspace_bytes(const SimPlan &p) { return layout(p, choose_tiling(p)).total; }
 
-int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
-                      float *output, void *workspace, size_t workspace_bytes, hipStream_t s)
+// Writes everything of the workspace that depends on the parameters only (one launch).
+int sim_direct_prepare(const SimPlan &p, const float *templates, const float *weights, void *workspace,
+                       size_t workspace_bytes, hipStream_t s)
 {
     const Tiling t = choose_tiling(p);
-    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
-    const size_t pa_bytes = align_up(((size_t)n_mtiles * p.K + 1) * t.MT * 2 * sizeof(float), 256);
-    if (workspace_bytes < sim_direct_workspace_bytes(p))
+    const Layout l = layout(p, t);
+    if (workspace_bytes < l.total)
         return SIMNETS_ERR_WORKSPACE;
-    float *pa = reinterpret_cast<float *>(workspace);
-    const size_t pc_bytes = align_up(((size_t)n_mtiles * p.K + 1) * t.MT * sizeof(float), 256);
-    float *pc = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + pa_bytes);
-    int *koff = reinterpret_cast<int *>(reinterpret_cast<char *>(workspace) + pa_bytes + pc_bytes);
-
+    char *ws = reinterpret_cast<char *>(workspace);
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
     const long long total = (long long)n_mtiles * p.K * t.MT;
     const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
     const bool sqrtw = use_sqrtw(p, t);
     const int mode = sqrtw ? (int)SIM_MODE_L2_SQRTW : p.mode;
-    const size_t koff_bytes = align_up(((size_t)p.K + 2) * sizeof(int), 256);
-    float *thr = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + pa_bytes + pc_bytes + koff_bytes);
-    int *flags = reinterpret_cast<int *>(reinterpret_cast<char *>(thr) + align_up((size_t)p.O * sizeof(float), 256));
-    if (sqrtw) {
-        const long long n_flags = guard_flags(p, t);
-        const int blocks = (int)std::min<long long>(std::max<long long>((p.O + 3) / 4, (n_flags + 255) / 256), 1024);
-        hipLaunchKernelGGL(sim_guard_prep_kernel, dim3(blocks), dim3(256), 0, s, templates, weights, p.O, p.K, thr,
-                           flags, n_flags);
-        if (hipGetLastError() != hipSuccess)
-            return SIMNETS_ERR_HIP;
-    }
-    hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights, p.O, p.K, t.MT,
-                       n_mtiles, mode, p.fudge, pa, pc, koff, p.bh * p.bw, p.bw, t.CC, t.TRmax * t.TC, t.TC);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
+    const int thr_blocks = sqrtw ? std::min((p.O + 3) / 4, 1024) : 0;
+    hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks + thr_blocks), dim3(256), 0, s, templates, weights, p.O,
+                       p.K, t.MT, n_mtiles, mode, p.fudge, reinterpret_cast<float *>(ws + l.pa),
+                       reinterpret_cast<float *>(ws + l.pc), reinterpret_cast<int *>(ws + l.koff), p.bh * p.bw, p.bw, t.CC,
+                       t.TRmax * t.TC, t.TC, sqrtw ? reinterpret_cast<float *>(ws + l.pa2) : nullptr,
+                       reinterpret_cast<float *>(ws + l.thr), pack_blocks);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+// The forward launches on a prepared workspace.
+int sim_direct_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
+                   hipStream_t s)
+{
+    const Tiling t = choose_tiling(p);
+    const Layout l = layout(p, t);
+    if (workspace_bytes < l.total)
+        return SIMNETS_ERR_WORKSPACE;
+    char *ws = reinterpret_cast<char *>(workspace);
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
+    const bool sqrtw = use_sqrtw(p, t);
+    const int mode = sqrtw ? (int)SIM_MODE_L2_SQRTW : p.mode;
 
     SimKernelArgs a;
-    a.in = input; a.out = output; a.pa = pa; a.pc = pc; a.koff = koff;
+    a.in = input; a.out = output;
+    a.pa = reinterpret_cast<const float *>(ws + l.pa); a.pc = reinterpret_cast<const float *>(ws + l.pc);
+    a.koff = reinterpret_cast<const int *>(ws + l.koff);
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
     a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw; a.K = p.K;
     a.G = t.G; a.gpi = t.gpi; a.tiles = t.tiles; a.nws = t.nws; a.n_mtiles = n_mtiles;
     a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
     a.vec_store = (p.ow % 4 == 0) && ((reinterpret_cast<uintptr_t>(output) & 15) == 0);
     a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC; a.fast_stage = t.fast_stage;
+    a.plds_off = (int)align_up((size_t)t.CC * t.TRmax * t.TC, 4);
     a.oob = p.oob;
     // Dtype(-0.5) * Dtype(K_) * std::log(2.0 * M_PI), rounded to float by Eigen's constant()
     a.norm_const = (p.mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)p.K) * std::log(2.0 * M_PI)) : 0.0f;
     a.norm_every_iteration = p.norm_const_every_iteration;
-    a.templates = templates; a.weights = weights; a.thr = thr; a.flags = flags;
+    a.pa2 = reinterpret_cast<const float *>(ws + l.pa2);
+    a.thr = reinterpret_cast<const float *>(ws + l.thr);
+    a.flags = reinterpret_cast<int *>(ws + l.flags);
 
+    const bool plds = use_plds(p, t);
     hipError_t e;
     switch (mode) {
-    case SIM_MODE_L1: e = launch_mode<SIM_MODE_L1>(a, t, s); break;
-    case SIM_MODE_L2: e = launch_mode<SIM_MODE_L2>(a, t, s); break;
-    case SIM_MODE_L2_NORM: e = launch_mode<SIM_MODE_L2_NORM>(a, t, s); break;
-    case SIM_MODE_L2_NORM_IGNORE_NAN: e = launch_mode<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, s); break;
-    default: e = launch_mode<SIM_MODE_L2_SQRTW>(a, t, s); break;
+    case SIM_MODE_L1: e = launch_mode<SIM_MODE_L1>(a, t, plds, s); break;
+    case SIM_MODE_L2: e = launch_mode<SIM_MODE_L2>(a, t, plds, s); break;
+    case SIM_MODE_L2_NORM: e = launch_mode<SIM_MODE_L2_NORM>(a, t, plds, s); break;
+    case SIM_MODE_L2_NORM_IGNORE_NAN: e = launch_mode<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, plds, s); break;
+    default: e = launch_mode<SIM_MODE_L2_SQRTW>(a, t, plds, s); break;
     }
-    if (e == hipSuccess && sqrtw) {
-        // same grid as the main kernel: a wave looks at its flag and, almost always, returns
-        const int nwm = kWaves / a.nws;
-        dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
-        if (t.PT == kBigPT && t.MT == kBigMT)
-            hipLaunchKernelGGL((sim_guard_fix_kernel<kBigPT, kBigMT>), grid, dim3(kThreads), 0, s, a);
-        else
-            hipLaunchKernelGGL((sim_guard_fix_kernel<kSmallPT, kSmallMT>), grid, dim3(kThreads), 0, s, a);
-        e = hipGetLastError();
-    }
+    if (e == hipSuccess && sqrtw)  // same grid: a workgroup looks at its waves' flags and, almost always, returns
+        e = launch_mode<SIM_MODE_L2, true>(a, t, false, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
+                      float *output, void *workspace, size_t workspace_bytes, hipStream_t s)
+{
+    const int rc = sim_direct_prepare(p, templates, weights, workspace, workspace_bytes, s);
+    return rc ? rc : sim_direct_run(p, input, output, workspace, workspace_bytes, s);
 }
 
 }  // namespace simnets

@@ -389,30 +389,52 @@ size_t sim_mfma_workspace_bytes(const SimPlan &p)
            align_up((size_t)p.C * sizeof(float), 256);
 }
 
-int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
-                    void *workspace, size_t workspace_bytes, hipStream_t s)
+namespace {
+struct MfmaLayout {
+    float *pm, *bias, *ctr;
+};
+MfmaLayout mfma_layout(const MfmaTiling &t, void *workspace)
+{
+    char *ws = reinterpret_cast<char *>(workspace);
+    MfmaLayout l;
+    l.pm = reinterpret_cast<float *>(ws);
+    l.bias = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256));
+    l.ctr = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256) +
+                                      align_up((size_t)t.Opad * sizeof(float), 256));
+    return l;
+}
+}  // namespace
+
+// Writes the parameter-only part of the workspace: channel centres, packed operands, per-template bias.
+int sim_mfma_prepare(const SimPlan &p, const float *templates, const float *weights, void *workspace,
+                     size_t workspace_bytes, hipStream_t s)
 {
     const MfmaTiling t = mfma_tiling(p);
     if (!t.ok)
         return SIMNETS_ERR_ALGO;  // image rows too long for the LDS tile of this path
     if (workspace_bytes < sim_mfma_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
-    char *ws = reinterpret_cast<char *>(workspace);
-    float *pm = reinterpret_cast<float *>(ws);
-    float *bias = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256));
-    float *ctr = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256) +
-                                           align_up((size_t)t.Opad * sizeof(float), 256));
+    const MfmaLayout l = mfma_layout(t, workspace);
     const int bhw = p.bh * p.bw;
-    hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, bhw, ctr);
+    hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, bhw, l.ctr);
     const long long total = (long long)t.pm_floats;
     hipLaunchKernelGGL(mfma_pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 8192)), dim3(256), 0, s,
-                       templates, weights, ctr, p.O, t.Opad, p.C, p.bh, p.bw, total, pm);
-    hipLaunchKernelGGL(mfma_bias_kernel, dim3(t.Opad), dim3(256), 0, s, templates, weights, ctr, p.O, p.C, bhw, bias);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
+                       templates, weights, l.ctr, p.O, t.Opad, p.C, p.bh, p.bw, total, l.pm);
+    hipLaunchKernelGGL(mfma_bias_kernel, dim3(t.Opad), dim3(256), 0, s, templates, weights, l.ctr, p.O, p.C, bhw, l.bias);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
 
+int sim_mfma_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
+                 hipStream_t s)
+{
+    const MfmaTiling t = mfma_tiling(p);
+    if (!t.ok)
+        return SIMNETS_ERR_ALGO;
+    if (workspace_bytes < sim_mfma_workspace_bytes(p))
+        return SIMNETS_ERR_WORKSPACE;
+    const MfmaLayout l = mfma_layout(t, workspace);
     MfmaArgs a;
-    a.in = input; a.out = output; a.pm = pm; a.bias = bias; a.ctr = ctr;
+    a.in = input; a.out = output; a.pm = l.pm; a.bias = l.bias; a.ctr = l.ctr;
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.Opad = t.Opad;
     a.oh = p.oh; a.ow = p.ow; a.npix = p.oh * p.ow;
     a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
@@ -423,6 +445,13 @@ int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates
     const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
     hipLaunchKernelGGL(sim_mfma_kernel<false>, grid, dim3(kThreads), lds_bytes, s, a);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+int sim_mfma_launch(const SimPlan &p, const float *input, const float *templates, const float *weights, float *output,
+                    void *workspace, size_t workspace_bytes, hipStream_t s)
+{
+    const int rc = sim_mfma_prepare(p, templates, weights, workspace, workspace_bytes, s);
+    return rc ? rc : sim_mfma_run(p, input, output, workspace, workspace_bytes, s);
 }
 
 namespace {

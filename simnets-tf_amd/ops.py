@@ -567,3 +567,155 @@ def sum_pooling_input_grad(output_grad, input_shape, pool_size=(2, 2)):
         _check(_lib.lib().simnets_hip_sum_pool_input_grad((C.c_int * 4)(B, Cc, H, W), ph, pw, g.data_ptr(),
                                                           dx.data_ptr(), stream))
     return dx
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# Prepared forward calls: the work that depends on the parameters alone (packing the templates / weights / offsets
+# for the kernels) done once, for callers whose parameters stay fixed across calls (inference).  The reference
+# redoes its counterpart on every call (interlace, src/kernels/similarity_kernel_gpu.cu:70; offsets copy,
+# src/kernels/mex_kernel_gpu.cu:98-112).
+# ---------------------------------------------------------------------------------------------------------------
+class Prepared:
+    """A forward operator bound to packed parameters and one input shape; call it with the input.
+
+    Made by `similarity_prepare`, `mex_prepare`, `mex_sum_pool_prepare` or `similarity_mex_sum_pool_prepare`.  The
+    results are those of the plain call, bit for bit.  The buffer also serves as the per-call scratch of the kernels,
+    so calls of one object must not overlap (keep them on one stream).  Later changes of the parameter tensors are
+    not seen: prepare again.
+    """
+
+    def __init__(self, input_shape, output_shape, buffer, run):
+        self.input_shape = tuple(int(v) for v in input_shape)
+        self.output_shape = tuple(int(v) for v in output_shape)
+        self.buffer = buffer
+        self._run = run
+
+    def __call__(self, input, out=None):
+        x = _require_cuda_f32("input", input)
+        if tuple(x.shape) != self.input_shape or x.device != self.buffer.device:
+            raise SimnetsError(-15)
+        if out is None:
+            out = torch.empty(self.output_shape, dtype=torch.float32, device=x.device)
+        else:
+            assert out.is_contiguous() and tuple(out.shape) == self.output_shape and out.dtype == torch.float32 \
+                and out.device == x.device
+        with _on_device(x.device):
+            _check(self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream(x.device).cuda_stream))
+        return out
+
+
+def _prepared_buffer(device, nbytes):
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def similarity_prepare(input_shape, templates, weights, similarity_function=None, blocks=None, strides=None,
+                       padding=None, normalization_term=None, normalization_term_fudge=None, ignore_nan_input=None,
+                       out_of_bounds_value=None, algo=None, norm_const_every_iteration=False):
+    """`similarity(input, templates, weights, ...)` with the parameter packing done here, once: returns a `Prepared`
+    whose call takes the input (of exactly `input_shape`, batch size included) and runs only the forward kernels."""
+    t = _require_cuda_f32("templates", templates)
+    w = _require_cuda_f32("weights", weights)
+    if len(input_shape) != 4 or t.dim() != 4 or w.dim() != 4:
+        raise SimnetsError(-15)
+    l = _lib.lib()
+    a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+                         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+                         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
+                         norm_const_every_iteration=norm_const_every_iteration)
+    I4 = C.c_int * 4
+    xs, ts, wsh = I4(*[int(v) for v in input_shape]), I4(*t.shape), I4(*w.shape)
+    oshape = I4()
+    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
+    buf = _prepared_buffer(t.device, nbytes.value)
+    with _on_device(t.device):
+        stream = torch.cuda.current_stream(t.device).cuda_stream
+        _check(l.simnets_hip_similarity_prepare(C.byref(a), xs, ts, wsh, t.data_ptr(), w.data_ptr(), buf.data_ptr(),
+                                                buf.numel(), stream))
+
+    def run(x_ptr, out_ptr, stream):
+        return l.simnets_hip_similarity_fwd_prepared(C.byref(a), xs, ts, x_ptr, buf.data_ptr(), buf.numel(), out_ptr,
+                                                     stream)
+    return Prepared(input_shape, tuple(oshape), buf, run)
+
+
+def mex_prepare(input_shape, offsets, num_instances, normalize_offsets=False, **attrs):
+    """`mex(input, offsets, num_instances, ...)` with the offsets packed here, once (keyword arguments as `mex`)."""
+    off = _require_cuda_f32("offsets", offsets)
+    if len(input_shape) != 4:
+        raise SimnetsError(-15)
+    l = _lib.lib()
+    a = mex_attrs(num_instances, normalize_offsets=normalize_offsets, **attrs)
+    xs = (C.c_int * 4)(*[int(v) for v in input_shape])
+    oshape = (C.c_int * 4)()
+    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
+    buf = _prepared_buffer(off.device, nbytes.value)
+    with _on_device(off.device):
+        stream = torch.cuda.current_stream(off.device).cuda_stream
+        _check(l.simnets_hip_mex_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), buf.data_ptr(), buf.numel(),
+                                         stream))
+
+    def run(x_ptr, out_ptr, stream):
+        return l.simnets_hip_mex_fwd_prepared(C.byref(a), xs, x_ptr, buf.data_ptr(), buf.numel(), out_ptr, stream)
+    return Prepared(input_shape, tuple(oshape), buf, run)
+
+
+def mex_sum_pool_prepare(input_shape, offsets, num_instances, pool_size=(2, 2), normalize_offsets=False, **attrs):
+    """`mex_sum_pool(input, offsets, num_instances, pool_size, ...)` with the offsets packed here, once."""
+    off = _require_cuda_f32("offsets", offsets)
+    if len(input_shape) != 4:
+        raise SimnetsError(-15)
+    l = _lib.lib()
+    a = mex_attrs(num_instances, normalize_offsets=normalize_offsets, **attrs)
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    xs = (C.c_int * 4)(*[int(v) for v in input_shape])
+    oshape = (C.c_int * 4)()
+    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
+    buf = _prepared_buffer(off.device, nbytes.value)
+    with _on_device(off.device):
+        stream = torch.cuda.current_stream(off.device).cuda_stream
+        _check(l.simnets_hip_mex_sum_pool_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), ph, pw, buf.data_ptr(),
+                                                  buf.numel(), stream))
+
+    def run(x_ptr, out_ptr, stream):
+        return l.simnets_hip_mex_sum_pool_fwd_prepared(C.byref(a), xs, x_ptr, ph, pw, buf.data_ptr(), buf.numel(),
+                                                       out_ptr, stream)
+    return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
+
+
+def similarity_mex_sum_pool_prepare(input_shape, templates, weights, offsets, num_instances, pool_size=(2, 2),
+                                    similarity=None, mex=None):
+    """`similarity_mex_sum_pool(input, templates, weights, offsets, ...)` with all parameters packed here, once."""
+    t = _require_cuda_f32("templates", templates)
+    w = _require_cuda_f32("weights", weights)
+    off = _require_cuda_f32("offsets", offsets)
+    if len(input_shape) != 4 or t.dim() != 4 or tuple(w.shape) != tuple(t.shape):
+        raise SimnetsError(-15)
+    sa = similarity_attrs(**(similarity or {}))
+    ma = mex_attrs(num_instances, **(mex or {}))
+    ph, pw = int(pool_size[0]), int(pool_size[1])
+    l = _lib.lib()
+    I4 = C.c_int * 4
+    xs, ts = I4(*[int(v) for v in input_shape]), I4(*t.shape)
+    mid, oshape = I4(), I4()
+    _check(l.simnets_similarity_out_shape(C.byref(sa), xs, ts, ts, mid))
+    _check(l.simnets_mex_out_shape(C.byref(ma), mid, C.byref(oshape), None))
+    nbytes = C.c_size_t()
+    _check(l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), xs, ts, C.byref(ma), ph, pw,
+                                                                 C.byref(nbytes)))
+    buf = _prepared_buffer(t.device, nbytes.value)
+    with _on_device(t.device):
+        stream = torch.cuda.current_stream(t.device).cuda_stream
+        _check(l.simnets_hip_similarity_mex_sum_pool_prepare(C.byref(sa), xs, ts, t.data_ptr(), w.data_ptr(),
+                                                             C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
+                                                             buf.data_ptr(), buf.numel(), stream))
+
+    def run(x_ptr, out_ptr, stream):
+        return l.simnets_hip_similarity_mex_sum_pool_fwd_prepared(C.byref(sa), xs, ts, x_ptr, C.byref(ma), ph, pw,
+                                                                  buf.data_ptr(), buf.numel(), out_ptr, stream)
+    return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
