@@ -130,7 +130,11 @@ constexpr int lds_budget_floats(int pt, int mt) { return pt * mt <= 64 ? kLdsBud
 //        on the second packed copy, bit-identical to SIMNETS_ALGO_DIRECT).
 // PLDS:  the workgroup's packed parameters (all K) are copied to LDS once and read from there by broadcast:
 //        for short K the step-ahead global loads would cost one memory latency per k.
-template <int MODE, int PT, int MT, int SWT, bool GATED = false, bool PLDS = false>
+// ROW3:  3 x 3 templates at stride 1 (the convolution-like layers): the k loop walks (channel, dh) rows of the
+//        staged tile; a lane reads the PT + 2 values of a row once and the three taps of the row take their
+//        operands from those registers (x of tap dw, pixel p = value dw + p), instead of PT LDS values per tap
+//        through a table of offsets: a third of the LDS instructions, no per-k address arithmetic.
+template <int MODE, int PT, int MT, int SWT, bool GATED = false, bool PLDS = false, bool ROW3 = false>
 __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
 {
     extern __shared__ float lds[];
@@ -227,6 +231,11 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
     // LDS offsets of the patch elements, one scalar load per k, fetched two steps ahead
     const int SIMNETS_CONST_AS *kt = (const int SIMNETS_CONST_AS *)(a.koff);
+    // sqrt-weight form: the thresholds of the wave's MT templates, one per lane (lane % MT), requested now and
+    // read after the first chunk
+    float thr_lane = 0.0f;
+    if (MODE == SIM_MODE_L2_SQRTW)
+        thr_lane = a.thr[min(mtile_c * MT + (lane % MT), a.O - 1)];
 
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
@@ -240,7 +249,67 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
         __syncthreads();
         if (PLDS && ch0 == 0)
             fetch_params(pa0, pc0);  // the parameter copy is in place behind the same barrier
-        if (wave_active) {
+        if (PT % 2 == 0 && (MODE == SIM_MODE_L2_SQRTW || MODE == SIM_MODE_L2))
+            sim_pin_pairs<PT, MT>(acc);
+        if (ROW3 && wave_active) {
+            // ---- rows (channel, dh) of the chunk in k order; per row: the next row's values and, per tap, the
+            //      next tap's parameters are requested before the arithmetic on the current ones ----
+            const int nrow = ccn * 3;
+            int roff = a.TC, rdh = 1;   // LDS offset and dh of the row to request next (row 1 at first)
+            float xa[PT + 2], xb[PT + 2];
+#pragma unroll
+            for (int j = 0; j < PT + 2; ++j)
+                xa[j] = lds[lds_base + j];
+            auto tap = [&](const float *xr, const float (&pac)[2 * MT], const float (&pcc)[MT], float (&panx)[2 * MT],
+                           float (&pcnx)[MT]) {
+                fetch_params(panx, pcnx);  // one k of slack exists behind the arrays
+                __builtin_amdgcn_sched_barrier(0);
+                float xs[PT];
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    xs[p] = xr[p];
+                sim_step<MODE, PT, MT, true>(acc, xs, pac, pcc);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            auto row = [&](int r, const float (&cur)[PT + 2], float (&nxt)[PT + 2], float (&pA)[2 * MT], float (&cA)[MT],
+                           float (&pB)[2 * MT], float (&cB)[MT]) {
+                // everything outstanding was issued a whole tap ago
+                __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+                __builtin_amdgcn_sched_barrier(0);
+                const int off = r + 1 < nrow ? roff : 0;  // behind the chunk's last row: any valid address
+#pragma unroll
+                for (int j = 0; j < PT + 2; ++j)
+                    nxt[j] = lds[lds_base + off + j];
+                rdh += 1;
+                roff += a.TC;
+                if (rdh == 3) {
+                    rdh = 0;
+                    roff += chan_lds - 3 * a.TC;
+                }
+                tap(cur, pA, cA, pB, cB);
+                __builtin_amdgcn_s_waitcnt(0x0070);
+                __builtin_amdgcn_sched_barrier(0);
+                tap(cur + 1, pB, cB, pA, cA);
+                __builtin_amdgcn_s_waitcnt(0x0070);
+                __builtin_amdgcn_sched_barrier(0);
+                tap(cur + 2, pA, cA, pB, cB);
+            };
+            int r = 0;
+            for (; r + 2 <= nrow; r += 2) {
+                row(r, xa, xb, pa0, pc0, pa1, pc1);
+                row(r + 1, xb, xa, pa1, pc1, pa0, pc0);
+            }
+            if (r < nrow) {
+                row(r, xa, xb, pa0, pc0, pa1, pc1);
+#pragma unroll
+                for (int i = 0; i < 2 * MT; ++i)
+                    pa0[i] = pa1[i];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    pc0[i] = pc1[i];
+            }
+        }
+        if (!ROW3 && wave_active) {
             // ---- accumulate over the k of these channels, in k order.  Software pipeline: the pixel
             //      values and the parameters of step k+1 are requested before the arithmetic of step k,
             //      ping-ponging between two register sets (no copies) ----
@@ -284,7 +353,7 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
             }
         }
         if (MODE == SIM_MODE_L2_SQRTW && ch0 == 0) {
-            // Guard of the sqrt-weight form.  The terms are all <= 0, so -acc only grows from here on: a partial sum
+            // Guard of the sqrt-weight form.  The terms all have one sign, so |acc| only grows from here on: a partial sum
             // that already lies beyond the template's threshold proves the final output does; a wave with a partial
             // sum that does not (or is NaN) stops here and leaves its outputs to the recomputing pass.
             bool suspect = false;
@@ -294,10 +363,10 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
                     const int mm = mtile * MT + m;
                     if (mm >= a.O)
                         break;
-                    const float thr = a.thr[mm];
+                    const float thr = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, thr_lane), m));
 #pragma unroll
                     for (int p = 0; p < PT; ++p)
-                        suspect |= gw * PT + p < a.ow && !(-acc[m][p] >= thr);
+                        suspect |= gw * PT + p < a.ow && !(acc[m][p] >= thr);  // (this form accumulates +d*d)
                 }
             }
             const bool bail = __any(suspect);
@@ -323,7 +392,9 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
         float v[PT];
 #pragma unroll
         for (int p = 0; p < PT; ++p) {
-            v[p] = acc[m][p];
+            // the sqrt-weight form summed +d*d: 0 - acc is its exact negative, with +0 for an empty sum like the
+            // reference's 0 + (-0)
+            v[p] = MODE == SIM_MODE_L2_SQRTW ? 0.0f - acc[m][p] : acc[m][p];
             for (int r = 0; r < reps; ++r)
                 v[p] += a.norm_const;
         }
@@ -393,7 +464,7 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
         const int mm = mtile * MT + m;
         if (mm >= a.O)
             break;
-        float v = acc[m][0];
+        float v = MODE == SIM_MODE_L2_SQRTW ? 0.0f - acc[m][0] : acc[m][0];
         for (int r = 0; r < reps; ++r)
             v += a.norm_const;
         a.out[(((size_t)b * a.O + mm) * a.oh + h) * a.ow + w] = v;
@@ -534,6 +605,14 @@ Tiling choose_tiling(const SimPlan &p)
 template <int MODE, int PT, int MT, bool GATED, bool PLDS>
 hipError_t launch_direct(const SimKernelArgs &a, dim3 grid, size_t lds_bytes, hipStream_t s)
 {
+    // (the normalized modes keep the table-driven loop: with their extra operands the row form does not fit the
+    // register file)
+    constexpr bool kRow3 = PT == kBigPT && !PLDS && (MODE == SIM_MODE_L1 || MODE == SIM_MODE_L2 || MODE == SIM_MODE_L2_SQRTW);
+    if (kRow3 && a.sw == 1 && a.bh == 3 && a.bw == 3) {
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, GATED, false, kRow3>), grid, dim3(kThreads), lds_bytes, s,
+                           a);
+        return hipGetLastError();
+    }
     if (a.sw == 1)
         hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     else if (a.sw == 2)
