@@ -39,7 +39,7 @@ SIM_CASES = [
                                             normalization_term=True, ignore_nan_input=True,
                                             out_of_bounds_value=float("nan")), nan=0.25),      # parameters through LDS
     dict(shape=(3, 3, 20, 31), O=21, kw=dict(similarity_function="L1", blocks=[3, 3], strides=[1, 2], padding=[1, 0]), nan=0),
-    dict(shape=(2, 40, 34, 34), O=40, kw=dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1]), nan=0),  # 16x8 tile, 4 chunks
+    dict(shape=(2, 40, 34, 34), O=40, kw=dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1]), nan=0),  # several chunks
     dict(shape=(2, 40, 34, 34), O=40, kw=dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1], algo="direct"), nan=0),
     dict(shape=(2, 40, 34, 34), O=40, kw=dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1], algo="mfma"), nan=0),
     dict(shape=(2, 70, 12, 12), O=12, kw=dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1],
@@ -211,7 +211,7 @@ def test_unfused_pairs_prepared(pkg):
 
 
 # ---- sqrt-weight form over several channel chunks -----------------------------------------------------------------
-CHUNKED = dict(shape=(2, 40, 34, 34), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1])   # 16x8 tile, 4 chunks
+CHUNKED = dict(shape=(2, 40, 34, 34), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1])   # 4x8 tile, 3 chunks
 CHUNKED_SMALL = dict(shape=(2, 70, 12, 12), O=12, blocks=[3, 3], strides=[1, 1], padding=[1, 1])  # 4x8 tile
 
 
@@ -258,3 +258,57 @@ def test_similarity_sqrt_weight_form_over_channel_chunks(pkg, geom, kind):
         assert np.array_equal(got[:, 1::4], exact_form[:, 1::4], equal_nan=True)
     if kind == "ordinary":
         assert not np.array_equal(got, exact_form)      # nothing is recomputed: the two forms round differently
+
+
+# ---- the wide lane tile (16 pixels x 8 templates) needs a grid of 1536 waves: 96 images of 32 x 32 --------------------
+def big_tile_case(C, seed):
+    g = np.random.default_rng(seed)
+    x = (g.normal(size=(96, C, 32, 32)) * 3 + 50).astype(np.float32)
+    t = (g.normal(size=(128, C, 3, 3)) * 3 + 50).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    return x, t, w, dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+
+
+@pytest.mark.parametrize("C", [5, 14, 27])      # one chunk; two chunks of 7 (odd number of rows); three chunks of 9
+@pytest.mark.parametrize("func,algo", [("L2", None), ("L2", "direct"), ("L1", None)])
+def test_similarity_wide_tile_row_loop(pkg, C, func, algo):
+    """3 x 3 templates at stride 1 on the wide lane tile: the k loop walks (channel, dh) rows; sampled images
+    against the oracle."""
+    x, t, w, kw = big_tile_case(C, 51)
+    got = pkg.similarity(dev(x), dev(t), dev(w), similarity_function=func, algo=algo, **kw).cpu().numpy()
+    pick = [0, 37, 95]
+    assert rel_err(got[pick], orc.similarity_fwd(x[pick], t, w, similarity_function=func, threads=8, **kw)) <= SIM_TOL
+
+
+@pytest.mark.parametrize("kind", ["exact", "first_chunk_equal", "all_close", "negative_weights"])
+def test_similarity_wide_tile_sqrt_weight_guard(pkg, kind):
+    x, t, w, kw = big_tile_case(27, 52)
+    g = np.random.default_rng(53)
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1)))
+    hits = []
+    if kind in ("exact", "first_chunk_equal"):
+        for m in range(0, 128, 5):
+            b, i, j = int(g.integers(3)) * 47, int(g.integers(32)), int(g.integers(32))
+            patch = xp[b, :, i:i + 3, j:j + 3]
+            if kind == "exact":
+                t[m] = patch
+                hits.append((b, m, i, j))
+            else:
+                t[m, :9] = patch[:9]
+    elif kind == "all_close":
+        x = (g.normal(size=x.shape) + 1000).astype(np.float32)
+        t = (g.normal(size=t.shape) + 1000).astype(np.float32)
+    else:
+        w[3::16] *= -1.0
+    X, T, W = dev(x), dev(t), dev(w)
+    got = pkg.similarity(X, T, W, **kw).cpu().numpy()
+    exact_form = pkg.similarity(X, T, W, algo="direct", **kw).cpu().numpy()
+    pick = [0, 47, 94]
+    assert rel_err(got[pick], orc.similarity_fwd(x[pick], t, w, threads=8, **kw)) <= SIM_TOL
+    assert rel_err(got, exact_form) <= SIM_TOL
+    for b, m, i, j in hits:
+        assert got[b, m, i, j] == 0.0
+    if kind == "all_close":
+        assert np.array_equal(got, exact_form)
+    if kind == "negative_weights":
+        assert np.array_equal(got[:, 3::16], exact_form[:, 3::16], equal_nan=True)
