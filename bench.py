@@ -3,12 +3,14 @@
 
 One "step" = one Similarity L2 forward over benchmark configuration 3 (input 256x64x32x32, 128
 templates 64x3x3, stride 1, padding 1 -> 256x128x32x32; 19.33 G generalized MACs), inputs already
-resident in HBM, called through the C ABI exactly as an op layer would.  The other configurations
-(1, 2, 3-L1, 4, and the backward operators of configuration 5) and the alternative evaluation paths
-are timed in the same run and reported under "others".  Prints ONE JSON line.
+resident in HBM, called through the C ABI exactly as an op layer would (the self-packing entry
+point: parameter packing included in every step).  The other configurations (1, 2, 3-L1, 4, and the
+backward operators of configuration 5) and the alternative evaluation paths are timed in the same
+run and reported under "others", each beside the CPU oracle timed on a bounded sample of the same
+workload.  Prints ONE JSON line.
 
-The CPU baseline leg times the CPU oracle (a restatement of the reference's CPU kernels) on a
-bounded sample of the same workload; it is the only place this file touches oracle/.
+The CPU baseline legs time the CPU oracle (a restatement of the reference's CPU kernels); they are
+the only places this file touches oracle/, and they run after the GPU timings.
 """
 import argparse
 import json
@@ -23,12 +25,16 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 PEAK_FP32_TFLOPS = 157.3   # MI355X published FP32 vector / FP32 matrix peak (256 CU x 128 FMA lanes x 2.4 GHz x 2)
 PEAK_HBM_GBS = 8000.0
-EXP_RATE = 19.66e12        # v_exp_f32 at a quarter of the 128 lanes/clk/CU VALU rate (17.6e12 measured on the box)
+EXP_RATE_STATED = 9.83e12  # exponentials per second the work table of the baseline document prices MEX against
+EXP_RATE_MEASURED = 19.66e12  # v_exp_f32 at a quarter of the 128 lanes/clk/CU VALU rate (17.6e12 measured on the box)
 
-# HBM bytes per launch of the dominant kernel, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs of this
-# same workload scaled by a copy kernel of known size (profiles/sim_direct_l2_config3.md).
-# Keyed by evaluation path; None where no counter run exists for the current kernel.
-MEASURED_TRAFFIC_BYTES = {"sqrtw": 311.3e6, "direct": 287.0e6, "mfma": 223.3e6}
+# HBM bytes per launch of the dominant kernel of the headline workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
+# scaled by a copy kernel of known size; not measured inside this run: "traffic_source" names the committed summary.
+MEASURED_TRAFFIC = {
+    "sqrtw": (None, "profiles/sim_direct_l2_config3.md"),
+    "direct": (None, "profiles/sim_direct_l2_config3.md"),
+    "mfma": (223.3e6, "profiles/sim_direct_l2_config3_other_forms.md"),
+}
 
 
 def main():
@@ -40,13 +46,13 @@ def main():
                     help="seconds of untimed load before the warm-up steps (lets the clocks of an idle GPU settle)")
     ap.add_argument("--algo", default=None, choices=[None, "direct", "sqrtw", "mfma"],
                     help="evaluation path of the headline Similarity kernel (default: the library default)")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--no-others", action="store_true", help="time only the headline workload")
     ap.add_argument("--pmc-calib", action="store_true",
                     help="also run three 256 MiB device-to-device copies (a plain copy kernel of known size, "
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters)")
-    ap.add_argument("--cpu-images", type=int, default=24,
-                    help="images of configuration 3 the single-threaded CPU baseline times (24 ~ 6 s)")
+    ap.add_argument("--cpu-images", type=int, default=12,
+                    help="images of configuration 3 the single-threaded CPU baseline times per function (12 ~ 3 s)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path is data parallel over the batch; "
@@ -56,7 +62,7 @@ def main():
     import numpy as np
     import torch
     from __graft_entry__ import load_package, build
-    from util import config1, config2, config3
+    from util import config1, config2, config3, config4_stack, rel_err
 
     if not os.path.exists(os.path.join(ROOT, "simnets-tf_amd", "libsimnets_hip.so")):
         build()
@@ -64,6 +70,8 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU: there is no CPU fallback"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+    host_cpus = os.cpu_count() or 1
+    threads = min(host_cpus, 16)
 
     def to_dev(a):
         return torch.from_numpy(np.ascontiguousarray(a)).to(dev)
@@ -84,6 +92,20 @@ def main():
         torch.cuda.synchronize()
         wall = (time.perf_counter() - t0) * 1e3 / steps
         return wall, start.elapsed_time(stop) / steps
+
+    def graph_of(fn, reps):
+        """A HIP graph of `reps` back-to-back calls: per-call time without the host's share of a launch."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            fn()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(reps):
+                fn()
+        return g
 
     if args.pmc_calib:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
@@ -115,6 +137,8 @@ def main():
     gmacs = gmac3 / (ev_ms * 1e-3)
     flop_per_gmac = 4
     achieved_tflops = gmacs * flop_per_gmac / 1e12
+    path = args.algo or "sqrtw"
+    traffic, traffic_source = MEASURED_TRAFFIC[path]
     result = {
         "metric": "Similarity L2 fwd generalized-GMAC/s (config 3), 1 MI355X",
         "value": round(gmac3 / (wall_ms * 1e-3) / 1e9, 1),
@@ -125,14 +149,16 @@ def main():
         "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config3: Similarity L2 fwd 256x64x32x32, 128 templates 64x3x3, s1 p1 "
                                "-> 256x128x32x32 (M=262144 N=128 K=576)",
-                   "algo": args.algo or "auto (sqrt-weight form + exact recomputation of near-zero outputs)",
+                   "algo": args.algo or "auto (sqrt-weight form; waves with a partial sum near zero are recomputed "
+                                        "term by term)",
+                   "entry_point": "simnets_hip_similarity_fwd (packs the parameters in every step)",
                    "gmac_per_step": gmac3},
-        # compute bound at the FP32 peak, which is the same figure for the vector ALU and the FP32 matrix
-        # cores; "engine" says which of the two the kernel runs on
-        "roofline": {"bound": "mfma", "engine": "mfma" if args.algo == "mfma" else "valu",
+        # compute bound: the FP32 vector ALU ("valu") unless the matrix-core path is asked for; the two peaks are
+        # the same 157.3 TFLOP/s
+        "roofline": {"bound": "mfma" if args.algo == "mfma" else "valu",
                      "achieved": round(achieved_tflops, 2), "peak": PEAK_FP32_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(achieved_tflops / PEAK_FP32_TFLOPS, 4),
-                     "traffic": MEASURED_TRAFFIC_BYTES.get(args.algo or "sqrtw"),
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel_ms": round(ev_ms, 4), "flop_per_gmac": flop_per_gmac,
                      "algorithmic_bytes": bytes3,
                      "hbm_frac": round(bytes3 / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)},
@@ -140,95 +166,170 @@ def main():
 
     # ------------------------------------------------------------------ the other configurations
     others = {}
-    if not args.no_others:
-        def entry(ms, gmac, nbytes, flop=None, exp_bound=False):
-            e = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(gmac / (ms * 1e-3) / 1e9, 1),
-                 "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
-            if flop:
-                e["valu_frac"] = round(gmac / (ms * 1e-3) * flop / 1e12 / PEAK_FP32_TFLOPS, 4)
-            if exp_bound:
-                # MEX: 1 exp + 5 flop per gMAC
-                e["exp_frac"] = round(gmac / (ms * 1e-3) / EXP_RATE, 4)
-                e["valu_frac"] = round(gmac / (ms * 1e-3) * 5 / 1e12 / PEAK_FP32_TFLOPS, 4)
-            return e
+    cpu_jobs = []   # (name, callable returning the cpu_baseline dict): run after all GPU timings, once `oracle` is imported
+    oracle = None
 
+    def entry(ms, gmac, nbytes, bound, flop=None):
+        """bound: which roofline prices this shape ("valu", "mfma", "hbm", "exp"); frac is taken against it."""
+        rate = gmac / (ms * 1e-3)
+        e = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(rate / 1e9, 1), "bound": bound,
+             "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4)}
+        if flop:
+            e["valu_frac"] = round(rate * flop / 1e12 / PEAK_FP32_TFLOPS, 4)
+        if bound == "exp":
+            # MEX: 1 exp + 5 flop per generalized MAC in the reference's formulation.  The product form used here
+            # takes one exp per patch element, not per term, so a fraction above 1 is possible.
+            e["exp_frac"] = round(rate / EXP_RATE_STATED, 4)
+            e["exp_frac_measured_rate"] = round(rate / EXP_RATE_MEASURED, 4)
+        e["frac"] = {"valu": e.get("valu_frac"), "mfma": e.get("valu_frac"), "hbm": e["hbm_frac"],
+                     "exp": e.get("exp_frac")}[bound]
+        return e
+
+    def cpu_leg(sample, run_single, run_all, gmac_single, gmac_all, err):
+        t0 = time.perf_counter()
+        run_single()
+        dt = time.perf_counter() - t0
+        t0 = time.perf_counter()
+        run_all()
+        dta = time.perf_counter() - t0
+        return {"value": round(gmac_single / dt / 1e9, 4), "unit": "GMAC/s", "cores": 1, "kind": "port",
+                "sample": sample, "seconds": round(dt, 2),
+                "all_cores": {"value": round(gmac_all / dta / 1e9, 4), "threads": threads,
+                              "note": "batch loop spread over threads; not reference behaviour"},
+                "host_cpus": host_cpus, "max_rel_err_gpu_vs_cpu": err}
+
+    if not args.no_others:
+        def mex_err(got, x, off, n, **kw):
+            want = oracle.mex_fwd(x, off, n, threads=threads, **kw)
+            shift = oracle.mex_fwd(x, off, n, threads=threads,
+                                   **dict(kw, epsilon=math.copysign(math.inf, kw.get("epsilon", 1.0))))
+            return rel_err(got, want, floor=np.maximum(np.abs(shift), np.abs(off).max()))
+
+        # ---- configuration 3, other functions and forms
         _, ms = timed(sim3("L1", None), args.steps, args.warmup)
-        others["config3_L1_direct"] = entry(ms, gmac3, bytes3, flop=3)
+        others["config3_L1_direct"] = entry(ms, gmac3, bytes3, "valu", flop=3)
+        prep3 = pkg.similarity_prepare(x3.shape, T3, W3, similarity_function="L2", algo=args.algo, **kw3)
+        _, ms = timed(lambda: prep3(X3, out=out3), args.steps, args.warmup)
+        others["config3_L2_prepared"] = entry(ms, gmac3, bytes3, "mfma" if args.algo == "mfma" else "valu", flop=4)
+        others["config3_L2_prepared"]["entry_point"] = "simnets_hip_similarity_fwd_prepared (parameters packed once)"
+        del prep3
         for algo in ("direct", "sqrtw", "mfma"):
-            if algo == (args.algo or "sqrtw"):
+            if algo == path:
                 continue
             try:
                 _, ms = timed(sim3("L2", algo), args.steps, args.warmup)
-                others["config3_L2_" + algo] = entry(ms, gmac3, bytes3, flop=4)
+                others["config3_L2_" + algo] = entry(ms, gmac3, bytes3, "mfma" if algo == "mfma" else "valu", flop=4)
             except pkg.SimnetsError as e:
                 others["config3_L2_" + algo] = {"error": str(e)}
+        # worst case of the sqrt-weight form's guard: every wave stops after the first channel chunk and is
+        # recomputed term by term (inputs and templates 1000 +- 3: all outputs far below the thresholds)
+        g = np.random.default_rng(77)
+        XA = to_dev((g.normal(size=x3.shape) + 1000).astype(np.float32))
+        TA = to_dev((g.normal(size=t3.shape) + 1000).astype(np.float32))
+        _, ms_w = timed(lambda: pkg.similarity(XA, TA, W3, out=out3, **kw3), args.steps, args.warmup)
+        got_w = out3.clone()
+        _, ms_d = timed(lambda: pkg.similarity(XA, TA, W3, out=out3, algo="direct", **kw3), args.steps, args.warmup)
+        others["config3_L2_guard_worst_case"] = {
+            "kernel_ms": round(ms_w, 4), "direct_same_data_ms": round(ms_d, 4), "ratio": round(ms_w / ms_d, 3),
+            "bit_identical_to_direct": bool(torch.equal(got_w, out3)),
+            "data": "inputs and templates ~ N(1000, 1): every wave is flagged"}
+        del XA, TA, got_w
 
+        def cpu3(func):
+            def job():
+                n_img = max(1, args.cpu_images)
+                xm = x3[:min(256, threads * 4)]
+                ref = [None]
+
+                def single():
+                    ref[0] = oracle.similarity_fwd(x3[:n_img], t3, w3, similarity_function=func, **kw3)
+                got = pkg.similarity(X3[:n_img], T3, W3, similarity_function=func, algo=args.algo if func == "L2" else None,
+                                     **kw3).cpu().numpy()
+                leg = cpu_leg("%d of 256 images of config 3 (%s), single thread like the reference; -O2, no fast-math"
+                              % (n_img, func), single,
+                              lambda: oracle.similarity_fwd(xm, t3, w3, similarity_function=func, threads=threads, **kw3),
+                              n_img * 128 * 1024 * 576, len(xm) * 128 * 1024 * 576, None)
+                leg["max_rel_err_gpu_vs_cpu"] = rel_err(got, ref[0])
+                return leg
+            return job
+        cpu_jobs.append(("config3_L1_direct", cpu3("L1")))
+
+        # ---- configuration 1
         x1, t1, w1, kw1 = config1(batch=64, nan_frac=0.0)
         X1, T1, W1 = to_dev(x1), to_dev(t1), to_dev(w1)
         o1 = torch.empty((64, 32, 16, 16), device=dev)
         _, ms = timed(lambda: pkg.similarity(X1, T1, W1, out=o1, **kw1), args.steps, args.warmup)
-        others["config1_similarity"] = entry(ms, 2097152, 2298880, flop=6)
+        others["config1_similarity"] = entry(ms, 2097152, 2298880, "hbm", flop=6)
+        prep1 = pkg.similarity_prepare(x1.shape, T1, W1, **kw1)
+        _, ms_p = timed(lambda: prep1(X1, out=o1), 4 * args.steps, args.warmup)
+        _, ms_g = timed(graph_of(lambda: prep1(X1, out=o1), 20).replay, args.steps, args.warmup)
+        others["config1_similarity"].update({
+            "prepared_ms": round(ms_p, 4), "prepared_hip_graph_ms_per_call": round(ms_g / 20, 4),
+            "note": "latency bound: one launch of 64 workgroups; the eager prepared figure is bounded by the host's "
+                    "share of a launch, the graph figure by the kernel"})
 
+        def cpu1():
+            got = o1.cpu().numpy()
+            return cpu_leg("all 64 images of config 1, single thread", lambda: oracle.similarity_fwd(x1, t1, w1, **kw1),
+                           lambda: oracle.similarity_fwd(x1, t1, w1, threads=threads, **kw1), 2097152, 2097152,
+                           rel_err(got, oracle.similarity_fwd(x1, t1, w1, **kw1)))
+        cpu_jobs.append(("config1_similarity", cpu1))
+
+        # ---- configuration 2
         x2, off2, n2, kw2 = config2()
         X2, O2 = to_dev(x2), to_dev(off2)
         o2 = torch.empty((64, 64, 16, 16), device=dev)
         _, ms = timed(lambda: pkg.mex(X2, O2, n2, normalize_offsets=True, out=o2, **kw2), args.steps, args.warmup)
-        others["config2_mex"] = entry(ms, 33554432, 6324224, exp_bound=True)
+        others["config2_mex"] = entry(ms, 33554432, 6324224, "exp", flop=5)
+        prep2 = pkg.mex_prepare(x2.shape, O2, n2, normalize_offsets=True, **kw2)
+        _, ms_p = timed(lambda: prep2(X2, out=o2), 4 * args.steps, args.warmup)
+        _, ms_g = timed(graph_of(lambda: prep2(X2, out=o2), 20).replay, args.steps, args.warmup)
+        others["config2_mex"].update({
+            "prepared_ms": round(ms_p, 4), "prepared_hip_graph_ms_per_call": round(ms_g / 20, 4),
+            "note": "latency bound at this size; the product form takes one exp per patch element (2 M), not per "
+                    "term (33.5 M), so exp_frac prices the reference's formulation, not this kernel's work"})
 
-        # configuration 4: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10), batch 512
-        x4, t4, w4, kw4 = config1(batch=512, nan_frac=0.25)
+        def cpu2():
+            got = o2.cpu().numpy()
+            noff = oracle.normalize_offsets(off2)
+            return cpu_leg("all 64 images of config 2, single thread", lambda: oracle.mex_fwd(x2, noff, n2, **kw2),
+                           lambda: oracle.mex_fwd(x2, noff, n2, threads=threads, **kw2), 33554432, 33554432,
+                           mex_err(got, x2, noff, n2, **kw2))
+        cpu_jobs.append(("config2_mex", cpu2))
+
+        # ---- configuration 4: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10), batch 512
+        x4, t4, w4, kw4, layers_np, (offl_np, nl, kwl) = config4_stack(512)
         X4, T4, W4 = to_dev(x4), to_dev(t4), to_dev(w4)
-        g = np.random.default_rng(4567)
-        layers, ch, size = [], 32, 16
-        for _ in range(4):
-            n = ch * 2
-            off = to_dev((g.normal(size=(4 if size > 1 else 1, n, ch, 1, 1)) * 0.1).astype(np.float32))
-            layers.append((off, n, dict(softmax_mode=True, blocks=[ch, 1, 1], strides=[ch, 1, 1],
-                                        unshared_offset_region=[2])))
-            ch, size = n, size // 2
-        offl = to_dev((g.normal(size=(1, 10, ch, 1, 1)) * 0.1).astype(np.float32))
+        layers = [(to_dev(off), n, kw) for off, n, kw in layers_np]
+        offl = to_dev(offl_np)
 
         def stack():
             cur = pkg.similarity(X4, T4, W4, **kw4)
             for off, n, kw in layers:
                 cur = pkg.sum_pooling(pkg.mex(cur, off, n, normalize_offsets=True, **kw), (2, 2))
-            return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
-                           strides=[ch, 1, 1], shared_offset_region=[1])
+            return pkg.mex(cur, offl, nl, normalize_offsets=True, **kwl)
 
         _, ms = timed(stack, args.steps, args.warmup)
         # the same stack captured once into a HIP graph and replayed: 15 launches without per-launch host work
-        stack()
-        torch.cuda.synchronize()
-        side = torch.cuda.Stream()
-        side.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(side):
-            stack()
-        torch.cuda.current_stream().wait_stream(side)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            graph_out = stack()
+        graph = graph_of(stack, 1)
         _, ms_graph = timed(graph.replay, args.steps, args.warmup)
-        graph_ok = bool(torch.equal(graph_out, stack()))
         gmac4 = 512 * 32 * 256 * 4 + 4 * 268435456 + 512 * 10 * 512
-        others["config4_stack"] = {"kernel_ms": round(ms, 4), "gmac_per_s_G": round(gmac4 / (ms * 1e-3) / 1e9, 1),
-                                   "exp_frac": round(gmac4 / (ms * 1e-3) / EXP_RATE, 4), "batch": 512,
-                                   "kernels": "similarity + 4 x (offset pack + mex + sum pool) + wave-per-pixel mex",
-                                   "hip_graph_replay_ms": round(ms_graph, 4), "hip_graph_matches_eager": graph_ok}
+        bytes4 = 117e6   # compulsory traffic of the six operators (inputs, parameters, outputs once)
+        e4 = entry(ms, gmac4, bytes4 + 79e6, "exp", flop=5)
+        e4.update({"batch": 512, "kernels": "similarity + 4 x (offset pack + mex + sum pool) + offset pack + "
+                                            "wave-per-pixel mex",
+                   "hip_graph_replay_ms": round(ms_graph, 4)})
+        others["config4_stack"] = e4
         # the same stack with every MEX + pooling pair as one call (a fused kernel for this geometry)
         def fused_stack():
             cur = pkg.similarity(X4, T4, W4, **kw4)
             for off, n, kw in layers:
                 cur = pkg.mex_sum_pool(cur, off, n, (2, 2), normalize_offsets=True, **kw)
-            return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
-                           strides=[ch, 1, 1], shared_offset_region=[1])
+            return pkg.mex(cur, offl, nl, normalize_offsets=True, **kwl)
 
         _, ms_fused = timed(fused_stack, args.steps, args.warmup)
-        ref4 = stack()
-        dev4 = float((fused_stack() - ref4).abs().max() / ref4.abs().max())
-        others["config4_stack"].update({"fused_pool_kernel_ms": round(ms_fused, 4),
-                                        "fused_pool_max_dev_of_scale": dev4})
-
-        # ... and with the Similarity layer evaluated inside the first of those kernels
+        e4["fused_pool_kernel_ms"] = round(ms_fused, 4)
+        # ... with the Similarity layer evaluated inside the first of those kernels
         off0, n0, kwm0 = layers[0]
 
         def fused_stack3():
@@ -236,13 +337,31 @@ def main():
                                               mex=dict(kwm0, normalize_offsets=True))
             for off, n, kw in layers[1:]:
                 cur = pkg.mex_sum_pool(cur, off, n, (2, 2), normalize_offsets=True, **kw)
-            return pkg.mex(cur, offl, 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
-                           strides=[ch, 1, 1], shared_offset_region=[1])
+            return pkg.mex(cur, offl, nl, normalize_offsets=True, **kwl)
 
         _, ms_fused3 = timed(fused_stack3, args.steps, args.warmup)
-        dev43 = float((fused_stack3() - ref4).abs().max() / ref4.abs().max())
-        others["config4_stack"].update({"fused_similarity_mex_pool_kernel_ms": round(ms_fused3, 4),
-                                        "fused_similarity_mex_pool_max_dev_of_scale": dev43})
+        e4["fused_similarity_mex_pool_kernel_ms"] = round(ms_fused3, 4)
+        # ... and with every layer prepared (parameters packed once): five launches per stack
+        shapes, ch, size = [], 32, 16
+        for _, n, _ in layers:
+            shapes.append((512, ch, size, size))
+            ch, size = n, size // 2
+        pf = pkg.similarity_mex_sum_pool_prepare(x4.shape, T4, W4, off0, n0, (2, 2), similarity=kw4,
+                                                 mex=dict(kwm0, normalize_offsets=True))
+        pp = [pkg.mex_sum_pool_prepare(shapes[i], layers[i][0], layers[i][1], (2, 2), normalize_offsets=True,
+                                       **layers[i][2]) for i in range(1, 4)]
+        pl = pkg.mex_prepare((512, ch, 1, 1), offl, nl, normalize_offsets=True, **kwl)
+
+        def prepared_stack():
+            cur = pf(X4)
+            for p in pp:
+                cur = p(cur)
+            return pl(cur)
+
+        _, ms_prep = timed(prepared_stack, args.steps, args.warmup)
+        e4.update({"fused_prepared_ms": round(ms_prep, 4),
+                   "fused_prepared_hbm_frac": round((bytes4 / 1e9) / (ms_prep * 1e-3) / PEAK_HBM_GBS, 4),
+                   "fused_prepared_bit_identical_to_fused": bool(torch.equal(prepared_stack(), fused_stack3()))})
         # a training step of the same stack through the differentiable layer functions: forward with the unfused
         # MEX calls (their gradients take the unpooled outputs), then every operator's gradient calls
         L = pkg.layers
@@ -255,33 +374,96 @@ def main():
             cur = L.similarity(X4, train_params[0], train_params[1], **kw4)
             for i, (_, n, kw) in enumerate(layers):
                 cur = L.mex_sum_pool(cur, train_params[2 + i], n, (2, 2), normalize_offsets=True, **kw)
-            out = L.mex(cur, train_params[-1], 10, normalize_offsets=True, softmax_mode=True, blocks=[ch, 1, 1],
-                        strides=[ch, 1, 1], shared_offset_region=[1])
+            out = L.mex(cur, train_params[-1], nl, normalize_offsets=True, **kwl)
             out.sum().backward()
 
         _, ms_train = timed(train_step, args.steps, args.warmup)
-        others["config4_stack"]["train_step_ms"] = round(ms_train, 4)
+        e4["train_step_ms"] = round(ms_train, 4)
         del train_params
-        # backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
+
+        def cpu4():
+            """The stack on the CPU oracle, layer by layer on 64 of the 512 images (single thread), all 512 with
+            threads; the GPU's fused, prepared result against the oracle's on the 64 images."""
+            def run(xb, th):
+                cur = oracle.similarity_fwd(xb, t4, w4, threads=th, **kw4)
+                for off, n, kw in layers_np:
+                    y = oracle.mex_fwd(cur, oracle.normalize_offsets(off), n, threads=th, **kw)
+                    B, Cc, H, W = y.shape
+                    cur = y.reshape(B, Cc, H // 2, 2, W // 2, 2).sum(axis=(3, 5), dtype=np.float32)
+                return oracle.mex_fwd(cur, oracle.normalize_offsets(offl_np), nl, threads=th, **kwl)
+            nb = 64
+            ref = [None]
+
+            def single():
+                ref[0] = run(x4[:nb], 1)
+            got = prepared_stack()[:nb].cpu().numpy()
+            leg = cpu_leg("%d of 512 images through the whole stack, single thread" % nb, single,
+                          lambda: run(x4, threads), gmac4 * nb / 512, gmac4, None)
+            leg["max_dev_of_scale_gpu_vs_cpu"] = float(np.abs(got - ref[0]).max() / np.abs(ref[0]).max())
+            del leg["max_rel_err_gpu_vs_cpu"]
+            return leg
+        cpu_jobs.append(("config4_stack", cpu4))
+
+        # ---- backward (configuration 5): gradients at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         G3 = to_dev(np.random.default_rng(6789).normal(size=(256, 128, 32, 32)).astype(np.float32))
         _, ms = timed(lambda: pkg.similarity_input_grad(X3, T3, W3, G3, similarity_function="L2", **kw3), args.steps,
                       args.warmup)
-        others["config5_similarity_input_grad_L2"] = entry(ms, gmac3, 2 * 67108864 + 589824 + 134217728, flop=4)
+        others["config5_similarity_input_grad_L2"] = entry(ms, gmac3, 2 * 67108864 + 589824 + 134217728, "mfma", flop=4)
         _, ms = timed(lambda: pkg.similarity_parameters_grad(X3, T3, W3, G3, similarity_function="L2", **kw3),
                       args.steps, args.warmup)
-        others["config5_similarity_params_grad_L2"] = entry(ms, gmac3, 67108864 + 3 * 589824 + 134217728, flop=5)
-        del G3
+        others["config5_similarity_params_grad_L2"] = entry(ms, gmac3, 67108864 + 3 * 589824 + 134217728, "mfma", flop=5)
         Y2 = pkg.mex(X2, O2, n2, normalize_offsets=True, **kw2)
         G2 = to_dev(np.random.default_rng(6789).normal(size=(64, 64, 16, 16)).astype(np.float32))
         _, ms = timed(lambda: pkg.mex_input_grad(X2, O2, Y2, G2, n2, normalize_offsets=True, **kw2), args.steps,
                       args.warmup)
-        others["config5_mex_input_grad"] = entry(ms, 33554432, 2 * 2097152 + 2 * 4194304 + 32768, exp_bound=True)
+        others["config5_mex_input_grad"] = entry(ms, 33554432, 2 * 2097152 + 2 * 4194304 + 32768, "exp", flop=5)
         _, ms = timed(lambda: pkg.mex_offsets_grad(X2, O2, Y2, G2, n2, normalize_offsets=True, **kw2), args.steps,
                       args.warmup)
-        others["config5_mex_offsets_grad"] = entry(ms, 33554432, 2097152 + 2 * 4194304 + 2 * 32768, exp_bound=True)
+        others["config5_mex_offsets_grad"] = entry(ms, 33554432, 2097152 + 2 * 4194304 + 2 * 32768, "exp", flop=5)
+
+        def cpu5():
+            """Achieved gradient errors against the fp64 oracle, beside the fp32 oracle's own: the error of an element
+            relative to max(|want|, 1 % of the tensor's largest |want|); Similarity on 2 images of the config-3
+            shape, MEX on 8 images of the config-2 shape."""
+            def gerr(got, want):
+                want = np.asarray(want)
+                return rel_err(got, want, floor=np.full(want.shape, 1e-2 * float(np.abs(want).max())))
+            f64 = lambda *a: [np.asarray(v, dtype=np.float64) for v in a]
+            nb = 2
+            xs, gs = x3[:nb], G3[:nb].cpu().numpy()
+            XS, GS = to_dev(xs), to_dev(gs)
+            out = {}
+            for func in ("L2", "L1"):
+                kw = dict(kw3, similarity_function=func)
+                dx = pkg.similarity_input_grad(XS, T3, W3, GS, **kw).cpu().numpy()
+                dt, dw = [v.cpu().numpy() for v in pkg.similarity_parameters_grad(XS, T3, W3, GS, **kw)]
+                d = f64(xs, t3, w3, gs)
+                tx = oracle.similarity_input_grad(*d, threads=threads, **kw)
+                tt, tw = oracle.similarity_params_grad(*d, threads=threads, **kw)
+                rx = oracle.similarity_input_grad(xs, t3, w3, gs, threads=threads, **kw)
+                rt, rw = oracle.similarity_params_grad(xs, t3, w3, gs, threads=threads, **kw)
+                out["similarity_" + func] = {"input": [gerr(dx, tx), gerr(rx, tx)], "templates": [gerr(dt, tt), gerr(rt, tt)],
+                                             "weights": [gerr(dw, tw), gerr(rw, tw)]}
+            nb = 8
+            xm, gm = x2[:nb], G2[:nb].cpu().numpy()
+            noff = oracle.normalize_offsets(off2)
+            ym = oracle.mex_fwd(xm, noff, n2, **kw2)
+            XM, GM, YM, NOFF = to_dev(xm), to_dev(gm), to_dev(ym), to_dev(noff)
+            di = pkg.mex_input_grad(XM, NOFF, YM, GM, n2, **kw2).cpu().numpy()
+            do = pkg.mex_offsets_grad(XM, NOFF, YM, GM, n2, **kw2).cpu().numpy()
+            d = f64(xm, noff)
+            y64 = oracle.mex_fwd(d[0], d[1], n2, **kw2)
+            ti = oracle.mex_input_grad(d[0], d[1], y64, gm.astype(np.float64), n2, **kw2)
+            to = oracle.mex_offsets_grad(d[0], d[1], y64, gm.astype(np.float64), n2, **kw2)
+            ri = oracle.mex_input_grad(xm, noff, ym, gm, n2, **kw2)
+            ro = oracle.mex_offsets_grad(xm, noff, ym, gm, n2, **kw2)
+            out["mex"] = {"input": [gerr(di, ti), gerr(ri, ti)], "offsets": [gerr(do, to), gerr(ro, to)]}
+            out["what"] = "[gpu, fp32 oracle] error against the fp64 oracle, relative to max(|want|, 1% of max|want|)"
+            return out
+        cpu_jobs.append(("config5_gradient_errors", cpu5))
     result["others"] = others
 
-    # ------------------------------------------------------------------ CPU baseline (bounded sample)
+    # ------------------------------------------------------------------ CPU baselines (bounded samples)
     if not args.no_cpu:
         from oracle import oracle
         n_img = max(1, args.cpu_images)
@@ -289,16 +471,13 @@ def main():
         t0 = time.perf_counter()
         ref = oracle.similarity_fwd(xs, t3, w3, similarity_function="L2", **kw3)
         dt = time.perf_counter() - t0
-        cores = os.cpu_count() or 1
-        threads = min(cores, 16)
-        xm = x3[:min(256, threads * n_img)]
+        xm = x3[:min(256, threads * 4)]
         t0 = time.perf_counter()
         oracle.similarity_fwd(xm, t3, w3, similarity_function="L2", threads=threads, **kw3)
         dtm = time.perf_counter() - t0
         gm = n_img * 128 * 1024 * 576
         gm_all = len(xm) * 128 * 1024 * 576
-        got = out3.cpu().numpy() if False else pkg.similarity(X3[:n_img], T3, W3, similarity_function="L2",
-                                                               algo=args.algo, **kw3).cpu().numpy()
+        got = pkg.similarity(X3[:n_img], T3, W3, similarity_function="L2", algo=args.algo, **kw3).cpu().numpy()
         err = float(np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-6 * np.abs(ref).max())))
         # the reference's own ggemm_cpu (its header, compiled as it lies; include/utils/ggemm_cpu.hpp:462-511) on the
         # im2col matrices of a few of the same images: the loop the reference's CPU kernel spends its time in
@@ -323,11 +502,17 @@ def main():
             "sample": "%d of 256 images of config 3 (L2), single thread like the reference; -O2, no fast-math" % n_img,
             "all_cores": {"value": round(gm_all / dtm / 1e9, 4), "threads": threads, "images": int(len(xm)),
                           "note": "batch loop spread over threads; not reference behaviour"},
-            "host_cpus": cores,
+            "host_cpus": host_cpus,
             "max_rel_err_gpu_vs_cpu": err,
         }
         if ref_ggemm is not None:
             result["cpu_baseline"]["reference_ggemm"] = ref_ggemm
+        for name, job in cpu_jobs:
+            leg = job()
+            if name in others:
+                others[name]["cpu_baseline"] = leg
+            else:
+                others[name] = leg
     print(json.dumps(result))
 
 

@@ -32,6 +32,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <type_traits>
 #include <cmath>
 
 #include "internal.h"
@@ -648,13 +649,35 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
     if (px.out_off < 0)
         return;  // ragged region edge (same for the whole wave)
 
+    const int m_first = blockIdx.y * kSmallMChunk;
+    const int m_end = min(a.M, m_first + kSmallMChunk);
+    const size_t row0 = (size_t)r * a.M;
+    constexpr int MG = 4;   // instances at a time: their shuffle reductions are independent, so the latencies overlap
+    bool kv[KL];
+#pragma unroll
+    for (int j = 0; j < KL; ++j)
+        kv[j] = lane + 64 * j < a.K;
+    // The packed rows of the next four instances are requested while the current four are reduced, the first four
+    // before anything else: exp2(o - row maximum) for finite epsilon (the product form; an instance whose range
+    // turns out too wide loads its plain row again), the plain rows otherwise.
+    const float *rows = (a.finite_eps ? a.offe : a.offp) + row0 * a.K;
+    float on[MG][KL];
+    auto fetch_rows = [&](int m0) __attribute__((always_inline)) {
+#pragma unroll
+        for (int g = 0; g < MG; ++g) {
+            const float *row = rows + (size_t)min(m0 + g, a.M - 1) * a.K;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                on[g][j] = row[kv[j] ? lane + 64 * j : 0];
+        }
+    };
+    fetch_rows(m_first);
+
     const int bhw = a.bh * a.bw;
     float x[KL];
-    bool kv[KL];
 #pragma unroll
     for (int j = 0; j < KL; ++j) {
         const int k = lane + 64 * j;
-        kv[j] = k < a.K;
         const int kk = kv[j] ? k : 0;
         const int dc = kk / bhw;
         const int rem = kk - dc * bhw;
@@ -663,27 +686,46 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
         const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
         x[j] = ok ? px.base[((ptrdiff_t)dc * a.H + dh) * a.W + dw] : a.oob;
     }
-    // four instances at a time: their shuffle reductions are independent, so the latencies overlap
-    constexpr int MG = 4;
-    auto wave_sum = [](float (&v)[MG]) {
-        for (int d = 32; d > 0; d >>= 1)
-#pragma unroll
-            for (int g = 0; g < MG; ++g)
-                v[g] += __shfl_xor(v[g], d, 64);
+    // Wave reductions through the data-parallel-primitive lane patterns (neighbour, pair, half-row mirror, row mirror:
+    // after the four steps every lane holds its 16-lane row's result) and four lane reads for the rows: VALU latencies
+    // instead of a round trip through the LDS crossbar per step.  All 64 lanes are active here.
+    auto dpp = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value,
+                                                                      0xF, 0xF, false));
     };
-    auto wave_best = [](float (&v)[MG], bool neg) {
-        for (int d = 32; d > 0; d >>= 1)
+    auto lane_of = [](float v, int l) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+    };
+    using std::integral_constant;
+    auto wave_sum = [&](float (&v)[MG]) {
 #pragma unroll
-            for (int g = 0; g < MG; ++g) {
-                const float o = __shfl_xor(v[g], d, 64);
-                v[g] = neg ? __builtin_fminf(v[g], o) : __builtin_fmaxf(v[g], o);
-            }
+        for (int g = 0; g < MG; ++g) v[g] += dpp(v[g], integral_constant<int, 0xB1>{});
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] += dpp(v[g], integral_constant<int, 0x4E>{});
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] += dpp(v[g], integral_constant<int, 0x141>{});
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] += dpp(v[g], integral_constant<int, 0x140>{});
+#pragma unroll
+        for (int g = 0; g < MG; ++g)
+            v[g] = (lane_of(v[g], 0) + lane_of(v[g], 16)) + (lane_of(v[g], 32) + lane_of(v[g], 48));
+    };
+    auto best2 = [](float p, float q, bool neg) { return neg ? __builtin_fminf(p, q) : __builtin_fmaxf(p, q); };
+    auto wave_best = [&](float (&v)[MG], bool neg) {
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] = best2(v[g], dpp(v[g], integral_constant<int, 0xB1>{}), neg);
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] = best2(v[g], dpp(v[g], integral_constant<int, 0x4E>{}), neg);
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] = best2(v[g], dpp(v[g], integral_constant<int, 0x141>{}), neg);
+#pragma unroll
+        for (int g = 0; g < MG; ++g) v[g] = best2(v[g], dpp(v[g], integral_constant<int, 0x140>{}), neg);
+#pragma unroll
+        for (int g = 0; g < MG; ++g)
+            v[g] = best2(best2(lane_of(v[g], 0), lane_of(v[g], 16), neg), best2(lane_of(v[g], 32), lane_of(v[g], 48), neg), neg);
     };
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
-    const int m_first = blockIdx.y * kSmallMChunk;
-    const int m_end = min(a.M, m_first + kSmallMChunk);
-    const size_t row0 = (size_t)r * a.M;
     // which form each instance of this wave takes (wave-uniform): bit g of `wide` set -> term by term
     unsigned wide = a.finite_eps ? 0u : 0xffffu;
     if (a.finite_eps) {
@@ -691,19 +733,6 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
             if (!(a.orng[row0 + m] <= kProductRange))
                 wide |= 1u << (m - m_first);
     }
-    // the offsets rows of the next four instances are requested while the current four are reduced
-    float on[MG][KL];
-    auto fetch_rows = [&](int m0) __attribute__((always_inline)) {
-#pragma unroll
-        for (int g = 0; g < MG; ++g) {
-            const int m = min(m0 + g, a.M - 1);
-            const float *row = (((wide >> (m - m_first)) & 1u) ? a.offp : a.offe) + (row0 + m) * a.K;
-#pragma unroll
-            for (int j = 0; j < KL; ++j)
-                on[g][j] = row[kv[j] ? lane + 64 * j : 0];
-        }
-    };
-    fetch_rows(m_first);
     // scaled patch values, their maximum and exponentials (finite epsilon)
     float ex[KL];
     float mp = -INFINITY;
@@ -714,8 +743,9 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
             mp = fmaxf(mp, x[j]);
     }
     if (a.finite_eps) {
-        for (int d = 32; d > 0; d >>= 1)
-            mp = fmaxf(mp, __shfl_xor(mp, d, 64));
+        float mpv[MG] = {mp, mp, mp, mp};
+        wave_best(mpv, false);
+        mp = mpv[0];
         const float m_sub = mp == -INFINITY ? 0.0f : mp;
 #pragma unroll
         for (int j = 0; j < KL; ++j)
@@ -753,9 +783,10 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
 #pragma unroll
             for (int g = 0; g < MG; ++g) {
                 best[g] = NEG ? INFINITY : -INFINITY;
+                const float *prow = a.offp + (row0 + min(m0 + g, a.M - 1)) * a.K;   // the plain (scaled) row
 #pragma unroll
                 for (int j = 0; j < KL; ++j) {
-                    v[g][j] = x[j] + o[g][j];   // patch + offset
+                    v[g][j] = x[j] + (a.finite_eps ? prow[kv[j] ? lane + 64 * j : 0] : o[g][j]);   // patch + offset
                     if (kv[j])
                         best[g] = NEG ? __builtin_fminf(best[g], v[g][j]) : __builtin_fmaxf(best[g], v[g][j]);
                 }

@@ -95,21 +95,23 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
         ppos[tid] = pos;
     }
 
-    bool prod;
-    {
+    // Product form or term by term: decided from the packed row ranges, after the first chunk's loads have been
+    // issued (those assume the product form; a workgroup that turns out wide loads again).
+    auto decide = [&]() {
         int wide = 0;
         if (tid < TM) {
 #pragma unroll
             for (int r = 0; r < R; ++r)
                 wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
         }
-        prod = !__syncthreads_or(wide);
-    }
+        return !__syncthreads_or(wide);
+    };
+    bool prod = true;
     float m_run = -INFINITY;  // running maximum of this thread's staging column
 
-    auto stage = [&](int k0, int kc) {
+    // patch elements k0 + sk + 4u of this thread's column (Similarity channels when SIMF): loads issued, not awaited
+    auto gather = [&](int k0, int kc, float (&v)[U]) {
         const bool full = kc == KC;
-        float v[U];
         if (SIMF) {
             if (k0 == 0) {
                 // taps of this column's Similarity patch (im2col_3d rule of that layer), once per workgroup
@@ -170,6 +172,12 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
                 v[u] = gp.base[ke.x];
             }
         }
+    };
+
+    auto stage = [&](int k0, int kc) {
+        const bool full = kc == KC;
+        float v[U];
+        gather(k0, kc, v);
         // offsets tiles of the R regions: straight copies of kc * TM floats each
         const int on = kc * (TM / 4);
 #pragma unroll
@@ -228,6 +236,28 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     const bool all_rows = m0 + MX <= a.M;                 // same for the whole wave
     float res[4][4];  // [tile][v]: MEX value of (pixel lr of the tile, instance m0 + 4*lq + v)
 
+    // ---- product form, software pipelined: the global loads of chunk i + 1 (patch elements and offsets tiles, into
+    //      registers) are issued before the matrix loop of chunk i and written to LDS after it ----
+    constexpr int TILE4 = KC * TM / 4;                       // float4 of one region's offsets tile
+    constexpr int NO = (TILE4 + kThreads - 1) / kThreads;    // ... per thread
+    float vn[U];
+    float4 on[R * NO];
+    auto issue = [&](int k0, int kc) {
+        const int cnt = kc * (TM / 4);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            const float4 *src = reinterpret_cast<const float4 *>(
+                a.offe + (((size_t)r * a.n_mgroups + mgroup) * a.K + k0) * TM);
+#pragma unroll
+            for (int j = 0; j < NO; ++j) {
+                const int i = tid + j * kThreads;
+                on[r * NO + j] = i < cnt ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);  // rows past kc: zeros
+            }
+        }
+        gather(k0, kc, vn);
+    };
+    issue(0, min(KC, a.K));
+    prod = decide();
     if (prod) {
         floatx4 acc[4];
 #pragma unroll
@@ -237,29 +267,60 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
         const float *oa = os + lq * TM + wm * MX + lr;
         for (int k0 = 0; k0 < a.K; k0 += KC) {
             const int kc = min(KC, a.K - k0);
-            __syncthreads();
-            stage(k0, kc);
-            __syncthreads();
-            if (!wave_active)
-                continue;
-            if (k0 > 0) {
+            // ---- registers -> LDS (the previous chunk's readers are behind the barrier that ended its loop) ----
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    acc[t] *= fsh[wh * 64 + t * 16 + lr];
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int j = 0; j < NO; ++j)
+                    if (TILE4 % kThreads == 0 || tid + j * kThreads < TILE4)
+                        reinterpret_cast<float4 *>(os + r * KC * TM)[tid + j * kThreads] = on[r * NO + j];
+            float pm = -INFINITY;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                vn[u] *= a.scale;
+                if (sk + u * KSTEP < kc)
+                    pm = fmaxf(pm, vn[u]);
             }
-            const int kend = (kc + 3) & ~3;
-            for (int kq = 0; kq < kend; kq += 4) {
-                float av[R], bv[4];
+            pmx[sk * XP + col] = pm;
+            __syncthreads();
 #pragma unroll
-                for (int r = 0; r < R; ++r)
-                    av[r] = oa[r * KC * TM + kq * TM];
+            for (int j = 0; j < KSTEP; ++j)
+                pm = fmaxf(pm, pmx[j * XP + col]);
+            const float m_new = fmaxf(m_run, pm);
+            const float m_sub = m_new == -INFINITY ? 0.0f : m_new;  // nothing finite yet: the terms are exp2(-inf) = 0
 #pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    bv[t] = xa[kq * XP + t * 16];
-#pragma unroll
-                for (int t = 0; t < 4; ++t)
-                    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t % R], bv[t], acc[t], 0, 0, 0);
+            for (int u = 0; u < U; ++u)   // rows past kc hold zeros (the matrix instruction takes 4 k at a time)
+                xs[(sk + u * KSTEP) * XP + col] = sk + u * KSTEP < kc ? __builtin_amdgcn_exp2f(vn[u] - m_sub) : 0.0f;
+            if (sk == 0) {
+                fsh[col] = m_run == m_new ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);
+                msh[col] = m_new;
             }
+            m_run = m_new;
+            __syncthreads();
+            if (k0 + KC < a.K)
+                issue(k0 + KC, min(KC, a.K - k0 - KC));
+            if (wave_active) {
+                if (k0 > 0) {
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        acc[t] *= fsh[wh * 64 + t * 16 + lr];
+                }
+                const int kend = (kc + 3) & ~3;
+                for (int kq = 0; kq < kend; kq += 4) {
+                    float av[R], bv[4];
+#pragma unroll
+                    for (int r = 0; r < R; ++r)
+                        av[r] = oa[r * KC * TM + kq * TM];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        bv[t] = xa[kq * XP + t * 16];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av[t % R], bv[t], acc[t], 0, 0, 0);
+                }
+            }
+            if (k0 + KC < a.K)
+                __syncthreads();  // everyone is done with this chunk's tiles
         }
         if (!wave_active)
             return;
@@ -401,7 +462,11 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     q.Wp = d.width_out / pw;
     // two column halves per workgroup whenever there are slots for both: the extra waves per compute unit pay even
     // when the launch then has fewer workgroups than compute units (measured on 512 images of 2x2 pixels)
-    const int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
+    // ... and four halves (16 waves) when there are many slots and the patches are short: the offsets tiles are
+    // then copied once per 256 pixel columns
+    int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
+    if (ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
+        nh = 4;
     q.spw = nh * 64 / (ph * pw);
     const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
     if (gx > 0x7fffffffLL || n_mgroups > 65535)
@@ -414,7 +479,8 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e;
     if (ph * pw == 4)
-        e = nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s);
+        e = nh == 4 ? launch_pool<4, 4>(a, q, grid, inside, s)
+                    : (nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s));
     else
         e = nh == 2 ? launch_pool<2, 2>(a, q, grid, inside, s) : launch_pool<2, 1>(a, q, grid, inside, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;

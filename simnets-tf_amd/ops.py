@@ -585,22 +585,34 @@ class Prepared:
     """
 
     def __init__(self, input_shape, output_shape, buffer, run):
-        self.input_shape = tuple(int(v) for v in input_shape)
+        self.input_shape = torch.Size(int(v) for v in input_shape)
         self.output_shape = tuple(int(v) for v in output_shape)
         self.buffer = buffer
         self._run = run
+        self._device = buffer.device
+        self._index = buffer.device.index
 
     def __call__(self, input, out=None):
-        x = _require_cuda_f32("input", input)
-        if tuple(x.shape) != self.input_shape or x.device != self.buffer.device:
+        # (kept short: for the small layers this host code, not the kernel, bounds the call rate)
+        x = input
+        if x.shape != self.input_shape or x.device != self._device or x.dtype is not torch.float32:
+            _require_cuda_f32("input", x)
             raise SimnetsError(-15)
+        if not x.is_contiguous():
+            x = x.contiguous()
         if out is None:
-            out = torch.empty(self.output_shape, dtype=torch.float32, device=x.device)
+            out = torch.empty(self.output_shape, dtype=torch.float32, device=self._device)
+        elif not (out.is_contiguous() and tuple(out.shape) == self.output_shape and out.dtype is torch.float32
+                  and out.device == self._device):
+            raise ValueError("out must be a contiguous float32 tensor of shape %s on %s"
+                             % (self.output_shape, self._device))
+        if torch.cuda.current_device() == self._index:
+            code = self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
         else:
-            assert out.is_contiguous() and tuple(out.shape) == self.output_shape and out.dtype == torch.float32 \
-                and out.device == x.device
-        with _on_device(x.device):
-            _check(self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream(x.device).cuda_stream))
+            with torch.cuda.device(self._device):
+                code = self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        if code != 0:
+            raise SimnetsError(code)
         return out
 
 
@@ -634,9 +646,10 @@ def similarity_prepare(input_shape, templates, weights, similarity_function=None
         _check(l.simnets_hip_similarity_prepare(C.byref(a), xs, ts, wsh, t.data_ptr(), w.data_ptr(), buf.data_ptr(),
                                                 buf.numel(), stream))
 
+    fn, ar, bp, bn = l.simnets_hip_similarity_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
+
     def run(x_ptr, out_ptr, stream):
-        return l.simnets_hip_similarity_fwd_prepared(C.byref(a), xs, ts, x_ptr, buf.data_ptr(), buf.numel(), out_ptr,
-                                                     stream)
+        return fn(ar, xs, ts, x_ptr, bp, bn, out_ptr, stream)
     return Prepared(input_shape, tuple(oshape), buf, run)
 
 
@@ -658,8 +671,10 @@ def mex_prepare(input_shape, offsets, num_instances, normalize_offsets=False, **
         _check(l.simnets_hip_mex_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), buf.data_ptr(), buf.numel(),
                                          stream))
 
+    fn, ar, bp, bn = l.simnets_hip_mex_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
+
     def run(x_ptr, out_ptr, stream):
-        return l.simnets_hip_mex_fwd_prepared(C.byref(a), xs, x_ptr, buf.data_ptr(), buf.numel(), out_ptr, stream)
+        return fn(ar, xs, x_ptr, bp, bn, out_ptr, stream)
     return Prepared(input_shape, tuple(oshape), buf, run)
 
 
@@ -682,9 +697,10 @@ def mex_sum_pool_prepare(input_shape, offsets, num_instances, pool_size=(2, 2), 
         _check(l.simnets_hip_mex_sum_pool_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), ph, pw, buf.data_ptr(),
                                                   buf.numel(), stream))
 
+    fn, ar, bp, bn = l.simnets_hip_mex_sum_pool_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
+
     def run(x_ptr, out_ptr, stream):
-        return l.simnets_hip_mex_sum_pool_fwd_prepared(C.byref(a), xs, x_ptr, ph, pw, buf.data_ptr(), buf.numel(),
-                                                       out_ptr, stream)
+        return fn(ar, xs, x_ptr, ph, pw, bp, bn, out_ptr, stream)
     return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
 
 
@@ -715,7 +731,9 @@ def similarity_mex_sum_pool_prepare(input_shape, templates, weights, offsets, nu
                                                              C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
                                                              buf.data_ptr(), buf.numel(), stream))
 
+    fn, sr, mr, bp, bn = (l.simnets_hip_similarity_mex_sum_pool_fwd_prepared, C.byref(sa), C.byref(ma), buf.data_ptr(),
+                          buf.numel())
+
     def run(x_ptr, out_ptr, stream):
-        return l.simnets_hip_similarity_mex_sum_pool_fwd_prepared(C.byref(sa), xs, ts, x_ptr, C.byref(ma), ph, pw,
-                                                                  buf.data_ptr(), buf.numel(), out_ptr, stream)
+        return fn(sr, xs, ts, x_ptr, mr, ph, pw, bp, bn, out_ptr, stream)
     return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
