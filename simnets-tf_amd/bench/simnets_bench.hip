@@ -128,6 +128,68 @@ static float time_ms(hipStream_t s, int reps, const std::function<void()> &fn)
     return ms / reps;
 }
 
+
+// ---------------------------------------------------------------- co-issue probes
+// Streams of unpacked FP32 VALU instructions on fixed registers, two waves per SIMD (the occupancy of the wide
+// Similarity tile): how the parity of the source registers and the number of sources change the issue rate.
+//   0: v_fma acc, a, x, acc with a, x, acc all in even registers      1: a in odd registers
+//   2: acc += d*d with d and acc of one parity                         3: d and acc of opposite parity
+//   4: (d = a*x + b ; acc += d*d), the sqrt-weight pair                5: (d = b - x ; acc = a*|d| + acc), the L1 pair
+//   6: (d = b - x ; q = a*d ; acc += q*d), the three-instruction L2 form
+template <int V>
+__global__ __launch_bounds__(256) void coissue_kernel(float *out, int iters)
+{
+    extern __shared__ float coissue_lds[];   // only to limit the workgroups per CU
+    float r;
+    asm volatile(
+        "v_cvt_f32_u32 v20, %2\n\t"
+        ".irp n,21,22,23,24,25,26,27,28,29,30,31,32,33,34,35,36,40,41,42,43,44,45,46,47,48,49,50,51,52,53,54,55,56,60,61,62,63,64,65,66,67,68,69,70,71,72,73,74,75,80,81,82\n\t"
+        "v_mul_f32 v\\n, 0x3a83126f, v20\n\t"
+        ".endr\n\t"
+        ".irp n,100,104,108,112,116,120,124,128\n\t"
+        "v_mov_b32 v\\n, 0\n\t"
+        ".endr\n\t"
+        "1:\n\t"
+        ".rept 16\n\t"
+        ".irp i,0,1,2,3,4,5,6,7\n\t"
+        ".if %3 == 0\n\t v_fma_f32 v[100+4*\\i], v80, v[20+2*\\i], v[100+4*\\i]\n\t .endif\n\t"
+        ".if %3 == 1\n\t v_fma_f32 v[100+4*\\i], v81, v[20+2*\\i], v[100+4*\\i]\n\t .endif\n\t"
+        ".if %3 == 2\n\t v_fmac_f32 v[100+4*\\i], v[40+2*\\i], v[40+2*\\i]\n\t .endif\n\t"
+        ".if %3 == 3\n\t v_fmac_f32 v[100+4*\\i], v[41+2*\\i], v[41+2*\\i]\n\t .endif\n\t"
+        ".if %3 == 4\n\t v_fma_f32 v[41+2*\\i], v81, v[20+2*\\i], v82\n\t .endif\n\t"
+        ".if %3 >= 5\n\t v_sub_f32 v[41+2*\\i], v82, v[20+2*\\i]\n\t .endif\n\t"
+        ".endr\n\t"
+        ".if %3 == 6\n\t .irp i,0,1,2,3,4,5,6,7\n\t v_mul_f32 v[60+2*\\i], v81, v[41+2*\\i]\n\t .endr\n\t .endif\n\t"
+        ".if %3 >= 4\n\t .irp i,0,1,2,3,4,5,6,7\n\t"
+        ".if %3 == 4\n\t v_fmac_f32 v[100+4*\\i], v[41+2*\\i], v[41+2*\\i]\n\t .endif\n\t"
+        ".if %3 == 5\n\t v_fma_f32 v[100+4*\\i], v81, |v[41+2*\\i]|, v[100+4*\\i]\n\t .endif\n\t"
+        ".if %3 == 6\n\t v_fmac_f32 v[100+4*\\i], v[60+2*\\i], v[41+2*\\i]\n\t .endif\n\t"
+        ".endr\n\t .endif\n\t"
+        ".endr\n\t"
+        "s_sub_u32 %1, %1, 1\n\t"
+        "s_cmp_lg_u32 %1, 0\n\t"
+        "s_cbranch_scc1 1b\n\t"
+        "v_add_f32 %0, v100, v128"
+        : "=v"(r), "+s"(iters)
+        : "v"(threadIdx.x), "n"(V)
+        : "memory", "scc", "v20", "v21", "v22", "v23", "v24", "v25", "v26", "v27", "v28", "v29", "v30", "v31", "v32", "v33", "v34",
+          "v35", "v36", "v40", "v41", "v42", "v43", "v44", "v45", "v46", "v47", "v48", "v49", "v50", "v51", "v52", "v53", "v54",
+          "v55", "v56", "v60", "v61", "v62", "v63", "v64", "v65", "v66", "v67", "v68", "v69", "v70", "v71", "v72", "v73", "v74",
+          "v75", "v80", "v81", "v82", "v100", "v104", "v108", "v112", "v116", "v120", "v124", "v128");
+    out[blockIdx.x * 256 + threadIdx.x] = r;
+}
+
+template <int V>
+static void run_coissue(const char *name, int valu_per_round, float *out, int cus, hipStream_t s)
+{
+    const int iters = 2000, blocks = cus * 2;   // 60 KB of LDS each: two workgroups per CU = two waves per SIMD
+    HIP_OK(hipFuncSetAttribute((const void *)coissue_kernel<V>, hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024));
+    float ms = time_ms(s, 5, [&] { hipLaunchKernelGGL(coissue_kernel<V>, dim3(blocks), dim3(256), 60 * 1024, s, out, iters); });
+    const double ops = (double)blocks * 256 * iters * 16.0 * valu_per_round;
+    printf("{\"probe\": \"%s\", \"waves_per_simd\": 2, \"lane_instr_per_s_T\": %.2f, \"ms\": %.4f}\n", name,
+           ops / (ms * 1e-3) / 1e12, ms);
+}
+
 static void run_peaks(hipStream_t s)
 {
     hipDeviceProp_t prop;
@@ -169,6 +231,13 @@ static void run_peaks(hipStream_t s)
         HIP_OK(hipFree(a));
         HIP_OK(hipFree(b));
     }
+    run_coissue<0>("fma, three sources in even registers", 8, out, cus, s);
+    run_coissue<1>("fma, sources of mixed parity", 8, out, cus, s);
+    run_coissue<2>("acc += d*d, d and acc of one parity", 8, out, cus, s);
+    run_coissue<3>("acc += d*d, d and acc of opposite parity", 8, out, cus, s);
+    run_coissue<4>("d = a*x + b ; acc += d*d (sqrt-weight pair)", 16, out, cus, s);
+    run_coissue<5>("d = b - x ; acc = a*|d| + acc (L1 pair)", 16, out, cus, s);
+    run_coissue<6>("d = b - x ; q = a*d ; acc += q*d (three-instruction L2)", 24, out, cus, s);
     HIP_OK(hipFree(out));
 }
 
@@ -330,11 +399,21 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) run_sim(c, s);
         float ms = time_ms(s, steps, [&] { run_sim(c, s); });
         report("config1 similarity L2 norm ignore-nan 64x1x28x28 -> 64x32x16x16", 2097152.0, 2298880.0, 6, ms, steps);
+        SN_OK(simnets_hip_similarity_prepare(&c.a, c.in, c.tp, c.tp, c.t, c.w, c.ws, c.ws_bytes, s));
+        auto prepared = [&] { SN_OK(simnets_hip_similarity_fwd_prepared(&c.a, c.in, c.tp, c.x, c.ws, c.ws_bytes, c.y, s)); };
+        for (int i = 0; i < warmup; ++i) prepared();
+        ms = time_ms(s, 10 * steps, prepared);
+        report("config1, parameters prepared once (simnets_hip_similarity_fwd_prepared)", 2097152.0, 2298880.0, 6, ms, 10 * steps);
     } else if (config == 2) {
         MexCase c = make_mex(64, 32, 16, 64, false, nullptr);
         for (int i = 0; i < warmup; ++i) run_mex(c, s);
         float ms = time_ms(s, steps, [&] { run_mex(c, s); });
         report("config2 mex 64x32x16x16 -> 64x64x16x16", 33554432.0, 6324224.0, 5, ms, steps);
+        SN_OK(simnets_hip_mex_prepare(&c.a, c.in, c.o, c.off_count, c.ws, c.ws_bytes, s));
+        auto prepared = [&] { SN_OK(simnets_hip_mex_fwd_prepared(&c.a, c.in, c.x, c.ws, c.ws_bytes, c.y, s)); };
+        for (int i = 0; i < warmup; ++i) prepared();
+        ms = time_ms(s, 10 * steps, prepared);
+        report("config2, offsets prepared once (simnets_hip_mex_fwd_prepared)", 33554432.0, 6324224.0, 5, ms, 10 * steps);
     } else if (config == 3) {
         for (int l1 = 0; l1 < 2; ++l1) {
             if (l1 && algo != SIMNETS_ALGO_AUTO && algo != SIMNETS_ALGO_DIRECT)
@@ -343,6 +422,10 @@ int main(int argc, char **argv)
             for (int i = 0; i < warmup; ++i) run_sim(c, s);
             float ms = time_ms(s, steps, [&] { run_sim(c, s); });
             report(l1 ? "config3 similarity L1 256x64x32x32 x 128 templates 3x3" : "config3 similarity L2 256x64x32x32 x 128 templates 3x3",
+                   19327352832.0, 201916416.0, l1 ? 3 : 4, ms, steps);
+            SN_OK(simnets_hip_similarity_prepare(&c.a, c.in, c.tp, c.tp, c.t, c.w, c.ws, c.ws_bytes, s));
+            ms = time_ms(s, steps, [&] { SN_OK(simnets_hip_similarity_fwd_prepared(&c.a, c.in, c.tp, c.x, c.ws, c.ws_bytes, c.y, s)); });
+            report(l1 ? "config3 similarity L1, parameters prepared once" : "config3 similarity L2, parameters prepared once",
                    19327352832.0, 201916416.0, l1 ? 3 : 4, ms, steps);
         }
     } else if (config == 4) {
@@ -406,6 +489,25 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) fused3();
         ms = time_ms(s, steps, fused3);
         report("config4 missing-data stack batch 512, Similarity + MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        // ... and with every layer's parameters packed once (the *_prepare / *_fwd_prepared entry points): the
+        // workspaces above double as the prepared buffers, five launches per stack
+        SN_OK(simnets_hip_similarity_mex_sum_pool_prepare(&sc.a, sc.in, sc.tp, sc.t, sc.w, &mex[0].a, mex[0].o,
+                                                          mex[0].off_count, 2, 2, f0ws, f0bytes, s));
+        for (int l = 1; l < 4; ++l)
+            SN_OK(simnets_hip_mex_sum_pool_prepare(&mex[l].a, mex[l].in, mex[l].o, mex[l].off_count, 2, 2, fws[l],
+                                                   fbytes[l], s));
+        SN_OK(simnets_hip_mex_prepare(&mex[4].a, mex[4].in, mex[4].o, mex[4].off_count, mex[4].ws, mex[4].ws_bytes, s));
+        auto prepared = [&] {
+            SN_OK(simnets_hip_similarity_mex_sum_pool_fwd_prepared(&sc.a, sc.in, sc.tp, sc.x, &mex[0].a, 2, 2, f0ws, f0bytes,
+                                                                   pooled[0], s));
+            for (int l = 1; l < 4; ++l)
+                SN_OK(simnets_hip_mex_sum_pool_fwd_prepared(&mex[l].a, mex[l].in, mex[l].x, 2, 2, fws[l], fbytes[l],
+                                                            pooled[l], s));
+            SN_OK(simnets_hip_mex_fwd_prepared(&mex[4].a, mex[4].in, mex[4].x, mex[4].ws, mex[4].ws_bytes, mex[4].y, s));
+        };
+        for (int i = 0; i < warmup; ++i) prepared();
+        ms = time_ms(s, steps, prepared);
+        report("config4 missing-data stack batch 512, fused, parameters prepared once", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 117e6, 5, ms, steps);
     }
     else if (config == 5) {
         // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
