@@ -346,3 +346,45 @@ def test_static_scratch_entry_point_validates_and_bounds_its_scratch(pkg):
     assert f(C.byref(a), I4(1, 63, 8, 8), small, small, 256, 256, 256, 256, None) == -8        # channel mismatch
     bad = pkg.ops.similarity_attrs(blocks=[3, 3], ignore_nan_input=True)
     assert f(C.byref(bad), I4(1, 64, 8, 8), small, small, 256, 256, 256, 256, None) == -7
+
+
+def test_prepared_entry_points_validate_on_the_host(pkg):
+    # the *_prepare / *_fwd_prepared pairs run the same checks as the self-packing calls before anything is launched
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    a = pkg.ops.similarity_attrs(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    xs, ts = I4(2, 8, 12, 12), I4(5, 8, 3, 3)
+    need = C.c_size_t()
+    assert l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(need)) == 0 and need.value > 0
+    prep, run = l.simnets_hip_similarity_prepare, l.simnets_hip_similarity_fwd_prepared
+    assert prep(C.byref(a), xs, ts, ts, None, 256, 256, need.value, None) == -1              # null templates
+    assert prep(C.byref(a), xs, ts, ts, 256, 256, None, need.value, None) == -17             # no buffer
+    assert prep(C.byref(a), xs, ts, ts, 256, 256, 256, need.value - 1, None) == -17          # buffer too small
+    assert prep(C.byref(a), xs, ts, ts, 256, 256, 257, need.value, None) == -17              # misaligned buffer
+    assert prep(C.byref(a), xs, I4(5, 7, 3, 3), I4(5, 7, 3, 3), 256, 256, 256, need.value, None) == -8
+    assert run(C.byref(a), xs, ts, None, 256, need.value, 256, None) == -1                   # null input
+    assert run(C.byref(a), xs, ts, 256, 256, need.value - 1, 256, None) == -17
+    assert run(C.byref(a), I4(0, 8, 12, 12), ts, None, None, 0, None, None) == 0             # empty batch: nothing to do
+    m = pkg.ops.mex_attrs(4, blocks=[8, 1, 1], strides=[8, 1, 1], unshared_offset_region=[2])
+    ms = I4(2, 8, 6, 6)
+    assert l.simnets_hip_mex_workspace_bytes(C.byref(m), ms, C.byref(need)) == 0 and need.value > 0
+    n_off = 4 * 4 * 8
+    assert l.simnets_hip_mex_prepare(C.byref(m), ms, 256, n_off - 1, 256, need.value, None) == -15   # too few offsets
+    assert l.simnets_hip_mex_prepare(C.byref(m), ms, None, n_off, 256, need.value, None) == -1
+    assert l.simnets_hip_mex_prepare(C.byref(m), ms, 256, n_off, 256, need.value - 1, None) == -17
+    assert l.simnets_hip_mex_fwd_prepared(C.byref(m), ms, None, 256, need.value, 256, None) == -1
+    assert l.simnets_hip_mex_fwd_prepared(C.byref(m), ms, 256, 256, need.value - 1, 256, None) == -17
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(m), ms, 2, 2, C.byref(need)) == 0
+    assert l.simnets_hip_mex_sum_pool_prepare(C.byref(m), ms, 256, n_off, 0, 2, 256, need.value, None) == -15   # pool size
+    assert l.simnets_hip_mex_sum_pool_prepare(C.byref(m), ms, 256, n_off, 2, 2, None, need.value, None) == -17
+    assert l.simnets_hip_mex_sum_pool_fwd_prepared(C.byref(m), ms, 256, 8, 8, 256, need.value, 256, None) == -16  # empty output
+    sa = pkg.ops.similarity_attrs(blocks=[2, 2], strides=[2, 2], padding=[0, 0])
+    sx, st = I4(2, 1, 12, 12), I4(8, 1, 2, 2)
+    assert l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), sx, st, C.byref(m), 2, 2,
+                                                                 C.byref(need)) == 0
+    f = l.simnets_hip_similarity_mex_sum_pool_prepare
+    assert f(C.byref(sa), sx, st, 256, None, C.byref(m), 256, n_off, 2, 2, 256, need.value, None) == -1         # null weights
+    assert f(C.byref(sa), sx, st, 256, 256, C.byref(m), 256, n_off - 1, 2, 2, 256, need.value, None) == -15
+    g = l.simnets_hip_similarity_mex_sum_pool_fwd_prepared
+    assert g(C.byref(sa), sx, st, None, C.byref(m), 2, 2, 256, need.value, 256, None) == -1
+    assert g(C.byref(sa), sx, st, 256, C.byref(m), 2, 2, 256, need.value - 1, 256, None) == -17
