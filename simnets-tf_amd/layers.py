@@ -151,6 +151,7 @@ class Similarity(torch.nn.Module):
         self.channels_last = channels_last
         self.templates = torch.nn.UninitializedParameter()
         self.sweights = torch.nn.UninitializedParameter()
+        self._prepared = None   # (key, ops.Prepared) of the last inference call
 
     @staticmethod
     def _init(param, how):
@@ -185,7 +186,16 @@ class Similarity(torch.nn.Module):
             self.to(x.device)
         if self.channels_last:
             x = x.permute(0, 3, 1, 2).contiguous()
-        out = similarity(x, self.templates, self.sweights.abs(), **self.attrs())
+        if not torch.is_grad_enabled() and x.is_cuda:
+            # inference: the parameters are packed once per (input shape, parameter version); calls run the forward
+            # kernels on the prepared buffer
+            key = (tuple(x.shape), x.device, self.templates._version, self.sweights._version)
+            if self._prepared is None or self._prepared[0] != key:
+                self._prepared = (key, ops.similarity_prepare(x.shape, self.templates.detach(),
+                                                              self.sweights.detach().abs(), **self.attrs()))
+            out = self._prepared[1](x)
+        else:
+            out = similarity(x, self.templates, self.sweights.abs(), **self.attrs())
         return out.permute(0, 2, 3, 1) if self.channels_last else out
 
     def compute_output_shape(self, input_shape):
@@ -226,6 +236,7 @@ class Mex(torch.nn.Module):
         self.offsets_initializer = offsets_initializer
         self.channels_last = channels_last
         self.offsets = torch.nn.UninitializedParameter()
+        self._prepared = None   # (key, ops.Prepared) of the last inference call
 
     def build(self, input_shape):
         shape = list(input_shape)
@@ -264,7 +275,15 @@ class Mex(torch.nn.Module):
             self.to(x.device)
         if self.channels_last:
             x = x.permute(0, 3, 1, 2).contiguous()
-        out = mex(x, self.offsets, self.num_instances, **self.attrs())
+        if not torch.is_grad_enabled() and x.is_cuda:
+            # inference: the offsets are packed once per (input shape, parameter version)
+            key = (tuple(x.shape), x.device, self.offsets._version)
+            if self._prepared is None or self._prepared[0] != key:
+                self._prepared = (key, ops.mex_prepare(x.shape, self.offsets.detach(), self.num_instances,
+                                                       **self.attrs()))
+            out = self._prepared[1](x)
+        else:
+            out = mex(x, self.offsets, self.num_instances, **self.attrs())
         return out.permute(0, 2, 3, 1) if self.channels_last else out
 
     def compute_output_shape(self, input_shape):

@@ -272,3 +272,27 @@ def test_gradient_calls_replay_from_a_hip_graph(pkg):
         torch.cuda.synchronize()
         for a, b, name in zip(got, want, ("dX", "dT", "dW", "mex dX", "mex dOff")):
             assert torch.equal(a, b), "replay %d: %s" % (trial, name)
+
+
+def test_modules_pack_parameters_once_for_inference(pkg):
+    """Under no_grad the Similarity / Mex modules run the prepared calls: same bits as the training-mode forward, one
+    buffer per (input shape, parameter version), a fresh one after the parameters change."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    sim = pkg.Similarity(12, blocks=[3, 3], strides=[1, 1], padding=[1, 1]).cuda()
+    mexl = pkg.Mex(7, blocks=[-1, 1, 1], strides=[12, 1, 1], softmax_mode=True, normalize_offsets=True,
+                   unshared_offset_region=[2]).cuda()
+    x = torch.randn((3, 5, 10, 10), device="cuda", generator=g)
+    y_train = mexl(sim(x))
+    with torch.no_grad():
+        y1 = mexl(sim(x))
+        first = (sim._prepared[1], mexl._prepared[1])
+        y2 = mexl(sim(x))
+        assert sim._prepared[1] is first[0] and mexl._prepared[1] is first[1]      # reused
+        assert torch.equal(y1, y_train.detach()) and torch.equal(y2, y1)
+        sim.templates.add_(0.25)
+        mexl.offsets.mul_(0.5)
+        y3 = mexl(sim(x))
+        assert sim._prepared[1] is not first[0] and mexl._prepared[1] is not first[1]
+    assert torch.equal(y3, mexl(sim(x)).detach()) and not torch.equal(y3, y1)
+    with torch.no_grad():
+        assert mexl(sim(x[:2])).shape[0] == 2                                      # another input shape: prepared anew
