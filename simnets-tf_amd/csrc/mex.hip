@@ -271,7 +271,6 @@ __global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
                     acc[t] *= fsh[t * 16 + lr];
             }
             const int kend = min((kc + 3) & ~3, (wk + 1) * KW);  // rows kc .. kend - 1 hold zeros
-#pragma unroll 2
             for (int kq = wk * KW; kq < kend; kq += 4) {
                 const float av = oa[kq * TM];
                 float bv[NT];
