@@ -24,6 +24,7 @@
 
 #include <cmath>
 
+#include "fast_div.h"
 #include "internal.h"
 #include "stage.h"
 #include "valu_tile.h"
@@ -36,6 +37,7 @@ namespace {
 constexpr int kWaves = 4;                 // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr int kLdsBudgetFloats = 16384;   // 64 KiB of input tile per workgroup
+constexpr int kSmWaves = 4, kSmThreads = 64 * kSmWaves;   // the small-map kernel's workgroup (eight waves measured slower)
 constexpr int kStagePos = 6;              // tile elements per thread and channel (a channel's tile holds at most
                                           // kStagePos * kThreads floats; larger geometries use the gather kernel)
 constexpr int kStageChan = 6;             // channels whose loads are in flight at once while staging
@@ -62,6 +64,8 @@ struct SimKernelArgs {
     int norm_every_iteration;
     int vec_store;     // output rows are 16-byte aligned: store float4
     int fast_stage;    // the channel tile has at most kStagePos * kThreads elements: division-free staging
+    int NI, img_lds;   // small-map kernel: images per workgroup and LDS floats of one image's tile (one channel)
+    FastDiv d_chan, d_img, d_tc;   // ... divisions of its staging loop: by NI * img_lds, img_lds, TC
     int plds_off;      // PLDS variants: where the workgroup's parameter copy starts in LDS (floats, multiple of 4)
     // sqrt-weight form only (see the guard in sim_direct_kernel)
     const float *pa2;  // [mtile][K][MT][2]  (template, negative weight): what the recomputing pass reads
@@ -413,6 +417,182 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     }
 }
 
+// Small maps (an image has fewer pixel groups than a wave has lanes, or the grid of the tiled kernel would leave
+// most SIMDs idle - hundreds of templates over 7 x 7 or 14 x 14 images at small batch): a wave covers NI images
+// (lane -> (image, pixel group)), a workgroup one tile of MT templates, and its four waves split K: each walks a
+// quarter of every staged channel chunk, the partial sums are added through LDS in wave order at the end (so the
+// summation order over k is by quarters of a chunk, not strictly ascending).  Same LDS staging rule (out-of-image ->
+// out_of_bounds_value), same packed parameters and offset table, same combine step as the tiled kernel.
+template <int MODE>
+__global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKernelArgs a)
+{
+    constexpr int PT = kSmallPT, MT = kSmallMT;
+    constexpr int NP = 4;   // tile elements per thread and channel the fast staging covers (NP * 256 per channel)
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int img_l = lane / a.gpi, g_l = lane - img_l * a.gpi;
+    const int b0 = blockIdx.x * a.NI;
+    const bool lane_valid = img_l < a.NI && b0 + img_l < a.B;
+    const int img = lane_valid ? img_l : 0, g = lane_valid ? g_l : 0;
+    const int b = b0 + img;
+    const int h = g / a.G, gw = g - h * a.G;
+    const int lds_base = img * a.img_lds + h * a.sh * a.TC + gw * PT * a.sw;
+    const int mtile = blockIdx.y;
+    const int taps = a.bh * a.bw;
+    const int chan_lds = a.NI * a.img_lds;
+    const size_t plane = (size_t)a.H * a.W;
+
+    float acc[MT][PT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            acc[m][p] = 0.0f;
+    const float *pa_t = a.pa + (size_t)mtile * a.K * MT * 2;
+    const float *pc_t = a.pc + (size_t)mtile * a.K * MT;
+    const int SIMNETS_CONST_AS *koff = (const int SIMNETS_CONST_AS *)(a.koff);
+
+    // where this thread's tile elements of a channel come from: every channel of a chunk has the same geometry
+    const bool fast = chan_lds <= NP * kSmThreads;
+    long long gofs[NP];   // offset from the image block's channel plane; -1: outside the image, -2: no such element
+#pragma unroll
+    for (int j = 0; j < NP; ++j) {
+        const int pos = tid + j * kSmThreads;
+        const int pc = min(pos, chan_lds - 1);
+        const int im = (int)fast_div((unsigned)pc, a.d_img), r2 = pc - im * a.img_lds;
+        const int r = (int)fast_div((unsigned)r2, a.d_tc), c = r2 - r * a.TC;
+        const int ih = r - a.ph, iw = c - a.pw, bb = b0 + im;
+        gofs[j] = -1;
+        if (bb < a.B && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
+            gofs[j] = (long long)bb * a.C * (long long)plane + (long long)ih * a.W + iw;
+        if (pos >= chan_lds)
+            gofs[j] = -2;
+    }
+
+    for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
+        const int ccn = min(a.CC, a.C - ch0);
+        __syncthreads();
+        // ---- the chunk's tile ----
+        if (fast) {
+            for (int cc0 = 0; cc0 < ccn; cc0 += 4) {
+                float v[4][NP];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float *chan = a.in + (size_t)(ch0 + min(cc0 + i, ccn - 1)) * plane;
+#pragma unroll
+                    for (int j = 0; j < NP; ++j)
+                        v[i][j] = gofs[j] >= 0 ? chan[gofs[j]] : a.oob;
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+#pragma unroll
+                    for (int j = 0; j < NP; ++j)
+                        if (cc0 + i < ccn && gofs[j] != -2)
+                            lds[(cc0 + i) * chan_lds + tid + j * kSmThreads] = v[i][j];
+            }
+        } else {
+            const int total = ccn * chan_lds;
+            for (int idx = tid; idx < total; idx += kSmThreads) {
+                const int cc = (int)fast_div((unsigned)idx, a.d_chan), r1 = idx - cc * chan_lds;
+                const int im = (int)fast_div((unsigned)r1, a.d_img), r2 = r1 - im * a.img_lds;
+                const int r = (int)fast_div((unsigned)r2, a.d_tc), c = r2 - r * a.TC;
+                const int ih = r - a.ph, iw = c - a.pw, bb = b0 + im;
+                float v = a.oob;
+                if (bb < a.B && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
+                    v = a.in[((size_t)bb * a.C + ch0 + cc) * plane + (size_t)ih * a.W + iw];
+                lds[idx] = v;   // == cc * chan_lds + im * img_lds + r * TC + c
+            }
+        }
+        __syncthreads();
+        const int cpw = (ccn + kSmWaves - 1) / kSmWaves;
+        const int c_lo = min(wave * cpw, ccn), c_hi = min(c_lo + cpw, ccn);
+        const int kl0 = c_lo * taps, nk = (c_hi - c_lo) * taps;   // this wave's steps, counted inside the chunk
+        // Software pipeline: the pixel values (LDS) and the parameters of step j + 1 are requested before the
+        // arithmetic of step j, two register sets.  The parameters come through scalar loads (one s_load_dwordx16
+        // per step) and are moved to VGPRs once per step by the combine (sim_step without VP): on this narrow tile a
+        // step has only 64-96 VALU instructions, and four lane-uniform vector or LDS loads per step - 16 / 8 cycles of
+        // the compute unit's one texture / LDS pipe each, shared by its four SIMDs - would bound the loop.
+        if (nk > 0) {
+            const int kg0 = ch0 * taps + kl0;   // this wave's first step, counted over all K
+            const int SIMNETS_CONST_AS *kt = koff + kg0;
+            const float SIMNETS_CONST_AS *pw = (const float SIMNETS_CONST_AS *)(pa_t) + (size_t)kg0 * (2 * MT);
+            const float SIMNETS_CONST_AS *pq = (const float SIMNETS_CONST_AS *)(pc_t) + (size_t)kg0 * MT;
+            float x0[PT], x1[PT], pa0[2 * MT], pa1[2 * MT], pc0[MT], pc1[MT];
+            {
+                const int off0 = kt[0];
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    x0[p] = lds[lds_base + off0 + p * a.sw];
+            }
+            load_params<MODE, MT>(pa0, pc0, pw, pq);
+            int off_next = kt[1];   // (the table has two entries of slack, the packed arrays one step)
+            auto step = [&](int j, const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT],
+                            float (&xn)[PT], float (&pan)[2 * MT], float (&pcn)[MT]) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): issued a whole step ago
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    xn[p] = lds[lds_base + off_next + p * a.sw];
+                off_next = kt[j + 2];
+                load_params<MODE, MT>(pan, pcn, pw + (size_t)(j + 1) * (2 * MT), pq + (size_t)(j + 1) * MT);
+                __builtin_amdgcn_sched_barrier(0);
+                sim_step<MODE, PT, MT, false>(acc, xc, pac, pcc);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            int j = 0;
+            for (; j + 2 <= nk; j += 2) {
+                step(j, x0, pa0, pc0, x1, pa1, pc1);
+                step(j + 1, x1, pa1, pc1, x0, pa0, pc0);
+            }
+            if (j < nk)
+                step(j, x0, pa0, pc0, x1, pa1, pc1);
+        }
+    }
+    // ---- partial sums of waves 1..3 -> wave 0, in wave order; the tile's LDS is reused ----
+    constexpr int kPart = MT * PT * 64;
+    __syncthreads();
+    if (wave > 0) {
+        float *dst = lds + (size_t)(wave - 1) * kPart + lane;
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                dst[(m * PT + p) * 64] = acc[m][p];
+    }
+    __syncthreads();
+    if (wave > 0 || !lane_valid)
+        return;
+    for (int w = 1; w < kSmWaves; ++w) {
+        const float *src = lds + (size_t)(w - 1) * kPart + lane;
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                acc[m][p] += src[(m * PT + p) * 64];
+    }
+    int reps = 0;
+    if (MODE == SIM_MODE_L2_NORM)
+        reps = a.norm_every_iteration ? (a.B - b) : 1;
+    const int w0 = gw * PT;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int mm = mtile * MT + m;
+        if (mm >= a.O)
+            break;
+        float *o = a.out + (((size_t)b * a.O + mm) * a.oh + h) * a.ow + w0;
+#pragma unroll
+        for (int p = 0; p < PT; ++p) {
+            float v = acc[m][p];
+            for (int r = 0; r < reps; ++r)
+                v += a.norm_const;
+            if (w0 + p < a.ow)
+                o[p] = v;
+        }
+    }
+}
+
 // Fallback for geometries whose input rows do not fit the LDS budget: one output pixel per
 // lane, patch elements gathered straight from global memory with bounds checks.
 template <int MODE, int MT>
@@ -537,6 +717,8 @@ __global__ __launch_bounds__(256) void sim_pack_params_kernel(const float *__res
 
 struct Tiling {
     int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
+    int NI;            // > 0: the small-map kernel with NI images per workgroup (CC, chan_pitch are then that kernel's)
+    int chan_pitch;    // LDS floats of one staged channel
     bool lds_ok;       // the rows of a workgroup's pixel groups fit the LDS tile (else: gather kernel)
     bool fast_stage;   // ... and the division-free staging (at most kStagePos elements per thread and channel)
 };
@@ -563,8 +745,12 @@ Tiling try_tiling(const SimPlan &p, int PT, int MT, int nws)
         const int chunks = (p.C + cc_max - 1) / cc_max;
         t.CC = (p.C + chunks - 1) / chunks;
     }
+    t.NI = 0;
+    t.chan_pitch = t.TRmax * t.TC;
     return t;
 }
+
+constexpr int kSmallMapLdsFloats = 8192;   // 32 KiB of tile per workgroup of the small-map kernel
 
 // Lane tile and workgroup shape for a problem.
 Tiling choose_tiling(const SimPlan &p)
@@ -599,7 +785,24 @@ Tiling choose_tiling(const SimPlan &p)
         if (big.lds_ok && waves(big) >= 1536)
             return big;
     }
-    return pick(kSmallPT, kSmallMT);
+    Tiling t = pick(kSmallPT, kSmallMT);
+    // Small maps: a whole image is one tile of at most 64 pixel groups, and either several images fit a wave or the
+    // tiled grid has at most one wave per SIMD while K is long enough to split over the four waves.
+    if (t.lds_ok && t.nws == 1 && t.tiles == 1 && p.C >= kSmWaves) {
+        const int NI = (int)std::max(1, std::min(p.B, 64 / t.gpi));
+        const long long per_chan = 1LL * NI * t.TRmax * t.TC;
+        if ((NI >= 2 || waves(t) <= 1024) && per_chan <= kSmallMapLdsFloats) {
+            t.NI = NI;
+            t.chan_pitch = (int)per_chan;
+            const int cc_max = (int)std::min<long long>(p.C, kSmallMapLdsFloats / per_chan);
+            const int chunks = (p.C + cc_max - 1) / cc_max;
+            t.CC = (p.C + chunks - 1) / chunks;
+            // the waves of the workgroup split a chunk's channels: a multiple of their number keeps them even
+            if (t.CC >= kSmWaves && t.CC % kSmWaves)
+                t.CC = t.CC / kSmWaves * kSmWaves;
+        }
+    }
+    return t;
 }
 
 template <int MODE, int PT, int MT, bool GATED, bool PLDS>
@@ -628,7 +831,7 @@ size_t plds_floats(const SimPlan &p, const Tiling &t) { return (size_t)(kWaves /
 // Short K on the small lane tile: the parameters go through LDS (one memory latency instead of one per k).
 bool use_plds(const SimPlan &p, const Tiling &t)
 {
-    return t.lds_ok && t.PT == kSmallPT && t.MT == kSmallMT && plds_floats(p, t) * sizeof(float) <= 16384;
+    return t.lds_ok && t.NI == 0 && t.PT == kSmallPT && t.MT == kSmallMT && plds_floats(p, t) * sizeof(float) <= 16384;
 }
 
 template <int MODE, bool GATED = false>
@@ -645,6 +848,12 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
             hipLaunchKernelGGL((sim_gather_kernel<MODE, 8>), grid, dim3(256), 0, s, a);
         return hipGetLastError();
     }
+    if (t.NI > 0) {
+        dim3 grid((unsigned)((a.B + t.NI - 1) / t.NI), (unsigned)a.n_mtiles);
+        const size_t floats = std::max<size_t>((size_t)t.CC * t.chan_pitch, (size_t)(kSmWaves - 1) * kSmallMT * kSmallPT * 64);
+        hipLaunchKernelGGL((sim_small_map_kernel<MODE>), grid, dim3(kSmThreads), floats * sizeof(float), s, a);
+        return hipGetLastError();
+    }
     const int nwm = kWaves / a.nws;
     dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
     size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
@@ -658,7 +867,7 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
 }
 
 // the sqrt-weight form runs on the tiled kernel only
-bool use_sqrtw(const SimPlan &p, const Tiling &t) { return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok; }
+bool use_sqrtw(const SimPlan &p, const Tiling &t) { return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && t.NI == 0; }
 
 long long guard_flags(const SimPlan &p, const Tiling &t)
 {
@@ -716,7 +925,7 @@ int sim_direct_prepare(const SimPlan &p, const float *templates, const float *we
     hipLaunchKernelGGL(sim_pack_params_kernel, dim3(pack_blocks + thr_blocks), dim3(256), 0, s, templates, weights, p.O,
                        p.K, t.MT, n_mtiles, mode, p.fudge, reinterpret_cast<float *>(ws + l.pa),
                        reinterpret_cast<float *>(ws + l.pc), reinterpret_cast<int *>(ws + l.koff), p.bh * p.bw, p.bw, t.CC,
-                       t.TRmax * t.TC, t.TC, sqrtw ? reinterpret_cast<float *>(ws + l.pa2) : nullptr,
+                       t.chan_pitch, t.TC, sqrtw ? reinterpret_cast<float *>(ws + l.pa2) : nullptr,
                        reinterpret_cast<float *>(ws + l.thr), pack_blocks);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
@@ -744,7 +953,10 @@ int sim_direct_run(const SimPlan &p, const float *input, float *output, void *wo
     a.nws_log2 = t.nws == 4 ? 2 : (t.nws == 2 ? 1 : 0);
     a.vec_store = (p.ow % 4 == 0) && ((reinterpret_cast<uintptr_t>(output) & 15) == 0);
     a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC; a.fast_stage = t.fast_stage;
-    a.plds_off = (int)align_up((size_t)t.CC * t.TRmax * t.TC, 4);
+    a.plds_off = (int)align_up((size_t)t.CC * t.chan_pitch, 4);
+    a.NI = t.NI; a.img_lds = t.TRmax * t.TC;
+    a.d_chan = make_fast_div((unsigned)std::max(1, t.chan_pitch)); a.d_img = make_fast_div((unsigned)std::max(1, a.img_lds));
+    a.d_tc = make_fast_div((unsigned)std::max(1, t.TC));
     a.oob = p.oob;
     // Dtype(-0.5) * Dtype(K_) * std::log(2.0 * M_PI), rounded to float by Eigen's constant()
     a.norm_const = (p.mode == SIM_MODE_L2_NORM) ? (float)((double)(-0.5f * (float)p.K) * std::log(2.0 * M_PI)) : 0.0f;

@@ -212,7 +212,7 @@ def test_unfused_pairs_prepared(pkg):
 
 # ---- sqrt-weight form over several channel chunks -----------------------------------------------------------------
 CHUNKED = dict(shape=(2, 40, 34, 34), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1])   # 4x8 tile, 3 chunks
-CHUNKED_SMALL = dict(shape=(2, 70, 12, 12), O=12, blocks=[3, 3], strides=[1, 1], padding=[1, 1])  # 4x8 tile
+CHUNKED_SMALL = dict(shape=(2, 70, 20, 20), O=12, blocks=[3, 3], strides=[1, 1], padding=[1, 1])  # 4x8 tile, 2 tiles per image
 
 
 @pytest.mark.parametrize("geom", [CHUNKED, CHUNKED_SMALL])
@@ -312,3 +312,35 @@ def test_similarity_wide_tile_sqrt_weight_guard(pkg, kind):
         assert np.array_equal(got, exact_form)
     if kind == "negative_weights":
         assert np.array_equal(got[:, 3::16], exact_form[:, 3::16], equal_nan=True)
+
+
+# ---- small maps: several images per wave, K split over the waves of a workgroup ---------------------------------------
+SMALL_MAPS = [
+    dict(shape=(9, 24, 7, 7), O=20, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),        # 4 images per wave, ragged batch
+    dict(shape=(5, 10, 5, 6), O=9, blocks=[2, 3], strides=[1, 1], padding=[0, 1], out_of_bounds_value=0.5),
+    dict(shape=(3, 37, 14, 14), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),      # one image per wave, K split only
+    dict(shape=(2, 16, 13, 9), O=8, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),        # stride 2
+    dict(shape=(70, 6, 3, 3), O=5, blocks=[3, 3], strides=[1, 1], padding=[0, 0]),         # 1 x 1 outputs: 64 images per wave
+]
+
+
+@pytest.mark.parametrize("mode", [dict(similarity_function="L1"), dict(similarity_function="L2"),
+                                  dict(similarity_function="L2", normalization_term=True),
+                                  dict(similarity_function="L2", normalization_term=True, ignore_nan_input=True)])
+@pytest.mark.parametrize("geom", SMALL_MAPS)
+def test_similarity_small_maps(pkg, geom, mode):
+    g = np.random.default_rng(61)
+    shape, O = geom["shape"], geom["O"]
+    kw = dict({k: v for k, v in geom.items() if k not in ("shape", "O")}, **mode)
+    x = g.normal(size=shape).astype(np.float32)
+    if mode.get("ignore_nan_input"):
+        x[g.random(size=shape) < 0.1] = np.nan
+        kw["out_of_bounds_value"] = float("nan")
+    t = g.normal(size=(O, shape[1]) + tuple(geom["blocks"])).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    X, T, W = dev(x), dev(t), dev(w)
+    got = pkg.similarity(X, T, W, **kw)
+    assert rel_err(got.cpu().numpy(), orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+    assert same_bits(pkg.similarity_prepare(shape, T, W, **kw)(X), got)
+    if not mode.get("normalization_term"):
+        assert rel_err(pkg.similarity(X, T, W, algo="direct", **kw).cpu().numpy(), got.cpu().numpy()) <= SIM_TOL
