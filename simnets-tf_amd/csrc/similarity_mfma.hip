@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <vector>
 
 #include "internal.h"
 #include "stage.h"
@@ -45,6 +46,20 @@ constexpr int kLdsBudgetFloats = 12288;  // 48 KiB input tile per workgroup
 constexpr int kStagePos = 8;             // tile elements per thread and channel (at most kStagePos * 256 floats)
 constexpr int kStageChan = 4;            // channels whose loads are in flight at once while staging
 
+// Geometry of one launch grid: the forward op's, or one stride phase of the input gradient.
+struct MfmaGeom {
+    int ow, npix;            // output grid width and size
+    int bh, bw, sh, sw, ph, pw;
+    int tiles;               // workgroup pixel tiles per image
+    int TC, chan_lds, CC;
+    int oy0, ox0;            // input gradient: first input row / column of the phase
+    long long pm_off;        // this grid's packed operands inside pm, floats
+};
+
+constexpr int kMaxPhases = 16;
+constexpr int kMaxTaps = 64;    // window size limit of the kernel that interleaves the stride phases
+constexpr int kPmAhead = 8;     // ... and the steps per block of parameter operands it requests ahead
+
 struct MfmaArgs {
     const float *in;
     float *out;
@@ -54,14 +69,21 @@ struct MfmaArgs {
     const float *x;     // input-gradient variant: the forward op's input (one value per output element)
     int x_channels;     // ... and its channel count (rows of the product that exist)
     int ignore_nan;     // ... NaN inputs get gradient 0
-    int B, C, H, W, O, Opad, oh, ow, npix;
-    int bh, bw, sh, sw, ph, pw;
-    int tiles;          // workgroup pixel tiles per image
-    int TC, TRmax, chan_lds, CC;
+    // ... where pixel (r, c) of a phase's grid sits in the forward op's input plane: row oy0 + r * oys,
+    // column ox0 + c * oxs of a plane x_w wide and x_plane large (the whole plane at stride 1)
+    int oys, oxs, x_w, x_plane;
+    int B, C, H, W, O, Opad;
+    int grid_tiles;     // pixel tiles per image in blockIdx.x (the largest phase's count)
     float oob;
+    MfmaGeom g;         // the forward op's grid
 };
 
-// GRAD: the same contraction machinery computes the input gradient of the L2 modes at stride 1.  With
+// The stride phases of one input-gradient launch, one per blockIdx.z.
+struct MfmaPhases {
+    MfmaGeom g[kMaxPhases];
+};
+
+// GRAD: the same contraction machinery computes the input gradient of the L2 modes.  At stride 1, with
 // P0 = s w (t - c), P1 = s w (s = 2, or 1 with the normalization term; c = the channel's centre),
 //   dX[b,ch,y,x] = sum_{m,dh,dw} g[b,m,y+ph-dh,x+pw-dw] (P0 - (X - c) P1)[m,ch,dh,dw] = A - (X[b,ch,y,x] - c) B,
 // two products over (m, dh, dw) whose right operand is the output gradient read like an input image padded by
@@ -69,9 +91,14 @@ struct MfmaArgs {
 // same sums term by term).  Here the "image" is g (its channels are the templates), the rows are input channels:
 // row tile 0 of a wave accumulates A and row tile 1 accumulates B for the same 32 channels, so a lane ends up
 // with both values of an element and combines them with X at the store.
+// At stride (sh, sw) the input pixels fall into sh * sw phases, (ry, rx) = ((y + ph) mod sh, (x + pw) mod sw).
+// Only the taps dh = ry + sh a, dw = rx + sw b reach a pixel of that phase, and with Y = (y + ph - ry) / sh the
+// window rows they come from are Y - a: each phase is a stride-1 problem of the same kind over its own taps,
+// on the grid of its pixels, and gets a launch of its own that stores to (and reads X at) the phase's pixels.
 template <bool GRAD>
-__global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
+__global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a, const MfmaPhases phases)
 {
+    const MfmaGeom &g = GRAD ? phases.g[blockIdx.z] : a.g;
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -79,14 +106,16 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
     const int wm = wave & 1, wp = wave >> 1;
     const int col = lane & 31, half = lane >> 5;
 
-    const int b = blockIdx.x / a.tiles;
-    const int tile = blockIdx.x - b * a.tiles;
+    const int b = blockIdx.x / a.grid_tiles;
+    const int tile = blockIdx.x - b * a.grid_tiles;
+    if (tile >= g.tiles)
+        return;  // a phase with fewer pixel tiles than the largest one
     const int p_first = tile * WG_PIX;
-    const int p_last = min(p_first + WG_PIX, a.npix) - 1;
-    const int h_first = p_first / a.ow;
-    const int nrows = p_last / a.ow - h_first + 1;
-    const int TR = (nrows - 1) * a.sh + a.bh;
-    const int in_row0 = h_first * a.sh - a.ph;
+    const int p_last = min(p_first + WG_PIX, g.npix) - 1;
+    const int h_first = p_first / g.ow;
+    const int nrows = p_last / g.ow - h_first + 1;
+    const int TR = (nrows - 1) * g.sh + g.bh;
+    const int in_row0 = h_first * g.sh - g.ph;
     const int mbase = GRAD ? blockIdx.y * (WG_TPL / 2) + wm * 32 : blockIdx.y * WG_TPL + wm * (RM * 32);
 
     // per pixel tile: LDS address of this lane's pixel (k-pair half folded in)
@@ -96,8 +125,8 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
         const int p = p_first + (wp * RP + j) * 32 + col;
         pix[j] = p;
         const int pc = min(p, p_last);
-        const int h = pc / a.ow, w = pc - h * a.ow;
-        xbase[j] = (h - h_first) * a.sh * a.TC + w * a.sw + half * a.chan_lds;
+        const int h = pc / g.ow, w = pc - h * g.ow;
+        xbase[j] = (h - h_first) * g.sh * g.TC + w * g.sw + half * g.chan_lds;
     }
 
     floatx16 acc[RM][RP];
@@ -114,7 +143,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
 
     // parameter operand: this lane's element within a [type][half][Opad] step record
     const int step_stride = 4 * a.Opad;
-    const float *pm = a.pm + half * a.Opad + mbase + col;
+    const float *pm = a.pm + g.pm_off + half * a.Opad + mbase + col;
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
 
     float pw_cur[RM], pt_cur[RM], pw_nxt[RM], pt_nxt[RM];
@@ -132,19 +161,19 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
     pm += 2 * step_stride;
 
     TilePositions<kStagePos> tp;
-    tp.template init<kThreads>(a.H, a.W, TR, a.TC, in_row0, a.pw);
+    tp.template init<kThreads>(a.H, a.W, TR, g.TC, in_row0, g.pw);
 
-    for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
-        const int ccn = min(a.CC, a.C - ch0);
+    for (int ch0 = 0; ch0 < a.C; ch0 += g.CC) {
+        const int ccn = min(g.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
-        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, a.chan_lds, a.oob,
+        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, g.chan_lds, a.oob,
                                                      GRAD ? nullptr : a.ctr, tp);
         __syncthreads();
 
         // steps of this chunk in (channel pair, dh, dw) order; the pixel operand of step s+1 and the
         // parameter operand of step s+2 are requested before the MFMAs of step s are issued
-        const int nsteps = (ccp / 2) * a.bh * a.bw;
+        const int nsteps = (ccp / 2) * g.bh * g.bw;
         int dh = 0, dw = 0, row_off = 0, off = 0;
         float xn[RP];
 #pragma unroll
@@ -156,13 +185,13 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
             for (int j = 0; j < RP; ++j)
                 x[j] = xn[j];
             int ndw = dw + 1, ndh = dh, nrow = row_off;
-            if (ndw == a.bw) {
+            if (ndw == g.bw) {
                 ndw = 0;
                 ++ndh;
-                nrow += a.TC;
-                if (ndh == a.bh) {
+                nrow += g.TC;
+                if (ndh == g.bh) {
                     ndh = 0;
-                    nrow += 2 * a.chan_lds - a.bh * a.TC;
+                    nrow += 2 * g.chan_lds - g.bh * g.TC;
                 }
             }
             int noff = nrow + ndw;
@@ -208,25 +237,28 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
         }
     }
 
-    const size_t plane = (size_t)a.npix;
+    const size_t plane = (size_t)g.npix;
     if constexpr (GRAD) {
         // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel ----
-        float *ob = a.out + (size_t)b * a.x_channels * plane;
-        const float *xb = a.x + (size_t)b * a.x_channels * plane;
+        const size_t xplane = (size_t)a.x_plane;
+        float *ob = a.out + (size_t)b * a.x_channels * xplane;
+        const float *xb = a.x + (size_t)b * a.x_channels * xplane;
 #pragma unroll
         for (int j = 0; j < RP; ++j) {
             if (pix[j] > p_last)
                 continue;
+            const int pr = pix[j] / g.ow, pc = pix[j] - pr * g.ow;
+            const size_t at = (size_t)(g.oy0 + pr * a.oys) * a.x_w + (g.ox0 + pc * a.oxs);
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int ch = mbase + 8 * (v / 4) + 4 * half + (v % 4);
                 if (ch >= a.x_channels)
                     continue;
-                const float xin = xb[(size_t)ch * plane + pix[j]];
+                const float xin = xb[(size_t)ch * xplane + at];
                 float d = __builtin_fmaf(-(xin - a.ctr[ch]), acc[1][j][v], acc[0][j][v]);
                 if (a.ignore_nan && xin != xin)
                     d = 0.0f;
-                ob[(size_t)ch * plane + pix[j]] = d;
+                ob[(size_t)ch * xplane + at] = d;
             }
         }
         return;
@@ -245,6 +277,203 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a)
                 if (m < a.O)
                     ob[(size_t)m * plane + pix[j]] = acc[i][j][v];
             }
+    }
+}
+
+// Input gradient at strides whose phases number two or four (1x2, 2x1, 2x2), all phases in one workgroup.
+// Input pixel (y, x) = (sh Yb + ry, sw Xb + rx): the residue (ry, rx) names the phase, (Yb, Xb) the position on a
+// grid common to all phases.  Tap (i, j) reaches the pixels of one phase only, those with (ry + ph - i) divisible by
+// sh, and comes from window row Yb + (ry + ph - i) / sh: a fixed offset from the position for every tap.  A wave's
+// four pixel tiles are its 32 positions in each of four phases (two phases: 2 x 32 positions each), so one staged
+// tile of the output gradient serves every phase, and a step - one tap of one template pair - feeds the pixel
+// tiles of the tap's phase.  q.tap[t] = (phase << 24) | LDS offset of tap t relative to the position.
+struct MfmaStrideArgs {
+    int nXb, npos, tiles;   // position grid: width, size, workgroup tiles per image
+    int T;                  // taps (bh * bw <= kMaxTaps)
+    int TC, chan_lds, CC;
+    int row_min, col_min;   // window row / column of tile element (0, 0), relative to the first position row / column 0
+    int row_ext;            // tile rows = position rows - 1 + row_ext
+    int tap[kMaxTaps];
+};
+
+template <int NPH>
+__global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(const MfmaArgs a, const MfmaStrideArgs q)
+{
+    constexpr int PB = RP / NPH;          // 32-position blocks per wave
+    constexpr int WG_POS = 2 * PB * 32;   // positions per workgroup (2 pixel waves)
+    extern __shared__ float lds[];
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 1, wp = wave >> 1;
+    const int col = lane & 31, half = lane >> 5;
+
+    const int b = blockIdx.x / q.tiles;
+    const int tile = blockIdx.x - b * q.tiles;
+    const int p_first = tile * WG_POS;
+    const int p_last = min(p_first + WG_POS, q.npos) - 1;
+    const int h_first = p_first / q.nXb;
+    const int nrows = p_last / q.nXb - h_first + 1;
+    const int TR = nrows - 1 + q.row_ext;
+    const int mbase = blockIdx.y * (WG_TPL / 2) + wm * 32;
+
+    int xbase[PB], pos_h[PB], pos_w[PB];
+#pragma unroll
+    for (int j = 0; j < PB; ++j) {
+        const int p = p_first + (wp * PB + j) * 32 + col;
+        const int pc = min(p, p_last);
+        const int h = pc / q.nXb, w = pc - h * q.nXb;
+        pos_h[j] = p <= p_last ? h : -1;
+        pos_w[j] = w;
+        xbase[j] = (h - h_first) * q.TC + w + half * q.chan_lds;
+    }
+
+    floatx16 acc[2][RP];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < RP; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v)
+                acc[i][j][v] = 0.0f;
+
+    // parameter operand: [step][type][half][Cpad] in the order of use (chunk, tap, template pair)
+    const int step_stride = 4 * a.Opad;
+    const float *pm = a.pm + half * a.Opad + mbase + col;
+    const float *img = a.in + (size_t)b * a.C * a.H * a.W;
+    float pa[kPmAhead], pb[kPmAhead];
+#pragma unroll
+    for (int i = 0; i < kPmAhead; ++i) {
+        pa[i] = pm[i * step_stride];
+        pb[i] = pm[i * step_stride + 2 * a.Opad];
+    }
+
+    // Staging: the tile of a channel is small here (a few rows of the position grid), so a thread's kStagePos
+    // elements span a group of G channels and every thread has that many loads in flight.
+    const int per_chan = TR * q.TC;
+    const int G = max(1, min(kStagePos * kThreads / per_chan, q.CC));
+    const int plane_g = a.H * a.W;
+    int gofs[kStagePos], lofs[kStagePos], gchan[kStagePos];
+#pragma unroll
+    for (int j = 0; j < kStagePos; ++j) {
+        const int e = tid + j * kThreads;
+        const int cc = e / per_chan;
+        const int pos = e - cc * per_chan;
+        const int r = pos / q.TC, c = pos - r * q.TC;
+        const int ih = h_first + q.row_min + r, iw = c + q.col_min;
+        gchan[j] = cc < G ? cc : (1 << 20);   // beyond the group: never staged
+        lofs[j] = cc * q.chan_lds + pos;
+        gofs[j] = (ih >= 0 && ih < a.H && iw >= 0 && iw < a.W) ? cc * plane_g + ih * a.W + iw : -1;
+    }
+
+    for (int ch0 = 0; ch0 < a.C; ch0 += q.CC) {
+        const int ccn = min(q.CC, a.C - ch0);
+        const int ccp = (ccn + 1) & ~1;
+        __syncthreads();
+        for (int c0 = 0; c0 < ccp; c0 += G) {
+            const float *src = img + (size_t)(ch0 + c0) * plane_g;
+            float v[kStagePos];
+#pragma unroll
+            for (int j = 0; j < kStagePos; ++j) {
+                v[j] = 0.0f;
+                if (c0 + gchan[j] < ccn && gofs[j] >= 0)
+                    v[j] = src[gofs[j]];
+            }
+#pragma unroll
+            for (int j = 0; j < kStagePos; ++j)
+                if (c0 + gchan[j] < ccp)
+                    lds[c0 * q.chan_lds + lofs[j]] = v[j];
+        }
+        __syncthreads();
+
+        // taps outside, template pairs inside: the inner loop has one phase and walks the channel slots of the tile
+        const int np = ccp / 2;
+        int e_next = q.tap[0];
+        float xn[PB];
+#pragma unroll
+        for (int j = 0; j < PB; ++j)
+            xn[j] = lds[xbase[j] + (e_next & 0xffffff)];
+        for (int t = 0; t < q.T; ++t) {
+            const int e_cur = e_next;
+            e_next = q.tap[t + 1 < q.T ? t + 1 : t];
+            const int off = e_cur & 0xffffff, off_next = e_next & 0xffffff;
+            const int phase = e_cur >> 24;
+#pragma unroll
+            for (int f = 0; f < NPH; ++f) {
+                if (phase != f)
+                    continue;
+                int lo = off;
+                // blocks of kPmAhead steps: the parameters of the next block (which may belong to the next tap or
+                // chunk: the stream is continuous) are requested before the first step of this one
+                for (int mp0 = 0; mp0 < np; mp0 += kPmAhead) {
+                    const int n = min(kPmAhead, np - mp0);
+                    const float *pmn = pm + n * step_stride;
+                    float qa[kPmAhead], qb[kPmAhead];
+#pragma unroll
+                    for (int u = 0; u < kPmAhead; ++u) {
+                        qa[u] = pmn[u * step_stride];
+                        qb[u] = pmn[u * step_stride + 2 * a.Opad];
+                    }
+#pragma unroll
+                    for (int u = 0; u < kPmAhead; ++u) {
+                        if (u >= n)
+                            break;
+                        float x[PB];
+#pragma unroll
+                        for (int j = 0; j < PB; ++j)
+                            x[j] = xn[j];
+                        lo += 2 * q.chan_lds;
+                        const int noff = mp0 + u + 1 < np ? lo : off_next;
+#pragma unroll
+                        for (int j = 0; j < PB; ++j)
+                            xn[j] = lds[xbase[j] + noff];
+                        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                        for (int j = 0; j < PB; ++j)
+                            acc[0][f * PB + j] =
+                                __builtin_amdgcn_mfma_f32_32x32x2f32(pa[u], x[j], acc[0][f * PB + j], 0, 0, 0);
+#pragma unroll
+                        for (int j = 0; j < PB; ++j)
+                            acc[1][f * PB + j] =
+                                __builtin_amdgcn_mfma_f32_32x32x2f32(pb[u], x[j], acc[1][f * PB + j], 0, 0, 0);
+                    }
+                    pm = pmn;
+#pragma unroll
+                    for (int u = 0; u < kPmAhead; ++u) {
+                        pa[u] = qa[u];
+                        pb[u] = qb[u];
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel per phase ----
+    const size_t xplane = (size_t)a.x_plane;
+    const int x_h = a.x_plane / a.x_w;
+    float *ob = a.out + (size_t)b * a.x_channels * xplane;
+    const float *xb = a.x + (size_t)b * a.x_channels * xplane;
+#pragma unroll
+    for (int f = 0; f < NPH; ++f) {
+        const int ry = f / a.oxs, rx = f - ry * a.oxs;
+#pragma unroll
+        for (int j = 0; j < PB; ++j) {
+            const int y = pos_h[j] * a.oys + ry, xx = pos_w[j] * a.oxs + rx;
+            if (pos_h[j] < 0 || y >= x_h || xx >= a.x_w)
+                continue;
+            const size_t at = (size_t)y * a.x_w + xx;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int ch = mbase + 8 * (v / 4) + 4 * half + (v % 4);
+                if (ch >= a.x_channels)
+                    continue;
+                const float xin = xb[(size_t)ch * xplane + at];
+                float d = __builtin_fmaf(-(xin - a.ctr[ch]), acc[1][f * PB + j][v], acc[0][f * PB + j][v]);
+                if (a.ignore_nan && xin != xin)
+                    d = 0.0f;
+                ob[(size_t)ch * xplane + at] = d;
+            }
+        }
     }
 }
 
@@ -324,11 +553,50 @@ __global__ __launch_bounds__(256) void mfma_bias_kernel(const float *__restrict_
         bias[m] = -red[0];
 }
 
-// Input-gradient variant: pm[step][type][half][Cpad], step = ((mpair * bh) + dh) * bw + dw over the flipped taps,
-// template m = 2 * mpair + half, row = input channel: type 0 = s w (t - ctr), type 1 = s w.
+// Input-gradient variant: pm[step][type][half][Cpad], step = ((mpair * na) + dh) * nb + dw over the flipped taps
+// of one stride phase (tap rows ry + sh a, a < na, columns rx + sw b, b < nb; all bh x bw taps at stride 1),
+// template m = 2 * mpair + half, row = input channel: type 0 = s w (t - ctr), type 1 = s w.  blockIdx.y = phase.
+struct MfmaGradPack {
+    struct Phase {
+        int ry, rx, na, nb;
+        long long pm_off, total;
+    } p[kMaxPhases];
+    long long max_floats;
+};
+
 __global__ void mfma_grad_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
-                                      const float *__restrict__ ctr, int O, int C, int Cpad, int bh, int bw,
-                                      float scale, long long total, float *__restrict__ pm)
+                                      const float *__restrict__ ctr, int O, int C, int Cpad, int bh, int bw, int sh,
+                                      int sw, float scale, const MfmaGradPack pk, float *__restrict__ pm)
+{
+    const MfmaGradPack::Phase &q = pk.p[blockIdx.y];
+    pm += q.pm_off;
+    for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < q.total;
+         i += (long long)gridDim.x * blockDim.x) {
+        const int c = (int)(i % Cpad);
+        long long r = i / Cpad;
+        const int half = (int)(r & 1); r >>= 1;
+        const int type = (int)(r & 1); r >>= 1;
+        const int dw = (int)(r % q.nb); r /= q.nb;
+        const int dh = (int)(r % q.na);
+        const int mpair = (int)(r / q.na);
+        const int m = 2 * mpair + half;
+        float v = 0.0f;
+        if (m < O && c < C) {
+            const size_t idx =
+                (((size_t)m * C + c) * bh + (q.ry + sh * (q.na - 1 - dh))) * bw + (q.rx + sw * (q.nb - 1 - dw));
+            const float w = scale * weights[idx];
+            v = type == 0 ? w * (templates[idx] - ctr[c]) : w;
+        }
+        pm[i] = v;
+    }
+}
+
+// Parameters of the kernel that interleaves the stride phases: pm[step][type][half][Cpad] with the steps in the
+// kernel's order: chunks of CC templates, inside a chunk the taps (i * bw + j, unflipped: the tap table holds where
+// each tap reads), inside a tap the chunk's template pairs.
+__global__ void mfma_grad_strided_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
+                                              const float *__restrict__ ctr, int O, int C, int Cpad, int T, int CC,
+                                              float scale, long long total, float *__restrict__ pm)
 {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < total;
          i += (long long)gridDim.x * blockDim.x) {
@@ -336,13 +604,20 @@ __global__ void mfma_grad_pack_kernel(const float *__restrict__ templates, const
         long long r = i / Cpad;
         const int half = (int)(r & 1); r >>= 1;
         const int type = (int)(r & 1); r >>= 1;
-        const int dw = (int)(r % bw); r /= bw;
-        const int dh = (int)(r % bh);
-        const int mpair = (int)(r / bh);
-        const int m = 2 * mpair + half;
+        // step r: chunk k covers the pairs [k CC/2, min((k+1) CC/2, pairs)), T * (pairs in the chunk) steps
+        const long long per_chunk = (long long)(CC / 2) * T;
+        const int chunk = (int)(r / per_chunk);
+        const int in_chunk = (int)(r - chunk * per_chunk);
+        const int np = min(CC / 2, (O + 1) / 2 - chunk * (CC / 2));
+        int m = O;
+        int tap = 0;
+        if (np > 0 && in_chunk < np * T) {
+            tap = in_chunk / np;
+            m = 2 * (chunk * (CC / 2) + in_chunk - tap * np) + half;
+        }
         float v = 0.0f;
         if (m < O && c < C) {
-            const size_t idx = (((size_t)m * C + c) * bh + (bh - 1 - dh)) * bw + (bw - 1 - dw);
+            const size_t idx = ((size_t)m * C + c) * T + tap;
             const float w = scale * weights[idx];
             v = type == 0 ? w * (templates[idx] - ctr[c]) : w;
         }
@@ -378,6 +653,16 @@ MfmaTiling mfma_tiling(const SimPlan &p)
     // two steps of slack: the parameter loads run two steps ahead
     t.pm_floats = (size_t)(t.steps + 2) * 4 * t.Opad;
     return t;
+}
+
+MfmaGeom mfma_geom(const SimPlan &p, const MfmaTiling &t)
+{
+    MfmaGeom g = {};
+    g.ow = p.ow; g.npix = p.oh * p.ow;
+    g.bh = p.bh; g.bw = p.bw; g.sh = p.sh; g.sw = p.sw; g.ph = p.ph; g.pw = p.pw;
+    g.tiles = (g.npix + WG_PIX - 1) / WG_PIX;
+    g.TC = t.TC; g.chan_lds = t.chan_lds; g.CC = t.CC;
+    return g;
 }
 
 }  // namespace
@@ -433,17 +718,15 @@ int sim_mfma_run(const SimPlan &p, const float *input, float *output, void *work
     if (workspace_bytes < sim_mfma_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     const MfmaLayout l = mfma_layout(t, workspace);
-    MfmaArgs a;
+    MfmaArgs a = {};
     a.in = input; a.out = output; a.pm = l.pm; a.bias = l.bias; a.ctr = l.ctr;
     a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.Opad = t.Opad;
-    a.oh = p.oh; a.ow = p.ow; a.npix = p.oh * p.ow;
-    a.bh = p.bh; a.bw = p.bw; a.sh = p.sh; a.sw = p.sw; a.ph = p.ph; a.pw = p.pw;
-    a.tiles = (a.npix + WG_PIX - 1) / WG_PIX;
-    a.TC = t.TC; a.TRmax = t.TRmax; a.chan_lds = t.chan_lds; a.CC = t.CC;
+    a.g = mfma_geom(p, t);
+    a.grid_tiles = a.g.tiles;
     a.oob = p.oob;
-    dim3 grid((unsigned)(p.B * a.tiles), (unsigned)(t.Opad / WG_TPL));
+    dim3 grid((unsigned)(p.B * a.g.tiles), (unsigned)(t.Opad / WG_TPL));
     const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
-    hipLaunchKernelGGL(sim_mfma_kernel<false>, grid, dim3(kThreads), lds_bytes, s, a);
+    hipLaunchKernelGGL(sim_mfma_kernel<false>, grid, dim3(kThreads), lds_bytes, s, a, MfmaPhases{});
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
@@ -467,32 +750,150 @@ MfmaTiling mfma_grad_tiling(const SimPlan &q)
     return t;
 }
 
-SimPlan grad_as_forward(const SimPlan &p)
+// One stride phase of the input gradient as a stride-1 forward problem: the output gradient is the image (its
+// channels are the templates), the phase's pixels are the output grid, the phase's taps the window.
+struct GradPhase {
+    SimPlan q;
+    int ry, rx, na, nb;   // tap rows ry + sh a (a < na), tap columns rx + sw b (b < nb)
+    int oy0, ox0;         // first input row / column of the phase
+    MfmaTiling t;
+};
+
+// Phases with pixels, in (ry, rx) order.  Returns false when a phase with pixels has no tap (stride larger than
+// the window: its gradient is zero and this path leaves it to the caller's other kernel).
+bool grad_phases(const SimPlan &p, std::vector<GradPhase> &out)
 {
-    SimPlan q = p;
-    q.C = p.O; q.H = p.oh; q.W = p.ow;
-    q.O = p.C; q.oh = p.H; q.ow = p.W;
-    q.ph = p.bh - 1 - p.ph; q.pw = p.bw - 1 - p.pw;
-    q.K = p.O * p.bh * p.bw;
-    return q;
+    out.clear();
+    for (int ry = 0; ry < p.sh; ++ry)
+        for (int rx = 0; rx < p.sw; ++rx) {
+            GradPhase g;
+            g.ry = ry; g.rx = rx;
+            g.na = ry < p.bh ? (p.bh - ry + p.sh - 1) / p.sh : 0;
+            g.nb = rx < p.bw ? (p.bw - rx + p.sw - 1) / p.sw : 0;
+            // pixels y = sh Y + ry - ph in [0, H): Y from Y0 = ceil((ph - ry) / sh) (>= 0 as ry < sh)
+            const int Y0 = p.ph > ry ? (p.ph - ry + p.sh - 1) / p.sh : 0;
+            const int X0 = p.pw > rx ? (p.pw - rx + p.sw - 1) / p.sw : 0;
+            g.oy0 = p.sh * Y0 + ry - p.ph;
+            g.ox0 = p.sw * X0 + rx - p.pw;
+            const int nY = g.oy0 < p.H ? (p.H - 1 - g.oy0) / p.sh + 1 : 0;
+            const int nX = g.ox0 < p.W ? (p.W - 1 - g.ox0) / p.sw + 1 : 0;
+            if (nY <= 0 || nX <= 0)
+                continue;
+            if (g.na == 0 || g.nb == 0)
+                return false;
+            SimPlan q = p;
+            q.C = p.O; q.H = p.oh; q.W = p.ow;
+            q.O = p.C; q.oh = nY; q.ow = nX;
+            q.bh = g.na; q.bw = g.nb; q.sh = 1; q.sw = 1;
+            // phase row r reads window rows Y0 + r - a = r - (na - 1 - Y0) + (na - 1 - a)
+            q.ph = g.na - 1 - Y0; q.pw = g.nb - 1 - X0;
+            q.K = p.O * g.na * g.nb;
+            g.q = q;
+            g.t = mfma_grad_tiling(q);
+            out.push_back(g);
+        }
+    return true;
+}
+
+// Tiling of the kernel that interleaves the stride phases (two or four of them, windows of at most kMaxTaps taps).
+struct StrideTiling {
+    bool ok;
+    int nph, Cpad;
+    size_t pm_floats, lds_bytes;
+    MfmaStrideArgs q;
+};
+
+// residue r of an input coordinate that tap i reaches, and the window coordinate it comes from relative to the
+// position: input = stride * position + r, (r + pad - i) divisible by stride, window = position + (r + pad - i) / stride
+void stride_tap(int i, int stride, int pad, int *r, int *d)
+{
+    *r = ((i - pad) % stride + stride) % stride;
+    *d = (*r + pad - i) / stride;   // exact division; negative for taps beyond the padding
+}
+
+StrideTiling stride_tiling(const SimPlan &p)
+{
+    StrideTiling t = {};
+    t.nph = p.sh * p.sw;
+    const int T = p.bh * p.bw;
+    if ((t.nph != 2 && t.nph != 4) || p.sh > p.bh || p.sw > p.bw || T > kMaxTaps)
+        return t;
+    const int PB = RP / t.nph, wg_pos = 2 * PB * 32;
+    const int nYb = (p.H + p.sh - 1) / p.sh, nXb = (p.W + p.sw - 1) / p.sw;
+    int rmin = 1 << 30, rmax = -(1 << 30), cmin = 1 << 30, cmax = -(1 << 30);
+    for (int i = 0; i < p.bh; ++i) {
+        int r, d;
+        stride_tap(i, p.sh, p.ph, &r, &d);
+        rmin = std::min(rmin, d); rmax = std::max(rmax, d);
+    }
+    for (int j = 0; j < p.bw; ++j) {
+        int r, d;
+        stride_tap(j, p.sw, p.pw, &r, &d);
+        cmin = std::min(cmin, d); cmax = std::max(cmax, d);
+    }
+    MfmaStrideArgs &q = t.q;
+    q.nXb = nXb; q.npos = nYb * nXb; q.tiles = (q.npos + wg_pos - 1) / wg_pos;
+    q.T = T;
+    q.row_min = rmin; q.col_min = cmin; q.row_ext = rmax - rmin + 1;
+    q.TC = nXb - 1 + (cmax - cmin + 1);
+    const int max_rows = std::min(nYb, (wg_pos + nXb - 1) / nXb + 1);
+    const int TRmax = max_rows - 1 + q.row_ext;
+    long long pitch = 1LL * TRmax * q.TC;
+    pitch = (pitch + 31) / 64 * 64 + 32;
+    if (pitch < 1LL * TRmax * q.TC)
+        pitch += 64;
+    if (2 * pitch > kLdsBudgetFloats || 1LL * TRmax * q.TC > kStagePos * kThreads)
+        return t;
+    q.chan_lds = (int)pitch;
+    int cc_max = (int)(kLdsBudgetFloats / pitch) & ~1;
+    cc_max = std::min(cc_max, (p.O + 1) & ~1);
+    const int chunks = (p.O + cc_max - 1) / cc_max;
+    q.CC = ((p.O + chunks - 1) / chunks + 1) & ~1;
+    for (int i = 0; i < p.bh; ++i)
+        for (int j = 0; j < p.bw; ++j) {
+            int ry, dy, rx, dx;
+            stride_tap(i, p.sh, p.ph, &ry, &dy);
+            stride_tap(j, p.sw, p.pw, &rx, &dx);
+            q.tap[i * p.bw + j] = ((ry * p.sw + rx) << 24) | ((dy - rmin) * q.TC + (dx - cmin));
+        }
+    t.Cpad = (p.C + WG_TPL / 2 - 1) / (WG_TPL / 2) * (WG_TPL / 2);
+    t.pm_floats = ((size_t)((p.O + 1) / 2) * T + kPmAhead) * 4 * t.Cpad;
+    t.lds_bytes = (size_t)q.CC * q.chan_lds * sizeof(float);
+    t.ok = true;
+    return t;
 }
 
 }  // namespace
 
 bool sim_mfma_grad_input_supported(const SimPlan &p)
 {
-    if (p.mode == SIM_MODE_L1 || p.exact_terms || p.sh != 1 || p.sw != 1 || p.ph > p.bh - 1 || p.pw > p.bw - 1)
+    if (p.mode == SIM_MODE_L1 || p.exact_terms || p.ph > p.bh - 1 || p.pw > p.bw - 1)
         return false;
     // 32 channels per row tile, two templates per step: smaller problems leave the tiles mostly empty
     if (p.C < 24 || p.O < 8 || p.B == 0)
         return false;
-    return mfma_grad_tiling(grad_as_forward(p)).ok;
+    if (stride_tiling(p).ok)
+        return true;
+    std::vector<GradPhase> ph;
+    if (p.sh * p.sw > kMaxPhases || !grad_phases(p, ph) || ph.empty())
+        return false;
+    for (const GradPhase &g : ph)
+        if (!g.t.ok)
+            return false;
+    return true;
 }
 
 size_t sim_mfma_grad_input_workspace_bytes(const SimPlan &p)
 {
-    const MfmaTiling t = mfma_grad_tiling(grad_as_forward(p));
-    return align_up(t.pm_floats * sizeof(float), 256) + align_up((size_t)p.C * sizeof(float), 256);
+    const StrideTiling st = stride_tiling(p);
+    if (st.ok)
+        return align_up((size_t)p.C * sizeof(float), 256) + align_up(st.pm_floats * sizeof(float), 256);
+    std::vector<GradPhase> ph;
+    grad_phases(p, ph);
+    size_t bytes = align_up((size_t)p.C * sizeof(float), 256);
+    for (const GradPhase &g : ph)
+        bytes += align_up(g.t.pm_floats * sizeof(float), 256);
+    return bytes;
 }
 
 int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
@@ -500,35 +901,73 @@ int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float
                                void *stream)
 {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const SimPlan q = grad_as_forward(p);
-    const MfmaTiling t = mfma_grad_tiling(q);
-    if (!t.ok)
+    const StrideTiling st = stride_tiling(p);
+    if (st.ok) {
+        if (workspace_bytes < sim_mfma_grad_input_workspace_bytes(p))
+            return SIMNETS_ERR_WORKSPACE;
+        char *ws = reinterpret_cast<char *>(workspace);
+        float *ctr = reinterpret_cast<float *>(ws);
+        float *pm = reinterpret_cast<float *>(ws + align_up((size_t)p.C * sizeof(float), 256));
+        const bool norm = p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+        hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, p.bh * p.bw, ctr);
+        const long long total = (long long)st.pm_floats;
+        hipLaunchKernelGGL(mfma_grad_strided_pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 8192)),
+                           dim3(256), 0, s, templates, weights, ctr, p.O, p.C, st.Cpad, st.q.T, st.q.CC,
+                           norm ? 1.0f : 2.0f, total, pm);
+        MfmaArgs a = {};
+        a.in = output_grad; a.out = input_grad; a.pm = pm; a.ctr = ctr;
+        a.x = input; a.x_channels = p.C; a.ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
+        a.oys = p.sh; a.oxs = p.sw; a.x_w = p.W; a.x_plane = p.H * p.W;
+        a.B = p.B; a.C = p.O; a.H = p.oh; a.W = p.ow; a.O = p.C; a.Opad = st.Cpad;
+        dim3 grid((unsigned)(p.B * st.q.tiles), (unsigned)(st.Cpad / (WG_TPL / 2)));
+        if (st.nph == 4)
+            hipLaunchKernelGGL(sim_mfma_grad_strided_kernel<4>, grid, dim3(kThreads), st.lds_bytes, s, a, st.q);
+        else
+            hipLaunchKernelGGL(sim_mfma_grad_strided_kernel<2>, grid, dim3(kThreads), st.lds_bytes, s, a, st.q);
+        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
+    std::vector<GradPhase> phases;
+    if (!grad_phases(p, phases) || phases.empty())
         return SIMNETS_ERR_ALGO;
+    for (const GradPhase &g : phases)
+        if (!g.t.ok)
+            return SIMNETS_ERR_ALGO;
     if (workspace_bytes < sim_mfma_grad_input_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     char *ws = reinterpret_cast<char *>(workspace);
-    float *pm = reinterpret_cast<float *>(ws);
-    float *ctr = reinterpret_cast<float *>(ws + align_up(t.pm_floats * sizeof(float), 256));
+    float *ctr = reinterpret_cast<float *>(ws);
+    ws += align_up((size_t)p.C * sizeof(float), 256);
     const bool norm = p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     hipLaunchKernelGGL(mfma_center_kernel, dim3(p.C), dim3(256), 0, s, templates, p.O, p.C, p.bh * p.bw, ctr);
-    const long long total = (long long)t.pm_floats;
-    hipLaunchKernelGGL(mfma_grad_pack_kernel, dim3((unsigned)std::min<long long>((total + 255) / 256, 8192)), dim3(256),
-                       0, s, templates, weights, ctr, p.O, p.C, t.Opad, p.bh, p.bw, norm ? 1.0f : 2.0f, total, pm);
-    if (hipGetLastError() != hipSuccess)
-        return SIMNETS_ERR_HIP;
-
-    MfmaArgs a;
+    MfmaArgs a = {};
+    MfmaPhases ph = {};
+    MfmaGradPack pk = {};
+    const int Cpad = phases[0].t.Opad;
+    long long pm_off = 0;
+    size_t lds_bytes = 0;
+    for (size_t i = 0; i < phases.size(); ++i) {
+        const GradPhase &g = phases[i];
+        ph.g[i] = mfma_geom(g.q, g.t);
+        ph.g[i].oy0 = g.oy0; ph.g[i].ox0 = g.ox0;
+        ph.g[i].pm_off = pm_off;
+        pk.p[i] = {g.ry, g.rx, g.na, g.nb, pm_off, (long long)g.t.pm_floats};
+        pm_off += (long long)(align_up(g.t.pm_floats * sizeof(float), 256) / sizeof(float));
+        a.grid_tiles = std::max(a.grid_tiles, ph.g[i].tiles);
+        lds_bytes = std::max(lds_bytes, (size_t)g.t.CC * g.t.chan_lds * sizeof(float));
+        pk.max_floats = std::max(pk.max_floats, (long long)g.t.pm_floats);
+    }
+    float *pm = reinterpret_cast<float *>(ws);
+    hipLaunchKernelGGL(mfma_grad_pack_kernel,
+                       dim3((unsigned)std::min<long long>((pk.max_floats + 255) / 256, 4096), (unsigned)phases.size()),
+                       dim3(256), 0, s, templates, weights, ctr, p.O, p.C, Cpad, p.bh, p.bw, p.sh, p.sw,
+                       norm ? 1.0f : 2.0f, pk, pm);
     a.in = output_grad; a.out = input_grad; a.pm = pm; a.bias = nullptr; a.ctr = ctr;
     a.x = input; a.x_channels = p.C; a.ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
-    a.B = q.B; a.C = q.C; a.H = q.H; a.W = q.W; a.O = q.O; a.Opad = t.Opad;
-    a.oh = q.oh; a.ow = q.ow; a.npix = q.oh * q.ow;
-    a.bh = q.bh; a.bw = q.bw; a.sh = 1; a.sw = 1; a.ph = q.ph; a.pw = q.pw;
-    a.tiles = (a.npix + WG_PIX - 1) / WG_PIX;
-    a.TC = t.TC; a.TRmax = t.TRmax; a.chan_lds = t.chan_lds; a.CC = t.CC;
+    a.oys = p.sh; a.oxs = p.sw; a.x_w = p.W; a.x_plane = p.H * p.W;
+    a.B = p.B; a.C = p.O; a.H = p.oh; a.W = p.ow; a.O = p.C; a.Opad = Cpad;
     a.oob = 0.0f;
-    dim3 grid((unsigned)(q.B * a.tiles), (unsigned)(t.Opad / (WG_TPL / 2)));
-    const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
-    hipLaunchKernelGGL(sim_mfma_kernel<true>, grid, dim3(kThreads), lds_bytes, s, a);
+    dim3 grid((unsigned)(p.B * a.grid_tiles), (unsigned)(Cpad / (WG_TPL / 2)), (unsigned)phases.size());
+    hipLaunchKernelGGL(sim_mfma_kernel<true>, grid, dim3(kThreads), lds_bytes, s, a, ph);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

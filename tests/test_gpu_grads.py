@@ -490,18 +490,29 @@ def test_similarity_params_grad_row_staged_matrix_form(pkg, case, func, norm, ig
     dict(shape=(1, 70, 9, 40), O=33, blocks=[2, 4], padding=[0, 3]),       # two channel tiles, asymmetric block
     dict(shape=(3, 24, 20, 20), O=16, blocks=[5, 5], padding=[4, 0]),      # padding = block - 1
     dict(shape=(2, 32, 6, 300), O=12, blocks=[1, 3], padding=[0, 1]),      # several pixel tiles per row
+    dict(shape=(2, 24, 14, 15), O=10, blocks=[3, 3], padding=[1, 1], strides=[2, 2]),   # four phases: 4, 2, 2, 1 taps
+    dict(shape=(1, 40, 23, 22), O=9, blocks=[7, 7], padding=[3, 3], strides=[2, 2]),    # 16, 12, 12, 9 taps
+    dict(shape=(2, 26, 12, 17), O=8, blocks=[3, 2], padding=[2, 0], strides=[2, 1]),    # a phase starting past the padding
+    dict(shape=(1, 30, 11, 20), O=11, blocks=[3, 4], padding=[0, 2], strides=[3, 2]),   # leftover rows no window covers
+    dict(shape=(2, 24, 9, 9), O=8, blocks=[2, 2], padding=[0, 0], strides=[2, 2]),      # disjoint windows, one tap a phase
+    dict(shape=(3, 64, 37, 41), O=19, blocks=[3, 3], padding=[1, 1], strides=[2, 2]),   # several position tiles, odd O
+    dict(shape=(1, 25, 8, 70), O=12, blocks=[1, 4], padding=[0, 1], strides=[1, 2]),    # two phases along the width
+    dict(shape=(1, 33, 19, 16), O=8, blocks=[3, 3], padding=[1, 1], strides=[3, 3]),    # nine phases, one launch grid each
 ])
 def test_similarity_input_grad_matrix_form(pkg, case, func, norm, ign):
-    """Stride 1, at least 24 channels: the L2 modes' input gradient is A - (x - c) B with both products on the
-    matrix cores.  Data sit away from zero (the centre c matters); algo='direct' takes the term-by-term kernel."""
+    """At least 24 channels, strides no larger than the window: the L2 modes' input gradient is A - (x - c) B with
+    both products on the matrix cores.  Two or four stride phases share a workgroup's tile of the output gradient;
+    other strides run one grid per phase.  Data sit away from zero (the centre c matters); algo='direct' takes the
+    term-by-term kernel."""
     g = np.random.default_rng(52)
     x = (3.0 + g.normal(size=case["shape"])).astype(np.float32)
     t = (3.0 + g.normal(size=(case["O"], case["shape"][1]) + tuple(case["blocks"]))).astype(np.float32)
     w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
     if ign:
         x[g.random(size=x.shape) < 0.15] = np.nan
-    kw = dict(similarity_function=func, blocks=case["blocks"], strides=[1, 1], padding=case["padding"],
-              normalization_term=norm, ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else 1.5)
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case.get("strides", [1, 1]),
+              padding=case["padding"], normalization_term=norm, ignore_nan_input=ign,
+              out_of_bounds_value=float("nan") if ign else 1.5)
     out = orc.similarity_fwd(x, t, w, **kw)
     og = g.normal(size=out.shape).astype(np.float32)
     want = orc.similarity_input_grad(x, t, w, og, **kw)
