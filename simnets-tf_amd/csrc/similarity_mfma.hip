@@ -44,7 +44,7 @@ constexpr int WG_PIX = 2 * RP * 32;   // 256 pixels per workgroup (2 pixel waves
 constexpr int WG_TPL = 2 * RM * 32;   // 128 templates per workgroup (2 template waves)
 constexpr int kLdsBudgetFloats = 12288;  // 48 KiB input tile per workgroup
 constexpr int kStagePos = 8;             // tile elements per thread and channel (at most kStagePos * 256 floats)
-constexpr int kStageChan = 4;            // channels whose loads are in flight at once while staging
+constexpr int kStageGroups = 2;          // channel groups whose loads are in flight at once while staging
 
 // Geometry of one launch grid: the forward op's, or one stride phase of the input gradient.
 struct MfmaGeom {
@@ -52,6 +52,7 @@ struct MfmaGeom {
     int bh, bw, sh, sw, ph, pw;
     int tiles;               // workgroup pixel tiles per image
     int TC, chan_lds, CC;
+    int NI;                  // images per workgroup (maps of at most half a pixel tile; then tiles == 1), else 1
     int oy0, ox0;            // input gradient: first input row / column of the phase
     long long pm_off;        // this grid's packed operands inside pm, floats
 };
@@ -75,6 +76,12 @@ struct MfmaArgs {
     int B, C, H, W, O, Opad;
     int grid_tiles;     // pixel tiles per image in blockIdx.x (the largest phase's count)
     float oob;
+    // input gradient with few workgroups: blockIdx.z = phase * nsplit + split, split s takes the chunks
+    // [s n / nsplit, (s + 1) n / nsplit) of the output gradient's channels and writes its partial result to
+    // part + s * part_stride (same layout as out); a second kernel adds the parts in order
+    int nsplit;
+    float *part;
+    long long part_stride;
     MfmaGeom g;         // the forward op's grid
 };
 
@@ -98,7 +105,8 @@ struct MfmaPhases {
 template <bool GRAD>
 __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a, const MfmaPhases phases)
 {
-    const MfmaGeom &g = GRAD ? phases.g[blockIdx.z] : a.g;
+    const int split = GRAD ? blockIdx.z % a.nsplit : 0;
+    const MfmaGeom &g = GRAD ? phases.g[blockIdx.z / a.nsplit] : a.g;
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -106,27 +114,33 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     const int wm = wave & 1, wp = wave >> 1;
     const int col = lane & 31, half = lane >> 5;
 
-    const int b = blockIdx.x / a.grid_tiles;
-    const int tile = blockIdx.x - b * a.grid_tiles;
-    if (tile >= g.tiles)
-        return;  // a phase with fewer pixel tiles than the largest one
+    // a workgroup covers a tile of one image's pixels, or all pixels of g.NI images (positions = image, pixel)
+    const bool multi = g.NI > 1;
+    const int b = multi ? blockIdx.x * g.NI : blockIdx.x / a.grid_tiles;
+    const int tile = multi ? 0 : blockIdx.x - b * a.grid_tiles;
+    if (tile >= g.tiles || b >= a.B)
+        return;  // a phase with fewer workgroups than the largest one
+    const int nimg = multi ? min(g.NI, a.B - b) : 1;
     const int p_first = tile * WG_PIX;
-    const int p_last = min(p_first + WG_PIX, g.npix) - 1;
+    const int p_last = multi ? nimg * g.npix - 1 : min(p_first + WG_PIX, g.npix) - 1;
     const int h_first = p_first / g.ow;
-    const int nrows = p_last / g.ow - h_first + 1;
+    const int nrows = (multi ? g.npix - 1 : p_last) / g.ow - h_first + 1;
     const int TR = (nrows - 1) * g.sh + g.bh;
     const int in_row0 = h_first * g.sh - g.ph;
     const int mbase = GRAD ? blockIdx.y * (WG_TPL / 2) + wm * 32 : blockIdx.y * WG_TPL + wm * (RM * 32);
 
     // per pixel tile: LDS address of this lane's pixel (k-pair half folded in)
-    int xbase[RP], pix[RP];
+    int xbase[RP], pix[RP], pimg[RP];   // pixel inside its image, image (-1: none)
 #pragma unroll
     for (int j = 0; j < RP; ++j) {
         const int p = p_first + (wp * RP + j) * 32 + col;
-        pix[j] = p;
         const int pc = min(p, p_last);
-        const int h = pc / g.ow, w = pc - h * g.ow;
-        xbase[j] = (h - h_first) * g.sh * g.TC + w * g.sw + half * g.chan_lds;
+        const int il = multi ? pc / g.npix : 0;
+        const int pr = pc - il * g.npix;
+        pix[j] = pr;
+        pimg[j] = p <= p_last ? b + il : -1;
+        const int h = pr / g.ow, w = pr - h * g.ow;
+        xbase[j] = il * (TR * g.TC) + (h - h_first) * g.sh * g.TC + w * g.sw + half * g.chan_lds;
     }
 
     floatx16 acc[RM][RP];
@@ -144,6 +158,10 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     // parameter operand: this lane's element within a [type][half][Opad] step record
     const int step_stride = 4 * a.Opad;
     const float *pm = a.pm + g.pm_off + half * a.Opad + mbase + col;
+    if (GRAD && a.nsplit > 1) {
+        const int nchunks = (a.C + g.CC - 1) / g.CC;
+        pm += (size_t)(split * nchunks / a.nsplit) * (g.CC / 2) * g.bh * g.bw * step_stride;
+    }
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
 
     float pw_cur[RM], pt_cur[RM], pw_nxt[RM], pt_nxt[RM];
@@ -160,15 +178,22 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     load_params(pm + step_stride, pw_nxt, pt_nxt);
     pm += 2 * step_stride;
 
-    TilePositions<kStagePos> tp;
-    tp.template init<kThreads>(a.H, a.W, TR, g.TC, in_row0, g.pw);
+    GroupedTile<kStagePos> gt;
+    gt.template init<kThreads>(a.H, a.W, TR, g.TC, in_row0, g.pw, g.NI, nimg, a.C * a.H * a.W, g.chan_lds, g.CC);
 
-    for (int ch0 = 0; ch0 < a.C; ch0 += g.CC) {
+    // this workgroup's chunks of the image channels (all of them unless the input gradient is split)
+    int ch_first = 0, ch_end = a.C;
+    if (GRAD && a.nsplit > 1) {
+        const int nchunks = (a.C + g.CC - 1) / g.CC;
+        ch_first = split * nchunks / a.nsplit * g.CC;
+        ch_end = min(a.C, (split + 1) * nchunks / a.nsplit * g.CC);
+    }
+    for (int ch0 = ch_first; ch0 < ch_end; ch0 += g.CC) {
         const int ccn = min(g.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
-        stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.H, a.W, ch0, ccp, ccn, g.chan_lds, a.oob,
-                                                     GRAD ? nullptr : a.ctr, tp);
+        gt.template stage<kStageGroups>(lds, img + (size_t)ch0 * a.H * a.W, a.H * a.W, ccp, ccn, g.chan_lds, a.oob,
+                                      GRAD ? nullptr : a.ctr + ch0);
         __syncthreads();
 
         // steps of this chunk in (channel pair, dh, dw) order; the pixel operand of step s+1 and the
@@ -241,12 +266,13 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     if constexpr (GRAD) {
         // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel ----
         const size_t xplane = (size_t)a.x_plane;
-        float *ob = a.out + (size_t)b * a.x_channels * xplane;
-        const float *xb = a.x + (size_t)b * a.x_channels * xplane;
+        float *out = a.nsplit > 1 ? a.part + split * a.part_stride : a.out;
 #pragma unroll
         for (int j = 0; j < RP; ++j) {
-            if (pix[j] > p_last)
+            if (pimg[j] < 0)
                 continue;
+            float *ob = out + (size_t)pimg[j] * a.x_channels * xplane;
+            const float *xb = a.x + (size_t)pimg[j] * a.x_channels * xplane;
             const int pr = pix[j] / g.ow, pc = pix[j] - pr * g.ow;
             const size_t at = (size_t)(g.oy0 + pr * a.oys) * a.x_w + (g.ox0 + pc * a.oxs);
 #pragma unroll
@@ -264,11 +290,11 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
         return;
     }
     // ---- store: lane holds, per tile, 16 templates of one pixel ----
-    float *ob = a.out + (size_t)b * a.O * plane;
 #pragma unroll
     for (int j = 0; j < RP; ++j) {
-        if (pix[j] > p_last)
+        if (pimg[j] < 0)
             continue;
+        float *ob = a.out + (size_t)pimg[j] * a.O * plane;
 #pragma unroll
         for (int i = 0; i < RM; ++i)
 #pragma unroll
@@ -348,42 +374,14 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(cons
         pb[i] = pm[i * step_stride + 2 * a.Opad];
     }
 
-    // Staging: the tile of a channel is small here (a few rows of the position grid), so a thread's kStagePos
-    // elements span a group of G channels and every thread has that many loads in flight.
-    const int per_chan = TR * q.TC;
-    const int G = max(1, min(kStagePos * kThreads / per_chan, q.CC));
-    const int plane_g = a.H * a.W;
-    int gofs[kStagePos], lofs[kStagePos], gchan[kStagePos];
-#pragma unroll
-    for (int j = 0; j < kStagePos; ++j) {
-        const int e = tid + j * kThreads;
-        const int cc = e / per_chan;
-        const int pos = e - cc * per_chan;
-        const int r = pos / q.TC, c = pos - r * q.TC;
-        const int ih = h_first + q.row_min + r, iw = c + q.col_min;
-        gchan[j] = cc < G ? cc : (1 << 20);   // beyond the group: never staged
-        lofs[j] = cc * q.chan_lds + pos;
-        gofs[j] = (ih >= 0 && ih < a.H && iw >= 0 && iw < a.W) ? cc * plane_g + ih * a.W + iw : -1;
-    }
+    GroupedTile<kStagePos> gt;
+    gt.template init<kThreads>(a.H, a.W, TR, q.TC, h_first + q.row_min, -q.col_min, 1, 1, 0, q.chan_lds, q.CC);
 
     for (int ch0 = 0; ch0 < a.C; ch0 += q.CC) {
         const int ccn = min(q.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
-        for (int c0 = 0; c0 < ccp; c0 += G) {
-            const float *src = img + (size_t)(ch0 + c0) * plane_g;
-            float v[kStagePos];
-#pragma unroll
-            for (int j = 0; j < kStagePos; ++j) {
-                v[j] = 0.0f;
-                if (c0 + gchan[j] < ccn && gofs[j] >= 0)
-                    v[j] = src[gofs[j]];
-            }
-#pragma unroll
-            for (int j = 0; j < kStagePos; ++j)
-                if (c0 + gchan[j] < ccp)
-                    lds[c0 * q.chan_lds + lofs[j]] = v[j];
-        }
+        gt.template stage<kStageGroups>(lds, img + (size_t)ch0 * a.H * a.W, a.H * a.W, ccp, ccn, q.chan_lds, 0.0f, nullptr);
         __syncthreads();
 
         // taps outside, template pairs inside: the inner loop has one phase and walks the channel slots of the tile
@@ -625,8 +623,33 @@ __global__ void mfma_grad_strided_pack_kernel(const float *__restrict__ template
     }
 }
 
+// out[i] = part[0][i] + part[1][i] + ... in that order (the partial input gradients of a split contraction)
+__global__ __launch_bounds__(256) void mfma_sum_parts_kernel(const float *__restrict__ part, int nsplit, long long n,
+                                                             float *__restrict__ out)
+{
+    for (long long i = ((long long)blockIdx.x * blockDim.x + threadIdx.x) * 4; i < n;
+         i += (long long)gridDim.x * blockDim.x * 4) {
+        if (i + 4 <= n && (n & 3) == 0 && (reinterpret_cast<size_t>(out) & 15) == 0) {
+            float4 acc = *reinterpret_cast<const float4 *>(part + i);
+            for (int z = 1; z < nsplit; ++z) {
+                const float4 v = *reinterpret_cast<const float4 *>(part + z * n + i);
+                acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+            }
+            *reinterpret_cast<float4 *>(out + i) = acc;
+        } else {
+            for (long long k = i; k < min(i + 4, n); ++k) {
+                float acc = part[k];
+                for (int z = 1; z < nsplit; ++z)
+                    acc += part[z * n + k];
+                out[k] = acc;
+            }
+        }
+    }
+}
+
 struct MfmaTiling {
     int Opad, steps, TC, TRmax, chan_lds, CC;
+    int NI;   // images per workgroup (small maps), else 1
     bool ok;
     size_t pm_floats;
 };
@@ -639,12 +662,23 @@ MfmaTiling mfma_tiling(const SimPlan &p)
     t.TC = (p.ow - 1) * p.sw + p.bw;
     const int max_rows = std::min(p.oh, (WG_PIX + p.ow - 1) / p.ow + 1);
     t.TRmax = (max_rows - 1) * p.sh + p.bh;
+    // maps of at most half a pixel tile: a workgroup takes several images, their tiles side by side in a channel slot
+    t.NI = 1;
+    const int npix = p.oh * p.ow;
+    if (2 * npix <= WG_PIX && p.B >= 2) {
+        const long long img_elems = 1LL * ((p.oh - 1) * p.sh + p.bh) * t.TC;
+        int ni = std::min(WG_PIX / npix, p.B);
+        while (ni > 1 && (ni * img_elems > kStagePos * kThreads || 2 * (ni * img_elems + 64) > kLdsBudgetFloats))
+            --ni;
+        t.NI = ni;
+    }
+    const long long per_chan = t.NI > 1 ? t.NI * 1LL * ((p.oh - 1) * p.sh + p.bh) * t.TC : 1LL * t.TRmax * t.TC;
     // channel pitch = 32 mod 64 floats: the two k-pair halves of a wave land in disjoint LDS banks
-    long long pitch = 1LL * t.TRmax * t.TC;
+    long long pitch = per_chan;
     pitch = (pitch + 31) / 64 * 64 + 32;
-    if (pitch < 1LL * t.TRmax * t.TC)
+    if (pitch < per_chan)
         pitch += 64;
-    t.ok = 2 * pitch <= kLdsBudgetFloats && 1LL * t.TRmax * t.TC <= kStagePos * kThreads;
+    t.ok = 2 * pitch <= kLdsBudgetFloats && per_chan <= kStagePos * kThreads;
     t.chan_lds = (int)pitch;
     int cc_max = t.ok ? (int)(kLdsBudgetFloats / pitch) & ~1 : 2;
     cc_max = std::min(cc_max, (p.C + 1) & ~1);
@@ -661,7 +695,7 @@ MfmaGeom mfma_geom(const SimPlan &p, const MfmaTiling &t)
     g.ow = p.ow; g.npix = p.oh * p.ow;
     g.bh = p.bh; g.bw = p.bw; g.sh = p.sh; g.sw = p.sw; g.ph = p.ph; g.pw = p.pw;
     g.tiles = (g.npix + WG_PIX - 1) / WG_PIX;
-    g.TC = t.TC; g.chan_lds = t.chan_lds; g.CC = t.CC;
+    g.TC = t.TC; g.chan_lds = t.chan_lds; g.CC = t.CC; g.NI = t.NI;
     return g;
 }
 
@@ -724,7 +758,8 @@ int sim_mfma_run(const SimPlan &p, const float *input, float *output, void *work
     a.g = mfma_geom(p, t);
     a.grid_tiles = a.g.tiles;
     a.oob = p.oob;
-    dim3 grid((unsigned)(p.B * a.g.tiles), (unsigned)(t.Opad / WG_TPL));
+    a.nsplit = 1;
+    dim3 grid((unsigned)(t.NI > 1 ? (p.B + t.NI - 1) / t.NI : p.B * a.g.tiles), (unsigned)(t.Opad / WG_TPL));
     const size_t lds_bytes = (size_t)t.CC * t.chan_lds * sizeof(float);
     hipLaunchKernelGGL(sim_mfma_kernel<false>, grid, dim3(kThreads), lds_bytes, s, a, MfmaPhases{});
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
@@ -863,6 +898,30 @@ StrideTiling stride_tiling(const SimPlan &p)
     return t;
 }
 
+// Workgroups along blockIdx.x of one phase's grid.
+unsigned grad_phase_blocks(const SimPlan &p, const GradPhase &g)
+{
+    const int tiles = (g.q.oh * g.q.ow + WG_PIX - 1) / WG_PIX;
+    return (unsigned)(g.t.NI > 1 ? (p.B + g.t.NI - 1) / g.t.NI : p.B * tiles);
+}
+
+// Small problems give the chip too few workgroups: the channels of the output gradient (the contraction) are then
+// split over up to 16 workgroups whose partial results a second kernel adds in order.
+int grad_split(const SimPlan &p, const std::vector<GradPhase> &ph)
+{
+    if (ph.empty())
+        return 1;
+    long long wgs = 0;
+    int min_chunks = 1 << 30;
+    for (const GradPhase &g : ph) {
+        wgs += (long long)grad_phase_blocks(p, g) * (g.t.Opad / (WG_TPL / 2));
+        min_chunks = std::min(min_chunks, (g.q.C + g.t.CC - 1) / g.t.CC);
+    }
+    if (wgs >= 256)
+        return 1;
+    return (int)std::max<long long>(1, std::min<long long>(std::min(min_chunks, 16), (512 + wgs - 1) / wgs));
+}
+
 }  // namespace
 
 bool sim_mfma_grad_input_supported(const SimPlan &p)
@@ -893,6 +952,9 @@ size_t sim_mfma_grad_input_workspace_bytes(const SimPlan &p)
     size_t bytes = align_up((size_t)p.C * sizeof(float), 256);
     for (const GradPhase &g : ph)
         bytes += align_up(g.t.pm_floats * sizeof(float), 256);
+    const int nsplit = grad_split(p, ph);
+    if (nsplit > 1)
+        bytes += align_up((size_t)nsplit * p.B * p.C * p.H * p.W * sizeof(float), 256);
     return bytes;
 }
 
@@ -945,6 +1007,7 @@ int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float
     const int Cpad = phases[0].t.Opad;
     long long pm_off = 0;
     size_t lds_bytes = 0;
+    unsigned blocks_x = 0;
     for (size_t i = 0; i < phases.size(); ++i) {
         const GradPhase &g = phases[i];
         ph.g[i] = mfma_geom(g.q, g.t);
@@ -952,22 +1015,32 @@ int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float
         ph.g[i].pm_off = pm_off;
         pk.p[i] = {g.ry, g.rx, g.na, g.nb, pm_off, (long long)g.t.pm_floats};
         pm_off += (long long)(align_up(g.t.pm_floats * sizeof(float), 256) / sizeof(float));
-        a.grid_tiles = std::max(a.grid_tiles, ph.g[i].tiles);
+        if (g.t.NI == 1)
+            a.grid_tiles = std::max(a.grid_tiles, ph.g[i].tiles);
+        blocks_x = std::max(blocks_x, grad_phase_blocks(p, g));
         lds_bytes = std::max(lds_bytes, (size_t)g.t.CC * g.t.chan_lds * sizeof(float));
         pk.max_floats = std::max(pk.max_floats, (long long)g.t.pm_floats);
     }
+    a.grid_tiles = std::max(a.grid_tiles, 1);
     float *pm = reinterpret_cast<float *>(ws);
     hipLaunchKernelGGL(mfma_grad_pack_kernel,
                        dim3((unsigned)std::min<long long>((pk.max_floats + 255) / 256, 4096), (unsigned)phases.size()),
                        dim3(256), 0, s, templates, weights, ctr, p.O, p.C, Cpad, p.bh, p.bw, p.sh, p.sw,
                        norm ? 1.0f : 2.0f, pk, pm);
+    const long long n_in = (long long)p.B * p.C * p.H * p.W;
+    a.nsplit = grad_split(p, phases);
+    a.part = reinterpret_cast<float *>(ws + (size_t)pm_off * sizeof(float));
+    a.part_stride = n_in;
     a.in = output_grad; a.out = input_grad; a.pm = pm; a.bias = nullptr; a.ctr = ctr;
     a.x = input; a.x_channels = p.C; a.ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
     a.oys = p.sh; a.oxs = p.sw; a.x_w = p.W; a.x_plane = p.H * p.W;
     a.B = p.B; a.C = p.O; a.H = p.oh; a.W = p.ow; a.O = p.C; a.Opad = Cpad;
     a.oob = 0.0f;
-    dim3 grid((unsigned)(p.B * a.grid_tiles), (unsigned)(Cpad / (WG_TPL / 2)), (unsigned)phases.size());
+    dim3 grid(blocks_x, (unsigned)(Cpad / (WG_TPL / 2)), (unsigned)(phases.size() * a.nsplit));
     hipLaunchKernelGGL(sim_mfma_kernel<true>, grid, dim3(kThreads), lds_bytes, s, a, ph);
+    if (a.nsplit > 1)
+        hipLaunchKernelGGL(mfma_sum_parts_kernel, dim3((unsigned)std::min<long long>((n_in + 1023) / 1024, 4096)),
+                           dim3(256), 0, s, a.part, a.nsplit, n_in, input_grad);
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

@@ -110,4 +110,75 @@ __device__ __forceinline__ void stage_input_tile_fast(float *lds, const float *i
     }
 }
 
+// Variant for small tiles: a thread's NPOS elements span a group of G channels (and, with several images per
+// workgroup, the images' tiles side by side inside a channel slot), so that every thread has NPOS loads in flight
+// however small the tile of one channel is.  LDS element (cc, image il, r, c) sits at cc * chan_pitch +
+// il * TR * TC + r * TC + c and holds input[b0 + il][ch0 + cc][row0 + r][c - pad_w].
+template <int NPOS>
+struct GroupedTile {
+    int gofs[NPOS];  // offset from (image b0, first channel of the group); -1: pad value; -2: not an element
+    int lofs[NPOS];  // LDS offset from the group's first channel slot | channel inside the group << 16
+    int G;           // channels per group
+
+    // nslots images have a tile in a channel slot, the first nimg of them exist; image_stride = floats per image
+    template <int NTHREADS>
+    __device__ __forceinline__ void init(int H, int W, int TR, int TC, int row0, int pad_w, int nslots, int nimg,
+                                         int image_stride, int chan_pitch, int max_group)
+    {
+        const int img_elems = TR * TC;
+        const int per_chan = nslots * img_elems;
+        G = max(1, min(NPOS * NTHREADS / per_chan, max_group));
+#pragma unroll
+        for (int j = 0; j < NPOS; ++j) {
+            const int e = threadIdx.x + j * NTHREADS;
+            const int cc = e / per_chan;
+            const int rem = e - cc * per_chan;
+            const int il = rem / img_elems;
+            const int pos = rem - il * img_elems;
+            const int r = pos / TC, c = pos - r * TC;
+            const int ih = row0 + r, iw = c - pad_w;
+            lofs[j] = (cc * chan_pitch + rem) | (cc << 16);
+            if (cc >= G)
+                gofs[j] = -2;
+            else if (il < nimg && ih >= 0 && ih < H && iw >= 0 && iw < W)
+                gofs[j] = il * image_stride + cc * H * W + ih * W + iw;
+            else
+                gofs[j] = -1;
+        }
+    }
+
+    // src: channel ch0 of image b0; channels [0, nvalid) exist, [nvalid, nchan) are zero filled; shift: per-channel
+    // value subtracted from the staged elements (indexed from channel ch0), or null.  R groups per round: R * NPOS
+    // loads of a thread are in flight before its first LDS store.
+    template <int R>
+    __device__ __forceinline__ void stage(float *lds, const float *src, int plane, int nchan, int nvalid,
+                                          int chan_pitch, float oob, const float *shift) const
+    {
+        for (int c0 = 0; c0 < nchan; c0 += R * G) {
+            float v[R][NPOS];
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float *from = src + (size_t)(c0 + r * G) * plane;
+#pragma unroll
+                for (int j = 0; j < NPOS; ++j) {
+                    const int ch = c0 + r * G + (lofs[j] >> 16);
+                    float val = 0.0f;
+                    if (gofs[j] != -2 && ch < nvalid) {
+                        val = gofs[j] >= 0 ? from[gofs[j]] : oob;
+                        if (shift != nullptr)
+                            val -= shift[ch];
+                    }
+                    v[r][j] = val;
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int j = 0; j < NPOS; ++j)
+                    if (gofs[j] != -2 && c0 + r * G + (lofs[j] >> 16) < nchan)
+                        lds[(c0 + r * G) * chan_pitch + (lofs[j] & 0xffff)] = v[r][j];
+        }
+    }
+};
+
 }  // namespace simnets

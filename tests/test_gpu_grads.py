@@ -498,6 +498,10 @@ def test_similarity_params_grad_row_staged_matrix_form(pkg, case, func, norm, ig
     dict(shape=(3, 64, 37, 41), O=19, blocks=[3, 3], padding=[1, 1], strides=[2, 2]),   # several position tiles, odd O
     dict(shape=(1, 25, 8, 70), O=12, blocks=[1, 4], padding=[0, 1], strides=[1, 2]),    # two phases along the width
     dict(shape=(1, 33, 19, 16), O=8, blocks=[3, 3], padding=[1, 1], strides=[3, 3]),    # nine phases, one launch grid each
+    dict(shape=(7, 48, 7, 7), O=100, blocks=[3, 3], padding=[1, 1]),      # 5 + 2 images per workgroup, contraction split
+    dict(shape=(3, 30, 5, 9), O=64, blocks=[2, 3], padding=[1, 2]),       # 45 pixels: one group of 3 images
+    dict(shape=(1, 64, 20, 20), O=300, blocks=[3, 3], padding=[1, 1]),    # two pixel tiles, contraction split 11 ways
+    dict(shape=(6, 24, 9, 10), O=90, blocks=[3, 3], padding=[1, 1], strides=[3, 3]),    # small phase grids, split
 ])
 def test_similarity_input_grad_matrix_form(pkg, case, func, norm, ign):
     """At least 24 channels, strides no larger than the window: the L2 modes' input gradient is A - (x - c) B with

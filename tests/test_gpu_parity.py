@@ -182,6 +182,9 @@ def test_similarity_l2_default_form_recomputes_outputs_near_zero(pkg, geom, kind
     dict(shape=(2, 4, 31, 29), O=130, blocks=[2, 3], strides=[2, 1], padding=[0, 2]),    # two template groups
     dict(shape=(1, 3, 40, 40), O=5, blocks=[5, 5], strides=[2, 2], padding=[2, 2]),
     dict(shape=(2, 1, 28, 28), O=32, blocks=[2, 2], strides=[2, 2], padding=[2, 2]),     # single channel
+    dict(shape=(7, 20, 7, 7), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),      # 5 + 2 images per workgroup
+    dict(shape=(3, 9, 12, 11), O=12, blocks=[3, 2], strides=[2, 1], padding=[0, 0]),     # 50 pixels: 3 images a group
+    dict(shape=(12, 6, 4, 4), O=9, blocks=[2, 2], strides=[1, 1], padding=[1, 1]),       # 25 pixels: 10 + 2 images
 ])
 def test_similarity_mfma_algorithm_matches_direct(pkg, case):
     x, t, w = sim_inputs(8, case["shape"], case["O"], case["blocks"])
