@@ -53,6 +53,9 @@ def main():
                          "used to scale the FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--cpu-images", type=int, default=12,
                     help="images of configuration 3 the single-threaded CPU baseline times per function (12 ~ 3 s)")
+    ap.add_argument("--shapes", action="store_true",
+                    help="instead of the benchmark line: time Similarity forward, input gradient and parameter "
+                         "gradients on network-like shapes away from the benchmark configurations (one JSON object)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path is data parallel over the batch; "
@@ -106,6 +109,40 @@ def main():
             for _ in range(reps):
                 fn()
         return g
+
+    if args.shapes:
+        # (name, input shape, templates, block, stride, padding): layers of a residual-network-like stack at batch 32
+        shapes = [
+            ("3x224x224->64 7x7 s2 p3", (32, 3, 224, 224), 64, 7, 2, 3),
+            ("64x56x56->64 3x3 s1 p1", (32, 64, 56, 56), 64, 3, 1, 1),
+            ("128x28x28->128 3x3 s1 p1", (32, 128, 28, 28), 128, 3, 1, 1),
+            ("256x14x14->256 3x3 s1 p1", (32, 256, 14, 14), 256, 3, 1, 1),
+            ("512x7x7->512 3x3 s1 p1", (32, 512, 7, 7), 512, 3, 1, 1),
+            ("64x56x56->128 3x3 s2 p1", (32, 64, 56, 56), 128, 3, 2, 1),
+            ("256x56x56->64 1x1", (32, 256, 56, 56), 64, 1, 1, 0),
+            ("64x32x32->128 3x3 s1 p1 batch 256", (256, 64, 32, 32), 128, 3, 1, 1),
+        ]
+        table = {}
+        torch.manual_seed(1234)
+        for name, shp, n_templates, blk, stride, pad in shapes:
+            xs = torch.randn(*shp, device=dev)
+            ts = torch.randn(n_templates, shp[1], blk, blk, device=dev)
+            ws = torch.rand_like(ts) + 0.1
+            kws = dict(blocks=[blk, blk], strides=[stride, stride], padding=[pad, pad])
+            outs = pkg.similarity(xs, ts, ws, **kws)
+            gs = torch.randn_like(outs)
+            gmac = outs.numel() * shp[1] * blk * blk
+            row = {}
+            for key, fn in (("forward", lambda: pkg.similarity(xs, ts, ws, out=outs, **kws)),
+                            ("input_grad", lambda: pkg.similarity_input_grad(xs, ts, ws, gs, **kws)),
+                            ("params_grad", lambda: pkg.similarity_parameters_grad(xs, ts, ws, gs, **kws))):
+                reps = [timed(fn, args.steps, args.warmup)[1] for _ in range(3)]   # the fastest of three batches
+                ms = min(reps)
+                row[key] = {"ms": round(ms, 4), "T_gMAC_per_s": round(gmac / ms / 1e9, 2),
+                            "slowest_batch_ms": round(max(reps), 4)}
+            table[name] = row
+        print(json.dumps({"similarity_shapes": table, "steps": args.steps, "warmup": args.warmup, "dtype": "f32"}))
+        return
 
     if args.pmc_calib:
         src = torch.ones(64 * 1024 * 1024, dtype=torch.float32, device=dev)
