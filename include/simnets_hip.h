@@ -158,9 +158,11 @@ int simnets_hip_similarity_grad_workspace_bytes(const simnets_similarity_attrs *
  * SimilarityInputGradKernelGPU<float>::Compute (src/kernels/similarity_grad_kernel_gpu.cu), i.e. per image
  * im2col_3d_gpu + ggemm_readc_gpu<TRANSPOSE_A> with sim_*_backward_bottom + col2im_3d_gpu.
  * output_grad has the forward output's shape, input_grad the input's.  attrs->algo: SIMNETS_ALGO_DIRECT sums
- * the reference's terms one by one in every case; otherwise the L2 modes at stride 1 with 24 channels or more
- * evaluate A - (x - c) B with A = sum g s w (t - c), B = sum g s w on the fp32 matrix cores (same sum, other
- * rounding; c = the channel's mean template value). */
+ * the reference's terms one by one in every case; otherwise the L2 modes with 24 channels or more (strides no
+ * larger than the window, padding smaller than the window) evaluate A - (x - c) B with A = sum g s w (t - c),
+ * B = sum g s w on the fp32 matrix cores (same sum, other rounding; c = the channel's mean template value).
+ * Small grids split that sum over workgroups and add the parts in a fixed order: results do not vary from
+ * run to run. */
 int simnets_hip_similarity_input_grad(const simnets_similarity_attrs *attrs, const int input_shape[4],
                                       const int templates_shape[4], const int weights_shape[4], const float *input,
                                       const float *templates, const float *weights, const float *output_grad,

@@ -1,4 +1,5 @@
-// Similarity forward, plain L2 only, on the fp32 matrix cores (gfx950 v_mfma_f32_32x32x2_f32).
+// Similarity on the fp32 matrix cores (gfx950 v_mfma_f32_32x32x2_f32): the plain L2 forward (opt-in) and the input
+// gradient of the L2 modes (sim_mfma_kernel<GRAD = true>, sim_mfma_grad_strided_kernel; described at the kernels).
 //
 // The weighted squared distance is expanded into dense contractions over k:
 //   out[b,m,p] = -sum_k w (t - x)^2
@@ -16,9 +17,11 @@
 // templates; wave (wm, wp) owns 64 templates x 128 pixels = 2 x 4 MFMA tiles of 32x32 (128
 // accumulator VGPRs).  Templates are the MFMA row index and pixels the column index, so each lane
 // ends up with 16 values of ONE pixel column and stores run along w: coalesced.
-//   * input rows are staged, a few channels at a time, into LDS (out of image -> out_of_bounds_value,
+//   * input rows are staged, a chunk of channels at a time, into LDS (out of image -> out_of_bounds_value,
 //     shift applied); a lane reads the pixel operand with one ds_read_b32 per tile and k-pair and
 //     squares it in the VALU, which is otherwise idle;
+//   * maps of at most 128 output pixels: the 256 pixel columns of a workgroup are the pixels of several images,
+//     whose tiles sit side by side in a channel's LDS slot;
 //   * the two k of an MFMA k-pair are the same tap (dh, dw) of two adjacent channels, so the
 //     per-lane LDS address is base + uniform offset;
 //   * the parameter operand is read straight from a pre-packed global array in consumption order
