@@ -114,3 +114,51 @@ def test_mex_random_geometry(pkg, seed):
                           orc.mex_input_grad(x64, off64, out64, g64, n, **kw), "dX %s" % kw)
         assert_grad_close(doff, orc.mex_offsets_grad(x, off, want, go, n, **kw),
                           orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "dOff %s" % kw)
+
+
+def random_matrix_gradient_case(g):
+    """Geometries the matrix-core gradient kernels take (L2 modes, at least 24 channels and 8 templates): small maps
+    that share a workgroup tile, strides with two, four or more phases, contractions long enough to be split."""
+    while True:
+        C = int(g.choice([24, 25, 31, 33, 48, 64, 70]))
+        O = int(g.choice([8, 9, 17, 30, 65, 100, 131]))
+        small = bool(g.integers(0, 2))
+        H, W = (int(g.integers(2, 12)), int(g.integers(2, 12))) if small else (int(g.integers(12, 34)), int(g.integers(12, 60)))
+        bh, bw = int(g.integers(1, min(H, 5) + 1)), int(g.integers(1, min(W, 5) + 1))
+        sh, sw = int(g.integers(1, min(bh, 3) + 1)), int(g.integers(1, min(bw, 3) + 1))
+        ph, pw = int(g.integers(0, bh)), int(g.integers(0, bw))
+        mode = int(g.integers(1, 4))
+        B = int(g.integers(1, 10)) if small else int(g.integers(1, 4))
+        kw = dict(similarity_function="L2", blocks=[bh, bw], strides=[sh, sw], padding=[ph, pw],
+                  normalization_term=mode >= 2, ignore_nan_input=mode == 3,
+                  out_of_bounds_value=float("nan") if mode == 3 else float(g.normal()))
+        try:
+            oh, ow = orc.similarity_out_dims(orc.similarity_args((B, C, H, W), O, **kw))
+        except ValueError:
+            continue
+        if B * O * C * bh * bw * oh * ow > 40_000_000:
+            continue
+        x = (2.0 + g.normal(size=(B, C, H, W))).astype(np.float32)
+        if mode == 3:
+            x[g.random(size=x.shape) < 0.2] = np.nan
+        t = (2.0 + g.normal(size=(O, C, bh, bw))).astype(np.float32)
+        w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+        return x, t, w, kw
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_similarity_matrix_gradient_random_geometry(pkg, seed):
+    g = np.random.default_rng(3000 + seed)
+    x, t, w, kw = random_matrix_gradient_case(g)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    go = g.normal(size=out.shape).astype(np.float32)
+    dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(go), **kw).cpu().numpy()
+    dt, dw = [a.cpu().numpy() for a in pkg.similarity_parameters_grad(dev(x), dev(t), dev(w), dev(go), **kw)]
+    d = f64(x, t, w, go)
+    want = orc.similarity_input_grad(x, t, w, go, **kw)
+    assert np.array_equal(np.isnan(dx), np.isnan(want)), kw
+    assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(orc.similarity_input_grad(*d, **kw)),
+                      "dX %s %s" % (x.shape, kw))
+    w32, w64 = orc.similarity_params_grad(x, t, w, go, **kw), orc.similarity_params_grad(*d, **kw)
+    assert_grad_close(dt, w32[0], w64[0], "dT %s" % kw)
+    assert_grad_close(np.nan_to_num(dw), np.nan_to_num(w32[1]), np.nan_to_num(w64[1]), "dW %s" % kw)
