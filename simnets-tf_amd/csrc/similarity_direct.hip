@@ -423,7 +423,7 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
 // quarter of every staged channel chunk, the partial sums are added through LDS in wave order at the end (so the
 // summation order over k is by quarters of a chunk, not strictly ascending).  Same LDS staging rule (out-of-image ->
 // out_of_bounds_value), same packed parameters and offset table, same combine step as the tiled kernel.
-template <int MODE>
+template <int MODE, bool GATED = false>
 __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKernelArgs a)
 {
     constexpr int PT = kSmallPT, MT = kSmallMT;
@@ -432,6 +432,12 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int flag_at = blockIdx.y * gridDim.x + blockIdx.x;   // sqrt-weight form: one flag per workgroup
+    if (GATED) {
+        const int SIMNETS_CONST_AS *fl = (const int SIMNETS_CONST_AS *)(a.flags);
+        if (fl[flag_at] == 0)
+            return;
+    }
     const int img_l = lane / a.gpi, g_l = lane - img_l * a.gpi;
     const int b0 = blockIdx.x * a.NI;
     const bool lane_valid = img_l < a.NI && b0 + img_l < a.B;
@@ -450,7 +456,7 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
 #pragma unroll
         for (int p = 0; p < PT; ++p)
             acc[m][p] = 0.0f;
-    const float *pa_t = a.pa + (size_t)mtile * a.K * MT * 2;
+    const float *pa_t = (GATED ? a.pa2 : a.pa) + (size_t)mtile * a.K * MT * 2;
     const float *pc_t = a.pc + (size_t)mtile * a.K * MT;
     const int SIMNETS_CONST_AS *koff = (const int SIMNETS_CONST_AS *)(a.koff);
 
@@ -562,7 +568,7 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
                 dst[(m * PT + p) * 64] = acc[m][p];
     }
     __syncthreads();
-    if (wave > 0 || !lane_valid)
+    if (wave > 0)
         return;
     for (int w = 1; w < kSmWaves; ++w) {
         const float *src = lds + (size_t)(w - 1) * kPart + lane;
@@ -572,10 +578,28 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
             for (int p = 0; p < PT; ++p)
                 acc[m][p] += src[(m * PT + p) * 64];
     }
+    const int w0 = gw * PT;
+    if (MODE == SIM_MODE_L2_SQRTW) {
+        // guard of the sqrt-weight form on the finished sums: a workgroup with an output below its template's
+        // threshold (or a template with a negative weight: threshold +inf) raises its flag and is recomputed
+        const float SIMNETS_CONST_AS *thr = (const float SIMNETS_CONST_AS *)(a.thr);
+        bool suspect = false;
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+            const float th = thr[min(mtile * MT + m, a.O - 1)];
+#pragma unroll
+            for (int p = 0; p < PT; ++p)
+                suspect |= lane_valid && mtile * MT + m < a.O && w0 + p < a.ow && !(acc[m][p] >= th);
+        }
+        const int bail = __any(suspect) ? 1 : 0;
+        if (lane == 0)
+            a.flags[flag_at] = bail;
+    }
+    if (!lane_valid)
+        return;
     int reps = 0;
     if (MODE == SIM_MODE_L2_NORM)
         reps = a.norm_every_iteration ? (a.B - b) : 1;
-    const int w0 = gw * PT;
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int mm = mtile * MT + m;
@@ -584,7 +608,7 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
         float *o = a.out + (((size_t)b * a.O + mm) * a.oh + h) * a.ow + w0;
 #pragma unroll
         for (int p = 0; p < PT; ++p) {
-            float v = acc[m][p];
+            float v = MODE == SIM_MODE_L2_SQRTW ? 0.0f - acc[m][p] : acc[m][p];
             for (int r = 0; r < reps; ++r)
                 v += a.norm_const;
             if (w0 + p < a.ow)
@@ -851,7 +875,7 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     if (t.NI > 0) {
         dim3 grid((unsigned)((a.B + t.NI - 1) / t.NI), (unsigned)a.n_mtiles);
         const size_t floats = std::max<size_t>((size_t)t.CC * t.chan_pitch, (size_t)(kSmWaves - 1) * kSmallMT * kSmallPT * 64);
-        hipLaunchKernelGGL((sim_small_map_kernel<MODE>), grid, dim3(kSmThreads), floats * sizeof(float), s, a);
+        hipLaunchKernelGGL((sim_small_map_kernel<MODE, GATED>), grid, dim3(kSmThreads), floats * sizeof(float), s, a);
         return hipGetLastError();
     }
     const int nwm = kWaves / a.nws;
@@ -866,12 +890,19 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     return launch_direct<MODE, kSmallPT, kSmallMT, GATED, false>(a, grid, lds_bytes, s);
 }
 
-// the sqrt-weight form runs on the tiled kernel only
-bool use_sqrtw(const SimPlan &p, const Tiling &t) { return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && t.NI == 0; }
+// The sqrt-weight form runs on the tiled kernels and on the small-map kernel; there only with enough pixels per
+// parameter, or packing the second copy of the parameters costs more than the shorter inner loop saves.
+bool use_sqrtw(const SimPlan &p, const Tiling &t)
+{
+    return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && (t.NI == 0 || (long long)p.B * p.oh * p.ow >= 4096);
+}
 
+// flags of the guard: one per wave of the tiled kernels' grid, one per workgroup of the small-map kernel's
 long long guard_flags(const SimPlan &p, const Tiling &t)
 {
     const int n_mtiles = (p.O + t.MT - 1) / t.MT, nwm = kWaves / t.nws;
+    if (t.NI > 0)
+        return (long long)((p.B + t.NI - 1) / t.NI) * n_mtiles;
     return (long long)p.B * t.tiles * ((n_mtiles + nwm - 1) / nwm) * kWaves;
 }
 

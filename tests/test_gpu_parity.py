@@ -129,6 +129,8 @@ def test_similarity_sqrtw_algorithm_matches_direct(pkg):
     dict(shape=(3, 6, 40, 40), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # 16 x 8 lane tiles
     dict(shape=(2, 5, 17, 13), O=19, blocks=[3, 2], strides=[2, 1], padding=[0, 1]),     # 4 x 8 lane tiles, ragged
     dict(shape=(2, 3, 9, 50), O=9, blocks=[2, 2], strides=[1, 2], padding=[1, 0], out_of_bounds_value=0.75),
+    dict(shape=(9, 6, 7, 7), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),       # small maps: images share a wave,
+    dict(shape=(5, 8, 6, 9), O=19, blocks=[2, 3], strides=[1, 1], padding=[0, 1]),       # one guard flag per workgroup
 ])
 @pytest.mark.parametrize("kind", ["exact", "near", "negative_weights", "nan_input", "all_zero"])
 def test_similarity_l2_default_form_recomputes_outputs_near_zero(pkg, geom, kind):
