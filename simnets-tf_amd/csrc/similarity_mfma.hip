@@ -182,7 +182,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     pm += 2 * step_stride;
 
     GroupedTile<kStagePos> gt;
-    gt.template init<kThreads>(a.H, a.W, TR, g.TC, in_row0, g.pw, g.NI, nimg, a.C * a.H * a.W, g.chan_lds, g.CC);
+    gt.template init<kThreads>(a.H, a.W, TR, g.TC, in_row0, g.pw, g.NI, nimg, multi ? a.C * a.H * a.W : 0, g.chan_lds, g.CC);
 
     // this workgroup's chunks of the image channels (all of them unless the input gradient is split)
     int ch_first = 0, ch_end = a.C;
@@ -687,6 +687,10 @@ MfmaTiling mfma_tiling(const SimPlan &p)
     cc_max = std::min(cc_max, (p.C + 1) & ~1);
     const int chunks = (p.C + cc_max - 1) / cc_max;
     t.CC = ((p.C + chunks - 1) / chunks + 1) & ~1;
+    // the staging addresses a group of channels (and the images of a tile) with 32-bit offsets
+    const long long group = std::max<long long>(1, std::min<long long>(kStagePos * kThreads / std::max<long long>(per_chan, 1), t.CC));
+    if ((group + 1) * p.H * p.W + (t.NI > 1 ? 1LL * t.NI * p.C * p.H * p.W : 0) >= (1LL << 31))
+        t.ok = false;
     // two steps of slack: the parameter loads run two steps ahead
     t.pm_floats = (size_t)(t.steps + 2) * 4 * t.Opad;
     return t;
@@ -887,6 +891,10 @@ StrideTiling stride_tiling(const SimPlan &p)
     cc_max = std::min(cc_max, (p.O + 1) & ~1);
     const int chunks = (p.O + cc_max - 1) / cc_max;
     q.CC = ((p.O + chunks - 1) / chunks + 1) & ~1;
+    // the staging addresses a group of channels with 32-bit offsets
+    const long long group = std::max<long long>(1, std::min<long long>(kStagePos * kThreads / (1LL * TRmax * q.TC), q.CC));
+    if ((group + 1) * p.oh * p.ow >= (1LL << 31))
+        return t;
     for (int i = 0; i < p.bh; ++i)
         for (int j = 0; j < p.bw; ++j) {
             int ry, dy, rx, dx;
