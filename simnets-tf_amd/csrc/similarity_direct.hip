@@ -37,7 +37,8 @@ namespace {
 constexpr int kWaves = 4;                 // waves per workgroup
 constexpr int kThreads = 64 * kWaves;
 constexpr int kLdsBudgetFloats = 16384;   // 64 KiB of input tile per workgroup
-constexpr int kSmWaves = 4, kSmThreads = 64 * kSmWaves;   // the small-map kernel's workgroup (eight waves measured slower)
+constexpr int kSmWaves = 4;   // the small-map kernel's workgroup: four waves, eight when the grid would otherwise give the
+                              // SIMDs at most one wave each (with more waves in the grid, eight measured slower)
 constexpr int kStagePos = 6;              // tile elements per thread and channel (a channel's tile holds at most
                                           // kStagePos * kThreads floats; larger geometries use the gather kernel)
 constexpr int kStageChan = 6;             // channels whose loads are in flight at once while staging
@@ -125,6 +126,7 @@ __device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT]
 #endif
 constexpr int kBigPT = SIMNETS_BIG_PT, kBigMT = SIMNETS_BIG_MT;
 constexpr int kSmallPT = 4, kSmallMT = 8;
+constexpr int kSmStageGroups = 2;   // small-map kernel: channel groups whose loads are in flight at once while staging
 // waves per SIMD the register budget is sized for: 64 accumulators leave room for 4, 128 for 2
 constexpr int waves_per_simd(int pt, int mt) { return pt * mt <= 64 ? 4 : 2; }
 constexpr int lds_budget_floats(int pt, int mt) { return pt * mt <= 64 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
@@ -423,9 +425,10 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
 // quarter of every staged channel chunk, the partial sums are added through LDS in wave order at the end (so the
 // summation order over k is by quarters of a chunk, not strictly ascending).  Same LDS staging rule (out-of-image ->
 // out_of_bounds_value), same packed parameters and offset table, same combine step as the tiled kernel.
-template <int MODE, bool GATED = false>
-__global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKernelArgs a)
+template <int MODE, bool GATED = false, int WAVES = kSmWaves>
+__global__ __launch_bounds__(64 * WAVES) void sim_small_map_kernel(const SimKernelArgs a)
 {
+    constexpr int kSmThreads = 64 * WAVES;
     constexpr int PT = kSmallPT, MT = kSmallMT;
     constexpr int NP = 4;   // tile elements per thread and channel the fast staging covers (NP * 256 per channel)
     extern __shared__ float lds[];
@@ -460,44 +463,21 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
     const float *pc_t = a.pc + (size_t)mtile * a.K * MT;
     const int SIMNETS_CONST_AS *koff = (const int SIMNETS_CONST_AS *)(a.koff);
 
-    // where this thread's tile elements of a channel come from: every channel of a chunk has the same geometry
+    // where this thread's tile elements come from: its NP elements span a group of channels (every group of a chunk
+    // has the same geometry), several groups are in flight at once
     const bool fast = chan_lds <= NP * kSmThreads;
-    long long gofs[NP];   // offset from the image block's channel plane; -1: outside the image, -2: no such element
-#pragma unroll
-    for (int j = 0; j < NP; ++j) {
-        const int pos = tid + j * kSmThreads;
-        const int pc = min(pos, chan_lds - 1);
-        const int im = (int)fast_div((unsigned)pc, a.d_img), r2 = pc - im * a.img_lds;
-        const int r = (int)fast_div((unsigned)r2, a.d_tc), c = r2 - r * a.TC;
-        const int ih = r - a.ph, iw = c - a.pw, bb = b0 + im;
-        gofs[j] = -1;
-        if (bb < a.B && ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
-            gofs[j] = (long long)bb * a.C * (long long)plane + (long long)ih * a.W + iw;
-        if (pos >= chan_lds)
-            gofs[j] = -2;
-    }
+    GroupedTile<NP> gt;
+    if (fast)
+        gt.template init<kSmThreads>(a.H, a.W, a.img_lds / a.TC, a.TC, -a.ph, a.pw, a.NI, min(a.NI, a.B - b0),
+                                     a.C * a.H * a.W, chan_lds, a.CC);
 
     for (int ch0 = 0; ch0 < a.C; ch0 += a.CC) {
         const int ccn = min(a.CC, a.C - ch0);
         __syncthreads();
         // ---- the chunk's tile ----
         if (fast) {
-            for (int cc0 = 0; cc0 < ccn; cc0 += 4) {
-                float v[4][NP];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float *chan = a.in + (size_t)(ch0 + min(cc0 + i, ccn - 1)) * plane;
-#pragma unroll
-                    for (int j = 0; j < NP; ++j)
-                        v[i][j] = gofs[j] >= 0 ? chan[gofs[j]] : a.oob;
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i)
-#pragma unroll
-                    for (int j = 0; j < NP; ++j)
-                        if (cc0 + i < ccn && gofs[j] != -2)
-                            lds[(cc0 + i) * chan_lds + tid + j * kSmThreads] = v[i][j];
-            }
+            gt.template stage<kSmStageGroups>(lds, a.in + ((size_t)b0 * a.C + ch0) * plane, (int)plane, ccn, ccn, chan_lds,
+                                              a.oob, nullptr);
         } else {
             const int total = ccn * chan_lds;
             for (int idx = tid; idx < total; idx += kSmThreads) {
@@ -512,48 +492,65 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
             }
         }
         __syncthreads();
-        const int cpw = (ccn + kSmWaves - 1) / kSmWaves;
+        const int cpw = (ccn + WAVES - 1) / WAVES;
         const int c_lo = min(wave * cpw, ccn), c_hi = min(c_lo + cpw, ccn);
         const int kl0 = c_lo * taps, nk = (c_hi - c_lo) * taps;   // this wave's steps, counted inside the chunk
-        // Software pipeline: the pixel values (LDS) and the parameters of step j + 1 are requested before the
-        // arithmetic of step j, two register sets.  The parameters come through scalar loads (one s_load_dwordx16
-        // per step) and are moved to VGPRs once per step by the combine (sim_step without VP): on this narrow tile a
-        // step has only 64-96 VALU instructions, and four lane-uniform vector or LDS loads per step - 16 / 8 cycles of
-        // the compute unit's one texture / LDS pipe each, shared by its four SIMDs - would bound the loop.
+        // Software pipeline: the pixel values (LDS) and the parameters of the next U steps are requested before the
+        // arithmetic of the current U, two register sets.  The parameters come through scalar loads (one
+        // s_load_dwordx16 per step) and are moved to VGPRs once per step by the combine (sim_step without VP): on this
+        // narrow tile a step has only 64-96 VALU instructions, and four lane-uniform vector or LDS loads per step -
+        // 16 / 8 cycles of the compute unit's one texture / LDS pipe each, shared by its four SIMDs - would bound the
+        // loop (a coalesced vector load per eight steps with the values taken out of the lanes by v_readlane measured
+        // slower as well: 0.53 against 0.44 ms on 512x7x7 at batch 32).  Scalar loads return in any order, so the wait
+        // is for all of them: two steps per wait (where the scalar registers allow it: the modes without a
+        // per-template constant) double the time a load has to arrive.
+        constexpr int U = (MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN) ? 1 : 2;
         if (nk > 0) {
             const int kg0 = ch0 * taps + kl0;   // this wave's first step, counted over all K
             const int SIMNETS_CONST_AS *kt = koff + kg0;
             const float SIMNETS_CONST_AS *pw = (const float SIMNETS_CONST_AS *)(pa_t) + (size_t)kg0 * (2 * MT);
             const float SIMNETS_CONST_AS *pq = (const float SIMNETS_CONST_AS *)(pc_t) + (size_t)kg0 * MT;
-            float x0[PT], x1[PT], pa0[2 * MT], pa1[2 * MT], pc0[MT], pc1[MT];
-            {
-                const int off0 = kt[0];
+            float x0[U][PT], x1[U][PT], pa0[U][2 * MT], pa1[U][2 * MT], pc0[U][MT], pc1[U][MT];
+            int offn[U];   // LDS offsets of the steps the next fetch reads (steps beyond the wave's last repeat it)
 #pragma unroll
-                for (int p = 0; p < PT; ++p)
-                    x0[p] = lds[lds_base + off0 + p * a.sw];
-            }
-            load_params<MODE, MT>(pa0, pc0, pw, pq);
-            int off_next = kt[1];   // (the table has two entries of slack, the packed arrays one step)
-            auto step = [&](int j, const float (&xc)[PT], const float (&pac)[2 * MT], const float (&pcc)[MT],
-                            float (&xn)[PT], float (&pan)[2 * MT], float (&pcn)[MT]) {
-                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): issued a whole step ago
-                __builtin_amdgcn_sched_barrier(0);
+            for (int u = 0; u < U; ++u)
+                offn[u] = kt[min(u, nk - 1)];
+            auto fetch = [&](int j, float (&xs)[U][PT], float (&pas)[U][2 * MT], float (&pcs)[U][MT]) {
 #pragma unroll
-                for (int p = 0; p < PT; ++p)
-                    xn[p] = lds[lds_base + off_next + p * a.sw];
-                off_next = kt[j + 2];
-                load_params<MODE, MT>(pan, pcn, pw + (size_t)(j + 1) * (2 * MT), pq + (size_t)(j + 1) * MT);
-                __builtin_amdgcn_sched_barrier(0);
-                sim_step<MODE, PT, MT, false>(acc, xc, pac, pcc);
-                __builtin_amdgcn_sched_barrier(0);
+                for (int u = 0; u < U; ++u) {
+                    const int jj = min(j + u, nk - 1);
+#pragma unroll
+                    for (int p = 0; p < PT; ++p)
+                        xs[u][p] = lds[lds_base + offn[u] + p * a.sw];
+                    load_params<MODE, MT>(pas[u], pcs[u], pw + (size_t)jj * (2 * MT), pq + (size_t)jj * MT);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    offn[u] = kt[min(j + U + u, nk - 1)];
             };
-            int j = 0;
-            for (; j + 2 <= nk; j += 2) {
-                step(j, x0, pa0, pc0, x1, pa1, pc1);
-                step(j + 1, x1, pa1, pc1, x0, pa0, pc0);
+            auto run = [&](int j, const float (&xs)[U][PT], const float (&pas)[U][2 * MT], const float (&pcs)[U][MT]) {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (j + u < nk)
+                        sim_step<MODE, PT, MT, false>(acc, xs[u], pas[u], pcs[u]);
+            };
+            fetch(0, x0, pa0, pc0);
+            for (int j = 0; j < nk; j += 2 * U) {
+                __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): issued a whole block of steps ago
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(j + U, x1, pa1, pc1);
+                __builtin_amdgcn_sched_barrier(0);
+                run(j, x0, pa0, pc0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (j + U >= nk)
+                    break;
+                __builtin_amdgcn_s_waitcnt(0xC07F);
+                __builtin_amdgcn_sched_barrier(0);
+                fetch(j + 2 * U, x0, pa0, pc0);
+                __builtin_amdgcn_sched_barrier(0);
+                run(j + U, x1, pa1, pc1);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            if (j < nk)
-                step(j, x0, pa0, pc0, x1, pa1, pc1);
         }
     }
     // ---- partial sums of waves 1..3 -> wave 0, in wave order; the tile's LDS is reused ----
@@ -570,7 +567,7 @@ __global__ __launch_bounds__(kSmThreads) void sim_small_map_kernel(const SimKern
     __syncthreads();
     if (wave > 0)
         return;
-    for (int w = 1; w < kSmWaves; ++w) {
+    for (int w = 1; w < WAVES; ++w) {
         const float *src = lds + (size_t)(w - 1) * kPart + lane;
 #pragma unroll
         for (int m = 0; m < MT; ++m)
@@ -742,6 +739,7 @@ __global__ __launch_bounds__(256) void sim_pack_params_kernel(const float *__res
 struct Tiling {
     int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
     int NI;            // > 0: the small-map kernel with NI images per workgroup (CC, chan_pitch are then that kernel's)
+    int sm_waves;      // ... and its waves per workgroup
     int chan_pitch;    // LDS floats of one staged channel
     bool lds_ok;       // the rows of a workgroup's pixel groups fit the LDS tile (else: gather kernel)
     bool fast_stage;   // ... and the division-free staging (at most kStagePos elements per thread and channel)
@@ -818,12 +816,15 @@ Tiling choose_tiling(const SimPlan &p)
         if ((NI >= 2 || waves(t) <= 1024) && per_chan <= kSmallMapLdsFloats) {
             t.NI = NI;
             t.chan_pitch = (int)per_chan;
+            const int n_mtiles = (p.O + t.MT - 1) / t.MT;
+            const long long wgs = (long long)((p.B + NI - 1) / NI) * n_mtiles;
+            t.sm_waves = (wgs * kSmWaves <= 1024 && p.C >= 2 * kSmWaves) ? 2 * kSmWaves : kSmWaves;
             const int cc_max = (int)std::min<long long>(p.C, kSmallMapLdsFloats / per_chan);
             const int chunks = (p.C + cc_max - 1) / cc_max;
             t.CC = (p.C + chunks - 1) / chunks;
             // the waves of the workgroup split a chunk's channels: a multiple of their number keeps them even
-            if (t.CC >= kSmWaves && t.CC % kSmWaves)
-                t.CC = t.CC / kSmWaves * kSmWaves;
+            if (t.CC >= t.sm_waves && t.CC % t.sm_waves)
+                t.CC = t.CC / t.sm_waves * t.sm_waves;
         }
     }
     return t;
@@ -874,8 +875,13 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     }
     if (t.NI > 0) {
         dim3 grid((unsigned)((a.B + t.NI - 1) / t.NI), (unsigned)a.n_mtiles);
-        const size_t floats = std::max<size_t>((size_t)t.CC * t.chan_pitch, (size_t)(kSmWaves - 1) * kSmallMT * kSmallPT * 64);
-        hipLaunchKernelGGL((sim_small_map_kernel<MODE, GATED>), grid, dim3(kSmThreads), floats * sizeof(float), s, a);
+        const size_t floats = std::max<size_t>((size_t)t.CC * t.chan_pitch, (size_t)(t.sm_waves - 1) * kSmallMT * kSmallPT * 64);
+        if (t.sm_waves == kSmWaves)
+            hipLaunchKernelGGL((sim_small_map_kernel<MODE, GATED, kSmWaves>), grid, dim3(64 * kSmWaves),
+                               floats * sizeof(float), s, a);
+        else
+            hipLaunchKernelGGL((sim_small_map_kernel<MODE, GATED, 2 * kSmWaves>), grid, dim3(128 * kSmWaves),
+                               floats * sizeof(float), s, a);
         return hipGetLastError();
     }
     const int nwm = kWaves / a.nws;

@@ -321,6 +321,8 @@ SMALL_MAPS = [
     dict(shape=(3, 37, 14, 14), O=40, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),      # one image per wave, K split only
     dict(shape=(2, 16, 13, 9), O=8, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),        # stride 2
     dict(shape=(70, 6, 3, 3), O=5, blocks=[3, 3], strides=[1, 1], padding=[0, 0]),         # 1 x 1 outputs: 64 images per wave
+    dict(shape=(64, 9, 7, 7), O=132, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),       # 272 workgroups: four waves each
+                                                                                           # (smaller grids above: eight)
 ]
 
 
