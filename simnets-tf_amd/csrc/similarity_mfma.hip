@@ -368,7 +368,15 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(cons
 
     // parameter operand: [step][type][half][Cpad] in the order of use (chunk, tap, template pair)
     const int step_stride = 4 * a.Opad;
-    const float *pm = a.pm + half * a.Opad + mbase + col;
+    // this workgroup's chunks of the output gradient's channels (all of them unless the contraction is split)
+    const int split = blockIdx.z;
+    int ch_first = 0, ch_end = a.C;
+    if (a.nsplit > 1) {
+        const int nchunks = (a.C + q.CC - 1) / q.CC;
+        ch_first = split * nchunks / a.nsplit * q.CC;
+        ch_end = min(a.C, (split + 1) * nchunks / a.nsplit * q.CC);
+    }
+    const float *pm = a.pm + half * a.Opad + mbase + col + (size_t)(ch_first / 2) * q.T * step_stride;
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
     float pa[kPmAhead], pb[kPmAhead];
 #pragma unroll
@@ -380,7 +388,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(cons
     GroupedTile<kStagePos> gt;
     gt.template init<kThreads>(a.H, a.W, TR, q.TC, h_first + q.row_min, -q.col_min, 1, 1, 0, q.chan_lds, q.CC);
 
-    for (int ch0 = 0; ch0 < a.C; ch0 += q.CC) {
+    for (int ch0 = ch_first; ch0 < ch_end; ch0 += q.CC) {
         const int ccn = min(q.CC, a.C - ch0);
         const int ccp = (ccn + 1) & ~1;
         __syncthreads();
@@ -452,7 +460,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(cons
     // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel per phase ----
     const size_t xplane = (size_t)a.x_plane;
     const int x_h = a.x_plane / a.x_w;
-    float *ob = a.out + (size_t)b * a.x_channels * xplane;
+    float *ob = (a.nsplit > 1 ? a.part + split * a.part_stride : a.out) + (size_t)b * a.x_channels * xplane;
     const float *xb = a.x + (size_t)b * a.x_channels * xplane;
 #pragma unroll
     for (int f = 0; f < NPH; ++f) {
@@ -909,6 +917,16 @@ StrideTiling stride_tiling(const SimPlan &p)
     return t;
 }
 
+// The same split for the kernel that interleaves the stride phases.
+int stride_split(const SimPlan &p, const StrideTiling &st)
+{
+    const long long wgs = (long long)p.B * st.q.tiles * (st.Cpad / (WG_TPL / 2));
+    const int nchunks = (p.O + st.q.CC - 1) / st.q.CC;
+    if (wgs >= 256)
+        return 1;
+    return (int)std::max<long long>(1, std::min<long long>(std::min(nchunks, 16), (512 + wgs - 1) / wgs));
+}
+
 // Workgroups along blockIdx.x of one phase's grid.
 unsigned grad_phase_blocks(const SimPlan &p, const GradPhase &g)
 {
@@ -956,8 +974,11 @@ bool sim_mfma_grad_input_supported(const SimPlan &p)
 size_t sim_mfma_grad_input_workspace_bytes(const SimPlan &p)
 {
     const StrideTiling st = stride_tiling(p);
-    if (st.ok)
-        return align_up((size_t)p.C * sizeof(float), 256) + align_up(st.pm_floats * sizeof(float), 256);
+    if (st.ok) {
+        const int nsplit = stride_split(p, st);
+        return align_up((size_t)p.C * sizeof(float), 256) + align_up(st.pm_floats * sizeof(float), 256) +
+               (nsplit > 1 ? align_up((size_t)nsplit * p.B * p.C * p.H * p.W * sizeof(float), 256) : 0);
+    }
     std::vector<GradPhase> ph;
     grad_phases(p, ph);
     size_t bytes = align_up((size_t)p.C * sizeof(float), 256);
@@ -992,11 +1013,19 @@ int sim_mfma_grad_input_launch(const SimPlan &p, const float *input, const float
         a.x = input; a.x_channels = p.C; a.ignore_nan = p.mode == SIM_MODE_L2_NORM_IGNORE_NAN;
         a.oys = p.sh; a.oxs = p.sw; a.x_w = p.W; a.x_plane = p.H * p.W;
         a.B = p.B; a.C = p.O; a.H = p.oh; a.W = p.ow; a.O = p.C; a.Opad = st.Cpad;
-        dim3 grid((unsigned)(p.B * st.q.tiles), (unsigned)(st.Cpad / (WG_TPL / 2)));
+        const long long n_in = (long long)p.B * p.C * p.H * p.W;
+        a.nsplit = stride_split(p, st);
+        a.part = reinterpret_cast<float *>(ws + align_up((size_t)p.C * sizeof(float), 256) +
+                                           align_up(st.pm_floats * sizeof(float), 256));
+        a.part_stride = n_in;
+        dim3 grid((unsigned)(p.B * st.q.tiles), (unsigned)(st.Cpad / (WG_TPL / 2)), (unsigned)a.nsplit);
         if (st.nph == 4)
             hipLaunchKernelGGL(sim_mfma_grad_strided_kernel<4>, grid, dim3(kThreads), st.lds_bytes, s, a, st.q);
         else
             hipLaunchKernelGGL(sim_mfma_grad_strided_kernel<2>, grid, dim3(kThreads), st.lds_bytes, s, a, st.q);
+        if (a.nsplit > 1)
+            hipLaunchKernelGGL(mfma_sum_parts_kernel, dim3((unsigned)std::min<long long>((n_in + 1023) / 1024, 4096)),
+                               dim3(256), 0, s, a.part, a.nsplit, n_in, input_grad);
         return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
     }
     std::vector<GradPhase> phases;

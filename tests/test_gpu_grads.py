@@ -502,6 +502,8 @@ def test_similarity_params_grad_row_staged_matrix_form(pkg, case, func, norm, ig
     dict(shape=(3, 30, 5, 9), O=64, blocks=[2, 3], padding=[1, 2]),       # 45 pixels: one group of 3 images
     dict(shape=(1, 64, 20, 20), O=300, blocks=[3, 3], padding=[1, 1]),    # two pixel tiles, contraction split 11 ways
     dict(shape=(6, 24, 9, 10), O=90, blocks=[3, 3], padding=[1, 1], strides=[3, 3]),    # small phase grids, split
+    dict(shape=(2, 24, 10, 11), O=300, blocks=[3, 3], padding=[1, 1], strides=[2, 2]),  # interleaved phases, split
+    dict(shape=(1, 32, 12, 40), O=260, blocks=[2, 4], padding=[1, 0], strides=[1, 2]),  # two phases, split
 ])
 def test_similarity_input_grad_matrix_form(pkg, case, func, norm, ign):
     """At least 24 channels, strides no larger than the window: the L2 modes' input gradient is A - (x - c) B with
