@@ -66,6 +66,8 @@ struct GradXArgs {
     int ignore_nan;
     int fast_stage;    // the g tile of a channel has at most kStagePos * kThreads elements: division-free staging
     int row_limit, col_limit;  // phase rows h <= row_limit (columns v <= col_limit) are covered by a window
+    int NI;            // small phase grids (MULTI variant): a wave covers NI images (lane -> image, pixel group); their
+                       // g tiles sit side by side in a channel's LDS slot
 };
 
 template <int MODE, int PT, int MT>
@@ -108,7 +110,8 @@ __device__ __forceinline__ void gx_step(float (&acc)[MT][PT], const float (&xv)[
 constexpr int gx_waves_per_simd(int pt, int mt) { return pt * mt <= 32 ? 3 : 2; }
 constexpr int gx_lds_budget(int pt, int mt) { return pt * mt <= 32 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
 
-template <int MODE, int PT, int MT>
+// MULTI: small phase grids, a wave covers a.NI images.
+template <int MODE, int PT, int MT, bool MULTI = false>
 __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_input_kernel(const GradXArgs a)
 {
     extern __shared__ float lds[];
@@ -116,11 +119,13 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    const int b = blockIdx.x / a.tiles;
-    const int tile = blockIdx.x - b * a.tiles;
-    const int ws = wave & (a.nws - 1);
-    const int wm = wave >> a.nws_log2;
-    const int nwm = kWaves >> a.nws_log2;
+    constexpr bool multi = MULTI;
+    const int b0 = multi ? blockIdx.x * a.NI : blockIdx.x / a.tiles;
+    const int tile = multi ? 0 : blockIdx.x - b0 * a.tiles;
+    // (MULTI: the four waves of a workgroup share one channel tile and split the steps of every chunk)
+    const int ws = multi ? 0 : wave & (a.nws - 1);
+    const int wm = multi ? 0 : wave >> a.nws_log2;
+    const int nwm = multi ? 1 : kWaves >> a.nws_log2;
     const int ctile = blockIdx.y * nwm + wm;
     const bool wave_active = ctile < a.n_ctiles;
 
@@ -131,12 +136,15 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
     const int TR = nrows - 1 + a.nI;
     const int in_row0 = row_first - a.padh;
 
-    int grp = g_first + ws * 64 + lane;
-    const bool lane_valid = grp <= g_last;
+    // this lane's pixel group: of image b0 (a tile of its groups), or - small grids - of image b0 + lane / gpi
+    const int img_l = multi ? lane / a.gpi : 0;
+    int grp = multi ? lane - img_l * a.gpi : g_first + ws * 64 + lane;
+    const bool lane_valid = multi ? (img_l < a.NI && b0 + img_l < a.B) : grp <= g_last;
     grp = min(grp, g_last);
+    const int b = lane_valid ? b0 + img_l : b0;
     const int h = grp / a.G;
     const int gw = grp - h * a.G;
-    const int lds_base = (h - row_first) * a.TC + gw * PT;
+    const int lds_base = (lane_valid ? img_l : 0) * (TR * a.TC) + (h - row_first) * a.TC + gw * PT;
     const int v0 = gw * PT;
 
     // the X values of this lane's tile (NaN -> 0 when NaN inputs are ignored: their gradient is 0)
@@ -172,18 +180,25 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
         }
         pb_off += 2 * MT * sizeof(float);
     };
-    const float *img = a.g + (size_t)b * a.O * a.oh * a.ow;
-    const int chan_lds = a.TRmax * a.TC;
+    const float *img = a.g + (size_t)b0 * a.O * a.oh * a.ow;
+    const int chan_lds = (multi ? a.NI : 1) * a.TRmax * a.TC;
     float pb0[2 * MT], pb1[2 * MT];
     fetch_params(pb0);
-    TilePositions<kStagePos> tp;
-    tp.template init<kThreads>(a.oh, a.ow, TR, a.TC, in_row0, a.padw);
+    TilePositions<multi ? 1 : kStagePos> tp;
+    GroupedTile<multi ? kStagePos : 1> gt;
+    if constexpr (multi)
+        gt.template init<kThreads>(a.oh, a.ow, TR, a.TC, in_row0, a.padw, a.NI, min(a.NI, a.B - b0), a.O * a.oh * a.ow,
+                                   chan_lds, a.CC);
+    else
+        tp.template init<kThreads>(a.oh, a.ow, TR, a.TC, in_row0, a.padw);
     const int SIMNETS_CONST_AS *kt = (const int SIMNETS_CONST_AS *)(a.koff);
 
     for (int ch0 = 0; ch0 < a.O; ch0 += a.CC) {
         const int ccn = min(a.CC, a.O - ch0);
         __syncthreads();
-        if (a.fast_stage)
+        if constexpr (multi)
+            gt.template stage<1>(lds, img + (size_t)ch0 * a.oh * a.ow, a.oh * a.ow, ccn, ccn, chan_lds, 0.0f, nullptr);
+        else if (a.fast_stage)
             stage_input_tile_fast<kStagePos, kStageChan>(lds, img, a.oh, a.ow, ch0, ccn, ccn, chan_lds, 0.0f, nullptr, tp);
         else
             stage_input_tile<kThreads, 8>(lds, img, a.oh, a.ow, ch0, ccn, ccn, TR, a.TC, chan_lds, in_row0, a.padw, 0.0f,
@@ -193,7 +208,18 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
             continue;
         // software pipeline over the (o, tap) steps of this chunk: the g values and the parameters of
         // the next step are requested before the arithmetic of the current one
-        const int nk = ccn * a.nI * a.nJ;
+        int nk = ccn * a.nI * a.nJ;
+        if constexpr (multi) {
+            // this wave's quarter of the chunk's templates
+            const int taps = a.nI * a.nJ;
+            const int cpw = (ccn + kWaves - 1) / kWaves;
+            const int c_lo = min(wave * cpw, ccn), c_hi = min(c_lo + cpw, ccn);
+            const int k_first = (ch0 + c_lo) * taps;
+            nk = (c_hi - c_lo) * taps;
+            kt = (const int SIMNETS_CONST_AS *)(a.koff) + k_first;
+            pb_off = zero_v + (unsigned)k_first * (unsigned)(2 * MT * sizeof(float));
+            fetch_params(pb0);
+        }
         int off_next = kt[1];
         auto step = [&](const float (&gc)[PT], const float (&pbc)[2 * MT], float (&gnx)[PT], float (&pbnx)[2 * MT]) {
             __builtin_amdgcn_s_waitcnt(0xC07F);  // lgkmcnt(0): issued a whole step ago
@@ -228,6 +254,27 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
         }
     }
 
+    if constexpr (multi) {
+        // partial sums of waves 1..3 -> wave 0, in wave order; the tile's LDS is reused
+        constexpr int kPart = MT * PT * 64;
+        __syncthreads();
+        if (wave > 0) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    lds[(wave - 1) * kPart + (m * PT + p) * 64 + lane] = acc[m][p];
+        }
+        __syncthreads();
+        if (wave > 0)
+            return;
+        for (int w = 1; w < kWaves; ++w)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int p = 0; p < PT; ++p)
+                    acc[m][p] += lds[(w - 1) * kPart + (m * PT + p) * 64 + lane];
+    }
     if (!wave_active || !lane_valid)
         return;
     const bool row_covered = h <= a.row_limit;
@@ -382,6 +429,9 @@ Phase make_phase(const SimPlan &p, int ry, int rx)
 
 struct GxTiling {
     int PT, MT, nws, G, gpi, tiles, TC, TRmax, CC;
+    int NI;   // images per wave (small phase grids), else 1
+    bool ksplit;   // the variant for small grids: a wave covers NI >= 1 whole images, the four waves of a workgroup
+                   // share a channel tile and split the templates
     bool lds_ok, fast_stage;
 };
 
@@ -397,7 +447,20 @@ GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws)
     t.TC |= 1;
     const int max_rows = std::min(f.na, (64 * nws + t.G - 1) / t.G + 1);
     t.TRmax = max_rows - 1 + f.nI;
-    const long long per_chan = 1LL * t.TRmax * t.TC;
+    // a phase grid of at most 32 pixel groups: a wave takes several images
+    t.NI = 1;
+    if (nws == 1 && t.tiles == 1 && 2 * t.gpi <= 64 && p.B >= 2) {
+        int ni = std::min(64 / t.gpi, p.B);
+        while (ni > 1 && (1LL * ni * t.TRmax * t.TC > kStagePos * kThreads || 1LL * ni * t.TRmax * t.TC > budget ||
+                          1LL * ni * p.O * p.oh * p.ow >= (1LL << 31)))
+            --ni;
+        t.NI = ni;
+    }
+    // ... and so does a grid that would give the SIMDs at most one wave each (one image per wave then)
+    const long long plain_waves = (long long)p.B * (((p.C + t.MT - 1) / t.MT + kWaves - 1) / kWaves) * kWaves;
+    t.ksplit = t.NI > 1 || (nws == 1 && t.tiles == 1 && t.gpi <= 64 && plain_waves <= 1024 && p.O >= kWaves &&
+                            1LL * t.TRmax * t.TC <= kStagePos * kThreads);
+    const long long per_chan = 1LL * t.NI * t.TRmax * t.TC;
     t.lds_ok = per_chan <= budget;
     t.fast_stage = per_chan <= kStagePos * kThreads;
     t.CC = 1;
@@ -405,6 +468,9 @@ GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws)
         const int cc_max = (int)std::min<long long>(p.O, budget / per_chan);
         const int chunks = (p.O + cc_max - 1) / cc_max;
         t.CC = (p.O + chunks - 1) / chunks;
+        // several images per wave: the four waves split a chunk's templates, a multiple of four keeps them even
+        if (t.ksplit && t.CC > kWaves && t.CC % kWaves)
+            t.CC = t.CC / kWaves * kWaves;
     }
     return t;
 }
@@ -463,6 +529,13 @@ template <int MODE>
 hipError_t gx_launch_phase(const GradXArgs &a, const GxTiling &t, hipStream_t s)
 {
     const int nwm = kWaves / a.nws;
+    if (t.ksplit) {
+        // four waves per channel tile; the LDS also holds three waves' partial sums at the end
+        dim3 mgrid((unsigned)((a.B + a.NI - 1) / a.NI), (unsigned)a.n_ctiles);
+        const size_t floats = std::max<size_t>((size_t)a.CC * a.NI * a.TRmax * a.TC, (size_t)(kWaves - 1) * 8 * 4 * 64);
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8, true>), mgrid, dim3(kThreads), floats * sizeof(float), s, a);
+        return hipGetLastError();
+    }
     dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_ctiles + nwm - 1) / nwm));
     const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
     if (t.PT == 8)
@@ -543,7 +616,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
             hipLaunchKernelGGL(sim_grad_input_pack_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights,
                                p.O, p.C, p.bh, p.bw, p.sh, p.sw, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, (int)l1, scale,
-                               pb, koff, t.CC, t.TRmax * t.TC, t.TC);
+                               pb, koff, t.CC, t.NI * t.TRmax * t.TC, t.TC);
             if (hipGetLastError() != hipSuccess)
                 return SIMNETS_ERR_HIP;
 
@@ -561,6 +634,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             a.n_ctiles = n_ctiles; a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC;
             a.ignore_nan = ignore_nan;
             a.fast_stage = t.fast_stage;
+            a.NI = t.NI;
             // phase row h (a = a0 + h) is covered by some window iff a - (nI-1) <= oh-1
             a.row_limit = p.oh - 1 + f.nI - 1 - f.a0;
             a.col_limit = p.ow - 1 + f.nJ - 1 - f.b0;

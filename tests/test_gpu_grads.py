@@ -569,3 +569,25 @@ def test_mex_grads_in_one_call_equal_the_two_calls(pkg, case, normalize):
     do1 = pkg.mex_offsets_grad(X, O, Y, G, case["n"], **kw)
     assert torch.equal(do1, doff)
     assert torch.equal(dx1, dx)
+
+
+@pytest.mark.parametrize("func,norm,ign", [("L1", False, False), ("L2", False, False), ("L2", True, True)])
+@pytest.mark.parametrize("case", [
+    dict(shape=(9, 12, 7, 7), O=20, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),     # 14 pixel groups: 4 images a wave
+    dict(shape=(7, 5, 5, 6), O=33, blocks=[2, 3], strides=[1, 1], padding=[0, 2]),      # ragged image groups, odd sizes
+    dict(shape=(11, 40, 9, 8), O=9, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),     # stride phases of 5x4 pixels
+    dict(shape=(70, 3, 3, 3), O=6, blocks=[3, 3], strides=[1, 1], padding=[0, 0]),      # 3 groups an image: 21 images a wave
+])
+def test_similarity_input_grad_small_maps_share_a_wave(pkg, case, func, norm, ign):
+    """Phase grids of at most 32 pixel groups: a wave of the term-by-term input-gradient kernel covers several
+    images (L1 always takes that kernel; the L2 modes with fewer than 24 channels, or with algo='direct')."""
+    x, t, w = sim_inputs(77, case["shape"], case["O"], case["blocks"], nan_frac=0.15 if ign else 0.0)
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+              normalization_term=norm, ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else 0.25)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = np.random.default_rng(5).normal(size=out.shape).astype(np.float32)
+    want = orc.similarity_input_grad(x, t, w, og, **kw)
+    true = orc.similarity_input_grad(*f64(x, t, w, og), **kw)
+    dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), algo="direct", **kw).cpu().numpy()
+    assert np.array_equal(np.isnan(dx), np.isnan(want))
+    assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad")
