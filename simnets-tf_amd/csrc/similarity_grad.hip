@@ -26,6 +26,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <vector>
 #include <cmath>
 
 #include "internal.h"
@@ -68,6 +69,12 @@ struct GradXArgs {
     int row_limit, col_limit;  // phase rows h <= row_limit (columns v <= col_limit) are covered by a window
     int NI;            // small phase grids (MULTI variant): a wave covers NI images (lane -> image, pixel group); their
                        // g tiles sit side by side in a channel's LDS slot
+    int grid_x, grid_y;  // workgroups of this phase (a launch covers several phases: blockIdx.z)
+};
+
+constexpr int kGxMaxPhases = 16;   // stride phases per launch
+struct GradXPhases {
+    GradXArgs p[kGxMaxPhases];
 };
 
 template <int MODE, int PT, int MT>
@@ -112,8 +119,11 @@ constexpr int gx_lds_budget(int pt, int mt) { return pt * mt <= 32 ? kLdsBudgetF
 
 // MULTI: small phase grids, a wave covers a.NI images.
 template <int MODE, int PT, int MT, bool MULTI = false>
-__global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_input_kernel(const GradXArgs a)
+__global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_input_kernel(const GradXPhases phases)
 {
+    const GradXArgs &a = phases.p[blockIdx.z];
+    if ((int)blockIdx.x >= a.grid_x || (int)blockIdx.y >= a.grid_y)
+        return;   // a phase with fewer workgroups than the largest of the launch
     extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -360,13 +370,26 @@ __global__ void fill_zero_kernel(float *__restrict__ p, long long n)
         p[i] = 0.0f;
 }
 
-// Packs one phase's (template, weight) pairs as [ctile][k = (o, dh, dw)][MT][2] with the taps flipped
-// (dh = nI-1-ii, original tap i = ry + sh*ii) and the per-mode scaling folded in.
+// Packs the (template, weight) pairs of the stride phases (blockIdx.y) as [ctile][k = (o, dh, dw)][MT][2] with the
+// taps flipped (dh = nI-1-ii, original tap i = ry + sh*ii) and the per-mode scaling folded in.
+struct GxPackPhase {
+    float *pb;
+    int *koff;
+    int ry, rx, nI, nJ, MT, n_ctiles, CC, chan_pitch, TC;
+};
+struct GxPackPhases {
+    GxPackPhase p[kGxMaxPhases];
+};
+
 __global__ void sim_grad_input_pack_kernel(const float *__restrict__ templates, const float *__restrict__ weights,
-                                           int O, int C, int bh, int bw, int sh, int sw, int ry, int rx, int nI,
-                                           int nJ, int MT, int n_ctiles, int l1, float scale, float *__restrict__ pb,
-                                           int *__restrict__ koff, int CC, int chan_pitch, int TC)
+                                           int O, int C, int bh, int bw, int sh, int sw, int l1, float scale,
+                                           const GxPackPhases phases)
 {
+    const GxPackPhase &q = phases.p[blockIdx.y];
+    const int ry = q.ry, rx = q.rx, nI = q.nI, nJ = q.nJ, MT = q.MT, n_ctiles = q.n_ctiles, CC = q.CC;
+    const int chan_pitch = q.chan_pitch, TC = q.TC;
+    float *__restrict__ pb = q.pb;
+    int *__restrict__ koff = q.koff;
     const int K = O * nI * nJ;
     for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < K + 2; k += gridDim.x * blockDim.x) {
         int off = 0;
@@ -525,23 +548,29 @@ bool gx_all_phases_fit(const SimPlan &p)
     return true;
 }
 
+// One launch for the phases that share a kernel variant (lane tile, small-grid form).
 template <int MODE>
-hipError_t gx_launch_phase(const GradXArgs &a, const GxTiling &t, hipStream_t s)
+hipError_t gx_launch_phases(const GradXPhases &ph, int n, int PT, bool ksplit, hipStream_t s)
 {
-    const int nwm = kWaves / a.nws;
-    if (t.ksplit) {
-        // four waves per channel tile; the LDS also holds three waves' partial sums at the end
-        dim3 mgrid((unsigned)((a.B + a.NI - 1) / a.NI), (unsigned)a.n_ctiles);
-        const size_t floats = std::max<size_t>((size_t)a.CC * a.NI * a.TRmax * a.TC, (size_t)(kWaves - 1) * 8 * 4 * 64);
-        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8, true>), mgrid, dim3(kThreads), floats * sizeof(float), s, a);
-        return hipGetLastError();
+    unsigned gx = 1, gy = 1;
+    size_t lds_floats = 0;
+    for (int i = 0; i < n; ++i) {
+        const GradXArgs &a = ph.p[i];
+        gx = std::max(gx, (unsigned)a.grid_x);
+        gy = std::max(gy, (unsigned)a.grid_y);
+        size_t floats = (size_t)a.CC * std::max(a.NI, 1) * a.TRmax * a.TC;
+        if (ksplit)  // the LDS also holds three waves' partial sums at the end
+            floats = std::max<size_t>(floats, (size_t)(kWaves - 1) * 8 * 4 * 64);
+        lds_floats = std::max(lds_floats, floats);
     }
-    dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_ctiles + nwm - 1) / nwm));
-    const size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
-    if (t.PT == 8)
-        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 8, 8>), grid, dim3(kThreads), lds_bytes, s, a);
+    dim3 grid(gx, gy, (unsigned)n);
+    const size_t lds_bytes = lds_floats * sizeof(float);
+    if (ksplit)
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8, true>), grid, dim3(kThreads), lds_bytes, s, ph);
+    else if (PT == 8)
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 8, 8>), grid, dim3(kThreads), lds_bytes, s, ph);
     else
-        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8>), grid, dim3(kThreads), lds_bytes, s, ph);
     return hipGetLastError();
 }
 
@@ -598,6 +627,15 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             return SIMNETS_ERR_HIP;
     }
 
+    // the phases' arguments, grouped by kernel variant (lane tile, small-grid form): one pack launch and one main
+    // launch per group of at most kGxMaxPhases phases (ordinarily one group: the phase grids differ by a row or column)
+    struct Job {
+        GradXArgs a;
+        GxPackPhase q;
+        int PT;
+        bool ksplit;
+    };
+    std::vector<Job> jobs;
     char *ws = reinterpret_cast<char *>(workspace);
     for (int ry = 0; ry < p.sh; ++ry)
         for (int rx = 0; rx < p.sw; ++rx) {
@@ -612,15 +650,10 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             int *koff = reinterpret_cast<int *>(ws);
             ws += gx_phase_table_bytes(p, f);
 
-            const long long total = (long long)n_ctiles * (K + 1) * t.MT;
-            const int pack_blocks = (int)std::min<long long>((total + 255) / 256, 4096);
-            hipLaunchKernelGGL(sim_grad_input_pack_kernel, dim3(pack_blocks), dim3(256), 0, s, templates, weights,
-                               p.O, p.C, p.bh, p.bw, p.sh, p.sw, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, (int)l1, scale,
-                               pb, koff, t.CC, t.NI * t.TRmax * t.TC, t.TC);
-            if (hipGetLastError() != hipSuccess)
-                return SIMNETS_ERR_HIP;
-
-            GradXArgs a;
+            Job j;
+            j.PT = t.PT; j.ksplit = t.ksplit;
+            j.q = {pb, koff, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, t.CC, t.NI * t.TRmax * t.TC, t.TC};
+            GradXArgs &a = j.a;
             a.g = output_grad; a.x = input; a.dx = input_grad; a.pb = pb; a.koff = koff;
             a.B = p.B; a.C = p.C; a.H = p.H; a.W = p.W; a.O = p.O; a.oh = p.oh; a.ow = p.ow;
             a.nI = f.nI; a.nJ = f.nJ;
@@ -638,10 +671,37 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             // phase row h (a = a0 + h) is covered by some window iff a - (nI-1) <= oh-1
             a.row_limit = p.oh - 1 + f.nI - 1 - f.a0;
             a.col_limit = p.ow - 1 + f.nJ - 1 - f.b0;
-            const hipError_t e = l1 ? gx_launch_phase<GX_L1>(a, t, s) : gx_launch_phase<GX_L2>(a, t, s);
-            if (e != hipSuccess)
-                return SIMNETS_ERR_HIP;
+            const int nwm = kWaves / t.nws;
+            a.grid_x = t.ksplit ? (p.B + t.NI - 1) / t.NI : p.B * t.tiles;
+            a.grid_y = t.ksplit ? n_ctiles : (n_ctiles + nwm - 1) / nwm;
+            jobs.push_back(j);
         }
+    std::vector<bool> done(jobs.size(), false);
+    for (size_t first = 0; first < jobs.size(); ++first) {
+        if (done[first])
+            continue;
+        GradXPhases ph;
+        GxPackPhases pk;
+        int n = 0;
+        long long pack_total = 0;
+        for (size_t i = first; i < jobs.size() && n < kGxMaxPhases; ++i)
+            if (!done[i] && jobs[i].PT == jobs[first].PT && jobs[i].ksplit == jobs[first].ksplit) {
+                ph.p[n] = jobs[i].a;
+                pk.p[n] = jobs[i].q;
+                pack_total = std::max(pack_total, (long long)jobs[i].q.n_ctiles * (jobs[i].a.K + 1) * jobs[i].q.MT);
+                done[i] = true;
+                ++n;
+            }
+        const int pack_blocks = (int)std::min<long long>((pack_total + 255) / 256, 4096);
+        hipLaunchKernelGGL(sim_grad_input_pack_kernel, dim3(pack_blocks, n), dim3(256), 0, s, templates, weights, p.O, p.C,
+                           p.bh, p.bw, p.sh, p.sw, (int)l1, scale, pk);
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+        const hipError_t e = l1 ? gx_launch_phases<GX_L1>(ph, n, jobs[first].PT, jobs[first].ksplit, s)
+                                : gx_launch_phases<GX_L2>(ph, n, jobs[first].PT, jobs[first].ksplit, s);
+        if (e != hipSuccess)
+            return SIMNETS_ERR_HIP;
+    }
     return SIMNETS_OK;
 }
 
