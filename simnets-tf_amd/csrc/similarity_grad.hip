@@ -458,10 +458,10 @@ struct GxTiling {
     bool lds_ok, fast_stage;
 };
 
-GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws)
+GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws, int MT = 8)
 {
     GxTiling t;
-    t.PT = PT; t.MT = 8; t.nws = nws;
+    t.PT = PT; t.MT = MT; t.nws = nws;
     const int budget = gx_lds_budget(t.PT, t.MT);
     t.G = (f.nb + t.PT - 1) / t.PT;
     t.gpi = f.na * t.G;
@@ -481,7 +481,9 @@ GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws)
     }
     // ... and so does a grid that would give the SIMDs at most one wave each (one image per wave then)
     const long long plain_waves = (long long)p.B * (((p.C + t.MT - 1) / t.MT + kWaves - 1) / kWaves) * kWaves;
-    t.ksplit = t.NI > 1 || (nws == 1 && t.tiles == 1 && t.gpi <= 64 && plain_waves <= 1024 && p.O >= kWaves &&
+    if (MT != 8)
+        t.NI = 1;   // (the small-grid variant has the 4 x 8 lane tile)
+    t.ksplit = MT != 8 ? false : t.NI > 1 || (nws == 1 && t.tiles == 1 && t.gpi <= 64 && plain_waves <= 1024 && p.O >= kWaves &&
                             1LL * t.TRmax * t.TC <= kStagePos * kThreads);
     const long long per_chan = 1LL * t.NI * t.TRmax * t.TC;
     t.lds_ok = per_chan <= budget;
@@ -515,6 +517,18 @@ GxTiling gx_tiling(const SimPlan &p, const Phase &f)
         }
         return t;
     };
+    // Three or four channels (an image): 8 pixels x 4 channels per lane, all pixel waves on the one channel tile
+    if (p.C <= 4 && f.nb >= 16) {
+        const int gpi = f.na * ((f.nb + 7) / 8);
+        int nws = gpi >= 256 ? 4 : (gpi >= 128 ? 2 : 1);
+        GxTiling t = gx_try(p, f, 8, nws, 4);
+        while (nws > 1 && !(t.lds_ok && t.fast_stage)) {
+            nws >>= 1;
+            t = gx_try(p, f, 8, nws, 4);
+        }
+        if (t.lds_ok && !pick(4).ksplit)
+            return t;
+    }
     // 8 x 8 lane tile for wide phase grids with many channels, if the grid then still gives every SIMD two waves
     if (f.nb >= 32 && p.C >= 32) {
         const GxTiling big = pick(8);
@@ -550,7 +564,7 @@ bool gx_all_phases_fit(const SimPlan &p)
 
 // One launch for the phases that share a kernel variant (lane tile, small-grid form).
 template <int MODE>
-hipError_t gx_launch_phases(const GradXPhases &ph, int n, int PT, bool ksplit, hipStream_t s)
+hipError_t gx_launch_phases(const GradXPhases &ph, int n, int PT, int MT, bool ksplit, hipStream_t s)
 {
     unsigned gx = 1, gy = 1;
     size_t lds_floats = 0;
@@ -567,6 +581,8 @@ hipError_t gx_launch_phases(const GradXPhases &ph, int n, int PT, bool ksplit, h
     const size_t lds_bytes = lds_floats * sizeof(float);
     if (ksplit)
         hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 4, 8, true>), grid, dim3(kThreads), lds_bytes, s, ph);
+    else if (MT == 4)
+        hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 8, 4>), grid, dim3(kThreads), lds_bytes, s, ph);
     else if (PT == 8)
         hipLaunchKernelGGL((sim_grad_input_kernel<MODE, 8, 8>), grid, dim3(kThreads), lds_bytes, s, ph);
     else
@@ -632,7 +648,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
     struct Job {
         GradXArgs a;
         GxPackPhase q;
-        int PT;
+        int PT, MT;
         bool ksplit;
     };
     std::vector<Job> jobs;
@@ -651,7 +667,7 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
             ws += gx_phase_table_bytes(p, f);
 
             Job j;
-            j.PT = t.PT; j.ksplit = t.ksplit;
+            j.PT = t.PT; j.MT = t.MT; j.ksplit = t.ksplit;
             j.q = {pb, koff, ry, rx, f.nI, f.nJ, t.MT, n_ctiles, t.CC, t.NI * t.TRmax * t.TC, t.TC};
             GradXArgs &a = j.a;
             a.g = output_grad; a.x = input; a.dx = input_grad; a.pb = pb; a.koff = koff;
@@ -685,7 +701,8 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
         int n = 0;
         long long pack_total = 0;
         for (size_t i = first; i < jobs.size() && n < kGxMaxPhases; ++i)
-            if (!done[i] && jobs[i].PT == jobs[first].PT && jobs[i].ksplit == jobs[first].ksplit) {
+            if (!done[i] && jobs[i].PT == jobs[first].PT && jobs[i].MT == jobs[first].MT &&
+                jobs[i].ksplit == jobs[first].ksplit) {
                 ph.p[n] = jobs[i].a;
                 pk.p[n] = jobs[i].q;
                 pack_total = std::max(pack_total, (long long)jobs[i].q.n_ctiles * (jobs[i].a.K + 1) * jobs[i].q.MT);
@@ -697,8 +714,8 @@ int sim_grad_input(const SimPlan &p, const float *input, const float *templates,
                            p.bh, p.bw, p.sh, p.sw, (int)l1, scale, pk);
         if (hipGetLastError() != hipSuccess)
             return SIMNETS_ERR_HIP;
-        const hipError_t e = l1 ? gx_launch_phases<GX_L1>(ph, n, jobs[first].PT, jobs[first].ksplit, s)
-                                : gx_launch_phases<GX_L2>(ph, n, jobs[first].PT, jobs[first].ksplit, s);
+        const hipError_t e = l1 ? gx_launch_phases<GX_L1>(ph, n, jobs[first].PT, jobs[first].MT, jobs[first].ksplit, s)
+                                : gx_launch_phases<GX_L2>(ph, n, jobs[first].PT, jobs[first].MT, jobs[first].ksplit, s);
         if (e != hipSuccess)
             return SIMNETS_ERR_HIP;
     }

@@ -591,3 +591,23 @@ def test_similarity_input_grad_small_maps_share_a_wave(pkg, case, func, norm, ig
     dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), algo="direct", **kw).cpu().numpy()
     assert np.array_equal(np.isnan(dx), np.isnan(want))
     assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad")
+
+
+@pytest.mark.parametrize("func,norm,ign", [("L1", False, False), ("L2", False, False), ("L2", True, True)])
+@pytest.mark.parametrize("case", [
+    dict(shape=(2, 3, 40, 50), O=9, blocks=[7, 7], strides=[2, 2], padding=[3, 3]),     # an image-like first layer
+    dict(shape=(1, 4, 20, 33), O=17, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),    # four channels, ragged rows
+    dict(shape=(3, 3, 9, 130), O=5, blocks=[2, 5], strides=[1, 3], padding=[0, 2]),     # wide rows: several pixel waves
+])
+def test_similarity_input_grad_of_few_channels(pkg, case, func, norm, ign):
+    """Three or four input channels: the term-by-term input-gradient kernel runs 8 pixels x 4 channels per lane."""
+    x, t, w = sim_inputs(78, case["shape"], case["O"], case["blocks"], nan_frac=0.15 if ign else 0.0)
+    kw = dict(similarity_function=func, blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+              normalization_term=norm, ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else -0.5)
+    out = orc.similarity_fwd(x, t, w, **kw)
+    og = np.random.default_rng(6).normal(size=out.shape).astype(np.float32)
+    want = orc.similarity_input_grad(x, t, w, og, **kw)
+    true = orc.similarity_input_grad(*f64(x, t, w, og), **kw)
+    dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), **kw).cpu().numpy()
+    assert np.array_equal(np.isnan(dx), np.isnan(want))
+    assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad")
