@@ -104,7 +104,8 @@ struct MfmaPhases {
 // At stride (sh, sw) the input pixels fall into sh * sw phases, (ry, rx) = ((y + ph) mod sh, (x + pw) mod sw).
 // Only the taps dh = ry + sh a, dw = rx + sw b reach a pixel of that phase, and with Y = (y + ph - ry) / sh the
 // window rows they come from are Y - a: each phase is a stride-1 problem of the same kind over its own taps,
-// on the grid of its pixels, and gets a launch of its own that stores to (and reads X at) the phase's pixels.
+// on the grid of its pixels, and gets a grid of its own (blockIdx.z) that stores to (and reads X at) the phase's
+// pixels.
 template <bool GRAD>
 __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a, const MfmaPhases phases)
 {
