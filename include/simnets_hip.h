@@ -72,9 +72,9 @@ enum {
                                 could exceed 4e-6 relative only for outputs closer to zero than sum_k w t^2 / 1024.
                                 The terms all have one sign, so a wave (64 pixel groups x 8 templates) whose partial
                                 sums after the first channel chunk all lie beyond that bound is safe; a wave with one
-                                that does not (or with a template of negative or NaN weight) stops there and a second,
-                                flag-gated pass recomputes all its outputs with DIRECT's arithmetic, bit-identical
-                                to SIMNETS_ALGO_DIRECT */
+                                that does not (or with a template of negative or NaN weight) stops there and a second
+                                pass of its workgroup recomputes all its outputs with DIRECT's arithmetic,
+                                bit-identical to SIMNETS_ALGO_DIRECT */
     SIMNETS_ALGO_MFMA = 3    /* plain L2 only, inputs free of NaN/Inf: sum w x^2 - 2 sum (w t) x + sum w t^2
                                 as dense fp32 matrix-core contractions */
 };

@@ -131,19 +131,20 @@ constexpr int kSmStageGroups = 2;   // small-map kernel: channel groups whose lo
 constexpr int waves_per_simd(int pt, int mt) { return pt * mt <= 64 ? 4 : 2; }
 constexpr int lds_budget_floats(int pt, int mt) { return pt * mt <= 64 ? kLdsBudgetFloats / 2 : kLdsBudgetFloats; }
 
-// GATED: the recomputing pass of the sqrt-weight form - same grid as the main launch, a workgroup none of whose
-//        waves raised its flag returns at once, the others recompute the flagged waves' outputs (MODE = SIM_MODE_L2
-//        on the second packed copy, bit-identical to SIMNETS_ALGO_DIRECT).
+// GATED: the recomputing pass of the sqrt-weight form, run by a workgroup with a flagged wave behind the main pass:
+//        the flagged waves recompute their outputs (MODE = SIM_MODE_L2 on the second packed copy, bit-identical to
+//        SIMNETS_ALGO_DIRECT), the others only help staging.
 // PLDS:  the workgroup's packed parameters (all K) are copied to LDS once and read from there by broadcast:
 //        for short K the step-ahead global loads would cost one memory latency per k.
 // ROW3:  3 x 3 templates at stride 1 (the convolution-like layers): the k loop walks (channel, dh) rows of the
 //        staged tile; a lane reads the PT + 2 values of a row once and the three taps of the row take their
 //        operands from those registers (x of tap dw, pixel p = value dw + p), instead of PT LDS values per tap
 //        through a table of offsets: a third of the LDS instructions, no per-k address arithmetic.
-template <int MODE, int PT, int MT, int SWT, bool GATED = false, bool PLDS = false, bool ROW3 = false>
-__global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
+// The kernel's body.  wave_bail: sqrt-weight form - out: this wave's guard flag; GATED - in: the flag that selects the
+// waves to recompute.
+template <int MODE, int PT, int MT, int SWT, bool GATED, bool PLDS, bool ROW3>
+__device__ __forceinline__ void sim_direct_body(const SimKernelArgs &a, float *lds, int &wave_bail)
 {
-    extern __shared__ float lds[];
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -153,13 +154,8 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     const int b = lp.b, mtile = lp.mtile, h = lp.h, gw = lp.gw;
     const bool lane_valid = lp.lane_valid;
     bool wave_active = lp.wave_active;
-    const size_t flag0 = ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * kWaves;
-    if (GATED) {
-        const int SIMNETS_CONST_AS *f = (const int SIMNETS_CONST_AS *)(a.flags) + flag0;
-        if ((f[0] | f[1] | f[2] | f[3]) == 0)
-            return;
-        wave_active = wave_active && f[wave] != 0;  // the other waves only help staging
-    }
+    if (GATED)
+        wave_active = wave_active && wave_bail != 0;  // the other waves only help staging
 
     // pixel groups of this workgroup and the input rows they need
     const int row_first = lp.row_first;
@@ -376,8 +372,7 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
                 }
             }
             const bool bail = __any(suspect);
-            if (lane == 0)
-                a.flags[flag0 + wave] = bail ? 1 : 0;
+            wave_bail = bail ? 1 : 0;
             if (bail)
                 wave_active = false;
         }
@@ -416,6 +411,21 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
                 if (w0 + p < a.ow)
                     o[p] = v[p];
         }
+    }
+}
+
+// The kernel: one pass of the body; the sqrt-weight form follows it, in the (rare) workgroups with a flagged wave, by
+// the recomputing pass - MODE = SIM_MODE_L2 on the second packed copy for the flagged waves, bit-identical to
+// SIMNETS_ALGO_DIRECT - as a cold path of the same launch.
+template <int MODE, int PT, int MT, int SWT, bool PLDS = false, bool ROW3 = false>
+__global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
+{
+    extern __shared__ float lds[];
+    int wave_bail = 0;
+    sim_direct_body<MODE, PT, MT, SWT, false, PLDS, ROW3>(a, lds, wave_bail);
+    if constexpr (MODE == SIM_MODE_L2_SQRTW) {
+        if (__syncthreads_or(wave_bail))
+            sim_direct_body<SIM_MODE_L2, PT, MT, SWT, true, false, ROW3>(a, lds, wave_bail);
     }
 }
 
@@ -830,23 +840,23 @@ Tiling choose_tiling(const SimPlan &p)
     return t;
 }
 
-template <int MODE, int PT, int MT, bool GATED, bool PLDS>
+template <int MODE, int PT, int MT, bool PLDS>
 hipError_t launch_direct(const SimKernelArgs &a, dim3 grid, size_t lds_bytes, hipStream_t s)
 {
     // (the normalized modes keep the table-driven loop: with their extra operands the row form does not fit the
     // register file)
     constexpr bool kRow3 = PT == kBigPT && !PLDS && (MODE == SIM_MODE_L1 || MODE == SIM_MODE_L2 || MODE == SIM_MODE_L2_SQRTW);
     if (kRow3 && a.sw == 1 && a.bh == 3 && a.bw == 3) {
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, GATED, false, kRow3>), grid, dim3(kThreads), lds_bytes, s,
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, false, kRow3>), grid, dim3(kThreads), lds_bytes, s,
                            a);
         return hipGetLastError();
     }
     if (a.sw == 1)
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 1, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     else if (a.sw == 2)
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 2, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 2, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     else
-        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 0, GATED, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
+        hipLaunchKernelGGL((sim_direct_kernel<MODE, PT, MT, 0, PLDS>), grid, dim3(kThreads), lds_bytes, s, a);
     return hipGetLastError();
 }
 
@@ -887,13 +897,15 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     const int nwm = kWaves / a.nws;
     dim3 grid((unsigned)(a.B * a.tiles), (unsigned)((a.n_mtiles + nwm - 1) / nwm));
     size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
+    if (GATED)
+        return hipSuccess;   // the tiled kernels recompute flagged waves inside the main launch
     if (t.PT == kBigPT && t.MT == kBigMT)
-        return launch_direct<MODE, kBigPT, kBigMT, GATED, false>(a, grid, lds_bytes, s);
-    if (plds && !GATED) {
+        return launch_direct<MODE, kBigPT, kBigMT, false>(a, grid, lds_bytes, s);
+    if (plds) {
         lds_bytes = ((size_t)a.plds_off + (size_t)nwm * (a.K + 1) * kSmallMT * 3) * sizeof(float);
-        return launch_direct<MODE, kSmallPT, kSmallMT, false, true>(a, grid, lds_bytes, s);
+        return launch_direct<MODE, kSmallPT, kSmallMT, true>(a, grid, lds_bytes, s);
     }
-    return launch_direct<MODE, kSmallPT, kSmallMT, GATED, false>(a, grid, lds_bytes, s);
+    return launch_direct<MODE, kSmallPT, kSmallMT, false>(a, grid, lds_bytes, s);
 }
 
 // The sqrt-weight form runs on the tiled kernels and on the small-map kernel; there only with enough pixels per
@@ -903,18 +915,17 @@ bool use_sqrtw(const SimPlan &p, const Tiling &t)
     return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && (t.NI == 0 || (long long)p.B * p.oh * p.ow >= 4096);
 }
 
-// flags of the guard: one per wave of the tiled kernels' grid, one per workgroup of the small-map kernel's
+// flags of the guard that live in the workspace: one per workgroup of the small-map kernel (the tiled kernels keep
+// theirs in registers)
 long long guard_flags(const SimPlan &p, const Tiling &t)
 {
-    const int n_mtiles = (p.O + t.MT - 1) / t.MT, nwm = kWaves / t.nws;
-    if (t.NI > 0)
-        return (long long)((p.B + t.NI - 1) / t.NI) * n_mtiles;
-    return (long long)p.B * t.tiles * ((n_mtiles + nwm - 1) / nwm) * kWaves;
+    const int n_mtiles = (p.O + t.MT - 1) / t.MT;
+    return t.NI > 0 ? (long long)((p.B + t.NI - 1) / t.NI) * n_mtiles : 0;
 }
 
 // Where the pieces of the workspace lie.  The first three are what every mode reads; the sqrt-weight form adds
-// the second packed copy, the thresholds (all written by the pack kernel) and the wave flags (written by every
-// main launch, read by the recomputing launch behind it).
+// the second packed copy and the thresholds (all written by the pack kernel) and, for the small-map kernel, the
+// workgroup flags (written by every main launch, read by the recomputing launch behind it).
 struct Layout {
     size_t pa, pc, koff, pa2, thr, flags, total;
 };
@@ -1011,7 +1022,7 @@ int sim_direct_run(const SimPlan &p, const float *input, float *output, void *wo
     case SIM_MODE_L2_NORM_IGNORE_NAN: e = launch_mode<SIM_MODE_L2_NORM_IGNORE_NAN>(a, t, plds, s); break;
     default: e = launch_mode<SIM_MODE_L2_SQRTW>(a, t, plds, s); break;
     }
-    if (e == hipSuccess && sqrtw)  // same grid: a workgroup looks at its waves' flags and, almost always, returns
+    if (e == hipSuccess && sqrtw)  // small maps: same grid, a workgroup looks at its flag and, almost always, returns
         e = launch_mode<SIM_MODE_L2, true>(a, t, false, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
