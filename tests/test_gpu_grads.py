@@ -611,3 +611,27 @@ def test_similarity_input_grad_of_few_channels(pkg, case, func, norm, ign):
     dx = pkg.similarity_input_grad(dev(x), dev(t), dev(w), dev(og), **kw).cpu().numpy()
     assert np.array_equal(np.isnan(dx), np.isnan(want))
     assert_grad_close(np.nan_to_num(dx), np.nan_to_num(want), np.nan_to_num(true), "input grad")
+
+
+@pytest.mark.parametrize("case", [
+    dict(shape=(32, 64, 56, 56), O=128, blocks=[3, 3], strides=[2, 2], padding=[1, 1]),   # interleaved stride phases
+    dict(shape=(32, 512, 7, 7), O=512, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),    # images share a tile, split
+    dict(shape=(32, 256, 14, 14), O=256, blocks=[3, 3], strides=[1, 1], padding=[1, 1]),  # split contraction
+    dict(shape=(8, 64, 57, 55), O=96, blocks=[3, 3], strides=[3, 2], padding=[1, 1]),     # six phase grids
+])
+def test_similarity_input_grad_forms_agree_at_network_sizes(pkg, case):
+    """Sizes the oracle would take minutes for: the matrix-core form against the term-by-term kernel (which the small
+    cases pin to the oracle), L2 with and without the normalization term."""
+    g = torch.Generator(device="cuda").manual_seed(11)
+    shape, O = case["shape"], case["O"]
+    x = torch.randn(shape, device="cuda", generator=g) + 1.5
+    t = torch.randn((O, shape[1]) + tuple(case["blocks"]), device="cuda", generator=g) + 1.5
+    w = torch.rand(t.shape, device="cuda", generator=g) + 0.1
+    for norm in (False, True):
+        kw = dict(similarity_function="L2", blocks=case["blocks"], strides=case["strides"], padding=case["padding"],
+                  normalization_term=norm)
+        og = torch.randn(pkg.similarity_output_shape(shape, t.shape, **kw), device="cuda", generator=g)
+        fast = pkg.similarity_input_grad(x, t, w, og, **kw)
+        exact = pkg.similarity_input_grad(x, t, w, og, algo="direct", **kw)
+        scale = exact.abs().max().item()
+        assert (fast - exact).abs().max().item() <= 1e-4 * scale, (case, norm)
