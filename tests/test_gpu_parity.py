@@ -568,3 +568,18 @@ def test_mex_overlapping_3d_blocks_network_like(pkg):
     assert got.shape == (6, 32, 28, 28)
     for b in (0, 5):
         assert mex_err(got[b:b + 1], x[b:b + 1], off, 32, **kw) <= MEX_TOL
+
+
+@pytest.mark.parametrize("shape,O", [((128, 512, 7, 7), 512), ((32, 256, 14, 14), 256), ((64, 128, 8, 8), 128)])
+def test_similarity_small_map_forms_agree_at_network_sizes(pkg, shape, O):
+    """Deep, small maps at sizes the oracle would take minutes for: the default form (sqrt-weight arithmetic with its
+    guard on the small-map kernel) against algo='direct' (the reference's arithmetic, pinned to the oracle by the
+    small cases), to the forward tolerance."""
+    g = torch.Generator(device="cuda").manual_seed(12)
+    x = torch.randn(shape, device="cuda", generator=g)
+    t = torch.randn((O, shape[1], 3, 3), device="cuda", generator=g)
+    w = torch.rand(t.shape, device="cuda", generator=g) + 0.1
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    fast = pkg.similarity(x, t, w, **kw).cpu().numpy()
+    exact = pkg.similarity(x, t, w, algo="direct", **kw).cpu().numpy()
+    assert rel_err(fast, exact) <= SIM_TOL
