@@ -782,7 +782,8 @@ Tiling try_tiling(const SimPlan &p, int PT, int MT, int nws)
     return t;
 }
 
-constexpr int kSmallMapLdsFloats = 8192;   // 32 KiB of tile per workgroup of the small-map kernel
+constexpr int kSmallMapLdsFloats = 8192;   // 32 KiB of tile per workgroup of the small-map kernel; twice that when the
+                                           // grid has at most two workgroups per compute unit (half as many chunk phases)
 
 // Lane tile and workgroup shape for a problem.
 Tiling choose_tiling(const SimPlan &p)
@@ -829,7 +830,8 @@ Tiling choose_tiling(const SimPlan &p)
             const int n_mtiles = (p.O + t.MT - 1) / t.MT;
             const long long wgs = (long long)((p.B + NI - 1) / NI) * n_mtiles;
             t.sm_waves = (wgs * kSmWaves <= 1024 && p.C >= 2 * kSmWaves) ? 2 * kSmWaves : kSmWaves;
-            const int cc_max = (int)std::min<long long>(p.C, kSmallMapLdsFloats / per_chan);
+            const int lds_floats = wgs <= 512 ? 2 * kSmallMapLdsFloats : kSmallMapLdsFloats;
+            const int cc_max = (int)std::min<long long>(p.C, lds_floats / per_chan);
             const int chunks = (p.C + cc_max - 1) / cc_max;
             t.CC = (p.C + chunks - 1) / chunks;
             // the waves of the workgroup split a chunk's channels: a multiple of their number keeps them even
