@@ -127,8 +127,8 @@ int simnets_hip_similarity_fwd(const simnets_similarity_attrs *attrs, const int 
  * caller-owned buffer of simnets_hip_similarity_workspace_bytes bytes (256-byte aligned), and
  * simnets_hip_similarity_fwd_prepared runs only the forward kernels on it.  attrs, input_shape (batch size
  * included: the tiling depends on it) and templates_shape must be the ones the buffer was prepared with; results
- * are those of simnets_hip_similarity_fwd bit for bit.  The buffer also holds a few bytes of per-call scratch (the
- * wave flags of the sqrt-weight form), so calls that share one prepared buffer must not overlap. */
+ * are those of simnets_hip_similarity_fwd bit for bit.  The buffer may also hold a few bytes of per-call scratch (the
+ * workgroup flags of the sqrt-weight form on small maps), so calls that share one prepared buffer must not overlap. */
 int simnets_hip_similarity_prepare(const simnets_similarity_attrs *attrs, const int input_shape[4],
                                    const int templates_shape[4], const int weights_shape[4], const float *templates,
                                    const float *weights, void *prepared, size_t prepared_bytes, void *stream);
