@@ -790,17 +790,24 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     const int wo = wave % WO, wk = wave / WO;
     const int lo = lane & 7, lk = lane >> 3;
     // blockIdx.x -> (pixel split, tile): the tiles of one split get ids that agree mod 8, so they run on the
-    // same XCD close in time and share the split's g and x chunks through that XCD's L2
+    // same XCD close in time and share the split's g and x chunks through that XCD's L2.  Fewer than 8 splits
+    // (1, 2 or 4: many tiles, few pixels) spread over all 8 XCDs, 8 / S of them per split.
     int split, tile_id;
-    {
+    if (a.S >= 8) {
         const int per_super = 8 * a.n_tiles;
         const int super = blockIdx.x / per_super;
         const int within = blockIdx.x - super * per_super;
         tile_id = within >> 3;
         split = super * 8 + (within & 7);
+        if (split >= a.S)
+            return;  // padding of the last group of 8 splits (uniform for the workgroup)
+    } else {
+        const int xcd = blockIdx.x & 7;
+        split = xcd & (a.S - 1);
+        tile_id = (blockIdx.x >> 3) * (8 / a.S) + xcd / a.S;
+        if (tile_id >= a.n_tiles)
+            return;
     }
-    if (split >= a.S)
-        return;  // padding of the last group of 8 splits (uniform for the workgroup)
     const int ktile = tile_id % a.n_ktiles, otile = tile_id / a.n_ktiles;
     const int o_wg = otile * OWG, k_wg = ktile * KWG;
 
@@ -1360,14 +1367,34 @@ GpTiling gp_tiling(const SimPlan &p)
     S = std::max(S, 1);
     t.cps = (t.nchunks + S - 1) / S;
     t.S = t.cps > 0 ? (t.nchunks + t.cps - 1) / t.cps : 1;
+    if (t.S < 8) {
+        // a power of two, so that 8 / S XCDs serve each split (a split past the last chunk adds zeros)
+        const int want = t.S >= 6 ? 8 : (t.S >= 3 ? 4 : t.S);
+        int s2 = 1;
+        while (s2 < want && s2 * 2 <= std::max(t.nchunks, 1))
+            s2 *= 2;
+        t.S = s2;
+        t.cps = (std::max(t.nchunks, 1) + s2 - 1) / s2;
+    }
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
     return t;
+}
+
+// workgroups of a launch: splits in groups of 8 (one per XCD) times the tiles; below 8 splits, 8 XCD slots times the
+// tiles each slot takes
+long long gp_blocks(const GpTiling &t)
+{
+    const long long tiles = (long long)t.n_otiles * t.n_ktiles;
+    if (t.S >= 8)
+        return (long long)(t.S + 7) / 8 * 8 * tiles;
+    const int per_split = 8 / t.S;
+    return 8 * ((tiles + per_split - 1) / per_split);
 }
 
 template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
-    dim3 grid((unsigned)((t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles));
+    dim3 grid((unsigned)gp_blocks(t));
     constexpr bool L2M = MODE != SIM_MODE_L1;
     if (t.fast && L2M && a.ow % PC == 0) {
         if (t.WO == 2)
@@ -1408,7 +1435,7 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
     if (workspace_bytes < sim_grad_params_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     const GpTiling t = gp_tiling(p);
-    if (p.bh > 0xffff || p.bw > 0xffff || (long long)(t.S + 7) / 8 * 8 * t.n_otiles * t.n_ktiles > 0x7fffffffLL)
+    if (p.bh > 0xffff || p.bw > 0xffff || gp_blocks(t) > 0x7fffffffLL)
         return SIMNETS_ERR_TOO_LARGE;
     GradPArgs a;
     a.g = output_grad; a.x = input; a.templates = templates;
