@@ -849,7 +849,10 @@ MexTiling mex_tiling(const MexPlan &p)
     const long long mtiles = (p.d.M + MX - 1) / MX;
     auto waves = [&](int px) { return p.d.num_regions * ((slots + 64 * px - 1) / (64 * px)) * mtiles; };
     MexTiling t;
-    t.px = 4;
+    // two pixels per lane at most: with four the kernel holds 220 VGPRs, one workgroup per compute unit, and every
+    // dependent phase (gather, barrier, matrix loop, stores) shows (32x16x16 -> 64 at batch 4096: 0.229 ms with four,
+    // 0.150 ms with two)
+    t.px = 2;
     while (t.px > 1 && waves(t.px) < SIMNETS_MEX_WAVES)
         t.px >>= 1;
     t.ks = 1;
@@ -986,9 +989,7 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     // finite eps: values are pre-multiplied by eps*log2(e), so the shift is always the maximum
     const bool neg = !a.finite_eps && p.epsilon < 0;
     hipError_t e;
-    if (t.px == 4)
-        e = launch_variant<4, 1, kChunkMin>(a, grid, neg, inside, s);
-    else if (t.px == 2)
+    if (t.px == 2)
         e = launch_variant<2, 1, kChunkMin>(a, grid, neg, inside, s);
     else if (t.ks == 1)
         e = launch_px1<1>(a, grid, neg, inside, t.kc, s);
