@@ -577,6 +577,7 @@ __global__ __launch_bounds__(64 * WAVES) void sim_small_map_kernel(const SimKern
     __syncthreads();
     if (wave > 0)
         return;
+#pragma unroll 1
     for (int w = 1; w < WAVES; ++w) {
         const float *src = lds + (size_t)(w - 1) * kPart + lane;
 #pragma unroll
