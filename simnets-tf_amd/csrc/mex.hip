@@ -55,7 +55,7 @@ constexpr int cmax(int a, int b) { return a > b ? a : b; }
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 template <int PX, int KS, int KC, bool NEG, bool CHECK>
-__global__ __launch_bounds__(256) void mex_fwd_kernel(const MexKernelArgs a)
+__global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const MexKernelArgs a)
 {
     constexpr int WM = 4 / KS;            // instance waves per workgroup
     constexpr int TM = WM * MX;           // instances per workgroup
