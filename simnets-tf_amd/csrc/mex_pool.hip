@@ -399,6 +399,352 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     }
 }
 
+// Panel form of the kernel above for the deep layers of such a stack: 2x2 windows, patches that are exactly the C
+// channels of a pixel (blocks [C, 1, 1], stride 1, no padding), C = 32 * NCH = 64, 128 or 256.  The pixels of a workgroup's
+// windows are then whole rows of a few images, i.e. per channel one contiguous run of floats, and the K values of all
+// its 64 * NH columns ("the panel") fit its registers (K / 16 float4 per thread).  The workgroup loads the panel once
+// with coalesced 16-byte loads (lanes along the run, then along k), takes each column's maximum over all of K once
+// (through LDS), and the chunk loop is left with two barriers: exponentials of 32 panel rows and the offsets tiles go
+// to LDS, the next offsets tiles are requested, the matrix loop runs.  Against the kernel above (per chunk: a gather
+// of dwords an image apart, a running maximum with its own barrier, rescaling of the accumulators) the chunk takes
+// about half the time where one workgroup per compute unit is all a layer offers.
+// LDS tiles are stored with column ^ swizzle(k): bits 4-5 of the column take k & 3, so that the four k rows a matrix
+// instruction's operand fetch touches (lane >> 4) fall into different banks; for the panel tile bits 2-3 take
+// (k >> 2) & 3 as well, which spreads the lanes of the staging writes that hold one column at 16 different k.
+constexpr int kPanelWorkgroups = 256;   // below this many two-half workgroups (one per compute unit) the panel form runs one-half ones
+
+struct PanelArgs {
+    int lgF;          // log2 of the float4 per (part, k): run / 4
+    int lgTPP;        // log2 of the threads per part
+    int lgW, Ws, RS;  // log2(width); windows per row; windows per image
+    int run;          // pixels of a part: whole rows of one image, contiguous per channel
+    int nparts;       // parts per workgroup
+    int ppi;          // parts per image
+    int total_parts;  // B * ppi
+    int HW;
+};
+
+template <int NH, int NCH>
+__global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKernelArgs a, const PoolArgs q,
+                                                                  const PanelArgs g)
+{
+    constexpr int R = 4;
+    constexpr int XP = 64 * NH;
+    constexpr int kThreads = 256 * NH;
+    constexpr int NV = 2 * NCH;   // float4 of the panel per thread: rows kslot + 16 u
+    __shared__ __attribute__((aligned(16))) float xs[KC * XP];       // [k][column ^ swizzle]
+    __shared__ __attribute__((aligned(16))) float os[R * KC * TM];   // [region][k][instance ^ swizzle]
+    __shared__ __attribute__((aligned(16))) float pmx[16 * XP];      // [kslot][column]: partial column maxima
+    __shared__ float msh[XP];                                        // column maxima
+    __shared__ long long ppos[16 * NH];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = wave & 3, wh = wave >> 2;
+    const int chunk = blockIdx.x, mgroup = blockIdx.y;
+    const int m0 = mgroup * TM + wm * MX;
+    const bool wave_active = m0 < a.M;
+
+    // ---- offsets tiles of a chunk: kThreads float4 per region and round ----
+    constexpr int TILE4 = KC * TM / 4;
+    constexpr int NO = TILE4 / kThreads;
+    static_assert(TILE4 % kThreads == 0, "offsets tile copy");
+    static_assert((NO == 1 || NO == 2) && R == 4, "offsets tile registers");
+    float4 on0, on1, on2, on3, on4, on5, on6, on7;   // float4 i: region i / NO, round i % NO
+    const float4 *osrc = reinterpret_cast<const float4 *>(a.offe + (size_t)mgroup * a.K * TM) + tid;
+    const size_t ostep = (size_t)a.n_mgroups * a.K * (TM / 4);   // float4 between the regions' tiles
+#define SIMNETS_PANEL_LOAD(i, k0) \
+    on##i = osrc[(size_t)((i) / NO) * ostep + ((i) % NO) * kThreads + (size_t)(k0) * (TM / 4)];
+#define SIMNETS_PANEL_ISSUE(k0)                                                                              \
+    {                                                                                                        \
+        SIMNETS_PANEL_LOAD(0, k0) SIMNETS_PANEL_LOAD(1, k0) SIMNETS_PANEL_LOAD(2, k0) SIMNETS_PANEL_LOAD(3, k0) \
+        if constexpr (NO == 2) {                                                                             \
+            SIMNETS_PANEL_LOAD(4, k0) SIMNETS_PANEL_LOAD(5, k0) SIMNETS_PANEL_LOAD(6, k0) SIMNETS_PANEL_LOAD(7, k0) \
+        }                                                                                                    \
+    }
+
+    // ---- the panel: this thread's float4 (4 neighbouring pixels of one channel) of rows kslot + 16 u ----
+    const int part = tid >> g.lgTPP;
+    const int jj = tid & ((1 << g.lgTPP) - 1);
+    const int pg = jj & ((1 << g.lgF) - 1);
+    const int kslot = jj >> g.lgF;   // 0 .. 15
+    const int gpart = chunk * g.nparts + part;
+    const bool pvalid = gpart < g.total_parts;
+    const int pb = pvalid ? gpart / g.ppi : 0;
+    const int po = pvalid ? (gpart - pb * g.ppi) * g.run : 0;   // first pixel of the part inside its image
+    float4 pv[NV];
+    {
+        const float *src = a.in + (size_t)pb * a.K * g.HW + po + 4 * pg + (size_t)kslot * g.HW;
+#pragma unroll
+        for (int u = 0; u < NV; ++u)
+            pv[u] = *reinterpret_cast<const float4 *>(src + (size_t)(16 * u) * g.HW);
+    }
+    SIMNETS_PANEL_ISSUE(0)
+
+    int wide = 0;
+    if (tid < TM) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+            wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
+    }
+
+    if (tid < 16 * NH) {
+        const int slot = chunk * (16 * NH) + tid;
+        long long pos = -1;
+        if (slot < a.slots) {
+            const int b = (int)fast_div((unsigned)slot, a.dRS);
+            const int sq = slot - b * a.RS;
+            const int qw = (int)fast_div((unsigned)sq, a.dWs);
+            const int i = sq - qw * a.Ws;
+            pos = (long long)b * a.M * ((long long)q.Hp * q.Wp) + (long long)qw * q.Wp + i;
+        }
+        ppos[tid] = pos;
+    }
+
+    // columns of the four pixels: tile (column half, region) x slot inside the half
+    int colx[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const int pix = po + 4 * pg + e;
+        const int h = pix >> g.lgW, w = pix & ((1 << g.lgW) - 1);
+        const int sl = pb * g.RS + (h >> 1) * g.Ws + (w >> 1) - chunk * (16 * NH);
+        colx[e] = pvalid ? (sl >> 4) * 64 + ((h & 1) * 2 + (w & 1)) * 16 + (sl & 15) : 0;
+    }
+
+    // ---- column maxima over all of K ----
+    {
+        float4 pm = make_float4(-INFINITY, -INFINITY, -INFINITY, -INFINITY);
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            pv[u].x *= a.scale; pv[u].y *= a.scale; pv[u].z *= a.scale; pv[u].w *= a.scale;
+            pm.x = fmaxf(pm.x, pv[u].x); pm.y = fmaxf(pm.y, pv[u].y);
+            pm.z = fmaxf(pm.z, pv[u].z); pm.w = fmaxf(pm.w, pv[u].w);
+        }
+        const int cg = (part << g.lgF) | pg;   // 0 .. XP / 4 - 1
+        reinterpret_cast<float4 *>(pmx)[kslot * (XP / 4) + cg] = pm;
+    }
+    const bool prod = !__syncthreads_or(wide);
+    float msub[4];
+    {
+        const int cg = (part << g.lgF) | pg;
+        float4 m = reinterpret_cast<const float4 *>(pmx)[cg];
+#pragma unroll
+        for (int s = 1; s < 16; ++s) {
+            const float4 o = reinterpret_cast<const float4 *>(pmx)[s * (XP / 4) + cg];
+            m.x = fmaxf(m.x, o.x); m.y = fmaxf(m.y, o.y); m.z = fmaxf(m.z, o.z); m.w = fmaxf(m.w, o.w);
+        }
+        if (kslot == 0 && pvalid) {
+            msh[colx[0]] = m.x; msh[colx[1]] = m.y; msh[colx[2]] = m.z; msh[colx[3]] = m.w;
+        }
+        // nothing finite in the column: the terms are exp2(-inf) = 0
+        msub[0] = m.x == -INFINITY ? 0.0f : m.x; msub[1] = m.y == -INFINITY ? 0.0f : m.y;
+        msub[2] = m.z == -INFINITY ? 0.0f : m.z; msub[3] = m.w == -INFINITY ? 0.0f : m.w;
+    }
+
+    const int lr = lane & 15, lq = lane >> 4;
+    const size_t plane_p = (size_t)q.Hp * q.Wp;
+    const size_t row0 = (size_t)(m0 + 4 * lq) * plane_p;
+    const bool all_rows = m0 + MX <= a.M;
+    float res[4][4];  // [region][v]: MEX value of (slot lr of this half, instance m0 + 4*lq + v)
+
+    if (prod) {
+        floatx4 acc[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+        const int sw = ((kslot & 3) << 4) | (((kslot >> 2) & 3) << 2);
+        const float *oa = os + lq * TM + ((wm ^ lq) << 4) + lr;
+        int xo[4];   // column of tile t in row lq (+ 4 j): ((t ^ lq) << 4 | lr) ^ (j & 3) << 2
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            xo[t] = lq * XP + wh * 64 + ((t ^ lq) << 4) + lr;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            // ---- registers -> LDS (the previous chunk's readers are behind the barrier that ended its loop) ----
+            {
+                float4 *dst = reinterpret_cast<float4 *>(os) + ((tid & ~15) | ((tid & 15) ^ (((tid >> 4) & 3) << 2)));
+#define SIMNETS_PANEL_PUT(i) dst[((i) / NO) * TILE4 + ((i) % NO) * kThreads] = on##i;
+                SIMNETS_PANEL_PUT(0) SIMNETS_PANEL_PUT(1) SIMNETS_PANEL_PUT(2) SIMNETS_PANEL_PUT(3)
+                if constexpr (NO == 2) {
+                    SIMNETS_PANEL_PUT(4) SIMNETS_PANEL_PUT(5) SIMNETS_PANEL_PUT(6) SIMNETS_PANEL_PUT(7)
+                }
+#undef SIMNETS_PANEL_PUT
+            }
+            // (columns of parts past the batch stay unwritten: a column only reaches its own, unstored, outputs)
+            if (pvalid) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 v = pv[2 * c + h];
+                    float *row = xs + (kslot + 16 * h) * XP;
+                    row[colx[0] ^ sw] = __builtin_amdgcn_exp2f(v.x - msub[0]);
+                    row[colx[1] ^ sw] = __builtin_amdgcn_exp2f(v.y - msub[1]);
+                    row[colx[2] ^ sw] = __builtin_amdgcn_exp2f(v.z - msub[2]);
+                    row[colx[3] ^ sw] = __builtin_amdgcn_exp2f(v.w - msub[3]);
+                }
+            }
+            __syncthreads();
+            // the matrix loop, with the requests for the next chunk's offsets tiles spread between its steps (a
+            // compute unit's vector memory path takes 64 bytes a cycle: issued in one go they hold the waves up)
+            const bool more = c + 1 < NCH;
+            const int kn = (c + 1) * KC;
+#define SIMNETS_PANEL_RD(set, it, t)            \
+    av##set[t] = oa[(t) * KC * TM + 4 * (it) * TM]; \
+    bv##set[t] = xs[4 * (it) * XP + (xo[t] ^ (((it) & 3) << 2))];
+#define SIMNETS_PANEL_READ(set, it) \
+    SIMNETS_PANEL_RD(set, it, 0) SIMNETS_PANEL_RD(set, it, 1) SIMNETS_PANEL_RD(set, it, 2) SIMNETS_PANEL_RD(set, it, 3)
+#define SIMNETS_PANEL_MM(set, t) \
+    acc[t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av##set[t], bv##set[t], acc[t], 0, 0, 0);
+#define SIMNETS_PANEL_FENCE __builtin_amdgcn_sched_barrier(0);
+// the four matrix instructions of a step, each followed by the LDS reads of one tile of the step two ahead
+#define SIMNETS_PANEL_STEP(cur, nxt, itn)                                        \
+    SIMNETS_PANEL_MM(cur, 0) SIMNETS_PANEL_RD(nxt, itn, 0) SIMNETS_PANEL_FENCE   \
+    SIMNETS_PANEL_MM(cur, 1) SIMNETS_PANEL_RD(nxt, itn, 1) SIMNETS_PANEL_FENCE   \
+    SIMNETS_PANEL_MM(cur, 2) SIMNETS_PANEL_RD(nxt, itn, 2) SIMNETS_PANEL_FENCE   \
+    SIMNETS_PANEL_MM(cur, 3) SIMNETS_PANEL_RD(nxt, itn, 3)
+#define SIMNETS_PANEL_LAST(cur) \
+    SIMNETS_PANEL_MM(cur, 0) SIMNETS_PANEL_MM(cur, 1) SIMNETS_PANEL_MM(cur, 2) SIMNETS_PANEL_MM(cur, 3)
+#define SIMNETS_PANEL_NEXT(i2, i1)                    \
+    if (more) {                                       \
+        if constexpr (NO == 2) {                      \
+            SIMNETS_PANEL_LOAD(i2, kn)                \
+        } else if constexpr ((i2) % 2 == 0) {         \
+            SIMNETS_PANEL_LOAD(i1, kn)                \
+        }                                             \
+    }                                                 \
+    __builtin_amdgcn_sched_barrier(0);
+            {
+                // (waves past the last instance compute on the padding rows of the packed offsets: no branch whose
+                // other side would leave loads pending in the registers used here)
+                // operands of step i + 2 are read from LDS between the matrix instructions of step i: a wave issues
+                // in order, so reads bunched in front of a step's four matrix instructions would idle the matrix unit
+                float avA[R], bvA[4], avB[R], bvB[4], avC[R], bvC[4];
+                SIMNETS_PANEL_READ(A, 0) SIMNETS_PANEL_READ(B, 1) SIMNETS_PANEL_FENCE
+                SIMNETS_PANEL_STEP(A, C, 2) SIMNETS_PANEL_NEXT(0, 0)
+                SIMNETS_PANEL_STEP(B, A, 3) SIMNETS_PANEL_NEXT(1, 0)
+                SIMNETS_PANEL_STEP(C, B, 4) SIMNETS_PANEL_NEXT(2, 1)
+                SIMNETS_PANEL_STEP(A, C, 5) SIMNETS_PANEL_NEXT(3, 1)
+                SIMNETS_PANEL_STEP(B, A, 6) SIMNETS_PANEL_NEXT(4, 2)
+                SIMNETS_PANEL_STEP(C, B, 7) SIMNETS_PANEL_NEXT(5, 2)
+                SIMNETS_PANEL_LAST(A) SIMNETS_PANEL_NEXT(6, 3)
+                SIMNETS_PANEL_LAST(B) SIMNETS_PANEL_NEXT(7, 3)
+            }
+#undef SIMNETS_PANEL_RD
+#undef SIMNETS_PANEL_READ
+#undef SIMNETS_PANEL_MM
+#undef SIMNETS_PANEL_FENCE
+#undef SIMNETS_PANEL_STEP
+#undef SIMNETS_PANEL_LAST
+#undef SIMNETS_PANEL_NEXT
+            if (c + 1 < NCH)
+                __syncthreads();  // everyone is done with this chunk's tiles
+        }
+        if (!wave_active)
+            return;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const float *omax = a.omax + ((size_t)t * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
+            const float mp = msh[wh * 64 + t * 16 + lr];
+            // an infinite column bound makes the result NaN, as the reference's exp(inf - inf) does
+            const float mpt = (mp - mp) + mp + a.c0;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                res[t][v] = (__builtin_amdgcn_logf(acc[t][v]) + (mpt + omax[v])) * a.ln2_over_eps;
+        }
+    } else {
+        // offsets too far apart for the product form: term by term from global memory (rare, slow)
+        if (!wave_active)
+            return;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const PixelRef gp = locate(a, t, chunk * (16 * NH) + wh * 16 + lr);
+            const float *orow = a.offp + (((size_t)t * a.n_mgroups + mgroup) * a.K) * TM + wm * MX + 4 * lq;
+            float best[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+            for (int k = 0; k < a.K; ++k) {
+                const float x = gp.base[(size_t)k * g.HW] * a.scale;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    best[v] = fmaxf(best[v], x + orow[(size_t)k * TM + v]);
+            }
+            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (int k = 0; k < a.K; ++k) {
+                const float x = gp.base[(size_t)k * g.HW] * a.scale;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    sum[v] += __builtin_amdgcn_exp2f(x + orow[(size_t)k * TM + v] -
+                                                     (best[v] == -INFINITY ? 0.0f : best[v]));
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const float b = best[v];
+                res[t][v] = (__builtin_amdgcn_logf(sum[v]) + ((b - b) + b + a.c0)) * a.ln2_over_eps;
+            }
+        }
+    }
+
+    // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
+    const long long pos = ppos[wh * 16 + lr];  // written before the first barrier
+    if (pos < 0)
+        return;
+    float *o = q.pooled + pos + row0;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const float w = ((res[0][v] + res[1][v]) + res[2][v]) + res[3][v];
+        if (all_rows || m0 + 4 * lq + v < a.M)
+            o[v * plane_p] = w;
+    }
+}
+
+// Geometry of the panel form for workgroups of nh column halves; false when the layer does not have it.
+bool panel_geometry(const MexPlan &p, int ph, int pw, const float *input, int nh, PanelArgs *g)
+{
+    const simnets_mex_dims &d = p.d;
+    if (ph != 2 || pw != 2 || d.block_c != p.C || d.block_h != 1 || d.block_w != 1 || d.stride_h != 1 ||
+        d.stride_w != 1 || d.pad_c != 0 || d.pad_h != 0 || d.pad_w != 0 || d.channels_out != 1 || (p.H & 1) ||
+        (p.W & 1) || (p.W & (p.W - 1)) != 0)
+        return false;
+    if (d.K != 64 && d.K != 128 && d.K != 256)   // (one chunk: nothing to gain over the kernel above)
+        return false;
+    if (reinterpret_cast<uintptr_t>(input) % 16 != 0)
+        return false;
+    const int spw = 16 * nh, Ws = p.W / 2, RS = (p.H / 2) * Ws, HW = p.H * p.W;
+    if (d.region_size != RS)
+        return false;
+    int run;
+    if (spw % RS == 0)
+        run = HW;        // whole images
+    else if (RS % spw == 0 && spw % Ws == 0)
+        run = 4 * spw;   // whole window rows of one image
+    else
+        return false;
+    auto lg = [](int v) { int l = 0; while ((1 << l) < v) ++l; return l; };
+    g->run = run;
+    g->nparts = 4 * spw / run;
+    g->ppi = HW / run;
+    g->total_parts = p.B * g->ppi;
+    g->HW = HW;
+    g->lgF = lg(run / 4);
+    g->lgTPP = lg(256 * nh / g->nparts);
+    g->lgW = lg(p.W);
+    g->Ws = Ws;
+    g->RS = RS;
+    return true;
+}
+
+template <int NH>
+hipError_t launch_panel(const MexKernelArgs &a, const PoolArgs &q, const PanelArgs &g, dim3 grid, hipStream_t s)
+{
+    switch (a.K / KC) {
+    case 2: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 2>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    case 4: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 4>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    default: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 8>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    }
+    return hipGetLastError();
+}
+
+#undef SIMNETS_PANEL_ISSUE
+#undef SIMNETS_PANEL_LOAD
+
 template <int R, int NH>
 hipError_t launch_pool(const MexKernelArgs &a, const PoolArgs &q, dim3 grid, bool inside, hipStream_t s)
 {
@@ -467,6 +813,16 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
     if (ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
         nh = 4;
+    // panel form: one column half per workgroup while two would leave compute units without a workgroup
+    PanelArgs pg;
+    bool panel = false;
+    if (!sp && a.slots > 16) {
+        const int pnh = ((long long)a.slots + 31) / 32 * n_mgroups < kPanelWorkgroups ? 1 : 2;
+        panel = panel_geometry(p, ph, pw, input, pnh, &pg) ||
+                (pnh == 1 && panel_geometry(p, ph, pw, input, 2, &pg));
+        if (panel)
+            nh = pg.nparts * pg.run / 64;   // columns of a workgroup / 64
+    }
     q.spw = nh * 64 / (ph * pw);
     const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
     if (gx > 0x7fffffffLL || n_mgroups > 65535)
@@ -478,7 +834,9 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     dim3 grid((unsigned)gx, (unsigned)n_mgroups);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e;
-    if (ph * pw == 4)
+    if (panel)
+        e = nh == 1 ? launch_panel<1>(a, q, pg, grid, s) : launch_panel<2>(a, q, pg, grid, s);
+    else if (ph * pw == 4)
         e = nh == 4 ? launch_pool<4, 4>(a, q, grid, inside, s)
                     : (nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s));
     else

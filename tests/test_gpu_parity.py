@@ -359,6 +359,16 @@ def pooled(y, ph, pw):
     dict(im=(36, 8, 16, 32), n=70, pool=(1, 2)),
     dict(im=(33, 7, 31, 33), n=20, pool=(2, 2), blocks=[7, 3, 3], padding=[0, 1, 1]),  # the same with ragged edges
     dict(im=(3, 6, 12, 12), n=24, pool=(2, 2), blocks=[2, 1, 1], strides=[2, 1, 1]),   # several output channels
+    # whole-channel patches of 64 / 128 / 256 channels on power-of-two widths: the panel form of the kernel
+    dict(im=(37, 64, 8, 8), n=70, pool=(2, 2)),                        # one image per workgroup, a partial instance group
+    dict(im=(21, 128, 4, 4), n=64, pool=(2, 2)),                       # four images per workgroup, the last one part full
+    dict(im=(45, 256, 2, 2), n=130, pool=(2, 2)),                      # one window per image, 16 images per workgroup
+    dict(im=(5, 64, 16, 16), n=64, pool=(2, 2)),                       # four workgroups per image
+    dict(im=(3, 64, 24, 16), n=16, pool=(2, 2)),                       # six workgroups per image
+    dict(im=(3, 128, 4, 32), n=16, pool=(2, 2)),                       # wide and flat: two workgroups per image
+    dict(im=(2, 64, 4, 64), n=16, pool=(2, 2)),                        # rows too wide for one-half workgroups: two halves
+    dict(im=(2, 64, 4, 128), n=16, pool=(2, 2)),                       # rows too wide for it: the general kernel
+    dict(im=(64, 64, 16, 16), n=256, pool=(2, 2)),                     # enough workgroups for its two-half form
 ])
 @pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("wide", 1.0), ("mixed", 3.0)])
 def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
@@ -386,6 +396,34 @@ def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
     # and it is the two separate calls, up to the rounding of the MEX values
     two = pkg.sum_pooling(pkg.mex(dev(x), dev(off), n, **kw), (ph, pw)).cpu().numpy()
     assert rel_err(got, two, floor=shift) <= 1e-5
+
+
+@pytest.mark.parametrize("im,n", [((19, 64, 8, 8), 40), ((40, 256, 2, 2), 64), ((6, 128, 16, 16), 64)])
+@pytest.mark.parametrize("eps", [1.0, -0.5])
+def test_mex_sum_pool_panel_form_with_infinite_and_missing_inputs(pkg, im, n, eps):
+    # pixels whose channels are all -inf (+inf for negative epsilon), single infinite or NaN channels, huge values:
+    # the fused kernel gives what MEX followed by sum pooling gives, NaN for NaN
+    g = np.random.default_rng(44)
+    kw = dict(softmax_mode=True, blocks=[im[1], 1, 1], strides=[im[1], 1, 1], epsilon=eps, use_unshared_regions=True,
+              unshared_offset_region=[1, 2, 2])
+    x = (g.normal(size=im) * 30).astype(np.float32)
+    lo = -math.inf if eps > 0 else math.inf
+    x[g.random(size=im) < 0.05] = lo
+    x[0, :, 0, 0] = lo                      # an empty column
+    x[1, 3, 1, 1] = -lo                     # a column with an infinite maximum
+    x[2, 5, 0, 1] = np.nan
+    x[3] *= 1e4                             # maxima far from zero
+    off = g.normal(size=(4, n, im[1], 1, 1)).astype(np.float32)
+    got = pkg.mex_sum_pool(dev(x), dev(off), n, (2, 2), **kw).cpu().numpy()
+    two = pkg.sum_pooling(pkg.mex(dev(x), dev(off), n, **kw), (2, 2)).cpu().numpy()
+    assert np.array_equal(np.isnan(got), np.isnan(two))
+    assert np.isnan(got[2]).any() and not np.isnan(got[4:]).any()
+    with np.errstate(invalid="ignore"):
+        want = pooled(orc.mex_fwd(x, off, n, **kw), 2, 2)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    fin = np.isfinite(want)
+    assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+    assert np.abs(got[fin] - want[fin]).max() <= MEX_TOL * max(1.0, np.abs(want[fin]).max())
 
 
 @pytest.mark.parametrize("kw,pool", [
