@@ -849,6 +849,14 @@ MexTiling mex_tiling(const MexPlan &p)
     const long long mtiles = (p.d.M + MX - 1) / MX;
     auto waves = [&](int px) { return p.d.num_regions * ((slots + 64 * px - 1) / (64 * px)) * mtiles; };
     MexTiling t;
+    if (mex_panel_geometry(p)) {
+        // the panel kernel's packing: 64 instances per group; its fallback for unaligned inputs is the plain tiling
+        t.px = 1; t.ks = 1;
+        t.kc = p.d.K >= 128 ? 128 : 64;
+        t.tm = 4 * MX;
+        t.n_mgroups = (p.d.M + t.tm - 1) / t.tm;
+        return t;
+    }
     // two pixels per lane at most: with four the kernel holds 220 VGPRs, one workgroup per compute unit, and every
     // dependent phase (gather, barrier, matrix loop, stores) shows (32x16x16 -> 64 at batch 4096: 0.229 ms with four,
     // 0.150 ms with two)
@@ -972,6 +980,11 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     const int rc = mex_pack_offsets(p, offsets, t.tm, t.n_mgroups, workspace, &a, stream, nullptr, pack);
     if (rc || !(phase & kMexRun))
         return rc;
+    if (mex_panel_geometry(p)) {
+        const int prc = mex_panel_launch(p, a, input, output, stream);
+        if (prc != SIMNETS_PANEL_NOT_TAKEN)
+            return prc;
+    }
     a.in = input; a.out = output;
     a.kgather = t.px == 1 && t.ks >= 2 && d.region_size == 1;
 

@@ -139,4 +139,13 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
                      void *stream, const SimPackJob *job = nullptr, bool launch = true);
 
+
+// Panel form of the tiled forward kernel (csrc/mex_pool.hip) for layers with 2x2 unshared offsets over whole-channel
+// patches of 64, 128 or 256 channels: mex_panel_geometry says whether a layer has its geometry (its offsets are then
+// packed in groups of 64 instances); mex_panel_launch runs it on offsets packed that way, or returns
+// SIMNETS_PANEL_NOT_TAKEN without launching anything (input not 16-byte aligned).
+constexpr int SIMNETS_PANEL_NOT_TAKEN = 1;
+bool mex_panel_geometry(const MexPlan &p);
+int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *input, float *output, void *stream);
+
 }  // namespace simnets

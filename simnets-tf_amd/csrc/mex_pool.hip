@@ -424,7 +424,8 @@ struct PanelArgs {
     int HW;
 };
 
-template <int NH, int NCH>
+// POOL = false: the same tiling without the pooling, every MEX value stored (the plain MEX call on such a layer).
+template <int NH, int NCH, bool POOL>
 __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKernelArgs a, const PoolArgs q,
                                                                   const PanelArgs g)
 {
@@ -436,7 +437,9 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
     __shared__ __attribute__((aligned(16))) float os[R * KC * TM];   // [region][k][instance ^ swizzle]
     __shared__ __attribute__((aligned(16))) float pmx[16 * XP];      // [kslot][column]: partial column maxima
     __shared__ float msh[XP];                                        // column maxima
-    __shared__ long long ppos[16 * NH];  // per slot: where instance 0 goes in the pooled tensor, -1 = no window
+    // per slot: where instance 0 goes in the pooled tensor (POOL = false: where the window's first pixel goes in the
+    // MEX output), -1 = no window
+    __shared__ long long ppos[16 * NH];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -497,7 +500,10 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
             const int sq = slot - b * a.RS;
             const int qw = (int)fast_div((unsigned)sq, a.dWs);
             const int i = sq - qw * a.Ws;
-            pos = (long long)b * a.M * ((long long)q.Hp * q.Wp) + (long long)qw * q.Wp + i;
+            if (POOL)
+                pos = (long long)b * a.M * ((long long)q.Hp * q.Wp) + (long long)qw * q.Wp + i;
+            else
+                pos = (long long)b * a.M * g.HW + ((long long)(2 * qw) << g.lgW) + 2 * i;
         }
         ppos[tid] = pos;
     }
@@ -543,7 +549,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
     }
 
     const int lr = lane & 15, lq = lane >> 4;
-    const size_t plane_p = (size_t)q.Hp * q.Wp;
+    const size_t plane_p = POOL ? (size_t)q.Hp * q.Wp : (size_t)g.HW;   // floats per instance of the stored tensor
     const size_t row0 = (size_t)(m0 + 4 * lq) * plane_p;
     const bool all_rows = m0 + MX <= a.M;
     float res[4][4];  // [region][v]: MEX value of (slot lr of this half, instance m0 + 4*lq + v)
@@ -687,11 +693,21 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
     if (pos < 0)
         return;
     float *o = q.pooled + pos + row0;
+    if (POOL) {
 #pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const float w = ((res[0][v] + res[1][v]) + res[2][v]) + res[3][v];
-        if (all_rows || m0 + 4 * lq + v < a.M)
-            o[v * plane_p] = w;
+        for (int v = 0; v < 4; ++v) {
+            const float w = ((res[0][v] + res[1][v]) + res[2][v]) + res[3][v];
+            if (all_rows || m0 + 4 * lq + v < a.M)
+                o[v * plane_p] = w;
+        }
+    } else {
+        // region t is pixel (t / 2, t % 2) of the window
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (all_rows || m0 + 4 * lq + v < a.M)
+                    o[v * plane_p + ((size_t)(t >> 1) << g.lgW) + (t & 1)] = res[t][v];
     }
 }
 
@@ -731,15 +747,27 @@ bool panel_geometry(const MexPlan &p, int ph, int pw, const float *input, int nh
     return true;
 }
 
-template <int NH>
+template <int NH, bool POOL>
 hipError_t launch_panel(const MexKernelArgs &a, const PoolArgs &q, const PanelArgs &g, dim3 grid, hipStream_t s)
 {
     switch (a.K / KC) {
-    case 2: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 2>), grid, dim3(256 * NH), 0, s, a, q, g); break;
-    case 4: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 4>), grid, dim3(256 * NH), 0, s, a, q, g); break;
-    default: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 8>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    case 2: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 2, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    case 4: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 4, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    default: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 8, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
     }
     return hipGetLastError();
+}
+
+// Workgroup shape of the panel form for this layer (column halves), 0 when the layer does not have its geometry.
+int panel_halves(const MexPlan &p, int ph, int pw, const float *input, int slots, int n_mgroups, PanelArgs *g)
+{
+    if (slots <= 16)
+        return 0;
+    // one column half per workgroup while two would leave compute units without a workgroup
+    const int pnh = ((long long)slots + 31) / 32 * n_mgroups < kPanelWorkgroups ? 1 : 2;
+    if (panel_geometry(p, ph, pw, input, pnh, g))
+        return pnh;
+    return pnh == 1 && panel_geometry(p, ph, pw, input, 2, g) ? 2 : 0;
 }
 
 #undef SIMNETS_PANEL_ISSUE
@@ -813,16 +841,10 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
     if (ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
         nh = 4;
-    // panel form: one column half per workgroup while two would leave compute units without a workgroup
     PanelArgs pg;
-    bool panel = false;
-    if (!sp && a.slots > 16) {
-        const int pnh = ((long long)a.slots + 31) / 32 * n_mgroups < kPanelWorkgroups ? 1 : 2;
-        panel = panel_geometry(p, ph, pw, input, pnh, &pg) ||
-                (pnh == 1 && panel_geometry(p, ph, pw, input, 2, &pg));
-        if (panel)
-            nh = pg.nparts * pg.run / 64;   // columns of a workgroup / 64
-    }
+    const int panel = sp ? 0 : panel_halves(p, ph, pw, input, a.slots, n_mgroups, &pg);
+    if (panel)
+        nh = panel;
     q.spw = nh * 64 / (ph * pw);
     const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
     if (gx > 0x7fffffffLL || n_mgroups > 65535)
@@ -835,7 +857,7 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     hipError_t e;
     if (panel)
-        e = nh == 1 ? launch_panel<1>(a, q, pg, grid, s) : launch_panel<2>(a, q, pg, grid, s);
+        e = nh == 1 ? launch_panel<1, true>(a, q, pg, grid, s) : launch_panel<2, true>(a, q, pg, grid, s);
     else if (ph * pw == 4)
         e = nh == 4 ? launch_pool<4, 4>(a, q, grid, inside, s)
                     : (nh == 2 ? launch_pool<4, 2>(a, q, grid, inside, s) : launch_pool<4, 1>(a, q, grid, inside, s));
@@ -845,6 +867,40 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
 }
 
 }  // namespace
+
+bool mex_panel_geometry(const MexPlan &p)
+{
+    PanelArgs g;
+    const long long slots = (long long)p.B * p.d.region_size;
+    if (!fusable(p, 2, 2) || slots > 0x7fffffffLL)
+        return false;
+    // (the pointer is checked by the launch; any 16-byte aligned one stands in here)
+    return panel_halves(p, 2, 2, reinterpret_cast<const float *>(uintptr_t(16)), (int)slots, (p.d.M + TM - 1) / TM,
+                        &g) != 0;
+}
+
+int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *input, float *output, void *stream)
+{
+    PanelArgs g;
+    const int nh = panel_halves(p, 2, 2, input, a.slots, a.n_mgroups, &g);
+    if (!nh)
+        return SIMNETS_PANEL_NOT_TAKEN;
+    PoolArgs q;
+    q.sx = nullptr;
+    q.pooled = output;
+    q.Hp = p.d.height_out / 2;
+    q.Wp = p.d.width_out / 2;
+    q.spw = 16 * nh;
+    const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
+    if (gx > 0x7fffffffLL || a.n_mgroups > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    MexKernelArgs b = a;
+    b.in = input;
+    dim3 grid((unsigned)gx, (unsigned)a.n_mgroups);
+    hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    const hipError_t e = nh == 1 ? launch_panel<1, false>(b, q, g, grid, s) : launch_panel<2, false>(b, q, g, grid, s);
+    return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
 
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw)
 {

@@ -398,6 +398,33 @@ def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
     assert rel_err(got, two, floor=shift) <= 1e-5
 
 
+@pytest.mark.parametrize("im,n", [
+    ((37, 64, 8, 8), 70), ((21, 128, 4, 4), 64), ((45, 256, 2, 2), 130), ((5, 64, 16, 16), 64), ((3, 64, 24, 16), 16),
+    ((2, 64, 4, 64), 16), ((64, 64, 16, 16), 256),
+])
+@pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("mixed", 3.0)])
+def test_mex_panel_form_of_the_plain_call(pkg, im, n, spread, eps):
+    # 2x2 unshared offsets over whole-channel patches of 64 / 128 / 256 channels: the plain MEX call runs the panel
+    # kernel without its pooling; an input that is not 16-byte aligned takes the general tiled kernel on the same
+    # packed offsets
+    g = np.random.default_rng(46)
+    kw = dict(softmax_mode=False, blocks=[im[1], 1, 1], strides=[im[1], 1, 1], epsilon=eps, use_unshared_regions=True,
+              unshared_offset_region=[1, 2, 2])
+    x = (g.normal(size=im) * 5).astype(np.float32)
+    off = (g.normal(size=(4, n, im[1], 1, 1)) * 0.3).astype(np.float32)
+    if spread == "mixed":
+        off[:, n // 2:] *= 400
+    got = run_mex(pkg, x, off, n, **kw)
+    assert got.shape == (im[0], n, im[2], im[3])
+    assert mex_err(got, x, off, n, **kw) <= MEX_TOL
+    flat = torch.empty(x.size + 1, device="cuda")
+    shifted = flat[1:].view(*im)
+    shifted.copy_(dev(x))
+    assert shifted.data_ptr() % 16 == 4
+    other = pkg.mex(shifted, dev(off), n, **kw).cpu().numpy()
+    assert mex_err(other, x, off, n, **kw) <= MEX_TOL
+
+
 @pytest.mark.parametrize("im,n", [((19, 64, 8, 8), 40), ((40, 256, 2, 2), 64), ((6, 128, 16, 16), 64)])
 @pytest.mark.parametrize("eps", [1.0, -0.5])
 def test_mex_sum_pool_panel_form_with_infinite_and_missing_inputs(pkg, im, n, eps):
