@@ -852,7 +852,7 @@ MexTiling mex_tiling(const MexPlan &p)
     if (mex_panel_geometry(p)) {
         // the panel kernel's packing: 64 instances per group; its fallback for unaligned inputs is the plain tiling
         t.px = 1; t.ks = 1;
-        t.kc = p.d.K >= 128 ? 128 : 64;
+        t.kc = p.d.K >= 128 ? 128 : (p.d.K >= 64 ? 64 : kChunkMin);
         t.tm = 4 * MX;
         t.n_mgroups = (p.d.M + t.tm - 1) / t.tm;
         return t;

@@ -141,7 +141,7 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
 
 
 // Panel form of the tiled forward kernel (csrc/mex_pool.hip) for layers with 2x2 unshared offsets over whole-channel
-// patches of 64, 128 or 256 channels: mex_panel_geometry says whether a layer has its geometry (its offsets are then
+// patches of 32 (small grids), 64, 128 or 256 channels: mex_panel_geometry says whether a layer has its geometry (its offsets are then
 // packed in groups of 64 instances); mex_panel_launch runs it on offsets packed that way, or returns
 // SIMNETS_PANEL_NOT_TAKEN without launching anything (input not 16-byte aligned).
 constexpr int SIMNETS_PANEL_NOT_TAKEN = 1;

@@ -400,7 +400,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
 }
 
 // Panel form of the kernel above for the deep layers of such a stack: 2x2 windows, patches that are exactly the C
-// channels of a pixel (blocks [C, 1, 1], stride 1, no padding), C = 32 * NCH = 64, 128 or 256.  The pixels of a workgroup's
+// channels of a pixel (blocks [C, 1, 1], stride 1, no padding), C = 32 * NCH = 32 (plain call on a small grid only), 64, 128 or 256.  The pixels of a workgroup's
 // windows are then whole rows of a few images, i.e. per channel one contiguous run of floats, and the K values of all
 // its 64 * NH columns ("the panel") fit its registers (K / 16 float4 per thread).  The workgroup loads the panel once
 // with coalesced 16-byte loads (lanes along the run, then along k), takes each column's maximum over all of K once
@@ -719,7 +719,7 @@ bool panel_geometry(const MexPlan &p, int ph, int pw, const float *input, int nh
         d.stride_w != 1 || d.pad_c != 0 || d.pad_h != 0 || d.pad_w != 0 || d.channels_out != 1 || (p.H & 1) ||
         (p.W & 1) || (p.W & (p.W - 1)) != 0)
         return false;
-    if (d.K != 64 && d.K != 128 && d.K != 256)   // (one chunk: nothing to gain over the kernel above)
+    if (d.K != 32 && d.K != 64 && d.K != 128 && d.K != 256)
         return false;
     if (reinterpret_cast<uintptr_t>(input) % 16 != 0)
         return false;
@@ -751,6 +751,7 @@ template <int NH, bool POOL>
 hipError_t launch_panel(const MexKernelArgs &a, const PoolArgs &q, const PanelArgs &g, dim3 grid, hipStream_t s)
 {
     switch (a.K / KC) {
+    case 1: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 1, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
     case 2: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 2, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
     case 4: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 4, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
     default: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 8, POOL>), grid, dim3(256 * NH), 0, s, a, q, g); break;
@@ -759,12 +760,18 @@ hipError_t launch_panel(const MexKernelArgs &a, const PoolArgs &q, const PanelAr
 }
 
 // Workgroup shape of the panel form for this layer (column halves), 0 when the layer does not have its geometry.
-int panel_halves(const MexPlan &p, int ph, int pw, const float *input, int slots, int n_mgroups, PanelArgs *g)
+int panel_halves(const MexPlan &p, int ph, int pw, const float *input, int slots, int n_mgroups, PanelArgs *g,
+                 bool pool)
 {
     if (slots <= 16)
         return 0;
     // one column half per workgroup while two would leave compute units without a workgroup
     const int pnh = ((long long)slots + 31) / 32 * n_mgroups < kPanelWorkgroups ? 1 : 2;
+    // a single chunk (32 channels): only the plain call on a small grid gains (64 x 32x16x16 -> 64: 7.2 -> 6.0 us per
+    // call, 512 images: 20.5 -> 21.3 us); with pooling the kernel above stays, and with it the first layer's results
+    // stay those of its form with the Similarity inside, bit for bit
+    if (p.d.K == 32 && (pool || pnh != 1))
+        return 0;
     if (panel_geometry(p, ph, pw, input, pnh, g))
         return pnh;
     return pnh == 1 && panel_geometry(p, ph, pw, input, 2, g) ? 2 : 0;
@@ -842,7 +849,7 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     if (ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
         nh = 4;
     PanelArgs pg;
-    const int panel = sp ? 0 : panel_halves(p, ph, pw, input, a.slots, n_mgroups, &pg);
+    const int panel = sp ? 0 : panel_halves(p, ph, pw, input, a.slots, n_mgroups, &pg, true);
     if (panel)
         nh = panel;
     q.spw = nh * 64 / (ph * pw);
@@ -876,13 +883,13 @@ bool mex_panel_geometry(const MexPlan &p)
         return false;
     // (the pointer is checked by the launch; any 16-byte aligned one stands in here)
     return panel_halves(p, 2, 2, reinterpret_cast<const float *>(uintptr_t(16)), (int)slots, (p.d.M + TM - 1) / TM,
-                        &g) != 0;
+                        &g, false) != 0;
 }
 
 int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *input, float *output, void *stream)
 {
     PanelArgs g;
-    const int nh = panel_halves(p, 2, 2, input, a.slots, a.n_mgroups, &g);
+    const int nh = panel_halves(p, 2, 2, input, a.slots, a.n_mgroups, &g, false);
     if (!nh)
         return SIMNETS_PANEL_NOT_TAKEN;
     PoolArgs q;

@@ -400,11 +400,11 @@ def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
 
 @pytest.mark.parametrize("im,n", [
     ((37, 64, 8, 8), 70), ((21, 128, 4, 4), 64), ((45, 256, 2, 2), 130), ((5, 64, 16, 16), 64), ((3, 64, 24, 16), 16),
-    ((2, 64, 4, 64), 16), ((64, 64, 16, 16), 256),
+    ((2, 64, 4, 64), 16), ((64, 64, 16, 16), 256), ((9, 32, 16, 16), 64), ((3, 32, 4, 8), 20),
 ])
 @pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("mixed", 3.0)])
 def test_mex_panel_form_of_the_plain_call(pkg, im, n, spread, eps):
-    # 2x2 unshared offsets over whole-channel patches of 64 / 128 / 256 channels: the plain MEX call runs the panel
+    # 2x2 unshared offsets over whole-channel patches of 32 / 64 / 128 / 256 channels: the plain MEX call runs the panel
     # kernel without its pooling; an input that is not 16-byte aligned takes the general tiled kernel on the same
     # packed offsets
     g = np.random.default_rng(46)
