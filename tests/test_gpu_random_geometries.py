@@ -116,6 +116,51 @@ def test_mex_random_geometry(pkg, seed):
                           orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "dOff %s" % kw)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_mex_whole_channel_layers_random_geometry(pkg, seed):
+    # 2x2 unshared offsets over all channels of a pixel, channel counts and power-of-two maps around what the panel
+    # kernel takes (and just outside: odd channel counts, widths that are no power of two), plain and with pooling
+    g = np.random.default_rng(7000 + seed)
+    C = int(g.choice([32, 64, 128, 256, 48, 96]))
+    H = int(g.choice([2, 4, 8, 16, 6]))
+    W = int(g.choice([2, 4, 8, 16, 32, 64, 12]))
+    B = int(g.integers(1, 24))
+    while B * C * H * W > 600_000:
+        B = max(1, B // 2)
+        if B == 1:
+            break
+    n = int(g.choice([1, 10, 16, 63, 64, 65, 130]))
+    if B * C * H * W * n > 30_000_000:
+        n = 10
+    eps = float(g.choice([1.0, 0.25, 4.0, -1.5]))
+    kw = dict(softmax_mode=bool(g.integers(0, 2)), blocks=[C, 1, 1], strides=[C, 1, 1], epsilon=eps,
+              use_unshared_regions=True, unshared_offset_region=[1, 2, 2])
+    x = (g.normal(size=(B, C, H, W)) * float(g.choice([0.5, 5.0, 40.0]))).astype(np.float32)
+    off = (g.normal(size=(4, n, C, 1, 1)) * float(g.choice([0.1, 1.0, 30.0]))).astype(np.float32)
+    if g.random() < 0.3:
+        off[:, n // 2:] *= 20
+    if g.random() < 0.3:
+        x[g.random(size=x.shape) < 0.1] = -math.inf if eps > 0 else math.inf
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = orc.mex_fwd(x, off, n, **kw)
+        shift = np.abs(orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, eps))))
+    got = pkg.mex(dev(x), dev(off), n, **kw).cpu().numpy()
+    fused = pkg.mex_sum_pool(dev(x), dev(off), n, (2, 2), **kw).cpu().numpy()
+    assert np.array_equal(np.isfinite(got), np.isfinite(want)), kw
+    fin = np.isfinite(want)
+    assert np.array_equal(got[~fin], want[~fin], equal_nan=True), kw
+    bar = np.maximum(np.abs(want), shift)
+    assert (np.abs(got[fin] - want[fin]) <= 1e-4 * np.maximum(bar[fin], 1e-30)).all(), kw
+
+    def pool(y):
+        return y.reshape(B, n, H // 2, 2, W // 2, 2).sum(axis=(3, 5))
+    with np.errstate(invalid="ignore"):
+        wantp, barp = pool(want), pool(bar)
+    finp = np.isfinite(wantp)
+    assert np.array_equal(np.isfinite(fused), finp), kw
+    assert (np.abs(fused[finp] - wantp[finp]) <= 1e-4 * np.maximum(barp[finp], 1e-30)).all(), kw
+
+
 def random_matrix_gradient_case(g):
     """Geometries the matrix-core gradient kernels take (L2 modes, at least 24 channels and 8 templates): small maps
     that share a workgroup tile, strides with two, four or more phases, contractions long enough to be split."""
