@@ -241,7 +241,9 @@ int simnets_hip_mex_workspace_bytes(const simnets_mex_attrs *attrs, const int in
 /* Forward: replaces MEXKernelGPU<float>::Compute (src/kernels/mex_kernel_gpu.cu:60-159), i.e. the
  * offsets copy + per-image im2col_3d_gpu + split_patches_gpu + ggemm_gpu (max pass) +
  * ggemm_readc_gpu (exp/sum/log pass) + reverse split_patches_gpu.
- * offsets_count = number of floats behind `offsets`; must be >= num_regions*num_instances*K. */
+ * offsets_count = number of floats behind `offsets`; must be >= num_regions*num_instances*K.
+ * `input` may have any float alignment; on layers with 2x2 unshared offsets over whole-channel patches a 16-byte
+ * aligned input takes a faster kernel, whose results differ from the general kernel's in the last bits. */
 int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                         const float *offsets, size_t offsets_count, float *output, void *workspace,
                         size_t workspace_bytes, void *stream);
@@ -252,7 +254,7 @@ int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4]
  * exponentials, row maxima and ranges, and the patch element table) into a caller-owned buffer of
  * simnets_hip_mex_workspace_bytes bytes (256-byte aligned) and simnets_hip_mex_fwd_prepared runs only the forward
  * kernel on it.  attrs and input_shape (batch size included) must be the ones the buffer was prepared with; results
- * are those of simnets_hip_mex_fwd bit for bit. */
+ * are those of simnets_hip_mex_fwd (on an input of the same alignment) bit for bit. */
 int simnets_hip_mex_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
                             size_t offsets_count, void *prepared, size_t prepared_bytes, void *stream);
 int simnets_hip_mex_fwd_prepared(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
