@@ -1032,9 +1032,25 @@ __global__ void sum_pool_kernel(const float *__restrict__ in, float *__restrict_
         out[idx] = acc;
     }
 }
-}  // namespace
 
-namespace {
+// 2x2 windows on maps whose width is a multiple of 4 (16-byte aligned tensors, fewer than 2^31 elements): a thread
+// takes two neighbouring windows - one 16-byte load per input row, one 8-byte store - and the row index comes from
+// a multiply-high instead of divisions.  Same order of additions as the kernel above.
+__global__ __launch_bounds__(256) void sum_pool_2x2_kernel(const float4 *__restrict__ in, float2 *__restrict__ out,
+                                                          unsigned pairs, unsigned W4, FastDiv dW4)
+{
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;   // (image-channel-output row, pair of windows)
+    if (idx >= pairs)
+        return;
+    const unsigned row = fast_div(idx, dW4);                // output row over all images and channels
+    const unsigned c = idx - row * W4;
+    const float4 a = in[(size_t)(2 * row) * W4 + c], b = in[(size_t)(2 * row + 1) * W4 + c];
+    float2 r;
+    r.x = (((0.0f + a.x) + a.y) + b.x) + b.y;
+    r.y = (((0.0f + a.z) + a.w) + b.z) + b.w;
+    out[idx] = r;
+}
+
 // gradient of the sum pooling: every input element of a window receives the window's gradient, the elements
 // of a dropped trailing row or column receive 0
 template <typename I>
@@ -1050,6 +1066,29 @@ __global__ void sum_pool_grad_kernel(const float *__restrict__ gout, float *__re
         gin[idx] = (ho < Ho && wo < Wo) ? gout[((size_t)bc * Ho + ho) * Wo + wo] : 0.0f;
     }
 }
+
+// ... and of the 2x2 case above: a thread reads the gradients of two neighbouring windows and writes their four input
+// elements of both rows
+__global__ __launch_bounds__(256) void sum_pool_grad_2x2_kernel(const float2 *__restrict__ gout, float4 *__restrict__ gin,
+                                                               unsigned pairs, unsigned W4, FastDiv dW4)
+{
+    const unsigned idx = blockIdx.x * 256u + threadIdx.x;
+    if (idx >= pairs)
+        return;
+    const unsigned row = fast_div(idx, dW4);
+    const unsigned c = idx - row * W4;
+    const float2 g = gout[idx];
+    const float4 v = make_float4(g.x, g.x, g.y, g.y);
+    gin[(size_t)(2 * row) * W4 + c] = v;
+    gin[(size_t)(2 * row + 1) * W4 + c] = v;
+}
+
+// the 2x2 kernels' case: even height, width a multiple of 4, 16-byte aligned tensors, 32-bit element counts
+bool pool_2x2_fast(long long planes, int H, int W, int ph, int pw, const void *full, const void *pooled)
+{
+    return ph == 2 && pw == 2 && H % 2 == 0 && W % 4 == 0 && planes * H * W < 0x7fffffffLL &&
+           reinterpret_cast<uintptr_t>(full) % 16 == 0 && reinterpret_cast<uintptr_t>(pooled) % 8 == 0;
+}
 }  // namespace
 
 int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float *output_grad, float *input_grad,
@@ -1058,8 +1097,15 @@ int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float
     const long long total = (long long)B * C * H * W;
     if (total == 0)
         return SIMNETS_OK;
-    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (pool_2x2_fast((long long)B * C, H, W, ph, pw, input_grad, output_grad)) {
+        const unsigned pairs = (unsigned)(total / 8), W4 = (unsigned)(W / 4);
+        hipLaunchKernelGGL(sum_pool_grad_2x2_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s,
+                           reinterpret_cast<const float2 *>(output_grad), reinterpret_cast<float4 *>(input_grad), pairs, W4,
+                           make_fast_div(W4));
+        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
     if (total + 256LL * blocks < 0x7fffffffLL)
         hipLaunchKernelGGL(sum_pool_grad_kernel<int>, dim3(blocks), dim3(256), 0, s, output_grad, input_grad, (int)total,
                            H, W, H / ph, W / pw, ph, pw);
@@ -1075,8 +1121,15 @@ int sum_pool_launch(int B, int C, int H, int W, int ph, int pw, const float *inp
     const long long total = (long long)B * C * Ho * Wo;
     if (total == 0)
         return SIMNETS_OK;
-    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+    if (pool_2x2_fast((long long)B * C, H, W, ph, pw, input, output)) {
+        const unsigned pairs = (unsigned)(total / 2), W4 = (unsigned)(W / 4);
+        hipLaunchKernelGGL(sum_pool_2x2_kernel, dim3((pairs + 255) / 256), dim3(256), 0, s,
+                           reinterpret_cast<const float4 *>(input), reinterpret_cast<float2 *>(output), pairs, W4,
+                           make_fast_div(W4));
+        return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+    }
+    const int blocks = (int)std::min<long long>((total + 255) / 256, 1 << 20);
     if (total + 256LL * blocks < 0x7fffffffLL)
         hipLaunchKernelGGL(sum_pool_kernel<int>, dim3(blocks), dim3(256), 0, s, input, output, (int)total, H, W, Ho, Wo,
                            ph, pw);

@@ -538,6 +538,30 @@ def test_sum_pooling(pkg):
     np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6)
 
 
+@pytest.mark.parametrize("shape", [(4, 6, 8, 16), (2, 3, 2, 4), (5, 7, 6, 28), (64, 64, 16, 16)])
+def test_sum_pooling_2x2_vector_kernels(pkg, shape):
+    # 2x2 windows on even heights and widths that are multiples of 4: the kernels that move 16 bytes per thread give
+    # what the general kernels give (taken here on a copy that is not 16-byte aligned), bit for bit, forward and gradient
+    g = np.random.default_rng(17)
+    x = dev(g.normal(size=shape).astype(np.float32))
+    B, Cc, H, W = shape
+    got = pkg.sum_pooling(x, (2, 2))
+    want = x.cpu().numpy().reshape(B, Cc, H // 2, 2, W // 2, 2).sum(axis=(3, 5))
+    np.testing.assert_allclose(got.cpu().numpy(), want, rtol=1e-6, atol=1e-6)
+    flat = torch.empty(x.numel() + 1, device="cuda")
+    shifted = flat[1:].view(*shape)
+    shifted.copy_(x)
+    assert shifted.data_ptr() % 16 == 4
+    assert torch.equal(got, pkg.sum_pooling(shifted, (2, 2)))
+    go = dev(g.normal(size=(B, Cc, H // 2, W // 2)).astype(np.float32))
+    gi = pkg.sum_pooling_input_grad(go, shape, (2, 2))
+    assert torch.equal(gi, go.repeat_interleave(2, dim=2).repeat_interleave(2, dim=3))
+    gflat = torch.empty(go.numel() + 1, device="cuda")
+    gshift = gflat[1:].view(*go.shape)
+    gshift.copy_(go)
+    assert torch.equal(gi, pkg.sum_pooling_input_grad(gshift, shape, (2, 2)))
+
+
 def test_missing_data_stack_end_to_end(pkg):
     # benchmark configuration 4 at a reduced batch: Similarity -> 4 x (MEX + 2x2 sum pool) -> MEX(10).
     # Each layer is checked on the GPU's own previous activations, so tolerances do not compound.
