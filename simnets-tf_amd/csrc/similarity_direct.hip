@@ -912,10 +912,12 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
 }
 
 // The sqrt-weight form runs on the tiled kernels and on the small-map kernel; there only with enough pixels per
-// parameter, or packing the second copy of the parameters costs more than the shorter inner loop saves.
+// parameter, or packing the second copy of the parameters costs more than the shorter inner loop saves (512
+// templates over 512 x 7 x 7 inputs: at 32 images 0.425 -> 0.391 ms per self-packing call and 0.413 -> 0.358 ms
+// prepared, at 16 images 0.222 -> 0.223 and 0.212 -> 0.190 ms, at 8 images the same ratios).
 bool use_sqrtw(const SimPlan &p, const Tiling &t)
 {
-    return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && (t.NI == 0 || (long long)p.B * p.oh * p.ow >= 4096);
+    return p.algo == SIMNETS_ALGO_SQRTW && t.lds_ok && (t.NI == 0 || (long long)p.B * p.oh * p.ow >= 512);
 }
 
 // flags of the guard that live in the workspace: one per workgroup of the small-map kernel (the tiled kernels keep
