@@ -752,7 +752,8 @@ struct Tiling {
     int NI;            // > 0: the small-map kernel with NI images per workgroup (CC, chan_pitch are then that kernel's)
     int sm_waves;      // ... and its waves per workgroup
     int chan_pitch;    // LDS floats of one staged channel
-    bool lds_ok;       // the rows of a workgroup's pixel groups fit the LDS tile (else: gather kernel)
+    bool lds_ok;       // the tiled kernels run: the rows of a workgroup's pixel groups fit the LDS tile and the
+                       // patches are not too short to be worth staging (else: gather kernel)
     bool fast_stage;   // ... and the division-free staging (at most kStagePos elements per thread and channel)
 };
 
@@ -783,6 +784,7 @@ Tiling try_tiling(const SimPlan &p, int PT, int MT, int nws)
     return t;
 }
 
+constexpr int kGatherMaxK = 12;            // patch lengths up to which the gather kernel replaces the tiled ones
 constexpr int kSmallMapLdsFloats = 8192;   // 32 KiB of tile per workgroup of the small-map kernel; twice that when the
                                            // grid has at most two workgroups per compute unit (half as many chunk phases)
 
@@ -820,6 +822,15 @@ Tiling choose_tiling(const SimPlan &p)
             return big;
     }
     Tiling t = pick(kSmallPT, kSmallMT);
+    // Short patches (the 2x2 first layer of the missing-data network, 1x1 and 3x3 patches of one channel): a pixel's
+    // whole patch is a handful of loads, and staging rows through LDS behind a barrier only adds dependent phases -
+    // one pixel per lane straight from global memory, four template tiles per pixel group of 256 (1x28x28 -> 32, 2x2
+    // s2 p2: 8.3 -> 4.0 us per prepared call at 64 images, 11.6 -> 9.5 at 512, 26.3 -> 24.8 at 2048; 3x3 of one channel
+    // 10.2 -> 6.6 / 28.2 -> 25.0; 12 elements 11.8 -> 8.1 / 37.7 -> 33.5; 16 and more: no gain on large grids)
+    if (p.K <= kGatherMaxK) {
+        t.lds_ok = false;
+        return t;
+    }
     // Small maps: a whole image is one tile of at most 64 pixel groups, and either several images fit a wave or the
     // tiled grid has at most one wave per SIMD while K is long enough to split over the four waves.
     if (t.lds_ok && t.nws == 1 && t.tiles == 1 && p.C >= kSmWaves) {
