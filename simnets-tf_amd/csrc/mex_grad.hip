@@ -247,6 +247,25 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     const int mg_begin = blockIdx.z * ga.mg_per_split, mg_end = min(n_mg, mg_begin + ga.mg_per_split);
     float *dxo = ga.msplit > 1 ? ga.dx_splits + (size_t)blockIdx.z * a.B * a.C * a.H * a.W : ga.dx;
     const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
+    // (everything the product form reads first is requested before the barriers that decide on it: the pixel, its
+    // table entries, the first output value of the bound, the patch element records of this lane's gradients)
+    const int lr = lane & 15, lq = lane >> 4;
+    int4 kel[4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v)
+        kel[v] = a.ktab[min(k0 + wave * 16 + 4 * lq + v, a.K - 1)];
+    const PixelRef px = locate(a, r, chunk * 64 + lane);
+    const bool valid = px.out_off >= 0;
+    if (wave == 0) {
+        pb[lane] = valid ? px.b : -1;
+        pc0[lane] = px.ci0; ph0[lane] = px.hi0; pw0[lane] = px.wi0;
+        pout[lane] = px.out_off;
+    }
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const float o_first = op[(size_t)min(wave, a.M - 1) * plane];
+    const float lo_first = omax_r[min(wave, a.M - 1)] - orng_r[min(wave, a.M - 1)];
     int roomy;  // some instance's offsets range is large enough for the choice of the bound to matter (below)
     {
         int wide = 0, big = 0;
@@ -266,16 +285,6 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             return;
         }
     }
-    const PixelRef px = locate(a, r, chunk * 64 + lane);
-    const bool valid = px.out_off >= 0;
-    if (wave == 0) {
-        pb[lane] = valid ? px.b : -1;
-        pc0[lane] = px.ci0; ph0[lane] = px.hi0; pw0[lane] = px.wi0;
-        pout[lane] = px.out_off;
-    }
-    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
-    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
-    const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const bool buffered = ga.wbuf != nullptr;   // W and 2^(xs - a) come from mex_grad_factors_kernel
     const size_t row0 = (size_t)r * ga.slots_pad + (size_t)chunk * 64;
     // the pixel's bound a = min_m (outs_m - c0 - lo_m).  Every single term of the minimum is a valid bound
@@ -286,7 +295,8 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     const int m_scan = buffered ? 0 : (roomy ? a.M : min(a.M, 4));
     float amin = INFINITY;
     for (int m = wave; m < m_scan; m += 4)
-        amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
+        amin = fminf(amin, m == wave ? __builtin_fmaf(o_first, a.c1, -(a.c0 + lo_first))
+                                     : __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
     pmn[wave * 64 + lane] = amin;
     __syncthreads();
     if (wave == 0)
@@ -294,17 +304,67 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     __syncthreads();
     const float a_p = ap[lane];
 
-    const int lr = lane & 15, lq = lane >> 4;
+    // where this lane's 16 gradients go (the pixel tables are in place behind the barriers above) and the input
+    // values their factors 2^(xs_k - a) are made of: requested here, used after the matrix loop (a load in front of
+    // each store made the lane wait for 16 memory round trips in turn, 45 % of the kernel on a 64 x 32 x 16 x 16 -> 64
+    // layer)
+    const size_t chw = (size_t)a.C * a.H * a.W;
+    size_t at[4][4];
+    float xin[4][4];
+    bool ok[4][4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int k = k0 + wave * 16 + 4 * lq + v;
+        const int dc = kel[v].y, dh = kel[v].z, dw = kel[v].w;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const int p = t * 16 + lr;
+            const int b = pb[p];
+            const int ci = pc0[p] + dc, hi = ph0[p] + dh, wi = pw0[p] + dw;
+            ok[v][t] = k < a.K && b >= 0 && ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+            at[v][t] = ok[v][t] ? (size_t)b * chw + ((size_t)ci * a.H + hi) * a.W + wi : 0;
+            if (buffered)
+                xin[v][t] = ga.exbuf[ok[v][t] ? (row0 + p) * ga.Kp + k : 0];
+            else
+                xin[v][t] = a.in[at[v][t]];
+        }
+    }
+
     floatx4 acc[4];
 #pragma unroll
     for (int t = 0; t < 4; ++t)
         acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    // operands of an instance group: the offsets tile (two float4 per thread) and, unless the pixel factors come from
+    // the buffers, this thread's eight output and gradient values - requested a group ahead
+    constexpr int EO4 = GM_KT * (GM_TM / 4) / 256;
+    float4 eo_n[EO4];
+    float ov_n[GM_TM / 4], gv_n[GM_TM / 4], om_n[GM_TM / 4];
+    auto request = [&](int mg) {
+        const float4 *src = reinterpret_cast<const float4 *>(a.offe + (((size_t)r * n_mg + mg) * a.K + k0) * GM_TM);
+#pragma unroll
+        for (int j = 0; j < EO4; ++j) {
+            const int i = tid + j * 256;
+            eo_n[j] = k0 + i / (GM_TM / 4) < a.K ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+        if (!buffered) {
+#pragma unroll
+            for (int i = 0; i < GM_TM / 4; ++i) {
+                const int m = min(mg * GM_TM + wave + 4 * i, a.M - 1);
+                ov_n[i] = op[(size_t)m * plane];
+                gv_n[i] = gp[(size_t)m * plane];
+                om_n[i] = omax_r[m];
+            }
+        }
+    };
+    if (mg_begin < mg_end)
+        request(mg_begin);
     for (int mg = mg_begin; mg < mg_end; ++mg) {
         __syncthreads();  // the previous chunk's matrix instructions are done with eo / wt
-        const float4 *src = reinterpret_cast<const float4 *>(a.offe + (((size_t)r * n_mg + mg) * a.K + k0) * GM_TM);
-        for (int i = tid; i < GM_KT * (GM_TM / 4); i += 256) {
+#pragma unroll
+        for (int j = 0; j < EO4; ++j) {
+            const int i = tid + j * 256;
             const int row = i / (GM_TM / 4), c4 = i % (GM_TM / 4);
-            const float4 v = k0 + row < a.K ? src[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            const float4 v = eo_n[j];
             float *d = eo + row * (GM_TM + 1) + 4 * c4;
             d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
         }
@@ -321,12 +381,14 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
                 float w = 0.0f;
                 if (valid && m < a.M) {
                     // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
-                    const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
-                    w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+                    const float e = __builtin_fmaf(-ov_n[i], a.c1, a_p) + (om_n[i] + a.c0);
+                    w = gv_n[i] * __builtin_amdgcn_exp2f(e);
                 }
                 wt[mm * 65 + lane] = w;
             }
         }
+        if (mg + 1 < mg_end)
+            request(mg + 1);   // in flight during the matrix steps
         __syncthreads();
 #pragma unroll
         for (int ms = 0; ms < GM_TM; ms += 4) {
@@ -337,30 +399,20 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
         }
     }
     // ---- d patch_k = 2^(xs_k - a) * acc, scattered to the input element the patch element is ----
-    const size_t chw = (size_t)a.C * a.H * a.W;
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int k = k0 + wave * 16 + 4 * lq + v;
-        if (k >= a.K)
-            continue;
-        const int4 ke = a.ktab[k];
-        const int dc = ke.y, dh = ke.z, dw = ke.w;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
+            if (!ok[v][t])
+                continue;
             const int p = t * 16 + lr;
-            const int b = pb[p];
-            if (b < 0)
-                continue;
-            const int ci = pc0[p] + dc, hi = ph0[p] + dh, wi = pw0[p] + dw;
-            if (!(ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W))
-                continue;
-            const size_t at = (size_t)b * chw + ((size_t)ci * a.H + hi) * a.W + wi;
-            const float val = acc[t][v] * (buffered ? ga.exbuf[(row0 + p) * ga.Kp + k]
-                                                    : __builtin_amdgcn_exp2f(__builtin_fmaf(a.in[at], a.c1, -ap[p])));
+            const float val = acc[t][v] * (buffered ? xin[v][t]
+                                                    : __builtin_amdgcn_exp2f(__builtin_fmaf(xin[v][t], a.c1, -ap[p])));
             if (ga.overlap)
-                ga.col[((size_t)b * plane + pout[p]) * a.K + k] = val;
+                ga.col[((size_t)pb[p] * plane + pout[p]) * a.K + k] = val;
             else
-                dxo[at] = val;
+                dxo[at[v][t]] = val;
         }
     }
 }
@@ -540,6 +592,9 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
         acc[t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
     // this thread's instances when staging (16 of the tile, the same for the whole wave) and their constants
     const int ms0 = m0 + wave * 16;
+    // the records of the wave's 16 patch elements: one vector load (lane i holds element i), read back lane by lane
+    // where they are used - as 16 wave-uniform loads in front of the 16 gathers each was waited for on its own
+    const int4 kl = a.ktab[min(k0 + wave * 16 + (lane & 15), a.K - 1)];
     const bool buffered = ga.wbuf != nullptr;   // W and 2^(xs - a) come from mex_grad_factors_kernel
     // global loads of a group of 64 pixel slots: this thread's pixel, its 16 instances' output and gradient values
     // and 16 of the tile's patch elements; the loads of group s + 1 are issued before group s is processed
@@ -567,10 +622,12 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             const int k = k0 + wave * 16 + i;
             q.xr[i] = 0.0f;
             if (q.valid && k < a.K) {
-                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
-                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
+                // {offset inside an image, dc, dh, dw} of element i
+                const int kx = __builtin_amdgcn_readlane(kl.x, i), ky = __builtin_amdgcn_readlane(kl.y, i);
+                const int kz = __builtin_amdgcn_readlane(kl.z, i), kw = __builtin_amdgcn_readlane(kl.w, i);
+                const int ci = px.ci0 + ky, hi = px.hi0 + kz, wi = px.wi0 + kw;
                 const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-                q.xr[i] = ok ? px.base[ke.x] : a.oob;
+                q.xr[i] = ok ? px.base[kx] : a.oob;
             }
         }
     };
