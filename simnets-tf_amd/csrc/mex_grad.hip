@@ -703,17 +703,26 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     }
     // ---- partial sums of this pixel chunk: acc * 2^(os_mk - mo_m) ----
     float *dst = ga.partial + ((size_t)chunk * a.R + r) * a.M * a.K;
+    // (the 16 offset exponentials first, on clamped indices, then the products and stores)
+    float eov[4][4];
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int m = min(m0 + wave * 16 + 4 * lq + v, a.M - 1);
+        const float *eo = a.offe + (((size_t)r * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            eov[v][t] = eo[(size_t)min(k0 + t * 16 + lr, a.K - 1) * GM_TM];
+    }
 #pragma unroll
     for (int v = 0; v < 4; ++v) {
         const int m = m0 + wave * 16 + 4 * lq + v;
         if (m >= a.M)
             continue;
-        const float *eo = a.offe + (((size_t)r * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
             const int k = k0 + t * 16 + lr;
             if (k < a.K)
-                dst[(size_t)m * a.K + k] = acc[t][v] * eo[(size_t)k * GM_TM];
+                dst[(size_t)m * a.K + k] = acc[t][v] * eov[v][t];
         }
     }
 }

@@ -271,6 +271,9 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
         // ---- store: lane holds A (tile 0) and B (tile 1) of 16 channels of one pixel ----
         const size_t xplane = (size_t)a.x_plane;
         float *out = a.nsplit > 1 ? a.part + split * a.part_stride : a.out;
+        // (per pixel the 16 input values and channel centres are loaded first, on clamped channel indices, then the
+        // 16 gradients are formed and stored: with each load under its channel bound, in front of its store, a lane
+        // waited for 64 memory round trips in turn)
 #pragma unroll
         for (int j = 0; j < RP; ++j) {
             if (pimg[j] < 0)
@@ -279,14 +282,20 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
             const float *xb = a.x + (size_t)pimg[j] * a.x_channels * xplane;
             const int pr = pix[j] / g.ow, pc = pix[j] - pr * g.ow;
             const size_t at = (size_t)(g.oy0 + pr * a.oys) * a.x_w + (g.ox0 + pc * a.oxs);
+            float xin[16], cen[16];
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int ch = min(mbase + 8 * (v / 4) + 4 * half + (v % 4), a.x_channels - 1);
+                xin[v] = xb[(size_t)ch * xplane + at];
+                cen[v] = a.ctr[ch];
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int ch = mbase + 8 * (v / 4) + 4 * half + (v % 4);
                 if (ch >= a.x_channels)
                     continue;
-                const float xin = xb[(size_t)ch * xplane + at];
-                float d = __builtin_fmaf(-(xin - a.ctr[ch]), acc[1][j][v], acc[0][j][v]);
-                if (a.ignore_nan && xin != xin)
+                float d = __builtin_fmaf(-(xin[v] - cen[v]), acc[1][j][v], acc[0][j][v]);
+                if (a.ignore_nan && xin[v] != xin[v])
                     d = 0.0f;
                 ob[(size_t)ch * xplane + at] = d;
             }
@@ -472,14 +481,20 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_grad_strided_kernel(cons
             if (pos_h[j] < 0 || y >= x_h || xx >= a.x_w)
                 continue;
             const size_t at = (size_t)y * a.x_w + xx;
+            float xin[16], cen[16];   // loaded first, on clamped channel indices (see sim_mfma_kernel)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int ch = min(mbase + 8 * (v / 4) + 4 * half + (v % 4), a.x_channels - 1);
+                xin[v] = xb[(size_t)ch * xplane + at];
+                cen[v] = a.ctr[ch];
+            }
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const int ch = mbase + 8 * (v / 4) + 4 * half + (v % 4);
                 if (ch >= a.x_channels)
                     continue;
-                const float xin = xb[(size_t)ch * xplane + at];
-                float d = __builtin_fmaf(-(xin - a.ctr[ch]), acc[1][f * PB + j][v], acc[0][f * PB + j][v]);
-                if (a.ignore_nan && xin != xin)
+                float d = __builtin_fmaf(-(xin[v] - cen[v]), acc[1][f * PB + j][v], acc[0][f * PB + j][v]);
+                if (a.ignore_nan && xin[v] != xin[v])
                     d = 0.0f;
                 ob[(size_t)ch * xplane + at] = d;
             }
