@@ -33,13 +33,25 @@ def _fill(dst, values, cap):
 
 _workspaces = {}
 
+# The current stream's handle without building a torch.cuda.Stream object (a few microseconds per call, as much as
+# a small kernel runs); the public API where this build of torch lacks the direct accessor.
+_raw_stream_of = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
-def _workspace(device, nbytes):
+
+def _current_stream(device):
+    if _raw_stream_of is not None:
+        return _raw_stream_of(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _workspace(device, nbytes, stream=None):
     """A scratch tensor per (device, current stream), grown on demand and reused across calls: the kernels that
     use it are ordered on that stream, and calls on different streams never share one."""
     # a buffer first allocated during stream capture lives in that graph's private pool: kept apart from the
     # eager calls' buffer, which a later replay of the graph must not share
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream, torch.cuda.is_current_stream_capturing())
+    if stream is None:
+        stream = _current_stream(device)
+    key = (device.index, stream, torch.cuda.is_current_stream_capturing())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
@@ -50,15 +62,35 @@ def _workspace(device, nbytes):
 _plans = {}
 
 
+_PLAIN_KEY_TYPES = frozenset((int, str, bool, type(None), torch.Size))
+
+
+def _freeze(v):
+    if isinstance(v, (list, tuple)):
+        return tuple(_freeze(e) for e in v)
+    if isinstance(v, dict):
+        return tuple(sorted((k, _freeze(e)) for k, e in v.items()))
+    return repr(v) if isinstance(v, float) else v
+
+
+def _key_part(v):
+    t = type(v)
+    if t in _PLAIN_KEY_TYPES:
+        return v
+    if t is float:
+        return repr(v)
+    if t is list or t is tuple:
+        for e in v:
+            if type(e) is not int:
+                return _freeze(v)
+        return tuple(v)
+    return _freeze(v)
+
+
 def _plan_key(*parts):
-    """Hashable key of shapes and attribute values (floats by repr: NaN out-of-bounds values must compare equal)."""
-    def freeze(v):
-        if isinstance(v, (list, tuple)):
-            return tuple(freeze(e) for e in v)
-        if isinstance(v, dict):
-            return tuple(sorted((k, freeze(e)) for k, e in v.items()))
-        return repr(v) if isinstance(v, float) else v
-    return freeze(parts)
+    """Hashable key of shapes and attribute values (floats by repr: NaN out-of-bounds values must compare equal).
+    Called on every op call: values of the usual plain types and lists of ints take the short way."""
+    return tuple([v if type(v) in _PLAIN_KEY_TYPES else _key_part(v) for v in parts])
 
 
 def _cached_plan(key, make):
@@ -170,13 +202,13 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
         _plan_key("similarity", x.shape, t.shape, w.shape, similarity_function, blocks, strides, padding,
                   normalization_term, normalization_term_fudge, ignore_nan_input, out_of_bounds_value, algo,
                   norm_const_every_iteration), make)
-    ws = _workspace(x.device, nbytes)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes, stream)
     if out is None:
         out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_fwd(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                             out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out
@@ -189,13 +221,18 @@ def _similarity_grad_setup(input, templates, weights, output_grad, kw):
     g = _require_cuda_f32("output_grad", output_grad)
     if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
         raise SimnetsError(-15)
-    a = similarity_attrs(**kw)
     l = _lib.lib()
-    I4 = C.c_int * 4
-    xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
-    oshape = I4()
-    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
-    if tuple(g.shape) != tuple(oshape):
+
+    def make():
+        a = similarity_attrs(**kw)
+        I4 = C.c_int * 4
+        xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
+        oshape = I4()
+        _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
+        return a, xs, ts, wsh, tuple(oshape)
+
+    a, xs, ts, wsh, oshape = _cached_plan(_plan_key("similarity_grad", x.shape, t.shape, w.shape, *kw.values()), make)
+    if tuple(g.shape) != oshape:
         raise SimnetsError(-15)
     return l, a, x, t, w, g, xs, ts, wsh
 
@@ -211,10 +248,10 @@ def similarity_input_grad(input, templates, weights, output_grad, similarity_fun
         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes), None))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     dx = torch.empty_like(x)
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_input_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                                    g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return dx
@@ -234,10 +271,10 @@ def similarity_parameters_grad(input, templates, weights, output_grad, similarit
         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, None, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     dt, dw = torch.empty_like(t), torch.empty_like(w)
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_params_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(),
                                                     w.data_ptr(), g.data_ptr(), dt.data_ptr(), dw.data_ptr(),
                                                     ws.data_ptr(), ws.numel(), stream))
@@ -353,13 +390,13 @@ def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=
         _plan_key("mex", x.shape, num_instances, softmax_mode, padding, strides, blocks, epsilon,
                   blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
                   unshared_offset_region, normalize_offsets), make)
-    ws = _workspace(x.device, nbytes)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes, stream)
     if out is None:
         out = torch.empty(oshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
                                      ws.data_ptr(), ws.numel(), stream))
     return out
@@ -372,12 +409,17 @@ def _mex_grad_setup(input, offsets, output, output_grad, num_instances, kw):
     g = _require_cuda_f32("output_grad", output_grad)
     if x.dim() != 4:
         raise SimnetsError(-15)
-    a = mex_attrs(num_instances, **kw)
     l = _lib.lib()
-    xs = (C.c_int * 4)(*x.shape)
-    oshape = (C.c_int * 4)()
-    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-    if tuple(y.shape) != tuple(oshape) or tuple(g.shape) != tuple(oshape):
+
+    def make():
+        a = mex_attrs(num_instances, **kw)
+        xs = (C.c_int * 4)(*x.shape)
+        oshape = (C.c_int * 4)()
+        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
+        return a, xs, tuple(oshape)
+
+    a, xs, oshape = _cached_plan(_plan_key("mex_grad", x.shape, num_instances, *kw.values()), make)
+    if tuple(y.shape) != oshape or tuple(g.shape) != oshape:
         raise SimnetsError(-15)
     return l, a, x, off, y, g, xs
 
@@ -395,10 +437,10 @@ def mex_input_grad(input, offsets, output, output_grad, num_instances, softmax_m
         unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, C.byref(nbytes), None))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     dx = torch.empty_like(x)
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_input_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
                                             g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return dx
@@ -417,10 +459,10 @@ def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax
         unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, None, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     doff = torch.empty_like(off)
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_offsets_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
                                               g.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return doff
@@ -440,10 +482,10 @@ def mex_grads(input, offsets, output, output_grad, num_instances, softmax_mode=N
         unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
     nbytes = C.c_size_t()
     _check(l.simnets_hip_mex_grads_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     dx, doff = torch.empty_like(x), torch.empty_like(off)
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_grads(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
                                        g.data_ptr(), dx.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(),
                                        stream))
@@ -481,13 +523,13 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
         _plan_key("mex_sum_pool", x.shape, num_instances, ph, pw, softmax_mode, padding, strides, blocks, epsilon,
                   blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
                   unshared_offset_region, normalize_offsets), make)
-    ws = _workspace(x.device, nbytes)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes, stream)
     if out is None:
         out = torch.empty(pshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_mex_sum_pool_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), ph, pw,
                                               out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
     return out
@@ -518,14 +560,14 @@ def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, p
     nbytes = C.c_size_t()
     _check(l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), xs, ts, C.byref(ma), ph, pw,
                                                                  C.byref(nbytes)))
-    ws = _workspace(x.device, nbytes.value)
+    stream = _current_stream(x.device)
+    ws = _workspace(x.device, nbytes.value, stream)
     pshape = (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw)
     if out is None:
         out = torch.empty(pshape, dtype=torch.float32, device=x.device)
     else:
         assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
         _check(l.simnets_hip_similarity_mex_sum_pool_fwd(C.byref(sa), xs, ts, x.data_ptr(), t.data_ptr(), w.data_ptr(),
                                                          C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
                                                          out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
@@ -547,7 +589,7 @@ def sum_pooling(input, pool_size=(2, 2), out=None):
         assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32 \
             and out.device == x.device
     with _on_device(x.device):
-        stream = torch.cuda.current_stream(x.device).cuda_stream
+        stream = _current_stream(x.device)
         _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),
                                                    stream))
     return out
@@ -563,7 +605,7 @@ def sum_pooling_input_grad(output_grad, input_shape, pool_size=(2, 2)):
         raise SimnetsError(-15)
     dx = torch.empty((B, Cc, H, W), dtype=torch.float32, device=g.device)
     with _on_device(g.device):
-        stream = torch.cuda.current_stream(g.device).cuda_stream
+        stream = _current_stream(g.device)
         _check(_lib.lib().simnets_hip_sum_pool_input_grad((C.c_int * 4)(B, Cc, H, W), ph, pw, g.data_ptr(),
                                                           dx.data_ptr(), stream))
     return dx
@@ -607,10 +649,10 @@ class Prepared:
             raise ValueError("out must be a contiguous float32 tensor of shape %s on %s"
                              % (self.output_shape, self._device))
         if torch.cuda.current_device() == self._index:
-            code = self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+            code = self._run(x.data_ptr(), out.data_ptr(), _current_stream(self._device))
         else:
             with torch.cuda.device(self._device):
-                code = self._run(x.data_ptr(), out.data_ptr(), torch.cuda.current_stream().cuda_stream)
+                code = self._run(x.data_ptr(), out.data_ptr(), _current_stream(self._device))
         if code != 0:
             raise SimnetsError(code)
         return out
@@ -642,7 +684,7 @@ def similarity_prepare(input_shape, templates, weights, similarity_function=None
     _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
     buf = _prepared_buffer(t.device, nbytes.value)
     with _on_device(t.device):
-        stream = torch.cuda.current_stream(t.device).cuda_stream
+        stream = _current_stream(t.device)
         _check(l.simnets_hip_similarity_prepare(C.byref(a), xs, ts, wsh, t.data_ptr(), w.data_ptr(), buf.data_ptr(),
                                                 buf.numel(), stream))
 
@@ -667,7 +709,7 @@ def mex_prepare(input_shape, offsets, num_instances, normalize_offsets=False, **
     _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
     buf = _prepared_buffer(off.device, nbytes.value)
     with _on_device(off.device):
-        stream = torch.cuda.current_stream(off.device).cuda_stream
+        stream = _current_stream(off.device)
         _check(l.simnets_hip_mex_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), buf.data_ptr(), buf.numel(),
                                          stream))
 
@@ -693,7 +735,7 @@ def mex_sum_pool_prepare(input_shape, offsets, num_instances, pool_size=(2, 2), 
     _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
     buf = _prepared_buffer(off.device, nbytes.value)
     with _on_device(off.device):
-        stream = torch.cuda.current_stream(off.device).cuda_stream
+        stream = _current_stream(off.device)
         _check(l.simnets_hip_mex_sum_pool_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), ph, pw, buf.data_ptr(),
                                                   buf.numel(), stream))
 
@@ -726,7 +768,7 @@ def similarity_mex_sum_pool_prepare(input_shape, templates, weights, offsets, nu
                                                                  C.byref(nbytes)))
     buf = _prepared_buffer(t.device, nbytes.value)
     with _on_device(t.device):
-        stream = torch.cuda.current_stream(t.device).cuda_stream
+        stream = _current_stream(t.device)
         _check(l.simnets_hip_similarity_mex_sum_pool_prepare(C.byref(sa), xs, ts, t.data_ptr(), w.data_ptr(),
                                                              C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
                                                              buf.data_ptr(), buf.numel(), stream))
