@@ -72,6 +72,9 @@ struct SimKernelArgs {
     const float *pa2;  // [mtile][K][MT][2]  (template, negative weight): what the recomputing pass reads
     const float *thr;  // [O] a partial sum of template m above -thr[m] sends its wave to the recomputing pass
     int *flags;        // [workgroups * kWaves] 1: the wave left its outputs to the recomputing pass
+    // self-packing gather kernel only: the parameters as the caller holds them, [O][K] each
+    const float *raw_t, *raw_w;
+    float fudge;
 };
 
 // Output positions of a lane.
@@ -126,6 +129,7 @@ __device__ __forceinline__ void load_params(float (&pa)[2 * MT], float (&pc)[MT]
 #endif
 constexpr int kBigPT = SIMNETS_BIG_PT, kBigMT = SIMNETS_BIG_MT;
 constexpr int kSmallPT = 4, kSmallMT = 8;
+constexpr int kGatherMaxK = 12;            // patch lengths up to which the gather kernel replaces the tiled ones
 constexpr int kSmStageGroups = 2;   // small-map kernel: channel groups whose loads are in flight at once while staging
 // waves per SIMD the register budget is sized for: 64 accumulators leave room for 4, 128 for 2
 constexpr int waves_per_simd(int pt, int mt) { return pt * mt <= 64 ? 4 : 2; }
@@ -683,6 +687,83 @@ __global__ __launch_bounds__(256) void sim_gather_kernel(const SimKernelArgs a)
     }
 }
 
+// The gather kernel for patches of at most kGatherMaxK elements when the caller's parameters have not been packed
+// (the self-packing forward call): the workgroup packs the parameters of its template tile into LDS itself (the same
+// sim_pack_element, so the same values) and reads them from there, which saves the pack launch, at this size as long
+// as the kernel itself.  Same order over k, same combine step: results identical to sim_gather_kernel's.
+template <int MODE, int MT>
+__global__ __launch_bounds__(256) void sim_gather_selfpack_kernel(const SimKernelArgs a)
+{
+    constexpr bool HAS_PC = MODE == SIM_MODE_L2_NORM || MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
+    __shared__ float spa[kGatherMaxK * 2 * MT];
+    __shared__ float spc[kGatherMaxK * MT];
+    const int mtile = blockIdx.y;
+    for (int i = threadIdx.x; i < a.K * MT; i += 256) {
+        const int k = i / MT, m = mtile * MT + (i - k * MT);
+        float t = 0.0f, w = 0.0f;
+        if (m < a.O) {
+            t = a.raw_t[(size_t)m * a.K + k];
+            w = a.raw_w[(size_t)m * a.K + k];
+        }
+        sim_pack_element(MODE, m < a.O, t, w, a.fudge, spa[2 * i], spa[2 * i + 1], spc[i]);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const long long pix0 = ((long long)blockIdx.x * kWaves + wave) * 64;
+    const long long npix = (long long)a.B * a.oh * a.ow;
+    if (pix0 >= npix)
+        return;
+    long long pix = pix0 + lane;
+    const bool lane_valid = pix < npix;
+    if (!lane_valid)
+        pix = npix - 1;
+    const int b = (int)(pix / (a.oh * a.ow));
+    const int rem = (int)(pix - (long long)b * a.oh * a.ow);
+    const int h = rem / a.ow, w = rem - h * a.ow;
+    const float *img = a.in + (size_t)b * a.C * a.H * a.W;
+    const float *pa = spa, *pc = spc;
+    float acc[MT][1];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+        acc[m][0] = 0.0f;
+    for (int c = 0; c < a.C; ++c)
+        for (int dh = 0; dh < a.bh; ++dh) {
+            const int ih = h * a.sh - a.ph + dh;
+            for (int dw = 0; dw < a.bw; ++dw) {
+                const int iw = w * a.sw - a.pw + dw;
+                float x[1] = {a.oob};
+                if (ih >= 0 && ih < a.H && iw >= 0 && iw < a.W)
+                    x[0] = img[((size_t)c * a.H + ih) * a.W + iw];
+                float pav[2 * MT], pcv[MT];
+#pragma unroll
+                for (int i = 0; i < 2 * MT; ++i)
+                    pav[i] = pa[i];
+#pragma unroll
+                for (int i = 0; i < MT; ++i)
+                    pcv[i] = HAS_PC ? pc[i] : 0.0f;
+                sim_step<MODE, 1, MT, true>(acc, x, pav, pcv);
+                pa += 2 * MT;
+                pc += MT;
+            }
+        }
+    if (!lane_valid)
+        return;
+    int reps = 0;
+    if (MODE == SIM_MODE_L2_NORM)
+        reps = a.norm_every_iteration ? (a.B - b) : 1;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int mm = mtile * MT + m;
+        if (mm >= a.O)
+            break;
+        float v = acc[m][0];
+        for (int r = 0; r < reps; ++r)
+            v += a.norm_const;
+        a.out[(((size_t)b * a.O + mm) * a.oh + h) * a.ow + w] = v;
+    }
+}
+
 // Packs (template, weight) into the k-major, MT-interleaved layout the parameter loads walk, with
 // the sign and the 1/2 of the normalized modes folded into the weight, and precomputes the
 // per-(m,k) logarithm term.  Replaces interlace_kernel (include/utils/ggemm.cuh:70-87).
@@ -784,7 +865,6 @@ Tiling try_tiling(const SimPlan &p, int PT, int MT, int nws)
     return t;
 }
 
-constexpr int kGatherMaxK = 12;            // patch lengths up to which the gather kernel replaces the tiled ones
 constexpr int kSmallMapLdsFloats = 8192;   // 32 KiB of tile per workgroup of the small-map kernel; twice that when the
                                            // grid has at most two workgroups per compute unit (half as many chunk phases)
 
@@ -889,7 +969,10 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     if (!t.lds_ok) {
         const long long npix = (long long)a.B * a.oh * a.ow;
         dim3 grid((unsigned)((npix + 255) / 256), (unsigned)a.n_mtiles);
-        if (t.MT == 4)
+        if (a.raw_t != nullptr) {
+            if constexpr (MODE != SIM_MODE_L2_SQRTW && !GATED)
+                hipLaunchKernelGGL((sim_gather_selfpack_kernel<MODE, kSmallMT>), grid, dim3(256), 0, s, a);
+        } else if (t.MT == 4)
             hipLaunchKernelGGL((sim_gather_kernel<MODE, 4>), grid, dim3(256), 0, s, a);
         else if (t.MT == 16)
             hipLaunchKernelGGL((sim_gather_kernel<MODE, 16>), grid, dim3(256), 0, s, a);
@@ -994,9 +1077,16 @@ int sim_direct_prepare(const SimPlan &p, const float *templates, const float *we
     return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
-// The forward launches on a prepared workspace.
-int sim_direct_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
-                   hipStream_t s)
+// The self-packing call of a short-patch geometry on the gather kernel needs no packed parameters.
+static bool gather_packs_itself(const SimPlan &p, const Tiling &t)
+{
+    return !t.lds_ok && p.K <= kGatherMaxK && t.MT == kSmallMT;
+}
+
+// raw_templates / raw_weights: non-null for a geometry that packs inside the kernel (gather_packs_itself).
+static int sim_direct_run_on(const SimPlan &p, const float *input, float *output, void *workspace,
+                             size_t workspace_bytes, hipStream_t s, const float *raw_templates,
+                             const float *raw_weights)
 {
     const Tiling t = choose_tiling(p);
     const Layout l = layout(p, t);
@@ -1028,6 +1118,7 @@ int sim_direct_run(const SimPlan &p, const float *input, float *output, void *wo
     a.pa2 = reinterpret_cast<const float *>(ws + l.pa2);
     a.thr = reinterpret_cast<const float *>(ws + l.thr);
     a.flags = reinterpret_cast<int *>(ws + l.flags);
+    a.raw_t = raw_templates; a.raw_w = raw_weights; a.fudge = p.fudge;
 
     const bool plds = use_plds(p, t);
     hipError_t e;
@@ -1043,9 +1134,18 @@ int sim_direct_run(const SimPlan &p, const float *input, float *output, void *wo
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
+// The forward launches on a prepared workspace.
+int sim_direct_run(const SimPlan &p, const float *input, float *output, void *workspace, size_t workspace_bytes,
+                   hipStream_t s)
+{
+    return sim_direct_run_on(p, input, output, workspace, workspace_bytes, s, nullptr, nullptr);
+}
+
 int sim_direct_launch(const SimPlan &p, const float *input, const float *templates, const float *weights,
                       float *output, void *workspace, size_t workspace_bytes, hipStream_t s)
 {
+    if (gather_packs_itself(p, choose_tiling(p)))
+        return sim_direct_run_on(p, input, output, workspace, workspace_bytes, s, templates, weights);
     const int rc = sim_direct_prepare(p, templates, weights, workspace, workspace_bytes, s);
     return rc ? rc : sim_direct_run(p, input, output, workspace, workspace_bytes, s);
 }

@@ -67,6 +67,37 @@ def test_similarity_prepared_matches_plain_call_and_oracle(pkg, case):
         assert rel_err(got.cpu().numpy(), orc.similarity_fwd(x, t, w, **okw)) <= SIM_TOL
 
 
+SHORT_PATCH_MODES = [
+    dict(similarity_function="L1"),
+    dict(similarity_function="L2"),
+    dict(similarity_function="L2", algo="direct"),
+    dict(similarity_function="L2", normalization_term=True),
+    dict(similarity_function="L2", normalization_term=True, ignore_nan_input=True, out_of_bounds_value=float("nan")),
+]
+
+
+@pytest.mark.parametrize("mode", SHORT_PATCH_MODES)
+@pytest.mark.parametrize("geom", [((7, 3, 13, 17), 19, [2, 2], [2, 1], [1, 0]), ((4, 1, 9, 9), 8, [3, 3], [1, 1], [1, 1]),
+                                  ((3, 12, 5, 6), 33, [1, 1], [1, 1], [0, 0]), ((2, 2, 6, 70), 5, [2, 3], [1, 2], [0, 2])])
+def test_short_patches_self_packing_call_matches_prepared_and_oracle(pkg, mode, geom):
+    """Patches of at most 12 elements: the self-packing call packs inside its one kernel, the prepared call reads
+    parameters packed by the pack kernel; same bits, every mode, template counts off the tile size."""
+    shape, O, blocks, strides, padding = geom
+    kw = dict(mode, blocks=blocks, strides=strides, padding=padding)
+    g = np.random.default_rng(11)
+    t = g.normal(size=(O, shape[1]) + tuple(blocks)).astype(np.float32)
+    w = (np.abs(g.normal(size=t.shape)) + 0.05).astype(np.float32)
+    w[0].flat[0] = 0.0
+    x = g.normal(size=shape).astype(np.float32)
+    if mode.get("ignore_nan_input"):
+        x[g.random(size=shape) < 0.2] = np.nan
+    X, T, W = dev(x), dev(t), dev(w)
+    plain = pkg.similarity(X, T, W, **kw)
+    assert same_bits(pkg.similarity_prepare(shape, T, W, **kw)(X), plain)
+    okw = {k: v for k, v in kw.items() if k != "algo"}
+    assert rel_err(plain.cpu().numpy(), orc.similarity_fwd(x, t, w, **okw)) <= SIM_TOL
+
+
 def test_similarity_prepared_config1_full(pkg):
     x, t, w, kw = config1(batch=64, nan_frac=0.25)
     prep = pkg.similarity_prepare(x.shape, dev(t), dev(w), **kw)
