@@ -489,7 +489,8 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                                                               int finite_eps, float *__restrict__ offp,
                                                               float *__restrict__ offe, float *__restrict__ omax,
                                                               float *__restrict__ orng, int4 *__restrict__ ktab, int H,
-                                                              int W, int bh, int bw, int row_blocks, SimPackJob job)
+                                                              int W, int bh, int bw, int row_blocks, SimPackJob job,
+                                                              float *__restrict__ normalized_out)
 {
     if ((int)blockIdx.x >= row_blocks) {
         // extra workgroups: the parameters of a Similarity layer evaluated inside the MEX staging
@@ -573,6 +574,10 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         for (int d = 32; d > 0; d >>= 1)
             sum += __shfl_xor(sum, d, 64);
         lse = logf(sum) + mxv;
+    }
+    if (normalized_out != nullptr) {   // the same values as mex_normalize_rows_kernel writes
+        float *nd = normalized_out + ((size_t)r * M + m) * K;
+        each([&](int k, float x) { nd[k] = x - lse; });
     }
     if (!finite_eps) {
         each([&](int k, float x) { dst[(size_t)k * tm] = (x - lse) * scale; });
@@ -889,7 +894,7 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups)
 }
 
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream, const SimPackJob *job, bool launch)
+                     void *stream, const SimPackJob *job, bool launch, float *normalized_out)
 {
     const simnets_mex_dims &d = p.d;
     const long long rows = (long long)d.num_regions * n_mgroups * tm;
@@ -919,7 +924,7 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
 #define SIMNETS_PACK_LAUNCH(KL)                                                                                        \
     hipLaunchKernelGGL(mex_pack_offsets_kernel<KL>, grid, dim3(256), 0, hs, offsets, d.num_regions, d.M, d.K, n_mgroups, \
                        tm, p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W,         \
-                       d.block_h, d.block_w, row_blocks, pj)
+                       d.block_h, d.block_w, row_blocks, pj, normalized_out)
     if (d.K <= 64)
         SIMNETS_PACK_LAUNCH(1);
     else if (d.K <= 256)

@@ -136,8 +136,11 @@ struct SimPackJob {
 };
 size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
 // launch = false: the arrays were packed by an earlier call with the same arguments; only the pointers are set.
+// normalized_out: if not null, the launch also writes the offsets minus their rows' logsumexp there, [region][M][K]
+// (what the gradient kernels' term-by-term path and the chain rule through the normalisation read).
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream, const SimPackJob *job = nullptr, bool launch = true);
+                     void *stream, const SimPackJob *job = nullptr, bool launch = true,
+                     float *normalized_out = nullptr);
 
 
 // Panel form of the tiled forward kernel (csrc/mex_pool.hip) for layers with 2x2 unshared offsets over whole-channel

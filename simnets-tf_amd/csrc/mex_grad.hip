@@ -798,6 +798,55 @@ __global__ __launch_bounds__(256) void mex_normalize_rows_backward_kernel(const 
         gr[k] -= expf(n[k]) * sum;
 }
 
+// Both of the above for short rows, one wave per (region, instance) row: element k of the row is the sum of its
+// partial sums in the order of mex_grad_offsets_finish_kernel (eight interleaved sums in chunk order, added in
+// order), then, if `normalized` is given, the chain rule of mex_normalize_rows_backward_kernel with the same
+// reduction over the row: the same values as the two launches, in one.
+constexpr int kFinishRowsMaxK = 1024;
+__global__ __launch_bounds__(256) void mex_grad_offsets_finish_rows_kernel(const float *__restrict__ partial, long long n,
+                                                                          int chunks, long long rows, int K,
+                                                                          const float *__restrict__ normalized,
+                                                                          float *__restrict__ doff)
+{
+    const int lane = threadIdx.x & 63;
+    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= rows)
+        return;
+    float *gr = doff + (size_t)row * K;
+    const float *pr = partial + (size_t)row * K;
+    float sum = 0.0f;
+    for (int k = lane; k < K; k += 64) {
+        float s8[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j)
+            s8[j] = 0.0f;
+        for (int c0 = 0; c0 < chunks; c0 += 8) {
+            // all eight requests first, those past the last chunk on its address (a load inside the condition
+            // would be waited for before the next one is issued)
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                v[j] = pr[(size_t)min(c0 + j, chunks - 1) * n + k];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                s8[j] = c0 + j < chunks ? s8[j] + v[j] : s8[j];
+        }
+        float t = s8[0];
+#pragma unroll
+        for (int j = 1; j < 8; ++j)
+            t += s8[j];
+        gr[k] = t;
+        sum += t;
+    }
+    if (normalized == nullptr)
+        return;
+    for (int d = 32; d > 0; d >>= 1)
+        sum += __shfl_xor(sum, d, 64);
+    const float *nr = normalized + (size_t)row * K;
+    for (int k = lane; k < K; k += 64)
+        gr[k] -= expf(nr[k]) * sum;   // reads back what this lane stored above
+}
+
 __global__ void mex_fill_zero_kernel(float *__restrict__ p, long long n)
 {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
@@ -968,7 +1017,14 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     MexGradArgs ga;
     ga.k = mex_kernel_args(p);
     ga.k.in = input;
-    int rc = prepare_offsets(p, offsets, ws + w.norm, s, &ga.off);
+    // the offsets as the forward op used them: with the matrix kernels the pack launch below writes the normalised
+    // copy as well, otherwise a launch of its own does
+    const bool pack_normalizes = t.mfma && p.normalize_offsets;
+    int rc = SIMNETS_OK;
+    if (pack_normalizes)
+        ga.off = reinterpret_cast<const float *>(ws + w.norm);
+    else
+        rc = prepare_offsets(p, offsets, ws + w.norm, s, &ga.off);
     if (rc)
         return rc;
     ga.out = output; ga.g = output_grad;
@@ -982,7 +1038,8 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
     if (t.mfma) {
-        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream);
+        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream, nullptr, true,
+                              pack_normalizes ? reinterpret_cast<float *>(ws + w.norm) : nullptr);
         if (rc)
             return rc;
         if (w.use_factors) {
@@ -1065,13 +1122,20 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
         }
         if (hipGetLastError() != hipSuccess)
             return SIMNETS_ERR_HIP;
+        const long long rows = (long long)d.num_regions * d.M;
+        if (d.K <= kFinishRowsMaxK && (rows + 3) / 4 <= 0x7fffffffLL) {
+            // short rows: the sum over the pixel chunks and the chain rule through the normalisation in one launch
+            hipLaunchKernelGGL(mex_grad_offsets_finish_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s,
+                               go.partial, n_off, go.cpr, rows, d.K, p.normalize_offsets ? go.off : nullptr,
+                               offsets_grad);
+            return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+        }
         hipLaunchKernelGGL(mex_grad_offsets_finish_kernel,
                            dim3((unsigned)std::min<long long>((n_off + 31) / 32, 65535)), dim3(256), 0, s, go.partial,
                            n_off, go.cpr, offsets_grad);
         if (hipGetLastError() != hipSuccess)
             return SIMNETS_ERR_HIP;
         if (p.normalize_offsets) {
-            const long long rows = (long long)d.num_regions * d.M;
             hipLaunchKernelGGL(mex_normalize_rows_backward_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s,
                                go.off, rows, d.K, offsets_grad);
             if (hipGetLastError() != hipSuccess)
