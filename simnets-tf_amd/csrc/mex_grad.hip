@@ -180,24 +180,35 @@ __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const int m_scan = roomy ? a.M : min(a.M, 4);   // see mex_grad_input_mfma_kernel
     float amin = INFINITY;
-    for (int m = wave; m < m_scan; m += 4)
+#pragma unroll 4
+    for (int m = wave; m < m_scan; m += 4)   // (unrolled: four loads in flight instead of one)
         amin = fminf(amin, __builtin_fmaf(op[(size_t)m * plane], a.c1, -(a.c0 + (omax_r[m] - orng_r[m]))));
     pmn[wave * 64 + lane] = amin;
     __syncthreads();
     const float a_p = valid ? fminf(fminf(pmn[lane], pmn[64 + lane]), fminf(pmn[128 + lane], pmn[192 + lane])) : 0.0f;
+    // (below, all loads of a block go out first, those past the last instance or patch element on a clamped
+    // address: a load inside the condition would be waited for before the next one is issued)
     // rows of this chunk; thread (column c, pixels pr, pr + 8, ...) writes the tile out
     const size_t row0 = (size_t)r * ga.slots_pad + (size_t)chunk * 64;
     const int c = tid & 31, pr = tid >> 5;
     // grid.y: one block of 32 columns per workgroup - the instance groups first, then the patch-element blocks
     if ((int)blockIdx.y < n_mg) {
         const int mg = blockIdx.y;
+        float ovv[GM_TM / 4], gvv[GM_TM / 4], omv[GM_TM / 4];
+#pragma unroll
+        for (int i = 0; i < GM_TM / 4; ++i) {
+            const int mc = min(mg * GM_TM + wave + 4 * i, a.M - 1);
+            ovv[i] = op[(size_t)mc * plane];
+            gvv[i] = gp[(size_t)mc * plane];
+            omv[i] = omax_r[mc];
+        }
 #pragma unroll
         for (int i = 0; i < GM_TM / 4; ++i) {
             const int mm = wave + 4 * i, m = mg * GM_TM + mm;
             float w = 0.0f;
             if (valid && m < a.M) {
-                const float e = __builtin_fmaf(-op[(size_t)m * plane], a.c1, a_p) + (omax_r[m] + a.c0);
-                w = gp[(size_t)m * plane] * __builtin_amdgcn_exp2f(e);
+                const float e = __builtin_fmaf(-ovv[i], a.c1, a_p) + (omv[i] + a.c0);
+                w = gvv[i] * __builtin_amdgcn_exp2f(e);
             }
             tile[mm * 65 + lane] = w;
         }
@@ -207,15 +218,26 @@ __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs
             ga.wbuf[(row0 + pr + 8 * j) * ga.Mp + mg * GM_TM + c] = tile[c * 65 + pr + 8 * j];
     } else {
         const int kb = ((int)blockIdx.y - n_mg) * 32;
+        int4 ke[8];  // wave-uniform: {offset inside an image, dc, dh, dw}
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            ke[i] = a.ktab[min(kb + wave + 4 * i, a.K - 1)];
+        float xg[8];
+        unsigned inside = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int ci = px.ci0 + ke[i].y, hi = px.hi0 + ke[i].z, wi = px.wi0 + ke[i].w;
+            const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+            inside |= ok ? 1u << i : 0u;
+            const float *src = ok ? px.base + ke[i].x : a.in;
+            xg[i] = *src;
+        }
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int kk = wave + 4 * i, k = kb + kk;
             float e = 0.0f;
             if (valid && k < a.K) {
-                const int4 ke = a.ktab[k];  // wave-uniform: {offset inside an image, dc, dh, dw}
-                const int ci = px.ci0 + ke.y, hi = px.hi0 + ke.z, wi = px.wi0 + ke.w;
-                const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-                const float x = ok ? px.base[ke.x] : a.oob;
+                const float x = (inside >> i) & 1u ? xg[i] : a.oob;
                 e = __builtin_amdgcn_exp2f(__builtin_fmaf(x, a.c1, -a_p));
             }
             tile[kk * 65 + lane] = e;
@@ -641,11 +663,24 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             const size_t row0 = (size_t)r * ga.slots_pad + (size_t)grp * 64;
             const int cc = tid & 63, pq = tid >> 6;
             __syncthreads();  // the previous group's matrix instructions are done with wt / ex
+            // (sixteen loads at a time, columns past the buffers' rows on a clamped address: inside the condition
+            // each would be waited for in front of its LDS write)
+            const int mcol_c = min(m0 + cc, ga.Mp - 1), kcol_c = min(k0 + cc, ga.Kp - 1);
 #pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const int pp = pq + 4 * j;
-                wt[pp * 65 + cc] = m0 + cc < ga.Mp ? ga.wbuf[(row0 + pp) * ga.Mp + m0 + cc] : 0.0f;
-                ex[pp * 65 + cc] = k0 + cc < ga.Kp ? ga.exbuf[(row0 + pp) * ga.Kp + k0 + cc] : 0.0f;
+            for (int j0 = 0; j0 < 16; j0 += 8) {
+                float wv[8], ev[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int pp = pq + 4 * (j0 + j);
+                    wv[j] = ga.wbuf[(row0 + pp) * ga.Mp + mcol_c];
+                    ev[j] = ga.exbuf[(row0 + pp) * ga.Kp + kcol_c];
+                }
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int pp = pq + 4 * (j0 + j);
+                    wt[pp * 65 + cc] = m0 + cc < ga.Mp ? wv[j] : 0.0f;
+                    ex[pp * 65 + cc] = k0 + cc < ga.Kp ? ev[j] : 0.0f;
+                }
             }
             __syncthreads();
 #pragma unroll 4

@@ -158,20 +158,32 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
     const int v0 = gw * PT;
 
     // the X values of this lane's tile (NaN -> 0 when NaN inputs are ignored: their gradient is 0)
+    // All of them are requested first, elements outside the tile on a clamped address: a load inside the condition
+    // would be waited for before the next one is issued.  nan_at: bit m * PT + p = that element is a NaN whose
+    // gradient is 0 (what the stores at the end need to know).
     float acc[MT][PT], xv[MT][PT];
     const size_t plane = (size_t)a.H * a.W;
     const float *xrow = a.x + (size_t)b * a.C * plane + (size_t)(a.y0 + a.sh * h) * a.W + a.x0;
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+        const int c = min(ctile * MT + m, a.C - 1);
+#pragma unroll
+        for (int p = 0; p < PT; ++p)
+            xv[m][p] = xrow[(size_t)c * plane + (size_t)a.sw * max(min(v0 + p, a.nb - 1), 0)];
+    }
+    unsigned long long nan_at = 0;
+    static_assert(MT * PT <= 64, "one bit per element of the lane tile");
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
         const int c = ctile * MT + m;
 #pragma unroll
         for (int p = 0; p < PT; ++p) {
             acc[m][p] = 0.0f;
-            float val = 0.0f;
-            if (wave_active && lane_valid && c < a.C && v0 + p < a.nb)
-                val = xrow[(size_t)c * plane + (size_t)a.sw * (v0 + p)];
-            if ((a.ignore_nan || MODE == GX_L1) && !(val == val))
+            float val = (wave_active && lane_valid && c < a.C && v0 + p < a.nb) ? xv[m][p] : 0.0f;
+            if ((a.ignore_nan || MODE == GX_L1) && !(val == val)) {
                 val = 0.0f;
+                nan_at |= 1ull << (m * PT + p);
+            }
             xv[m][p] = val;
         }
     }
@@ -300,11 +312,8 @@ __global__ __launch_bounds__(kThreads, gx_waves_per_simd(PT, MT)) void sim_grad_
                 continue;
             const size_t o = (size_t)c * plane + (size_t)a.sw * (v0 + p);
             float val = (row_covered && v0 + p <= a.col_limit) ? acc[m][p] : 0.0f;
-            if (a.ignore_nan || MODE == GX_L1) {
-                const float xin = xrow[o];
-                if (!(xin == xin))
-                    val = 0.0f;
-            }
+            if ((nan_at >> (m * PT + p)) & 1)
+                val = 0.0f;
             drow[o] = val;
         }
     }
@@ -832,8 +841,16 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     for (int oo = 0; oo < LO; ++oo)
 #pragma unroll
         for (int kk = 0; kk < LK; ++kk) {
+            // (a clamped address rather than a load inside the condition: each of those would be waited for in turn)
+            if constexpr (!MF)
+                t[oo][kk] = a.templates[(size_t)min(lane_o(oo), a.O - 1) * a.K + min(k0 + kk, a.K - 1)];
+        }
+#pragma unroll
+    for (int oo = 0; oo < LO; ++oo)
+#pragma unroll
+        for (int kk = 0; kk < LK; ++kk) {
             const bool ok = !MF && lane_o(oo) < a.O && k0 + kk < a.K;
-            t[oo][kk] = ok ? a.templates[(size_t)lane_o(oo) * a.K + k0 + kk] : 0.0f;
+            t[oo][kk] = ok ? t[oo][kk] : 0.0f;
             if constexpr (SGN)
                 t[oo][kk] *= 0x1p64f;
             at[oo][kk] = 0.0f;
