@@ -168,7 +168,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
     }
     const float *img = a.in + (size_t)b * a.C * a.H * a.W;
 
-    float pw_cur[RM], pt_cur[RM], pw_nxt[RM], pt_nxt[RM];
+    float pw_cur[RM], pt_cur[RM], pw_nxt[RM], pt_nxt[RM], pw_nn[RM], pt_nn[RM];
     auto load_params = [&](const float *p, float (&w_)[RM], float (&t_)[RM]) {
 #pragma unroll
         for (int i = 0; i < RM; ++i) {
@@ -208,7 +208,10 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
 #pragma unroll
         for (int j = 0; j < RP; ++j)
             xn[j] = lds[xbase[j]];
-        for (int st = 0; st < nsteps; ++st) {
+        // one step: the MFMAs on the operands in (w_use, t_use), the parameter loads of the step after next into
+        // (w_load, t_load)
+        auto do_step = [&](int st, const float (&w_use)[RM], const float (&t_use)[RM], float (&w_load)[RM],
+                           float (&t_load)[RM]) {
             float x[RP], x2[RP];
 #pragma unroll
             for (int j = 0; j < RP; ++j)
@@ -229,17 +232,16 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
 #pragma unroll
             for (int j = 0; j < RP; ++j)
                 xn[j] = lds[xbase[j] + noff];
-            float pw_nn[RM], pt_nn[RM];
-            load_params(pm, pw_nn, pt_nn);
+            load_params(pm, w_load, t_load);
             pm += step_stride;
             __builtin_amdgcn_sched_barrier(0);
             if constexpr (GRAD) {
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
-                    acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[0], x[j], acc[0][j], 0, 0, 0);
+                    acc[0][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(w_use[0], x[j], acc[0][j], 0, 0, 0);
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
-                    acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[0], x[j], acc[1][j], 0, 0, 0);
+                    acc[1][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(t_use[0], x[j], acc[1][j], 0, 0, 0);
             } else {
 #pragma unroll
                 for (int j = 0; j < RP; ++j)
@@ -248,13 +250,26 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
                 for (int i = 0; i < RM; ++i)
 #pragma unroll
                     for (int j = 0; j < RP; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pw_cur[i], x2[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(w_use[i], x2[j], acc[i][j], 0, 0, 0);
 #pragma unroll
                 for (int i = 0; i < RM; ++i)
 #pragma unroll
                     for (int j = 0; j < RP; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(pt_cur[i], x[j], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(t_use[i], x[j], acc[i][j], 0, 0, 0);
             }
+            dw = ndw; dh = ndh; row_off = nrow; off = noff;
+        };
+        // Three steps per round, the three parameter sets taking turns as (in use, next, being loaded): a load
+        // lands in the registers it is consumed from two steps later, and is waited for there.  (With one set
+        // moved to the next after every step, each move waited for loads issued a single step earlier.)
+        int st = 0;
+        for (; st + 3 <= nsteps; st += 3) {
+            do_step(st, pw_cur, pt_cur, pw_nn, pt_nn);
+            do_step(st + 1, pw_nxt, pt_nxt, pw_cur, pt_cur);
+            do_step(st + 2, pw_nn, pt_nn, pw_nxt, pt_nxt);
+        }
+        for (; st < nsteps; ++st) {
+            do_step(st, pw_cur, pt_cur, pw_nn, pt_nn);
 #pragma unroll
             for (int i = 0; i < RM; ++i) {
                 if (GRAD && i > 0)
@@ -262,7 +277,6 @@ __global__ __launch_bounds__(kThreads, 2) void sim_mfma_kernel(const MfmaArgs a,
                 pw_cur[i] = pw_nxt[i]; pt_cur[i] = pt_nxt[i];
                 pw_nxt[i] = pw_nn[i];  pt_nxt[i] = pt_nn[i];
             }
-            dw = ndw; dh = ndh; row_off = nrow; off = noff;
         }
     }
 
