@@ -56,6 +56,9 @@ def main():
     ap.add_argument("--shapes", action="store_true",
                     help="instead of the benchmark line: time Similarity forward, input gradient and parameter "
                          "gradients on network-like shapes away from the benchmark configurations (one JSON object)")
+    ap.add_argument("--train", action="store_true",
+                    help="instead of the benchmark line: time only the training step of the config-4 stack (the run "
+                         "to put under a kernel trace; one JSON object)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the path is data parallel over the batch; "
@@ -109,6 +112,32 @@ def main():
             for _ in range(reps):
                 fn()
         return g
+
+    def config4_training_step(X4, T4, W4, kw4, layer_offsets, offl, nl, kwl):
+        """A training step of the config-4 stack through the differentiable layer functions: forward with the
+        unfused MEX calls (their gradients take the unpooled outputs), then every operator's gradient calls."""
+        L = pkg.layers
+        params = [T4.clone().requires_grad_(), W4.clone().requires_grad_()] + \
+                 [off.clone().requires_grad_() for off, _, _ in layer_offsets] + [offl.clone().requires_grad_()]
+
+        def train_step():
+            for q in params:
+                q.grad = None
+            cur = L.similarity(X4, params[0], params[1], **kw4)
+            for i, (_, n, kw) in enumerate(layer_offsets):
+                cur = L.mex_sum_pool(cur, params[2 + i], n, (2, 2), normalize_offsets=True, **kw)
+            out = L.mex(cur, params[-1], nl, normalize_offsets=True, **kwl)
+            out.sum().backward()
+        return train_step
+
+    if args.train:
+        x4, t4, w4, kw4, layers_np, (offl_np, nl, kwl) = config4_stack(512)
+        step = config4_training_step(to_dev(x4), to_dev(t4), to_dev(w4), kw4,
+                                     [(to_dev(o), n, kw) for o, n, kw in layers_np], to_dev(offl_np), nl, kwl)
+        _, ms = timed(step, args.steps, args.warmup)
+        print(json.dumps({"config4_train_step_ms": round(ms, 4), "batch": 512, "steps": args.steps,
+                          "warmup": args.warmup, "dtype": "f32"}))
+        return
 
     if args.shapes:
         # (name, input shape, templates, block, stride, padding): layers of a residual-network-like stack at batch 32
@@ -411,24 +440,10 @@ def main():
         e4.update({"fused_prepared_ms": round(ms_prep, 4),
                    "fused_prepared_hbm_frac": round((bytes4 / 1e9) / (ms_prep * 1e-3) / PEAK_HBM_GBS, 4),
                    "fused_prepared_bit_identical_to_fused": bool(torch.equal(prepared_stack(), fused_stack3()))})
-        # a training step of the same stack through the differentiable layer functions: forward with the unfused
-        # MEX calls (their gradients take the unpooled outputs), then every operator's gradient calls
-        L = pkg.layers
-        train_params = [T4.clone().requires_grad_(), W4.clone().requires_grad_()] + \
-                       [off.clone().requires_grad_() for off, _, _ in layers] + [offl.clone().requires_grad_()]
-
-        def train_step():
-            for q in train_params:
-                q.grad = None
-            cur = L.similarity(X4, train_params[0], train_params[1], **kw4)
-            for i, (_, n, kw) in enumerate(layers):
-                cur = L.mex_sum_pool(cur, train_params[2 + i], n, (2, 2), normalize_offsets=True, **kw)
-            out = L.mex(cur, train_params[-1], nl, normalize_offsets=True, **kwl)
-            out.sum().backward()
-
+        train_step = config4_training_step(X4, T4, W4, kw4, layers, offl, nl, kwl)
         _, ms_train = timed(train_step, args.steps, args.warmup)
         e4["train_step_ms"] = round(ms_train, 4)
-        del train_params
+        del train_step
 
         def cpu4():
             """The stack on the CPU oracle, layer by layer on 64 of the 512 images (single thread), all 512 with
