@@ -44,6 +44,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--settle", type=float, default=1.5,
                     help="seconds of untimed load before the warm-up steps (lets the clocks of an idle GPU settle)")
+    ap.add_argument("--settle-others", type=float, default=0.25,
+                    help="seconds of untimed load before every other timed workload")
     ap.add_argument("--algo", default=None, choices=[None, "direct", "sqrtw", "mfma"],
                     help="evaluation path of the headline Similarity kernel (default: the library default)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
@@ -85,7 +87,14 @@ def main():
     def timed(fn, steps, warmup):
         """(wall ms per step, HIP-event ms per step) for `steps` calls after `warmup` calls.
         The events are recorded on the stream the kernels are launched on (torch's current stream,
-        whose handle the op layer passes through the C ABI)."""
+        whose handle the op layer passes through the C ABI).  Like the headline, every workload first runs
+        untimed for a moment (--settle-others): the host-side set-up between two workloads leaves the chip idle
+        long enough for its clocks to drop."""
+        until = time.perf_counter() + args.settle_others
+        while time.perf_counter() < until:
+            for _ in range(10):
+                fn()
+            torch.cuda.synchronize()
         for _ in range(warmup):
             fn()
         torch.cuda.synchronize()
