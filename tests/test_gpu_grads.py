@@ -400,6 +400,32 @@ def test_mex_offsets_grad_through_the_offset_normalisation(pkg):
     assert grad_err(got_dx, orc.mex_input_grad(x, norm, out, g, n, **kw)) <= GRAD_TOL
 
 
+@pytest.mark.parametrize("shape,blocks,n,shared", [
+    ((3, 5, 16, 16), [5, 16, 16], 3, None),        # rows of 1280 elements: two launches
+    ((6, 4, 16, 16), [4, 16, 16], 5, None),        # rows of 1024: one launch
+    ((40, 3, 6, 6), [3, 2, 2], 7, [-1])])          # one region of 360 pixel slots: several pixel chunks
+@pytest.mark.parametrize("normalize", [False, True])
+def test_mex_offsets_grad_sum_over_pixel_chunks_and_chain_rule(pkg, shape, blocks, n, shared, normalize):
+    """The offsets gradient's last step - partial sums of the pixel chunks added up, then the chain rule through
+    the normalisation - runs as one launch for rows of at most 1024 elements and as two for longer ones."""
+    g_ = np.random.default_rng(21)
+    x = g_.normal(size=shape).astype(np.float32)
+    kw = dict(blocks=blocks, strides=blocks, epsilon=1.0, softmax_mode=True)
+    if shared is not None:
+        kw.update(use_unshared_regions=False, shared_offset_region=shared)
+    off = (0.3 * g_.normal(size=(1, n) + tuple(blocks))).astype(np.float32)
+    used = orc.normalize_offsets(off) if normalize else off
+    out = orc.mex_fwd(x, used, n, **kw)
+    g = g_.normal(size=out.shape).astype(np.float32)
+    G = orc.mex_offsets_grad(x.astype(np.float64), used.astype(np.float64), out.astype(np.float64),
+                             g.astype(np.float64), n, **kw)
+    want = G - np.exp(used.astype(np.float64)) * G.sum(axis=(2, 3, 4), keepdims=True) if normalize else G
+    got = pkg.mex_offsets_grad(dev(x), dev(off), dev(out), dev(g), n, normalize_offsets=normalize, **kw)
+    assert grad_err(got.cpu().numpy(), want) <= GRAD_TOL
+    both = pkg.mex_grads(dev(x), dev(off), dev(out), dev(g), n, normalize_offsets=normalize, **kw)
+    assert np.array_equal(both[1].cpu().numpy().view(np.uint32), got.cpu().numpy().view(np.uint32))
+
+
 def test_mex_offsets_grad_is_reproducible_and_additive(pkg):
     x, off, n, kw = config2(batch=64)
     off = orc.normalize_offsets(off)
