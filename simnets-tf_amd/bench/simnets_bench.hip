@@ -5,9 +5,14 @@
 //   simnets_bench --config N [--algo A] [--steps K] [--warmup W]     (N = 1..4 forward, 5 backward)
 //                                              N in 1..4: times that benchmark configuration through the
 //                                              C ABI with hipEvents on its own stream
-// Prints one JSON object per measurement.  Inputs are synthetic (fixed-seed counter-based generator),
-// resident in HBM before timing starts.  Parity is not checked here (tests/ does that through the same
-// ABI); this binary links only the product library.
+//   ... --dump DIR                             also writes the synthetic inputs of the configuration to DIR as
+//                                              raw float32 files (<tag>_x.bin, <tag>_t.bin, ...)
+// Prints one JSON object per line: the measurements, and for every configuration a checksum of the
+// output tensors its calls produced ({"checksum": name, "value": "<hex>", "elements": n}; the value is
+// sum_i (bits(out[i]) + 1) * (2 i + 1) mod 2^64 over the fp32 bit patterns), so that a caller of the same
+// library on the dumped inputs can be compared bit for bit.  Inputs are synthetic (fixed-seed
+// counter-based generator), resident in HBM before timing starts.  Parity with the CPU oracle is not
+// checked here (tests/ does that through the same ABI); this binary links only the product library.
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
@@ -262,6 +267,31 @@ static void fill_normal(std::vector<float> &v, uint64_t seed, float sigma)
         v[i] = sigma * std::sqrt(-2.0f * std::log(u1)) * std::cos(6.2831853f * u2);
     }
 }
+static std::string g_dump_dir;
+static void dump(const std::string &name, const std::vector<float> &v)
+{
+    if (g_dump_dir.empty())
+        return;
+    const std::string path = g_dump_dir + "/" + name + ".bin";
+    FILE *f = fopen(path.c_str(), "wb");
+    if (!f || fwrite(v.data(), sizeof(float), v.size(), f) != v.size()) {
+        fprintf(stderr, "cannot write %s\n", path.c_str());
+        exit(1);
+    }
+    fclose(f);
+}
+// checksum of a device tensor's bit patterns, printed as one JSON line
+static void checksum(const char *name, const float *dev, size_t n, hipStream_t s)
+{
+    std::vector<uint32_t> h(n);
+    HIP_OK(hipStreamSynchronize(s));
+    HIP_OK(hipMemcpy(h.data(), dev, n * sizeof(float), hipMemcpyDeviceToHost));
+    uint64_t acc = 0;
+    for (size_t i = 0; i < n; ++i)
+        acc += ((uint64_t)h[i] + 1) * (2 * (uint64_t)i + 1);
+    printf("{\"checksum\": \"%s\", \"value\": \"%016llx\", \"elements\": %zu}\n", name, (unsigned long long)acc, n);
+}
+static size_t count4(const int *d) { return (size_t)d[0] * d[1] * d[2] * d[3]; }
 static float *upload(const std::vector<float> &v)
 {
     float *d;
@@ -278,7 +308,8 @@ struct SimCase {
     size_t ws_bytes;
 };
 
-static SimCase make_similarity(int B, int C, int H, int W, int O, int bh, int bw, int s, int p, bool missing, int algo, int l1)
+static SimCase make_similarity(const std::string &tag, int B, int C, int H, int W, int O, int bh, int bw, int s, int p,
+                               bool missing, int algo, int l1)
 {
     SimCase c;
     simnets_similarity_attrs_default(&c.a);
@@ -306,6 +337,7 @@ static SimCase make_similarity(int B, int C, int H, int W, int O, int bh, int bw
         fill_normal(t, 2345, 1.0f);
         fill_uniform(w, 3456, 0.1f, 2.0f);
     }
+    dump(tag + "_x", x); dump(tag + "_t", t); dump(tag + "_w", w);
     c.x = upload(x); c.t = upload(t); c.w = upload(w);
     HIP_OK(hipMalloc(&c.y, (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3] * sizeof(float)));
     SN_OK(simnets_hip_similarity_workspace_bytes(&c.a, c.in, c.tp, &c.ws_bytes));
@@ -321,7 +353,7 @@ struct MexCase {
     size_t ws_bytes, off_count;
 };
 
-static MexCase make_mex(int B, int C, int HW, int M, bool shared1, const float *input)
+static MexCase make_mex(const std::string &tag, int B, int C, int HW, int M, bool shared1, const float *input)
 {
     MexCase c;
     simnets_mex_attrs_default(&c.a);
@@ -340,12 +372,14 @@ static MexCase make_mex(int B, int C, int HW, int M, bool shared1, const float *
     c.off_count = (size_t)c.off[0] * c.off[1] * c.off[2] * c.off[3] * c.off[4];
     std::vector<float> off(c.off_count);
     fill_normal(off, 4567 + C, 0.1f);
+    dump(tag + "_off", off);
     c.o = upload(off);
     if (input) {
         c.x = const_cast<float *>(input);
     } else {
         std::vector<float> x((size_t)B * C * HW * HW);
         fill_normal(x, 1234, 1.0f);
+        dump(tag + "_x", x);
         c.x = upload(x);
     }
     HIP_OK(hipMalloc(&c.y, (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3] * sizeof(float)));
@@ -382,11 +416,12 @@ int main(int argc, char **argv)
         else if (a == "--config" && i + 1 < argc) config = atoi(argv[++i]);
         else if (a == "--steps" && i + 1 < argc) steps = atoi(argv[++i]);
         else if (a == "--warmup" && i + 1 < argc) warmup = atoi(argv[++i]);
+        else if (a == "--dump" && i + 1 < argc) g_dump_dir = argv[++i];
         else if (a == "--algo" && i + 1 < argc) {
             std::string v = argv[++i];
             algo = v == "direct" ? SIMNETS_ALGO_DIRECT : v == "sqrtw" ? SIMNETS_ALGO_SQRTW : v == "mfma" ? SIMNETS_ALGO_MFMA : SIMNETS_ALGO_AUTO;
         } else {
-            fprintf(stderr, "usage: %s --peaks | --config N [--algo direct|sqrtw|mfma] [--steps K] [--warmup W]\n", argv[0]);
+            fprintf(stderr, "usage: %s --peaks | --config N [--algo direct|sqrtw|mfma] [--steps K] [--warmup W] [--dump DIR]\n", argv[0]);
             return 2;
         }
     }
@@ -395,30 +430,36 @@ int main(int argc, char **argv)
     if (peaks)
         run_peaks(s);
     if (config == 1) {
-        SimCase c = make_similarity(64, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
+        SimCase c = make_similarity("c1", 64, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
         for (int i = 0; i < warmup; ++i) run_sim(c, s);
         float ms = time_ms(s, steps, [&] { run_sim(c, s); });
         report("config1 similarity L2 norm ignore-nan 64x1x28x28 -> 64x32x16x16", 2097152.0, 2298880.0, 6, ms, steps);
+        checksum("config1", c.y, count4(c.out), s);
+        HIP_OK(hipMemsetAsync(c.y, 0xff, count4(c.out) * sizeof(float), s));
         SN_OK(simnets_hip_similarity_prepare(&c.a, c.in, c.tp, c.tp, c.t, c.w, c.ws, c.ws_bytes, s));
         auto prepared = [&] { SN_OK(simnets_hip_similarity_fwd_prepared(&c.a, c.in, c.tp, c.x, c.ws, c.ws_bytes, c.y, s)); };
         for (int i = 0; i < warmup; ++i) prepared();
         ms = time_ms(s, 10 * steps, prepared);
         report("config1, parameters prepared once (simnets_hip_similarity_fwd_prepared)", 2097152.0, 2298880.0, 6, ms, 10 * steps);
+        checksum("config1 prepared", c.y, count4(c.out), s);
     } else if (config == 2) {
-        MexCase c = make_mex(64, 32, 16, 64, false, nullptr);
+        MexCase c = make_mex("c2", 64, 32, 16, 64, false, nullptr);
         for (int i = 0; i < warmup; ++i) run_mex(c, s);
         float ms = time_ms(s, steps, [&] { run_mex(c, s); });
         report("config2 mex 64x32x16x16 -> 64x64x16x16", 33554432.0, 6324224.0, 5, ms, steps);
+        checksum("config2", c.y, count4(c.out), s);
+        HIP_OK(hipMemsetAsync(c.y, 0xff, count4(c.out) * sizeof(float), s));
         SN_OK(simnets_hip_mex_prepare(&c.a, c.in, c.o, c.off_count, c.ws, c.ws_bytes, s));
         auto prepared = [&] { SN_OK(simnets_hip_mex_fwd_prepared(&c.a, c.in, c.x, c.ws, c.ws_bytes, c.y, s)); };
         for (int i = 0; i < warmup; ++i) prepared();
         ms = time_ms(s, 10 * steps, prepared);
         report("config2, offsets prepared once (simnets_hip_mex_fwd_prepared)", 33554432.0, 6324224.0, 5, ms, 10 * steps);
+        checksum("config2 prepared", c.y, count4(c.out), s);
     } else if (config == 3) {
         for (int l1 = 0; l1 < 2; ++l1) {
             if (l1 && algo != SIMNETS_ALGO_AUTO && algo != SIMNETS_ALGO_DIRECT)
                 break;
-            SimCase c = make_similarity(256, 64, 32, 32, 128, 3, 3, 1, 1, false, algo, l1);
+            SimCase c = make_similarity("c3", 256, 64, 32, 32, 128, 3, 3, 1, 1, false, algo, l1);
             for (int i = 0; i < warmup; ++i) run_sim(c, s);
             float ms = time_ms(s, steps, [&] { run_sim(c, s); });
             report(l1 ? "config3 similarity L1 256x64x32x32 x 128 templates 3x3" : "config3 similarity L2 256x64x32x32 x 128 templates 3x3",
@@ -427,16 +468,18 @@ int main(int argc, char **argv)
             ms = time_ms(s, steps, [&] { SN_OK(simnets_hip_similarity_fwd_prepared(&c.a, c.in, c.tp, c.x, c.ws, c.ws_bytes, c.y, s)); });
             report(l1 ? "config3 similarity L1, parameters prepared once" : "config3 similarity L2, parameters prepared once",
                    19327352832.0, 201916416.0, l1 ? 3 : 4, ms, steps);
+            checksum(l1 ? "config3 L1" : "config3 L2", c.y, count4(c.out), s);
+            HIP_OK(hipFree(c.x)); HIP_OK(hipFree(c.y)); HIP_OK(hipFree(c.ws));
         }
     } else if (config == 4) {
         const int B = 512;
-        SimCase sc = make_similarity(B, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
+        SimCase sc = make_similarity("c4", B, 1, 28, 28, 32, 2, 2, 2, 2, true, algo, 0);
         std::vector<MexCase> mex;
         std::vector<float *> pooled;
         const float *cur = sc.y;
         int ch = 32, hw = 16;
         for (int l = 0; l < 4; ++l) {
-            mex.push_back(make_mex(B, ch, hw, 2 * ch, false, cur));
+            mex.push_back(make_mex("c4_mex" + std::to_string(l), B, ch, hw, 2 * ch, false, cur));
             float *p;
             HIP_OK(hipMalloc(&p, (size_t)B * 2 * ch * (hw / 2) * (hw / 2) * sizeof(float)));
             pooled.push_back(p);
@@ -444,7 +487,8 @@ int main(int argc, char **argv)
             ch *= 2;
             hw /= 2;
         }
-        mex.push_back(make_mex(B, ch, 1, 10, true, cur));
+        mex.push_back(make_mex("c4_mex4", B, ch, 1, 10, true, cur));
+        const size_t n_final = count4(mex[4].out);
         auto stack = [&] {
             run_sim(sc, s);
             for (int l = 0; l < 4; ++l) {
@@ -456,6 +500,8 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) stack();
         float ms = time_ms(s, steps, stack);
         report("config4 missing-data stack batch 512", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        checksum("config4 separate calls", mex[4].y, n_final, s);
+        HIP_OK(hipMemsetAsync(mex[4].y, 0xff, n_final * sizeof(float), s));
         // the same stack with each MEX + pooling pair as one call (simnets_hip_mex_sum_pool_fwd)
         std::vector<void *> fws(4);
         std::vector<size_t> fbytes(4);
@@ -473,6 +519,8 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) fused();
         ms = time_ms(s, steps, fused);
         report("config4 missing-data stack batch 512, MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        checksum("config4 fused pooling", mex[4].y, n_final, s);
+        HIP_OK(hipMemsetAsync(mex[4].y, 0xff, n_final * sizeof(float), s));
         // ... and with the Similarity layer evaluated inside the first of those kernels
         size_t f0bytes = 0;
         SN_OK(simnets_hip_similarity_mex_sum_pool_workspace_bytes(&sc.a, sc.in, sc.tp, &mex[0].a, 2, 2, &f0bytes));
@@ -489,6 +537,8 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) fused3();
         ms = time_ms(s, steps, fused3);
         report("config4 missing-data stack batch 512, Similarity + MEX + pooling fused", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 0, 5, ms, steps);
+        checksum("config4 fused similarity and pooling", mex[4].y, n_final, s);
+        HIP_OK(hipMemsetAsync(mex[4].y, 0xff, n_final * sizeof(float), s));
         // ... and with every layer's parameters packed once (the *_prepare / *_fwd_prepared entry points): the
         // workspaces above double as the prepared buffers, five launches per stack
         SN_OK(simnets_hip_similarity_mex_sum_pool_prepare(&sc.a, sc.in, sc.tp, sc.t, sc.w, &mex[0].a, mex[0].o,
@@ -508,14 +558,16 @@ int main(int argc, char **argv)
         for (int i = 0; i < warmup; ++i) prepared();
         ms = time_ms(s, steps, prepared);
         report("config4 missing-data stack batch 512, fused, parameters prepared once", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 117e6, 5, ms, steps);
+        checksum("config4 fused prepared", mex[4].y, n_final, s);
     }
     else if (config == 5) {
         // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)
         for (int l1 = 0; l1 < 2; ++l1) {
-            SimCase c = make_similarity(256, 64, 32, 32, 128, 3, 3, 1, 1, false, SIMNETS_ALGO_AUTO, l1);
+            SimCase c = make_similarity("c5", 256, 64, 32, 32, 128, 3, 3, 1, 1, false, SIMNETS_ALGO_AUTO, l1);
             const size_t n_out = (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3];
             std::vector<float> g(n_out);
             fill_normal(g, 6789, 1.0f);
+            dump("c5_g", g);
             float *dg = upload(g), *dx, *dt, *dw;
             HIP_OK(hipMalloc(&dx, (size_t)256 * 64 * 32 * 32 * sizeof(float)));
             HIP_OK(hipMalloc(&dt, (size_t)128 * 64 * 9 * sizeof(float)));
@@ -534,15 +586,19 @@ int main(int argc, char **argv)
             ms = time_ms(s, steps, gp);
             report(l1 ? "config5 similarity params grad L1 (config-3 shape)" : "config5 similarity params grad L2 (config-3 shape)",
                    19327352832.0, (n_out + 256.0 * 64 * 32 * 32) * 4, l1 ? 6 : 5, ms, steps);
+            checksum(l1 ? "config5 L1 input grad" : "config5 L2 input grad", dx, (size_t)256 * 64 * 32 * 32, s);
+            checksum(l1 ? "config5 L1 templates grad" : "config5 L2 templates grad", dt, (size_t)128 * 64 * 9, s);
+            checksum(l1 ? "config5 L1 weights grad" : "config5 L2 weights grad", dw, (size_t)128 * 64 * 9, s);
             HIP_OK(hipFree(dg)); HIP_OK(hipFree(dx)); HIP_OK(hipFree(dt)); HIP_OK(hipFree(dw)); HIP_OK(hipFree(ws));
             HIP_OK(hipFree(c.x)); HIP_OK(hipFree(c.y));
         }
         {
-            MexCase c = make_mex(64, 32, 16, 64, false, nullptr);
+            MexCase c = make_mex("c5_mex", 64, 32, 16, 64, false, nullptr);
             run_mex(c, s);
             const size_t n_out = (size_t)c.out[0] * c.out[1] * c.out[2] * c.out[3];
             std::vector<float> g(n_out);
             fill_normal(g, 6789, 1.0f);
+            dump("c5_mex_g", g);
             float *dg = upload(g), *dx, *doff;
             HIP_OK(hipMalloc(&dx, (size_t)64 * 32 * 16 * 16 * sizeof(float)));
             HIP_OK(hipMalloc(&doff, c.off_count * sizeof(float)));
@@ -557,6 +613,8 @@ int main(int argc, char **argv)
             report("config5 mex input grad (config-2 shape)", 33554432.0, (2.0 * n_out + 2.0 * 64 * 32 * 256) * 4, 5, ms, steps);
             ms = time_ms(s, steps, go);
             report("config5 mex offsets grad (config-2 shape)", 33554432.0, (2.0 * n_out + 64.0 * 32 * 256) * 4, 5, ms, steps);
+            checksum("config5 mex input grad", dx, (size_t)64 * 32 * 16 * 16, s);
+            checksum("config5 mex offsets grad", doff, c.off_count, s);
         }
     }
     HIP_OK(hipStreamSynchronize(s));

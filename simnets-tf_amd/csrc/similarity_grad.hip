@@ -498,6 +498,11 @@ GxTiling gx_try(const SimPlan &p, const Phase &f, int PT, int nws, int MT = 8)
     t.lds_ok = per_chan <= budget;
     t.fast_stage = per_chan <= kStagePos * kThreads;
     t.CC = 1;
+    if (t.NI > 1 && !grouped_tile_fits(kStagePos * kThreads, per_chan, per_chan, p.O)) {
+        // (cannot happen while the loop above bounds NI * tile by kStagePos * kThreads; kept as the staging's own check)
+        t.NI = 1;
+        t.lds_ok = false;
+    }
     if (t.lds_ok) {
         const int cc_max = (int)std::min<long long>(p.O, budget / per_chan);
         const int chunks = (p.O + cc_max - 1) / cc_max;

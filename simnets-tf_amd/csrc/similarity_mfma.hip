@@ -719,7 +719,8 @@ MfmaTiling mfma_tiling(const SimPlan &p)
     pitch = (pitch + 31) / 64 * 64 + 32;
     if (pitch < per_chan)
         pitch += 64;
-    t.ok = 2 * pitch <= kLdsBudgetFloats && per_chan <= kStagePos * kThreads;
+    t.ok = 2 * pitch <= kLdsBudgetFloats && per_chan <= kStagePos * kThreads &&
+           grouped_tile_fits(kStagePos * kThreads, per_chan, pitch, (p.C + 1) & ~1);
     t.chan_lds = (int)pitch;
     int cc_max = t.ok ? (int)(kLdsBudgetFloats / pitch) & ~1 : 2;
     cc_max = std::min(cc_max, (p.C + 1) & ~1);
@@ -922,7 +923,8 @@ StrideTiling stride_tiling(const SimPlan &p)
     pitch = (pitch + 31) / 64 * 64 + 32;
     if (pitch < 1LL * TRmax * q.TC)
         pitch += 64;
-    if (2 * pitch > kLdsBudgetFloats || 1LL * TRmax * q.TC > kStagePos * kThreads)
+    if (2 * pitch > kLdsBudgetFloats || 1LL * TRmax * q.TC > kStagePos * kThreads ||
+        !grouped_tile_fits(kStagePos * kThreads, 1LL * TRmax * q.TC, pitch, (p.O + 1) & ~1))
         return t;
     q.chan_lds = (int)pitch;
     int cc_max = (int)(kLdsBudgetFloats / pitch) & ~1;

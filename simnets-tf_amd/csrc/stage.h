@@ -114,6 +114,25 @@ __device__ __forceinline__ void stage_input_tile_fast(float *lds, const float *i
 // workgroup, the images' tiles side by side inside a channel slot), so that every thread has NPOS loads in flight
 // however small the tile of one channel is.  LDS element (cc, image il, r, c) sits at cc * chan_pitch +
 // il * TR * TC + r * TC + c and holds input[b0 + il][ch0 + cc][row0 + r][c - pad_w].
+// Preconditions, which the host checks with grouped_tile_fits() where it picks this staging (a violation would drop
+// tile elements or mix the two fields of `lofs` without any visible error):
+//   * one channel slot has at most NPOS * NTHREADS elements (per_chan = nslots * TR * TC): with more, G = 1 would
+//     cover only the first NPOS * NTHREADS of them;
+//   * the LDS offsets of a group, (G - 1) * chan_pitch + per_chan, stay below 65536 (16 bits of `lofs`), and the
+//     channel inside the group (< G <= max_group) fits the 15 bits above them.
+__host__ __device__ inline bool grouped_tile_fits(long long elems_per_round, long long per_chan, long long chan_pitch,
+                                                  long long max_group)
+{
+    if (per_chan < 1 || per_chan > elems_per_round)
+        return false;
+    long long G = elems_per_round / per_chan;
+    if (G > max_group)
+        G = max_group;
+    if (G < 1)
+        G = 1;
+    return (G - 1) * chan_pitch + per_chan <= 65536 && G < 32768;
+}
+
 template <int NPOS>
 struct GroupedTile {
     int gofs[NPOS];  // offset from (image b0, first channel of the group); -1: pad value; -2: not an element

@@ -9,6 +9,7 @@
 Everything computes in fp32 on a HIP device through libsimnets_hip.so; there is no CPU path.
 """
 import math
+import weakref
 
 import numpy as np
 import torch
@@ -121,6 +122,54 @@ def dirichlet_init(shape, alpha=1.0, generator=None):
     return torch.from_numpy(np.log(sample).astype(np.float32).reshape(shape))
 
 
+class _PreparedCache:
+    """The packed-parameter buffers of a module's inference calls, one per stream (a buffer also holds the per-call
+    scratch of its kernels, so calls on different streams must not share one).
+
+    A buffer is reused while the parameters are the same tensor objects (held by weak reference: the address of a
+    freed parameter may be handed to its replacement) at the same storage address and version counter, and the
+    rest of the key (input shape, device, layer attributes) is unchanged.  In-place operations on a parameter bump
+    its version; rebinding the attribute or `load_state_dict(assign=True)` changes the object.  Writes through
+    `.data` touch none of these: the modules' `invalidate_prepared()` is for them."""
+
+    def __init__(self):
+        self._slots = {}
+
+    @staticmethod
+    def _same(refs, marks, params):
+        for r, m, p in zip(refs, marks, params):
+            if r() is not p or m != (p.data_ptr(), p._version):
+                return False
+        return True
+
+    def get(self, stream, params, key, make):
+        slot = self._slots.get(stream)
+        if slot is None or slot[0] != key or not self._same(slot[1], slot[2], params):
+            if len(self._slots) >= 8:
+                self._slots.clear()
+            slot = self._slots[stream] = (key, [weakref.ref(p) for p in params],
+                                          [(p.data_ptr(), p._version) for p in params], make())
+        return slot[3]
+
+    def last(self, stream=None):
+        """The Prepared object last made for `stream` (default: for any stream), or None."""
+        if stream is None:
+            slot = next(reversed(self._slots.values())) if self._slots else None
+        else:
+            slot = self._slots.get(stream)
+        return None if slot is None else slot[3]
+
+    def clear(self):
+        self._slots.clear()
+
+    # copies and pickles of a module start with an empty cache (the buffers belong to the original's calls)
+    def __deepcopy__(self, memo):
+        return _PreparedCache()
+
+    def __reduce__(self):
+        return (_PreparedCache, ())
+
+
 def _resolve_padding(padding, blocks):
     if isinstance(padding, str):
         if padding.upper() not in ("SAME", "VALID"):
@@ -151,7 +200,7 @@ class Similarity(torch.nn.Module):
         self.channels_last = channels_last
         self.templates = torch.nn.UninitializedParameter()
         self.sweights = torch.nn.UninitializedParameter()
-        self._prepared = None   # (key, ops.Prepared) of the last inference call
+        self._prepared = _PreparedCache()
 
     @staticmethod
     def _init(param, how):
@@ -187,16 +236,22 @@ class Similarity(torch.nn.Module):
         if self.channels_last:
             x = x.permute(0, 3, 1, 2).contiguous()
         if not torch.is_grad_enabled() and x.is_cuda:
-            # inference: the parameters are packed once per (input shape, parameter version); calls run the forward
-            # kernels on the prepared buffer
-            key = (tuple(x.shape), x.device, self.templates._version, self.sweights._version)
-            if self._prepared is None or self._prepared[0] != key:
-                self._prepared = (key, ops.similarity_prepare(x.shape, self.templates.detach(),
-                                                              self.sweights.detach().abs(), **self.attrs()))
-            out = self._prepared[1](x)
+            # inference: the parameters are packed once per (input shape, parameter identity and version, layer
+            # attributes, stream); calls run the forward kernels on the prepared buffer
+            attrs = self.attrs()
+            key = (tuple(x.shape), x.device, ops._freeze(attrs))
+            out = self._prepared.get(
+                ops._current_stream(x.device), (self.templates, self.sweights), key, lambda: ops.similarity_prepare(
+                    x.shape, self.templates.detach(), self.sweights.detach().abs(), **attrs))(x)
         else:
             out = similarity(x, self.templates, self.sweights.abs(), **self.attrs())
         return out.permute(0, 2, 3, 1) if self.channels_last else out
+
+    def invalidate_prepared(self):
+        """Drop the packed-parameter buffers of the inference path.  Needed only after the parameters were written
+        through `.data` (or any other way that bypasses torch's version counter): in-place operations on the
+        parameters, rebinding them and changes of the layer's attributes are noticed without it."""
+        self._prepared.clear()
 
     def compute_output_shape(self, input_shape):
         shape = list(input_shape)
@@ -236,7 +291,7 @@ class Mex(torch.nn.Module):
         self.offsets_initializer = offsets_initializer
         self.channels_last = channels_last
         self.offsets = torch.nn.UninitializedParameter()
-        self._prepared = None   # (key, ops.Prepared) of the last inference call
+        self._prepared = _PreparedCache()
 
     def build(self, input_shape):
         shape = list(input_shape)
@@ -276,15 +331,21 @@ class Mex(torch.nn.Module):
         if self.channels_last:
             x = x.permute(0, 3, 1, 2).contiguous()
         if not torch.is_grad_enabled() and x.is_cuda:
-            # inference: the offsets are packed once per (input shape, parameter version)
-            key = (tuple(x.shape), x.device, self.offsets._version)
-            if self._prepared is None or self._prepared[0] != key:
-                self._prepared = (key, ops.mex_prepare(x.shape, self.offsets.detach(), self.num_instances,
-                                                       **self.attrs()))
-            out = self._prepared[1](x)
+            # inference: the offsets are packed once per (input shape, parameter identity and version, layer
+            # attributes, stream)
+            attrs = self.attrs()
+            key = (tuple(x.shape), x.device, self.num_instances, ops._freeze(attrs))
+            out = self._prepared.get(ops._current_stream(x.device), (self.offsets,), key, lambda: ops.mex_prepare(
+                x.shape, self.offsets.detach(), self.num_instances, **attrs))(x)
         else:
             out = mex(x, self.offsets, self.num_instances, **self.attrs())
         return out.permute(0, 2, 3, 1) if self.channels_last else out
+
+    def invalidate_prepared(self):
+        """Drop the packed-parameter buffers of the inference path.  Needed only after the parameters were written
+        through `.data` (or any other way that bypasses torch's version counter): in-place operations on the
+        parameters, rebinding them and changes of the layer's attributes are noticed without it."""
+        self._prepared.clear()
 
     def compute_output_shape(self, input_shape):
         shape = list(input_shape)

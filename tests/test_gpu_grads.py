@@ -5,10 +5,13 @@ Gradients are sums of many signed terms and cross zero, so
   * the error of an element is taken relative to max(|want|, 1e-2 * max|want|): element-wise for
     everything above a hundredth of the tensor's scale, relative to that hundredth below it (the
     rounding noise of an fp32 sum is proportional to the magnitude of its terms, not of its value);
-  * it is measured against the oracle's fp64 instantiation (the exact value of the sum), and the bar
-    is 1e-4 or twice the error the reference's own fp32 arithmetic (the oracle's fp32 instantiation)
-    makes on the same inputs, whichever is larger: where the sum cancels, no fp32 summation order
-    is closer to another than both are to the exact value.
+  * it is measured against the oracle's fp64 instantiation (the exact value of the sum).  The bar is
+    the plain 1e-4 at the benchmark shapes (configuration 5: the config-3, config-2 and config-1
+    layer shapes, `strict=True`) and wherever the data are of order one.  Only the stress cases that
+    put the data far off centre or make the sums cancel (named where they pass `strict=False`) may
+    use 1e-4 or twice the error the reference's own fp32 arithmetic (the oracle's fp32
+    instantiation) makes on the same inputs, whichever is larger: where the sum cancels, no fp32
+    summation order is closer to another than both are to the exact value.
 """
 import itertools
 import math
@@ -35,10 +38,11 @@ def grad_err(got, want):
     return rel_err(got, want, floor=np.full(want.shape, 1e-2 * scale))
 
 
-def assert_grad_close(got, want32, want64, what):
+def assert_grad_close(got, want32, want64, what, strict=True):
     e_gpu, e_ref = grad_err(got, want64), grad_err(want32, want64)
     print("%s: gpu %.3g, fp32 reference %.3g (of max(|want|, 1%% of the scale), against fp64)" % (what, e_gpu, e_ref))
-    assert e_gpu <= max(GRAD_TOL, 2.0 * e_ref), "%s: gpu %.3g, fp32 reference %.3g" % (what, e_gpu, e_ref)
+    bar = GRAD_TOL if strict else max(GRAD_TOL, 2.0 * e_ref)
+    assert e_gpu <= bar, "%s: gpu %.3g, fp32 reference %.3g, bar %.3g" % (what, e_gpu, e_ref, bar)
 
 
 def f64(*arrays):
@@ -52,7 +56,7 @@ def sim_grads_gpu(pkg, x, t, w, g, **kw):
     return dx.cpu().numpy(), dt.cpu().numpy(), dw.cpu().numpy()
 
 
-def check_sim_grads(pkg, x, t, w, seed=99, **kw):
+def check_sim_grads(pkg, x, t, w, seed=99, strict=True, **kw):
     out = orc.similarity_fwd(x, t, w, **kw)
     g = np.random.default_rng(seed).normal(size=out.shape).astype(np.float32)
     dx, dt, dw = sim_grads_gpu(pkg, x, t, w, g, **kw)
@@ -61,9 +65,9 @@ def check_sim_grads(pkg, x, t, w, seed=99, **kw):
     d = f64(x, t, w, g)
     true_dx = orc.similarity_input_grad(*d, **kw)
     true_dt, true_dw = orc.similarity_params_grad(*d, **kw)
-    assert_grad_close(dx, want_dx, true_dx, "input grad")
-    assert_grad_close(dt, want_dt, true_dt, "templates grad")
-    assert_grad_close(dw, want_dw, true_dw, "weights grad")
+    assert_grad_close(dx, want_dx, true_dx, "input grad", strict)
+    assert_grad_close(dt, want_dt, true_dt, "templates grad", strict)
+    assert_grad_close(dw, want_dw, true_dw, "weights grad", strict)
 
 
 # ---- the reference's own gradient test matrix (python/simnets/test/__init__.py:55-103, :143-154) ------------
@@ -191,13 +195,13 @@ def test_similarity_grads_nan_input_without_ignore_propagates_like_the_reference
 
 def test_similarity_grads_first_layer_of_the_missing_data_network(pkg):
     x, t, w, kw = config1(batch=8, nan_frac=0.25)
-    check_sim_grads(pkg, x, t, w, **kw)
+    check_sim_grads(pkg, x, t, w, strict=True, **kw)
 
 
 @pytest.mark.parametrize("func", ["L2", "L1"])
 def test_similarity_grads_conv_scale_shape_small_batch(pkg, func):
     x, t, w, kw = config3(batch=3)
-    check_sim_grads(pkg, x, t, w, similarity_function=func, **kw)
+    check_sim_grads(pkg, x, t, w, similarity_function=func, strict=True, **kw)
 
 
 def oracle_params_grad_over_batch(x, t, w, g, kw, dtype, threads=8):
@@ -230,7 +234,7 @@ def test_similarity_grads_conv_scale_full_batch_against_the_oracle(pkg, func, re
     for b in (0, 131, 255):
         want = orc.similarity_input_grad(x[b:b + 1], t, w, g[b:b + 1], **kw)
         true = orc.similarity_input_grad(*f64(x[b:b + 1], t, w, g[b:b + 1]), **kw)
-        assert_grad_close(dx[b:b + 1].cpu().numpy(), want, true, "input grad of image %d" % b)
+        assert_grad_close(dx[b:b + 1].cpu().numpy(), want, true, "input grad of image %d" % b, strict=True)
     idx = [0, 1, 37, 63, 64, 100, 126, 127]
     gs = np.ascontiguousarray(g[:, idx])
     ref_dt, ref_dw = oracle_params_grad_over_batch(x, t[idx], w[idx], gs, kw, np.float32)
@@ -242,10 +246,7 @@ def test_similarity_grads_conv_scale_full_batch_against_the_oracle(pkg, func, re
         print("config-3 %s parameter gradients, 256 images, algo=%s: templates %.3g, weights %.3g of the scale "
               "(fp32 oracle: %.3g, %.3g)" % (func, algo, e[0], e[1], e_ref[0], e_ref[1]))
         record_property("params_grad_err_%s_%s" % (func, algo), e)
-        if algo == "direct":
-            assert max(e) <= GRAD_TOL, e
-        else:
-            assert e[0] <= max(GRAD_TOL, 2 * e_ref[0]) and e[1] <= max(GRAD_TOL, 2 * e_ref[1]), (e, e_ref)
+        assert max(e) <= GRAD_TOL, (algo, e, e_ref)        # the plain bar, default forms included
         dt3, dw3 = pkg.similarity_parameters_grad(X, T, W, 2.0 * G, algo=algo, **kw)
         assert torch.equal(dt3, 2.0 * dt) and torch.equal(dw3, 2.0 * dw)      # scaling by 2 is exact in fp32
 
@@ -281,7 +282,7 @@ def mex_case(seed, im_dims, num_instances, **kw):
     return x, off
 
 
-def check_mex_grads(pkg, x, off, n, seed=77, **kw):
+def check_mex_grads(pkg, x, off, n, seed=77, strict=True, **kw):
     out = orc.mex_fwd(x, off, n, **kw)
     g = np.random.default_rng(seed).normal(size=out.shape).astype(np.float32)
     X, O, Y, G = dev(x), dev(off), dev(out), dev(g)
@@ -290,9 +291,9 @@ def check_mex_grads(pkg, x, off, n, seed=77, **kw):
     x64, off64, g64 = f64(x, off, g)
     out64 = orc.mex_fwd(x64, off64, n, **kw)
     assert_grad_close(dx, orc.mex_input_grad(x, off, out, g, n, **kw), orc.mex_input_grad(x64, off64, out64, g64, n, **kw),
-                      "input grad")
+                      "input grad", strict)
     assert_grad_close(doff, orc.mex_offsets_grad(x, off, out, g, n, **kw),
-                      orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "offsets grad")
+                      orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw), "offsets grad", strict)
 
 
 # the reference's gradient tests (python/simnets/test/__init__.py:329-372)
@@ -360,7 +361,11 @@ def test_mex_grads_offset_ranges_product_and_term_by_term_forms(pkg, geom, sprea
         off *= 300
     elif spread == "mixed":
         off[::2] *= 300
-    check_mex_grads(pkg, x, off, geom["n"], **kw)
+    # Stress case that needs the allowance (strict=False): inputs spanning +-16 and offsets spanning up to +-300,
+    # times epsilon up to 12, put exponents of several hundred next to each other; the forward output the gradients
+    # are formed from is then known to about 1e-5 of such an exponent, and the reference's own fp32 arithmetic is
+    # 2e-4 ... 3e-3 away from the exact gradient here (the GPU's error equals it to two digits).
+    check_mex_grads(pkg, x, off, geom["n"], strict=False, **kw)
 
 
 @pytest.mark.parametrize("eps", [2.0, -math.inf])
@@ -381,7 +386,7 @@ def test_mex_input_grad_of_overlapping_patches_is_reproducible(pkg, eps):
 def test_mex_grads_config2_shape(pkg):
     x, off, n, kw = config2(batch=64)
     off = orc.normalize_offsets(off)
-    check_mex_grads(pkg, x, off, n, **kw)
+    check_mex_grads(pkg, x, off, n, strict=True, **kw)
 
 
 def test_mex_offsets_grad_through_the_offset_normalisation(pkg):
@@ -568,7 +573,9 @@ def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, sp
     off = off * 0.3
     if spread == "mixed":
         off[::2] *= 300
-    check_mex_grads(pkg, x, off, 200, **kw)
+    # 'mixed' is a stress case that needs the allowance (offsets spanning +-300: the fp32 reference itself is more
+    # than 1e-4 from the exact gradient); the narrow case meets the plain bar
+    check_mex_grads(pkg, x, off, 200, strict=spread != "mixed", **kw)
 
 
 @pytest.mark.parametrize("case", [

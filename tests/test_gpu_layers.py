@@ -285,14 +285,69 @@ def test_modules_pack_parameters_once_for_inference(pkg):
     y_train = mexl(sim(x))
     with torch.no_grad():
         y1 = mexl(sim(x))
-        first = (sim._prepared[1], mexl._prepared[1])
+        first = (sim._prepared.last(), mexl._prepared.last())
         y2 = mexl(sim(x))
-        assert sim._prepared[1] is first[0] and mexl._prepared[1] is first[1]      # reused
+        assert sim._prepared.last() is first[0] and mexl._prepared.last() is first[1]      # reused
         assert torch.equal(y1, y_train.detach()) and torch.equal(y2, y1)
         sim.templates.add_(0.25)
         mexl.offsets.mul_(0.5)
         y3 = mexl(sim(x))
-        assert sim._prepared[1] is not first[0] and mexl._prepared[1] is not first[1]
+        assert sim._prepared.last() is not first[0] and mexl._prepared.last() is not first[1]
     assert torch.equal(y3, mexl(sim(x)).detach()) and not torch.equal(y3, y1)
     with torch.no_grad():
         assert mexl(sim(x[:2])).shape[0] == 2                                      # another input shape: prepared anew
+
+
+def test_modules_notice_rebound_parameters_changed_attributes_and_other_streams(pkg):
+    """The inference cache must never serve a stale packed buffer: rebinding a parameter (a new tensor object whose
+    version counter starts at 0 again), `load_state_dict(assign=True)`, and a changed layer attribute each prepare
+    anew; a write through `.data` (invisible to torch's version counter) needs `invalidate_prepared()`; every stream
+    gets a buffer of its own.  Each result equals the grad-mode forward, which packs on every call."""
+    g = torch.Generator(device="cuda").manual_seed(11)
+    sim = pkg.Similarity(9, blocks=[3, 3], strides=[1, 1], padding=[1, 1]).cuda()
+    mexl = pkg.Mex(5, blocks=[-1, 1, 1], strides=[9, 1, 1], softmax_mode=True, normalize_offsets=True,
+                   unshared_offset_region=[2]).cuda()
+    x = torch.randn((2, 4, 8, 8), device="cuda", generator=g)
+
+    def both():
+        with torch.no_grad():
+            fast = mexl(sim(x))
+        slow = mexl(sim(x)).detach()
+        assert torch.equal(fast, slow)
+        return fast
+
+    y0 = both()
+    # rebinding: fresh Parameter objects (version 0, like the ones they replace)
+    sim.templates = torch.nn.Parameter(torch.randn(sim.templates.shape, device="cuda", generator=g))
+    mexl.offsets = torch.nn.Parameter(torch.randn(mexl.offsets.shape, device="cuda", generator=g))
+    y1 = both()
+    assert not torch.equal(y1, y0)
+    # load_state_dict(assign=True) swaps the tensors as well
+    state = {k: torch.randn(v.shape, device="cuda", generator=g) for k, v in sim.state_dict().items()}
+    sim.load_state_dict(state, assign=True)
+    y2 = both()
+    assert not torch.equal(y2, y1)
+    # a layer attribute changed after the first call
+    sim.out_of_bounds_value = 3.0
+    mexl.epsilon = 2.0
+    y3 = both()
+    assert not torch.equal(y3, y2)
+    # .data writes are invisible to the version counter: the documented way is invalidate_prepared()
+    sim.sweights.data.mul_(1.5)
+    mexl.offsets.data.add_(0.5 * torch.randn(mexl.offsets.shape, device="cuda", generator=g))
+    sim.invalidate_prepared()
+    mexl.invalidate_prepared()
+    y4 = both()
+    assert not torch.equal(y4, y3)
+    # another stream: its own buffer, the first stream's one kept
+    main = sim._prepared.last()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side), torch.no_grad():
+        y5 = mexl(sim(x))
+        assert sim._prepared.last() is not main
+    side.synchronize()
+    assert torch.equal(y5, y4)
+    with torch.no_grad():
+        mexl(sim(x))
+    assert sim._prepared.last(pkg.ops._current_stream(x.device)) is main

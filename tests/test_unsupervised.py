@@ -109,3 +109,83 @@ def test_nan_patches_are_skipped_and_bad_kind_is_rejected():
     assert torch.isfinite(layer.templates).all()
     with pytest.raises(ValueError):
         uns.similarity_unsupervised_init("svm", layer, data, batch_size=8)
+
+
+# ---- single steps against what the mathematics fixes ------------------------------------------------------------
+def test_one_kmeans_step_from_a_fixed_start_is_assignment_plus_mean():
+    """With zero counts, one mini-batch step moves every centre that received points to the plain mean of its points
+    (brute-force nearest-centre assignment in float64) and leaves the others alone: one Lloyd step."""
+    g = np.random.default_rng(21)
+    pts = g.normal(size=(300, 6)).astype(np.float32)
+    start = np.concatenate([pts[[3, 50, 120, 200]], np.full((1, 6), 40.0, np.float32)])   # the last centre gets nothing
+    km = uns.MiniBatchKMeans(5)
+    km.centers = torch.from_numpy(start.copy())
+    km.counts = torch.zeros(5)
+    km.partial_fit(torch.from_numpy(pts))
+    d = ((pts[:, None].astype(np.float64) - start[None].astype(np.float64)) ** 2).sum(-1)
+    assign = d.argmin(1)
+    assert set(assign) == {0, 1, 2, 3}
+    for c in range(4):
+        np.testing.assert_allclose(km.centers[c].numpy(), pts[assign == c].astype(np.float64).mean(0), rtol=0, atol=1e-5)
+    assert np.array_equal(km.centers[4].numpy(), start[4])
+    assert np.array_equal(km.counts.numpy(), np.bincount(assign, minlength=5).astype(np.float32))
+    # a second batch: the centre is the mean of everything it has been given (the 1/count step rule, summed)
+    more = g.normal(size=(100, 6)).astype(np.float32) + km.centers[0].numpy()
+    before, n0 = km.centers.clone().double().numpy(), km.counts.clone().numpy()
+    km.partial_fit(torch.from_numpy(more))
+    d2 = ((more[:, None].astype(np.float64) - before[None]) ** 2).sum(-1).argmin(1)
+    for c in range(5):
+        sel = more[d2 == c].astype(np.float64)
+        want = before[c] if len(sel) == 0 else (before[c] * n0[c] + sel.sum(0)) / (n0[c] + len(sel))
+        np.testing.assert_allclose(km.centers[c].numpy(), want, rtol=0, atol=1e-5)
+
+
+def _diag_gmm_loglik(pts, means, covs):
+    """Mean log-likelihood of a uniform mixture of diagonal Gaussians, float64, straight from the definition."""
+    pts, means, covs = (np.asarray(a, dtype=np.float64) for a in (pts, means, covs))
+    diff = pts[:, None, :] - means[None]
+    logp = -0.5 * ((diff ** 2) / covs[None] + np.log(2 * np.pi * covs)[None]).sum(-1) - np.log(len(means))
+    m = logp.max(1, keepdims=True)
+    return float((m[:, 0] + np.log(np.exp(logp - m).sum(1))).mean())
+
+
+def test_em_steps_never_decrease_the_likelihood_and_follow_the_textbook_update():
+    g = np.random.default_rng(22)
+    centres = g.normal(size=(3, 5)) * 3
+    pts = np.concatenate([c + g.normal(size=(150, 5)) * s for c, s in zip(centres, (0.5, 1.0, 1.5))]).astype(np.float32)
+    gmm = uns.DiagonalGMM(3, generator=torch.Generator().manual_seed(2), min_var=1e-6)
+    T = torch.from_numpy(pts)
+    gmm.partial_fit(T)                       # seeds, then one step
+    ll = [_diag_gmm_loglik(pts, gmm.means, gmm.covs)]
+    for _ in range(8):
+        means0, covs0 = gmm.means.double().numpy(), gmm.covs.double().numpy()
+        gmm.partial_fit(T)
+        ll.append(_diag_gmm_loglik(pts, gmm.means, gmm.covs))
+        # the textbook EM update from (means0, covs0), in float64: responsibilities sum to 1 per point
+        diff = pts[:, None, :].astype(np.float64) - means0[None]
+        logp = -0.5 * ((diff ** 2) / covs0[None] + np.log(covs0)[None]).sum(-1)
+        resp = np.exp(logp - logp.max(1, keepdims=True))
+        resp /= resp.sum(1, keepdims=True)
+        np.testing.assert_allclose(resp.sum(1), 1.0, atol=1e-12)
+        mass = resp.sum(0)
+        means1 = resp.T @ pts.astype(np.float64) / mass[:, None]
+        covs1 = (resp[:, :, None] * (pts[:, None, :] - means1[None]) ** 2).sum(0) / mass[:, None]
+        np.testing.assert_allclose(gmm.means.numpy(), means1, rtol=2e-4, atol=2e-4)
+        np.testing.assert_allclose(gmm.covs.numpy(), np.maximum(covs1, 1e-6), rtol=2e-3, atol=2e-4)
+    assert all(b >= a - 1e-6 for a, b in zip(ll, ll[1:])), ll
+
+
+def test_pca_components_are_the_eigenvectors_torch_eigh_finds():
+    g = torch.Generator().manual_seed(23)
+    data = torch.randn(30, 2, 6, 6, generator=g) * torch.tensor([1.0, 3.0]).view(1, 2, 1, 1) + 0.7
+    pca = uns.RunningPCA()
+    for i in range(0, 30, 7):                                   # ragged batches: the running moments must not care
+        pca.partial_fit(uns.extract_patches(data[i:i + 7], (2, 3), (1, 2)))
+    patches = uns.extract_patches(data, (2, 3), (1, 2)).double()
+    mu = patches.mean(0)
+    cov = (patches - mu).t() @ (patches - mu) / patches.shape[0]
+    w, v = torch.linalg.eigh(cov)
+    order = torch.argsort(w, descending=True)
+    comps = pca.components(4)
+    for a, b in zip(comps, v[:, order[:4]].t()):
+        assert min(float((a - b).abs().max()), float((a + b).abs().max())) < 1e-8

@@ -3,7 +3,9 @@ inside the library) against simnets_hip_similarity_fwd (caller workspace), throu
 
 Both run the same kernels, so the outputs must be identical bit for bit; the oracle bounds them both (1e-5).
 The second call of every pair uses a smaller input than the first: the static array still holds the first call's
-packed parameters, thresholds and flags, and none of them may leak into the second result."""
+packed parameters, thresholds and (small-map kernel only: the tiled kernels keep them in registers) guard flags, and
+none of them may leak into the second result.  Every pair also checks that the static call leaves the device's free
+memory and torch's allocator statistics untouched."""
 import ctypes as C
 
 import numpy as np
@@ -42,6 +44,16 @@ def _call_pair(pkg, x, t, w, **kw):
                                              got.data_ptr(), stream)
     assert rc == 0, _lib.strerror(rc)
     torch.cuda.synchronize()
+    first = got.clone()
+    # the call again, now that its kernels' code is resident: nothing may be allocated, by the library or through torch
+    before = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    rc = l.simnets_hip_similarity_fwd_static(C.byref(a), xs, ts, ts, X.data_ptr(), T.data_ptr(), W.data_ptr(),
+                                             got.data_ptr(), stream)
+    assert rc == 0, _lib.strerror(rc)
+    torch.cuda.synchronize()
+    after = (torch.cuda.mem_get_info()[0], torch.cuda.memory_allocated(), torch.cuda.memory_reserved())
+    assert after == before, "the static-scratch call changed the device's memory state: %s -> %s" % (before, after)
+    assert torch.equal(got, first)
     return got.cpu().numpy(), want.cpu().numpy()
 
 
@@ -56,7 +68,7 @@ def _inputs(seed, shape, O, blocks, spread=1.0):
 def _check(pkg, x, t, w, **kw):
     got, want = _call_pair(pkg, x, t, w, **kw)
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), "static-scratch result differs from workspace result"
-    assert rel_err(got, orc.similarity_fwd(x, t, w, **kw)) <= SIM_TOL
+    assert rel_err(got, orc.similarity_fwd(x, t, w, **{k: v for k, v in kw.items() if k != "algo"})) <= SIM_TOL
 
 
 @pytest.mark.parametrize("func", ["L2", "L1"])
@@ -77,6 +89,29 @@ def test_static_scratch_guard_state_does_not_leak(pkg):
     w[4, 0, 0, 0] = -0.5           # sqrt undefined: every output of template 4 is recomputed
     _check(pkg, x, t, w, **kw)
     _check(pkg, *_inputs(22, (1, 4, 7, 9), 2, (2, 2)), **kw)
+
+
+def test_static_scratch_small_map_guard_flags_do_not_leak(pkg):
+    """The small-map kernel (several 7x7 images per wave) with the sqrt-weight form is the one path that keeps its
+    guard flags - one per workgroup - in the scratch: the main launch writes them, the recomputing launch reads them.
+    First call: an exact-match template and a negative-weight template raise flags; the second call (fewer images,
+    ordinary data, same geometry) must recompute nothing it should not and miss nothing."""
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1])
+    x, t, w = _inputs(31, (32, 16, 7, 7), 24, (3, 3))
+    t[3] = x[1, :, 2:5, 3:6]       # the patch of output pixel (3, 4) of image 1
+    w[5, 0, 0, 0] = -0.5
+    _check(pkg, x, t, w, **kw)
+    _check(pkg, *_inputs(32, (16, 16, 7, 7), 24, (3, 3)), **kw)
+    x, t, w = _inputs(33, (12, 16, 7, 7), 9, (3, 3))
+    t[8] = x[11, :, 4:7, 0:3]
+    _check(pkg, x, t, w, **kw)
+
+
+def test_static_scratch_matrix_core_path(pkg):
+    """algo='mfma' keeps its packed operand, bias and per-channel centre arrays in the scratch."""
+    kw = dict(blocks=[3, 3], strides=[1, 1], padding=[1, 1], algo="mfma")
+    _check(pkg, *_inputs(41, (4, 24, 20, 20), 70, (3, 3)), **kw)
+    _check(pkg, *_inputs(42, (2, 5, 9, 13), 3, (3, 3)), **kw)
 
 
 def test_static_scratch_normalized_ignore_nan(pkg):
