@@ -298,7 +298,10 @@ def main():
             shift = oracle.mex_fwd(x, off, n, threads=threads,
                                    **dict(kw, epsilon=math.copysign(math.inf, kw.get("epsilon", 1.0))))
             exact = oracle.mex_fwd(x.astype(np.float64), off.astype(np.float64), n, threads=threads, **kw)
-            return {"floor_max_term": rel_err(got, want, floor=shift), "plain_metric": rel_err(got, want),
+            # (the largest term's magnitude, or the largest offset's where the terms of the maximum cancel: the rounding of
+            # a normalised offset is of that size)
+            floor = np.maximum(np.abs(shift), np.abs(off).max() if np.isfinite(off).all() else 0.0)
+            return {"floor_max_term": rel_err(got, want, floor=floor), "plain_metric": rel_err(got, want),
                     "max_abs_dev": float(np.abs(got - want).max()), "max_abs_term": float(np.abs(shift).max()),
                     "plain_metric_gpu_vs_fp64_oracle": rel_err(got, exact),
                     "plain_metric_fp32_oracle_vs_fp64_oracle": rel_err(want, exact),
@@ -399,6 +402,54 @@ def main():
                     "prepared_kernel_ms (main kernel alone) are device times per call, from a HIP graph of 20 calls; "
                     "the fractions are taken on kernel_ms; the eager figures are back-to-back calls through the "
                     "Python op layer, bounded by the host's share of a call"})
+
+        # ---- the same layer on the paths that do not take the product form: offsets too far apart for it (every row's
+        #      scaled range far above 90: a max-tracked log-sum-exp on the VALU from the staged tiles) and an infinite
+        #      epsilon (the maximum alone)
+        def other_forms(tag, X, off_np, n, kw, gmac, nbytes, shape_out):
+            """device time per prepared call (HIP graph of 20) of the product form, wide offsets and eps = inf"""
+            res = {}
+            o = torch.empty(shape_out, device=dev)
+            variants = (("product_form", off_np, kw), ("wide_offsets", off_np * 1000.0, kw),
+                        ("eps_inf", off_np, dict(kw, epsilon=math.inf)))
+            for name, off_v, kw_v in variants:
+                OV = to_dev(off_v.astype(np.float32))
+                prep = pkg.mex_prepare(tuple(X.shape), OV, n, normalize_offsets=True, **kw_v)
+                _, ms_v = timed(graph_of(lambda: prep(X, out=o), 20).replay, args.steps, args.warmup)
+                res[name] = (ms_v / 20, OV, kw_v, o.clone())
+            base = res["product_form"][0]
+            out = {}
+            for name in ("wide_offsets", "eps_inf"):
+                ms_v = res[name][0]
+                e = entry(ms_v, gmac, nbytes, "hbm", flop=5, mex=True)
+                e.update({"product_form_kernel_ms": round(base, 4), "ratio_to_product_form": round(ms_v / base, 2),
+                          "entry_point": "simnets_hip_mex_fwd_prepared (device time per call, HIP graph of 20)"})
+                out["%s_%s" % (tag, name)] = e
+            return out, res
+
+        forms2, keep2 = other_forms("config2_mex", X2, off2, n2, kw2, 33554432, 6324224, (64, 64, 16, 16))
+        others.update(forms2)
+        # one deep layer of the config-4 stack (128 x 4 x 4 -> 256 instances at batch 512: the panel kernel)
+        xl3 = np.random.default_rng(1234).normal(size=(512, 128, 4, 4)).astype(np.float32)
+        offl3 = (np.random.default_rng(4567).normal(size=(4, 256, 128, 1, 1)) * 0.1).astype(np.float32)
+        kwl3 = dict(softmax_mode=True, blocks=[128, 1, 1], strides=[128, 1, 1], unshared_offset_region=[2])
+        XL3 = to_dev(xl3)
+        bytes_l3 = (xl3.size + offl3.size + 512 * 256 * 16) * 4
+        forms3, keep3 = other_forms("config4_layer3_mex", XL3, offl3, 256, kwl3, 268435456, bytes_l3, (512, 256, 4, 4))
+        others.update(forms3)
+
+        def cpu_forms():
+            """max error of the wide-offsets and infinite-epsilon results against the oracle (config-2 layer: all
+            images; deep layer: 64 of the 512 images)"""
+            out = {}
+            for tag, keep, xs_np, off_np, n, nb in (("config2_mex", keep2, x2, off2, n2, 64),
+                                                    ("config4_layer3_mex", keep3, xl3, offl3, 256, 64)):
+                for name in ("wide_offsets", "eps_inf"):
+                    _, OV, kw_v, got = keep[name]
+                    noff = oracle.normalize_offsets(OV.cpu().numpy())
+                    out["%s_%s" % (tag, name)] = mex_err(got[:nb].cpu().numpy(), xs_np[:nb], noff, n, **kw_v)["floor_max_term"]
+            return out
+        cpu_jobs.append(("mex_other_forms_max_rel_err_gpu_vs_cpu", cpu_forms))
 
         def cpu2():
             got = o2.cpu().numpy()

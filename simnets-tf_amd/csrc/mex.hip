@@ -23,10 +23,13 @@
 //   * the 4 waves of a workgroup split the instances (WM ways) and, when the grid would otherwise
 //     leave SIMDs idle, K (KS ways, WM*KS = 4): each K-split wave keeps its own (max, sum) pair and
 //     the pairs are merged through LDS at the end: sum = sum_i s_i * exp(eps*(m_i - max_i m_i)).
-//   * two sweeps over K like the reference (max, then sum of exp relative to the max).  For finite
-//     eps the patch values (when staged) and the offsets (when packed) are multiplied by eps*log2(e)
-//     once, so a term of the second sweep is add, subtract, v_exp_f32, add; a negative eps turns the
-//     reference's minimum into a maximum of the scaled values.  When K fits one chunk the second sweep reuses the LDS tile.
+//   * default for finite eps: the product form on the fp32 matrix cores (below).  Offsets too far apart for it, and
+//     infinite eps, take one pass over K with a max-tracked ("online") log-sum-exp at chunk granularity: per staged
+//     chunk the maximum of patch + offset first, then the running sums are rescaled to the new maximum and the
+//     chunk's exponentials added (the reference sweeps K twice: maximum, then sum of exp relative to it,
+//     src/kernels/mex_kernel_cpu.cpp:11-38).  For finite eps the patch values (when staged) and the offsets (when
+//     packed) are multiplied by eps*log2(e) once, so a term is add, subtract, v_exp_f32, add; a negative eps turns
+//     the reference's minimum into a maximum of the scaled values.
 //   * workgroups that own the different regions of the same pixel chunk are numbered a multiple of
 //     8 apart, so they run on the same XCD and their interleaved partial cache lines meet in one L2.
 #include <hip/hip_runtime.h>
@@ -234,7 +237,6 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
         for (int m = 0; m < MX; ++m)
             mx[p][m] = NEG ? INFINITY : -INFINITY;
 
-    const bool single_chunk = a.K <= KC;
     const float *xl = xs + lane;                 // this lane's pixels: xl[kk*TP + p*64]
     const float *ol = os + wm * MX;              // this wave's instances: ol[kk*TM + m]
 
@@ -338,8 +340,12 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
         }
         return;
     }
-    {
-    // ---- sweep 1: running max (min for negative epsilon) of patch + offset ----
+    // ---- one pass over K, chunk by chunk (wide offsets, infinite epsilon): per chunk first the maximum (minimum for a
+    //      negative infinite epsilon) of patch + offset over the chunk's k, then - finite epsilon - the running sums are
+    //      rescaled to the new running maximum and the chunk's exponentials added: a max-tracked ("online") log-sum-exp
+    //      at chunk granularity, one exponential per term and one per output and chunk; the patch elements and the
+    //      offsets are fetched once.  Patch values and offsets are already multiplied by eps*log2(e), so a term is
+    //      exp2 of a plain difference.  Infinite epsilon stops after the maximum. ----
     for (int k0 = 0; k0 < a.K; k0 += KC) {
         const int kc = min(KC, a.K - k0);
         __syncthreads();
@@ -348,75 +354,72 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
         if (!wave_active)
             continue;
         const int kend = min(kc, (wk + 1) * KW);
-        for (int kk = wk * KW; kk < kend; ++kk) {
-            float x[PX], o[MX];
+        // (one pixel of the lane and eight of the wave's instances at a time: the chunk maxima of those eight outputs
+        // are all that is held beside the running pairs, which keeps this path inside the register budget of the
+        // product form above)
+        constexpr int HM = 8;
 #pragma unroll
-            for (int p = 0; p < PX; ++p)
-                x[p] = xl[kk * XP + p * 64];
+        for (int ph = 0; ph < PX * (MX / HM); ++ph) {
+            const int p = ph / (MX / HM), h0 = (ph % (MX / HM)) * HM;
+            const float *xp = xl + p * 64;
+            const float *op = ol + h0;
+            float cm[HM];
 #pragma unroll
-            for (int m = 0; m < MX; ++m)
-                o[m] = ol[kk * TM + m];
-            // stage by stage across the 16 instances: a dependent VALU instruction issued right
-            // behind its producer stalls, so producers and consumers are kept 16 instructions apart
-#pragma unroll
-            for (int p = 0; p < PX; ++p) {
-                float v[MX];
-#pragma unroll
-                for (int m = 0; m < MX; ++m)
-                    v[m] = x[p] + o[m];
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int m = 0; m < MX; ++m)
-                    mx[p][m] = NEG ? __builtin_fminf(mx[p][m], v[m]) : __builtin_fmaxf(mx[p][m], v[m]);
-                __builtin_amdgcn_sched_barrier(0);
-            }
-        }
-    }
-
-    if (a.finite_eps) {
-        // ---- sweep 2: sum of exp(eps * (v - max)): patch values and offsets are already multiplied by
-        //      eps*log2(e), so the term is exp2 of a plain difference ----
-        for (int k0 = 0; k0 < a.K; k0 += KC) {
-            const int kc = min(KC, a.K - k0);
-            if (!single_chunk) {
-                __syncthreads();
-                stage(k0, kc);
-                __syncthreads();
-            }
-            if (!wave_active)
-                continue;
-            const int kend = min(kc, (wk + 1) * KW);
+            for (int m = 0; m < HM; ++m)
+                cm[m] = NEG ? INFINITY : -INFINITY;
+#pragma nounroll
             for (int kk = wk * KW; kk < kend; ++kk) {
-                float x[PX], o[MX];
+                const float x = xp[kk * XP];
+                float v[HM];
+                // stage by stage across the instances: a dependent VALU instruction issued right behind its producer
+                // stalls, so producers and consumers are kept apart
 #pragma unroll
-                for (int p = 0; p < PX; ++p)
-                    x[p] = xl[kk * XP + p * 64];
+                for (int m = 0; m < HM; ++m)
+                    v[m] = x + op[kk * TM + m];
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int m = 0; m < MX; ++m)
-                    o[m] = ol[kk * TM + m];
+                for (int m = 0; m < HM; ++m)
+                    cm[m] = NEG ? __builtin_fminf(cm[m], v[m]) : __builtin_fmaxf(cm[m], v[m]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if (!a.finite_eps) {
 #pragma unroll
-                for (int p = 0; p < PX; ++p) {
-                    float v[MX];
+                for (int m = 0; m < HM; ++m)
+                    mx[p][h0 + m] = NEG ? __builtin_fminf(mx[p][h0 + m], cm[m]) : __builtin_fmaxf(mx[p][h0 + m], cm[m]);
+                continue;
+            }
+            // new running maximum; sums so far rescaled to it (a maximum that did not move: factor 1, which also keeps
+            // -inf - -inf out of the exponent while nothing finite has been seen)
 #pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        v[m] = x[p] + o[m];
-                    __builtin_amdgcn_sched_barrier(0);
+            for (int m = 0; m < HM; ++m) {
+                const float mo = mx[p][h0 + m];
+                const float mn = __builtin_fmaxf(mo, cm[m]);
+                s[p][h0 + m] *= mn == mo ? 1.0f : __builtin_amdgcn_exp2f(mo - mn);
+                mx[p][h0 + m] = mn;
+                cm[m] = mn == -INFINITY ? 0.0f : mn;   // what the chunk's terms subtract
+            }
+#pragma nounroll
+            for (int kk = wk * KW; kk < kend; ++kk) {
+                const float x = xp[kk * XP];
+                float v[HM];
 #pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        v[m] = v[m] - mx[p][m];
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int m = 0; m < HM; ++m)
+                    v[m] = x + op[kk * TM + m];
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        v[m] = __builtin_amdgcn_exp2f(v[m]);
-                    __builtin_amdgcn_sched_barrier(0);
+                for (int m = 0; m < HM; ++m)
+                    v[m] = v[m] - cm[m];
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                    for (int m = 0; m < MX; ++m)
-                        s[p][m] += v[m];
-                    __builtin_amdgcn_sched_barrier(0);
-                }
+                for (int m = 0; m < HM; ++m)
+                    v[m] = __builtin_amdgcn_exp2f(v[m]);
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int m = 0; m < HM; ++m)
+                    s[p][h0 + m] += v[m];
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-    }
     }
 
     if (KS > 1) {
@@ -570,22 +573,22 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         if (!(fabsf(mxv) < INFINITY))
             mxv = 0.0f;
         float sum = 0.0f;
-        each([&](int, float x) { sum += expf(x - mxv); });
+        each([&](int, float x) { sum += mex_exp_term(x - mxv); });
         for (int d = 32; d > 0; d >>= 1)
             sum += __shfl_xor(sum, d, 64);
-        lse = logf(sum) + mxv;
+        lse = mex_lse_of(sum, mxv);
     }
     if (normalized_out != nullptr) {   // the same values as mex_normalize_rows_kernel writes
         float *nd = normalized_out + ((size_t)r * M + m) * K;
         each([&](int k, float x) { nd[k] = x - lse; });
     }
     if (!finite_eps) {
-        each([&](int k, float x) { dst[(size_t)k * tm] = (x - lse) * scale; });
+        each([&](int k, float x) { dst[(size_t)k * tm] = mex_scaled_offset(x, lse, scale); });
         return;
     }
     float hi = -INFINITY, lo = INFINITY;
     each([&](int, float x) {
-        const float v = (x - lse) * scale;
+        const float v = mex_scaled_offset(x, lse, scale);
         hi = fmaxf(hi, v);
         lo = fminf(lo, v);
     });
@@ -594,7 +597,7 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         lo = fminf(lo, __shfl_xor(lo, d, 64));
     }
     each([&](int k, float x) {
-        const float v = (x - lse) * scale;
+        const float v = mex_scaled_offset(x, lse, scale);
         dst[(size_t)k * tm] = v;
         dste[(size_t)k * tm] = __builtin_amdgcn_exp2f(v - hi);
     });
@@ -982,6 +985,13 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
     }
     const MexTiling t = mex_tiling(p);
     MexKernelArgs a = mex_kernel_args(p);
+    if (pack && (phase & kMexRun) && mex_panel_geometry(p)) {
+        // a whole self-packing call of a small single-chunk layer: one launch that packs inside its workgroups
+        a.n_mgroups = t.n_mgroups;
+        const int src = mex_panel_launch_selfpack(p, a, input, offsets, output, stream);
+        if (src != SIMNETS_PANEL_NOT_TAKEN)
+            return src;
+    }
     const int rc = mex_pack_offsets(p, offsets, t.tm, t.n_mgroups, workspace, &a, stream, nullptr, pack);
     if (rc || !(phase & kMexRun))
         return rc;

@@ -122,6 +122,29 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     return a;
 }
 
+// The scaled, normalised offset every packing path stores (and exponentiates relative to its row maximum): kept out of
+// the compiler's multiply-add fusion so that the pack kernel and the kernels that pack for themselves agree bit for bit.
+__device__ __forceinline__ float mex_scaled_offset(float x, float lse, float scale)
+{
+#pragma clang fp contract(off)
+    return (x - lse) * scale;
+}
+
+// exp(d) for d <= 0 and the row's logsumexp from the sum of such terms, as the packing paths compute them for
+// normalize_offsets: one v_exp_f32 / v_log_f32 each (results within about an ulp of the library functions', at a
+// tenth of their instructions: a workgroup that packs for itself evaluates 32 of them per thread), in one place so
+// that every path rounds alike.  Terms below 2^-126 of the largest come out as 0.
+__device__ __forceinline__ float mex_exp_term(float d)
+{
+#pragma clang fp contract(off)
+    return __builtin_amdgcn_exp2f(d * 1.44269504088896341f);
+}
+__device__ __forceinline__ float mex_lse_of(float sum, float mxv)
+{
+#pragma clang fp contract(off)
+    return __builtin_amdgcn_logf(sum) * 0.693147180559945309f + mxv;
+}
+
 // Packs the offsets for the forward kernels (k-major tiles of tm instances per group: scaled values, their
 // exponentials relative to the row maximum, row maxima and ranges) and the patch element table into `workspace`
 // (mex_packed_bytes), and points the argument block at them.
@@ -150,5 +173,11 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
 constexpr int SIMNETS_PANEL_NOT_TAKEN = 1;
 bool mex_panel_geometry(const MexPlan &p);
 int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *input, float *output, void *stream);
+// The whole self-packing call of such a layer as ONE launch when its patches are a single chunk (32 channels) and the
+// grid is small: every workgroup packs the offsets rows it needs (4 regions x 64 instances, one row per thread) into
+// its LDS tile itself, with the pack kernel's arithmetic in the pack kernel's order (bit-identical results).  Returns
+// SIMNETS_PANEL_NOT_TAKEN without launching anything when the layer or the pointers do not qualify.
+int mex_panel_launch_selfpack(const MexPlan &p, const MexKernelArgs &a, const float *input, const float *offsets,
+                              float *output, void *stream);
 
 }  // namespace simnets

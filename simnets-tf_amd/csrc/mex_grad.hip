@@ -806,10 +806,10 @@ __global__ __launch_bounds__(256) void mex_normalize_rows_kernel(const float *__
         mxv = 0.0f;
     float sum = 0.0f;
     for (int k = lane; k < K; k += 64)
-        sum += expf(s[k] - mxv);
+        sum += mex_exp_term(s[k] - mxv);   // (the pack kernel's arithmetic: both write the same normalised rows)
     for (int d = 32; d > 0; d >>= 1)
         sum += __shfl_xor(sum, d, 64);
-    const float lse = logf(sum) + mxv;
+    const float lse = mex_lse_of(sum, mxv);
     for (int k = lane; k < K; k += 64)
         dst[(size_t)row * K + k] = s[k] - lse;
 }

@@ -11,7 +11,7 @@
 // Arithmetic as in the tiled forward kernel (finite epsilon): product form on the fp32 matrix cores,
 //   S[instance][pixel] = sum_k exp2(o_k - max o) * exp2(x_k - max x)   (v_mfma_f32_16x16x4_f32),
 // per 16-pixel tile with the offsets tile of that tile's region; workgroups whose offsets span too wide a range
-// for the product form evaluate the logsumexp term by term instead (slow, rare).
+// for the product form evaluate a max-tracked log-sum-exp on the VALU from the same LDS tiles instead (lse_chunk).
 #include <hip/hip_runtime.h>
 
 #include <cmath>
@@ -43,6 +43,58 @@ struct PoolArgs {
     float soob, snorm;      // out-of-bounds value; -0.5 K log(2 pi) of the normalized mode
     int snorm_every, sB;    // reproduce the reference's per-iteration addition of that constant
 };
+
+// Offsets too far apart for the product form: max-tracked ("online") log-sum-exp at chunk granularity on the VALU, on
+// the same LDS tiles and the same lane layout as the matrix form - lane (lr, lq) owns column lr of each of the four
+// 16-column tiles of its column half and instances 4*lq + v of its wave.  xs holds the scaled patch values of the
+// chunk ([k][column]), os the scaled offsets ([region][k][instance], not their exponentials); tile t belongs to
+// region t % R.  Per chunk: the maximum of patch + offset over the chunk's k, then the running sums are rescaled to the
+// new running maximum and the chunk's exponentials added - one exponential per term and one per output and chunk,
+// the tiles read twice from LDS and nothing again from memory.  SWZ: the panel kernel's swizzled tiles.
+template <int R, int XP, bool SWZ>
+__device__ __forceinline__ void lse_chunk(float (&best)[4][4], float (&sum)[4][4], const float *xs, const float *os,
+                                          int colbase, int wm, int lr, int lq, int kc)
+{
+    // (one tile at a time: four running pairs' worth of temporaries, so that this path stays inside the register
+    // budget of the matrix form, whose occupancy the whole kernel's allocation decides)
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        auto fetch = [&](int kk, float &x, float4 &o) {
+            const int sx = SWZ ? (((kk & 3) << 4) | (((kk >> 2) & 3) << 2)) : 0;
+            const int so = SWZ ? ((kk & 3) << 4) : 0;
+            x = xs[kk * XP + ((colbase + t * 16 + lr) ^ sx)];
+            o = *reinterpret_cast<const float4 *>(os + (t % R) * KC * TM + kk * TM + ((wm * MX + 4 * lq) ^ so));
+        };
+        float cb[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
+#pragma unroll 2
+        for (int kk = 0; kk < kc; ++kk) {
+            float x;
+            float4 o;
+            fetch(kk, x, o);
+            cb[0] = fmaxf(cb[0], x + o.x); cb[1] = fmaxf(cb[1], x + o.y);
+            cb[2] = fmaxf(cb[2], x + o.z); cb[3] = fmaxf(cb[3], x + o.w);
+        }
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const float bo = best[t][v];
+            const float nb = fmaxf(bo, cb[v]);
+            // (a maximum that did not move: factor 1, which also keeps -inf - -inf out of the exponent)
+            sum[t][v] *= bo == nb ? 1.0f : __builtin_amdgcn_exp2f(bo - nb);
+            best[t][v] = nb;
+            cb[v] = nb == -INFINITY ? 0.0f : nb;   // what the chunk's terms subtract
+        }
+#pragma unroll 2
+        for (int kk = 0; kk < kc; ++kk) {
+            float x;
+            float4 o;
+            fetch(kk, x, o);
+            sum[t][0] += __builtin_amdgcn_exp2f(x + o.x - cb[0]);
+            sum[t][1] += __builtin_amdgcn_exp2f(x + o.y - cb[1]);
+            sum[t][2] += __builtin_amdgcn_exp2f(x + o.z - cb[2]);
+            sum[t][3] += __builtin_amdgcn_exp2f(x + o.w - cb[3]);
+        }
+    }
+}
 
 // NH = column halves of a workgroup (64 pixel columns = 4 tiles of 16 each), 4 instance waves per half: two halves
 // share the offsets tiles and double the waves per SIMD the LDS budget allows, which is what hides the latencies of
@@ -335,7 +387,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
                 res[t][v] = (__builtin_amdgcn_logf(acc[t][v]) + (mpt + omax[v])) * a.ln2_over_eps;
         }
     } else {
-        // term by term: running (maximum, sum) per output, rescaled when a chunk raises the maximum
+        // wide offsets: running (maximum, sum) per output on the VALU, chunk by chunk from the staged tiles
         float best[4][4], sum[4][4];
 #pragma unroll
         for (int t = 0; t < 4; ++t)
@@ -349,25 +401,8 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
             __syncthreads();
             stage(k0, kc);
             __syncthreads();
-            if (!wave_active)
-                continue;
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v) {
-                    const float *xc = xs + wh * 64 + t * 16 + lr;
-                    const float *oc = os + (t % R) * KC * TM + wm * MX + 4 * lq + v;
-                    float cb = -INFINITY;
-                    for (int kk = 0; kk < kc; ++kk)
-                        cb = fmaxf(cb, xc[kk * XP] + oc[kk * TM]);
-                    const float nb = fmaxf(best[t][v], cb);
-                    const float nsub = nb == -INFINITY ? 0.0f : nb;
-                    float sacc = sum[t][v] * (best[t][v] == nb ? 1.0f : __builtin_amdgcn_exp2f(best[t][v] - nb));
-                    for (int kk = 0; kk < kc; ++kk)
-                        sacc += __builtin_amdgcn_exp2f(xc[kk * XP] + oc[kk * TM] - nsub);
-                    sum[t][v] = sacc;
-                    best[t][v] = nb;
-                }
+            if (wave_active)
+                lse_chunk<R, XP, false>(best, sum, xs, os, wh * 64, wm, lr, lq, kc);
         }
         if (!wave_active)
             return;
@@ -422,13 +457,54 @@ struct PanelArgs {
     int ppi;          // parts per image
     int total_parts;  // B * ppi
     int HW;
+    const float *raw_offsets;  // SELFPACK: the offsets as the caller holds them, [region][M][K]
+    int normalize;             // SELFPACK: subtract every row's logsumexp first (normalize_offsets)
 };
 
+// One offsets row of 32 elements packed by one thread, with the arithmetic of mex_pack_offsets_kernel<1> in its order:
+// the lanes of that kernel hold one element each and add their exponentials in a butterfly (partner lane ^ 32, 16, 8,
+// 4, 2, 1; the upper half of the wave holds zeros for a row of 32), which is the tree below.
+__device__ __forceinline__ void pack_row32(const float (&x)[32], int normalize, float scale, float &lse, float &hi,
+                                           float &lo)
+{
+    lse = 0.0f;
+    if (normalize) {
+        float mxv = -INFINITY;
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            mxv = fmaxf(mxv, x[k]);
+        if (!(fabsf(mxv) < INFINITY))
+            mxv = 0.0f;
+        float e[32];
+#pragma unroll
+        for (int k = 0; k < 32; ++k)
+            e[k] = mex_exp_term(x[k] - mxv);
+#pragma unroll
+        for (int d = 16; d > 0; d >>= 1)
+#pragma unroll
+            for (int k = 0; k < d; ++k)
+                e[k] = e[k] + e[k + d];
+        lse = mex_lse_of(e[0], mxv);
+    }
+    hi = -INFINITY;
+    lo = INFINITY;
+#pragma unroll
+    for (int k = 0; k < 32; ++k) {
+        const float v = mex_scaled_offset(x[k], lse, scale);
+        hi = fmaxf(hi, v);
+        lo = fminf(lo, v);
+    }
+}
+
 // POOL = false: the same tiling without the pooling, every MEX value stored (the plain MEX call on such a layer).
-template <int NH, int NCH, bool POOL>
+// SELFPACK (one column half, one chunk, no pooling): no packed offsets exist; thread (region tid / 64, instance
+// tid % 64) packs its row of the caller's offsets into the LDS tile itself (pack_row32), so that a self-packing call of
+// a small layer is this one launch.
+template <int NH, int NCH, bool POOL, bool SELFPACK = false>
 __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKernelArgs a, const PoolArgs q,
                                                                   const PanelArgs g)
 {
+    static_assert(!SELFPACK || (NH == 1 && NCH == 1 && !POOL), "in-kernel packing: one row per thread, one chunk");
     constexpr int R = 4;
     constexpr int XP = 64 * NH;
     constexpr int kThreads = 256 * NH;
@@ -437,6 +513,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
     __shared__ __attribute__((aligned(16))) float os[R * KC * TM];   // [region][k][instance ^ swizzle]
     __shared__ __attribute__((aligned(16))) float pmx[16 * XP];      // [kslot][column]: partial column maxima
     __shared__ float msh[XP];                                        // column maxima
+    __shared__ float omax_sh[SELFPACK ? R * TM : 1];                 // SELFPACK: row maxima of the scaled offsets
     // per slot: where instance 0 goes in the pooled tensor (POOL = false: where the window's first pixel goes in the
     // MEX output), -1 = no window
     __shared__ long long ppos[16 * NH];
@@ -483,10 +560,20 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         for (int u = 0; u < NV; ++u)
             pv[u] = *reinterpret_cast<const float4 *>(src + (size_t)(16 * u) * g.HW);
     }
-    SIMNETS_PANEL_ISSUE(0)
+    float4 rw[SELFPACK ? KC / 4 : 1];   // SELFPACK: this thread's row of the caller's offsets
+    const bool row_valid = SELFPACK && mgroup * TM + (tid & 63) < a.M;
+    if constexpr (SELFPACK) {
+        const float4 *src = reinterpret_cast<const float4 *>(
+            g.raw_offsets + ((size_t)(tid >> 6) * a.M + (row_valid ? mgroup * TM + (tid & 63) : 0)) * KC);
+#pragma unroll
+        for (int i = 0; i < KC / 4; ++i)
+            rw[i] = src[i];
+    } else {
+        SIMNETS_PANEL_ISSUE(0)
+    }
 
     int wide = 0;
-    if (tid < TM) {
+    if (!SELFPACK && tid < TM) {
 #pragma unroll
         for (int r = 0; r < R; ++r)
             wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
@@ -530,6 +617,22 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         const int cg = (part << g.lgF) | pg;   // 0 .. XP / 4 - 1
         reinterpret_cast<float4 *>(pmx)[kslot * (XP / 4) + cg] = pm;
     }
+    float rx[SELFPACK ? KC : 1];   // SELFPACK: the row, its logsumexp (0 without normalisation) and its scaled maximum
+    float row_lse = 0.0f, row_hi = 0.0f;
+    if constexpr (SELFPACK) {
+#pragma unroll
+        for (int i = 0; i < KC / 4; ++i) {
+            rx[4 * i] = rw[i].x; rx[4 * i + 1] = rw[i].y; rx[4 * i + 2] = rw[i].z; rx[4 * i + 3] = rw[i].w;
+        }
+        float lo;
+        pack_row32(rx, g.normalize, a.scale, row_lse, row_hi, lo);
+        if (row_valid) {
+            wide = !(row_hi - lo <= kProductRange);   // NaN or inf (infinite entries) sends the workgroup to the VALU form
+        } else {
+            row_hi = 0.0f;   // rows past the last instance: zeros, like the pack kernel's padding
+        }
+        omax_sh[tid] = row_hi;
+    }
     const bool prod = !__syncthreads_or(wide);
     float msub[4];
     {
@@ -568,7 +671,15 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
 #pragma unroll
         for (int c = 0; c < NCH; ++c) {
             // ---- registers -> LDS (the previous chunk's readers are behind the barrier that ended its loop) ----
-            {
+            if constexpr (SELFPACK) {
+                // this thread's row: exp2(scaled offset - row maximum) into the region's tile, [k][instance ^ swizzle]
+                float *orow = os + (tid >> 6) * KC * TM;
+                const int mi = tid & 63;
+#pragma unroll
+                for (int k = 0; k < KC; ++k)
+                    orow[k * TM + (mi ^ ((k & 3) << 4))] =
+                        row_valid ? __builtin_amdgcn_exp2f(mex_scaled_offset(rx[k], row_lse, a.scale) - row_hi) : 0.0f;
+            } else {
                 float4 *dst = reinterpret_cast<float4 *>(os) + ((tid & ~15) | ((tid & 15) ^ (((tid >> 4) & 3) << 2)));
 #define SIMNETS_PANEL_PUT(i) dst[((i) / NO) * TILE4 + ((i) % NO) * kThreads] = on##i;
                 SIMNETS_PANEL_PUT(0) SIMNETS_PANEL_PUT(1) SIMNETS_PANEL_PUT(2) SIMNETS_PANEL_PUT(3)
@@ -649,7 +760,8 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
             return;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            const float *omax = a.omax + ((size_t)t * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
+            const float *omax = SELFPACK ? omax_sh + t * TM + wm * MX + 4 * lq
+                                         : a.omax + ((size_t)t * a.n_mgroups + mgroup) * TM + wm * MX + 4 * lq;
             const float mp = msh[wh * 64 + t * 16 + lr];
             // an infinite column bound makes the result NaN, as the reference's exp(inf - inf) does
             const float mpt = (mp - mp) + mp + a.c0;
@@ -658,34 +770,59 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
                 res[t][v] = (__builtin_amdgcn_logf(acc[t][v]) + (mpt + omax[v])) * a.ln2_over_eps;
         }
     } else {
-        // offsets too far apart for the product form: term by term from global memory (rare, slow)
+        // offsets too far apart for the product form: the same chunks through the same (swizzled) LDS tiles - the
+        // panel's scaled values as they are and the scaled offsets instead of their exponentials - and a max-tracked
+        // log-sum-exp on the VALU (lse_chunk); the tiles requested for the product form are dropped
+        float best[4][4], sum[4][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                best[t][v] = -INFINITY;
+                sum[t][v] = 0.0f;
+            }
+        const int sw = ((kslot & 3) << 4) | (((kslot >> 2) & 3) << 2);
+        const float4 *psrc = reinterpret_cast<const float4 *>(a.offp + (size_t)mgroup * a.K * TM) + tid;
+        float4 *dst = reinterpret_cast<float4 *>(os) + ((tid & ~15) | ((tid & 15) ^ (((tid >> 4) & 3) << 2)));
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c > 0)
+                __syncthreads();  // everyone is done with the previous chunk's tiles
+            if constexpr (SELFPACK) {
+                float *orow = os + (tid >> 6) * KC * TM;
+                const int mi = tid & 63;
+#pragma unroll
+                for (int k = 0; k < KC; ++k)
+                    orow[k * TM + (mi ^ ((k & 3) << 4))] = row_valid ? mex_scaled_offset(rx[k], row_lse, a.scale) : 0.0f;
+            } else {
+#pragma unroll
+                for (int i = 0; i < R * NO; ++i)
+                    dst[(i / NO) * TILE4 + (i % NO) * kThreads] =
+                        psrc[(size_t)(i / NO) * ostep + (i % NO) * kThreads + (size_t)(c * KC) * (TM / 4)];
+            }
+            if (pvalid) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 v = pv[2 * c + h];
+                    float *row = xs + (kslot + 16 * h) * XP;
+                    row[colx[0] ^ sw] = v.x;
+                    row[colx[1] ^ sw] = v.y;
+                    row[colx[2] ^ sw] = v.z;
+                    row[colx[3] ^ sw] = v.w;
+                }
+            }
+            __syncthreads();
+            lse_chunk<R, XP, true>(best, sum, xs, os, wh * 64, wm, lr, lq, KC);
+        }
         if (!wave_active)
             return;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const PixelRef gp = locate(a, t, chunk * (16 * NH) + wh * 16 + lr);
-            const float *orow = a.offp + (((size_t)t * a.n_mgroups + mgroup) * a.K) * TM + wm * MX + 4 * lq;
-            float best[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-            for (int k = 0; k < a.K; ++k) {
-                const float x = gp.base[(size_t)k * g.HW] * a.scale;
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    best[v] = fmaxf(best[v], x + orow[(size_t)k * TM + v]);
-            }
-            float sum[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (int k = 0; k < a.K; ++k) {
-                const float x = gp.base[(size_t)k * g.HW] * a.scale;
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    sum[v] += __builtin_amdgcn_exp2f(x + orow[(size_t)k * TM + v] -
-                                                     (best[v] == -INFINITY ? 0.0f : best[v]));
-            }
+        for (int t = 0; t < 4; ++t)
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
-                const float b = best[v];
-                res[t][v] = (__builtin_amdgcn_logf(sum[v]) + ((b - b) + b + a.c0)) * a.ln2_over_eps;
+                const float b = best[t][v];
+                res[t][v] = (__builtin_amdgcn_logf(sum[t][v]) + ((b - b) + b + a.c0)) * a.ln2_over_eps;
             }
-        }
     }
 
     // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
@@ -744,6 +881,8 @@ bool panel_geometry(const MexPlan &p, int ph, int pw, const float *input, int nh
     g->lgW = lg(p.W);
     g->Ws = Ws;
     g->RS = RS;
+    g->raw_offsets = nullptr;
+    g->normalize = 0;
     return true;
 }
 
@@ -907,6 +1046,33 @@ int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *inpu
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const hipError_t e = nh == 1 ? launch_panel<1, false>(b, q, g, grid, s) : launch_panel<2, false>(b, q, g, grid, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+}
+
+int mex_panel_launch_selfpack(const MexPlan &p, const MexKernelArgs &a, const float *input, const float *offsets,
+                              float *output, void *stream)
+{
+    PanelArgs g;
+    if (p.d.K != KC || reinterpret_cast<uintptr_t>(offsets) % 16 != 0)
+        return SIMNETS_PANEL_NOT_TAKEN;
+    if (panel_halves(p, 2, 2, input, a.slots, a.n_mgroups, &g, false) != 1)
+        return SIMNETS_PANEL_NOT_TAKEN;
+    g.raw_offsets = offsets;
+    g.normalize = p.normalize_offsets;
+    PoolArgs q;
+    q.sx = nullptr;
+    q.pooled = output;
+    q.Hp = p.d.height_out / 2;
+    q.Wp = p.d.width_out / 2;
+    q.spw = 16;
+    const long long gx = ((long long)a.slots + q.spw - 1) / q.spw;
+    if (gx > 0x7fffffffLL || a.n_mgroups > 65535)
+        return SIMNETS_ERR_TOO_LARGE;
+    MexKernelArgs b = a;
+    b.in = input;
+    dim3 grid((unsigned)gx, (unsigned)a.n_mgroups);
+    hipLaunchKernelGGL((mex_pool_panel_kernel<1, 1, false, true>), grid, dim3(256), 0, reinterpret_cast<hipStream_t>(stream),
+                       b, q, g);
+    return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw)

@@ -68,6 +68,7 @@ struct SimKernelArgs {
     int NI, img_lds;   // small-map kernel: images per workgroup and LDS floats of one image's tile (one channel)
     FastDiv d_chan, d_img, d_tc;   // ... divisions of its staging loop: by NI * img_lds, img_lds, TC
     int plds_off;      // PLDS variants: where the workgroup's parameter copy starts in LDS (floats, multiple of 4)
+    int xcd_group;     // tiled kernel: number the workgroups so that the template groups of one pixel tile share an XCD
     // sqrt-weight form only (see the guard in sim_direct_kernel)
     const float *pa2;  // [mtile][K][MT][2]  (template, negative weight): what the recomputing pass reads
     const float *thr;  // [O] a partial sum of template m above -thr[m] sends its wave to the recomputing pass
@@ -79,6 +80,7 @@ struct SimKernelArgs {
 
 // Output positions of a lane.
 struct LanePos {
+    int bx, by;        // the workgroup's (pixel tile over the batch, template group)
     int b, tile, ws, mtile;
     int g_first, g_last, row_first;
     int h, gw;
@@ -88,12 +90,25 @@ struct LanePos {
 __device__ __forceinline__ LanePos lane_pos(const SimKernelArgs &a, int wave, int lane)
 {
     LanePos q;
-    q.b = blockIdx.x / a.tiles;
-    q.tile = blockIdx.x - q.b * a.tiles;
+    q.bx = blockIdx.x;
+    q.by = blockIdx.y;
+    if (a.xcd_group) {
+        // Workgroups are handed to the 8 XCDs in turn by their linear number.  The gridDim.y template groups that
+        // stage the same pixel tile take numbers a multiple of 8 apart and next to each other in time, so they run on
+        // one XCD in the same round and the tile is fetched from HBM once: linear number = ((tile / 8) * gridDim.y +
+        // group) * 8 + tile % 8.  (gridDim.x is a multiple of 8 when the host sets this.)
+        const unsigned l = blockIdx.x + gridDim.x * blockIdx.y;
+        const unsigned j = l >> 3;
+        const unsigned q8 = j / gridDim.y;
+        q.by = (int)(j - q8 * gridDim.y);
+        q.bx = (int)(q8 * 8 + (l & 7));
+    }
+    q.b = q.bx / a.tiles;
+    q.tile = q.bx - q.b * a.tiles;
     q.ws = wave & (a.nws - 1);                   // which 64 pixel groups of the tile
     const int wm = wave >> a.nws_log2;           // which MT templates
     const int nwm = kWaves >> a.nws_log2;
-    q.mtile = blockIdx.y * nwm + wm;
+    q.mtile = q.by * nwm + wm;
     q.wave_active = q.mtile < a.n_mtiles;
     q.g_first = q.tile * 64 * a.nws;
     q.g_last = min(q.g_first + 64 * a.nws, a.gpi) - 1;
@@ -195,7 +210,7 @@ __device__ __forceinline__ void sim_direct_body(const SimKernelArgs &a, float *l
         // copy the parameters of the workgroup's template tiles: [wm][pa: K*MT*2 | slack | pc: K*MT | slack]
         const int nwm = kWaves >> a.nws_log2;
         for (int j = 0; j < nwm; ++j) {
-            const int mt = min((int)blockIdx.y * nwm + j, a.n_mtiles - 1);
+            const int mt = min(lp.by * nwm + j, a.n_mtiles - 1);
             const float *ga = a.pa + (size_t)mt * a.K * MT * 2;
             float *la = lds + a.plds_off + j * 3 * pk;
             for (int i = tid; i < a.K * MT * 2; i += kThreads)
@@ -964,8 +979,9 @@ bool use_plds(const SimPlan &p, const Tiling &t)
 }
 
 template <int MODE, bool GATED = false>
-hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipStream_t s)
+hipError_t launch_mode(const SimKernelArgs &a0, const Tiling &t, bool plds, hipStream_t s)
 {
+    SimKernelArgs a = a0;
     if (!t.lds_ok) {
         const long long npix = (long long)a.B * a.oh * a.ow;
         dim3 grid((unsigned)((npix + 255) / 256), (unsigned)a.n_mtiles);
@@ -996,6 +1012,7 @@ hipError_t launch_mode(const SimKernelArgs &a, const Tiling &t, bool plds, hipSt
     size_t lds_bytes = (size_t)a.CC * a.TRmax * a.TC * sizeof(float);
     if (GATED)
         return hipSuccess;   // the tiled kernels recompute flagged waves inside the main launch
+    a.xcd_group = grid.y > 1 && grid.x % 8 == 0;
     if (t.PT == kBigPT && t.MT == kBigMT)
         return launch_direct<MODE, kBigPT, kBigMT, false>(a, grid, lds_bytes, s);
     if (plds) {
@@ -1108,6 +1125,7 @@ static int sim_direct_run_on(const SimPlan &p, const float *input, float *output
     a.vec_store = (p.ow % 4 == 0) && ((reinterpret_cast<uintptr_t>(output) & 15) == 0);
     a.TC = t.TC; a.TRmax = t.TRmax; a.CC = t.CC; a.fast_stage = t.fast_stage;
     a.plds_off = (int)align_up((size_t)t.CC * t.chan_pitch, 4);
+    a.xcd_group = 0;
     a.NI = t.NI; a.img_lds = t.TRmax * t.TC;
     a.d_chan = make_fast_div((unsigned)std::max(1, t.chan_pitch)); a.d_img = make_fast_div((unsigned)std::max(1, a.img_lds));
     a.d_tc = make_fast_div((unsigned)std::max(1, t.TC));

@@ -455,7 +455,7 @@ def test_mex_sum_pool_fused_kernel(pkg, case, spread, eps):
     ((37, 64, 8, 8), 70), ((21, 128, 4, 4), 64), ((45, 256, 2, 2), 130), ((5, 64, 16, 16), 64), ((3, 64, 24, 16), 16),
     ((2, 64, 4, 64), 16), ((64, 64, 16, 16), 256), ((9, 32, 16, 16), 64), ((3, 32, 4, 8), 20),
 ])
-@pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("mixed", 3.0)])
+@pytest.mark.parametrize("spread,eps", [("narrow", 1.0), ("narrow", -2.0), ("mixed", 3.0), ("wide", 1.0), ("wide", -2.0)])
 def test_mex_panel_form_of_the_plain_call(pkg, im, n, spread, eps):
     # 2x2 unshared offsets over whole-channel patches of 32 / 64 / 128 / 256 channels: the plain MEX call runs the panel
     # kernel without its pooling; an input that is not 16-byte aligned takes the general tiled kernel on the same
@@ -467,6 +467,8 @@ def test_mex_panel_form_of_the_plain_call(pkg, im, n, spread, eps):
     off = (g.normal(size=(4, n, im[1], 1, 1)) * 0.3).astype(np.float32)
     if spread == "mixed":
         off[:, n // 2:] *= 400
+    elif spread == "wide":      # every workgroup runs the max-tracked log-sum-exp on the VALU from the staged tiles
+        off *= 400
     got = run_mex(pkg, x, off, n, **kw)
     assert got.shape == (im[0], n, im[2], im[3])
     assert mex_err(got, x, off, n, **kw) <= MEX_TOL
@@ -536,8 +538,10 @@ def test_mex_sum_pool_other_geometries_run_the_two_kernels(pkg, kw, pool):
 @pytest.mark.parametrize("case", [
     dict(im=(9, 1, 28, 28), O=32, n=64), dict(im=(40, 1, 30, 34), O=40, n=70), dict(im=(3, 2, 13, 16), O=8, n=5),
 ])
-def test_similarity_mex_sum_pool_one_kernel(pkg, sim, case):
+@pytest.mark.parametrize("spread", ["narrow", "wide"])
+def test_similarity_mex_sum_pool_one_kernel(pkg, sim, case, spread):
     # Similarity channels = the MEX patch of a pixel, offsets unshared over the pooling window: a single kernel
+    # ("wide": offsets too far apart for the product form - the kernel's max-tracked log-sum-exp on the VALU)
     g = np.random.default_rng(23)
     im, O, n = case["im"], case["O"], case["n"]
     if im[1] * sim["blocks"][0] * sim["blocks"][1] > 16:
@@ -551,7 +555,7 @@ def test_similarity_mex_sum_pool_one_kernel(pkg, sim, case):
     mkw = dict(softmax_mode=True, blocks=[O, 1, 1], strides=[O, 1, 1], use_unshared_regions=True,
                unshared_offset_region=[1, 2, 2])
     d = orc.mex_dims(orc.mex_args(s_ref.shape, n, **mkw))
-    off = (g.normal(size=(d.num_regions, n, O, 1, 1)) * 0.2).astype(np.float32)
+    off = (g.normal(size=(d.num_regions, n, O, 1, 1)) * (60.0 if spread == "wide" else 0.2)).astype(np.float32)
     got = pkg.similarity_mex_sum_pool(dev(x), dev(t), dev(w), dev(off), n, (2, 2), similarity=sim,
                                       mex=dict(mkw, normalize_offsets=True)).cpu().numpy()
     offn = orc.normalize_offsets(off)

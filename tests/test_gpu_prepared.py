@@ -142,6 +142,39 @@ def test_mex_prepared_matches_plain_call_and_oracle(pkg, case, normalize, eps):
         assert mex_err(got.cpu().numpy(), x, ref_off, n, **kw) <= MEX_TOL
 
 
+@pytest.mark.parametrize("spread", ["narrow", "wide", "mixed", "masked"])
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("im,n", [((64, 32, 16, 16), 64), ((9, 32, 16, 16), 20), ((7, 32, 8, 16), 70), ((3, 32, 4, 8), 130)])
+def test_mex_small_single_chunk_layer_packs_inside_its_kernel(pkg, im, n, normalize, spread):
+    """A self-packing call of a layer with 2x2 unshared offsets over 32 channels on a small grid is one launch whose
+    workgroups pack their offsets rows themselves: the same bits as the prepared call (pack kernel + forward kernel),
+    with and without the logsumexp normalisation, for partial and several instance groups, and for rows too far apart
+    for the product form (which both paths then evaluate as a max-tracked log-sum-exp)."""
+    g = np.random.default_rng(31)
+    eps = 1.5
+    kw = dict(blocks=[32, 1, 1], strides=[32, 1, 1], unshared_offset_region=[2], epsilon=eps, softmax_mode=False)
+    off = (g.normal(size=(4, n, 32, 1, 1)) * 0.5).astype(np.float32)
+    if spread == "wide":
+        off *= 300
+    elif spread == "mixed":
+        off[1:3, n // 3:] *= 300
+    elif spread == "masked":
+        off[g.random(size=off.shape) < 0.2] = -math.inf
+    x = (g.normal(size=im) * 3).astype(np.float32)
+    X, OFF = dev(x), dev(off)
+    plain = pkg.mex(X, OFF, n, normalize_offsets=normalize, **kw)
+    prep = pkg.mex_prepare(im, OFF, n, normalize_offsets=normalize, **kw)(X)
+    assert same_bits(plain, prep)
+    ref_off = orc.normalize_offsets(off) if normalize else off
+    assert mex_err(plain.cpu().numpy(), x, ref_off, n, **kw) <= MEX_TOL
+    # offsets that are not 16-byte aligned take the pack kernel: still the same bits
+    flat = torch.empty(off.size + 1, device="cuda")
+    shifted = flat[1:].view(*off.shape)
+    shifted.copy_(OFF)
+    assert shifted.data_ptr() % 16 == 4
+    assert same_bits(pkg.mex(X, shifted, n, normalize_offsets=normalize, **kw), plain)
+
+
 def test_mex_prepared_config2_full(pkg):
     x, off, n, kw = config2()
     prep = pkg.mex_prepare(x.shape, dev(off), n, normalize_offsets=True, **kw)
