@@ -436,6 +436,24 @@ __device__ __forceinline__ void sim_direct_body(const SimKernelArgs &a, float *l
 // The kernel: one pass of the body; the sqrt-weight form follows it, in the (rare) workgroups with a flagged wave, by
 // the recomputing pass - MODE = SIM_MODE_L2 on the second packed copy for the flagged waves, bit-identical to
 // SIMNETS_ALGO_DIRECT - as a cold path of the same launch.
+// The recomputing pass as a function of its own, not inlined: its registers are allocated apart from the hot pass's,
+// which would otherwise spill to make room for it.  It reads the argument block from the kernel's argument segment
+// again instead of taking it from the caller (who would have to keep a copy for the call).  A callable function is not
+// given the segment's address (that value is only defined inside kernels), but it is given the address of the
+// implicit arguments, which follow the explicit ones - here the block, the kernel's only parameter - at the next
+// multiple of 8 bytes.
+#if defined(__HIP_DEVICE_COMPILE__)
+typedef __attribute__((address_space(3))) float lds_float;
+template <int PT, int MT, int SWT, bool ROW3>
+__device__ __noinline__ void sim_direct_recompute(lds_float *lds, int wave_bail)
+{
+    constexpr size_t kExplicitArgs = (sizeof(SimKernelArgs) + 7) & ~size_t(7);
+    const SimKernelArgs a = *reinterpret_cast<const SimKernelArgs *>(
+        reinterpret_cast<const char *>(__builtin_amdgcn_implicitarg_ptr()) - kExplicitArgs);
+    sim_direct_body<SIM_MODE_L2, PT, MT, SWT, true, false, ROW3>(a, (float *)lds, wave_bail);
+}
+#endif
+
 template <int MODE, int PT, int MT, int SWT, bool PLDS = false, bool ROW3 = false>
 __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_kernel(const SimKernelArgs a)
 {
@@ -443,8 +461,11 @@ __global__ __launch_bounds__(kThreads, waves_per_simd(PT, MT)) void sim_direct_k
     int wave_bail = 0;
     sim_direct_body<MODE, PT, MT, SWT, false, PLDS, ROW3>(a, lds, wave_bail);
     if constexpr (MODE == SIM_MODE_L2_SQRTW) {
-        if (__syncthreads_or(wave_bail))
-            sim_direct_body<SIM_MODE_L2, PT, MT, SWT, true, false, ROW3>(a, lds, wave_bail);
+        if (__syncthreads_or(wave_bail)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+            sim_direct_recompute<PT, MT, SWT, ROW3>((lds_float *)lds, wave_bail);
+#endif
+        }
     }
 }
 
