@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsimnets_hip.so")
+NATIVE = os.path.join(HERE, "_simnets_native.so")
 BENCH = os.path.join(HERE, "simnets_bench")
 OBJDIR = os.path.join(HERE, "build")
 
@@ -60,9 +61,30 @@ def build(extra=(), verbose=False):
     bench_src = os.path.join(HERE, "bench", "simnets_bench.hip")
     _run([HIPCC, bench_src, "-o", BENCH] + COMMON + DEVICE + extra +
          ["-L" + HERE, "-lsimnets_hip", "-Wl,-rpath,$ORIGIN"])
+    build_op_layer()
     if verbose:
-        print("built", LIB, "and", BENCH)
+        print("built", LIB, ",", NATIVE, "and", BENCH)
     return LIB
+
+
+def build_op_layer():
+    """The compiled operator layer (csrc/op_layer.cpp): host code only, built with the host compiler against torch's
+    headers and linked to libsimnets_hip.so next to it."""
+    import sysconfig
+
+    import torch
+    from torch.utils import cpp_extension as ce
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-o", NATIVE,
+           os.path.join(CSRC, "op_layer.cpp"), "-I" + os.path.join(ROOT, "include")]
+    cmd += ["-I" + p for p in ce.include_paths()] + ["-I" + sysconfig.get_paths()["include"], "-I/opt/rocm/include"]
+    cmd += ["-DUSE_ROCM=1", "-D__HIP_PLATFORM_AMD__=1", "-DHIPBLAS_V2", "-DTORCH_EXTENSION_NAME=_simnets_native",
+            "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch._C._GLIBCXX_USE_CXX11_ABI),
+            "-Wall", "-Wno-unused-function"]
+    cmd += ["-L" + tlib, "-L" + HERE, "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+            "-lsimnets_hip", "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + tlib]
+    _run(cmd)
+    return NATIVE
 
 
 if __name__ == "__main__":

@@ -1,16 +1,24 @@
 """Operator layer: the reference's Python op API (python/simnets/ops/similarity.py,
-python/simnets/ops/mex.py) over the C ABI, with torch tensors as device memory.
+python/simnets/ops/mex.py) with torch tensors as device memory.
 
 Argument names, defaults (None = the registered op default, src/ops/similarity_op.cpp:67-74 and
 src/ops/mex_op.cpp:62-73) and error conditions follow the reference; errors surface as
 SimnetsError carrying the status code and the reference's message.
+
+Every call that launches work is a thin front of the compiled operator layer (csrc/op_layer.cpp, the module
+`_simnets_native`), which checks the tensors, fills the attribute structs, allocates outputs and scratch and calls the
+C ABI of libsimnets_hip.so.  The host-only queries (shapes, dimensions, attribute structs) go to the C ABI through
+ctypes.
 """
 import ctypes as C
 
 import torch
 
 from . import _lib
+from . import _native
 from ._lib import MexAttrs, MexDims, SimilarityAttrs
+
+_n = _native.module()
 
 
 class SimnetsError(ValueError):
@@ -31,8 +39,6 @@ def _fill(dst, values, cap):
     return len(values)
 
 
-_workspaces = {}
-
 # The current stream's handle without building a torch.cuda.Stream object (a few microseconds per call, as much as
 # a small kernel runs); the public API where this build of torch lacks the direct accessor.
 _raw_stream_of = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -44,91 +50,13 @@ def _current_stream(device):
     return torch.cuda.current_stream(device).cuda_stream
 
 
-def _workspace(device, nbytes, stream=None):
-    """A scratch tensor per (device, current stream), grown on demand and reused across calls: the kernels that
-    use it are ordered on that stream, and calls on different streams never share one."""
-    # a buffer first allocated during stream capture lives in that graph's private pool: kept apart from the
-    # eager calls' buffer, which a later replay of the graph must not share
-    if stream is None:
-        stream = _current_stream(device)
-    key = (device.index, stream, torch.cuda.is_current_stream_capturing())
-    ws = _workspaces.get(key)
-    if ws is None or ws.numel() < nbytes:
-        ws = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-        _workspaces[key] = ws
-    return ws
-
-
-_plans = {}
-
-
-_PLAIN_KEY_TYPES = frozenset((int, str, bool, type(None), torch.Size))
-
-
 def _freeze(v):
+    """Hashable form of an attribute value (floats by repr: NaN out-of-bounds values must compare equal)."""
     if isinstance(v, (list, tuple)):
         return tuple(_freeze(e) for e in v)
     if isinstance(v, dict):
         return tuple(sorted((k, _freeze(e)) for k, e in v.items()))
     return repr(v) if isinstance(v, float) else v
-
-
-def _key_part(v):
-    t = type(v)
-    if t in _PLAIN_KEY_TYPES:
-        return v
-    if t is float:
-        return repr(v)
-    if t is list or t is tuple:
-        for e in v:
-            if type(e) is not int:
-                return _freeze(v)
-        return tuple(v)
-    return _freeze(v)
-
-
-def _plan_key(*parts):
-    """Hashable key of shapes and attribute values (floats by repr: NaN out-of-bounds values must compare equal).
-    Called on every op call: values of the usual plain types and lists of ints take the short way."""
-    return tuple([v if type(v) in _PLAIN_KEY_TYPES else _key_part(v) for v in parts])
-
-
-def _cached_plan(key, make):
-    """Attribute struct, shapes and workspace size of a call: the host-side queries are pure functions of the
-    shapes and attributes, and repeated calls of a layer would otherwise spend more time in them than the GPU
-    spends in a small kernel."""
-    plan = _plans.get(key)
-    if plan is None:
-        if len(_plans) >= 512:
-            _plans.clear()
-        plan = _plans[key] = make()
-    return plan
-
-
-class _NoSwitch:
-    def __enter__(self):
-        return None
-
-    def __exit__(self, *exc):
-        return False
-
-
-_NO_SWITCH = _NoSwitch()
-
-
-def _on_device(device):
-    """Context that makes `device` current for a launch; free when it already is (the usual case)."""
-    return _NO_SWITCH if torch.cuda.current_device() == device.index else torch.cuda.device(device)
-
-
-def _require_cuda_f32(name, t):
-    if not isinstance(t, torch.Tensor):
-        raise TypeError("%s must be a torch.Tensor" % name)
-    if t.dtype != torch.float32:
-        raise TypeError("%s must be float32 (the HIP path computes in fp32), got %s" % (name, t.dtype))
-    if not t.is_cuda:
-        raise RuntimeError("%s must live on a HIP device: simnets_tf_amd has no CPU fallback" % name)
-    return t.contiguous()
 
 
 def similarity_attrs(templates_shape=None, similarity_function=None, blocks=None, strides=None, padding=None,
@@ -178,63 +106,9 @@ def similarity(input, templates, weights, similarity_function=None, blocks=None,
     input [B,C,H,W], templates/weights [O,C,bh,bw] (weights non-negative) -> [B,O,oh,ow].
     Extensions: `algo` in {None,'direct','sqrtw','mfma'} (None: 'sqrtw' for plain L2, else 'direct'), `norm_const_every_iteration`, `out`.
     """
-    x = _require_cuda_f32("input", input)
-    t = _require_cuda_f32("templates", templates)
-    w = _require_cuda_f32("weights", weights)
-    if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-
-    def make():
-        a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
-                             normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-                             ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
-                             norm_const_every_iteration=norm_const_every_iteration)
-        I4 = C.c_int * 4
-        xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
-        oshape = I4()
-        _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
-        nbytes = C.c_size_t()
-        _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
-        return a, xs, ts, wsh, tuple(oshape), nbytes.value
-
-    a, xs, ts, wsh, oshape, nbytes = _cached_plan(
-        _plan_key("similarity", x.shape, t.shape, w.shape, similarity_function, blocks, strides, padding,
-                  normalization_term, normalization_term_fudge, ignore_nan_input, out_of_bounds_value, algo,
-                  norm_const_every_iteration), make)
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes, stream)
-    if out is None:
-        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
-    else:
-        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
-    with _on_device(x.device):
-        _check(l.simnets_hip_similarity_fwd(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
-                                            out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return out
-
-
-def _similarity_grad_setup(input, templates, weights, output_grad, kw):
-    x = _require_cuda_f32("input", input)
-    t = _require_cuda_f32("templates", templates)
-    w = _require_cuda_f32("weights", weights)
-    g = _require_cuda_f32("output_grad", output_grad)
-    if x.dim() != 4 or t.dim() != 4 or w.dim() != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-
-    def make():
-        a = similarity_attrs(**kw)
-        I4 = C.c_int * 4
-        xs, ts, wsh = I4(*x.shape), I4(*t.shape), I4(*w.shape)
-        oshape = I4()
-        _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
-        return a, xs, ts, wsh, tuple(oshape)
-
-    a, xs, ts, wsh, oshape = _cached_plan(_plan_key("similarity_grad", x.shape, t.shape, w.shape, *kw.values()), make)
-    if tuple(g.shape) != oshape:
-        raise SimnetsError(-15)
-    return l, a, x, t, w, g, xs, ts, wsh
+    return _n.similarity(input, templates, weights, similarity_function, blocks, strides, padding, normalization_term,
+                         normalization_term_fudge, ignore_nan_input, out_of_bounds_value, algo,
+                         bool(norm_const_every_iteration), out)
 
 
 def similarity_input_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None, strides=None,
@@ -242,19 +116,9 @@ def similarity_input_grad(input, templates, weights, output_grad, similarity_fun
                           ignore_nan_input=None, out_of_bounds_value=None, name=None, algo=None):
     """Gradient of `similarity` w.r.t. its input: the SimilarityInputGrad op
     (python/simnets/ops/similarity.py:33-37, src/ops/similarity_op.cpp:141-156)."""
-    l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
-        similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
-        normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes), None))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    dx = torch.empty_like(x)
-    with _on_device(x.device):
-        _check(l.simnets_hip_similarity_input_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(), w.data_ptr(),
-                                                   g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return dx
+    return _n.similarity_input_grad(input, templates, weights, output_grad, similarity_function, blocks, strides, padding,
+                                    normalization_term, normalization_term_fudge, ignore_nan_input, out_of_bounds_value,
+                                    algo)
 
 
 def similarity_parameters_grad(input, templates, weights, output_grad, similarity_function=None, blocks=None,
@@ -265,20 +129,9 @@ def similarity_parameters_grad(input, templates, weights, output_grad, similarit
 
     Extension: `algo='direct'` sums the reference's terms one by one; by default the L2 modes accumulate the
     moments sum g xc, sum g xc^2, sum g about a centre near the templates and combine them at the end."""
-    l, a, x, t, w, g, xs, ts, wsh = _similarity_grad_setup(input, templates, weights, output_grad, dict(
-        similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
-        normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_grad_workspace_bytes(C.byref(a), xs, ts, None, C.byref(nbytes)))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    dt, dw = torch.empty_like(t), torch.empty_like(w)
-    with _on_device(x.device):
-        _check(l.simnets_hip_similarity_params_grad(C.byref(a), xs, ts, wsh, x.data_ptr(), t.data_ptr(),
-                                                    w.data_ptr(), g.data_ptr(), dt.data_ptr(), dw.data_ptr(),
-                                                    ws.data_ptr(), ws.numel(), stream))
-    return dt, dw
+    return _n.similarity_parameters_grad(input, templates, weights, output_grad, similarity_function, blocks, strides,
+                                         padding, normalization_term, normalization_term_fudge, ignore_nan_input,
+                                         out_of_bounds_value, algo)
 
 
 def mex_attrs(num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
@@ -367,61 +220,9 @@ def mex(input, offsets, num_instances, softmax_mode=None, padding=None, strides=
     input [B,C,H,W], offsets [num_regions, num_instances, bc, bh, bw] -> [B, channels_out*num_instances, oh, ow].
     Extension: `normalize_offsets` applies the Keras layer's logsumexp normalisation on the device.
     """
-    x = _require_cuda_f32("input", input)
-    off = _require_cuda_f32("offsets", offsets)
-    if x.dim() != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-
-    def make():
-        a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
-                      epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
-                      blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
-                      shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
-                      normalize_offsets=normalize_offsets)
-        xs = (C.c_int * 4)(*x.shape)
-        oshape = (C.c_int * 4)()
-        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-        nbytes = C.c_size_t()
-        _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
-        return a, xs, tuple(oshape), nbytes.value
-
-    a, xs, oshape, nbytes = _cached_plan(
-        _plan_key("mex", x.shape, num_instances, softmax_mode, padding, strides, blocks, epsilon,
+    return _n.mex(input, offsets, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
                   blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
-                  unshared_offset_region, normalize_offsets), make)
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes, stream)
-    if out is None:
-        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
-    else:
-        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32
-    with _on_device(x.device):
-        _check(l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), out.data_ptr(),
-                                     ws.data_ptr(), ws.numel(), stream))
-    return out
-
-
-def _mex_grad_setup(input, offsets, output, output_grad, num_instances, kw):
-    x = _require_cuda_f32("input", input)
-    off = _require_cuda_f32("offsets", offsets)
-    y = _require_cuda_f32("output", output)
-    g = _require_cuda_f32("output_grad", output_grad)
-    if x.dim() != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-
-    def make():
-        a = mex_attrs(num_instances, **kw)
-        xs = (C.c_int * 4)(*x.shape)
-        oshape = (C.c_int * 4)()
-        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-        return a, xs, tuple(oshape)
-
-    a, xs, oshape = _cached_plan(_plan_key("mex_grad", x.shape, num_instances, *kw.values()), make)
-    if tuple(y.shape) != oshape or tuple(g.shape) != oshape:
-        raise SimnetsError(-15)
-    return l, a, x, off, y, g, xs
+                  unshared_offset_region, bool(normalize_offsets), out)
 
 
 def mex_input_grad(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
@@ -430,42 +231,20 @@ def mex_input_grad(input, offsets, output, output_grad, num_instances, softmax_m
                    normalize_offsets=False):
     """Gradient of `mex` w.r.t. its input: the MexInputGrad op (python/simnets/ops/mex.py:63-71,
     src/ops/mex_op.cpp:134-151).  `output` is the forward result."""
-    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
-        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
-        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
-        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
-        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, C.byref(nbytes), None))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    dx = torch.empty_like(x)
-    with _on_device(x.device):
-        _check(l.simnets_hip_mex_input_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
-                                            g.data_ptr(), dx.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return dx
+    return _n.mex_input_grad(input, offsets, output, output_grad, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
+                          blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                          unshared_offset_region, bool(normalize_offsets))
 
 
-def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None,
-                     strides=None, blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
+                     blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
                      use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
                      normalize_offsets=False):
     """Gradient of `mex` w.r.t. its offsets: the MexOffsetsGrad op (python/simnets/ops/mex.py:73-80,
     src/ops/mex_op.cpp:153-170).  With `normalize_offsets` the gradient is w.r.t. the raw offsets."""
-    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
-        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
-        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
-        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
-        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_grad_workspace_bytes(C.byref(a), xs, None, C.byref(nbytes)))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    doff = torch.empty_like(off)
-    with _on_device(x.device):
-        _check(l.simnets_hip_mex_offsets_grad(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
-                                              g.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return doff
+    return _n.mex_offsets_grad(input, offsets, output, output_grad, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
+                            blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                            unshared_offset_region, bool(normalize_offsets))
 
 
 def mex_grads(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
@@ -475,21 +254,9 @@ def mex_grads(input, offsets, output, output_grad, num_instances, softmax_mode=N
     """`(mex_input_grad(...), mex_offsets_grad(...))` as one call of the library: the same results bit for bit, with
     the work both share (offsets normalisation and packing, per-pixel factors) done once.  What the gradient
     registered for the Mex op (python/simnets/ops/mex.py:47-81) computes."""
-    l, a, x, off, y, g, xs = _mex_grad_setup(input, offsets, output, output_grad, num_instances, dict(
-        softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks, epsilon=epsilon,
-        blocks_out_of_bounds_value=blocks_out_of_bounds_value, blocks_round_down=blocks_round_down,
-        use_unshared_regions=use_unshared_regions, shared_offset_region=shared_offset_region,
-        unshared_offset_region=unshared_offset_region, normalize_offsets=normalize_offsets))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_grads_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    dx, doff = torch.empty_like(x), torch.empty_like(off)
-    with _on_device(x.device):
-        _check(l.simnets_hip_mex_grads(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(),
-                                       g.data_ptr(), dx.data_ptr(), doff.data_ptr(), ws.data_ptr(), ws.numel(),
-                                       stream))
-    return dx, doff
+    return _n.mex_grads(input, offsets, output, output_grad, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
+                     blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                     unshared_offset_region, bool(normalize_offsets))
 
 
 def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
@@ -499,40 +266,9 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
     """`sum_pooling(mex(...), pool_size)` as one call (forward only): the MEX layer + pooling pair of the reference's
     networks (README.md:108-129).  With unshared offset regions equal to the pooling window and a finite epsilon a
     single kernel writes only the pooled tensor; other geometries run the two kernels through scratch memory."""
-    x = _require_cuda_f32("input", input)
-    off = _require_cuda_f32("offsets", offsets)
-    if x.dim() != 4:
-        raise SimnetsError(-15)
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    l = _lib.lib()
-
-    def make():
-        a = mex_attrs(num_instances, softmax_mode=softmax_mode, padding=padding, strides=strides, blocks=blocks,
-                      epsilon=epsilon, blocks_out_of_bounds_value=blocks_out_of_bounds_value,
-                      blocks_round_down=blocks_round_down, use_unshared_regions=use_unshared_regions,
-                      shared_offset_region=shared_offset_region, unshared_offset_region=unshared_offset_region,
-                      normalize_offsets=normalize_offsets)
-        xs = (C.c_int * 4)(*x.shape)
-        oshape = (C.c_int * 4)()
-        _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-        nbytes = C.c_size_t()
-        _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
-        return a, xs, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), nbytes.value
-
-    a, xs, pshape, nbytes = _cached_plan(
-        _plan_key("mex_sum_pool", x.shape, num_instances, ph, pw, softmax_mode, padding, strides, blocks, epsilon,
-                  blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
-                  unshared_offset_region, normalize_offsets), make)
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes, stream)
-    if out is None:
-        out = torch.empty(pshape, dtype=torch.float32, device=x.device)
-    else:
-        assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
-    with _on_device(x.device):
-        _check(l.simnets_hip_mex_sum_pool_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), ph, pw,
-                                              out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return out
+    return _n.mex_sum_pool(input, offsets, int(num_instances), int(pool_size[0]), int(pool_size[1]), softmax_mode, padding,
+                           strides, blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions,
+                           shared_offset_region, unshared_offset_region, bool(normalize_offsets), out)
 
 
 def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, pool_size=(2, 2), similarity=None,
@@ -542,73 +278,20 @@ def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, p
     `mex` are dicts of the keyword arguments of those two functions.  One kernel when the MEX blocks are
     [templates, 1, 1], the offsets are unshared over exactly the pooling window and a Similarity patch has at most 16
     elements; the separate kernels through scratch memory otherwise."""
-    x = _require_cuda_f32("input", input)
-    t = _require_cuda_f32("templates", templates)
-    w = _require_cuda_f32("weights", weights)
-    off = _require_cuda_f32("offsets", offsets)
-    if x.dim() != 4 or t.dim() != 4 or tuple(w.shape) != tuple(t.shape):
-        raise SimnetsError(-15)
-    sa = similarity_attrs(**(similarity or {}))
-    ma = mex_attrs(num_instances, **(mex or {}))
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    l = _lib.lib()
-    I4 = C.c_int * 4
-    xs, ts = I4(*x.shape), I4(*t.shape)
-    mid, oshape = I4(), I4()
-    _check(l.simnets_similarity_out_shape(C.byref(sa), xs, ts, ts, mid))
-    _check(l.simnets_mex_out_shape(C.byref(ma), mid, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), xs, ts, C.byref(ma), ph, pw,
-                                                                 C.byref(nbytes)))
-    stream = _current_stream(x.device)
-    ws = _workspace(x.device, nbytes.value, stream)
-    pshape = (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw)
-    if out is None:
-        out = torch.empty(pshape, dtype=torch.float32, device=x.device)
-    else:
-        assert out.is_contiguous() and tuple(out.shape) == pshape and out.dtype == torch.float32
-    with _on_device(x.device):
-        _check(l.simnets_hip_similarity_mex_sum_pool_fwd(C.byref(sa), xs, ts, x.data_ptr(), t.data_ptr(), w.data_ptr(),
-                                                         C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
-                                                         out.data_ptr(), ws.data_ptr(), ws.numel(), stream))
-    return out
+    return _n.similarity_mex_sum_pool(input, templates, weights, offsets, int(num_instances), int(pool_size[0]),
+                                      int(pool_size[1]), _sim_dict(similarity), _mex_dict(mex), out)
 
 
 def sum_pooling(input, pool_size=(2, 2), out=None):
     """Non-overlapping 'valid' sum pooling: the AveragePooling2D * area glue of the reference's
     missing-data example (README.md:108-111)."""
-    x = _require_cuda_f32("input", input)
-    if x.dim() != 4:
-        raise SimnetsError(-15)
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    B, Cc, H, W = x.shape
-    oshape = (B, Cc, H // max(ph, 1), W // max(pw, 1))
-    if out is None:
-        out = torch.empty(oshape, dtype=torch.float32, device=x.device)
-    else:
-        assert out.is_contiguous() and tuple(out.shape) == oshape and out.dtype == torch.float32 \
-            and out.device == x.device
-    with _on_device(x.device):
-        stream = _current_stream(x.device)
-        _check(_lib.lib().simnets_hip_sum_pool_fwd((C.c_int * 4)(*x.shape), ph, pw, x.data_ptr(), out.data_ptr(),
-                                                   stream))
-    return out
+    return _n.sum_pooling(input, int(pool_size[0]), int(pool_size[1]), out)
 
 
 def sum_pooling_input_grad(output_grad, input_shape, pool_size=(2, 2)):
     """Gradient of `sum_pooling` w.r.t. its input: each element receives its window's gradient, elements of a
     dropped trailing row or column receive 0."""
-    g = _require_cuda_f32("output_grad", output_grad)
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    B, Cc, H, W = [int(v) for v in input_shape]
-    if tuple(g.shape) != (B, Cc, H // max(ph, 1), W // max(pw, 1)):
-        raise SimnetsError(-15)
-    dx = torch.empty((B, Cc, H, W), dtype=torch.float32, device=g.device)
-    with _on_device(g.device):
-        stream = _current_stream(g.device)
-        _check(_lib.lib().simnets_hip_sum_pool_input_grad((C.c_int * 4)(B, Cc, H, W), ph, pw, g.data_ptr(),
-                                                          dx.data_ptr(), stream))
-    return dx
+    return _n.sum_pooling_input_grad(output_grad, [int(v) for v in input_shape], int(pool_size[0]), int(pool_size[1]))
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -617,49 +300,32 @@ def sum_pooling_input_grad(output_grad, input_shape, pool_size=(2, 2)):
 # redoes its counterpart on every call (interlace, src/kernels/similarity_kernel_gpu.cu:70; offsets copy,
 # src/kernels/mex_kernel_gpu.cu:98-112).
 # ---------------------------------------------------------------------------------------------------------------
-class Prepared:
-    """A forward operator bound to packed parameters and one input shape; call it with the input.
-
-    Made by `similarity_prepare`, `mex_prepare`, `mex_sum_pool_prepare` or `similarity_mex_sum_pool_prepare`.  The
-    results are those of the plain call, bit for bit.  The buffer also serves as the per-call scratch of the kernels,
-    so calls of one object must not overlap (keep them on one stream).  Later changes of the parameter tensors are
-    not seen: prepare again.
-    """
-
-    def __init__(self, input_shape, output_shape, buffer, run):
-        self.input_shape = torch.Size(int(v) for v in input_shape)
-        self.output_shape = tuple(int(v) for v in output_shape)
-        self.buffer = buffer
-        self._run = run
-        self._device = buffer.device
-        self._index = buffer.device.index
-
-    def __call__(self, input, out=None):
-        # (kept short: for the small layers this host code, not the kernel, bounds the call rate)
-        x = input
-        if x.shape != self.input_shape or x.device != self._device or x.dtype is not torch.float32:
-            _require_cuda_f32("input", x)
-            raise SimnetsError(-15)
-        if not x.is_contiguous():
-            x = x.contiguous()
-        if out is None:
-            out = torch.empty(self.output_shape, dtype=torch.float32, device=self._device)
-        elif not (out.is_contiguous() and tuple(out.shape) == self.output_shape and out.dtype is torch.float32
-                  and out.device == self._device):
-            raise ValueError("out must be a contiguous float32 tensor of shape %s on %s"
-                             % (self.output_shape, self._device))
-        if torch.cuda.current_device() == self._index:
-            code = self._run(x.data_ptr(), out.data_ptr(), _current_stream(self._device))
-        else:
-            with torch.cuda.device(self._device):
-                code = self._run(x.data_ptr(), out.data_ptr(), _current_stream(self._device))
-        if code != 0:
-            raise SimnetsError(code)
-        return out
+Prepared = _n.Prepared
 
 
-def _prepared_buffer(device, nbytes):
-    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+_SIM_KEYS = ("similarity_function", "blocks", "strides", "padding", "normalization_term", "normalization_term_fudge",
+             "ignore_nan_input", "out_of_bounds_value", "algo", "norm_const_every_iteration")
+_MEX_KEYS = ("softmax_mode", "padding", "strides", "blocks", "epsilon", "blocks_out_of_bounds_value",
+             "blocks_round_down", "use_unshared_regions", "shared_offset_region", "unshared_offset_region",
+             "normalize_offsets")
+
+
+def _sim_dict(attrs):
+    attrs = dict(attrs or {})
+    attrs.pop("name", None)
+    unknown = set(attrs) - set(_SIM_KEYS)
+    if unknown:
+        raise TypeError("unknown Similarity attributes: %s" % sorted(unknown))
+    return attrs
+
+
+def _mex_dict(attrs):
+    attrs = dict(attrs or {})
+    attrs.pop("name", None)
+    unknown = set(attrs) - set(_MEX_KEYS)
+    if unknown:
+        raise TypeError("unknown Mex attributes: %s" % sorted(unknown))
+    return attrs
 
 
 def similarity_prepare(input_shape, templates, weights, similarity_function=None, blocks=None, strides=None,
@@ -667,115 +333,31 @@ def similarity_prepare(input_shape, templates, weights, similarity_function=None
                        out_of_bounds_value=None, algo=None, norm_const_every_iteration=False):
     """`similarity(input, templates, weights, ...)` with the parameter packing done here, once: returns a `Prepared`
     whose call takes the input (of exactly `input_shape`, batch size included) and runs only the forward kernels."""
-    t = _require_cuda_f32("templates", templates)
-    w = _require_cuda_f32("weights", weights)
-    if len(input_shape) != 4 or t.dim() != 4 or w.dim() != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-    a = similarity_attrs(similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
-                         normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
-                         ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
-                         norm_const_every_iteration=norm_const_every_iteration)
-    I4 = C.c_int * 4
-    xs, ts, wsh = I4(*[int(v) for v in input_shape]), I4(*t.shape), I4(*w.shape)
-    oshape = I4()
-    _check(l.simnets_similarity_out_shape(C.byref(a), xs, ts, wsh, oshape))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_workspace_bytes(C.byref(a), xs, ts, C.byref(nbytes)))
-    buf = _prepared_buffer(t.device, nbytes.value)
-    with _on_device(t.device):
-        stream = _current_stream(t.device)
-        _check(l.simnets_hip_similarity_prepare(C.byref(a), xs, ts, wsh, t.data_ptr(), w.data_ptr(), buf.data_ptr(),
-                                                buf.numel(), stream))
-
-    fn, ar, bp, bn = l.simnets_hip_similarity_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
-
-    def run(x_ptr, out_ptr, stream):
-        return fn(ar, xs, ts, x_ptr, bp, bn, out_ptr, stream)
-    return Prepared(input_shape, tuple(oshape), buf, run)
+    return _n.similarity_prepare([int(v) for v in input_shape], templates, weights, dict(
+        similarity_function=similarity_function, blocks=blocks, strides=strides, padding=padding,
+        normalization_term=normalization_term, normalization_term_fudge=normalization_term_fudge,
+        ignore_nan_input=ignore_nan_input, out_of_bounds_value=out_of_bounds_value, algo=algo,
+        norm_const_every_iteration=norm_const_every_iteration))
 
 
 def mex_prepare(input_shape, offsets, num_instances, normalize_offsets=False, **attrs):
     """`mex(input, offsets, num_instances, ...)` with the offsets packed here, once (keyword arguments as `mex`)."""
-    off = _require_cuda_f32("offsets", offsets)
-    if len(input_shape) != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-    a = mex_attrs(num_instances, normalize_offsets=normalize_offsets, **attrs)
-    xs = (C.c_int * 4)(*[int(v) for v in input_shape])
-    oshape = (C.c_int * 4)()
-    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)))
-    buf = _prepared_buffer(off.device, nbytes.value)
-    with _on_device(off.device):
-        stream = _current_stream(off.device)
-        _check(l.simnets_hip_mex_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), buf.data_ptr(), buf.numel(),
-                                         stream))
-
-    fn, ar, bp, bn = l.simnets_hip_mex_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
-
-    def run(x_ptr, out_ptr, stream):
-        return fn(ar, xs, x_ptr, bp, bn, out_ptr, stream)
-    return Prepared(input_shape, tuple(oshape), buf, run)
+    return _n.mex_prepare([int(v) for v in input_shape], offsets, int(num_instances),
+                          _mex_dict(dict(attrs, normalize_offsets=normalize_offsets)))
 
 
 def mex_sum_pool_prepare(input_shape, offsets, num_instances, pool_size=(2, 2), normalize_offsets=False, **attrs):
     """`mex_sum_pool(input, offsets, num_instances, pool_size, ...)` with the offsets packed here, once."""
-    off = _require_cuda_f32("offsets", offsets)
-    if len(input_shape) != 4:
-        raise SimnetsError(-15)
-    l = _lib.lib()
-    a = mex_attrs(num_instances, normalize_offsets=normalize_offsets, **attrs)
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    xs = (C.c_int * 4)(*[int(v) for v in input_shape])
-    oshape = (C.c_int * 4)()
-    _check(l.simnets_mex_out_shape(C.byref(a), xs, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, ph, pw, C.byref(nbytes)))
-    buf = _prepared_buffer(off.device, nbytes.value)
-    with _on_device(off.device):
-        stream = _current_stream(off.device)
-        _check(l.simnets_hip_mex_sum_pool_prepare(C.byref(a), xs, off.data_ptr(), off.numel(), ph, pw, buf.data_ptr(),
-                                                  buf.numel(), stream))
-
-    fn, ar, bp, bn = l.simnets_hip_mex_sum_pool_fwd_prepared, C.byref(a), buf.data_ptr(), buf.numel()
-
-    def run(x_ptr, out_ptr, stream):
-        return fn(ar, xs, x_ptr, ph, pw, bp, bn, out_ptr, stream)
-    return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
+    return _n.mex_sum_pool_prepare([int(v) for v in input_shape], offsets, int(num_instances), int(pool_size[0]),
+                                   int(pool_size[1]), _mex_dict(dict(attrs, normalize_offsets=normalize_offsets)))
 
 
 def similarity_mex_sum_pool_prepare(input_shape, templates, weights, offsets, num_instances, pool_size=(2, 2),
                                     similarity=None, mex=None):
     """`similarity_mex_sum_pool(input, templates, weights, offsets, ...)` with all parameters packed here, once."""
-    t = _require_cuda_f32("templates", templates)
-    w = _require_cuda_f32("weights", weights)
-    off = _require_cuda_f32("offsets", offsets)
-    if len(input_shape) != 4 or t.dim() != 4 or tuple(w.shape) != tuple(t.shape):
-        raise SimnetsError(-15)
-    sa = similarity_attrs(**(similarity or {}))
-    ma = mex_attrs(num_instances, **(mex or {}))
-    ph, pw = int(pool_size[0]), int(pool_size[1])
-    l = _lib.lib()
-    I4 = C.c_int * 4
-    xs, ts = I4(*[int(v) for v in input_shape]), I4(*t.shape)
-    mid, oshape = I4(), I4()
-    _check(l.simnets_similarity_out_shape(C.byref(sa), xs, ts, ts, mid))
-    _check(l.simnets_mex_out_shape(C.byref(ma), mid, C.byref(oshape), None))
-    nbytes = C.c_size_t()
-    _check(l.simnets_hip_similarity_mex_sum_pool_workspace_bytes(C.byref(sa), xs, ts, C.byref(ma), ph, pw,
-                                                                 C.byref(nbytes)))
-    buf = _prepared_buffer(t.device, nbytes.value)
-    with _on_device(t.device):
-        stream = _current_stream(t.device)
-        _check(l.simnets_hip_similarity_mex_sum_pool_prepare(C.byref(sa), xs, ts, t.data_ptr(), w.data_ptr(),
-                                                             C.byref(ma), off.data_ptr(), off.numel(), ph, pw,
-                                                             buf.data_ptr(), buf.numel(), stream))
+    return _n.similarity_mex_sum_pool_prepare([int(v) for v in input_shape], templates, weights, offsets,
+                                              int(num_instances), int(pool_size[0]), int(pool_size[1]),
+                                              _sim_dict(similarity), _mex_dict(mex))
 
-    fn, sr, mr, bp, bn = (l.simnets_hip_similarity_mex_sum_pool_fwd_prepared, C.byref(sa), C.byref(ma), buf.data_ptr(),
-                          buf.numel())
 
-    def run(x_ptr, out_ptr, stream):
-        return fn(sr, xs, ts, x_ptr, mr, ph, pw, bp, bn, out_ptr, stream)
-    return Prepared(input_shape, (oshape[0], oshape[1], oshape[2] // ph, oshape[3] // pw), buf, run)
+_n.set_error_class(SimnetsError)

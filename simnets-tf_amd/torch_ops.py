@@ -1,17 +1,15 @@
-"""`torch.library` registration of the operators: `torch.ops.simnets.similarity`, `torch.ops.simnets.mex` and
-their gradient ops, the counterpart of the reference's REGISTER_OP / @RegisterGradient pairs
-(src/ops/similarity_op.cpp:61-174, src/ops/mex_op.cpp:58-170, python/simnets/ops/similarity.py:18-45,
-python/simnets/ops/mex.py:47-81).  With fake (meta) implementations for shape inference, so that graphs
-containing the ops can be traced by torch.compile / torch.export; the real implementations call the C ABI
-through ops.py and exist for HIP devices only.
-"""
-from typing import List, Tuple
+"""`torch.ops.simnets.similarity`, `torch.ops.simnets.mex` and their gradient ops: the counterpart of the reference's
+REGISTER_OP / @RegisterGradient pairs (src/ops/similarity_op.cpp:61-174, src/ops/mex_op.cpp:58-170,
+python/simnets/ops/similarity.py:18-45, python/simnets/ops/mex.py:47-81).
 
+The operators and their HIP implementations are registered by the compiled operator layer (TORCH_LIBRARY in
+csrc/op_layer.cpp, loaded through ops.py).  This module attaches what a graph tracer and autograd need on top of
+that: fake (meta) implementations for shape inference, so that graphs containing the ops can be traced by
+torch.compile / torch.export, and the autograd formulas, which call the gradient operators.
+"""
 import torch
 
-from . import ops
-
-_lib_defined = False
+from . import ops  # noqa: F401  (loads the compiled layer, which defines the operators)
 
 
 def _sim_kw(similarity_function, blocks, strides, padding, normalization_term, normalization_term_fudge,
@@ -31,16 +29,7 @@ def _mex_kw(softmax_mode, padding, strides, blocks, epsilon, blocks_out_of_bound
                 normalize_offsets=normalize_offsets)
 
 
-@torch.library.custom_op("simnets::similarity", mutates_args=(), device_types="cuda")
-def similarity(input: torch.Tensor, templates: torch.Tensor, weights: torch.Tensor, similarity_function: str,
-               blocks: List[int], strides: List[int], padding: List[int], normalization_term: bool,
-               normalization_term_fudge: float, ignore_nan_input: bool, out_of_bounds_value: float) -> torch.Tensor:
-    return ops.similarity(input, templates, weights, **_sim_kw(similarity_function, blocks, strides, padding,
-                                                               normalization_term, normalization_term_fudge,
-                                                               ignore_nan_input, out_of_bounds_value))
-
-
-@similarity.register_fake
+@torch.library.register_fake("simnets::similarity")
 def _(input, templates, weights, similarity_function, blocks, strides, padding, normalization_term,
       normalization_term_fudge, ignore_nan_input, out_of_bounds_value):
     shape = ops.similarity_output_shape(tuple(input.shape), tuple(templates.shape), tuple(weights.shape),
@@ -49,33 +38,12 @@ def _(input, templates, weights, similarity_function, blocks, strides, padding, 
     return input.new_empty(shape)
 
 
-@torch.library.custom_op("simnets::similarity_input_grad", mutates_args=(), device_types="cuda")
-def similarity_input_grad(input: torch.Tensor, templates: torch.Tensor, weights: torch.Tensor,
-                          output_grad: torch.Tensor, similarity_function: str, blocks: List[int], strides: List[int],
-                          padding: List[int], normalization_term: bool, normalization_term_fudge: float,
-                          ignore_nan_input: bool, out_of_bounds_value: float) -> torch.Tensor:
-    return ops.similarity_input_grad(input, templates, weights, output_grad.contiguous(),
-                                     **_sim_kw(similarity_function, blocks, strides, padding, normalization_term,
-                                               normalization_term_fudge, ignore_nan_input, out_of_bounds_value))
-
-
-@similarity_input_grad.register_fake
+@torch.library.register_fake("simnets::similarity_input_grad")
 def _(input, templates, weights, output_grad, *attrs):
     return torch.empty_like(input)
 
 
-@torch.library.custom_op("simnets::similarity_parameters_grad", mutates_args=(), device_types="cuda")
-def similarity_parameters_grad(input: torch.Tensor, templates: torch.Tensor, weights: torch.Tensor,
-                               output_grad: torch.Tensor, similarity_function: str, blocks: List[int],
-                               strides: List[int], padding: List[int], normalization_term: bool,
-                               normalization_term_fudge: float, ignore_nan_input: bool,
-                               out_of_bounds_value: float) -> Tuple[torch.Tensor, torch.Tensor]:
-    return ops.similarity_parameters_grad(input, templates, weights, output_grad.contiguous(),
-                                          **_sim_kw(similarity_function, blocks, strides, padding, normalization_term,
-                                                    normalization_term_fudge, ignore_nan_input, out_of_bounds_value))
-
-
-@similarity_parameters_grad.register_fake
+@torch.library.register_fake("simnets::similarity_parameters_grad")
 def _(input, templates, weights, output_grad, *attrs):
     return torch.empty_like(templates), torch.empty_like(weights)
 
@@ -89,27 +57,16 @@ def _similarity_backward(ctx, grad):
     input, templates, weights = ctx.saved_tensors
     gi = gt = gw = None
     if ctx.needs_input_grad[0]:
-        gi = similarity_input_grad(input, templates, weights, grad, *ctx.attrs)
+        gi = torch.ops.simnets.similarity_input_grad(input, templates, weights, grad.contiguous(), *ctx.attrs)
     if ctx.needs_input_grad[1] or ctx.needs_input_grad[2]:
-        gt, gw = similarity_parameters_grad(input, templates, weights, grad, *ctx.attrs)
+        gt, gw = torch.ops.simnets.similarity_parameters_grad(input, templates, weights, grad.contiguous(), *ctx.attrs)
     return (gi, gt, gw) + (None,) * len(ctx.attrs)
 
 
-similarity.register_autograd(_similarity_backward, setup_context=_similarity_setup)
+torch.library.register_autograd("simnets::similarity", _similarity_backward, setup_context=_similarity_setup)
 
 
-@torch.library.custom_op("simnets::mex", mutates_args=(), device_types="cuda")
-def mex(input: torch.Tensor, offsets: torch.Tensor, num_instances: int, softmax_mode: bool, padding: List[int],
-        strides: List[int], blocks: List[int], epsilon: float, blocks_out_of_bounds_value: float,
-        blocks_round_down: bool, use_unshared_regions: bool, shared_offset_region: List[int],
-        unshared_offset_region: List[int], normalize_offsets: bool) -> torch.Tensor:
-    return ops.mex(input, offsets, num_instances,
-                   **_mex_kw(softmax_mode, padding, strides, blocks, epsilon, blocks_out_of_bounds_value,
-                             blocks_round_down, use_unshared_regions, shared_offset_region, unshared_offset_region,
-                             normalize_offsets))
-
-
-@mex.register_fake
+@torch.library.register_fake("simnets::mex")
 def _(input, offsets, num_instances, softmax_mode, padding, strides, blocks, epsilon, blocks_out_of_bounds_value,
       blocks_round_down, use_unshared_regions, shared_offset_region, unshared_offset_region, normalize_offsets):
     shape, _ = ops.mex_output_shape(tuple(input.shape), num_instances,
@@ -119,36 +76,12 @@ def _(input, offsets, num_instances, softmax_mode, padding, strides, blocks, eps
     return input.new_empty(shape)
 
 
-@torch.library.custom_op("simnets::mex_input_grad", mutates_args=(), device_types="cuda")
-def mex_input_grad(input: torch.Tensor, offsets: torch.Tensor, orig_output: torch.Tensor, output_grad: torch.Tensor,
-                   num_instances: int, softmax_mode: bool, padding: List[int], strides: List[int], blocks: List[int],
-                   epsilon: float, blocks_out_of_bounds_value: float, blocks_round_down: bool,
-                   use_unshared_regions: bool, shared_offset_region: List[int], unshared_offset_region: List[int],
-                   normalize_offsets: bool) -> torch.Tensor:
-    return ops.mex_input_grad(input, offsets, orig_output, output_grad.contiguous(), num_instances,
-                              **_mex_kw(softmax_mode, padding, strides, blocks, epsilon, blocks_out_of_bounds_value,
-                                        blocks_round_down, use_unshared_regions, shared_offset_region,
-                                        unshared_offset_region, normalize_offsets))
-
-
-@mex_input_grad.register_fake
+@torch.library.register_fake("simnets::mex_input_grad")
 def _(input, offsets, orig_output, output_grad, *attrs):
     return torch.empty_like(input)
 
 
-@torch.library.custom_op("simnets::mex_offsets_grad", mutates_args=(), device_types="cuda")
-def mex_offsets_grad(input: torch.Tensor, offsets: torch.Tensor, orig_output: torch.Tensor, output_grad: torch.Tensor,
-                     num_instances: int, softmax_mode: bool, padding: List[int], strides: List[int],
-                     blocks: List[int], epsilon: float, blocks_out_of_bounds_value: float, blocks_round_down: bool,
-                     use_unshared_regions: bool, shared_offset_region: List[int], unshared_offset_region: List[int],
-                     normalize_offsets: bool) -> torch.Tensor:
-    return ops.mex_offsets_grad(input, offsets, orig_output, output_grad.contiguous(), num_instances,
-                                **_mex_kw(softmax_mode, padding, strides, blocks, epsilon, blocks_out_of_bounds_value,
-                                          blocks_round_down, use_unshared_regions, shared_offset_region,
-                                          unshared_offset_region, normalize_offsets))
-
-
-@mex_offsets_grad.register_fake
+@torch.library.register_fake("simnets::mex_offsets_grad")
 def _(input, offsets, orig_output, output_grad, *attrs):
     return torch.empty_like(offsets)
 
@@ -162,10 +95,10 @@ def _mex_backward(ctx, grad):
     input, offsets, out = ctx.saved_tensors
     gi = go = None
     if ctx.needs_input_grad[0]:
-        gi = mex_input_grad(input, offsets, out, grad, *ctx.attrs)
+        gi = torch.ops.simnets.mex_input_grad(input, offsets, out, grad.contiguous(), *ctx.attrs)
     if ctx.needs_input_grad[1]:
-        go = mex_offsets_grad(input, offsets, out, grad, *ctx.attrs)
+        go = torch.ops.simnets.mex_offsets_grad(input, offsets, out, grad.contiguous(), *ctx.attrs)
     return (gi, go) + (None,) * len(ctx.attrs)
 
 
-mex.register_autograd(_mex_backward, setup_context=_mex_setup)
+torch.library.register_autograd("simnets::mex", _mex_backward, setup_context=_mex_setup)
