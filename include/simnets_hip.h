@@ -315,12 +315,21 @@ int simnets_hip_sum_pool_input_grad(const int input_shape[4], int pool_h, int po
  * unshared with regions [1, pool_h, pool_w] (a pooling window is then one pixel of every region), epsilon is finite
  * and the window has 2 or 4 pixels, one kernel computes the MEX values of a window in one lane, adds them in the
  * window's row-major order and writes only the pooled tensor; any other geometry runs the two kernels through
- * scratch memory.  No gradient entry point takes the pooled tensor: training keeps the two separate calls. */
+ * scratch memory.  No gradient entry point takes the pooled tensor alone: training uses the _both form below. */
 int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
                                              int pool_w, size_t *bytes);
 int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                                  const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
                                  void *workspace, size_t workspace_bytes, void *stream);
+
+/* The same call for training: it also stores the MEX output before pooling (mex_output, the shape
+ * simnets_mex_out_shape gives), which MexInputGrad / MexOffsetsGrad take as their `output` argument
+ * (src/ops/mex_op.cpp:134-170), so that a training step keeps the fused kernel and runs no pooling launch.  Both
+ * tensors hold the values of the two separate calls. */
+int simnets_hip_mex_sum_pool_fwd_both(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                      const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                      float *mex_output, float *output, void *workspace, size_t workspace_bytes,
+                                      void *stream);
 
 /* ... in two halves, like simnets_hip_mex_prepare / simnets_hip_mex_fwd_prepared: the buffer has
  * simnets_hip_mex_sum_pool_workspace_bytes bytes; when the geometry runs the two kernels through scratch memory the

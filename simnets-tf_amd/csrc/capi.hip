@@ -371,7 +371,8 @@ int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, con
 
 static int mex_sum_pool_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                               const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
-                              void *workspace, size_t workspace_bytes, void *stream, int phase)
+                              void *workspace, size_t workspace_bytes, void *stream, int phase,
+                              float *mex_output = nullptr)
 {
     MexPlan p;
     const int rc = mex_make_plan(attrs, input_shape, &p);
@@ -388,7 +389,19 @@ static int mex_sum_pool_phase(const simnets_mex_attrs *attrs, const int input_sh
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_pool_workspace_bytes(p, pool_h, pool_w)))
         return SIMNETS_ERR_WORKSPACE;
-    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream, phase);
+    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream, phase,
+                           mex_output);
+}
+
+int simnets_hip_mex_sum_pool_fwd_both(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                      const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                      float *mex_output, float *output, void *workspace, size_t workspace_bytes,
+                                      void *stream)
+{
+    if (!mex_output && input_shape[0] != 0)
+        return SIMNETS_ERR_NULL_POINTER;
+    return mex_sum_pool_phase(attrs, input_shape, input, offsets, offsets_count, pool_h, pool_w, output, workspace,
+                              workspace_bytes, stream, kMexWhole, mex_output);
 }
 
 int simnets_hip_mex_sum_pool_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,

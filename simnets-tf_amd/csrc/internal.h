@@ -88,8 +88,10 @@ int sum_pool_grad_launch(int B, int C, int H, int W, int ph, int pw, const float
 // MEX followed by non-overlapping sum pooling: one fused kernel when a pooling window is one pixel of every
 // offsets region, else MEX into scratch + pooling
 size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw);
+// `full` (optional): the launch also stores the MEX output before pooling there (what the gradient operators read)
 int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
-                    void *workspace, size_t workspace_bytes, void *stream, int phase = kMexWhole);
+                    void *workspace, size_t workspace_bytes, void *stream, int phase = kMexWhole,
+                    float *full = nullptr);
 // Similarity, then MEX over its output, then sum pooling; `mp` is the MEX plan for the Similarity output's shape.
 // One kernel when the MEX patch of a pixel is exactly the Similarity channels of that pixel (and the MEX + pooling
 // pair is fusable), else the separate kernels through scratch memory.

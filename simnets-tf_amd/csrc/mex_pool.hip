@@ -34,6 +34,7 @@ constexpr int kSimTaps = 16;       // longest Similarity patch the kernel evalua
 
 struct PoolArgs {
     float *pooled;
+    float *full;  // not null: the MEX values before pooling are stored there as well, [B][M * Co][Ho][Wo]
     int Hp, Wp;   // pooled height and width
     int spw;      // slots per workgroup: NH * 64 / R
     // SIMF: the MEX input is the output of a Similarity layer that is evaluated on the fly
@@ -415,6 +416,21 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
             }
     }
 
+    if (q.full != nullptr) {
+        // the MEX output itself, for the gradient operators: tile t = (slot group t / R, region t % R)
+        const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const PixelRef cp = locate(a, t % R, (chunk * NH + wh) * (16 * G) + (t / R) * 16 + lr);
+            if (cp.out_off < 0)
+                continue;
+            float *o = q.full + (size_t)cp.b * a.M * plane + cp.out_off + (size_t)(m0 + 4 * lq) * plane;
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (all_rows || m0 + 4 * lq + v < a.M)
+                    o[v * plane] = res[t][v];
+        }
+    }
     // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
 #pragma unroll
     for (int g = 0; g < G; ++g) {
@@ -517,6 +533,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
     // per slot: where instance 0 goes in the pooled tensor (POOL = false: where the window's first pixel goes in the
     // MEX output), -1 = no window
     __shared__ long long ppos[16 * NH];
+    __shared__ long long fpos[16 * NH];   // POOL with q.full: where the window's first pixel goes in the unpooled output
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -581,18 +598,17 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
 
     if (tid < 16 * NH) {
         const int slot = chunk * (16 * NH) + tid;
-        long long pos = -1;
+        long long pos = -1, fp = -1;
         if (slot < a.slots) {
             const int b = (int)fast_div((unsigned)slot, a.dRS);
             const int sq = slot - b * a.RS;
             const int qw = (int)fast_div((unsigned)sq, a.dWs);
             const int i = sq - qw * a.Ws;
-            if (POOL)
-                pos = (long long)b * a.M * ((long long)q.Hp * q.Wp) + (long long)qw * q.Wp + i;
-            else
-                pos = (long long)b * a.M * g.HW + ((long long)(2 * qw) << g.lgW) + 2 * i;
+            fp = (long long)b * a.M * g.HW + ((long long)(2 * qw) << g.lgW) + 2 * i;
+            pos = POOL ? (long long)b * a.M * ((long long)q.Hp * q.Wp) + (long long)qw * q.Wp + i : fp;
         }
         ppos[tid] = pos;
+        fpos[tid] = fp;
     }
 
     // columns of the four pixels: tile (column half, region) x slot inside the half
@@ -837,6 +853,16 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
             if (all_rows || m0 + 4 * lq + v < a.M)
                 o[v * plane_p] = w;
         }
+        if (q.full != nullptr) {
+            // ... and the MEX values themselves, for the gradient operators (region t = pixel (t / 2, t % 2))
+            float *f = q.full + fpos[wh * 16 + lr] + (size_t)(m0 + 4 * lq) * g.HW;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (all_rows || m0 + 4 * lq + v < a.M)
+                        f[(size_t)v * g.HW + ((size_t)(t >> 1) << g.lgW) + (t & 1)] = res[t][v];
+        }
     } else {
         // region t is pixel (t / 2, t % 2) of the window
 #pragma unroll
@@ -954,13 +980,14 @@ size_t sim_packed_bytes(const SimPlan &sp) { return align_up((size_t)((sp.O + 31
 
 int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
                 void *workspace, const SimPlan *sp, const float *templates, const float *weights, void *stream,
-                int phase)
+                int phase, float *full = nullptr)
 {
     const simnets_mex_dims &d = p.d;
     const int n_mgroups = (d.M + TM - 1) / TM;
     MexKernelArgs a = mex_kernel_args(p);
     PoolArgs q;
     q.sx = nullptr;
+    q.full = full;
     SimPackJob job;
     if (sp) {
         float *pa = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_packed_bytes(p, TM, n_mgroups));
@@ -1033,6 +1060,7 @@ int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *inpu
         return SIMNETS_PANEL_NOT_TAKEN;
     PoolArgs q;
     q.sx = nullptr;
+    q.full = nullptr;
     q.pooled = output;
     q.Hp = p.d.height_out / 2;
     q.Wp = p.d.width_out / 2;
@@ -1060,6 +1088,7 @@ int mex_panel_launch_selfpack(const MexPlan &p, const MexKernelArgs &a, const fl
     g.normalize = p.normalize_offsets;
     PoolArgs q;
     q.sx = nullptr;
+    q.full = nullptr;
     q.pooled = output;
     q.Hp = p.d.height_out / 2;
     q.Wp = p.d.width_out / 2;
@@ -1085,19 +1114,21 @@ size_t mex_pool_workspace_bytes(const MexPlan &p, int ph, int pw)
 }
 
 int mex_pool_launch(const MexPlan &p, int ph, int pw, const float *input, const float *offsets, float *pooled,
-                    void *workspace, size_t workspace_bytes, void *stream, int phase)
+                    void *workspace, size_t workspace_bytes, void *stream, int phase, float *full_out)
 {
     const simnets_mex_dims &d = p.d;
     if (workspace_bytes < mex_pool_workspace_bytes(p, ph, pw))
         return SIMNETS_ERR_WORKSPACE;
     if (!fusable(p, ph, pw)) {
-        float *full = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_workspace_bytes(p));
+        // the caller's tensor for the MEX output if it wants one, else scratch
+        float *full = full_out ? full_out
+                               : reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_workspace_bytes(p));
         const int rc = mex_launch(p, input, offsets, full, workspace, mex_workspace_bytes(p), stream, phase);
         if (rc || !(phase & kMexRun))
             return rc;
         return sum_pool_launch(p.B, d.M * d.channels_out, d.height_out, d.width_out, ph, pw, full, pooled, stream);
     }
-    return pool_launch(p, ph, pw, input, offsets, pooled, workspace, nullptr, nullptr, nullptr, stream, phase);
+    return pool_launch(p, ph, pw, input, offsets, pooled, workspace, nullptr, nullptr, nullptr, stream, phase, full_out);
 }
 
 // Similarity -> MEX -> sum pooling.  `mp` is the MEX plan over the Similarity output's shape.

@@ -396,6 +396,25 @@ at::Tensor mex_sum_pool_call(const simnets_mex_attrs &a, const at::Tensor &input
     return y;
 }
 
+// ... for training: (MEX output before pooling, pooled output) from the one call
+std::tuple<at::Tensor, at::Tensor> mex_sum_pool_both_call(const simnets_mex_attrs &a, const at::Tensor &input,
+                                                          const at::Tensor &offsets, int ph, int pw)
+{
+    const at::Tensor x = dense("input", input), off = dense("offsets", offsets);
+    const Shape4 xs = shape4(x);
+    int os[4];
+    check(simnets_mex_out_shape(&a, xs.v, os, nullptr));
+    size_t nbytes = 0;
+    check(simnets_hip_mex_sum_pool_workspace_bytes(&a, xs.v, ph, pw, &nbytes));
+    const int ps[4] = {os[0], os[1], os[2] / ph, os[3] / pw};
+    at::Tensor full = output_like(x, os, c10::nullopt), y = output_like(x, ps, c10::nullopt);
+    Launch l(x);
+    const auto wsp = l.workspace(nbytes, x);
+    check(simnets_hip_mex_sum_pool_fwd_both(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ph, pw, ptr(full), ptr(y),
+                                            wsp.first, wsp.second, l.stream));
+    return {full, y};
+}
+
 at::Tensor similarity_mex_sum_pool_call(const simnets_similarity_attrs &sa, const simnets_mex_attrs &ma,
                                         const at::Tensor &input, const at::Tensor &templates, const at::Tensor &weights,
                                         const at::Tensor &offsets, int ph, int pw, const c10::optional<at::Tensor> &out)
@@ -743,6 +762,14 @@ PYBIND11_MODULE(_simnets_native, m)
               return mex_sum_pool_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down, unshared,
                                                     shared_region, unshared_region, normalize),
                                        x, off, ph, pw, out);
+          });
+    m.def("mex_sum_pool_both",
+          [](const at::Tensor &x, const at::Tensor &off, int n, int ph, int pw, py::object softmax, py::object padding,
+             py::object strides, py::object blocks, py::object epsilon, py::object oob, py::object round_down,
+             py::object unshared, py::object shared_region, py::object unshared_region, bool normalize) {
+              return mex_sum_pool_both_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down,
+                                                         unshared, shared_region, unshared_region, normalize),
+                                            x, off, ph, pw);
           });
     // the attribute structs of the two-operator calls come from Python as dicts of keyword arguments
     auto sim_from_dict = [](const py::dict &d) {

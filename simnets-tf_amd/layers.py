@@ -64,6 +64,31 @@ class MexFunction(torch.autograd.Function):
         return gi, go, None, None
 
 
+class MexSumPoolFunction(torch.autograd.Function):
+    """`mex` followed by non-overlapping sum pooling as one forward call that also keeps the MEX output before pooling
+    (`ops.mex_sum_pool_both`): what the MEX gradient operators take."""
+
+    @staticmethod
+    def forward(ctx, input, offsets, num_instances, ph, pw, attrs):
+        ctx.attrs, ctx.num_instances, ctx.pool = attrs, num_instances, (ph, pw)
+        full, pooled = ops.mex_sum_pool_both(input, offsets, num_instances, (ph, pw), **attrs)
+        ctx.save_for_backward(input, offsets, full)
+        return pooled
+
+    @staticmethod
+    def backward(ctx, grad):
+        input, offsets, full = ctx.saved_tensors
+        g = ops.sum_pooling_input_grad(grad.contiguous(), full.shape, ctx.pool)
+        gi = go = None
+        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
+            gi, go = ops.mex_grads(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
+        elif ctx.needs_input_grad[0]:
+            gi = ops.mex_input_grad(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
+        elif ctx.needs_input_grad[1]:
+            go = ops.mex_offsets_grad(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
+        return gi, go, None, None, None, None
+
+
 class SumPoolFunction(torch.autograd.Function):
     """Non-overlapping 'valid' sum pooling (`ops.sum_pooling`) with its gradient."""
 
@@ -100,16 +125,15 @@ def mex(input, offsets, num_instances, **attrs):
 
 def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), **attrs):
     """`mex` followed by non-overlapping sum pooling (the MEX layer + pooling pair of the reference's networks,
-    README.md:108-129).  Without gradients the pair is one call of the library (a fused kernel when the offsets are
-    unshared over exactly the pooling window); when a gradient is needed the two steps stay separate, because the
-    MEX gradients take the unpooled output."""
+    README.md:108-129), one call of the library either way (a fused kernel when the offsets are unshared over exactly
+    the pooling window).  When a gradient is needed the call also stores the MEX output before pooling, which the MEX
+    gradient operators take."""
     unknown = set(attrs) - set(_MEX_KEYS)
     if unknown:
         raise TypeError("unknown Mex attributes: %s" % sorted(unknown))
     ph, pw = int(pool_size[0]), int(pool_size[1])
     if torch.is_grad_enabled() and (input.requires_grad or offsets.requires_grad):
-        y = MexFunction.apply(input, offsets, num_instances, attrs)
-        return SumPoolFunction.apply(y, ph, pw)
+        return MexSumPoolFunction.apply(input, offsets, num_instances, ph, pw, attrs)
     return ops.mex_sum_pool(input, offsets, num_instances, (ph, pw), **attrs)
 
 

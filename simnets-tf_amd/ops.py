@@ -271,6 +271,18 @@ def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=N
                            shared_offset_region, unshared_offset_region, bool(normalize_offsets), out)
 
 
+def mex_sum_pool_both(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
+                      blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+                      use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+                      normalize_offsets=False):
+    """`(mex(...), sum_pooling(mex(...), pool_size))` from the one call `mex_sum_pool` makes: the form a training step
+    uses, since the MEX gradient operators take the output before pooling (src/ops/mex_op.cpp:134-170)."""
+    return _n.mex_sum_pool_both(input, offsets, int(num_instances), int(pool_size[0]), int(pool_size[1]), softmax_mode,
+                                padding, strides, blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down,
+                                use_unshared_regions, shared_offset_region, unshared_offset_region,
+                                bool(normalize_offsets))
+
+
 def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, pool_size=(2, 2), similarity=None,
                             mex=None, out=None):
     """`sum_pooling(mex(similarity(input, templates, weights, **similarity), offsets, num_instances, **mex), pool_size)`

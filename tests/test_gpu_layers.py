@@ -201,6 +201,47 @@ def test_mex_sum_pool_functional_fused_without_gradients_split_with(pkg):
     assert torch.allclose(off.grad, want, rtol=1e-5, atol=1e-6)
 
 
+@pytest.mark.parametrize("case", [
+    dict(im=(9, 32, 16, 16), n=64, pool=(2, 2)),                        # fused kernel (first MEX layer of the stack)
+    dict(im=(7, 64, 8, 8), n=70, pool=(2, 2)),                          # panel form, a partial instance group
+    dict(im=(5, 256, 2, 2), n=130, pool=(2, 2)),                        # panel form, one window per image
+    dict(im=(3, 6, 9, 11), n=20, pool=(2, 2)),                          # odd sizes: pixels no window takes still get a MEX value
+    dict(im=(4, 8, 6, 10), n=33, pool=(1, 2)),                          # two-pixel windows
+    dict(im=(4, 12, 8, 8), n=10, pool=(2, 2), kw=dict(blocks=[3, 1, 1], strides=[3, 1, 1], shared_offset_region=[2],
+                                                      use_unshared_regions=False)),   # not fusable: two kernels
+])
+@pytest.mark.parametrize("spread", ["narrow", "wide"])
+def test_mex_sum_pool_for_training_keeps_the_mex_output(pkg, case, spread):
+    """`mex_sum_pool_both` (what `layers.mex_sum_pool` runs when a gradient is needed) returns the MEX output before
+    pooling and the pooled output from one call: the pooled tensor has the bits `mex_sum_pool` gives (the same kernel
+    with one more store), the MEX output the values of `mex` up to rounding (another kernel may serve the plain call),
+    and gradients through it agree with those of the two separate differentiable calls."""
+    g = torch.Generator(device="cuda").manual_seed(12)
+    im, n, pool = case["im"], case["n"], case["pool"]
+    kw = dict(dict(softmax_mode=True, blocks=[im[1], 1, 1], strides=[im[1], 1, 1],
+                   unshared_offset_region=[1, pool[0], pool[1]], epsilon=1.5), **case.get("kw", {}))
+    x = torch.randn(im, device="cuda", generator=g)
+    _, oshape = pkg.mex_output_shape(im, n, **kw)
+    off = torch.randn(oshape, device="cuda", generator=g) * (150.0 if spread == "wide" else 0.3)
+    full, pooled = pkg.mex_sum_pool_both(x, off, n, pool, normalize_offsets=True, **kw)
+    plain = pkg.mex(x, off, n, normalize_offsets=True, **kw)
+    scale = float(plain.abs().max())
+    assert full.shape == plain.shape and float((full - plain).abs().max()) <= 1e-5 * scale
+    assert torch.equal(pooled, pkg.mex_sum_pool(x, off, n, pool, normalize_offsets=True, **kw))
+    assert torch.equal(pooled, pkg.sum_pooling(full, pool))
+    # gradients: fused forward against the two separate differentiable calls
+    L = pkg.layers
+    leaves = [t.clone().requires_grad_() for t in (x, off, x, off)]
+    y1 = L.mex_sum_pool(leaves[0], leaves[1], n, pool, normalize_offsets=True, **kw)
+    y2 = L.sum_pooling(L.mex(leaves[2], leaves[3], n, normalize_offsets=True, **kw), pool)
+    assert float((y1 - y2).detach().abs().max()) <= 1e-5 * float(y2.detach().abs().max())
+    go = torch.randn(y1.shape, device="cuda", generator=g)
+    y1.backward(go)
+    y2.backward(go)
+    for a, b in ((leaves[0].grad, leaves[2].grad), (leaves[1].grad, leaves[3].grad)):
+        assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max())
+
+
 @pytest.mark.parametrize("shape,pool", [((3, 5, 8, 10), (2, 2)), ((2, 3, 7, 9), (2, 3)), ((1, 4, 5, 5), (5, 1))])
 def test_sum_pooling_gradient(pkg, shape, pool):
     """layers.sum_pooling: forward = avg_pool2d * area ('valid': trailing rows/columns dropped), the gradient spreads
