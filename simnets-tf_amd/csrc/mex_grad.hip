@@ -762,6 +762,457 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Row-wise forms of the two matrix kernels for the layers of the reference's networks: 2 x 2 unshared offsets over
+// whole-channel patches (blocks [C, 1, 1], stride 1, no padding) on maps whose height and width are powers of two.
+// There the pixel slots of a region are every other pixel of every other row.  A wave that walks one region's slots
+// touches 16 to 64 separate 32-byte sectors per load and uses half of each or less, the four regions write the
+// input gradient into each other's sectors at different times, and the address units, not the arithmetic, set the
+// time of the kernels above.  Here a workgroup takes the 64 slots of a chunk for ALL four regions - 256 pixels that
+// are whole rows of one image or whole small images - so that every plane (an instance of `out` / `g`, a channel
+// of the input or of its gradient) is read and written as one run of 1 KB, or runs of whole images, with 16-byte
+// accesses.  The values pass through LDS tiles [plane][column] with column = region * 64 + slot, and wave r does
+// the matrix steps of region r on its 64 columns.
+struct RowsArgs {
+    int lgW, Ws, RS;   // log2(width), windows per row, windows per image
+    int lgHW, HW;      // pixels of an image
+    int nx, ty, tz;    // workgroup numbering (rows_block): pixel groups, tiles along the two other grid dimensions
+};
+
+// Workgroups that read the same rows - the tiles (y, z) of one pixel group x - get consecutive turns on ONE
+// accelerator die (linear workgroup id mod 8), so that the rows come from memory once and from that die's L2 for the
+// other tiles.  The launch is one-dimensional with 8 * ceil(nx / 8) * ty * tz workgroups; false: no such group.
+__device__ __forceinline__ bool rows_block(const RowsArgs &g, int *x, int *y, int *z)
+{
+    const int l = blockIdx.x, tiles = g.ty * g.tz;
+    const int j = l >> 3, tile = j % tiles;
+    *x = (j / tiles) * 8 + (l & 7);
+    *y = tile % g.ty;
+    *z = tile / g.ty;
+    return *x < g.nx;
+}
+
+// A thread's four neighbouring pixels (a 16-byte piece of a row; width >= 4, so they share the row) of the chunk's
+// 256: image, first pixel, tile columns.  Pixels 0 and 2 belong to region rbase, 1 and 3 to rbase + 1.  A chunk
+// starts on an even row (or a whole image), so the columns and rbase depend on the quad alone, not on the chunk.
+struct RowsQuad {
+    int img, pix0, rbase;
+    bool img_ok;
+    int col[4];
+};
+
+__device__ __forceinline__ RowsQuad rows_quad(const MexKernelArgs &a, const RowsArgs &g, int chunk, int quad)
+{
+    RowsQuad q;
+    const int gpix = chunk * 256 + 4 * quad;
+    q.img = gpix >> g.lgHW;
+    q.pix0 = gpix & (g.HW - 1);
+    q.img_ok = q.img < a.B;
+    const int h = q.pix0 >> g.lgW, w0 = q.pix0 & ((1 << g.lgW) - 1);
+    q.rbase = (h & 1) * 2;
+    const int sl = q.img * g.RS + (h >> 1) * g.Ws + (w0 >> 1) - chunk * 64;
+    q.col[0] = (q.rbase << 6) + sl;
+    q.col[1] = q.col[0] + 64;
+    q.col[2] = q.col[0] + 1;
+    q.col[3] = q.col[1] + 1;
+    return q;
+}
+
+// per region: does some instance's offsets range exceed the product form's (flags[r]); returns whether some range
+// exceeds kLooseBoundRange.  All threads of the workgroup call it.
+__device__ __forceinline__ int rows_ranges(const MexKernelArgs &a, int tid, int *flags)
+{
+    if (tid < 4)
+        flags[tid] = 0;
+    __syncthreads();
+    const int per = a.n_mgroups * GM_TM;
+    int big = 0;
+    for (int i = tid; i < 4 * per; i += 256) {
+        const int r = i / per, m = i - r * per;
+        if (m < a.M) {
+            const float rg = a.orng[i];
+            big |= !(rg <= kLooseBoundRange);
+            if (!(rg <= kProductRange))
+                flags[r] = 1;   // (every writer writes the same value)
+        }
+    }
+    return __syncthreads_or(big);
+}
+
+// Input gradient.  Workgroup (rows_block) x: chunk of 256 pixels; y: tile of 16 * KSUB patch elements; z: split of the
+// instance groups.  Per instance group the pixel factors W [32][256] are formed from rows of `out` and `g`, the four
+// regions' offset exponentials [16 * KSUB][32] come from the packed offsets, and wave r accumulates region r's
+// 16 * KSUB x 64 gradients; these leave through a tile [patch element][column], times 2^(xs - a) from rows of the
+// input, as rows of the gradient.  A region with a wide offsets range is done term by term (the other three are not
+// held up by it).
+template <int KSUB>
+__global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_grad_input_rows_kernel(const MexGradArgs ga, const RowsArgs g)
+{
+    const MexKernelArgs &a = ga.k;
+    constexpr int KT = 16 * KSUB;
+    constexpr int WP = 272, EP = 36, OP = 260;   // row pitches: the matrix steps' and the tile's accesses hit 64 banks
+    constexpr int kWt = 32 * WP, kEo = 4 * KT * EP, kOt = KT * OP;
+    constexpr int kTile = kWt + kEo > kOt ? kWt + kEo : kOt;
+    __shared__ __attribute__((aligned(16))) float smem[kTile];
+    __shared__ float ap[256];          // per column: the pixel's bound (0 for an empty slot)
+    __shared__ float tab[2][128];      // per (region, instance of the group): omax + c0, for this group and the next
+    __shared__ int wide_sh[4];
+    float *wt = smem, *eo = smem + kWt, *ot = smem;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lq = lane >> 4;
+    int chunk, by, bz;
+    if (!rows_block(g, &chunk, &by, &bz))
+        return;
+    const int k0 = by * KT;
+    const int n_mg = a.n_mgroups, per = n_mg * GM_TM;
+    const int mg_begin = bz * ga.mg_per_split, mg_end = min(n_mg, mg_begin + ga.mg_per_split);
+    float *dxo = ga.msplit > 1 ? ga.dx_splits + (size_t)bz * a.B * a.C * a.H * a.W : ga.dx;
+    const RowsQuad q = rows_quad(a, g, chunk, lane);
+    const int pl0 = wave;              // this thread's planes of a block of 32: pl0, pl0 + 4, ...
+    const size_t HW = (size_t)g.HW;
+    const size_t img = q.img_ok ? q.img : 0;
+    // operands of an instance group: this thread's eight rows pieces of `out` and `g`, its share of the four regions'
+    // offset exponentials, the next group's instance constants - requested a group ahead (the first before the bound
+    // is worked out, the others while the matrix steps run)
+    float4 ov[8], gv[8], en[2 * KSUB];
+    float tn = 0.0f;
+    auto request = [&](int mg) {
+        // (those past the last instance, image or patch element on a clamped address or skipped)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int m = min(mg * GM_TM + pl0 + 4 * j, a.M - 1);
+            const size_t at = (img * a.M + m) * HW + q.pix0;
+            ov[j] = *reinterpret_cast<const float4 *>(ga.out + at);
+            gv[j] = *reinterpret_cast<const float4 *>(ga.g + at);
+        }
+#pragma unroll
+        for (int j = 0; j < 2 * KSUB; ++j) {
+            const int i = tid + 256 * j;
+            const int r = i / (KT * 8), row = (i % (KT * 8)) >> 3, c4 = i & 7;
+            en[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (k0 + row < a.K)
+                en[j] = *reinterpret_cast<const float4 *>(a.offe + (((size_t)r * n_mg + mg) * a.K + k0 + row) * GM_TM + 4 * c4);
+        }
+        if (tid < 128 && mg + 1 < mg_end)
+            tn = a.omax[(tid >> 5) * per + (mg + 1) * GM_TM + (tid & 31)] + a.c0;
+    };
+    if (mg_begin < mg_end)
+        request(mg_begin);
+    const int roomy = rows_ranges(a, tid, wide_sh);
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
+    // ---- the bound of every pixel: a = min over (a few) instances of outs_m - c0 - lo_m, see
+    //      mex_grad_input_mfma_kernel ----
+    const int m_scan = roomy ? a.M : min(a.M, 4);
+    float amin = INFINITY;             // of column tid
+    for (int mb = 0; mb < m_scan; mb += 32) {
+        if (tid < 128) {
+            const int m = min(mb + (tid & 31), a.M - 1);
+            tab[0][tid] = a.omax[(tid >> 5) * per + m] - a.orng[(tid >> 5) * per + m];
+        }
+        float4 bo[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int m = mb + pl0 + 4 * j;
+            bo[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (q.img_ok && m < m_scan)
+                bo[j] = *reinterpret_cast<const float4 *>(ga.out + (img * a.M + m) * HW + q.pix0);
+        }
+        __syncthreads();               // tab in place; the previous block's readers are done with the tile
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int pl = pl0 + 4 * j;
+            const bool use = q.img_ok && mb + pl < m_scan;
+            const float v[4] = {bo[j].x, bo[j].y, bo[j].z, bo[j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                wt[pl * WP + q.col[e]] =
+                    use ? __builtin_fmaf(v[e], a.c1, -(a.c0 + tab[0][(q.rbase + (e & 1)) * 32 + pl])) : INFINITY;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int pl = 0; pl < 32; ++pl)
+            amin = fminf(amin, wt[pl * WP + tid]);
+    }
+    ap[tid] = chunk * 64 + (tid & 63) < a.slots ? amin : 0.0f;
+    if (tid < 128 && mg_begin < mg_end)   // (the loop above is done with the table: its last readers passed the
+        tab[mg_begin & 1][tid] = a.omax[(tid >> 5) * per + mg_begin * GM_TM + (tid & 31)] + a.c0;   // barrier in front of the reduction)
+    __syncthreads();
+    float bound[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+        bound[e] = ap[q.col[e]];
+
+    floatx4 acc[KSUB][4];
+#pragma unroll
+    for (int ks = 0; ks < KSUB; ++ks)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+            acc[ks][t] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    constexpr int NJ = KT / 4;
+    float4 xv[NJ];                     // the epilogue's rows of the input, requested during the last matrix steps
+    for (int mg = mg_begin; mg < mg_end; ++mg) {
+        __syncthreads();               // the previous group's matrix steps are done with wt / eo
+        const float *tb = tab[mg & 1];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int pl = pl0 + 4 * j;
+            const bool use = q.img_ok && mg * GM_TM + pl < a.M;
+            const float o[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
+            const float gg[4] = {gv[j].x, gv[j].y, gv[j].z, gv[j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
+                const float ex = __builtin_fmaf(-o[e], a.c1, bound[e]) + tb[(q.rbase + (e & 1)) * 32 + pl];
+                wt[pl * WP + q.col[e]] = use ? gg[e] * __builtin_amdgcn_exp2f(ex) : 0.0f;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 2 * KSUB; ++j) {
+            const int i = tid + 256 * j;
+            const int r = i / (KT * 8), row = (i % (KT * 8)) >> 3, c4 = i & 7;
+            *reinterpret_cast<float4 *>(eo + (r * KT + row) * EP + 4 * c4) = en[j];
+        }
+        if (tid < 128)
+            tab[(mg + 1) & 1][tid] = tn;
+        if (mg + 1 < mg_end) {
+            request(mg + 1);
+        } else {
+#pragma unroll
+            for (int j = 0; j < NJ; ++j) {
+                const int k = min(k0 + pl0 + 4 * j, a.K - 1);
+                xv[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + k) * HW + q.pix0);
+            }
+        }
+        __syncthreads();
+        if (!my_wide) {
+#pragma unroll
+            for (int ms = 0; ms < GM_TM; ms += 4) {
+                float bv[4];
+#pragma unroll
+                for (int t = 0; t < 4; ++t)
+                    bv[t] = wt[(ms + lq) * WP + wave * 64 + t * 16 + lr];
+#pragma unroll
+                for (int ks = 0; ks < KSUB; ++ks) {
+                    const float av = eo[(wave * KT + ks * 16 + lr) * EP + ms + lq];
+#pragma unroll
+                    for (int t = 0; t < 4; ++t)
+                        acc[ks][t] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, bv[t], acc[ks][t], 0, 0, 0);
+                }
+            }
+        }
+    }
+    // ---- d patch_k = 2^(xs_k - a) * acc: through the tile [patch element][column] to rows of the gradient ----
+    if (mg_begin >= mg_end) {
+#pragma unroll
+        for (int j = 0; j < NJ; ++j)
+            xv[j] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    __syncthreads();                   // the last matrix steps are done with wt / eo, which the tile overlies
+#pragma unroll
+    for (int ks = 0; ks < KSUB; ++ks)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                ot[(ks * 16 + 4 * lq + v) * OP + wave * 64 + t * 16 + lr] = acc[ks][t][v];
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+        const int kl = pl0 + 4 * j, k = k0 + kl;
+        if (!q.img_ok || k >= a.K)
+            continue;
+        const float x[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
+        float d[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            d[e] = ot[kl * OP + q.col[e]] * __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], a.c1, -bound[e]));
+        float *dst = dxo + (img * a.K + k) * HW + q.pix0;
+        if (!any_wide) {
+            *reinterpret_cast<float4 *>(dst) = make_float4(d[0], d[1], d[2], d[3]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (!wide_sh[q.rbase + (e & 1)])
+                    dst[e] = d[e];
+        }
+    }
+    if (any_wide) {
+        // the regions with a wide offsets range, term by term: GX_KT patch elements of a region per wave and turn
+        constexpr int NSUB = KT / GX_KT;
+        for (int u = wave; u < 4 * NSUB; u += 4) {
+            const int r = u / NSUB, kk0 = k0 + (u % NSUB) * GX_KT;
+            if (wide_sh[r] && kk0 < a.K)
+                mex_grad_input_wave(ga, r, chunk, kk0, lane, min(a.M, mg_begin * GM_TM), min(a.M, mg_end * GM_TM), dxo);
+        }
+    }
+}
+
+// Offsets gradient.  Workgroup (rows_block) x: group of ga.pxl chunks of 256 pixels; y: tile of 32 instances; z: tile
+// of 32 patch elements.  Per chunk the tile's pixel factors W [32][256] and patch exponentials [32][256] are formed from
+// rows of `out`, `g` and the input - relative to the bound over the tile's own instances, which the rows just read
+// give - and wave r adds region r's 32 x 32 products over its 64 columns.  Partial sums [chunk group][region][M][K]
+// like mex_grad_offsets_mfma_kernel's.
+__global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGradArgs ga, const RowsArgs g)
+{
+    const MexKernelArgs &a = ga.k;
+    constexpr int TP = 260;
+    __shared__ float wt[32 * TP];      // [instance][column]
+    __shared__ float ex[32 * TP];      // [patch element][column]
+    __shared__ float pm[4 * 256];      // per column: the four waves' minima
+    __shared__ int wide_sh[4];
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int lr = lane & 15, lq = lane >> 4;
+    int bx, by, bz;
+    if (!rows_block(g, &bx, &by, &bz))
+        return;
+    const int m0 = by * 32, k0 = bz * 32;
+    const int n_mg = a.n_mgroups, per = n_mg * GM_TM;
+    const int pl0 = wave;
+    const size_t HW = (size_t)g.HW;
+    rows_ranges(a, tid, wide_sh);
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
+    // the constants of this thread's planes for its two regions (the same in every chunk)
+    const RowsQuad q0 = rows_quad(a, g, 0, lane);   // (the columns and regions are the same in every chunk)
+    const int rbase = q0.rbase;
+    float lo[8][2], omc[8][2];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+        for (int par = 0; par < 2; ++par) {
+            const int idx = (rbase + par) * per + min(m0 + pl0 + 4 * j, a.M - 1);
+            const float om = a.omax[idx];
+            lo[j][par] = a.c0 + (om - a.orng[idx]);
+            omc[j][par] = om + a.c0;
+        }
+    floatx4 acc[2][2];
+#pragma unroll
+    for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+        for (int kt = 0; kt < 2; ++kt)
+            acc[mt][kt] = floatx4{0.0f, 0.0f, 0.0f, 0.0f};
+    // the rows of a chunk: this thread's pieces of eight instances of `out` and `g` and of eight channels of the
+    // input; those of chunk s + 1 are requested as soon as chunk s has gone to LDS, in front of its matrix steps
+    float4 ov[8], gv[8], xv[8];
+    bool img_ok = false;
+    auto request = [&](int s) {
+        const RowsQuad q = rows_quad(a, g, bx * ga.pxl + s, lane);
+        img_ok = q.img_ok;
+        const size_t img = q.img_ok ? q.img : 0;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int m = min(m0 + pl0 + 4 * j, a.M - 1), k = min(k0 + pl0 + 4 * j, a.K - 1);
+            const size_t at = (img * a.M + m) * HW + q.pix0;
+            ov[j] = *reinterpret_cast<const float4 *>(ga.out + at);
+            gv[j] = *reinterpret_cast<const float4 *>(ga.g + at);
+            xv[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + k) * HW + q.pix0);
+        }
+    };
+    // chunks of this workgroup that hold pixels (uniform)
+    const int n_steps = min(ga.pxl, ga.slots_pad / 64 - bx * ga.pxl);
+    if (n_steps > 0)
+        request(0);
+    for (int s = 0; s < n_steps; ++s) {
+        const bool cur_ok = img_ok;
+        float cand[4] = {INFINITY, INFINITY, INFINITY, INFINITY};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (m0 + pl0 + 4 * j >= a.M)
+                continue;
+            const float o[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                cand[e] = fminf(cand[e], __builtin_fmaf(o[e], a.c1, -lo[j][e & 1]));
+        }
+        __syncthreads();               // the previous chunk's matrix steps are done with wt / ex, its readers with pm
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+            pm[pl0 * 256 + q0.col[e]] = cand[e];
+        __syncthreads();
+        float bound[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int c = q0.col[e];
+            bound[e] = cur_ok ? fminf(fminf(pm[c], pm[256 + c]), fminf(pm[512 + c], pm[768 + c])) : 0.0f;
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int pl = pl0 + 4 * j;
+            const bool use_m = cur_ok && m0 + pl < a.M, use_k = cur_ok && k0 + pl < a.K;
+            const float o[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
+            const float gg[4] = {gv[j].x, gv[j].y, gv[j].z, gv[j].w};
+            const float x[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float we = __builtin_fmaf(-o[e], a.c1, bound[e]) + omc[j][e & 1];
+                wt[pl * TP + q0.col[e]] = use_m ? gg[e] * __builtin_amdgcn_exp2f(we) : 0.0f;
+                ex[pl * TP + q0.col[e]] = use_k ? __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], a.c1, -bound[e])) : 0.0f;
+            }
+        }
+        if (s + 1 < n_steps)
+            request(s + 1);
+        __syncthreads();
+        if (!my_wide) {
+#pragma unroll 4
+            for (int ps = 0; ps < 64; ps += 4) {
+                float wa[2], xb[2];
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    wa[i] = wt[(i * 16 + lr) * TP + wave * 64 + ps + lq];
+                    xb[i] = ex[(i * 16 + lr) * TP + wave * 64 + ps + lq];
+                }
+#pragma unroll
+                for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+                        acc[mt][kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(wa[mt], xb[kt], acc[mt][kt], 0, 0, 0);
+            }
+        }
+    }
+    // ---- partial sums of this chunk group: acc * 2^(os_mk - mo_m) ----
+    if (!my_wide) {
+        float *dst = ga.partial + ((size_t)bx * a.R + wave) * a.M * a.K;
+        float eov[2][2][4];
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int m = min(m0 + mt * 16 + 4 * lq + v, a.M - 1);
+                const float *eo = a.offe + (((size_t)wave * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt)
+                    eov[mt][kt][v] = eo[(size_t)min(k0 + kt * 16 + lr, a.K - 1) * GM_TM];
+            }
+#pragma unroll
+        for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int m = m0 + mt * 16 + 4 * lq + v;
+                if (m >= a.M)
+                    continue;
+#pragma unroll
+                for (int kt = 0; kt < 2; ++kt) {
+                    const int k = k0 + kt * 16 + lr;
+                    if (k < a.K)
+                        dst[(size_t)m * a.K + k] = acc[mt][kt][v] * eov[mt][kt][v];
+                }
+            }
+    }
+    if (any_wide) {
+        // the regions with a wide offsets range, term by term: this workgroup's tile as GO_MT x GO_KT wave tiles
+        constexpr int NU = (32 / GO_MT) * (32 / GO_KT);
+        for (int u = wave; u < 4 * NU; u += 4) {
+            const int r = u / NU, i = u % NU;
+            const int mm0 = m0 + (i / (32 / GO_KT)) * GO_MT, kk0 = k0 + (i % (32 / GO_KT)) * GO_KT;
+            if (wide_sh[r] && mm0 < a.M && kk0 < a.K)
+                mex_grad_offsets_wave(ga, r, bx, mm0, kk0, lane);
+        }
+    }
+}
+
 // dOff[r,m,k] = sum over pixel chunks, in a fixed order (reproducible): a workgroup takes 32 consecutive elements,
 // its 8 groups of 32 threads each sum every 8th chunk in chunk order, and the 8 sums are added in group order.
 __global__ __launch_bounds__(256) void mex_grad_offsets_finish_kernel(const float *__restrict__ partial, long long n,
@@ -850,6 +1301,49 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_finish_rows_kernel(const
     float *gr = doff + (size_t)row * K;
     const float *pr = partial + (size_t)row * K;
     float sum = 0.0f;
+    if (K <= 32) {
+        // rows shorter than a wave: the lanes form 64 / Kp groups (Kp = 8, 16 or 32 >= K) that each take 8 / groups
+        // of the eight interleaved sums, four rounds of chunks requested at a time; every lane then adds the eight
+        // sums in order (read from the lanes that hold them), so the values are those of the loop below
+        const int lg = K <= 8 ? 3 : K <= 16 ? 4 : 5, Kp = 1 << lg;
+        const int per = 8 >> (6 - lg);               // sums per group: 1, 2 or 4
+        const int gi = lane >> lg, k = lane & (Kp - 1), kc = min(k, K - 1);
+        float sj[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        for (int c0 = 0; c0 < chunks; c0 += 32) {
+            float v[4][4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (i < per)
+                        v[u][i] = pr[(size_t)min(c0 + 8 * u + gi * per + i, chunks - 1) * n + kc];
+#pragma unroll
+            for (int u = 0; u < 4; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i)
+                    if (i < per && c0 + 8 * u + gi * per + i < chunks)
+                        sj[i] += v[u][i];
+        }
+        float t = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int i = j & (per - 1), src = ((j >> (lg - 3)) << lg) + k;   // sum j lives in group j / per, slot j % per
+            const float mine = i == 0 ? sj[0] : i == 1 ? sj[1] : i == 2 ? sj[2] : sj[3];
+            const float val = __shfl(mine, src, 64);
+            t = j == 0 ? val : t + val;
+        }
+        const bool owner = gi == 0 && k < K;
+        if (owner)
+            gr[k] = t;
+        if (normalized == nullptr)
+            return;
+        sum = owner ? t : 0.0f;
+        for (int d = 32; d > 0; d >>= 1)
+            sum += __shfl_xor(sum, d, 64);
+        if (owner)
+            gr[k] = t - expf(normalized[(size_t)row * K + k]) * sum;
+        return;
+    }
     for (int k = lane; k < K; k += 64) {
         float s8[8];
 #pragma unroll
@@ -902,7 +1396,35 @@ struct MexGradTiling {
     bool factors_input, factors_offsets;
     int slots_pad, Mp, Kp;
     size_t factor_bytes;
+    // the row-wise kernels (mex_grad_input_rows_kernel, mex_grad_offsets_rows_kernel): the layer qualifies (the
+    // pointers are checked at the launch), and their tiling
+    bool rows;
+    int rows_ksub;                        // input gradient: 16 * ksub patch elements per workgroup
+    int rows_msplit, rows_mg_per_split;   // ... and the split of its instance groups
+    int rows_pxl, rows_cpr;               // offsets gradient: chunks per workgroup, workgroups along the pixels
 };
+
+inline int log2_exact(int v)   // log2 of a power of two, -1 otherwise
+{
+    int l = 0;
+    while ((1 << l) < v)
+        ++l;
+    return v > 0 && (1 << l) == v ? l : -1;
+}
+
+// 2 x 2 unshared offsets over whole-channel patches on a map with power-of-two sides: see the row-wise kernels.
+// A chunk of 256 pixels must be whole images or an even number of whole rows (width <= 128), so that it holds
+// exactly the 64 slots [64 chunk, 64 chunk + 64) of each of the four regions; a 16-byte piece lies in one row
+// (width >= 4).
+bool rows_geometry(const MexPlan &p)
+{
+    const simnets_mex_dims &d = p.d;
+    return std::isfinite(p.epsilon) && p.use_unshared && d.offsets_c == 1 && d.offsets_h == 2 && d.offsets_w == 2 &&
+           d.channels_out == 1 && d.block_c == p.C && d.block_h == 1 && d.block_w == 1 && d.stride_h == 1 &&
+           d.stride_w == 1 && d.pad_c == 0 && d.pad_h == 0 && d.pad_w == 0 && d.height_out == p.H &&
+           d.width_out == p.W && log2_exact(p.H) >= 1 && log2_exact(p.W) >= 2 && p.W <= 128 &&
+           d.region_size == (p.H / 2) * (p.W / 2) && (long long)p.B * p.H * p.W <= 0x3fffffffLL;
+}
 
 MexGradTiling mex_grad_tiling(const MexPlan &p)
 {
@@ -948,6 +1470,34 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
     t.factors_input = t.mfma && k_tiles >= 4 && d.M >= 128;
     t.factors_offsets = t.mfma && m_tiles * ((d.K + GOM_KT - 1) / GOM_KT) >= 16;
     t.factor_bytes = align_up((size_t)d.num_regions * t.slots_pad * ((size_t)t.Mp + t.Kp) * sizeof(float), 256);
+    // Row-wise kernels: about two workgroups per compute unit at least.  The input gradient takes as many patch
+    // elements per workgroup as that allows (each tile of them reads all of `out` and `g`), then splits the instance
+    // groups; the offsets gradient walks as many chunks per workgroup as that allows (each workgroup writes a
+    // partial sum of its tile).
+    t.rows = rows_geometry(p);
+    t.rows_ksub = 1; t.rows_msplit = 1; t.rows_mg_per_split = n_mg; t.rows_pxl = 1; t.rows_cpr = 0;
+    if (t.rows) {
+        const long long chunks = t.slots_pad / 64;
+        auto ktiles = [&](int ksub) { return (long long)((d.K + 16 * ksub - 1) / (16 * ksub)); };
+        t.rows_ksub = std::min(4, (d.K + 15) / 16);
+        if (t.rows_ksub == 3)
+            t.rows_ksub = 4;
+        while (t.rows_ksub > 1 && chunks * ktiles(t.rows_ksub) < 512)
+            t.rows_ksub >>= 1;
+        const long long wgs_in = chunks * ktiles(t.rows_ksub);
+        if (wgs_in < 512 && n_mg >= 4)
+            t.rows_msplit = (int)std::max<long long>(1, std::min<long long>(std::min(8, n_mg / 2), 512 / std::max<long long>(wgs_in, 1)));
+        t.rows_mg_per_split = (n_mg + t.rows_msplit - 1) / t.rows_msplit;
+        t.rows_msplit = (n_mg + t.rows_mg_per_split - 1) / t.rows_mg_per_split;
+        if (t.rows_msplit > 1)
+            t.split_bytes = std::max(t.split_bytes, align_up((size_t)t.rows_msplit * p.B * p.C * p.H * p.W * sizeof(float), 256));
+        const long long tiles = (long long)((d.M + 31) / 32) * ((d.K + 31) / 32);
+        t.rows_pxl = 16;
+        while (t.rows_pxl > 1 && (chunks + t.rows_pxl - 1) / t.rows_pxl * tiles < 512)
+            t.rows_pxl >>= 1;
+        t.rows_cpr = (int)((chunks + t.rows_pxl - 1) / t.rows_pxl);
+        t.partial_bytes = std::max(t.partial_bytes, align_up(rmk * t.rows_cpr, 256));
+    }
     return t;
 }
 
@@ -1072,17 +1622,25 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
     ga.pxl = 1;
     ga.cpr = (ga.k.slots + 63) / 64;
+    // the row-wise kernels read and write 16 bytes at a time
+    auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
+    const bool use_rows = t.mfma && t.rows && aligned16(input) && aligned16(output) && aligned16(output_grad) &&
+                          (!want_input || aligned16(input_grad));
     if (t.mfma) {
         rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream, nullptr, true,
                               pack_normalizes ? reinterpret_cast<float *>(ws + w.norm) : nullptr);
         if (rc)
             return rc;
-        if (w.use_factors) {
+        if (w.use_factors && !use_rows) {
             rc = launch_factors(p, t, ga, ws + w.factors, s);
             if (rc)
                 return rc;
         }
     }
+    RowsArgs rg;
+    rg.lgW = log2_exact(p.W); rg.Ws = p.W / 2; rg.RS = d.region_size; rg.HW = p.H * p.W; rg.lgHW = log2_exact(rg.HW);
+    if (use_rows)
+        ga.slots_pad = t.slots_pad;
 
     if (want_input) {
         MexGradArgs gi = ga;
@@ -1101,7 +1659,31 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
                 return SIMNETS_ERR_HIP;
         }
         const long long gx = (long long)d.num_regions * gi.cpr;
-        if (t.mfma) {
+        if (use_rows) {
+            gi.wbuf = gi.exbuf = nullptr;
+            gi.msplit = t.rows_msplit; gi.mg_per_split = t.rows_mg_per_split;
+            const int kt = 16 * t.rows_ksub, gy = (d.K + kt - 1) / kt;
+            if (gy > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            rg.nx = t.slots_pad / 64; rg.ty = gy; rg.tz = t.rows_msplit;
+            const long long wgs = (long long)((rg.nx + 7) / 8 * 8) * gy * t.rows_msplit;
+            if (wgs > 0x7fffffffLL)
+                return SIMNETS_ERR_TOO_LARGE;
+            const dim3 grid((unsigned)wgs);
+            if (t.rows_ksub == 4)
+                hipLaunchKernelGGL(mex_grad_input_rows_kernel<4>, grid, dim3(256), 0, s, gi, rg);
+            else if (t.rows_ksub == 2)
+                hipLaunchKernelGGL(mex_grad_input_rows_kernel<2>, grid, dim3(256), 0, s, gi, rg);
+            else
+                hipLaunchKernelGGL(mex_grad_input_rows_kernel<1>, grid, dim3(256), 0, s, gi, rg);
+            if (t.rows_msplit > 1) {
+                if (hipGetLastError() != hipSuccess)
+                    return SIMNETS_ERR_HIP;
+                hipLaunchKernelGGL(mex_sum_splits_kernel,
+                                   dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)), dim3(256), 0, s,
+                                   gi.dx_splits, n_in, t.rows_msplit, input_grad);
+            }
+        } else if (t.mfma) {
             const int gy = (d.K + GM_KT - 1) / GM_KT;
             if (gx > 0x7fffffffLL || gy > 65535)
                 return SIMNETS_ERR_TOO_LARGE;
@@ -1141,7 +1723,19 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
         if (!t.factors_offsets)
             go.wbuf = go.exbuf = nullptr;
         const long long gx = (long long)d.num_regions * go.cpr;
-        if (t.mfma) {
+        if (use_rows) {
+            go.wbuf = go.exbuf = nullptr;
+            go.pxl = t.rows_pxl;
+            go.cpr = t.rows_cpr;
+            const int gy = (d.M + 31) / 32, gz = (d.K + 31) / 32;
+            if (gy > 65535 || gz > 65535)
+                return SIMNETS_ERR_TOO_LARGE;
+            rg.nx = t.rows_cpr; rg.ty = gy; rg.tz = gz;
+            const long long wgs = (long long)((rg.nx + 7) / 8 * 8) * gy * gz;
+            if (wgs > 0x7fffffffLL)
+                return SIMNETS_ERR_TOO_LARGE;
+            hipLaunchKernelGGL(mex_grad_offsets_rows_kernel, dim3((unsigned)wgs), dim3(256), 0, s, go, rg);
+        } else if (t.mfma) {
             const int gy = (d.M + GOM_MT - 1) / GOM_MT, gz = (d.K + GOM_KT - 1) / GOM_KT;
             if (gx > 0x7fffffffLL || gy > 65535 || gz > 65535)
                 return SIMNETS_ERR_TOO_LARGE;

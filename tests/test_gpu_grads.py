@@ -578,6 +578,47 @@ def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, sp
     check_mex_grads(pkg, x, off, 200, strict=spread != "mixed", **kw)
 
 
+@pytest.mark.parametrize("spread", ["narrow", "roomy", "mixed"])
+@pytest.mark.parametrize("im,n", [
+    ((3, 32, 16, 16), 64),     # a 256-pixel chunk is one image
+    ((5, 40, 8, 8), 70),       # four images a chunk; ragged instance and channel blocks; the last chunk is part empty
+    ((9, 16, 4, 4), 33),       # sixteen images a chunk
+    ((3, 12, 2, 8), 5),        # two rows
+    ((2, 8, 32, 64), 6),       # eight chunks an image, four rows each
+    ((1, 5, 8, 128), 3),       # widest map the row-wise kernel takes: two rows a chunk
+    ((2, 4, 4, 256), 3),       # wider: the gathering factors kernel
+])
+def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
+    """2 x 2 unshared offsets over whole-channel patches on maps with power-of-two sides: the pixel factors and patch
+    exponentials are formed from whole rows (16-byte loads along the rows, regions interleaved through LDS) and both
+    matrix kernels read them back.  'roomy': offsets ranges beyond the few-instances bound, 'mixed': every other
+    region beyond the product form's range (term by term there).  Also through views that are not 16-byte aligned,
+    which take the gathering kernel: same results to the same bar."""
+    kw = dict(blocks=[im[1], 1, 1], strides=[im[1], 1, 1], padding=[0, 0, 0], unshared_offset_region=[2], epsilon=1.5,
+              softmax_mode=False)
+    x, off = mex_case(71, im, n, **kw)
+    off = off * {"narrow": 0.5, "roomy": 2.5, "mixed": 0.3}[spread]
+    if spread == "mixed":
+        off[::2] *= 300
+    check_mex_grads(pkg, x, off, n, strict=spread != "mixed", **kw)
+    # unaligned views of the same tensors
+    out = orc.mex_fwd(x, off, n, **kw)
+    g = np.random.default_rng(3).normal(size=out.shape).astype(np.float32)
+
+    def shifted(a):
+        buf = torch.empty(a.size + 1, device="cuda", dtype=torch.float32)
+        v = buf[1:].view(a.shape)
+        v.copy_(torch.from_numpy(a))
+        return v
+
+    X, O, Y, G = dev(x), dev(off), dev(out), dev(g)
+    dx, doff = pkg.mex_grads(X, O, Y, G, n, **kw)
+    dx_u, doff_u = pkg.mex_grads(shifted(x), O, shifted(out), shifted(g), n, **kw)
+    scale_x, scale_o = float(dx.abs().max()), float(doff.abs().max())
+    assert float((dx - dx_u).abs().max()) <= 1e-4 * scale_x
+    assert float((doff - doff_u).abs().max()) <= 1e-4 * scale_o
+
+
 @pytest.mark.parametrize("case", [
     dict(im=(5, 40, 6, 6), n=70, kw=dict(blocks=[40, 1, 1], strides=[40, 1, 1], padding=[0, 0, 0],
                                          unshared_offset_region=[2], epsilon=2.0, softmax_mode=True)),
