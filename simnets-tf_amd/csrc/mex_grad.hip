@@ -818,25 +818,40 @@ __device__ __forceinline__ RowsQuad rows_quad(const MexKernelArgs &a, const Rows
     return q;
 }
 
-// per region: does some instance's offsets range exceed the product form's (flags[r]); returns whether some range
-// exceeds kLooseBoundRange.  All threads of the workgroup call it.
-__device__ __forceinline__ int rows_ranges(const MexKernelArgs &a, int tid, int *flags)
+// per region: does some instance's offsets range exceed the product form's (flags[r]); flags[4]: does some range
+// exceed kLooseBoundRange.  All threads of the workgroup call it; the flags are in place behind its last barrier.
+// (All loads go out before the first is looked at.)
+__device__ __forceinline__ void rows_ranges(const MexKernelArgs &a, int tid, int *flags)
 {
-    if (tid < 4)
+    if (tid < 5)
         flags[tid] = 0;
-    __syncthreads();
     const int per = a.n_mgroups * GM_TM;
-    int big = 0;
-    for (int i = tid; i < 4 * per; i += 256) {
-        const int r = i / per, m = i - r * per;
-        if (m < a.M) {
-            const float rg = a.orng[i];
-            big |= !(rg <= kLooseBoundRange);
-            if (!(rg <= kProductRange))
-                flags[r] = 1;   // (every writer writes the same value)
-        }
+    int big = 0, wide[4] = {0, 0, 0, 0};
+    for (int mb = 0; mb < a.M; mb += 1024) {
+        float v[4][4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                v[u][r] = a.orng[r * per + min(mb + 256 * u + tid, a.M - 1)];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int r = 0; r < 4; ++r)
+                if (mb + 256 * u + tid < a.M) {
+                    big |= !(v[u][r] <= kLooseBoundRange);
+                    wide[r] |= !(v[u][r] <= kProductRange);
+                }
     }
-    return __syncthreads_or(big);
+    __syncthreads();
+    const bool first = (tid & 63) == 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+        if (__any(wide[r]) && first)
+            flags[r] = 1;   // (every writer writes the same value)
+    if (__any(big) && first)
+        flags[4] = 1;
+    __syncthreads();
 }
 
 // Input gradient.  Workgroup (rows_block) x: chunk of 256 pixels; y: tile of 16 * KSUB patch elements; z: split of the
@@ -856,7 +871,7 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
     __shared__ __attribute__((aligned(16))) float smem[kTile];
     __shared__ float ap[256];          // per column: the pixel's bound (0 for an empty slot)
     __shared__ float tab[2][128];      // per (region, instance of the group): omax + c0, for this group and the next
-    __shared__ int wide_sh[4];
+    __shared__ int wide_sh[5];         // per region: wide offsets range; [4]: some range beyond the loose bound's
     float *wt = smem, *eo = smem + kWt, *ot = smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -899,19 +914,16 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
     };
     if (mg_begin < mg_end)
         request(mg_begin);
-    const int roomy = rows_ranges(a, tid, wide_sh);
-    const bool my_wide = wide_sh[wave] != 0;
-    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
     // ---- the bound of every pixel: a = min over (a few) instances of outs_m - c0 - lo_m, see
-    //      mex_grad_input_mfma_kernel ----
-    const int m_scan = roomy ? a.M : min(a.M, 4);
-    float amin = INFINITY;             // of column tid
-    for (int mb = 0; mb < m_scan; mb += 32) {
+    //      mex_grad_input_mfma_kernel.  The rows of the first four instances, which give it unless some offsets
+    //      range is large, are requested before the ranges are looked at ----
+    float4 bo[8];
+    float lo_n = 0.0f;
+    auto request_bound = [&](int mb, int m_scan) {
         if (tid < 128) {
             const int m = min(mb + (tid & 31), a.M - 1);
-            tab[0][tid] = a.omax[(tid >> 5) * per + m] - a.orng[(tid >> 5) * per + m];
+            lo_n = a.omax[(tid >> 5) * per + m] - a.orng[(tid >> 5) * per + m];
         }
-        float4 bo[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int m = mb + pl0 + 4 * j;
@@ -919,6 +931,19 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
             if (q.img_ok && m < m_scan)
                 bo[j] = *reinterpret_cast<const float4 *>(ga.out + (img * a.M + m) * HW + q.pix0);
         }
+    };
+    request_bound(0, min(a.M, 4));
+    rows_ranges(a, tid, wide_sh);
+    const int roomy = wide_sh[4];
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
+    const int m_scan = roomy ? a.M : min(a.M, 4);
+    float amin = INFINITY;             // of column tid
+    for (int mb = 0; mb < m_scan; mb += 32) {
+        if (roomy)
+            request_bound(mb, m_scan);
+        if (tid < 128)
+            tab[0][tid] = lo_n;
         __syncthreads();               // tab in place; the previous block's readers are done with the tile
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -1054,14 +1079,14 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
 // rows of `out`, `g` and the input - relative to the bound over the tile's own instances, which the rows just read
 // give - and wave r adds region r's 32 x 32 products over its 64 columns.  Partial sums [chunk group][region][M][K]
 // like mex_grad_offsets_mfma_kernel's.
-__global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGradArgs ga, const RowsArgs g)
+__global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const MexGradArgs ga, const RowsArgs g)
 {
     const MexKernelArgs &a = ga.k;
     constexpr int TP = 260;
     __shared__ float wt[32 * TP];      // [instance][column]
     __shared__ float ex[32 * TP];      // [patch element][column]
     __shared__ float pm[4 * 256];      // per column: the four waves' minima
-    __shared__ int wide_sh[4];
+    __shared__ int wide_sh[5];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 15, lq = lane >> 4;
@@ -1072,9 +1097,6 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGra
     const int n_mg = a.n_mgroups, per = n_mg * GM_TM;
     const int pl0 = wave;
     const size_t HW = (size_t)g.HW;
-    rows_ranges(a, tid, wide_sh);
-    const bool my_wide = wide_sh[wave] != 0;
-    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
     // the constants of this thread's planes for its two regions (the same in every chunk)
     const RowsQuad q0 = rows_quad(a, g, 0, lane);   // (the columns and regions are the same in every chunk)
     const int rbase = q0.rbase;
@@ -1115,6 +1137,11 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGra
     const int n_steps = min(ga.pxl, ga.slots_pad / 64 - bx * ga.pxl);
     if (n_steps > 0)
         request(0);
+    rows_ranges(a, tid, wide_sh);      // (behind the requests above: one wait for everything)
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
+    // the offset exponentials of the epilogue: requested in front of the last matrix steps
+    float eov[2][2][4];
     for (int s = 0; s < n_steps; ++s) {
         const bool cur_ok = img_ok;
         float cand[4] = {INFINITY, INFINITY, INFINITY, INFINITY};
@@ -1152,8 +1179,20 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGra
                 ex[pl * TP + q0.col[e]] = use_k ? __builtin_amdgcn_exp2f(__builtin_fmaf(x[e], a.c1, -bound[e])) : 0.0f;
             }
         }
-        if (s + 1 < n_steps)
+        if (s + 1 < n_steps) {
             request(s + 1);
+        } else {
+#pragma unroll
+            for (int mt = 0; mt < 2; ++mt)
+#pragma unroll
+                for (int v = 0; v < 4; ++v) {
+                    const int m = min(m0 + mt * 16 + 4 * lq + v, a.M - 1);
+                    const float *eo = a.offe + (((size_t)wave * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
+#pragma unroll
+                    for (int kt = 0; kt < 2; ++kt)
+                        eov[mt][kt][v] = eo[(size_t)min(k0 + kt * 16 + lr, a.K - 1) * GM_TM];
+                }
+        }
         __syncthreads();
         if (!my_wide) {
 #pragma unroll 4
@@ -1175,17 +1214,6 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_rows_kernel(const MexGra
     // ---- partial sums of this chunk group: acc * 2^(os_mk - mo_m) ----
     if (!my_wide) {
         float *dst = ga.partial + ((size_t)bx * a.R + wave) * a.M * a.K;
-        float eov[2][2][4];
-#pragma unroll
-        for (int mt = 0; mt < 2; ++mt)
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int m = min(m0 + mt * 16 + 4 * lq + v, a.M - 1);
-                const float *eo = a.offe + (((size_t)wave * n_mg + m / GM_TM) * a.K) * GM_TM + m % GM_TM;
-#pragma unroll
-                for (int kt = 0; kt < 2; ++kt)
-                    eov[mt][kt][v] = eo[(size_t)min(k0 + kt * 16 + lr, a.K - 1) * GM_TM];
-            }
 #pragma unroll
         for (int mt = 0; mt < 2; ++mt)
 #pragma unroll
