@@ -31,7 +31,7 @@ EXP_RATE_MEASURED = 19.66e12  # v_exp_f32 at a quarter of the 128 lanes/clk/CU V
 # HBM bytes per launch of the dominant kernel of the headline workload, from rocprofv3 FETCH_SIZE / WRITE_SIZE runs
 # scaled by a copy kernel of known size; not measured inside this run: "traffic_source" names the committed summary.
 MEASURED_TRAFFIC = {
-    "sqrtw": (298.2e6, "profiles/sim_direct_l2_config3.md"),
+    "sqrtw": (231.8e6, "profiles/sim_direct_l2_config3.md"),
     "direct": (None, "no counter run of the current three-instruction kernel"),
     "mfma": (223.3e6, "profiles/sim_direct_l2_config3_other_forms.md"),
 }
@@ -338,6 +338,44 @@ def main():
             "bit_identical_to_direct": bool(torch.equal(got_w, out3)),
             "data": "inputs and templates ~ N(1000, 1): every wave is flagged"}
         del XA, TA, got_w
+
+        # the reference's other L2 modes at this scale (include/utils/similarity_utils.hpp:38-80): the normalisation
+        # term (half the log-weight per element, and with NaN inputs ignored only for the elements present), 25 % of the
+        # input missing, NaN beyond the border.  Priced at the functor's 6 flop per term (subtract, square, weight,
+        # halve, add the log term, accumulate); the kernels spend 4 instructions on them.
+        def sim3_mode(X, mode):
+            return lambda: pkg.similarity(X, T3, W3, similarity_function="L2", out=out3, **dict(kw3, **mode))
+
+        xn3 = x3.copy()
+        xn3[np.random.default_rng(78).random(x3.shape) < 0.25] = np.nan
+        XN3 = to_dev(xn3)
+        modes3 = {
+            "config3_L2_normalized": (x3, X3, dict(normalization_term=True)),
+            "config3_L2_normalized_ignore_nan": (xn3, XN3, dict(normalization_term=True, ignore_nan_input=True,
+                                                                out_of_bounds_value=float("nan"))),
+        }
+        for name, (_, Xm, mode) in modes3.items():
+            _, ms = timed(sim3_mode(Xm, mode), args.steps, args.warmup)
+            others[name] = entry(ms, gmac3, bytes3, "valu", flop=6)
+            others[name]["flop_per_gmac"] = 6
+            others[name]["attrs"] = {k: (str(v) if isinstance(v, float) else v) for k, v in mode.items()}
+            if "ignore_nan_input" in mode:
+                others[name]["data"] = "25 % of the input elements are NaN"
+
+        def cpu3_mode(name):
+            def job():
+                xm, Xm, mode = modes3[name]
+                n_img = 256 if threads >= 8 else 8 * threads
+                want = oracle.similarity_fwd(xm[:n_img], t3, w3, similarity_function="L2", threads=threads,
+                                             **dict(kw3, **mode))
+                got = pkg.similarity(Xm[:n_img], T3, W3, similarity_function="L2", **dict(kw3, **mode)).cpu().numpy()
+                return {"kind": "port", "sample": "%d of 256 images, %d threads: parity only, not timed" % (n_img, threads),
+                        "max_rel_err_gpu_vs_cpu": rel_err(got, want),
+                        "nan_positions_identical": bool(np.array_equal(np.isnan(got), np.isnan(want))),
+                        "nan_outputs": int(np.isnan(want).sum())}
+            return job
+        for name in modes3:
+            cpu_jobs.append((name, cpu3_mode(name)))
 
         def cpu3(func):
             def job():

@@ -233,6 +233,27 @@ def test_config3_similarity_conv_scale_sampled(pkg, func):
     assert np.array_equal(got2, got[perm])
 
 
+@pytest.mark.parametrize("ignore_nan", [False, True])
+def test_config3_similarity_normalized_modes_at_conv_scale(pkg, ignore_nan):
+    # the reference's normalised L2 functors (include/utils/similarity_utils.hpp:38-80) at the full config-3 size;
+    # with NaN inputs ignored a quarter of the input is missing and the border is NaN.  The oracle checks 16 images,
+    # NaN positions included (rel_err asserts that they coincide); the whole batch through the permutation property.
+    x, t, w, kw = config3()
+    kw = dict(kw, normalization_term=True)
+    if ignore_nan:
+        x = x.copy()
+        x[np.random.default_rng(5).random(x.shape) < 0.25] = np.nan
+        kw.update(ignore_nan_input=True, out_of_bounds_value=float("nan"))
+    got = run_similarity(pkg, x, t, w, **kw)
+    assert got.shape == (256, 128, 32, 32)
+    idx = [0, 1, 31, 32, 63, 64, 101, 127, 128, 159, 160, 191, 192, 223, 254, 255]
+    want = orc.similarity_fwd(x[idx], t, w, threads=8, **kw)
+    assert rel_err(got[idx], want) <= SIM_TOL
+    perm = np.random.default_rng(1).permutation(256)
+    got2 = run_similarity(pkg, x[perm], t, w, **kw)
+    assert np.array_equal(got2, got[perm], equal_nan=True)
+
+
 def test_config2_mex(pkg):
     x, off, n, kw = config2()
     offn = orc.normalize_offsets(off)
