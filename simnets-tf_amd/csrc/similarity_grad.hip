@@ -1294,6 +1294,143 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
     }
 }
 
+// Few templates over short patches (K <= 9 and O <= 4 * (32 / K): the first layer of the reference's networks, 32
+// templates over 2 x 2 patches of one channel), L2 modes, moment form.  The tiled kernel above would run its 64 x 128
+// (template x patch element) tile on 32 x 4 of them.  Here lanes are output pixels: a wave keeps the moments S1, S2
+// (and, with NaN inputs ignored, G) of its 32 / K templates x K patch elements in registers - at most 96 accumulators -
+// over the 64-pixel groups of its workgroup's pixel range, gathers a pixel's K patch elements once (im2col rule) and
+// reads its templates' output gradients along the pixels; at the end the lanes' sums are added by a butterfly (a
+// fixed order: reproducible) and lane 0 writes the split's partial sums in the layout the finish kernel reads.
+// a.cps: pixels per split here (a multiple of 64).
+template <int MODE, int K>
+__global__ __launch_bounds__(256) void sim_grad_params_small_kernel(const GradPArgs a)
+{
+    constexpr bool IGN = MODE == SIM_MODE_L2_NORM_IGNORE_NAN;
+    constexpr int TPW = 32 / K;   // templates per wave
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int split = blockIdx.x;
+    const int o0 = wave * TPW;
+    // centre of the moments: the mean of the wave's templates, per patch element (see sim_grad_params_kernel)
+    float ctr[K];
+    {
+        const int n = max(0, min(TPW, a.O - o0));
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < TPW; ++i)
+                if (i < n)
+                    sum += a.templates[(size_t)(o0 + i) * K + k];
+            ctr[k] = n > 0 ? sum / (float)n : 0.0f;
+        }
+    }
+    // patch element k -> channel and tap
+    int kc[K], kdh[K], kdw[K];
+    {
+        const int bhw = a.bh * a.bw;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            kc[k] = k / bhw;
+            const int rem = k - kc[k] * bhw;
+            kdh[k] = rem / a.bw;
+            kdw[k] = rem - kdh[k] * a.bw;
+        }
+    }
+    float s1[TPW][K], s2[TPW][K], gk[TPW][IGN ? K : 1];
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            s1[i][k] = 0.0f;
+            s2[i][k] = 0.0f;
+        }
+#pragma unroll
+        for (int k = 0; k < (IGN ? K : 1); ++k)
+            gk[i][k] = 0.0f;
+    }
+    const int plane = a.oh * a.ow;
+    const long long p_begin = (long long)split * a.cps, p_end = min(a.npix, p_begin + a.cps);
+    for (long long p0 = p_begin; p0 < p_end; p0 += 64) {
+        const long long p = p0 + lane;
+        const bool valid = p < p_end;
+        const long long pc = valid ? p : p_begin;
+        const int b = (int)(pc / plane), rem = (int)(pc - (long long)b * plane);
+        const int y = rem / a.ow, xw = rem - y * a.ow;
+        // (all loads first)
+        float xv[K], gv[TPW];
+        bool inside[K];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const int hi = y * a.sh - a.ph + kdh[k], wi = xw * a.sw - a.pw + kdw[k];
+            inside[k] = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+            xv[k] = a.x[inside[k] ? (((size_t)b * a.C + kc[k]) * a.H + hi) * a.W + wi : 0];
+        }
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+            gv[i] = a.g[((size_t)b * a.O + min(o0 + i, a.O - 1)) * plane + rem];
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            float x = inside[k] ? xv[k] : a.oob;
+            float keep = 1.0f;
+            if constexpr (IGN) {
+                keep = x == x ? 1.0f : 0.0f;
+                x = x == x ? x : 0.0f;
+            }
+            if (!valid) {   // a lane past the range adds nothing (and no NaN of a pixel that is not its own)
+                x = ctr[k];
+                keep = 0.0f;
+            }
+            const float xc = x - ctr[k], xc2 = xc * xc;
+#pragma unroll
+            for (int i = 0; i < TPW; ++i) {
+                float g = valid && o0 + i < a.O ? gv[i] : 0.0f;
+                if constexpr (IGN) {
+                    g *= keep;
+                    gk[i][k] += g;
+                }
+                s1[i][k] = __builtin_fmaf(g, xc, s1[i][k]);
+                s2[i][k] = __builtin_fmaf(g, xc2, s2[i][k]);
+            }
+        }
+        if constexpr (!IGN) {
+#pragma unroll
+            for (int i = 0; i < TPW; ++i)
+                gk[i][0] += valid && o0 + i < a.O ? gv[i] : 0.0f;
+        }
+    }
+    // sums over the lanes, then the split's partial sums
+    auto reduce = [](float v) {
+        for (int d = 32; d > 0; d >>= 1)
+            v += __shfl_xor(v, d, 64);
+        return v;
+    };
+    const size_t slab = (size_t)a.Opad * a.Kpad;
+    float *pt = a.partial + (size_t)split * slab;
+    float *pw = a.partial + ((size_t)a.S + split) * slab;
+    float *pn = a.partial + ((size_t)2 * a.S + split) * slab;
+#pragma unroll
+    for (int i = 0; i < TPW; ++i) {
+        const int o = o0 + i;
+#pragma unroll
+        for (int k = 0; k < K; ++k) {
+            const float r1 = reduce(s1[i][k]), r2 = reduce(s2[i][k]);
+            float rg = 0.0f;
+            if (IGN || k == 0)
+                rg = reduce(gk[i][IGN ? k : 0]);
+            if (lane == 0 && o < a.O) {
+                const size_t at = (size_t)o * a.Kpad + k;
+                pt[at] = r1;
+                pw[at] = r2;
+                if (IGN || k == 0)
+                    pn[at] = rg;
+                if (split == 0)
+                    a.partial[(size_t)3 * a.S * slab + at] = ctr[k];
+            }
+        }
+    }
+}
+
 // Adds the partial sums in a fixed order and applies the pixel-independent factors.  256 threads = E elements x
 // 256 / E groups (E = 32, or 8 when there are few elements): group j adds the splits j, j + G, ..., the group sums
 // are added in group order through LDS.
@@ -1356,6 +1493,7 @@ __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
 
 struct GpTiling {
     int WO, OWG, KWG, n_otiles, n_ktiles, Opad, Kpad, nchunks, cps, S, nacc;
+    bool small;   // few templates over short patches: sim_grad_params_small_kernel (cps: pixels per split)
     bool fast;    // unless the caller asked for the term-by-term arithmetic (algo DIRECT): moment form (L2 modes),
                   // scaled-sign form (L1)
     bool moment;  // fast and an L2 mode
@@ -1399,6 +1537,17 @@ GpTiling gp_tiling(const SimPlan &p)
         t.cps = (std::max(t.nchunks, 1) + s2 - 1) / s2;
     }
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
+    t.small = t.moment && p.K >= 1 && p.K <= 9 && p.O <= 4 * (32 / p.K);
+    if (t.small) {
+        // unpadded slabs; about 512 pixels per workgroup (eight groups of 64 per wave), at most 512 workgroups
+        t.Opad = p.O;
+        t.Kpad = p.K;
+        const long long want = std::max<long long>(1, std::min<long long>(512, npix / 512));
+        long long per = (npix + want - 1) / want;
+        per = std::max<long long>(64, (per + 63) / 64 * 64);
+        t.cps = (int)std::min<long long>(per, 0x7fffffc0LL);
+        t.S = (int)std::max<long long>(1, (npix + t.cps - 1) / t.cps);
+    }
     return t;
 }
 
@@ -1416,8 +1565,24 @@ long long gp_blocks(const GpTiling &t)
 template <int MODE>
 hipError_t gp_launch(const GradPArgs &a, const GpTiling &t, hipStream_t s)
 {
-    dim3 grid((unsigned)gp_blocks(t));
     constexpr bool L2M = MODE != SIM_MODE_L1;
+    if constexpr (L2M) {
+        if (t.small) {
+            const dim3 sgrid((unsigned)t.S);
+#define SIMNETS_GP_SMALL(KK)                                                                                  \
+    case KK:                                                                                                   \
+        hipLaunchKernelGGL((sim_grad_params_small_kernel<MODE, KK>), sgrid, dim3(256), 0, s, a);               \
+        break;
+            switch (a.K) {
+                SIMNETS_GP_SMALL(1) SIMNETS_GP_SMALL(2) SIMNETS_GP_SMALL(3) SIMNETS_GP_SMALL(4) SIMNETS_GP_SMALL(5)
+                SIMNETS_GP_SMALL(6) SIMNETS_GP_SMALL(7) SIMNETS_GP_SMALL(8) SIMNETS_GP_SMALL(9)
+            default: return hipErrorInvalidValue;
+            }
+#undef SIMNETS_GP_SMALL
+            return hipGetLastError();
+        }
+    }
+    dim3 grid((unsigned)gp_blocks(t));
     if (t.fast && L2M && a.ow % PC == 0) {
         if (t.WO == 2)
             hipLaunchKernelGGL((sim_grad_params_kernel<MODE, 2, true, L2M, L2M>), grid, dim3(kThreads), 0, s, a);
@@ -1457,7 +1622,7 @@ int sim_grad_params(const SimPlan &p, const float *input, const float *templates
     if (workspace_bytes < sim_grad_params_workspace_bytes(p))
         return SIMNETS_ERR_WORKSPACE;
     const GpTiling t = gp_tiling(p);
-    if (p.bh > 0xffff || p.bw > 0xffff || gp_blocks(t) > 0x7fffffffLL)
+    if (p.bh > 0xffff || p.bw > 0xffff || (!t.small && gp_blocks(t) > 0x7fffffffLL))
         return SIMNETS_ERR_TOO_LARGE;
     GradPArgs a;
     a.g = output_grad; a.x = input; a.templates = templates;
