@@ -276,6 +276,63 @@ int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[
                      stream);
 }
 
+// scratch of simnets_hip_mex_sum_pool_grads: the gradient kernels' workspace, then the expanded pooling gradient
+static size_t mex_pool_grads_scratch(const MexPlan &p, size_t *expanded_at)
+{
+    const size_t grads = align_up(mex_grads_workspace_bytes(p, true, true), 256);
+    *expanded_at = grads;
+    return grads + align_up((size_t)p.B * p.d.M * p.d.channels_out * p.d.height_out * p.d.width_out * sizeof(float), 256);
+}
+
+int simnets_hip_mex_sum_pool_grads_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
+                                                   int pool_w, size_t *bytes)
+{
+    if (!bytes)
+        return SIMNETS_ERR_NULL_POINTER;
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    if (pool_h <= 0 || pool_w <= 0)
+        return SIMNETS_ERR_SHAPE;
+    size_t at;
+    *bytes = mex_pool_grads_scratch(p, &at);
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                   const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                   const float *mex_output, const float *pooled_output_grad, float *input_grad,
+                                   float *offsets_grad, void *workspace, size_t workspace_bytes, void *stream)
+{
+    MexPlan p;
+    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    if (rc)
+        return rc;
+    if (pool_h <= 0 || pool_w <= 0)
+        return SIMNETS_ERR_SHAPE;
+    if (p.d.height_out / pool_h <= 0 || p.d.width_out / pool_w <= 0)
+        return SIMNETS_ERR_EMPTY_OUTPUT;
+    if (!offsets || (!offsets_grad && !input_grad) ||
+        (p.B > 0 && (!input || !mex_output || !pooled_output_grad)))
+        return SIMNETS_ERR_NULL_POINTER;
+    size_t expanded_at;
+    const size_t need = mex_pool_grads_scratch(p, &expanded_at);
+    if (!workspace_ok(workspace, workspace_bytes, need))
+        return SIMNETS_ERR_WORKSPACE;
+    if (p.B > 0 && pool_h == 2 && pool_w == 2 && mex_grads_take_pooled(p, input, mex_output, pooled_output_grad, input_grad))
+        return mex_grads(p, input, offsets, mex_output, pooled_output_grad, input_grad, offsets_grad, workspace,
+                         expanded_at, stream, true);
+    float *expanded = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + expanded_at);
+    if (p.B > 0) {
+        const int erc = sum_pool_grad_launch(p.B, p.d.M * p.d.channels_out, p.d.height_out, p.d.width_out, pool_h, pool_w,
+                                             pooled_output_grad, expanded, stream);
+        if (erc)
+            return erc;
+    }
+    return mex_grads(p, input, offsets, mex_output, expanded, input_grad, offsets_grad, workspace, expanded_at, stream);
+}
+
 static int mex_fwd_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                          const float *offsets, size_t offsets_count, float *output, void *workspace,
                          size_t workspace_bytes, void *stream, int phase)

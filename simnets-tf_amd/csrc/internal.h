@@ -73,9 +73,14 @@ size_t mex_grad_input_workspace_bytes(const MexPlan &p);
 size_t mex_grad_offsets_workspace_bytes(const MexPlan &p);
 size_t mex_grads_workspace_bytes(const MexPlan &p, bool want_input, bool want_offsets);
 // either gradient or both: a null gradient pointer skips one
+// grad_is_pooled: output_grad is the gradient of the 2 x 2 sum-pooled output (only where mex_grads_take_pooled says so)
 int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
               const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
-              size_t workspace_bytes, void *stream);
+              size_t workspace_bytes, void *stream, bool grad_is_pooled = false);
+// whether the gradient kernels of this layer read the pooled gradient themselves (the row-wise kernels on suitably
+// aligned tensors; input_grad may be null)
+bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *output, const float *pooled_grad,
+                           const float *input_grad);
 int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,
                    const float *output_grad, float *input_grad, void *workspace, size_t workspace_bytes, void *stream);
 int mex_grad_offsets(const MexPlan &p, const float *input, const float *offsets, const float *output,

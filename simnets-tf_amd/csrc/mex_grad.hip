@@ -31,6 +31,8 @@ struct MexGradArgs {
     const float *off;      // [R][M][K] offsets as the forward op used them
     const float *out;      // forward output
     const float *g;        // output gradient
+    int gpool;             // row-wise kernels: g is the gradient of the 2 x 2 sum-pooled output, [B][M][H/2][W/2]: the
+                           // gradient of output pixel (h, w) is its window's, g[h / 2][w / 2]
     float *dx;             // input gradient
     float *partial;        // offsets gradient partial sums [chunk][R][M][K]
     int overlap;           // patches overlap: the per-patch gradients go to `col`, mex_col2im_kernel adds them up
@@ -46,6 +48,21 @@ struct MexGradArgs {
     int slots_pad, Mp, Kp;
     int pxl;               // pixel slots per lane (offsets gradient)
 };
+
+// Output gradient given as the gradient of the 2 x 2 sum-pooled output (ga.gpool; one output channel per instance,
+// even height and width): plane size and the offset of output pixel `out_off`'s window.
+__device__ __forceinline__ size_t pooled_g_plane(const MexGradArgs &ga, size_t plane)
+{
+    return ga.gpool ? plane >> 2 : plane;
+}
+
+__device__ __forceinline__ int pooled_g_offset(const MexGradArgs &ga, int out_off)
+{
+    if (!ga.gpool)
+        return out_off;
+    const int h = out_off / ga.k.Wo, w = out_off - h * ga.k.Wo;
+    return (h >> 1) * (ga.k.Wo >> 1) + (w >> 1);
+}
 
 // patch element k of the pixel -> value (im2col_3d rule) and, if inside the image, its offset from the
 // image start; -1 otherwise
@@ -91,12 +108,13 @@ __device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r
             xk[j] = patch_element(a, px, k0 + j, &io[j]);
     }
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
-    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const size_t gplane = pooled_g_plane(ga, plane);
+    const float *gp = ga.g + (size_t)px.b * a.M * gplane + (valid ? pooled_g_offset(ga, px.out_off) : 0);
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float SIMNETS_CONST_AS *off = (const float SIMNETS_CONST_AS *)(ga.off) + (size_t)r * a.M * a.K + k0;
     const bool finite = a.finite_eps != 0;
     for (int m = m_begin; m < m_end; ++m) {
-        const float g = valid ? gp[(size_t)m * plane] : 0.0f;
+        const float g = valid ? gp[(size_t)m * gplane] : 0.0f;
         const float o = op[(size_t)m * plane];
 #pragma unroll
         for (int j = 0; j < GX_KT; ++j) {
@@ -522,12 +540,13 @@ __device__ __forceinline__ void mex_grad_offsets_wave(const MexGradArgs &ga, int
             ptrdiff_t unused;
             xk[j] = (k0 + j < a.K) ? patch_element(a, px, k0 + j, &unused) : 0.0f;
         }
-        const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+        const size_t gplane = pooled_g_plane(ga, plane);
+        const float *gp = ga.g + (size_t)px.b * a.M * gplane + (valid ? pooled_g_offset(ga, px.out_off) : 0);
         const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
 #pragma unroll
         for (int i = 0; i < GO_MT; ++i) {
             const bool mok = valid && m0 + i < a.M;
-            const float g = mok ? gp[(size_t)(m0 + i) * plane] : 0.0f;
+            const float g = mok ? gp[(size_t)(m0 + i) * gplane] : 0.0f;
             const float o = mok ? op[(size_t)(m0 + i) * plane] : 0.0f;
 #pragma unroll
             for (int j = 0; j < GO_KT; ++j) {
@@ -818,6 +837,28 @@ __device__ __forceinline__ RowsQuad rows_quad(const MexKernelArgs &a, const Rows
     return q;
 }
 
+// The output gradients of a thread's pixel quad for plane (img, m) as they come from memory: 16 bytes of g, or - g
+// pooled - the two window gradients the quad's row lies in (x, y; each belongs to two pixels).  rows_quad_g expands
+// them where they are used: expanding here would wait for the load where it is issued.
+__device__ __forceinline__ float4 rows_load_g(const MexGradArgs &ga, const RowsArgs &g, const RowsQuad &q, size_t img,
+                                              int m)
+{
+    if (!ga.gpool)
+        return *reinterpret_cast<const float4 *>(ga.g + (img * ga.k.M + m) * (size_t)g.HW + q.pix0);
+    const int h = q.pix0 >> g.lgW, w0 = q.pix0 & ((1 << g.lgW) - 1);
+    const float2 v = *reinterpret_cast<const float2 *>(ga.g + (img * ga.k.M + m) * (size_t)(g.HW >> 2) +
+                                                       (size_t)(h >> 1) * g.Ws + (w0 >> 1));
+    return make_float4(v.x, v.y, 0.0f, 0.0f);
+}
+
+__device__ __forceinline__ void rows_quad_g(const MexGradArgs &ga, const float4 &v, float (&gg)[4])
+{
+    gg[0] = v.x;
+    gg[1] = ga.gpool ? v.x : v.y;
+    gg[2] = ga.gpool ? v.y : v.z;
+    gg[3] = ga.gpool ? v.y : v.w;
+}
+
 // per region: does some instance's offsets range exceed the product form's (flags[r]); flags[4]: does some range
 // exceed kLooseBoundRange.  All threads of the workgroup call it; the flags are in place behind its last barrier.
 // (All loads go out before the first is looked at.)
@@ -897,9 +938,8 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int m = min(mg * GM_TM + pl0 + 4 * j, a.M - 1);
-            const size_t at = (img * a.M + m) * HW + q.pix0;
-            ov[j] = *reinterpret_cast<const float4 *>(ga.out + at);
-            gv[j] = *reinterpret_cast<const float4 *>(ga.g + at);
+            ov[j] = *reinterpret_cast<const float4 *>(ga.out + (img * a.M + m) * HW + q.pix0);
+            gv[j] = rows_load_g(ga, g, q, img, m);
         }
 #pragma unroll
         for (int j = 0; j < 2 * KSUB; ++j) {
@@ -985,7 +1025,8 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
             const int pl = pl0 + 4 * j;
             const bool use = q.img_ok && mg * GM_TM + pl < a.M;
             const float o[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
-            const float gg[4] = {gv[j].x, gv[j].y, gv[j].z, gv[j].w};
+            float gg[4];
+            rows_quad_g(ga, gv[j], gg);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
@@ -1127,9 +1168,8 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int m = min(m0 + pl0 + 4 * j, a.M - 1), k = min(k0 + pl0 + 4 * j, a.K - 1);
-            const size_t at = (img * a.M + m) * HW + q.pix0;
-            ov[j] = *reinterpret_cast<const float4 *>(ga.out + at);
-            gv[j] = *reinterpret_cast<const float4 *>(ga.g + at);
+            ov[j] = *reinterpret_cast<const float4 *>(ga.out + (img * a.M + m) * HW + q.pix0);
+            gv[j] = rows_load_g(ga, g, q, img, m);
             xv[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + k) * HW + q.pix0);
         }
     };
@@ -1170,7 +1210,8 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
             const int pl = pl0 + 4 * j;
             const bool use_m = cur_ok && m0 + pl < a.M, use_k = cur_ok && k0 + pl < a.K;
             const float o[4] = {ov[j].x, ov[j].y, ov[j].z, ov[j].w};
-            const float gg[4] = {gv[j].x, gv[j].y, gv[j].z, gv[j].w};
+            float gg[4];
+            rows_quad_g(ga, gv[j], gg);
             const float x[4] = {xv[j].x, xv[j].y, xv[j].z, xv[j].w};
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
@@ -1602,9 +1643,17 @@ size_t mex_grad_offsets_workspace_bytes(const MexPlan &p) { return mex_grads_wor
 
 // Either gradient or both (a null pointer skips one).  The offsets as the forward op used them, their packed form
 // and, where used, the factor buffers are prepared once and shared.
+bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *output, const float *pooled_grad,
+                           const float *input_grad)
+{
+    auto aligned = [](const void *q, uintptr_t a) { return (reinterpret_cast<uintptr_t>(q) & (a - 1)) == 0; };
+    return std::isfinite(p.epsilon) && rows_geometry(p) && aligned(input, 16) && aligned(output, 16) &&
+           aligned(pooled_grad, 8) && (input_grad == nullptr || aligned(input_grad, 16));
+}
+
 int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
               const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
-              size_t workspace_bytes, void *stream)
+              size_t workspace_bytes, void *stream, bool grad_is_pooled)
 {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const bool want_input = input_grad != nullptr, want_offsets = offsets_grad != nullptr;
@@ -1641,6 +1690,7 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     if (rc)
         return rc;
     ga.out = output; ga.g = output_grad;
+    ga.gpool = grad_is_pooled ? 1 : 0;
     ga.dx = input_grad;
     ga.partial = reinterpret_cast<float *>(ws + w.partial);
     ga.overlap = 0;
@@ -1652,8 +1702,11 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     ga.cpr = (ga.k.slots + 63) / 64;
     // the row-wise kernels read and write 16 bytes at a time
     auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-    const bool use_rows = t.mfma && t.rows && aligned16(input) && aligned16(output) && aligned16(output_grad) &&
-                          (!want_input || aligned16(input_grad));
+    const bool use_rows = grad_is_pooled ||
+                          (t.mfma && t.rows && aligned16(input) && aligned16(output) && aligned16(output_grad) &&
+                           (!want_input || aligned16(input_grad)));
+    if (grad_is_pooled && !mex_grads_take_pooled(p, input, output, output_grad, input_grad))
+        return SIMNETS_ERR_ALGO;   // (the callers ask first)
     if (t.mfma) {
         rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream, nullptr, true,
                               pack_normalizes ? reinterpret_cast<float *>(ws + w.norm) : nullptr);

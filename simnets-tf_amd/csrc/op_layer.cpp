@@ -415,6 +415,36 @@ std::tuple<at::Tensor, at::Tensor> mex_sum_pool_both_call(const simnets_mex_attr
     return {full, y};
 }
 
+// the gradients of that pair from the gradient of the pooled output; a gradient that is not wanted is an undefined tensor
+std::tuple<at::Tensor, at::Tensor> mex_sum_pool_grads_call(const simnets_mex_attrs &a, const at::Tensor &input,
+                                                           const at::Tensor &offsets, const at::Tensor &mex_output,
+                                                           const at::Tensor &pooled_grad, int ph, int pw,
+                                                           bool want_input, bool want_offsets)
+{
+    const at::Tensor x = dense("input", input), off = dense("offsets", offsets), y = dense("mex_output", mex_output),
+                     g = dense("pooled_output_grad", pooled_grad);
+    const Shape4 xs = shape4(x);
+    int os[4];
+    check(simnets_mex_out_shape(&a, xs.v, os, nullptr));
+    if (ph <= 0 || pw <= 0)
+        throw SimnetsStatus(SIMNETS_ERR_SHAPE);
+    const int ps[4] = {os[0], os[1], os[2] / ph, os[3] / pw};
+    for (int i = 0; i < 4; ++i)
+        if (y.dim() != 4 || g.dim() != 4 || y.size(i) != os[i] || g.size(i) != ps[i])
+            throw SimnetsStatus(SIMNETS_ERR_SHAPE);
+    if (!want_input && !want_offsets)
+        return {at::Tensor(), at::Tensor()};
+    size_t nbytes = 0;
+    check(simnets_hip_mex_sum_pool_grads_workspace_bytes(&a, xs.v, ph, pw, &nbytes));
+    at::Tensor dx = want_input ? at::empty_like(x) : at::Tensor(), doff = want_offsets ? at::empty_like(off) : at::Tensor();
+    Launch l(x);
+    const auto wsp = l.workspace(nbytes, x);
+    check(simnets_hip_mex_sum_pool_grads(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ph, pw, ptr(y), ptr(g),
+                                         want_input ? ptr(dx) : nullptr, want_offsets ? ptr(doff) : nullptr, wsp.first,
+                                         wsp.second, l.stream));
+    return {dx, doff};
+}
+
 at::Tensor similarity_mex_sum_pool_call(const simnets_similarity_attrs &sa, const simnets_mex_attrs &ma,
                                         const at::Tensor &input, const at::Tensor &templates, const at::Tensor &weights,
                                         const at::Tensor &offsets, int ph, int pw, const c10::optional<at::Tensor> &out)
@@ -770,6 +800,15 @@ PYBIND11_MODULE(_simnets_native, m)
               return mex_sum_pool_both_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down,
                                                          unshared, shared_region, unshared_region, normalize),
                                             x, off, ph, pw);
+          });
+    m.def("mex_sum_pool_grads",
+          [](const at::Tensor &x, const at::Tensor &off, const at::Tensor &full, const at::Tensor &g, int n, int ph, int pw,
+             bool want_input, bool want_offsets, py::object softmax, py::object padding, py::object strides,
+             py::object blocks, py::object epsilon, py::object oob, py::object round_down, py::object unshared,
+             py::object shared_region, py::object unshared_region, bool normalize) {
+              return mex_sum_pool_grads_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down,
+                                                          unshared, shared_region, unshared_region, normalize),
+                                             x, off, full, g, ph, pw, want_input, want_offsets);
           });
     // the attribute structs of the two-operator calls come from Python as dicts of keyword arguments
     auto sim_from_dict = [](const py::dict &d) {

@@ -1302,6 +1302,7 @@ __global__ __launch_bounds__(kThreads, 2) void sim_grad_params_kernel(const Grad
 // reads its templates' output gradients along the pixels; at the end the lanes' sums are added by a butterfly (a
 // fixed order: reproducible) and lane 0 writes the split's partial sums in the layout the finish kernel reads.
 // a.cps: pixels per split here (a multiple of 64).
+constexpr int kGpSmallGroups = 4;   // groups of 64 pixels whose loads are in flight together
 template <int MODE, int K>
 __global__ __launch_bounds__(256) void sim_grad_params_small_kernel(const GradPArgs a)
 {
@@ -1317,11 +1318,16 @@ __global__ __launch_bounds__(256) void sim_grad_params_small_kernel(const GradPA
         const int n = max(0, min(TPW, a.O - o0));
 #pragma unroll
         for (int k = 0; k < K; ++k) {
+            // (all loads first, those past the last template on a clamped address: a load inside the condition would
+            // be waited for before the next one is issued)
+            float tv[TPW];
+#pragma unroll
+            for (int i = 0; i < TPW; ++i)
+                tv[i] = a.templates[(size_t)min(o0 + i, a.O - 1) * K + k];
             float sum = 0.0f;
 #pragma unroll
             for (int i = 0; i < TPW; ++i)
-                if (i < n)
-                    sum += a.templates[(size_t)(o0 + i) * K + k];
+                sum += i < n ? tv[i] : 0.0f;
             ctr[k] = n > 0 ? sum / (float)n : 0.0f;
         }
     }
@@ -1350,84 +1356,127 @@ __global__ __launch_bounds__(256) void sim_grad_params_small_kernel(const GradPA
             gk[i][k] = 0.0f;
     }
     const int plane = a.oh * a.ow;
-    const long long p_begin = (long long)split * a.cps, p_end = min(a.npix, p_begin + a.cps);
-    for (long long p0 = p_begin; p0 < p_end; p0 += 64) {
-        const long long p = p0 + lane;
-        const bool valid = p < p_end;
-        const long long pc = valid ? p : p_begin;
-        const int b = (int)(pc / plane), rem = (int)(pc - (long long)b * plane);
-        const int y = rem / a.ow, xw = rem - y * a.ow;
-        // (all loads first)
-        float xv[K], gv[TPW];
-        bool inside[K];
+    // (pixel numbers fit 32 bits: checked by the host)
+    const unsigned p_begin = (unsigned)split * (unsigned)a.cps, p_end = min((unsigned)a.npix, p_begin + (unsigned)a.cps);
+    // groups of 64 pixels, kGpSmallGroups at a time: all their loads go out before the first value is used (a group
+    // is a dozen loads and a hundred fused multiply-adds: one memory round trip per group would be the kernel's time)
+    for (unsigned pg = p_begin; pg < p_end; pg += 64 * kGpSmallGroups) {
+        float xv[kGpSmallGroups][K], gv[kGpSmallGroups][TPW];
+        bool inside[kGpSmallGroups][K], valid[kGpSmallGroups];
 #pragma unroll
-        for (int k = 0; k < K; ++k) {
-            const int hi = y * a.sh - a.ph + kdh[k], wi = xw * a.sw - a.pw + kdw[k];
-            inside[k] = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
-            xv[k] = a.x[inside[k] ? (((size_t)b * a.C + kc[k]) * a.H + hi) * a.W + wi : 0];
-        }
+        for (int u = 0; u < kGpSmallGroups; ++u) {
+            const unsigned p = pg + 64 * u + lane;
+            valid[u] = p < p_end;
+            const unsigned pc = valid[u] ? p : p_begin;
+            const int b = (int)(pc / (unsigned)plane), rem = (int)(pc - (unsigned)b * (unsigned)plane);
+            const int y = (int)((unsigned)rem / (unsigned)a.ow), xw = rem - y * a.ow;
 #pragma unroll
-        for (int i = 0; i < TPW; ++i)
-            gv[i] = a.g[((size_t)b * a.O + min(o0 + i, a.O - 1)) * plane + rem];
-#pragma unroll
-        for (int k = 0; k < K; ++k) {
-            float x = inside[k] ? xv[k] : a.oob;
-            float keep = 1.0f;
-            if constexpr (IGN) {
-                keep = x == x ? 1.0f : 0.0f;
-                x = x == x ? x : 0.0f;
+            for (int k = 0; k < K; ++k) {
+                const int hi = y * a.sh - a.ph + kdh[k], wi = xw * a.sw - a.pw + kdw[k];
+                inside[u][k] = hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+                xv[u][k] = a.x[inside[u][k] ? (((size_t)b * a.C + kc[k]) * a.H + hi) * a.W + wi : 0];
             }
-            if (!valid) {   // a lane past the range adds nothing (and no NaN of a pixel that is not its own)
-                x = ctr[k];
-                keep = 0.0f;
-            }
-            const float xc = x - ctr[k], xc2 = xc * xc;
-#pragma unroll
-            for (int i = 0; i < TPW; ++i) {
-                float g = valid && o0 + i < a.O ? gv[i] : 0.0f;
-                if constexpr (IGN) {
-                    g *= keep;
-                    gk[i][k] += g;
-                }
-                s1[i][k] = __builtin_fmaf(g, xc, s1[i][k]);
-                s2[i][k] = __builtin_fmaf(g, xc2, s2[i][k]);
-            }
-        }
-        if constexpr (!IGN) {
 #pragma unroll
             for (int i = 0; i < TPW; ++i)
-                gk[i][0] += valid && o0 + i < a.O ? gv[i] : 0.0f;
+                gv[u][i] = a.g[((size_t)b * a.O + min(o0 + i, a.O - 1)) * plane + rem];
+        }
+#pragma unroll
+        for (int u = 0; u < kGpSmallGroups; ++u) {
+#pragma unroll
+            for (int k = 0; k < K; ++k) {
+                float x = inside[u][k] ? xv[u][k] : a.oob;
+                float keep = 1.0f;
+                if constexpr (IGN) {
+                    keep = x == x ? 1.0f : 0.0f;
+                    x = x == x ? x : 0.0f;
+                }
+                if (!valid[u]) {   // a lane past the range adds nothing (and no NaN of a pixel that is not its own)
+                    x = ctr[k];
+                    keep = 0.0f;
+                }
+                const float xc = x - ctr[k], xc2 = xc * xc;
+#pragma unroll
+                for (int i = 0; i < TPW; ++i) {
+                    float g = valid[u] && o0 + i < a.O ? gv[u][i] : 0.0f;
+                    if constexpr (IGN) {
+                        g *= keep;
+                        gk[i][k] += g;
+                    }
+                    s1[i][k] = __builtin_fmaf(g, xc, s1[i][k]);
+                    s2[i][k] = __builtin_fmaf(g, xc2, s2[i][k]);
+                }
+            }
+            if constexpr (!IGN) {
+#pragma unroll
+                for (int i = 0; i < TPW; ++i)
+                    gk[i][0] += valid[u] && o0 + i < a.O ? gv[u][i] : 0.0f;
+            }
         }
     }
-    // sums over the lanes, then the split's partial sums
-    auto reduce = [](float v) {
-        for (int d = 32; d > 0; d >>= 1)
-            v += __shfl_xor(v, d, 64);
-        return v;
+    // Sums over the lanes, in a fixed order, through the data-parallel-primitive lane patterns (neighbour, pair,
+    // half-row mirror, row mirror: every lane then holds its 16-lane row's sum) and four lane reads for the rows -
+    // all accumulators stage by stage, so that the stages' latencies overlap -, then the split's partial sums.
+    auto dpp = [](float v, auto ctrl) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), decltype(ctrl)::value,
+                                                                      0xF, 0xF, false));
     };
+    auto lane_of = [](float v, int l) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+    };
+    using std::integral_constant;
+    auto wave_sum = [&](auto &arr, auto nk) {
+        constexpr int NK = decltype(nk)::value;
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int k = 0; k < NK; ++k) arr[i][k] += dpp(arr[i][k], integral_constant<int, 0xB1>{});
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int k = 0; k < NK; ++k) arr[i][k] += dpp(arr[i][k], integral_constant<int, 0x4E>{});
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int k = 0; k < NK; ++k) arr[i][k] += dpp(arr[i][k], integral_constant<int, 0x141>{});
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int k = 0; k < NK; ++k) arr[i][k] += dpp(arr[i][k], integral_constant<int, 0x140>{});
+#pragma unroll
+        for (int i = 0; i < TPW; ++i)
+#pragma unroll
+            for (int k = 0; k < NK; ++k)
+                arr[i][k] = (lane_of(arr[i][k], 0) + lane_of(arr[i][k], 16)) + (lane_of(arr[i][k], 32) + lane_of(arr[i][k], 48));
+    };
+    wave_sum(s1, integral_constant<int, K>{});
+    wave_sum(s2, integral_constant<int, K>{});
+    wave_sum(gk, integral_constant<int, IGN ? K : 1>{});
+    // every lane holds all sums now: lane j keeps pair j = (template j / K, element j % K) and the wave writes each
+    // array with one store (the slabs are unpadded here: a.Kpad = K, so the wave's pairs are consecutive floats)
     const size_t slab = (size_t)a.Opad * a.Kpad;
     float *pt = a.partial + (size_t)split * slab;
     float *pw = a.partial + ((size_t)a.S + split) * slab;
     float *pn = a.partial + ((size_t)2 * a.S + split) * slab;
+    float m1 = 0.0f, m2 = 0.0f, mg = 0.0f, mc = 0.0f;
 #pragma unroll
-    for (int i = 0; i < TPW; ++i) {
-        const int o = o0 + i;
+    for (int i = 0; i < TPW; ++i)
 #pragma unroll
         for (int k = 0; k < K; ++k) {
-            const float r1 = reduce(s1[i][k]), r2 = reduce(s2[i][k]);
-            float rg = 0.0f;
-            if (IGN || k == 0)
-                rg = reduce(gk[i][IGN ? k : 0]);
-            if (lane == 0 && o < a.O) {
-                const size_t at = (size_t)o * a.Kpad + k;
-                pt[at] = r1;
-                pw[at] = r2;
-                if (IGN || k == 0)
-                    pn[at] = rg;
-                if (split == 0)
-                    a.partial[(size_t)3 * a.S * slab + at] = ctr[k];
-            }
+            const bool me = lane == i * K + k;
+            m1 = me ? s1[i][k] : m1;
+            m2 = me ? s2[i][k] : m2;
+            mg = me ? gk[i][IGN ? k : 0] : mg;
+            mc = me ? ctr[k] : mc;
         }
+    const int my_o = o0 + lane / K, my_k = lane % K;
+    if (lane < TPW * K && my_o < a.O) {
+        const size_t at = (size_t)my_o * a.Kpad + my_k;
+        pt[at] = m1;
+        pw[at] = m2;
+        if (IGN || my_k == 0)
+            pn[at] = mg;
+        if (split == 0)
+            a.partial[(size_t)3 * a.S * slab + at] = mc;
     }
 }
 
@@ -1537,12 +1586,13 @@ GpTiling gp_tiling(const SimPlan &p)
         t.cps = (std::max(t.nchunks, 1) + s2 - 1) / s2;
     }
     t.nacc = (t.moment || p.mode == SIM_MODE_L2_NORM || p.mode == SIM_MODE_L2_NORM_IGNORE_NAN) ? 3 : 2;
-    t.small = t.moment && p.K >= 1 && p.K <= 9 && p.O <= 4 * (32 / p.K);
+    t.small = t.moment && p.K >= 1 && p.K <= 9 && p.O <= 4 * (32 / p.K) && npix < 0x7fffffffLL;
     if (t.small) {
-        // unpadded slabs; about 512 pixels per workgroup (eight groups of 64 per wave), at most 512 workgroups
+        // unpadded slabs; about 256 pixels per workgroup (one round of four groups of 64 per wave), at most 1024
+        // workgroups
         t.Opad = p.O;
         t.Kpad = p.K;
-        const long long want = std::max<long long>(1, std::min<long long>(512, npix / 512));
+        const long long want = std::max<long long>(1, std::min<long long>(1024, npix / 256));
         long long per = (npix + want - 1) / want;
         per = std::max<long long>(64, (per + 63) / 64 * 64);
         t.cps = (int)std::min<long long>(per, 0x7fffffc0LL);

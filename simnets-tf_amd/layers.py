@@ -78,14 +78,9 @@ class MexSumPoolFunction(torch.autograd.Function):
     @staticmethod
     def backward(ctx, grad):
         input, offsets, full = ctx.saved_tensors
-        g = ops.sum_pooling_input_grad(grad.contiguous(), full.shape, ctx.pool)
-        gi = go = None
-        if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
-            gi, go = ops.mex_grads(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
-        elif ctx.needs_input_grad[0]:
-            gi = ops.mex_input_grad(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
-        elif ctx.needs_input_grad[1]:
-            go = ops.mex_offsets_grad(input, offsets, full, g, ctx.num_instances, **ctx.attrs)
+        gi, go = ops.mex_sum_pool_grads(input, offsets, full, grad.contiguous(), ctx.num_instances, ctx.pool,
+                                        want_input=ctx.needs_input_grad[0], want_offsets=ctx.needs_input_grad[1],
+                                        **ctx.attrs)
         return gi, go, None, None, None, None
 
 

@@ -283,6 +283,21 @@ def mex_sum_pool_both(input, offsets, num_instances, pool_size=(2, 2), softmax_m
                                 bool(normalize_offsets))
 
 
+def mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, num_instances, pool_size=(2, 2), want_input=True,
+                       want_offsets=True, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
+                       blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
+                       shared_offset_region=None, unshared_offset_region=None, name=None, normalize_offsets=False):
+    """The gradients of `mex_sum_pool` w.r.t. (input, offsets) from the gradient of the POOLED output and the MEX
+    output before pooling (`mex_sum_pool_both`'s first result): `mex_grads(input, offsets, mex_output,
+    sum_pooling_input_grad(pooled_output_grad, ...))` in one call, without the expanded gradient tensor on the layers
+    of the reference's networks.  A gradient that is not wanted comes back as None."""
+    gi, go = _n.mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, int(num_instances), int(pool_size[0]),
+                                   int(pool_size[1]), bool(want_input), bool(want_offsets), softmax_mode, padding, strides,
+                                   blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions,
+                                   shared_offset_region, unshared_offset_region, bool(normalize_offsets))
+    return (gi if want_input else None), (go if want_offsets else None)
+
+
 def similarity_mex_sum_pool(input, templates, weights, offsets, num_instances, pool_size=(2, 2), similarity=None,
                             mex=None, out=None):
     """`sum_pooling(mex(similarity(input, templates, weights, **similarity), offsets, num_instances, **mex), pool_size)`

@@ -242,6 +242,52 @@ def test_mex_sum_pool_for_training_keeps_the_mex_output(pkg, case, spread):
         assert float((a - b).abs().max()) <= 1e-4 * float(b.abs().max())
 
 
+@pytest.mark.parametrize("spread", ["narrow", "mixed"])
+@pytest.mark.parametrize("im,n,pool,kw", [
+    ((5, 32, 16, 16), 64, (2, 2), {}),                      # row-wise kernels read the window gradients themselves
+    ((9, 40, 8, 8), 70, (2, 2), {}),                        # ... ragged blocks, part-empty last chunk
+    ((17, 16, 4, 4), 33, (2, 2), {}),                       # ... sixteen images a chunk
+    ((3, 8, 4, 32), 6, (2, 2), {}),
+    ((3, 12, 6, 10), 5, (2, 2), {}),                        # map sides no powers of two: expanded gradient
+    ((2, 6, 9, 8), 4, (3, 2), {}),                          # 3 x 2 windows, a row left over
+    ((4, 6, 8, 8), 5, (2, 2), dict(unshared_offset_region=[1, 4, 4])),   # window is not the region grid
+    ((3, 16, 8, 8), 7, (2, 2), dict(epsilon=float("inf"))),
+])
+def test_mex_sum_pool_grads_from_the_pooled_gradient(pkg, im, n, pool, kw, spread):
+    """`mex_sum_pool_grads` = `mex_grads` on the expanded pooling gradient, bit for bit - whether the gradient kernels
+    read the window gradients themselves or the call expands them first -, for both gradients, either alone, and
+    through unaligned views."""
+    g = torch.Generator(device="cuda").manual_seed(21)
+    kw = dict(dict(softmax_mode=True, blocks=[im[1], 1, 1], strides=[im[1], 1, 1],
+                   unshared_offset_region=[1, pool[0], pool[1]], epsilon=1.5, normalize_offsets=True), **kw)
+    x = torch.randn(im, device="cuda", generator=g)
+    _, oshape = pkg.mex_output_shape(im, n, **{k: v for k, v in kw.items() if k != "normalize_offsets"})
+    off = torch.randn(oshape, device="cuda", generator=g) * 0.3
+    if spread == "mixed":
+        off[::2] *= 300
+    full, pooled = pkg.mex_sum_pool_both(x, off, n, pool, **kw)
+    gp = torch.randn(pooled.shape, device="cuda", generator=g)
+    want_dx, want_doff = pkg.mex_grads(x, off, full, pkg.sum_pooling_input_grad(gp, full.shape, pool), n, **kw)
+    dx, doff = pkg.mex_sum_pool_grads(x, off, full, gp, n, pool, **kw)
+    assert torch.equal(dx, want_dx) and torch.equal(doff, want_doff)
+    only_dx, none = pkg.mex_sum_pool_grads(x, off, full, gp, n, pool, want_offsets=False, **kw)
+    assert none is None and torch.equal(only_dx, want_dx)
+    none, only_doff = pkg.mex_sum_pool_grads(x, off, full, gp, n, pool, want_input=False, **kw)
+    assert none is None and torch.equal(only_doff, want_doff)
+
+    def shifted(t):
+        buf = torch.empty(t.numel() + 1, device="cuda")
+        v = buf[1:].view(t.shape)
+        v.copy_(t)
+        return v
+
+    dx_u, doff_u = pkg.mex_sum_pool_grads(shifted(x), off, shifted(full), shifted(gp), n, pool, **kw)
+    assert float((dx_u - want_dx).abs().max()) <= 1e-4 * float(want_dx.abs().max())
+    assert float((doff_u - want_doff).abs().max()) <= 1e-4 * float(want_doff.abs().max())
+    with pytest.raises(pkg.SimnetsError):
+        pkg.mex_sum_pool_grads(x, off, full, gp[:, :, :-1], n, pool, **kw)
+
+
 @pytest.mark.parametrize("shape,pool", [((3, 5, 8, 10), (2, 2)), ((2, 3, 7, 9), (2, 3)), ((1, 4, 5, 5), (5, 1))])
 def test_sum_pooling_gradient(pkg, shape, pool):
     """layers.sum_pooling: forward = avg_pool2d * area ('valid': trailing rows/columns dropped), the gradient spreads
