@@ -587,6 +587,8 @@ def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, sp
     ((2, 8, 32, 64), 6),       # eight chunks an image, four rows each
     ((1, 5, 8, 128), 3),       # widest map the row-wise kernel takes: two rows a chunk
     ((2, 4, 4, 256), 3),       # wider: the gathering factors kernel
+    ((70, 24, 2, 2), 40),      # width 2: below the row-wise kernels' widths (their 16-byte pieces would be one per image)
+    ((5, 8, 8, 2), 6),
 ])
 def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
     """2 x 2 unshared offsets over whole-channel patches on maps with power-of-two sides: the pixel factors and patch

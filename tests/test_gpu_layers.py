@@ -248,6 +248,8 @@ def test_mex_sum_pool_for_training_keeps_the_mex_output(pkg, case, spread):
     ((9, 40, 8, 8), 70, (2, 2), {}),                        # ... ragged blocks, part-empty last chunk
     ((17, 16, 4, 4), 33, (2, 2), {}),                       # ... sixteen images a chunk
     ((3, 8, 4, 32), 6, (2, 2), {}),
+    ((70, 16, 2, 2), 20, (2, 2), {}),                       # width 2: expanded gradient, gathering kernels
+    ((6, 8, 8, 2), 5, (2, 2), {}),
     ((3, 12, 6, 10), 5, (2, 2), {}),                        # map sides no powers of two: expanded gradient
     ((2, 6, 9, 8), 4, (3, 2), {}),                          # 3 x 2 windows, a row left over
     ((4, 6, 8, 8), 5, (2, 2), dict(unshared_offset_region=[1, 4, 4])),   # window is not the region grid
