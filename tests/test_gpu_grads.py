@@ -621,6 +621,37 @@ def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
     assert float((doff - doff_u).abs().max()) <= 1e-4 * scale_o
 
 
+@pytest.mark.parametrize("eps", [1.0, -2.5, math.inf, -math.inf])
+@pytest.mark.parametrize("case", [
+    dict(im=(37, 512, 1, 1), n=10, kw=dict(blocks=[512, 1, 1], strides=[512, 1, 1], padding=[0, 0, 0],
+                                           use_unshared_regions=False, shared_offset_region=[-1])),   # classifier head
+    dict(im=(9, 100, 2, 2), n=13, kw=dict(blocks=[100, 1, 1], strides=[100, 1, 1], padding=[0, 0, 0],
+                                          unshared_offset_region=[2])),              # four regions, ragged K
+    dict(im=(3, 20, 5, 4), n=6, kw=dict(blocks=[20, 2, 2], strides=[20, 1, 1], padding=[0, 1, 0],
+                                        use_unshared_regions=False, shared_offset_region=[2])),   # overlapping patches, padding
+    dict(im=(2, 1000, 1, 3), n=4, kw=dict(blocks=[1000, 1, 1], strides=[1000, 1, 1], padding=[0, 0, 0],
+                                          use_unshared_regions=False, shared_offset_region=[1, 1, 2])),   # 16 elements a lane
+])
+def test_mex_grads_few_pixels_long_patches_few_instances(pkg, case, eps):
+    """Few pixels, 64 <= K <= 1024, few instances (the classifier head of the reference's networks, where the forward
+    pass runs its wave-per-pixel kernel): both gradients against the oracle for either epsilon; with the offsets
+    normalisation one call for both equals the two separate calls bit for bit and every row of the offsets gradient
+    sums to zero."""
+    kw = dict(case["kw"], epsilon=eps, softmax_mode=True)
+    x, off = mex_case(91, case["im"], case["n"], **kw)
+    check_mex_grads(pkg, x, off * 0.5, case["n"], **kw)
+    kwn = dict(kw, normalize_offsets=True)
+    X, O = dev(x), dev(off)
+    Y = pkg.mex(X, O, case["n"], **kwn)
+    G = torch.randn_like(Y)
+    dx, doff = pkg.mex_grads(X, O, Y, G, case["n"], **kwn)
+    assert torch.equal(dx, pkg.mex_input_grad(X, O, Y, G, case["n"], **kwn))
+    assert torch.equal(doff, pkg.mex_offsets_grad(X, O, Y, G, case["n"], **kwn))
+    # the sum of an instance's offsets gradient vanishes under the normalisation (d/do of o - logsumexp(o))
+    rows = doff.reshape(doff.shape[0], doff.shape[1], -1)
+    assert float(rows.sum(-1).abs().max()) <= 1e-3 * max(1.0, float(rows.abs().max()))
+
+
 @pytest.mark.parametrize("case", [
     dict(im=(5, 40, 6, 6), n=70, kw=dict(blocks=[40, 1, 1], strides=[40, 1, 1], padding=[0, 0, 0],
                                          unshared_offset_region=[2], epsilon=2.0, softmax_mode=True)),
