@@ -586,6 +586,7 @@ def test_mex_grads_many_instances_and_patch_elements_on_a_small_map(pkg, eps, sp
     ((3, 12, 2, 8), 5),        # two rows
     ((2, 8, 32, 64), 6),       # eight chunks an image, four rows each
     ((1, 5, 8, 128), 3),       # widest map the row-wise kernel takes: two rows a chunk
+    ((6, 24, 4, 4), 140),      # few pixels, five instance groups: the input gradient splits them over workgroups
     ((2, 4, 4, 256), 3),       # wider: the gathering factors kernel
     ((70, 24, 2, 2), 40),      # width 2: below the row-wise kernels' widths (their 16-byte pieces would be one per image)
     ((5, 8, 8, 2), 6),
@@ -619,6 +620,15 @@ def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
     scale_x, scale_o = float(dx.abs().max()), float(doff.abs().max())
     assert float((dx - dx_u).abs().max()) <= 1e-4 * scale_x
     assert float((doff - doff_u).abs().max()) <= 1e-4 * scale_o
+
+
+def test_mex_grads_row_wise_kernels_on_a_large_batch(pkg):
+    """512 chunks of 256 pixels and 64 channels: the input gradient takes 64 patch elements per workgroup."""
+    im, n = (512, 64, 16, 16), 4
+    kw = dict(blocks=[64, 1, 1], strides=[64, 1, 1], padding=[0, 0, 0], unshared_offset_region=[2], epsilon=1.0,
+              softmax_mode=True)
+    x, off = mex_case(72, im, n, **kw)
+    check_mex_grads(pkg, x, off * 0.5, n, **kw)
 
 
 @pytest.mark.parametrize("eps", [1.0, -2.5, math.inf, -math.inf])
