@@ -157,10 +157,15 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
 // 2^-range: d patch_k = 2^(xs_k - a) * sum_m W_m EO_mk is a GEMM over the instances (v_mfma_f32_16x16x4_f32 tiles:
 // 16 patch elements x 16 pixels x 4 instances) of the pixel factors W (computed from g and out, which the kernel
 // reads anyway: no pass over the patches is needed for the bound) with the packed offset exponentials EO of the
-// forward pass.  Used when every instance of the region has an offsets range of at most kProductRange; otherwise the
+// forward pass.  Used when every instance of the region has an offsets range of at most kGradProductRange; otherwise the
 // workgroup falls back to the term-by-term waves.
 // grid.x: (region, pixel chunk of 64 slots); grid.y: tile of GM_KT patch elements (16 per wave)
 constexpr int GM_TM = 32;   // instances per packed group = contraction chunk
+// Widest offsets range (an exponent of two) the gradients' product form takes.  Its factors 2^(xs - a), 2^(os - mo) and W
+// carry exponents of up to the range, each rounded once: an error of ulp(range) in an exponent is a relative error of
+// about 4e-8 * range in the factor, and measured against the fp64 oracle the gradients stay within the 1e-4 bar up to
+// ranges of about 35 (7e-5 there, 1.7e-4 at 50); the forward pass's 90 is a bound against overflow, not this one.
+constexpr float kGradProductRange = 32.0f;
 constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) up to which a few instances give the bound
 constexpr int GM_KT = 64;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -169,7 +174,7 @@ typedef float floatx4 __attribute__((ext_vector_type(4)));
 // (region, chunk) the bound a, W_m = g_m 2^(a + mo_m - outs_m + c0) for every instance and 2^(xs_k - a) for every
 // patch element, written as rows [slot][Mp] and [slot][Kp] (through LDS, so that the stores run along the rows);
 // a workgroup forms one block of 32 instances or 32 patch elements (grid.y), each from the same bound.
-// Regions with an offsets range beyond kProductRange are left alone: the matrix kernels fall back to the
+// Regions with an offsets range beyond kGradProductRange are left alone: the matrix kernels fall back to the
 // term-by-term waves there and never look at the buffers.
 __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs ga)
 {
@@ -185,7 +190,7 @@ __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs
     const float *omax_r = a.omax + (size_t)r * n_mg * GM_TM, *orng_r = a.orng + (size_t)r * n_mg * GM_TM;
     int wide = 0, big = 0;
     for (int m = tid; m < a.M; m += 256) {
-        wide |= !(orng_r[m] <= kProductRange);
+        wide |= !(orng_r[m] <= kGradProductRange);
         big |= !(orng_r[m] <= kLooseBoundRange);
     }
     const int roomy = __syncthreads_or(big);
@@ -310,7 +315,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
     {
         int wide = 0, big = 0;
         for (int m = tid; m < a.M; m += 256) {
-            wide |= !(orng_r[m] <= kProductRange);
+            wide |= !(orng_r[m] <= kGradProductRange);
             big |= !(orng_r[m] <= kLooseBoundRange);
         }
         roomy = __syncthreads_or(big);
@@ -614,7 +619,7 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     {
         int wide = 0;
         for (int m = tid; m < a.M; m += 256)
-            wide |= !(orng_r[m] <= kProductRange);
+            wide |= !(orng_r[m] <= kGradProductRange);
         if (__syncthreads_or(wide)) {
             // term by term: this workgroup's tile as GO_MT x GO_KT wave tiles
             for (int i = wave; i < (GOM_MT / GO_MT) * (GOM_KT / GO_KT); i += 4) {
@@ -881,7 +886,7 @@ __device__ __forceinline__ void rows_ranges(const MexKernelArgs &a, int tid, int
             for (int r = 0; r < 4; ++r)
                 if (mb + 256 * u + tid < a.M) {
                     big |= !(v[u][r] <= kLooseBoundRange);
-                    wide[r] |= !(v[u][r] <= kProductRange);
+                    wide[r] |= !(v[u][r] <= kGradProductRange);
                 }
     }
     __syncthreads();

@@ -600,7 +600,7 @@ def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
     kw = dict(blocks=[im[1], 1, 1], strides=[im[1], 1, 1], padding=[0, 0, 0], unshared_offset_region=[2], epsilon=1.5,
               softmax_mode=False)
     x, off = mex_case(71, im, n, **kw)
-    off = off * {"narrow": 0.5, "roomy": 2.5, "mixed": 0.3}[spread]
+    off = off * {"narrow": 0.5, "roomy": 4.0, "mixed": 0.3}[spread]
     if spread == "mixed":
         off[::2] *= 300
     check_mex_grads(pkg, x, off, n, strict=spread != "mixed", **kw)
@@ -620,6 +620,30 @@ def test_mex_grads_row_wise_factors_on_power_of_two_maps(pkg, im, n, spread):
     scale_x, scale_o = float(dx.abs().max()), float(doff.abs().max())
     assert float((dx - dx_u).abs().max()) <= 1e-4 * scale_x
     assert float((doff - doff_u).abs().max()) <= 1e-4 * scale_o
+
+
+def test_mex_grads_row_wise_kernels_random_geometries(pkg):
+    """Seeded sweep over the row-wise kernels' domain (power-of-two maps of width 4 ... 64, any batch, channel and
+    instance counts): both gradients against the oracle, and from the pooled gradient bit for bit what the expanded
+    gradient gives."""
+    rng = np.random.default_rng(2024)
+    for _ in range(24):
+        H, W = 1 << int(rng.integers(1, 5)), 1 << int(rng.integers(2, 7))
+        B = int(rng.integers(1, max(2, min(40, 4096 // (H * W)) + 1)))
+        C, n = int(rng.integers(1, 72)), int(rng.integers(1, 80))
+        eps = float(rng.choice([1.0, -1.5, 3.0]))
+        kw = dict(blocks=[C, 1, 1], strides=[C, 1, 1], padding=[0, 0, 0], unshared_offset_region=[2], epsilon=eps,
+                  softmax_mode=bool(rng.integers(0, 2)))
+        x, off = mex_case(int(rng.integers(1 << 30)), (B, C, H, W), n, **kw)
+        off = off * float(rng.choice([0.3, 1.0, 6.0]))
+        print("case", (B, C, H, W), n, eps, flush=True)
+        check_mex_grads(pkg, x, off, n, **kw)
+        X, O = dev(x), dev(off)
+        full, pooled = pkg.mex_sum_pool_both(X, O, n, (2, 2), **kw)
+        gp = torch.randn_like(pooled)
+        want = pkg.mex_grads(X, O, full, pkg.sum_pooling_input_grad(gp, full.shape, (2, 2)), n, **kw)
+        got = pkg.mex_sum_pool_grads(X, O, full, gp, n, (2, 2), **kw)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
 
 
 def test_mex_grads_row_wise_kernels_on_a_large_batch(pkg):
