@@ -86,6 +86,25 @@ def test_similarity_grads_reference_matrix(pkg, strides, blocks, func, norm, ign
     check_sim_grads(pkg, x, t, w, **kw)
 
 
+@pytest.mark.parametrize("func,norm,ign", [("L2", False, False), ("L2", True, False), ("L2", True, True)])
+def test_similarity_params_grad_few_templates_short_patches(pkg, func, norm, ign):
+    """Patches of 1 ... 9 elements with as many templates as the lanes-along-pixels kernel takes (4 * (32 // K)), one
+    fewer and one more (the tiled kernel), seeded shapes, strides and padding; NaN inputs where they are ignored."""
+    rng = np.random.default_rng(77)
+    for blocks, C in (([1, 1], 1), ([1, 2], 1), ([1, 1], 3), ([2, 2], 1), ([1, 1], 5), ([2, 3], 1), ([1, 1], 7),
+                      ([2, 2], 2), ([3, 3], 1)):
+        K = C * blocks[0] * blocks[1]
+        for O in (4 * (32 // K) - 1, 4 * (32 // K), 4 * (32 // K) + 1):
+            B, H, W = int(rng.integers(1, 9)), int(rng.integers(4, 20)), int(rng.integers(4, 20))
+            strides = [int(rng.integers(1, 3)), int(rng.integers(1, 3))]
+            padding = [int(rng.integers(0, 3)), int(rng.integers(0, 3))]
+            x, t, w = sim_inputs(int(rng.integers(1 << 30)), (B, C, H, W), O, blocks, nan_frac=0.2 if ign else 0.0)
+            kw = dict(similarity_function=func, blocks=blocks, strides=strides, padding=padding, normalization_term=norm,
+                      ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else 0.5)
+            print("case", (B, C, H, W), O, blocks, strides, padding, flush=True)
+            check_sim_grads(pkg, x, t, w, **kw)
+
+
 def sim_inputs(seed, shape, O, blocks, nan_frac=0.0):
     g = np.random.default_rng(seed)
     x = g.normal(size=shape).astype(np.float32)
