@@ -750,3 +750,98 @@ def test_similarity_small_map_forms_agree_at_network_sizes(pkg, shape, O):
     fast = pkg.similarity(x, t, w, **kw).cpu().numpy()
     exact = pkg.similarity(x, t, w, algo="direct", **kw).cpu().numpy()
     assert rel_err(fast, exact) <= SIM_TOL
+
+
+# ---- seeded sweeps: random geometries through whatever kernel the library picks -----------------------------------
+def mex_close(got, x, off, n, **kw):
+    """Within MEX_TOL of the fp32 oracle under mex_err's metric.  Where an output and its largest term both pass
+    through zero (short patches), that metric divides rounding noise by almost nothing, for the reference's own fp32
+    arithmetic as well: those elements must be within 1e-6 of the operands' size (max|x| + max|offsets|) of the exact
+    (fp64) value instead, a few ulps of the terms they are made of."""
+    if mex_err(got, x, off, n, **kw) <= MEX_TOL:
+        return True
+    want = orc.mex_fwd(x, off, n, **kw)
+    exact = orc.mex_fwd(x.astype(np.float64), off.astype(np.float64), n, **kw)
+    shift = orc.mex_fwd(x, off, n, **dict(kw, epsilon=math.copysign(math.inf, kw.get("epsilon", 1.0))))
+    floor = np.maximum(np.abs(want), np.abs(shift))
+    with np.errstate(invalid="ignore", divide="ignore"):
+        bad = ~(np.abs(got - want) <= MEX_TOL * floor) & ~((got == want) | (np.isnan(got) & np.isnan(want)))
+    size = float(np.abs(x).max() + np.abs(off[np.isfinite(off)]).max())
+    worst = float(np.abs(got[bad] - exact[bad]).max())
+    print("  %d of %d outputs beyond %g of the fp32 oracle, all with max(|want|, |m|) <= %.3g; against fp64 they are "
+          "off by at most %.3g (operands up to %.3g; the fp32 oracle: %.3g)"
+          % (bad.sum(), bad.size, MEX_TOL, floor[bad].max(), worst, size, np.abs(want[bad] - exact[bad]).max()))
+    return bool(np.isfinite(got[bad]).all() and floor[bad].max() <= 1e-2 * size and worst <= 1e-6 * size)
+
+
+def test_mex_forward_random_geometries(pkg):
+    """MEX, MEX + pooling (with and without the unpooled output) on seeded random layers: whole-channel patches on
+    power-of-two and ragged maps (the panel, fused, wave-per-pixel and tiled kernels), small 3-D blocks with padding,
+    shared and unshared regions, either sign of epsilon and +-inf, narrow and wide offsets, with and without the
+    offsets normalisation; every result against the oracle."""
+    rng = np.random.default_rng(4242)
+    for case in range(160):
+        whole = case % 4 != 3
+        if whole:
+            pow2 = bool(rng.integers(0, 2))
+            H = 1 << int(rng.integers(0, 5)) if pow2 else int(rng.integers(1, 13))
+            W = 1 << int(rng.integers(0, 5)) if pow2 else int(rng.integers(1, 13))
+            C = int(rng.choice([1, 3, 8, 32, 33, 64, 100, 128, 256, 300]))
+            blocks, strides, padding = [C, 1, 1], [C, 1, 1], [0, 0, 0]
+        else:
+            H, W, C = int(rng.integers(3, 11)), int(rng.integers(3, 11)), int(rng.integers(1, 9))
+            blocks = [int(rng.integers(1, C + 1)), int(rng.integers(1, 4)), int(rng.integers(1, 4))]
+            strides = [int(rng.integers(1, blocks[0] + 1)), int(rng.integers(1, 3)), int(rng.integers(1, 3))]
+            padding = [0, int(rng.integers(0, 2)), int(rng.integers(0, 2))]
+        n = int(rng.integers(1, 140)) if C <= 128 else int(rng.integers(1, 24))
+        B = int(rng.integers(1, max(2, min(24, 200000 // max(1, H * W * C * n // 8)) + 1)))
+        unshared = bool(rng.integers(0, 2))
+        region = [1, 2, 2] if rng.integers(0, 2) else [int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.integers(1, 4))]
+        eps = float(rng.choice([1.0, -1.0, 2.5, -0.4, math.inf, -math.inf]))
+        kw = dict(blocks=blocks, strides=strides, padding=padding, epsilon=eps, softmax_mode=bool(rng.integers(0, 2)),
+                  use_unshared_regions=unshared, blocks_out_of_bounds_value=float(rng.choice([0.0, -1.5])))
+        kw["unshared_offset_region" if unshared else "shared_offset_region"] = region
+        try:
+            d = orc.mex_dims(orc.mex_args((B, C, H, W), n, **kw))
+        except Exception:
+            continue   # a geometry the reference rejects
+        g = np.random.default_rng(int(rng.integers(1 << 30)))
+        x = g.normal(size=(B, C, H, W)).astype(np.float32)
+        off = (g.normal(size=(d.num_regions, n) + tuple(blocks)) * float(rng.choice([0.3, 2.0, 40.0]))).astype(np.float32)
+        normalize = bool(rng.integers(0, 2))
+        offn = orc.normalize_offsets(off) if normalize else off
+        print("case", case, (B, C, H, W), n, kw, "normalize" if normalize else "", flush=True)
+        got = run_mex(pkg, x, off, n, normalize_offsets=normalize, **kw)
+        assert mex_close(got, x, offn, n, **kw)
+        Ho, Wo = got.shape[2], got.shape[3]
+        if Ho >= 2 and Wo >= 2:
+            X, O = dev(x), dev(off)
+            full, pooled = pkg.mex_sum_pool_both(X, O, n, (2, 2), normalize_offsets=normalize, **kw)
+            assert mex_close(full.cpu().numpy(), x, offn, n, **kw)
+            assert torch.equal(pooled, pkg.sum_pooling(full, (2, 2)))
+            assert torch.equal(pooled, pkg.mex_sum_pool(X, O, n, (2, 2), normalize_offsets=normalize, **kw))
+
+
+def test_similarity_forward_random_geometries(pkg):
+    """Similarity on seeded random layers (all four modes, blocks 1 ... 5, strides 1 ... 3, padding, NaN inputs where
+    they are ignored, template counts around the tile sizes) against the oracle."""
+    rng = np.random.default_rng(777)
+    for case in range(120):
+        func = "L1" if case % 4 == 0 else "L2"
+        norm = func == "L2" and case % 4 >= 2
+        ign = norm and case % 4 == 3
+        C, H, W = int(rng.choice([1, 2, 3, 8, 24, 64])), int(rng.integers(3, 40)), int(rng.integers(3, 40))
+        blocks = [int(rng.integers(1, min(5, H) + 1)), int(rng.integers(1, min(5, W) + 1))]
+        strides = [int(rng.integers(1, 4)), int(rng.integers(1, 4))]
+        padding = [int(rng.integers(0, 3)), int(rng.integers(0, 3))]
+        O = int(rng.choice([1, 7, 8, 9, 31, 32, 33, 64, 130]))
+        B = int(rng.integers(1, max(2, min(20, 3000000 // (H * W * C * O * blocks[0] * blocks[1])) + 1)))
+        x, t, w = sim_inputs(int(rng.integers(1 << 30)), (B, C, H, W), O, blocks, nan_frac=0.2 if ign else 0.0)
+        kw = dict(similarity_function=func, blocks=blocks, strides=strides, padding=padding, normalization_term=norm,
+                  ignore_nan_input=ign, out_of_bounds_value=float("nan") if ign else float(rng.choice([0.0, 0.75])))
+        try:
+            want = orc.similarity_fwd(x, t, w, **kw)
+        except Exception:
+            continue
+        print("case", case, (B, C, H, W), O, kw, flush=True)
+        assert rel_err(run_similarity(pkg, x, t, w, **kw), want) <= SIM_TOL
