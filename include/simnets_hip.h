@@ -345,8 +345,34 @@ int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int inp
                                    const float *mex_output, const float *pooled_output_grad, float *input_grad,
                                    float *offsets_grad, void *workspace, size_t workspace_bytes, void *stream);
 
-/* ... in two halves, like simnets_hip_mex_prepare / simnets_hip_mex_fwd_prepared: the buffer has
- * simnets_hip_mex_sum_pool_workspace_bytes bytes; when the geometry runs the two kernels through scratch memory the
+/* A training step runs the forward op and then its gradients on the same offsets (python/simnets/ops/mex.py:47-81:
+ * the registered gradient receives the forward op's inputs and output).  Both sides re-order the offsets first
+ * (scaled, row maxima and ranges, exponentials, the normalised copy of normalize_offsets), in different group sizes.
+ * The *_saving forward calls leave the gradient kernels' form in `saved` (simnets_hip_mex_saved_bytes; 256-byte
+ * aligned; 0 bytes = this layer's gradient kernels read the offsets as they are, `saved` may then be NULL) from the
+ * launch that packs the forward's own, and the *_saved gradient calls read it instead of packing again.  Outputs
+ * and gradients are those of the plain calls, bit for bit.  `saved` is valid for the attributes, input shape and
+ * offsets VALUES of the forward call that wrote it; a gradient call given saved == NULL packs for itself. */
+int simnets_hip_mex_saved_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], size_t *bytes);
+int simnets_hip_mex_fwd_saving(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                               const float *offsets, size_t offsets_count, float *output, void *saved,
+                               size_t saved_bytes, void *workspace, size_t workspace_bytes, void *stream);
+int simnets_hip_mex_sum_pool_fwd_saving(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                        const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                        float *mex_output, float *output, void *saved, size_t saved_bytes,
+                                        void *workspace, size_t workspace_bytes, void *stream);
+int simnets_hip_mex_grads_saved(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                const float *offsets, size_t offsets_count, const float *output,
+                                const float *output_grad, const void *saved, size_t saved_bytes, float *input_grad,
+                                float *offsets_grad, void *workspace, size_t workspace_bytes, void *stream);
+int simnets_hip_mex_sum_pool_grads_saved(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                         const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                         const float *mex_output, const float *pooled_output_grad, const void *saved,
+                                         size_t saved_bytes, float *input_grad, float *offsets_grad, void *workspace,
+                                         size_t workspace_bytes, void *stream);
+
+/* ... simnets_hip_mex_sum_pool_fwd in two halves, like simnets_hip_mex_prepare / simnets_hip_mex_fwd_prepared: the
+ * buffer has simnets_hip_mex_sum_pool_workspace_bytes bytes; when the geometry runs the two kernels through scratch memory the
  * buffer holds that scratch as well, so calls that share one prepared buffer must not overlap. */
 int simnets_hip_mex_sum_pool_prepare(const simnets_mex_attrs *attrs, const int input_shape[4], const float *offsets,
                                      size_t offsets_count, int pool_h, int pool_w, void *prepared,

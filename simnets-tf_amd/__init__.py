@@ -17,6 +17,8 @@ from .ops import (  # noqa: F401
     mex_sum_pool,
     mex_sum_pool_both,
     mex_sum_pool_grads,
+    mex_saving,
+    mex_sum_pool_saving,
     similarity_mex_sum_pool,
     similarity_input_grad,
     similarity_parameters_grad,
@@ -39,5 +41,5 @@ from .layers import Similarity, Mex, dirichlet_init  # noqa: F401,E402
 
 __all__ = ["layers", "unsupervised", "torch_ops", "Similarity", "Mex", "dirichlet_init", "similarity", "mex", "sum_pooling", "mex_sum_pool", "similarity_mex_sum_pool", "similarity_output_shape", "mex_output_shape", "SimnetsError",
            "similarity_input_grad", "similarity_parameters_grad", "mex_input_grad", "mex_offsets_grad",
-           "sum_pooling_input_grad", "mex_grads", "mex_sum_pool_both", "mex_sum_pool_grads", "Prepared", "similarity_prepare", "mex_prepare", "mex_sum_pool_prepare",
+           "sum_pooling_input_grad", "mex_grads", "mex_sum_pool_both", "mex_sum_pool_grads", "mex_saving", "mex_sum_pool_saving", "Prepared", "similarity_prepare", "mex_prepare", "mex_sum_pool_prepare",
            "similarity_mex_sum_pool_prepare"]

@@ -18,6 +18,8 @@ EXPORTS = [
     "simnets_hip_mex_offsets_grad", "simnets_hip_mex_grads_workspace_bytes", "simnets_hip_mex_grads",
     "simnets_hip_mex_sum_pool_workspace_bytes", "simnets_hip_mex_sum_pool_fwd", "simnets_hip_mex_sum_pool_fwd_both",
     "simnets_hip_mex_sum_pool_grads_workspace_bytes", "simnets_hip_mex_sum_pool_grads",
+    "simnets_hip_mex_saved_bytes", "simnets_hip_mex_fwd_saving", "simnets_hip_mex_sum_pool_fwd_saving",
+    "simnets_hip_mex_grads_saved", "simnets_hip_mex_sum_pool_grads_saved",
     "simnets_hip_similarity_mex_sum_pool_workspace_bytes", "simnets_hip_similarity_mex_sum_pool_fwd",
     "simnets_hip_similarity_prepare", "simnets_hip_similarity_fwd_prepared",
     "simnets_hip_mex_prepare", "simnets_hip_mex_fwd_prepared",
@@ -121,6 +123,18 @@ def lib():
         l.simnets_hip_mex_sum_pool_grads.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int, P, P, P, P,
                                                      P, C.c_size_t, P]
         l.simnets_hip_mex_sum_pool_grads.restype = C.c_int
+        l.simnets_hip_mex_saved_bytes.argtypes = [C.POINTER(MexAttrs), I4, C.POINTER(C.c_size_t)]
+        l.simnets_hip_mex_fwd_saving.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, C.c_size_t, P,
+                                                 C.c_size_t, P]
+        l.simnets_hip_mex_sum_pool_fwd_saving.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int,
+                                                          P, P, P, C.c_size_t, P, C.c_size_t, P]
+        l.simnets_hip_mex_grads_saved.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, P, P, P, C.c_size_t, P, P,
+                                                  P, C.c_size_t, P]
+        l.simnets_hip_mex_sum_pool_grads_saved.argtypes = [C.POINTER(MexAttrs), I4, P, P, C.c_size_t, C.c_int, C.c_int,
+                                                           P, P, P, C.c_size_t, P, P, P, C.c_size_t, P]
+        for f in (l.simnets_hip_mex_saved_bytes, l.simnets_hip_mex_fwd_saving, l.simnets_hip_mex_sum_pool_fwd_saving,
+                  l.simnets_hip_mex_grads_saved, l.simnets_hip_mex_sum_pool_grads_saved):
+            f.restype = C.c_int
         SZ = C.POINTER(C.c_size_t)
         l.simnets_hip_similarity_mex_sum_pool_workspace_bytes.argtypes = [C.POINTER(SimilarityAttrs), I4, I4,
                                                                           C.POINTER(MexAttrs), C.c_int, C.c_int, SZ]

@@ -259,21 +259,46 @@ int simnets_hip_mex_grads_workspace_bytes(const simnets_mex_attrs *attrs, const 
     return SIMNETS_OK;
 }
 
-int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
-                          const float *offsets, size_t offsets_count, const float *output, const float *output_grad,
-                          float *input_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
-                          void *stream)
+// the buffer a saving forward call filled, if the caller has one and the layer's gradient kernels read one
+static int saved_pack(const MexPlan &p, const void *saved, size_t saved_bytes, const void **use)
+{
+    *use = nullptr;
+    const size_t need = mex_grad_pack_bytes(p);
+    if (saved == nullptr || need == 0)
+        return SIMNETS_OK;
+    if (!workspace_ok(saved, saved_bytes, need))
+        return SIMNETS_ERR_WORKSPACE;
+    *use = saved;
+    return SIMNETS_OK;
+}
+
+int simnets_hip_mex_grads_saved(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                const float *offsets, size_t offsets_count, const float *output,
+                                const float *output_grad, const void *saved, size_t saved_bytes, float *input_grad,
+                                float *offsets_grad, void *workspace, size_t workspace_bytes, void *stream)
 {
     MexPlan p;
-    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
     if (rc)
         return rc;
     if (!offsets || !offsets_grad || (p.B > 0 && (!input || !output || !output_grad || !input_grad)))
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_grads_workspace_bytes(p, true, true)))
         return SIMNETS_ERR_WORKSPACE;
+    const void *pack;
+    if ((rc = saved_pack(p, saved, saved_bytes, &pack)) != SIMNETS_OK)
+        return rc;
     return mex_grads(p, input, offsets, output, output_grad, input_grad, offsets_grad, workspace, workspace_bytes,
-                     stream);
+                     stream, false, pack);
+}
+
+int simnets_hip_mex_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                          const float *offsets, size_t offsets_count, const float *output, const float *output_grad,
+                          float *input_grad, float *offsets_grad, void *workspace, size_t workspace_bytes,
+                          void *stream)
+{
+    return simnets_hip_mex_grads_saved(attrs, input_shape, input, offsets, offsets_count, output, output_grad, nullptr,
+                                       0, input_grad, offsets_grad, workspace, workspace_bytes, stream);
 }
 
 // scratch of simnets_hip_mex_sum_pool_grads: the gradient kernels' workspace, then the expanded pooling gradient
@@ -305,8 +330,19 @@ int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int inp
                                    const float *mex_output, const float *pooled_output_grad, float *input_grad,
                                    float *offsets_grad, void *workspace, size_t workspace_bytes, void *stream)
 {
+    return simnets_hip_mex_sum_pool_grads_saved(attrs, input_shape, input, offsets, offsets_count, pool_h, pool_w,
+                                                mex_output, pooled_output_grad, nullptr, 0, input_grad, offsets_grad,
+                                                workspace, workspace_bytes, stream);
+}
+
+int simnets_hip_mex_sum_pool_grads_saved(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                         const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                         const float *mex_output, const float *pooled_output_grad, const void *saved,
+                                         size_t saved_bytes, float *input_grad, float *offsets_grad, void *workspace,
+                                         size_t workspace_bytes, void *stream)
+{
     MexPlan p;
-    const int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
+    int rc = mex_grad_checks(attrs, input_shape, offsets_count, &p);
     if (rc)
         return rc;
     if (pool_h <= 0 || pool_w <= 0)
@@ -320,9 +356,12 @@ int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int inp
     const size_t need = mex_pool_grads_scratch(p, &expanded_at);
     if (!workspace_ok(workspace, workspace_bytes, need))
         return SIMNETS_ERR_WORKSPACE;
+    const void *pack;
+    if ((rc = saved_pack(p, saved, saved_bytes, &pack)) != SIMNETS_OK)
+        return rc;
     if (p.B > 0 && pool_h == 2 && pool_w == 2 && mex_grads_take_pooled(p, input, mex_output, pooled_output_grad, input_grad))
         return mex_grads(p, input, offsets, mex_output, pooled_output_grad, input_grad, offsets_grad, workspace,
-                         expanded_at, stream, true);
+                         expanded_at, stream, true, pack);
     float *expanded = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + expanded_at);
     if (p.B > 0) {
         const int erc = sum_pool_grad_launch(p.B, p.d.M * p.d.channels_out, p.d.height_out, p.d.width_out, pool_h, pool_w,
@@ -330,15 +369,51 @@ int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int inp
         if (erc)
             return erc;
     }
-    return mex_grads(p, input, offsets, mex_output, expanded, input_grad, offsets_grad, workspace, expanded_at, stream);
+    return mex_grads(p, input, offsets, mex_output, expanded, input_grad, offsets_grad, workspace, expanded_at, stream,
+                     false, pack);
+}
+
+// A forward call that also leaves the offsets as the gradient kernels read them in `saved`: the plan asks the
+// forward's pack launch to write them; a forward that launched none (it packs inside its kernel) is followed by the
+// gradient kernels' own pack launch.
+static int saving_begin(MexPlan &p, MexGradPack *gp, void *saved, size_t saved_bytes)
+{
+    gp->buffer = nullptr; gp->written = false;
+    const size_t need = mex_grad_pack_bytes(p);
+    if (need == 0)
+        return SIMNETS_OK;
+    if (!workspace_ok(saved, saved_bytes, need))
+        return SIMNETS_ERR_WORKSPACE;
+    gp->buffer = saved;
+    p.grad_pack = gp;
+    return SIMNETS_OK;
+}
+static int saving_end(const MexPlan &p, const MexGradPack &gp, const float *offsets, void *stream)
+{
+    if (gp.buffer == nullptr || gp.written)
+        return SIMNETS_OK;
+    return mex_grad_pack_launch(p, offsets, gp.buffer, stream);
+}
+
+int simnets_hip_mex_saved_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], size_t *bytes)
+{
+    if (!bytes)
+        return SIMNETS_ERR_NULL_POINTER;
+    MexPlan p;
+    const int rc = mex_make_plan(attrs, input_shape, &p);
+    if (rc)
+        return rc;
+    *bytes = mex_grad_pack_bytes(p);
+    return SIMNETS_OK;
 }
 
 static int mex_fwd_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                          const float *offsets, size_t offsets_count, float *output, void *workspace,
-                         size_t workspace_bytes, void *stream, int phase)
+                         size_t workspace_bytes, void *stream, int phase, bool saving = false, void *saved = nullptr,
+                         size_t saved_bytes = 0)
 {
     MexPlan p;
-    const int rc = mex_make_plan(attrs, input_shape, &p);
+    int rc = mex_make_plan(attrs, input_shape, &p);
     if (rc)
         return rc;
     if ((phase & kMexPrepare) && offsets_count < (size_t)p.d.num_regions * p.d.M * p.d.K)
@@ -349,7 +424,19 @@ static int mex_fwd_phase(const simnets_mex_attrs *attrs, const int input_shape[4
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_workspace_bytes(p)))
         return SIMNETS_ERR_WORKSPACE;
-    return mex_launch(p, input, offsets, output, workspace, workspace_bytes, stream, phase);
+    MexGradPack gp;
+    if (saving && (rc = saving_begin(p, &gp, saved, saved_bytes)) != SIMNETS_OK)
+        return rc;
+    rc = mex_launch(p, input, offsets, output, workspace, workspace_bytes, stream, phase);
+    return rc != SIMNETS_OK || !saving ? rc : saving_end(p, gp, offsets, stream);
+}
+
+int simnets_hip_mex_fwd_saving(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                               const float *offsets, size_t offsets_count, float *output, void *saved,
+                               size_t saved_bytes, void *workspace, size_t workspace_bytes, void *stream)
+{
+    return mex_fwd_phase(attrs, input_shape, input, offsets, offsets_count, output, workspace, workspace_bytes, stream,
+                         kMexWhole, true, saved, saved_bytes);
 }
 
 int simnets_hip_mex_fwd(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
@@ -429,10 +516,11 @@ int simnets_hip_mex_sum_pool_workspace_bytes(const simnets_mex_attrs *attrs, con
 static int mex_sum_pool_phase(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
                               const float *offsets, size_t offsets_count, int pool_h, int pool_w, float *output,
                               void *workspace, size_t workspace_bytes, void *stream, int phase,
-                              float *mex_output = nullptr)
+                              float *mex_output = nullptr, bool saving = false, void *saved = nullptr,
+                              size_t saved_bytes = 0)
 {
     MexPlan p;
-    const int rc = mex_make_plan(attrs, input_shape, &p);
+    int rc = mex_make_plan(attrs, input_shape, &p);
     if (rc)
         return rc;
     if (pool_h <= 0 || pool_w <= 0 ||
@@ -446,8 +534,23 @@ static int mex_sum_pool_phase(const simnets_mex_attrs *attrs, const int input_sh
         return SIMNETS_ERR_NULL_POINTER;
     if (!workspace_ok(workspace, workspace_bytes, mex_pool_workspace_bytes(p, pool_h, pool_w)))
         return SIMNETS_ERR_WORKSPACE;
-    return mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream, phase,
-                           mex_output);
+    MexGradPack gp;
+    if (saving && (rc = saving_begin(p, &gp, saved, saved_bytes)) != SIMNETS_OK)
+        return rc;
+    rc = mex_pool_launch(p, pool_h, pool_w, input, offsets, output, workspace, workspace_bytes, stream, phase,
+                         mex_output);
+    return rc != SIMNETS_OK || !saving ? rc : saving_end(p, gp, offsets, stream);
+}
+
+int simnets_hip_mex_sum_pool_fwd_saving(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,
+                                        const float *offsets, size_t offsets_count, int pool_h, int pool_w,
+                                        float *mex_output, float *output, void *saved, size_t saved_bytes,
+                                        void *workspace, size_t workspace_bytes, void *stream)
+{
+    if (!mex_output && input_shape[0] != 0)
+        return SIMNETS_ERR_NULL_POINTER;
+    return mex_sum_pool_phase(attrs, input_shape, input, offsets, offsets_count, pool_h, pool_w, output, workspace,
+                              workspace_bytes, stream, kMexWhole, mex_output, true, saved, saved_bytes);
 }
 
 int simnets_hip_mex_sum_pool_fwd_both(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,

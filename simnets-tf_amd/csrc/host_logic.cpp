@@ -228,6 +228,7 @@ int mex_make_plan(const simnets_mex_attrs *a, const int in[4], MexPlan *p)
     p->oob = a->blocks_out_of_bounds_value;
     p->use_unshared = a->use_unshared_regions != 0;
     p->normalize_offsets = a->normalize_offsets != 0;
+    p->grad_pack = nullptr;
     if (std::isnan(a->epsilon) || a->epsilon == 0.0f)
         return SIMNETS_ERR_SHAPE;
     if (!fits_int32(1LL * p->B * p->d.region_size) || !fits_int32(1LL * p->d.num_regions * p->d.M * 1LL) )

@@ -38,6 +38,12 @@ int sim_prepare(const SimPlan &p, const float *templates, const float *weights, 
                 void *stream);
 int sim_run(const SimPlan &p, const float *input, float *output, void *prepared, size_t prepared_bytes, void *stream);
 
+// where a forward call leaves the offsets as the gradient kernels read them (mex_grad_pack_bytes)
+struct MexGradPack {
+    void *buffer;
+    bool written;   // set by the forward's pack launch when it wrote the buffer
+};
+
 struct MexPlan {
     int B, C, H, W;
     simnets_mex_dims d;
@@ -45,6 +51,7 @@ struct MexPlan {
     float epsilon, oob;
     int use_unshared;
     int normalize_offsets;
+    MexGradPack *grad_pack;   // forward calls that keep the gradient kernels' offsets layout; else null
 };
 
 int mex_make_plan(const simnets_mex_attrs *attrs, const int input_shape[4], MexPlan *plan);
@@ -76,7 +83,11 @@ size_t mex_grads_workspace_bytes(const MexPlan &p, bool want_input, bool want_of
 // grad_is_pooled: output_grad is the gradient of the 2 x 2 sum-pooled output (only where mex_grads_take_pooled says so)
 int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
               const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
-              size_t workspace_bytes, void *stream, bool grad_is_pooled = false);
+              size_t workspace_bytes, void *stream, bool grad_is_pooled = false, const void *saved = nullptr);
+// `saved`: the buffer (mex_grad_pack_bytes, declared with the packing in mex_common.h) that a forward call of the same
+// layer and offsets filled, through MexPlan::grad_pack or mex_grad_pack_launch; the call then packs nothing.
+size_t mex_grad_pack_bytes(const MexPlan &p);   // 0: the layer's gradient kernels read no packed offsets
+int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream);
 // whether the gradient kernels of this layer read the pooled gradient themselves (the row-wise kernels on suitably
 // aligned tensors; input_grad may be null)
 bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *output, const float *pooled_grad,

@@ -493,7 +493,7 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                                                               float *__restrict__ offe, float *__restrict__ omax,
                                                               float *__restrict__ orng, int4 *__restrict__ ktab, int H,
                                                               int W, int bh, int bw, int row_blocks, SimPackJob job,
-                                                              float *__restrict__ normalized_out)
+                                                              float *__restrict__ normalized_out, MexPackTwin tw)
 {
     if ((int)blockIdx.x >= row_blocks) {
         // extra workgroups: the parameters of a Similarity layer evaluated inside the MEX staging
@@ -519,30 +519,51 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
             const int rem = k - dc * bh * bw;
             const int dh = rem / bw, dw = rem - dh * bw;
             ktab[k] = make_int4((dc * H + dh) * W + dw, dc, dh, dw);
+            if (tw.offp != nullptr)
+                tw.ktab[k] = ktab[k];
         }
     }
+    // a wave per (region, instance) with the instances padded to the groups of the layout (of the wider of the two
+    // layouts when the launch writes a second one)
     const int lane = threadIdx.x & 63;
-    const long long row = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    const long long rows = (long long)R * n_mgroups * tm;
-    if (row >= rows)
+    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int Mp = n_mgroups * tm, Mp2 = tw.offp != nullptr ? tw.n_mgroups * tw.tm : 0;
+    const int Mw = max(Mp, Mp2);
+    if (wave >= (long long)R * Mw)
         return;
-    const int mi = (int)(row % tm);
-    const long long t = row / tm;
-    const int mgroup = (int)(t % n_mgroups);
-    const int r = (int)(t / n_mgroups);
-    const int m = mgroup * tm + mi;
-    const size_t at = ((size_t)r * n_mgroups + mgroup) * K * tm + mi;
-    float *dst = offp + at;
-    float *dste = offe + at;
+    const int m = (int)(wave % Mw), r = (int)(wave / Mw);
+    const long long row = (long long)r * Mp + m;
+    float *dst = offp + ((size_t)r * n_mgroups + m / tm) * K * tm + m % tm;
+    float *dste = offe + (dst - offp);
+    // the second layout (finite epsilon only): same values, its own group size
+    const int tm2 = tw.tm;
+    const long long row2 = (long long)r * Mp2 + m;
+    float *dst2 = nullptr, *dste2 = nullptr;
+    if (m < Mp2) {
+        dst2 = tw.offp + ((size_t)r * tw.n_mgroups + m / tm2) * K * tm2 + m % tm2;
+        dste2 = tw.offe + (dst2 - tw.offp);
+    }
     if (m >= M) {
         for (int k = lane; k < K; k += 64) {
-            dst[(size_t)k * tm] = 0.0f;
-            if (finite_eps)
-                dste[(size_t)k * tm] = 0.0f;
+            if (m < Mp) {
+                dst[(size_t)k * tm] = 0.0f;
+                if (finite_eps)
+                    dste[(size_t)k * tm] = 0.0f;
+            }
+            if (dst2 != nullptr) {
+                dst2[(size_t)k * tm2] = 0.0f;
+                dste2[(size_t)k * tm2] = 0.0f;
+            }
         }
         if (finite_eps && lane == 0) {
-            omax[row] = 0.0f;
-            orng[row] = 0.0f;
+            if (m < Mp) {
+                omax[row] = 0.0f;
+                orng[row] = 0.0f;
+            }
+            if (dst2 != nullptr) {
+                tw.omax[row2] = 0.0f;
+                tw.orng[row2] = 0.0f;
+            }
         }
         return;
     }
@@ -598,12 +619,21 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
     }
     each([&](int k, float x) {
         const float v = mex_scaled_offset(x, lse, scale);
+        const float e = __builtin_amdgcn_exp2f(v - hi);
         dst[(size_t)k * tm] = v;
-        dste[(size_t)k * tm] = __builtin_amdgcn_exp2f(v - hi);
+        dste[(size_t)k * tm] = e;
+        if (dst2 != nullptr) {
+            dst2[(size_t)k * tm2] = v;
+            dste2[(size_t)k * tm2] = e;
+        }
     });
     if (lane == 0) {
         omax[row] = hi;
         orng[row] = hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
+        if (dst2 != nullptr) {
+            tw.omax[row2] = hi;
+            tw.orng[row2] = hi - lo;
+        }
     }
 }
 
@@ -896,6 +926,33 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups)
     return 2 * packed + 2 * rows + align_up((size_t)p.d.K * sizeof(int4), 256);
 }
 
+size_t mex_grad_pack_bytes(const MexPlan &p)
+{
+    if (!std::isfinite(p.epsilon))
+        return 0;   // those gradient kernels read the offsets as they are
+    const size_t rmk = (size_t)p.d.num_regions * p.d.M * p.d.K * sizeof(float);
+    return mex_packed_bytes(p, kGradPackTm, (p.d.M + kGradPackTm - 1) / kGradPackTm) +
+           (p.normalize_offsets ? align_up(rmk, 256) : 0);
+}
+
+void mex_grad_pack_layout(const MexPlan &p, void *buffer, MexPackTwin *tw, float **normalized)
+{
+    const simnets_mex_dims &d = p.d;
+    tw->tm = kGradPackTm;
+    tw->n_mgroups = (d.M + kGradPackTm - 1) / kGradPackTm;
+    const long long rows = (long long)d.num_regions * tw->n_mgroups * tw->tm;
+    const size_t packed = align_up((size_t)rows * d.K * sizeof(float), 256);
+    const size_t row_bytes = align_up((size_t)rows * sizeof(float), 256);
+    char *ws = reinterpret_cast<char *>(buffer);
+    tw->offp = reinterpret_cast<float *>(ws);
+    tw->offe = reinterpret_cast<float *>(ws + packed);
+    tw->omax = reinterpret_cast<float *>(ws + 2 * packed);
+    tw->orng = reinterpret_cast<float *>(ws + 2 * packed + row_bytes);
+    tw->ktab = reinterpret_cast<int4 *>(ws + 2 * packed + 2 * row_bytes);
+    *normalized = p.normalize_offsets
+                      ? reinterpret_cast<float *>(ws + mex_packed_bytes(p, tw->tm, tw->n_mgroups)) : nullptr;
+}
+
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
                      void *stream, const SimPackJob *job, bool launch, float *normalized_out)
 {
@@ -915,7 +972,15 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
     a->n_mgroups = n_mgroups;
     if (!launch)
         return SIMNETS_OK;  // the arrays are in place already: only the pointers were wanted
-    const int row_blocks = (int)((rows + 3) / 4);
+    // a forward call that keeps the gradient kernels' layout as well: the same launch writes it
+    MexPackTwin tw = {nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+    long long waves = rows;
+    if (p.grad_pack != nullptr && normalized_out == nullptr && mex_grad_pack_bytes(p) > 0) {
+        mex_grad_pack_layout(p, p.grad_pack->buffer, &tw, &normalized_out);
+        waves = (long long)d.num_regions * std::max(n_mgroups * tm, tw.n_mgroups * tw.tm);
+        p.grad_pack->written = true;
+    }
+    const int row_blocks = (int)((waves + 3) / 4);
     SimPackJob pj = {nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0.0f};
     int extra = 0;
     if (job) {
@@ -927,7 +992,7 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
 #define SIMNETS_PACK_LAUNCH(KL)                                                                                        \
     hipLaunchKernelGGL(mex_pack_offsets_kernel<KL>, grid, dim3(256), 0, hs, offsets, d.num_regions, d.M, d.K, n_mgroups, \
                        tm, p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W,         \
-                       d.block_h, d.block_w, row_blocks, pj, normalized_out)
+                       d.block_h, d.block_w, row_blocks, pj, normalized_out, tw)
     if (d.K <= 64)
         SIMNETS_PACK_LAUNCH(1);
     else if (d.K <= 256)

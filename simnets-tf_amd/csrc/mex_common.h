@@ -158,6 +158,17 @@ struct SimPackJob {
     float fudge;
 };
 size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
+// A second packed layout written by the same launch: what the gradient kernels read (groups of kGradPackTm instances,
+// and the normalised offsets when the layer normalises them), kept by a forward call for the gradient call that
+// follows it.  A plan whose grad_pack is set makes the forward's pack launch write it (and say so in `written`; a
+// forward that packs inside its own kernel does not).
+constexpr int kGradPackTm = 32;
+struct MexPackTwin {
+    float *offp, *offe, *omax, *orng;
+    int4 *ktab;
+    int tm, n_mgroups;
+};
+void mex_grad_pack_layout(const MexPlan &p, void *buffer, MexPackTwin *tw, float **normalized);
 // launch = false: the arrays were packed by an earlier call with the same arguments; only the pointers are set.
 // normalized_out: if not null, the launch also writes the offsets minus their rows' logsumexp there, [region][M][K]
 // (what the gradient kernels' term-by-term path and the chain rule through the normalisation read).

@@ -160,7 +160,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
 // forward pass.  Used when every instance of the region has an offsets range of at most kGradProductRange; otherwise the
 // workgroup falls back to the term-by-term waves.
 // grid.x: (region, pixel chunk of 64 slots); grid.y: tile of GM_KT patch elements (16 per wave)
-constexpr int GM_TM = 32;   // instances per packed group = contraction chunk
+constexpr int GM_TM = kGradPackTm;   // (32) instances per packed group = contraction chunk
 // Widest offsets range (an exponent of two) the gradients' product form takes.  Its factors 2^(xs - a), 2^(os - mo) and W
 // carry exponents of up to the range, each rounded once: an error of ulp(range) in an exponent is a relative error of
 // about 4e-8 * range in the factor, and measured against the fp64 oracle the gradients stay within the 1e-4 bar up to
@@ -1656,9 +1656,20 @@ bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *ou
            aligned(pooled_grad, 8) && (input_grad == nullptr || aligned(input_grad, 16));
 }
 
+int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream)
+{
+    MexPlan q = p;
+    q.grad_pack = nullptr;
+    MexPackTwin tw;
+    float *norm;
+    mex_grad_pack_layout(q, buffer, &tw, &norm);
+    MexKernelArgs a = mex_kernel_args(q);
+    return mex_pack_offsets(q, offsets, GM_TM, tw.n_mgroups, buffer, &a, stream, nullptr, true, norm);
+}
+
 int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
               const float *output_grad, float *input_grad, float *offsets_grad, void *workspace,
-              size_t workspace_bytes, void *stream, bool grad_is_pooled)
+              size_t workspace_bytes, void *stream, bool grad_is_pooled, const void *saved)
 {
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
     const bool want_input = input_grad != nullptr, want_offsets = offsets_grad != nullptr;
@@ -1687,9 +1698,18 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     // the offsets as the forward op used them: with the matrix kernels the pack launch below writes the normalised
     // copy as well, otherwise a launch of its own does
     const bool pack_normalizes = t.mfma && p.normalize_offsets;
+    // ... or the forward call left them (and their packed form) in `saved`
+    const bool packed_already = saved != nullptr && t.mfma;
+    char *packed_at = ws + w.packed;
+    float *norm_at = reinterpret_cast<float *>(ws + w.norm);
+    if (packed_already) {
+        MexPackTwin tw;
+        packed_at = reinterpret_cast<char *>(const_cast<void *>(saved));
+        mex_grad_pack_layout(p, packed_at, &tw, &norm_at);
+    }
     int rc = SIMNETS_OK;
     if (pack_normalizes)
-        ga.off = reinterpret_cast<const float *>(ws + w.norm);
+        ga.off = norm_at;
     else
         rc = prepare_offsets(p, offsets, ws + w.norm, s, &ga.off);
     if (rc)
@@ -1713,8 +1733,8 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     if (grad_is_pooled && !mex_grads_take_pooled(p, input, output, output_grad, input_grad))
         return SIMNETS_ERR_ALGO;   // (the callers ask first)
     if (t.mfma) {
-        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, ws + w.packed, &ga.k, stream, nullptr, true,
-                              pack_normalizes ? reinterpret_cast<float *>(ws + w.norm) : nullptr);
+        rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed_at, &ga.k, stream, nullptr,
+                              !packed_already, pack_normalizes ? norm_at : nullptr);
         if (rc)
             return rc;
         if (w.use_factors && !use_rows) {

@@ -316,6 +316,41 @@ at::Tensor mex_call(const simnets_mex_attrs &a, const at::Tensor &input, const a
     return y;
 }
 
+// the buffer a saving forward call fills for the gradient call (empty when the layer's gradient kernels read none)
+at::Tensor saved_buffer(const simnets_mex_attrs &a, const Shape4 &xs, const at::Tensor &like)
+{
+    size_t nbytes = 0;
+    check(simnets_hip_mex_saved_bytes(&a, xs.v, &nbytes));
+    return at::empty({(int64_t)nbytes}, like.options().dtype(at::kByte));
+}
+std::pair<const void *, size_t> saved_arg(const c10::optional<at::Tensor> &saved)
+{
+    if (!saved.has_value() || !saved->defined() || saved->numel() == 0)
+        return {nullptr, 0};
+    if (saved->scalar_type() != at::kByte || !saved->is_contiguous() || !saved->is_cuda())
+        throw SimnetsStatus(SIMNETS_ERR_SHAPE);
+    return {saved->data_ptr(), (size_t)saved->numel()};
+}
+
+// ... for training: (output, the offsets as the gradient call reads them)
+std::tuple<at::Tensor, at::Tensor> mex_saving_call(const simnets_mex_attrs &a, const at::Tensor &input,
+                                                   const at::Tensor &offsets)
+{
+    const at::Tensor x = dense("input", input), off = dense("offsets", offsets);
+    const Shape4 xs = shape4(x);
+    int os[4];
+    check(simnets_mex_out_shape(&a, xs.v, os, nullptr));
+    size_t nbytes = 0;
+    check(simnets_hip_mex_workspace_bytes(&a, xs.v, &nbytes));
+    at::Tensor y = output_like(x, os, c10::nullopt), saved = saved_buffer(a, xs, x);
+    Launch l(x);
+    const auto wsp = l.workspace(nbytes, x);
+    check(simnets_hip_mex_fwd_saving(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ptr(y),
+                                     saved.numel() ? saved.data_ptr() : nullptr, (size_t)saved.numel(), wsp.first,
+                                     wsp.second, l.stream));
+    return {y, saved};
+}
+
 void mex_grad_setup(const simnets_mex_attrs &a, const at::Tensor &x, const at::Tensor &y, const at::Tensor &g, Shape4 &xs)
 {
     xs = shape4(x);
@@ -362,7 +397,8 @@ at::Tensor mex_offsets_grad_call(const simnets_mex_attrs &a, const at::Tensor &i
 
 std::tuple<at::Tensor, at::Tensor> mex_grads_call(const simnets_mex_attrs &a, const at::Tensor &input,
                                                   const at::Tensor &offsets, const at::Tensor &output,
-                                                  const at::Tensor &grad)
+                                                  const at::Tensor &grad,
+                                                  const c10::optional<at::Tensor> &saved = c10::nullopt)
 {
     const at::Tensor x = dense("input", input), off = dense("offsets", offsets), y = dense("output", output),
                      g = dense("output_grad", grad);
@@ -373,8 +409,9 @@ std::tuple<at::Tensor, at::Tensor> mex_grads_call(const simnets_mex_attrs &a, co
     at::Tensor dx = at::empty_like(x), doff = at::empty_like(off);
     Launch l(x);
     const auto wsp = l.workspace(nbytes, x);
-    check(simnets_hip_mex_grads(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ptr(y), ptr(g), ptr(dx), ptr(doff),
-                                wsp.first, wsp.second, l.stream));
+    const auto sv = saved_arg(saved);
+    check(simnets_hip_mex_grads_saved(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ptr(y), ptr(g), sv.first, sv.second,
+                                      ptr(dx), ptr(doff), wsp.first, wsp.second, l.stream));
     return {dx, doff};
 }
 
@@ -415,11 +452,34 @@ std::tuple<at::Tensor, at::Tensor> mex_sum_pool_both_call(const simnets_mex_attr
     return {full, y};
 }
 
+// ... and the offsets as the gradient call reads them
+std::tuple<at::Tensor, at::Tensor, at::Tensor> mex_sum_pool_saving_call(const simnets_mex_attrs &a,
+                                                                        const at::Tensor &input,
+                                                                        const at::Tensor &offsets, int ph, int pw)
+{
+    const at::Tensor x = dense("input", input), off = dense("offsets", offsets);
+    const Shape4 xs = shape4(x);
+    int os[4];
+    check(simnets_mex_out_shape(&a, xs.v, os, nullptr));
+    size_t nbytes = 0;
+    check(simnets_hip_mex_sum_pool_workspace_bytes(&a, xs.v, ph, pw, &nbytes));
+    const int ps[4] = {os[0], os[1], os[2] / ph, os[3] / pw};
+    at::Tensor full = output_like(x, os, c10::nullopt), y = output_like(x, ps, c10::nullopt),
+               saved = saved_buffer(a, xs, x);
+    Launch l(x);
+    const auto wsp = l.workspace(nbytes, x);
+    check(simnets_hip_mex_sum_pool_fwd_saving(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ph, pw, ptr(full), ptr(y),
+                                              saved.numel() ? saved.data_ptr() : nullptr, (size_t)saved.numel(),
+                                              wsp.first, wsp.second, l.stream));
+    return {full, y, saved};
+}
+
 // the gradients of that pair from the gradient of the pooled output; a gradient that is not wanted is an undefined tensor
 std::tuple<at::Tensor, at::Tensor> mex_sum_pool_grads_call(const simnets_mex_attrs &a, const at::Tensor &input,
                                                            const at::Tensor &offsets, const at::Tensor &mex_output,
                                                            const at::Tensor &pooled_grad, int ph, int pw,
-                                                           bool want_input, bool want_offsets)
+                                                           bool want_input, bool want_offsets,
+                                                           const c10::optional<at::Tensor> &saved)
 {
     const at::Tensor x = dense("input", input), off = dense("offsets", offsets), y = dense("mex_output", mex_output),
                      g = dense("pooled_output_grad", pooled_grad);
@@ -439,9 +499,10 @@ std::tuple<at::Tensor, at::Tensor> mex_sum_pool_grads_call(const simnets_mex_att
     at::Tensor dx = want_input ? at::empty_like(x) : at::Tensor(), doff = want_offsets ? at::empty_like(off) : at::Tensor();
     Launch l(x);
     const auto wsp = l.workspace(nbytes, x);
-    check(simnets_hip_mex_sum_pool_grads(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ph, pw, ptr(y), ptr(g),
-                                         want_input ? ptr(dx) : nullptr, want_offsets ? ptr(doff) : nullptr, wsp.first,
-                                         wsp.second, l.stream));
+    const auto sv = saved_arg(saved);
+    check(simnets_hip_mex_sum_pool_grads_saved(&a, xs.v, ptr(x), ptr(off), (size_t)off.numel(), ph, pw, ptr(y), ptr(g),
+                                               sv.first, sv.second, want_input ? ptr(dx) : nullptr,
+                                               want_offsets ? ptr(doff) : nullptr, wsp.first, wsp.second, l.stream));
     return {dx, doff};
 }
 
@@ -783,8 +844,31 @@ PYBIND11_MODULE(_simnets_native, m)
     });
     SIMNETS_MEX_GRAD("mex_input_grad", mex_input_grad_call)
     SIMNETS_MEX_GRAD("mex_offsets_grad", mex_offsets_grad_call)
-    SIMNETS_MEX_GRAD("mex_grads", mex_grads_call)
 #undef SIMNETS_MEX_GRAD
+    m.def("mex_grads", [](const at::Tensor &x, const at::Tensor &off, const at::Tensor &y, const at::Tensor &g, int n,
+                          py::object softmax, py::object padding, py::object strides, py::object blocks,
+                          py::object epsilon, py::object oob, py::object round_down, py::object unshared,
+                          py::object shared_region, py::object unshared_region, bool normalize, OptT saved) {
+        return mex_grads_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down, unshared,
+                                           shared_region, unshared_region, normalize),
+                              x, off, y, g, saved);
+    });
+    m.def("mex_saving",
+          [](const at::Tensor &x, const at::Tensor &off, int n, py::object softmax, py::object padding, py::object strides,
+             py::object blocks, py::object epsilon, py::object oob, py::object round_down, py::object unshared,
+             py::object shared_region, py::object unshared_region, bool normalize) {
+              return mex_saving_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down, unshared,
+                                                  shared_region, unshared_region, normalize),
+                                     x, off);
+          });
+    m.def("mex_sum_pool_saving",
+          [](const at::Tensor &x, const at::Tensor &off, int n, int ph, int pw, py::object softmax, py::object padding,
+             py::object strides, py::object blocks, py::object epsilon, py::object oob, py::object round_down,
+             py::object unshared, py::object shared_region, py::object unshared_region, bool normalize) {
+              return mex_sum_pool_saving_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down,
+                                                           unshared, shared_region, unshared_region, normalize),
+                                              x, off, ph, pw);
+          });
     m.def("mex_sum_pool",
           [](const at::Tensor &x, const at::Tensor &off, int n, int ph, int pw, py::object softmax, py::object padding,
              py::object strides, py::object blocks, py::object epsilon, py::object oob, py::object round_down,
@@ -805,10 +889,10 @@ PYBIND11_MODULE(_simnets_native, m)
           [](const at::Tensor &x, const at::Tensor &off, const at::Tensor &full, const at::Tensor &g, int n, int ph, int pw,
              bool want_input, bool want_offsets, py::object softmax, py::object padding, py::object strides,
              py::object blocks, py::object epsilon, py::object oob, py::object round_down, py::object unshared,
-             py::object shared_region, py::object unshared_region, bool normalize) {
+             py::object shared_region, py::object unshared_region, bool normalize, OptT saved) {
               return mex_sum_pool_grads_call(mex_attrs_py(n, softmax, padding, strides, blocks, epsilon, oob, round_down,
                                                           unshared, shared_region, unshared_region, normalize),
-                                             x, off, full, g, ph, pw, want_input, want_offsets);
+                                             x, off, full, g, ph, pw, want_input, want_offsets, saved);
           });
     // the attribute structs of the two-operator calls come from Python as dicts of keyword arguments
     auto sim_from_dict = [](const py::dict &d) {

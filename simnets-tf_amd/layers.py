@@ -46,17 +46,18 @@ class MexFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input, offsets, num_instances, attrs):
         ctx.attrs, ctx.num_instances = attrs, num_instances
-        out = ops.mex(input, offsets, num_instances, **attrs)
-        ctx.save_for_backward(input, offsets, out)
+        # (the call also keeps the offsets as the gradient kernels read them)
+        out, packed = ops.mex_saving(input, offsets, num_instances, **attrs)
+        ctx.save_for_backward(input, offsets, out, packed)
         return out
 
     @staticmethod
     def backward(ctx, grad):
-        input, offsets, out = ctx.saved_tensors
+        input, offsets, out, packed = ctx.saved_tensors
         grad = grad.contiguous()
         gi = go = None
         if ctx.needs_input_grad[0] and ctx.needs_input_grad[1]:
-            gi, go = ops.mex_grads(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
+            gi, go = ops.mex_grads(input, offsets, out, grad, ctx.num_instances, saved=packed, **ctx.attrs)
         elif ctx.needs_input_grad[0]:
             gi = ops.mex_input_grad(input, offsets, out, grad, ctx.num_instances, **ctx.attrs)
         elif ctx.needs_input_grad[1]:
@@ -66,21 +67,22 @@ class MexFunction(torch.autograd.Function):
 
 class MexSumPoolFunction(torch.autograd.Function):
     """`mex` followed by non-overlapping sum pooling as one forward call that also keeps the MEX output before pooling
-    (`ops.mex_sum_pool_both`): what the MEX gradient operators take."""
+    (what the MEX gradient operators take) and the offsets as the gradient kernels read them
+    (`ops.mex_sum_pool_saving`)."""
 
     @staticmethod
     def forward(ctx, input, offsets, num_instances, ph, pw, attrs):
         ctx.attrs, ctx.num_instances, ctx.pool = attrs, num_instances, (ph, pw)
-        full, pooled = ops.mex_sum_pool_both(input, offsets, num_instances, (ph, pw), **attrs)
-        ctx.save_for_backward(input, offsets, full)
+        full, pooled, packed = ops.mex_sum_pool_saving(input, offsets, num_instances, (ph, pw), **attrs)
+        ctx.save_for_backward(input, offsets, full, packed)
         return pooled
 
     @staticmethod
     def backward(ctx, grad):
-        input, offsets, full = ctx.saved_tensors
+        input, offsets, full, packed = ctx.saved_tensors
         gi, go = ops.mex_sum_pool_grads(input, offsets, full, grad.contiguous(), ctx.num_instances, ctx.pool,
                                         want_input=ctx.needs_input_grad[0], want_offsets=ctx.needs_input_grad[1],
-                                        **ctx.attrs)
+                                        saved=packed, **ctx.attrs)
         return gi, go, None, None, None, None
 
 

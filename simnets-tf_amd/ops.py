@@ -250,13 +250,26 @@ def mex_offsets_grad(input, offsets, output, output_grad, num_instances, softmax
 def mex_grads(input, offsets, output, output_grad, num_instances, softmax_mode=None, padding=None, strides=None,
               blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
               use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
-              normalize_offsets=False):
+              normalize_offsets=False, saved=None):
     """`(mex_input_grad(...), mex_offsets_grad(...))` as one call of the library: the same results bit for bit, with
     the work both share (offsets normalisation and packing, per-pixel factors) done once.  What the gradient
-    registered for the Mex op (python/simnets/ops/mex.py:47-81) computes."""
+    registered for the Mex op (python/simnets/ops/mex.py:47-81) computes.  `saved`: what `mex_saving` returned for
+    the same input shape, attributes and offsets values; the call then packs no offsets."""
     return _n.mex_grads(input, offsets, output, output_grad, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
                      blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
-                     unshared_offset_region, bool(normalize_offsets))
+                     unshared_offset_region, bool(normalize_offsets), saved)
+
+
+def mex_saving(input, offsets, num_instances, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
+               blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
+               shared_offset_region=None, unshared_offset_region=None, name=None, normalize_offsets=False):
+    """`mex(...)` for a training step: `(output, saved)`, where `saved` (a byte tensor, empty when the layer's
+    gradient kernels have no use for one) holds the offsets as the gradient kernels read them, written by the launch
+    that re-orders them for the forward kernel; `mex_grads(..., saved=saved)` then packs nothing.  The registered
+    gradient of the Mex op runs on the forward op's inputs (python/simnets/ops/mex.py:47-81)."""
+    return _n.mex_saving(input, offsets, int(num_instances), softmax_mode, padding, strides, blocks, epsilon,
+                         blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions, shared_offset_region,
+                         unshared_offset_region, bool(normalize_offsets))
 
 
 def mex_sum_pool(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
@@ -283,10 +296,23 @@ def mex_sum_pool_both(input, offsets, num_instances, pool_size=(2, 2), softmax_m
                                 bool(normalize_offsets))
 
 
+def mex_sum_pool_saving(input, offsets, num_instances, pool_size=(2, 2), softmax_mode=None, padding=None, strides=None,
+                        blocks=None, epsilon=None, blocks_out_of_bounds_value=None, blocks_round_down=None,
+                        use_unshared_regions=None, shared_offset_region=None, unshared_offset_region=None, name=None,
+                        normalize_offsets=False):
+    """`mex_sum_pool_both(...)` + `saved` as `mex_saving` returns it: `(mex_output, pooled, saved)`, for
+    `mex_sum_pool_grads(..., saved=saved)`."""
+    return _n.mex_sum_pool_saving(input, offsets, int(num_instances), int(pool_size[0]), int(pool_size[1]), softmax_mode,
+                                  padding, strides, blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down,
+                                  use_unshared_regions, shared_offset_region, unshared_offset_region,
+                                  bool(normalize_offsets))
+
+
 def mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, num_instances, pool_size=(2, 2), want_input=True,
                        want_offsets=True, softmax_mode=None, padding=None, strides=None, blocks=None, epsilon=None,
                        blocks_out_of_bounds_value=None, blocks_round_down=None, use_unshared_regions=None,
-                       shared_offset_region=None, unshared_offset_region=None, name=None, normalize_offsets=False):
+                       shared_offset_region=None, unshared_offset_region=None, name=None, normalize_offsets=False,
+                       saved=None):
     """The gradients of `mex_sum_pool` w.r.t. (input, offsets) from the gradient of the POOLED output and the MEX
     output before pooling (`mex_sum_pool_both`'s first result): `mex_grads(input, offsets, mex_output,
     sum_pooling_input_grad(pooled_output_grad, ...))` in one call, without the expanded gradient tensor on the layers
@@ -294,7 +320,7 @@ def mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, num_insta
     gi, go = _n.mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, int(num_instances), int(pool_size[0]),
                                    int(pool_size[1]), bool(want_input), bool(want_offsets), softmax_mode, padding, strides,
                                    blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions,
-                                   shared_offset_region, unshared_offset_region, bool(normalize_offsets))
+                                   shared_offset_region, unshared_offset_region, bool(normalize_offsets), saved)
     return (gi if want_input else None), (go if want_offsets else None)
 
 

@@ -1,4 +1,6 @@
 """The differentiable op layer and the module classes (python/simnets/keras.py of the reference) on the GPU."""
+import math
+
 import numpy as np
 import pytest
 import torch
@@ -288,6 +290,57 @@ def test_mex_sum_pool_grads_from_the_pooled_gradient(pkg, im, n, pool, kw, sprea
     assert float((doff_u - want_doff).abs().max()) <= 1e-4 * float(want_doff.abs().max())
     with pytest.raises(pkg.SimnetsError):
         pkg.mex_sum_pool_grads(x, off, full, gp[:, :, :-1], n, pool, **kw)
+
+
+@pytest.mark.parametrize("normalize", [False, True])
+@pytest.mark.parametrize("im,n,kw", [
+    ((64, 32, 16, 16), 64, {}),                            # one-launch forward that packs inside its kernel
+    ((8, 32, 16, 16), 70, {}),                             # instance count that pads both layouts differently (128 / 96)
+    ((16, 64, 8, 8), 128, {}),                             # panel kernel, row-wise gradient kernels
+    ((16, 256, 2, 2), 40, {}),                             # 2x2 maps: gathering gradient kernels
+    ((32, 100, 1, 1), 10, dict(unshared_offset_region=[1, 1, 1])),   # head: wave-per-pixel forward (groups of one)
+    ((3, 6, 9, 7), 21, dict(blocks=[3, 2, 2], strides=[2, 1, 1], padding=[1, 1, 0], unshared_offset_region=[2, 3, 2])),
+    ((4, 16, 8, 8), 33, dict(use_unshared_regions=False, shared_offset_region=[2])),
+    ((4, 16, 8, 8), 9, dict(epsilon=float("-inf"))),       # nothing to keep: the gradient kernels read the offsets
+    ((4, 600, 4, 4), 12, {}),                              # rows of more than 256 elements
+    ((0, 16, 8, 8), 5, {}),
+])
+def test_mex_forward_keeps_the_offsets_for_the_gradient_call(pkg, im, n, kw, normalize):
+    """`mex_saving` / `mex_sum_pool_saving` = the plain forward calls, and the gradient calls given what they kept =
+    the plain gradient calls, all bit for bit; the kept buffer stays valid while other layers run on the stream (it is
+    no part of the calls' scratch)."""
+    g = torch.Generator(device="cuda").manual_seed(5)
+    kw = dict(dict(softmax_mode=True, blocks=[im[1], 1, 1], strides=[im[1], 1, 1], unshared_offset_region=[1, 2, 2],
+                   epsilon=1.5, normalize_offsets=normalize), **kw)
+    x = torch.randn(im, device="cuda", generator=g)
+    _, oshape = pkg.mex_output_shape(im, n, **{k: v for k, v in kw.items() if k != "normalize_offsets"})
+    off = torch.randn(oshape, device="cuda", generator=g)
+    off[:, ::3] *= 40           # some instances beyond the product form
+    y = pkg.mex(x, off, n, **kw)
+    ys, kept = pkg.mex_saving(x, off, n, **kw)
+    assert torch.equal(y, ys) and kept.dtype == torch.uint8
+    assert (kept.numel() == 0) == (not math.isfinite(kw["epsilon"]))
+    # another layer in between: its calls reuse the scratch of this one's
+    other = pkg.mex(torch.randn(5, 8, 6, 6, device="cuda"), torch.randn(1, 3, 8, 1, 1, device="cuda"), 3,
+                    blocks=[8, 1, 1], strides=[8, 1, 1], use_unshared_regions=False, shared_offset_region=[-1])
+    gy = torch.randn(y.shape, device="cuda", generator=g)
+    want = pkg.mex_grads(x, off, y, gy, n, **kw)
+    got = pkg.mex_grads(x, off, y, gy, n, saved=kept, **kw)
+    assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+    assert other.shape == (5, 3, 6, 6)
+    if y.shape[2] >= 2 and y.shape[3] >= 2:
+        full, pooled = pkg.mex_sum_pool_both(x, off, n, (2, 2), **kw)
+        fulls, pooleds, kept2 = pkg.mex_sum_pool_saving(x, off, n, (2, 2), **kw)
+        assert torch.equal(full, fulls) and torch.equal(pooled, pooleds)
+        gp = torch.randn(pooled.shape, device="cuda", generator=g)
+        want = pkg.mex_sum_pool_grads(x, off, full, gp, n, (2, 2), **kw)
+        got = pkg.mex_sum_pool_grads(x, off, full, gp, n, (2, 2), saved=kept2, **kw)
+        assert torch.equal(got[0], want[0]) and torch.equal(got[1], want[1])
+        only = pkg.mex_sum_pool_grads(x, off, full, gp, n, (2, 2), want_input=False, saved=kept2, **kw)
+        assert only[0] is None and torch.equal(only[1], want[1])
+    if kept.numel():
+        with pytest.raises(pkg.SimnetsError):   # a buffer that is too small
+            pkg.mex_grads(x, off, y, gy, n, saved=kept[:256], **kw)
 
 
 @pytest.mark.parametrize("shape,pool", [((3, 5, 8, 10), (2, 2)), ((2, 3, 7, 9), (2, 3)), ((1, 4, 5, 5), (5, 1))])
