@@ -526,7 +526,14 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
     // a wave per (region, instance) with the instances padded to the groups of the layout (of the wider of the two
     // layouts when the launch writes a second one)
     const int lane = threadIdx.x & 63;
-    const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    // Workgroups go to the chip's eight dies in turn, each with an L2 of its own, and the 64 rows of a packed group
+    // interleave in 4-byte pieces of the same cache lines: the 16 workgroups of such a group are numbered 8 apart, so
+    // that one die's L2 collects their pieces into whole lines (pieces of a line written from several dies each reach
+    // memory as a partial line).
+    unsigned wg = blockIdx.x;
+    if (wg < ((unsigned)row_blocks & ~127u))
+        wg = (((wg >> 7) * 8 + (wg & 7)) << 4) + ((wg >> 3) & 15);
+    const long long wave = (long long)wg * 4 + (threadIdx.x >> 6);
     const int Mp = n_mgroups * tm, Mp2 = tw.offp != nullptr ? tw.n_mgroups * tw.tm : 0;
     const int Mw = max(Mp, Mp2);
     if (wave >= (long long)R * Mw)
