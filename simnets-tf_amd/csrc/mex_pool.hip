@@ -35,6 +35,8 @@ constexpr int kSimTaps = 16;       // longest Similarity patch the kernel evalua
 struct PoolArgs {
     float *pooled;
     float *full;  // not null: the MEX values before pooling are stored there as well, [B][M * Co][Ho][Wo]
+    int full_pairs, out_pairs;  // `full` / the unpooled output of the panel form may be stored 8 bytes at a time
+                                // (aligned, even row length: the two regions of a window row are one float2)
     int Hp, Wp;   // pooled height and width
     int spw;      // slots per workgroup: NH * 64 / R
     // SIMF: the MEX input is the output of a Similarity layer that is evaluated on the fly
@@ -419,16 +421,31 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     if (q.full != nullptr) {
         // the MEX output itself, for the gradient operators: tile t = (slot group t / R, region t % R)
         const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+        if (R == 4 && q.full_pairs) {
+            // regions 2 ry and 2 ry + 1 of a window are neighbours in a row: one 8-byte store
 #pragma unroll
-        for (int t = 0; t < 4; ++t) {
-            const PixelRef cp = locate(a, t % R, (chunk * NH + wh) * (16 * G) + (t / R) * 16 + lr);
-            if (cp.out_off < 0)
-                continue;
-            float *o = q.full + (size_t)cp.b * a.M * plane + cp.out_off + (size_t)(m0 + 4 * lq) * plane;
+            for (int ry = 0; ry < 2; ++ry) {
+                const PixelRef cp = locate(a, 2 * ry, (chunk * NH + wh) * 16 + lr);
+                if (cp.out_off < 0)
+                    continue;
+                float *o = q.full + (size_t)cp.b * a.M * plane + cp.out_off + (size_t)(m0 + 4 * lq) * plane;
 #pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (all_rows || m0 + 4 * lq + v < a.M)
-                    o[v * plane] = res[t][v];
+                for (int v = 0; v < 4; ++v)
+                    if (all_rows || m0 + 4 * lq + v < a.M)
+                        *reinterpret_cast<float2 *>(o + v * plane) = make_float2(res[2 * ry][v], res[(2 * ry + 1) % 4][v]);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const PixelRef cp = locate(a, t % R, (chunk * NH + wh) * (16 * G) + (t / R) * 16 + lr);
+                if (cp.out_off < 0)
+                    continue;
+                float *o = q.full + (size_t)cp.b * a.M * plane + cp.out_off + (size_t)(m0 + 4 * lq) * plane;
+#pragma unroll
+                for (int v = 0; v < 4; ++v)
+                    if (all_rows || m0 + 4 * lq + v < a.M)
+                        o[v * plane] = res[t][v];
+            }
         }
     }
     // ---- sum over the window (one pixel per region, row-major) and store the pooled pixel ----
@@ -462,6 +479,28 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
 // LDS tiles are stored with column ^ swizzle(k): bits 4-5 of the column take k & 3, so that the four k rows a matrix
 // instruction's operand fetch touches (lane >> 4) fall into different banks; for the panel tile bits 2-3 take
 // (k >> 2) & 3 as well, which spreads the lanes of the staging writes that hold one column at 16 different k.
+// The four MEX values of a 2x2 window (region t = pixel (t / 2, t % 2)) for instances v < live, planes `plane`
+// floats apart: the two pixels of a window row as one 8-byte store where the tensor allows it.
+__device__ __forceinline__ void store_window(float *o, size_t plane, int lgW, int pairs, const float (&res)[4][4], int live)
+{
+    if (pairs) {
+#pragma unroll
+        for (int ry = 0; ry < 2; ++ry)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (v < live)
+                    *reinterpret_cast<float2 *>(o + v * plane + ((size_t)ry << lgW)) =
+                        make_float2(res[2 * ry][v], res[2 * ry + 1][v]);
+    } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                if (v < live)
+                    o[v * plane + ((size_t)(t >> 1) << lgW) + (t & 1)] = res[t][v];
+    }
+}
+
 constexpr int kPanelWorkgroups = 256;   // below this many two-half workgroups (one per compute unit) the panel form runs one-half ones
 
 struct PanelArgs {
@@ -856,21 +895,10 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         if (q.full != nullptr) {
             // ... and the MEX values themselves, for the gradient operators (region t = pixel (t / 2, t % 2))
             float *f = q.full + fpos[wh * 16 + lr] + (size_t)(m0 + 4 * lq) * g.HW;
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-#pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    if (all_rows || m0 + 4 * lq + v < a.M)
-                        f[(size_t)v * g.HW + ((size_t)(t >> 1) << g.lgW) + (t & 1)] = res[t][v];
+            store_window(f, g.HW, g.lgW, q.full_pairs, res, all_rows ? 4 : a.M - (m0 + 4 * lq));
         }
     } else {
-        // region t is pixel (t / 2, t % 2) of the window
-#pragma unroll
-        for (int t = 0; t < 4; ++t)
-#pragma unroll
-            for (int v = 0; v < 4; ++v)
-                if (all_rows || m0 + 4 * lq + v < a.M)
-                    o[v * plane_p + ((size_t)(t >> 1) << g.lgW) + (t & 1)] = res[t][v];
+        store_window(o, plane_p, g.lgW, q.out_pairs, res, all_rows ? 4 : a.M - (m0 + 4 * lq));
     }
 }
 
@@ -988,6 +1016,8 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     PoolArgs q;
     q.sx = nullptr;
     q.full = full;
+    q.full_pairs = full != nullptr && reinterpret_cast<uintptr_t>(full) % 8 == 0 && d.width_out % 2 == 0;
+    q.out_pairs = 0;
     SimPackJob job;
     if (sp) {
         float *pa = reinterpret_cast<float *>(reinterpret_cast<char *>(workspace) + mex_packed_bytes(p, TM, n_mgroups));
@@ -1061,6 +1091,8 @@ int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *inpu
     PoolArgs q;
     q.sx = nullptr;
     q.full = nullptr;
+    q.full_pairs = 0;
+    q.out_pairs = reinterpret_cast<uintptr_t>(output) % 8 == 0;
     q.pooled = output;
     q.Hp = p.d.height_out / 2;
     q.Wp = p.d.width_out / 2;
@@ -1089,6 +1121,8 @@ int mex_panel_launch_selfpack(const MexPlan &p, const MexKernelArgs &a, const fl
     PoolArgs q;
     q.sx = nullptr;
     q.full = nullptr;
+    q.full_pairs = 0;
+    q.out_pairs = reinterpret_cast<uintptr_t>(output) % 8 == 0;
     q.pooled = output;
     q.Hp = p.d.height_out / 2;
     q.Wp = p.d.width_out / 2;

@@ -493,3 +493,47 @@ def test_modules_notice_rebound_parameters_changed_attributes_and_other_streams(
     with torch.no_grad():
         mexl(sim(x))
     assert sim._prepared.last(pkg.ops._current_stream(x.device)) is main
+
+
+@pytest.mark.parametrize("im,n", [((64, 32, 16, 16), 64),      # panel form, one chunk
+                                  ((16, 64, 8, 8), 128),       # panel form, two halves
+                                  ((40, 16, 8, 8), 20)])       # fused kernel
+def test_mex_outputs_that_are_only_4_byte_aligned(pkg, im, n):
+    """The kernels store the two pixels of a window row as one 8-byte piece where the output tensor allows it: outputs
+    (the MEX output, the pooled output, the unpooled output of the fused call) a float off that alignment, passed
+    through the C ABI, hold the same values."""
+    import ctypes as C
+    from simnets_tf_amd import _lib, ops
+    l = _lib.lib()
+    kw = dict(softmax_mode=True, blocks=[im[1], 1, 1], strides=[im[1], 1, 1], unshared_offset_region=[1, 2, 2], epsilon=1.5)
+    g = torch.Generator(device="cuda").manual_seed(9)
+    x = torch.randn(im, device="cuda", generator=g)
+    _, oshape = pkg.mex_output_shape(im, n, **kw)
+    off = torch.randn(oshape, device="cuda", generator=g)
+    want = pkg.mex(x, off, n, **kw)
+    want_full, want_pooled = pkg.mex_sum_pool_both(x, off, n, (2, 2), **kw)
+    a = ops.mex_attrs(n, **kw)
+    xs = (C.c_int * 4)(*im)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def off_by_one(shape):
+        buf = torch.zeros(int(np.prod(shape)) + 1, device="cuda")
+        v = buf[1:].view(tuple(shape))
+        assert v.data_ptr() % 8 == 4
+        return v
+
+    nbytes = C.c_size_t()
+    assert l.simnets_hip_mex_workspace_bytes(C.byref(a), xs, C.byref(nbytes)) == 0
+    ws = torch.empty(max(nbytes.value, 256), dtype=torch.uint8, device="cuda")
+    y = off_by_one(want.shape)
+    rc = l.simnets_hip_mex_fwd(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), y.data_ptr(), ws.data_ptr(),
+                               ws.numel(), stream)
+    assert rc == 0, _lib.strerror(rc)
+    assert torch.equal(y, want)
+    assert l.simnets_hip_mex_sum_pool_workspace_bytes(C.byref(a), xs, 2, 2, C.byref(nbytes)) == 0
+    ws = torch.empty(max(nbytes.value, 256), dtype=torch.uint8, device="cuda")
+    full, pooled = off_by_one(want_full.shape), off_by_one(want_pooled.shape)
+    rc = l.simnets_hip_mex_sum_pool_fwd_both(C.byref(a), xs, x.data_ptr(), off.data_ptr(), off.numel(), 2, 2,
+                                             full.data_ptr(), pooled.data_ptr(), ws.data_ptr(), ws.numel(), stream)
+    assert rc == 0, _lib.strerror(rc)
+    assert torch.equal(full, want_full) and torch.equal(pooled, want_pooled)
