@@ -474,6 +474,38 @@ __global__ __launch_bounds__(256) void mex_sum_splits_kernel(const float *__rest
     }
 }
 
+// ... four elements per thread with all the splits' loads (at most 8) in flight together: n a multiple of 4, 16-byte
+// aligned pointers.  The same additions in the same order.
+__global__ __launch_bounds__(256) void mex_sum_splits4_kernel(const float4 *__restrict__ parts, long long n4, int splits,
+                                                             float4 *__restrict__ dx)
+{
+    const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+    if (i >= n4)
+        return;
+    float4 v[8];
+#pragma unroll
+    for (int z = 0; z < 8; ++z)
+        v[z] = parts[(size_t)min(z, splits - 1) * n4 + i];
+    float4 s = v[0];
+#pragma unroll
+    for (int z = 1; z < 8; ++z)
+        if (z < splits) {
+            s.x += v[z].x; s.y += v[z].y; s.z += v[z].z; s.w += v[z].w;
+        }
+    dx[i] = s;
+}
+
+void launch_sum_splits(const float *parts, long long n, int splits, float *dx, hipStream_t s)
+{
+    if (splits <= 8 && n % 4 == 0 && reinterpret_cast<uintptr_t>(parts) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(dx) % 16 == 0 && (n / 4 + 255) / 256 <= 0x7fffffffLL)
+        hipLaunchKernelGGL(mex_sum_splits4_kernel, dim3((unsigned)((n / 4 + 255) / 256)), dim3(256), 0, s,
+                           reinterpret_cast<const float4 *>(parts), n / 4, splits, reinterpret_cast<float4 *>(dx));
+    else
+        hipLaunchKernelGGL(mex_sum_splits_kernel, dim3((unsigned)std::min<long long>((n + 255) / 256, 65535)), dim3(256),
+                           0, s, parts, n, splits, dx);
+}
+
 // Overlapping patches: input gradient = sum, over the patches that cover the element, of the patch-element
 // gradients in `col` (the reference's col2im_3d, src/utils/im2col.cpp:297-328), patches in ascending (c, h, w)
 // order.  One thread per input element; elements no patch covers get 0.
@@ -1358,6 +1390,50 @@ __global__ __launch_bounds__(256) void mex_normalize_rows_backward_kernel(const 
         gr[k] -= expf(n[k]) * sum;
 }
 
+// Elements lane, lane + 64, ... of one row of the offsets gradient from its partial sums (eight interleaved sums in
+// chunk order, added in order), E elements at a time; returns the lane's share of the row sum (in element order).
+template <int E>
+__device__ __forceinline__ float finish_long_row(const float *__restrict__ pr, float *__restrict__ gr, long long n,
+                                                 int chunks, int K, int lane)
+{
+    float sum = 0.0f;
+    for (int k0 = lane; k0 < K; k0 += 64 * E) {
+        float s8[E][8];
+#pragma unroll
+        for (int e = 0; e < E; ++e)
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                s8[e][j] = 0.0f;
+        for (int c0 = 0; c0 < chunks; c0 += 8) {
+            // all requests first, those past the last chunk or the row's end on a valid address (a load inside the
+            // condition would be waited for before the next one is issued)
+            float v[E][8];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    v[e][j] = pr[(size_t)min(c0 + j, chunks - 1) * n + min(k0 + 64 * e, K - 1)];
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    s8[e][j] = c0 + j < chunks ? s8[e][j] + v[e][j] : s8[e][j];
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            float t = s8[e][0];
+#pragma unroll
+            for (int j = 1; j < 8; ++j)
+                t += s8[e][j];
+            if (k0 + 64 * e < K) {
+                gr[k0 + 64 * e] = t;
+                sum += t;
+            }
+        }
+    }
+    return sum;
+}
+
 // Both of the above for short rows, one wave per (region, instance) row: element k of the row is the sum of its
 // partial sums in the order of mex_grad_offsets_finish_kernel (eight interleaved sums in chunk order, added in
 // order), then, if `normalized` is given, the chain rule of mex_normalize_rows_backward_kernel with the same
@@ -1375,6 +1451,59 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_finish_rows_kernel(const
     float *gr = doff + (size_t)row * K;
     const float *pr = partial + (size_t)row * K;
     float sum = 0.0f;
+    if (K <= 32 && (K & 3) == 0) {
+        // short rows of whole 16-byte pieces: lane (q, j) = (lane & 7, lane >> 3) takes piece q (elements 4 q ... 4 q + 3)
+        // of the chunks j, j + 8, ... - the interleaved sum j -, eight of them requested at a time; lane (q, 0) then
+        // adds the eight sums in order.  The values are those of the loops below.
+        const int Kq = K >> 2, q = lane & 7, j = lane >> 3, qc = min(q, Kq - 1);
+        const long long n4 = n >> 2;
+        const float4 *pr4 = reinterpret_cast<const float4 *>(pr) + qc;
+        float4 sj = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int c0 = j; c0 < chunks; c0 += 64) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                v[u] = pr4[(size_t)min(c0 + 8 * u, chunks - 1) * n4];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (c0 + 8 * u < chunks) {
+                    sj.x += v[u].x; sj.y += v[u].y; sj.z += v[u].z; sj.w += v[u].w;
+                }
+        }
+        float4 t4 = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int jj = 0; jj < 8; ++jj) {
+            const float4 val = make_float4(__shfl(sj.x, q + 8 * jj, 64), __shfl(sj.y, q + 8 * jj, 64),
+                                           __shfl(sj.z, q + 8 * jj, 64), __shfl(sj.w, q + 8 * jj, 64));
+            if (jj == 0)
+                t4 = val;
+            else {
+                t4.x += val.x; t4.y += val.y; t4.z += val.z; t4.w += val.w;
+            }
+        }
+        if (normalized == nullptr) {
+            if (j == 0 && q < Kq) {
+                if ((reinterpret_cast<uintptr_t>(gr) & 15) == 0)
+                    reinterpret_cast<float4 *>(gr)[q] = t4;
+                else {
+                    gr[4 * q] = t4.x; gr[4 * q + 1] = t4.y; gr[4 * q + 2] = t4.z; gr[4 * q + 3] = t4.w;
+                }
+            }
+            return;
+        }
+        // element k to lane k (it lives in lane k / 4), then the row sum and the chain rule as below
+        const int k = lane & 31;
+        const float a0 = __shfl(t4.x, k >> 2, 64), a1 = __shfl(t4.y, k >> 2, 64), a2 = __shfl(t4.z, k >> 2, 64),
+                    a3 = __shfl(t4.w, k >> 2, 64);
+        const float t = (k & 3) == 0 ? a0 : (k & 3) == 1 ? a1 : (k & 3) == 2 ? a2 : a3;
+        const bool owner = lane < K;
+        sum = owner ? t : 0.0f;
+        for (int d = 32; d > 0; d >>= 1)
+            sum += __shfl_xor(sum, d, 64);
+        if (owner)
+            gr[k] = t - expf(normalized[(size_t)row * K + k]) * sum;
+        return;
+    }
     if (K <= 32) {
         // rows shorter than a wave: the lanes form 64 / Kp groups (Kp = 8, 16 or 32 >= K) that each take 8 / groups
         // of the eight interleaved sums, four rounds of chunks requested at a time; every lane then adds the eight
@@ -1418,29 +1547,13 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_finish_rows_kernel(const
             gr[k] = t - expf(normalized[(size_t)row * K + k]) * sum;
         return;
     }
-    for (int k = lane; k < K; k += 64) {
-        float s8[8];
-#pragma unroll
-        for (int j = 0; j < 8; ++j)
-            s8[j] = 0.0f;
-        for (int c0 = 0; c0 < chunks; c0 += 8) {
-            // all eight requests first, those past the last chunk on its address (a load inside the condition
-            // would be waited for before the next one is issued)
-            float v[8];
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                v[j] = pr[(size_t)min(c0 + j, chunks - 1) * n + k];
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-                s8[j] = c0 + j < chunks ? s8[j] + v[j] : s8[j];
-        }
-        float t = s8[0];
-#pragma unroll
-        for (int j = 1; j < 8; ++j)
-            t += s8[j];
-        gr[k] = t;
-        sum += t;
-    }
+    // up to four elements of the row per lane at a time (64 apart): 8 requests each in flight
+    if (K <= 64)
+        sum = finish_long_row<1>(pr, gr, n, chunks, K, lane);
+    else if (K <= 128)
+        sum = finish_long_row<2>(pr, gr, n, chunks, K, lane);
+    else
+        sum = finish_long_row<4>(pr, gr, n, chunks, K, lane);
     if (normalized == nullptr)
         return;
     for (int d = 32; d > 0; d >>= 1)
@@ -1785,9 +1898,7 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
             if (t.rows_msplit > 1) {
                 if (hipGetLastError() != hipSuccess)
                     return SIMNETS_ERR_HIP;
-                hipLaunchKernelGGL(mex_sum_splits_kernel,
-                                   dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)), dim3(256), 0, s,
-                                   gi.dx_splits, n_in, t.rows_msplit, input_grad);
+                launch_sum_splits(gi.dx_splits, n_in, t.rows_msplit, input_grad, s);
             }
         } else if (t.mfma) {
             const int gy = (d.K + GM_KT - 1) / GM_KT;
@@ -1799,9 +1910,7 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
             if (gx > 0 && t.msplit > 1) {
                 if (hipGetLastError() != hipSuccess)
                     return SIMNETS_ERR_HIP;
-                hipLaunchKernelGGL(mex_sum_splits_kernel,
-                                   dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)), dim3(256), 0, s,
-                                   gi.dx_splits, n_in, t.msplit, input_grad);
+                launch_sum_splits(gi.dx_splits, n_in, t.msplit, input_grad, s);
             }
         } else {
             const int gy = (d.K + 4 * GX_KT - 1) / (4 * GX_KT);

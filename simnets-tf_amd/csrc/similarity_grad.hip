@@ -1504,13 +1504,29 @@ __global__ __launch_bounds__(256) void sim_grad_params_finish_kernel(
     // where the sum of g lives: per (o, k) with ignore-NaN, else once per template (see the kernel's epilogue)
     const size_t gsrc = moment && !ign ? (size_t)o * Kpad : src;
     float st = 0.0f, sw = 0.0f, sn = 0.0f;
-    if (live)
-        for (int s = grp; s < S; s += G) {
-            st += partial[(size_t)s * slab + src];
-            sw += partial[((size_t)S + s) * slab + src];
-            if (norm || moment)
-                sn += partial[((size_t)2 * S + s) * slab + gsrc];
+    if (live) {
+        // eight splits' loads in flight at a time (a load per addition would be waited for each in turn); the additions
+        // keep their order, a split past the end adds 0
+        const bool third = norm || moment;
+        for (int s0 = grp; s0 < S; s0 += 8 * G) {
+            float a[8], b[8], c[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int s = s0 + u * G;
+                const int sc = s < S ? s : grp;
+                a[u] = partial[(size_t)sc * slab + src];
+                b[u] = partial[((size_t)S + sc) * slab + src];
+                c[u] = third ? partial[((size_t)2 * S + sc) * slab + gsrc] : 0.0f;
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const bool in = s0 + u * G < S;
+                st += in ? a[u] : 0.0f;
+                sw += in ? b[u] : 0.0f;
+                sn += in ? c[u] : 0.0f;
+            }
         }
+    }
     sm[0][threadIdx.x] = st; sm[1][threadIdx.x] = sw; sm[2][threadIdx.x] = sn;
     __syncthreads();
     if (grp != 0 || !live)
