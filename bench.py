@@ -441,26 +441,34 @@ def main():
                     "the fractions are taken on kernel_ms; the eager figures are back-to-back calls through the "
                     "Python op layer, bounded by the host's share of a call"})
 
-        # ---- the same layer on the paths that do not take the product form: offsets too far apart for it (every row's
-        #      scaled range far above 90: a max-tracked log-sum-exp on the VALU from the staged tiles) and an infinite
-        #      epsilon (the maximum alone)
+        # ---- the same layer with offsets too far apart for the product form on their own (every row's scaled range far
+        #      above 90): still the product form while every pixel's patch spans at most 90 (the largest term is then
+        #      bounded through the patch instead), a max-tracked log-sum-exp on the VALU from the staged tiles when the
+        #      patches are wide as well (input x 40); and an infinite epsilon (the maximum alone)
+        OTHER_FORMS = {"wide_offsets": "rows beyond the product form's range, pixel patches within it: product form",
+                       "wide_offsets_wide_pixels": "rows and pixel patches beyond it: max-tracked log-sum-exp on the VALU",
+                       "eps_inf": "the maximum alone"}
+
         def other_forms(tag, X, off_np, n, kw, gmac, nbytes, shape_out):
             """device time per prepared call (HIP graph of 20) of the product form, wide offsets and eps = inf"""
             res = {}
             o = torch.empty(shape_out, device=dev)
-            variants = (("product_form", off_np, kw), ("wide_offsets", off_np * 1000.0, kw),
-                        ("eps_inf", off_np, dict(kw, epsilon=math.inf)))
-            for name, off_v, kw_v in variants:
+            variants = (("product_form", off_np, kw, 1.0), ("wide_offsets", off_np * 1000.0, kw, 1.0),
+                        ("wide_offsets_wide_pixels", off_np * 1000.0, kw, 40.0),
+                        ("eps_inf", off_np, dict(kw, epsilon=math.inf), 1.0))
+            for name, off_v, kw_v, xscale in variants:
                 OV = to_dev(off_v.astype(np.float32))
+                XV = X if xscale == 1.0 else X * xscale
                 prep = pkg.mex_prepare(tuple(X.shape), OV, n, normalize_offsets=True, **kw_v)
-                _, ms_v = timed(graph_of(lambda: prep(X, out=o), 20).replay, args.steps, args.warmup)
-                res[name] = (ms_v / 20, OV, kw_v, o.clone())
+                _, ms_v = timed(graph_of(lambda: prep(XV, out=o), 20).replay, args.steps, args.warmup)
+                res[name] = (ms_v / 20, OV, kw_v, o.clone(), xscale)
             base = res["product_form"][0]
             out = {}
-            for name in ("wide_offsets", "eps_inf"):
+            for name, what in OTHER_FORMS.items():
                 ms_v = res[name][0]
                 e = entry(ms_v, gmac, nbytes, "hbm", flop=5, mex=True)
-                e.update({"product_form_kernel_ms": round(base, 4), "ratio_to_product_form": round(ms_v / base, 2),
+                e.update({"what": what, "product_form_kernel_ms": round(base, 4),
+                          "ratio_to_product_form": round(ms_v / base, 2),
                           "entry_point": "simnets_hip_mex_fwd_prepared (device time per call, HIP graph of 20)"})
                 out["%s_%s" % (tag, name)] = e
             return out, res
@@ -482,10 +490,11 @@ def main():
             out = {}
             for tag, keep, xs_np, off_np, n, nb in (("config2_mex", keep2, x2, off2, n2, 64),
                                                     ("config4_layer3_mex", keep3, xl3, offl3, 256, 64)):
-                for name in ("wide_offsets", "eps_inf"):
-                    _, OV, kw_v, got = keep[name]
+                for name in OTHER_FORMS:
+                    _, OV, kw_v, got, xscale = keep[name]
                     noff = oracle.normalize_offsets(OV.cpu().numpy())
-                    out["%s_%s" % (tag, name)] = mex_err(got[:nb].cpu().numpy(), xs_np[:nb], noff, n, **kw_v)["floor_max_term"]
+                    xv = xs_np[:nb] if xscale == 1.0 else (xs_np[:nb] * np.float32(xscale))
+                    out["%s_%s" % (tag, name)] = mex_err(got[:nb].cpu().numpy(), xv, noff, n, **kw_v)["floor_max_term"]
             return out
         cpu_jobs.append(("mex_other_forms_max_rel_err_gpu_vs_cpu", cpu_forms))
 

@@ -771,11 +771,14 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
     const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
     float *out = a.out + (size_t)px.b * a.M * plane + px.out_off;
     // which form each instance of this wave takes (wave-uniform): bit g of `wide` set -> term by term
-    unsigned wide = a.finite_eps ? 0u : 0xffffu;
+    // (wide_finite: range beyond the product form's on its own, but finite - decided below, once the pixel is known)
+    unsigned wide = a.finite_eps ? 0u : 0xffffu, wide_finite = 0u;
     if (a.finite_eps) {
-        for (int m = m_first; m < m_end; ++m)
-            if (!(a.orng[row0 + m] <= kProductRange))
-                wide |= 1u << (m - m_first);
+        for (int m = m_first; m < m_end; ++m) {
+            const float rg = a.orng[row0 + m];
+            if (!(rg <= kProductRange))
+                (rg < INFINITY ? wide_finite : wide) |= 1u << (m - m_first);
+        }
     }
     // scaled patch values, their maximum and exponentials (finite epsilon)
     float ex[KL];
@@ -790,6 +793,19 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
         float mpv[MG] = {mp, mp, mp, mp};
         wave_best(mpv, false);
         mp = mpv[0];
+        if (wide_finite != 0u) {
+            // the largest term of sum_k exp2(x_k - max x) exp2(o_k - max o) is at least exp2(-range) of either factor:
+            // a pixel whose patch spans at most kProductRange keeps the product form whatever the offsets' range
+            float mn = INFINITY;
+#pragma unroll
+            for (int j = 0; j < KL; ++j)
+                if (kv[j])
+                    mn = fminf(mn, x[j]);
+            float mnv[MG] = {mn, mn, mn, mn};
+            wave_best(mnv, true);
+            if (!(mp - mnv[0] <= kProductRange))
+                wide |= wide_finite;
+        }
         const float m_sub = mp == -INFINITY ? 0.0f : mp;
 #pragma unroll
         for (int j = 0; j < KL; ++j)

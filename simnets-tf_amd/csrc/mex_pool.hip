@@ -628,11 +628,15 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         SIMNETS_PANEL_ISSUE(0)
     }
 
-    int wide = 0;
+    // wide: an offsets row whose range is beyond the product form's on its own; unbounded: ... and not even finite
+    int wide = 0, unbounded = 0;
     if (!SELFPACK && tid < TM) {
 #pragma unroll
-        for (int r = 0; r < R; ++r)
-            wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
+        for (int r = 0; r < R; ++r) {
+            const float rg = a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid];
+            wide |= !(rg <= kProductRange);
+            unbounded |= !(rg < INFINITY);
+        }
     }
 
     if (tid < 16 * NH) {
@@ -682,13 +686,14 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         float lo;
         pack_row32(rx, g.normalize, a.scale, row_lse, row_hi, lo);
         if (row_valid) {
-            wide = !(row_hi - lo <= kProductRange);   // NaN or inf (infinite entries) sends the workgroup to the VALU form
+            wide = !(row_hi - lo <= kProductRange);
+            unbounded = !(row_hi - lo < INFINITY);    // NaN or inf (infinite entries) sends the workgroup to the VALU form
         } else {
             row_hi = 0.0f;   // rows past the last instance: zeros, like the pack kernel's padding
         }
         omax_sh[tid] = row_hi;
     }
-    const bool prod = !__syncthreads_or(wide);
+    bool prod = !__syncthreads_or(wide);
     float msub[4];
     {
         const int cg = (part << g.lgF) | pg;
@@ -697,6 +702,31 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         for (int s = 1; s < 16; ++s) {
             const float4 o = reinterpret_cast<const float4 *>(pmx)[s * (XP / 4) + cg];
             m.x = fmaxf(m.x, o.x); m.y = fmaxf(m.y, o.y); m.z = fmaxf(m.z, o.z); m.w = fmaxf(m.w, o.w);
+        }
+        if (!prod) {
+            // Rows with a wide but finite range: the largest term of sum_k exp2(x_k - max x) exp2(o_k - max o) is at
+            // least exp2(-range) of the OTHER factor too (take k where the offsets peak), and terms that underflow are
+            // then below the sum's last bit.  So the product form still holds if every pixel column of the workgroup
+            // spans at most kProductRange: the column minima, through the tile that the chunk loop fills later.
+            const int any_unbounded = __syncthreads_or(unbounded);
+            float4 pn = make_float4(INFINITY, INFINITY, INFINITY, INFINITY);
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                pn.x = fminf(pn.x, pv[u].x); pn.y = fminf(pn.y, pv[u].y);
+                pn.z = fminf(pn.z, pv[u].z); pn.w = fminf(pn.w, pv[u].w);
+            }
+            reinterpret_cast<float4 *>(xs)[kslot * (XP / 4) + cg] = pn;
+            __syncthreads();
+            float4 n = reinterpret_cast<const float4 *>(xs)[cg];
+#pragma unroll
+            for (int s = 1; s < 16; ++s) {
+                const float4 o = reinterpret_cast<const float4 *>(xs)[s * (XP / 4) + cg];
+                n.x = fminf(n.x, o.x); n.y = fminf(n.y, o.y); n.z = fminf(n.z, o.z); n.w = fminf(n.w, o.w);
+            }
+            // (a column with a NaN or an infinite value, or nothing finite at all, is not narrow)
+            const bool narrow = !pvalid || (m.x - n.x <= kProductRange && m.y - n.y <= kProductRange &&
+                                            m.z - n.z <= kProductRange && m.w - n.w <= kProductRange);
+            prod = !__syncthreads_or(!narrow) && !any_unbounded;   // (the barrier also frees the tile again)
         }
         if (kslot == 0 && pvalid) {
             msh[colx[0]] = m.x; msh[colx[1]] = m.y; msh[colx[2]] = m.z; msh[colx[3]] = m.w;

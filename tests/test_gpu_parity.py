@@ -416,6 +416,55 @@ def test_mex_offset_ranges_product_and_two_sweep_forms(pkg, geom, spread, eps):
     assert mex_err(got, x, off, n, **kw) <= MEX_TOL
 
 
+@pytest.mark.parametrize("im,n", [((9, 32, 16, 16), 64), ((21, 128, 4, 4), 70), ((45, 256, 2, 2), 40)])
+@pytest.mark.parametrize("eps", [1.0, -2.0])
+@pytest.mark.parametrize("span", [80.0, 100.0])
+def test_mex_wide_offsets_with_patch_and_offsets_against_each_other(pkg, im, n, eps, span):
+    """Panel form, offsets rows spanning far more than the product form's range.  The workgroup still takes the product
+    form when every pixel's patch spans at most that range (span 80: below it, in units of the scaled exponent; 100:
+    above it, the max-tracked log-sum-exp).  The case that stresses the bound: patch values and offsets run against
+    each other, so the largest term is neither where the patch nor where the offsets peak, and the offsets of most
+    terms lie hundreds of units below their row's maximum."""
+    g = np.random.default_rng(61)
+    Cc = im[1]
+    kw = dict(softmax_mode=True, blocks=[Cc, 1, 1], strides=[Cc, 1, 1], epsilon=eps, use_unshared_regions=True,
+              unshared_offset_region=[1, 2, 2])
+    c1 = abs(eps) * math.log2(math.e)
+    ramp = np.linspace(-0.5, 0.5, Cc, dtype=np.float32)
+    x = (ramp[None, :, None, None] * (span / c1) * g.uniform(0.6, 0.97, size=(im[0], 1, im[2], im[3]))
+         + g.normal(size=im) * 0.01).astype(np.float32)
+    off = (-ramp[None, None, :, None, None] * g.uniform(0.5, 8.0, size=(4, n, 1, 1, 1)) * (span / c1)
+           + g.normal(size=(4, n, Cc, 1, 1)) * 0.3).astype(np.float32)
+    got = run_mex(pkg, x, off, n, **kw)
+    assert np.isfinite(got).all()
+    assert mex_err(got, x, off, n, **kw) <= MEX_TOL
+    full, pooled_out = pkg.mex_sum_pool_both(dev(x), dev(off), n, (2, 2), **kw)
+    assert mex_err(full.cpu().numpy(), x, off, n, **kw) <= MEX_TOL
+    assert torch.equal(pooled_out, pkg.sum_pooling(full, (2, 2)))
+
+
+@pytest.mark.parametrize("im,n", [((32, 512, 1, 1), 10), ((6, 200, 2, 2), 23)])
+@pytest.mark.parametrize("eps", [1.0, -2.0])
+@pytest.mark.parametrize("span", [80.0, 100.0])
+def test_mex_wide_offsets_on_few_pixels_with_long_patches(pkg, im, n, eps, span):
+    """The same two cases on the wave-per-pixel kernel (a network's head): every instance's offsets span far more than
+    the product form's range; pixels whose patch spans less keep the product form, the others go term by term."""
+    g = np.random.default_rng(62)
+    Cc = im[1]
+    kw = dict(softmax_mode=True, blocks=[Cc, 1, 1], strides=[Cc, 1, 1], epsilon=eps, use_unshared_regions=False,
+              shared_offset_region=[-1])
+    c1 = abs(eps) * math.log2(math.e)
+    ramp = np.linspace(-0.5, 0.5, Cc, dtype=np.float32)
+    x = (ramp[None, :, None, None] * (span / c1) * g.uniform(0.6, 0.97, size=(im[0], 1, im[2], im[3]))
+         + g.normal(size=im) * 0.01).astype(np.float32)
+    x[::3] *= 0.1          # some pixels far inside the range, next to ones at its edge
+    off = (-ramp[None, None, :, None, None] * g.uniform(2.0, 8.0, size=(1, n, 1, 1, 1)) * (span / c1)
+           + g.normal(size=(1, n, Cc, 1, 1)) * 0.3).astype(np.float32)
+    got = run_mex(pkg, x, off, n, **kw)
+    assert np.isfinite(got).all()
+    assert mex_err(got, x, off, n, **kw) <= MEX_TOL
+
+
 def pooled(y, ph, pw):
     B, Cc, H, W = y.shape
     return y[:, :, :H // ph * ph, :W // pw * pw].reshape(B, Cc, H // ph, ph, W // pw, pw).sum(axis=(3, 5))
