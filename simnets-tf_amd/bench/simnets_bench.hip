@@ -559,6 +559,23 @@ int main(int argc, char **argv)
         ms = time_ms(s, steps, prepared);
         report("config4 missing-data stack batch 512, fused, parameters prepared once", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 117e6, 5, ms, steps);
         checksum("config4 fused prepared", mex[4].y, n_final, s);
+        HIP_OK(hipMemsetAsync(mex[4].y, 0xff, n_final * sizeof(float), s));
+        // ... and the same five launches recorded once and replayed as a HIP graph (a serving loop: the calls are
+        // kernel launches on the caller's stream and nothing else, so a capture holds exactly those)
+        hipGraph_t graph;
+        hipGraphExec_t exec;
+        HIP_OK(hipStreamSynchronize(s));
+        HIP_OK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+        prepared();
+        HIP_OK(hipStreamEndCapture(s, &graph));
+        HIP_OK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+        auto replay = [&] { HIP_OK(hipGraphLaunch(exec, s)); };
+        for (int i = 0; i < warmup; ++i) replay();
+        ms = time_ms(s, steps, replay);
+        report("config4 missing-data stack batch 512, fused, parameters prepared once, replayed from a HIP graph", 512.0 * 32 * 256 * 4 + 4 * 268435456.0 + 512.0 * 10 * 512, 117e6, 5, ms, steps);
+        checksum("config4 fused prepared graph", mex[4].y, n_final, s);
+        HIP_OK(hipGraphExecDestroy(exec));
+        HIP_OK(hipGraphDestroy(graph));
     }
     else if (config == 5) {
         // backward at the config-3 and config-2 shapes, upstream gradients ~N(0,1)

@@ -111,6 +111,7 @@ def test_harness_config4(pkg, tmp_path):
     final = pkg.mex(cur, head[0], head[1], **head[2])
     expect(sums, "config4 fused similarity and pooling", final)
     expect(sums, "config4 fused prepared", final)      # the prepared calls run the same kernels on the same packing
+    expect(sums, "config4 fused prepared graph", final)   # ... and so does their replay from a HIP graph
 
 
 def test_harness_config5(pkg, tmp_path):
