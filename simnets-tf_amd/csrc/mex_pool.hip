@@ -990,10 +990,10 @@ int panel_halves(const MexPlan &p, int ph, int pw, const float *input, int slots
         return 0;
     // one column half per workgroup while two would leave compute units without a workgroup
     const int pnh = ((long long)slots + 31) / 32 * n_mgroups < kPanelWorkgroups ? 1 : 2;
-    // a single chunk (32 channels): only the plain call on a small grid gains (64 x 32x16x16 -> 64: 7.2 -> 6.0 us per
-    // call, 512 images: 20.5 -> 21.3 us); with pooling the kernel above stays, and with it the first layer's results
-    // stay those of its form with the Similarity inside, bit for bit
-    if (p.d.K == 32 && (pool || pnh != 1))
+    // a single chunk (32 channels): the plain call gains (64 x 32x16x16 -> 64: 7.2 -> 6.0 us per call; 512 images, with
+    // the window rows stored 8 bytes at a time: 20.7 -> 19.2 us); with pooling the kernel above stays, and with it the
+    // first layer's results stay those of its form with the Similarity inside, bit for bit
+    if (p.d.K == 32 && pool)
         return 0;
     if (panel_geometry(p, ph, pw, input, pnh, g))
         return pnh;
