@@ -150,17 +150,6 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
         ppos[tid] = pos;
     }
 
-    // Product form or term by term: decided from the packed row ranges, after the first chunk's loads have been
-    // issued (those assume the product form; a workgroup that turns out wide loads again).
-    auto decide = [&]() {
-        int wide = 0;
-        if (tid < TM) {
-#pragma unroll
-            for (int r = 0; r < R; ++r)
-                wide |= !(a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid] <= kProductRange);
-        }
-        return !__syncthreads_or(wide);
-    };
     bool prod = true;
     float m_run = -INFINITY;  // running maximum of this thread's staging column
 
@@ -310,6 +299,44 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
             }
         }
         gather(k0, kc, vn);
+    };
+    // Product form or term by term: decided from the packed row ranges, after the first chunk's loads have been
+    // issued (those assume the product form; a workgroup that turns out wide loads again).  Rows whose range is too
+    // wide on its own but finite keep the product form when the patch of every pixel column spans at most
+    // kProductRange (see there) - known here when the patch is a single chunk, which the registers then hold.
+    auto decide = [&]() {
+        int wide = 0, unbounded = 0;
+        if (tid < TM) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                const float rg = a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid];
+                wide |= !(rg <= kProductRange);
+                unbounded |= !(rg < INFINITY);
+            }
+        }
+        if (!__syncthreads_or(wide))
+            return true;
+        if (a.K > KC)
+            return false;
+        const int any_unbounded = __syncthreads_or(unbounded);
+        float hi = -INFINITY, lo = INFINITY;
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (sk + u * KSTEP < a.K) {
+                const float v = vn[u] * a.scale;
+                hi = fmaxf(hi, v);
+                lo = fminf(lo, v);
+            }
+        pmx[sk * XP + col] = hi;
+        xs[sk * XP + col] = lo;   // (the tile is filled later)
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < KSTEP; ++j) {
+            hi = fmaxf(hi, pmx[j * XP + col]);
+            lo = fminf(lo, xs[j * XP + col]);
+        }
+        // (a column with an infinite value, or with nothing finite, is not narrow; the barrier frees the arrays again)
+        return !__syncthreads_or(!(hi - lo <= kProductRange)) && !any_unbounded;
     };
     issue(0, min(KC, a.K));
     prod = decide();
