@@ -542,14 +542,13 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
     const long long row = (long long)r * Mp + m;
     float *dst = offp + ((size_t)r * n_mgroups + m / tm) * K * tm + m % tm;
     float *dste = offe + (dst - offp);
-    // the second layout (finite epsilon only): same values, its own group size
+    // the second layout (finite epsilon only; its readers, the gradient kernels, take the exponentials, the row maxima
+    // and the ranges, not the scaled values): same values, its own group size
     const int tm2 = tw.tm;
     const long long row2 = (long long)r * Mp2 + m;
-    float *dst2 = nullptr, *dste2 = nullptr;
-    if (m < Mp2) {
-        dst2 = tw.offp + ((size_t)r * tw.n_mgroups + m / tm2) * K * tm2 + m % tm2;
-        dste2 = tw.offe + (dst2 - tw.offp);
-    }
+    float *dste2 = nullptr;
+    if (m < Mp2)
+        dste2 = tw.offe + ((size_t)r * tw.n_mgroups + m / tm2) * K * tm2 + m % tm2;
     if (m >= M) {
         for (int k = lane; k < K; k += 64) {
             if (m < Mp) {
@@ -557,17 +556,15 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                 if (finite_eps)
                     dste[(size_t)k * tm] = 0.0f;
             }
-            if (dst2 != nullptr) {
-                dst2[(size_t)k * tm2] = 0.0f;
+            if (dste2 != nullptr)
                 dste2[(size_t)k * tm2] = 0.0f;
-            }
         }
         if (finite_eps && lane == 0) {
             if (m < Mp) {
                 omax[row] = 0.0f;
                 orng[row] = 0.0f;
             }
-            if (dst2 != nullptr) {
+            if (dste2 != nullptr) {
                 tw.omax[row2] = 0.0f;
                 tw.orng[row2] = 0.0f;
             }
@@ -629,15 +626,13 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         const float e = __builtin_amdgcn_exp2f(v - hi);
         dst[(size_t)k * tm] = v;
         dste[(size_t)k * tm] = e;
-        if (dst2 != nullptr) {
-            dst2[(size_t)k * tm2] = v;
+        if (dste2 != nullptr)
             dste2[(size_t)k * tm2] = e;
-        }
     });
     if (lane == 0) {
         omax[row] = hi;
         orng[row] = hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
-        if (dst2 != nullptr) {
+        if (dste2 != nullptr) {
             tw.omax[row2] = hi;
             tw.orng[row2] = hi - lo;
         }

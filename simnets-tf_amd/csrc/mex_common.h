@@ -163,8 +163,9 @@ struct SimPackJob {
     float fudge;
 };
 size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
-// A second packed layout written by the same launch: what the gradient kernels read (groups of kGradPackTm instances,
-// and the normalised offsets when the layer normalises them), kept by a forward call for the gradient call that
+// A second packed layout written by the same launch: what the gradient kernels read (groups of kGradPackTm instances:
+// the exponentials, row maxima and ranges - the scaled values, which those kernels do not take, stay unwritten - and
+// the normalised offsets when the layer normalises them), kept by a forward call for the gradient call that
 // follows it.  A plan whose grad_pack is set makes the forward's pack launch write it (and say so in `written`; a
 // forward that packs inside its own kernel does not).
 constexpr int kGradPackTm = 32;
