@@ -334,10 +334,10 @@ int simnets_hip_mex_sum_pool_fwd_both(const simnets_mex_attrs *attrs, const int 
 /* The gradients of that pair in one call: MexInputGrad and MexOffsetsGrad (src/ops/mex_op.cpp:134-170) applied to the
  * gradient of the pooling (the reference's AveragePooling2D x area, README.md:108-111), from the gradient of the POOLED
  * output `pooled_output_grad` [B, M*C_out, H_out/pool_h, W_out/pool_w] and the unpooled MEX output `mex_output`
- * (what simnets_hip_mex_sum_pool_fwd_both stores).  On the layers of the reference's networks (2 x 2 windows over
- * 2 x 2 unshared offsets, whole-channel patches, power-of-two maps) the gradient kernels read the window gradients
- * themselves; elsewhere the pooling gradient is expanded into the workspace first.  Either gradient pointer may be
- * NULL.  The values are those of simnets_hip_sum_pool_input_grad followed by simnets_hip_mex_grads, bit for bit. */
+ * (what simnets_hip_mex_sum_pool_fwd_both stores).  With 2 x 2 windows over an output of even height and width and one
+ * output channel per instance (every output pixel then has a window: the layers of the reference's networks) the
+ * gradient kernels read the window gradients themselves; elsewhere the pooling gradient is expanded into the
+ * workspace first.  Either gradient pointer may be NULL.  The values are those of simnets_hip_sum_pool_input_grad followed by simnets_hip_mex_grads, bit for bit. */
 int simnets_hip_mex_sum_pool_grads_workspace_bytes(const simnets_mex_attrs *attrs, const int input_shape[4], int pool_h,
                                                    int pool_w, size_t *bytes);
 int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int input_shape[4], const float *input,

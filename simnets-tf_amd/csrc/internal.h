@@ -88,8 +88,8 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
 // layer and offsets filled, through MexPlan::grad_pack or mex_grad_pack_launch; the call then packs nothing.
 size_t mex_grad_pack_bytes(const MexPlan &p);   // 0: the layer's gradient kernels read no packed offsets
 int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream);
-// whether the gradient kernels of this layer read the pooled gradient themselves (the row-wise kernels on suitably
-// aligned tensors; input_grad may be null)
+// whether the gradient kernels of this layer read the pooled gradient themselves (one output channel per instance,
+// even output height and width: every output pixel then has a window; input_grad may be null)
 bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *output, const float *pooled_grad,
                            const float *input_grad);
 int mex_grad_input(const MexPlan &p, const float *input, const float *offsets, const float *output,

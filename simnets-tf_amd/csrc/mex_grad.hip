@@ -31,8 +31,8 @@ struct MexGradArgs {
     const float *off;      // [R][M][K] offsets as the forward op used them
     const float *out;      // forward output
     const float *g;        // output gradient
-    int gpool;             // row-wise kernels: g is the gradient of the 2 x 2 sum-pooled output, [B][M][H/2][W/2]: the
-                           // gradient of output pixel (h, w) is its window's, g[h / 2][w / 2]
+    int gpool;             // g is the gradient of the 2 x 2 sum-pooled output, [B][M][H/2][W/2]: the gradient of output
+                           // pixel (h, w) is its window's, g[h / 2][w / 2]
     float *dx;             // input gradient
     float *partial;        // offsets gradient partial sums [chunk][R][M][K]
     int overlap;           // patches overlap: the per-patch gradients go to `col`, mex_col2im_kernel adds them up
@@ -198,8 +198,8 @@ __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs
         return;
     const PixelRef px = locate(a, r, chunk * 64 + lane);
     const bool valid = px.out_off >= 0;
-    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
-    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo, gplane = pooled_g_plane(ga, plane);
+    const float *gp = ga.g + (size_t)px.b * a.M * gplane + (valid ? pooled_g_offset(ga, px.out_off) : 0);
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const int m_scan = roomy ? a.M : min(a.M, 4);   // see mex_grad_input_mfma_kernel
     float amin = INFINITY;
@@ -222,7 +222,7 @@ __global__ __launch_bounds__(256) void mex_grad_factors_kernel(const MexGradArgs
         for (int i = 0; i < GM_TM / 4; ++i) {
             const int mc = min(mg * GM_TM + wave + 4 * i, a.M - 1);
             ovv[i] = op[(size_t)mc * plane];
-            gvv[i] = gp[(size_t)mc * plane];
+            gvv[i] = gp[(size_t)mc * gplane];
             omv[i] = omax_r[mc];
         }
 #pragma unroll
@@ -306,8 +306,8 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
         pc0[lane] = px.ci0; ph0[lane] = px.hi0; pw0[lane] = px.wi0;
         pout[lane] = px.out_off;
     }
-    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
-    const float *gp = ga.g + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo, gplane = pooled_g_plane(ga, plane);
+    const float *gp = ga.g + (size_t)px.b * a.M * gplane + (valid ? pooled_g_offset(ga, px.out_off) : 0);
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float o_first = op[(size_t)min(wave, a.M - 1) * plane];
     const float lo_first = omax_r[min(wave, a.M - 1)] - orng_r[min(wave, a.M - 1)];
@@ -396,7 +396,7 @@ __global__ __launch_bounds__(256) void mex_grad_input_mfma_kernel(const MexGradA
             for (int i = 0; i < GM_TM / 4; ++i) {
                 const int m = min(mg * GM_TM + wave + 4 * i, a.M - 1);
                 ov_n[i] = op[(size_t)m * plane];
-                gv_n[i] = gp[(size_t)m * plane];
+                gv_n[i] = gp[(size_t)m * gplane];
                 om_n[i] = omax_r[m];
             }
         }
@@ -662,7 +662,7 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             return;
         }
     }
-    const size_t plane = (size_t)a.Co * a.Ho * a.Wo;
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo, gplane = pooled_g_plane(ga, plane);
     const int lr = lane & 15, lq = lane >> 4;
     floatx4 acc[4];
 #pragma unroll
@@ -683,7 +683,7 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
     auto load_group = [&](int s, Group &q) {
         const PixelRef px = locate(a, r, (chunk * ga.pxl + s) * 64 + lane);
         q.valid = px.out_off >= 0;
-        const float *gp = ga.g + (size_t)px.b * a.M * plane + (q.valid ? px.out_off : 0);
+        const float *gp = ga.g + (size_t)px.b * a.M * gplane + (q.valid ? pooled_g_offset(ga, px.out_off) : 0);
         const float *op = ga.out + (size_t)px.b * a.M * plane + (q.valid ? px.out_off : 0);
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
@@ -692,7 +692,7 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
             q.gv[i] = 0.0f;
             if (m < a.M) {
                 q.ov[i] = op[(size_t)m * plane];
-                q.gv[i] = q.valid ? gp[(size_t)m * plane] : 0.0f;
+                q.gv[i] = q.valid ? gp[(size_t)m * gplane] : 0.0f;
             }
         }
 #pragma unroll
@@ -1764,9 +1764,10 @@ size_t mex_grad_offsets_workspace_bytes(const MexPlan &p) { return mex_grads_wor
 bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *output, const float *pooled_grad,
                            const float *input_grad)
 {
-    auto aligned = [](const void *q, uintptr_t a) { return (reinterpret_cast<uintptr_t>(q) & (a - 1)) == 0; };
-    return std::isfinite(p.epsilon) && rows_geometry(p) && aligned(input, 16) && aligned(output, 16) &&
-           aligned(pooled_grad, 8) && (input_grad == nullptr || aligned(input_grad, 16));
+    (void)input; (void)output; (void)pooled_grad; (void)input_grad;   // (any alignment: only the row-wise kernels care)
+    // every kernel maps an output pixel to its window (pooled_g_offset): one output channel per instance and no
+    // trailing row or column that the pooling dropped
+    return p.d.channels_out == 1 && p.d.height_out % 2 == 0 && p.d.width_out % 2 == 0;
 }
 
 int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream)
@@ -1840,9 +1841,10 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     ga.cpr = (ga.k.slots + 63) / 64;
     // the row-wise kernels read and write 16 bytes at a time
     auto aligned16 = [](const void *q) { return (reinterpret_cast<uintptr_t>(q) & 15) == 0; };
-    const bool use_rows = grad_is_pooled ||
-                          (t.mfma && t.rows && aligned16(input) && aligned16(output) && aligned16(output_grad) &&
-                           (!want_input || aligned16(input_grad)));
+    // (of a pooled gradient they read a window row's two values: 8 bytes)
+    const bool g_aligned = grad_is_pooled ? (reinterpret_cast<uintptr_t>(output_grad) & 7) == 0 : aligned16(output_grad);
+    const bool use_rows = t.mfma && t.rows && aligned16(input) && aligned16(output) && g_aligned &&
+                          (!want_input || aligned16(input_grad));
     if (grad_is_pooled && !mex_grads_take_pooled(p, input, output, output_grad, input_grad))
         return SIMNETS_ERR_ALGO;   // (the callers ask first)
     if (t.mfma) {

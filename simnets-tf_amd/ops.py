@@ -315,8 +315,8 @@ def mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, num_insta
                        saved=None):
     """The gradients of `mex_sum_pool` w.r.t. (input, offsets) from the gradient of the POOLED output and the MEX
     output before pooling (`mex_sum_pool_both`'s first result): `mex_grads(input, offsets, mex_output,
-    sum_pooling_input_grad(pooled_output_grad, ...))` in one call, without the expanded gradient tensor on the layers
-    of the reference's networks.  A gradient that is not wanted comes back as None."""
+    sum_pooling_input_grad(pooled_output_grad, ...))` in one call, without the expanded gradient tensor where every
+    output pixel has a window (2 x 2 pooling of an even-sized map, one output channel per instance).  A gradient that is not wanted comes back as None."""
     gi, go = _n.mex_sum_pool_grads(input, offsets, mex_output, pooled_output_grad, int(num_instances), int(pool_size[0]),
                                    int(pool_size[1]), bool(want_input), bool(want_offsets), softmax_mode, padding, strides,
                                    blocks, epsilon, blocks_out_of_bounds_value, blocks_round_down, use_unshared_regions,
