@@ -349,7 +349,8 @@ int simnets_hip_mex_sum_pool_grads(const simnets_mex_attrs *attrs, const int inp
  * the registered gradient receives the forward op's inputs and output).  Both sides re-order the offsets first
  * (scaled, row maxima and ranges, exponentials, the normalised copy of normalize_offsets), in different group sizes.
  * The *_saving forward calls leave the gradient kernels' form in `saved` (simnets_hip_mex_saved_bytes; 256-byte
- * aligned; 0 bytes = this layer's gradient kernels read the offsets as they are, `saved` may then be NULL) from the
+ * aligned; 0 bytes = this layer's gradient kernels read the offsets as they are, `saved` may then be NULL; layers of few
+ * instances over long patches keep the normalised copy alone) from the
  * launch that packs the forward's own, and the *_saved gradient calls read it instead of packing again.  Outputs
  * and gradients are those of the plain calls, bit for bit.  `saved` is valid for the attributes, input shape and
  * offsets VALUES of the forward call that wrote it; a gradient call given saved == NULL packs for itself. */

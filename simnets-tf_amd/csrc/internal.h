@@ -87,6 +87,9 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
 // `saved`: the buffer (mex_grad_pack_bytes, declared with the packing in mex_common.h) that a forward call of the same
 // layer and offsets filled, through MexPlan::grad_pack or mex_grad_pack_launch; the call then packs nothing.
 size_t mex_grad_pack_bytes(const MexPlan &p);   // 0: the layer's gradient kernels read no packed offsets
+// whether they read the packed layout at all (finite epsilon, not the kernel for few instances over long patches,
+// which takes the offsets - or the normalised copy, which the buffer then holds alone - as they are)
+bool mex_grads_read_packed(const MexPlan &p);
 int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream);
 // whether the gradient kernels of this layer read the pooled gradient themselves (one output channel per instance,
 // even output height and width: every output pixel then has a window; input_grad may be null)

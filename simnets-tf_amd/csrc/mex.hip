@@ -949,19 +949,25 @@ size_t mex_grad_pack_bytes(const MexPlan &p)
     if (!std::isfinite(p.epsilon))
         return 0;   // those gradient kernels read the offsets as they are
     const size_t rmk = (size_t)p.d.num_regions * p.d.M * p.d.K * sizeof(float);
-    return mex_packed_bytes(p, kGradPackTm, (p.d.M + kGradPackTm - 1) / kGradPackTm) +
+    return (mex_grads_read_packed(p) ? mex_packed_bytes(p, kGradPackTm, (p.d.M + kGradPackTm - 1) / kGradPackTm) : 0) +
            (p.normalize_offsets ? align_up(rmk, 256) : 0);
 }
 
 void mex_grad_pack_layout(const MexPlan &p, void *buffer, MexPackTwin *tw, float **normalized)
 {
     const simnets_mex_dims &d = p.d;
+    char *ws = reinterpret_cast<char *>(buffer);
+    if (!mex_grads_read_packed(p)) {
+        // only the normalised copy
+        *tw = MexPackTwin{nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0};
+        *normalized = p.normalize_offsets ? reinterpret_cast<float *>(ws) : nullptr;
+        return;
+    }
     tw->tm = kGradPackTm;
     tw->n_mgroups = (d.M + kGradPackTm - 1) / kGradPackTm;
     const long long rows = (long long)d.num_regions * tw->n_mgroups * tw->tm;
     const size_t packed = align_up((size_t)rows * d.K * sizeof(float), 256);
     const size_t row_bytes = align_up((size_t)rows * sizeof(float), 256);
-    char *ws = reinterpret_cast<char *>(buffer);
     tw->offp = reinterpret_cast<float *>(ws);
     tw->offe = reinterpret_cast<float *>(ws + packed);
     tw->omax = reinterpret_cast<float *>(ws + 2 * packed);

@@ -1392,32 +1392,37 @@ __global__ __launch_bounds__(256) void mex_normalize_rows_backward_kernel(const 
 
 // Elements lane, lane + 64, ... of one row of the offsets gradient from its partial sums (eight interleaved sums in
 // chunk order, added in order), E elements at a time; returns the lane's share of the row sum (in element order).
-template <int E>
+// (NB: rounds of eight chunks requested together; the additions keep the order of one round at a time)
+template <int E, int STRIDE = 64, int NB = 1>
 __device__ __forceinline__ float finish_long_row(const float *__restrict__ pr, float *__restrict__ gr, long long n,
                                                  int chunks, int K, int lane)
 {
     float sum = 0.0f;
-    for (int k0 = lane; k0 < K; k0 += 64 * E) {
+    for (int k0 = lane; k0 < K; k0 += STRIDE * E) {
         float s8[E][8];
 #pragma unroll
         for (int e = 0; e < E; ++e)
 #pragma unroll
             for (int j = 0; j < 8; ++j)
                 s8[e][j] = 0.0f;
-        for (int c0 = 0; c0 < chunks; c0 += 8) {
+        for (int c0 = 0; c0 < chunks; c0 += 8 * NB) {
             // all requests first, those past the last chunk or the row's end on a valid address (a load inside the
             // condition would be waited for before the next one is issued)
-            float v[E][8];
+            float v[NB][E][8];
 #pragma unroll
-            for (int e = 0; e < E; ++e)
+            for (int b = 0; b < NB; ++b)
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    v[e][j] = pr[(size_t)min(c0 + j, chunks - 1) * n + min(k0 + 64 * e, K - 1)];
+                for (int e = 0; e < E; ++e)
 #pragma unroll
-            for (int e = 0; e < E; ++e)
+                    for (int j = 0; j < 8; ++j)
+                        v[b][e][j] = pr[(size_t)min(c0 + 8 * b + j, chunks - 1) * n + min(k0 + STRIDE * e, K - 1)];
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    s8[e][j] = c0 + j < chunks ? s8[e][j] + v[e][j] : s8[e][j];
+            for (int b = 0; b < NB; ++b)
+#pragma unroll
+                for (int e = 0; e < E; ++e)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        s8[e][j] = c0 + 8 * b + j < chunks ? s8[e][j] + v[b][e][j] : s8[e][j];
         }
 #pragma unroll
         for (int e = 0; e < E; ++e) {
@@ -1425,8 +1430,8 @@ __device__ __forceinline__ float finish_long_row(const float *__restrict__ pr, f
 #pragma unroll
             for (int j = 1; j < 8; ++j)
                 t += s8[e][j];
-            if (k0 + 64 * e < K) {
-                gr[k0 + 64 * e] = t;
+            if (k0 + STRIDE * e < K) {
+                gr[k0 + STRIDE * e] = t;
                 sum += t;
             }
         }
@@ -1563,6 +1568,123 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_finish_rows_kernel(const
         gr[k] -= expf(nr[k]) * sum;   // reads back what this lane stored above
 }
 
+// The same for few long rows (a classifier head: 10 rows of 512): one workgroup per row, the four waves split its
+// elements (thread t takes t, t + 256, ...), the row sum of the chain rule goes through LDS.
+__global__ __launch_bounds__(256) void mex_grad_offsets_finish_wide_rows_kernel(const float *__restrict__ partial,
+                                                                               long long n, int chunks, int K,
+                                                                               const float *__restrict__ normalized,
+                                                                               float *__restrict__ doff)
+{
+    __shared__ float ws[4];
+    const long long row = blockIdx.x;
+    float *gr = doff + (size_t)row * K;
+    const float *pr = partial + (size_t)row * K;
+    const int tid = threadIdx.x;
+    float sum = K <= 256 ? finish_long_row<1, 256, 4>(pr, gr, n, chunks, K, tid)
+                         : (K <= 512 ? finish_long_row<2, 256, 2>(pr, gr, n, chunks, K, tid)
+                                     : finish_long_row<4, 256, 1>(pr, gr, n, chunks, K, tid));
+    if (normalized == nullptr)
+        return;
+    for (int d = 32; d > 0; d >>= 1)
+        sum += __shfl_xor(sum, d, 64);
+    if ((tid & 63) == 0)
+        ws[tid >> 6] = sum;
+    __syncthreads();
+    sum = (ws[0] + ws[1]) + (ws[2] + ws[3]);
+    const float *nr = normalized + (size_t)row * K;
+    for (int k = tid; k < K; k += 256)
+        gr[k] -= expf(nr[k]) * sum;   // reads back what this thread stored above
+}
+
+// Few instances over long patches on few pixels (a network's classifier head: 10 instances x 512 channels on one
+// pixel per image): the tiled kernels above would run a handful of workgroups in long serial chains, in three
+// launches.  Here a thread owns one patch element k (a workgroup spans K) and keeps the region's offsets for that
+// element in registers; the workgroup walks its share of the pixels, four at a time (their loads in flight
+// together), and forms every term as the reference does (mex_term: either epsilon, any offsets range): summed over
+// the instances it is the input gradient of (pixel, k), summed over the pixels - in registers - the offsets gradient
+// of (instance, k).  No LDS, no barriers; one partial sum [M][K] per workgroup for the finish kernel.
+constexpr int kHeadMaxM = 16, kHeadPixels = 4;
+template <int MH, bool FINITE>
+__global__ __launch_bounds__(1024) void mex_grad_head_kernel(const MexGradArgs ga, int wgs_per_region, int want_input,
+                                                             int want_offsets)
+{
+    static_assert(MH <= 16, "one lane per instance in the load of the gradients and outputs");
+    const MexKernelArgs &a = ga.k;
+    const int lane = threadIdx.x & 63;
+    const int r = blockIdx.x / wgs_per_region, wg = blockIdx.x - r * wgs_per_region;
+    const int k = threadIdx.x;
+    const bool kv = k < a.K;
+    const int kk = kv ? k : 0;
+    const int bhw = a.bh * a.bw;
+    const int dc = kk / bhw, rem = kk - dc * bhw, dh = rem / a.bw, dw = rem - dh * a.bw;
+    float of[MH], acc[MH];
+#pragma unroll
+    for (int m = 0; m < MH; ++m) {
+        of[m] = ga.off[((size_t)r * a.M + min(m, a.M - 1)) * a.K + kk];
+        acc[m] = 0.0f;
+    }
+    const size_t plane = (size_t)a.Co * a.Ho * a.Wo, gplane = pooled_g_plane(ga, plane);
+    const int ml = min(lane & 15, a.M - 1);
+    for (int s0 = wg * kHeadPixels; s0 < a.slots; s0 += wgs_per_region * kHeadPixels) {
+        float x[kHeadPixels], go[kHeadPixels];
+        int io[kHeadPixels];
+        bool valid[kHeadPixels];
+        size_t img[kHeadPixels], col[kHeadPixels];
+#pragma unroll
+        for (int p = 0; p < kHeadPixels; ++p) {
+            const int slot = s0 + p;
+            const PixelRef px = locate(a, r, min(slot, a.slots - 1));   // (the same pixel for the whole workgroup)
+            valid[p] = slot < a.slots && px.out_off >= 0;
+            const int ci = px.ci0 + dc, hi = px.hi0 + dh, wi = px.wi0 + dw;
+            const bool ok = kv && ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
+            io[p] = ok ? (ci * a.H + hi) * a.W + wi : -1;
+            img[p] = (size_t)px.b * a.C * a.H * a.W;
+            // (loads on addresses that are always valid, the choice made afterwards: a load inside a condition is
+            // waited for before the next one is issued)
+            const float xv = a.in[img[p] + (ok ? io[p] : 0)];
+            x[p] = ok ? xv : a.oob;
+            const int oo = valid[p] ? px.out_off : 0;
+            // every instance's gradient (lanes 0 ... 15) and output value (lanes 16 ... 31) through one load, read back
+            // lane by lane below
+            const float *src = (lane & 16) ? ga.out + ((size_t)px.b * a.M + ml) * plane + oo
+                                           : ga.g + ((size_t)px.b * a.M + ml) * gplane + pooled_g_offset(ga, oo);
+            go[p] = *src;
+            col[p] = ((size_t)px.b * plane + oo) * a.K;
+        }
+        // Straight-line arithmetic: instances past the last one repeat it with a zero gradient (their sums are never
+        // stored), threads past the last patch element compute on the out-of-bounds value (nothing of theirs is
+        // stored either); only an empty pixel slot is skipped.
+#pragma unroll
+        for (int p = 0; p < kHeadPixels; ++p) {
+            if (!valid[p])
+                continue;
+            float dxa = 0.0f;
+#pragma unroll
+            for (int m = 0; m < MH; ++m) {
+                float gm = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, go[p]), m));
+                const float om = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, go[p]), 16 + m));
+                gm = m < a.M ? gm : 0.0f;
+                const float e = mex_term(x[p] + of[m], om, gm, a.c1, a.c0, FINITE);
+                dxa += e;
+                acc[m] += e;
+            }
+            if (want_input && io[p] >= 0) {
+                if (ga.overlap)
+                    ga.col[col[p] + k] = dxa;
+                else
+                    ga.dx[img[p] + io[p]] = dxa;
+            }
+        }
+    }
+    if (!want_offsets || !kv)
+        return;
+    float *part = ga.partial + ((size_t)wg * a.R + r) * a.M * a.K + k;
+#pragma unroll
+    for (int m = 0; m < MH; ++m)
+        if (m < a.M)
+            part[(size_t)m * a.K] = acc[m];
+}
+
 __global__ void mex_fill_zero_kernel(float *__restrict__ p, long long n)
 {
     for (long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long long)gridDim.x * blockDim.x)
@@ -1571,6 +1693,8 @@ __global__ void mex_fill_zero_kernel(float *__restrict__ p, long long n)
 
 struct MexGradTiling {
     int pxl, cpr_offsets;
+    bool head;           // few instances over long patches on few pixels: mex_grad_head_kernel, both gradients
+    int head_wgs;        // ... with this many workgroups per region (= partial sums per region)
     bool mfma;           // finite epsilon: the matrix-core kernels, fed by the forward pass's packed offsets
     size_t norm_bytes, partial_bytes, packed_bytes;
     bool overlap;        // input gradient: patches overlap
@@ -1661,6 +1785,13 @@ MexGradTiling mex_grad_tiling(const MexPlan &p)
     // elements per workgroup as that allows (each tile of them reads all of `out` and `g`), then splits the instance
     // groups; the offsets gradient walks as many chunks per workgroup as that allows (each workgroup writes a
     // partial sum of its tile).
+    // The head kernel: terms few enough for one exponential each (a classifier head has 512 x 10 x 512 of them)
+    t.head = d.M <= kHeadMaxM && d.K >= 64 && d.K <= 1024 && slots >= 1 &&
+             (long long)d.num_regions * slots * d.M * d.K <= (16LL << 20) && (long long)p.C * p.H * p.W <= 0x7fffffffLL;
+    // (about 8 pixels per workgroup, at most 64 partial sums per region for the finish kernel)
+    t.head_wgs = (int)std::max<long long>(1, std::min<long long>((slots + 7) / 8, std::max(1, 64 / d.num_regions)));
+    if (t.head)
+        t.partial_bytes = std::max(t.partial_bytes, align_up(rmk * t.head_wgs, 256));
     t.rows = rows_geometry(p);
     t.rows_ksub = 1; t.rows_msplit = 1; t.rows_mg_per_split = n_mg; t.rows_pxl = 1; t.rows_cpr = 0;
     if (t.rows) {
@@ -1770,6 +1901,12 @@ bool mex_grads_take_pooled(const MexPlan &p, const float *input, const float *ou
     return p.d.channels_out == 1 && p.d.height_out % 2 == 0 && p.d.width_out % 2 == 0;
 }
 
+bool mex_grads_read_packed(const MexPlan &p)
+{
+    const MexGradTiling t = mex_grad_tiling(p);
+    return t.mfma && !t.head;
+}
+
 int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, void *stream)
 {
     MexPlan q = p;
@@ -1777,6 +1914,10 @@ int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, v
     MexPackTwin tw;
     float *norm;
     mex_grad_pack_layout(q, buffer, &tw, &norm);
+    if (tw.offp == nullptr) {   // only the normalised copy is kept
+        const float *used;
+        return prepare_offsets(q, offsets, norm, reinterpret_cast<hipStream_t>(stream), &used);
+    }
     MexKernelArgs a = mex_kernel_args(q);
     return mex_pack_offsets(q, offsets, GM_TM, tw.n_mgroups, buffer, &a, stream, nullptr, true, norm);
 }
@@ -1834,6 +1975,56 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     ga.partial = reinterpret_cast<float *>(ws + w.partial);
     ga.overlap = 0;
     ga.col = reinterpret_cast<float *>(ws + w.col);
+    if (grad_is_pooled && !mex_grads_take_pooled(p, input, output, output_grad, input_grad))
+        return SIMNETS_ERR_ALGO;   // (the callers ask first)
+    if (t.head) {
+        // one launch for both gradients, on the offsets as they are (or their normalised copy): nothing is packed
+        if (pack_normalizes && !packed_already) {
+            rc = prepare_offsets(p, offsets, ws + w.norm, s, &ga.off);
+            if (rc)
+                return rc;
+        }
+        ga.overlap = t.overlap ? 1 : 0;
+        if (want_input && !t.overlap && !t.tiles_input) {
+            hipLaunchKernelGGL(mex_fill_zero_kernel, dim3((unsigned)std::min<long long>((n_in + 255) / 256, 65535)),
+                               dim3(256), 0, s, input_grad, n_in);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
+        const dim3 grid((unsigned)(d.num_regions * t.head_wgs)), block((unsigned)((d.K + 63) / 64 * 64));
+        const int wi = want_input ? 1 : 0, wo = want_offsets ? 1 : 0;
+#define SIMNETS_HEAD_LAUNCH(MH)                                                                                      \
+    if (t.mfma)                                                                                                      \
+        hipLaunchKernelGGL((mex_grad_head_kernel<MH, true>), grid, block, 0, s, ga, t.head_wgs, wi, wo);              \
+    else                                                                                                             \
+        hipLaunchKernelGGL((mex_grad_head_kernel<MH, false>), grid, block, 0, s, ga, t.head_wgs, wi, wo)
+        if (d.M <= 4) {
+            SIMNETS_HEAD_LAUNCH(4);
+        } else if (d.M <= 8) {
+            SIMNETS_HEAD_LAUNCH(8);
+        } else if (d.M <= 12) {
+            SIMNETS_HEAD_LAUNCH(12);
+        } else {
+            SIMNETS_HEAD_LAUNCH(kHeadMaxM);
+        }
+#undef SIMNETS_HEAD_LAUNCH
+        if (hipGetLastError() != hipSuccess)
+            return SIMNETS_ERR_HIP;
+        if (want_input && t.overlap) {
+            hipLaunchKernelGGL(mex_col2im_kernel, dim3((unsigned)((n_in + 255) / 256)), dim3(256), 0, s, ga.k, ga.col,
+                               input_grad, n_in);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
+        if (want_offsets) {
+            const long long rows = (long long)d.num_regions * d.M;
+            hipLaunchKernelGGL(mex_grad_offsets_finish_wide_rows_kernel, dim3((unsigned)rows), dim3(256), 0, s, ga.partial,
+                               n_off, t.head_wgs, d.K, p.normalize_offsets ? ga.off : nullptr, offsets_grad);
+            if (hipGetLastError() != hipSuccess)
+                return SIMNETS_ERR_HIP;
+        }
+        return SIMNETS_OK;
+    }
     ga.msplit = 1; ga.mg_per_split = (d.M + GM_TM - 1) / GM_TM;
     ga.dx_splits = reinterpret_cast<float *>(ws + w.split);
     ga.wbuf = nullptr; ga.exbuf = nullptr; ga.slots_pad = 0; ga.Mp = 0; ga.Kp = 0;
@@ -1845,8 +2036,6 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
     const bool g_aligned = grad_is_pooled ? (reinterpret_cast<uintptr_t>(output_grad) & 7) == 0 : aligned16(output_grad);
     const bool use_rows = t.mfma && t.rows && aligned16(input) && aligned16(output) && g_aligned &&
                           (!want_input || aligned16(input_grad));
-    if (grad_is_pooled && !mex_grads_take_pooled(p, input, output, output_grad, input_grad))
-        return SIMNETS_ERR_ALGO;   // (the callers ask first)
     if (t.mfma) {
         rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed_at, &ga.k, stream, nullptr,
                               !packed_already, pack_normalizes ? norm_at : nullptr);
@@ -1969,6 +2158,12 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
         if (hipGetLastError() != hipSuccess)
             return SIMNETS_ERR_HIP;
         const long long rows = (long long)d.num_regions * d.M;
+        if (rows <= 64 && d.K >= 256 && d.K <= kFinishRowsMaxK) {
+            // few long rows: a workgroup per row
+            hipLaunchKernelGGL(mex_grad_offsets_finish_wide_rows_kernel, dim3((unsigned)rows), dim3(256), 0, s, go.partial,
+                               n_off, go.cpr, d.K, p.normalize_offsets ? go.off : nullptr, offsets_grad);
+            return hipGetLastError() == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
+        }
         if (d.K <= kFinishRowsMaxK && (rows + 3) / 4 <= 0x7fffffffLL) {
             // short rows: the sum over the pixel chunks and the chain rule through the normalisation in one launch
             hipLaunchKernelGGL(mex_grad_offsets_finish_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, s,
