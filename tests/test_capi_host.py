@@ -388,3 +388,51 @@ def test_prepared_entry_points_validate_on_the_host(pkg):
     g = l.simnets_hip_similarity_mex_sum_pool_fwd_prepared
     assert g(C.byref(sa), sx, st, None, C.byref(m), 2, 2, 256, need.value, 256, None) == -1
     assert g(C.byref(sa), sx, st, 256, C.byref(m), 2, 2, 256, need.value - 1, 256, None) == -17
+
+
+def test_saving_and_saved_entry_points_validate_on_the_host(pkg):
+    """simnets_hip_mex_saved_bytes sizes the buffer a training forward fills for the gradient call; the *_saving and
+    *_saved calls check it (size, 256-byte alignment, presence) before anything is launched."""
+    l = pkg._lib.lib()
+    I4 = C.c_int * 4
+    xs = I4(2, 32, 8, 8)
+    n_off = 4 * 6 * 32
+    m = pkg.ops.mex_attrs(6, blocks=[32, 1, 1], strides=[32, 1, 1], unshared_offset_region=[1, 2, 2], normalize_offsets=True)
+    kept = C.c_size_t()
+    assert l.simnets_hip_mex_saved_bytes(C.byref(m), xs, C.byref(kept)) == 0
+    # exponentials, scaled values and two row tables in groups of 32 instances, the element table, the normalised copy
+    assert kept.value >= (2 * 4 * 32 * 32 + 4 * 6 * 32) * 4 and kept.value % 256 == 0
+    assert l.simnets_hip_mex_saved_bytes(C.byref(m), xs, None) == -1
+    inf = pkg.ops.mex_attrs(6, blocks=[32, 1, 1], strides=[32, 1, 1], unshared_offset_region=[1, 2, 2], epsilon=float("inf"))
+    assert l.simnets_hip_mex_saved_bytes(C.byref(inf), xs, C.byref(kept)) == 0 and kept.value == 0
+    # few instances over long patches: only the normalised copy (nothing without normalisation)
+    head = pkg.ops.mex_attrs(10, blocks=[512, 1, 1], strides=[512, 1, 1], use_unshared_regions=False,
+                             shared_offset_region=[-1], normalize_offsets=True)
+    hs = I4(64, 512, 1, 1)
+    assert l.simnets_hip_mex_saved_bytes(C.byref(head), hs, C.byref(kept)) == 0 and kept.value == 10 * 512 * 4
+    head.normalize_offsets = 0
+    assert l.simnets_hip_mex_saved_bytes(C.byref(head), hs, C.byref(kept)) == 0 and kept.value == 0
+
+    assert l.simnets_hip_mex_saved_bytes(C.byref(m), xs, C.byref(kept)) == 0
+    ws = C.c_size_t()
+    assert l.simnets_hip_mex_workspace_bytes(C.byref(m), xs, C.byref(ws)) == 0
+    big = 1 << 30
+    # forward: no buffer, a short one, a misaligned one
+    assert l.simnets_hip_mex_fwd_saving(C.byref(m), xs, 256, 256, n_off, 256, None, 0, 256, big, None) == -17
+    assert l.simnets_hip_mex_fwd_saving(C.byref(m), xs, 256, 256, n_off, 256, 256, kept.value - 1, 256, big, None) == -17
+    assert l.simnets_hip_mex_fwd_saving(C.byref(m), xs, 256, 256, n_off, 256, 257, big, 256, big, None) == -17
+    assert l.simnets_hip_mex_fwd_saving(C.byref(m), xs, 256, 256, 5, 256, 256, big, 256, big, None) == -15     # short offsets
+    assert l.simnets_hip_mex_sum_pool_fwd_saving(C.byref(m), xs, 256, 256, n_off, 2, 2, 256, 256, 256, 16, 256, big,
+                                                 None) == -17
+    assert l.simnets_hip_mex_sum_pool_fwd_saving(C.byref(m), xs, 256, 256, n_off, 2, 2, None, 256, 256, big, 256, big,
+                                                 None) == -1                                                     # no MEX output
+    assert l.simnets_hip_mex_sum_pool_fwd_saving(C.byref(m), xs, 256, 256, n_off, 0, 2, 256, 256, 256, big, 256, big,
+                                                 None) == -15                                                    # window
+    # gradients: a buffer that is given must be whole and aligned (none at all = the plain call)
+    assert l.simnets_hip_mex_grads_saved(C.byref(m), xs, 256, 256, n_off, 256, 256, 256, 16, 256, 256, 256, big, None) == -17
+    assert l.simnets_hip_mex_grads_saved(C.byref(m), xs, 256, 256, n_off, 256, 256, 257, big, 256, 256, 256, big, None) == -17
+    assert l.simnets_hip_mex_grads_saved(C.byref(m), xs, 256, 256, n_off, 256, 256, 256, big, 256, None, 256, big, None) == -1
+    assert l.simnets_hip_mex_sum_pool_grads_saved(C.byref(m), xs, 256, 256, n_off, 2, 2, 256, 256, 256, 16, 256, 256,
+                                                  256, big, None) == -17
+    assert l.simnets_hip_mex_sum_pool_grads_saved(C.byref(m), xs, 256, 256, n_off, 2, 2, 256, 256, 256, big, None, None,
+                                                  256, big, None) == -1                                          # no gradient wanted
