@@ -77,7 +77,10 @@ __device__ __forceinline__ float patch_element(const MexKernelArgs &a, const Pix
     const bool ok = ci >= 0 && ci < a.C && hi >= 0 && hi < a.H && wi >= 0 && wi < a.W;
     const ptrdiff_t o = ((ptrdiff_t)ci * a.H + hi) * a.W + wi;
     *img_off = ok ? o : -1;
-    return ok ? a.in[(size_t)px.b * a.C * a.H * a.W + o] : a.oob;
+    // (the load on an address that is always valid, the choice afterwards: loads inside conditions are waited for one
+    // by one)
+    const float v = a.in[(size_t)px.b * a.C * a.H * a.W + (ok ? o : 0)];
+    return ok ? v : a.oob;
 }
 
 __device__ __forceinline__ float mex_term(float x_plus_off, float out, float g, float c1, float c0, bool finite)
@@ -113,13 +116,26 @@ __device__ __forceinline__ void mex_grad_input_wave(const MexGradArgs &ga, int r
     const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
     const float SIMNETS_CONST_AS *off = (const float SIMNETS_CONST_AS *)(ga.off) + (size_t)r * a.M * a.K + k0;
     const bool finite = a.finite_eps != 0;
-    for (int m = m_begin; m < m_end; ++m) {
-        const float g = valid ? gp[(size_t)m * gplane] : 0.0f;
-        const float o = op[(size_t)m * plane];
+    // four instances at a time: their gradient and output values requested together (the additions keep their order)
+    for (int m4 = m_begin; m4 < m_end; m4 += 4) {
+        float gv[4], ov[4];
 #pragma unroll
-        for (int j = 0; j < GX_KT; ++j) {
-            const float of = (k0 + j < a.K) ? off[(size_t)m * a.K + j] : 0.0f;
-            acc[j] += mex_term(xk[j] + of, o, g, a.c1, a.c0, finite);
+        for (int u = 0; u < 4; ++u) {
+            const int mc = min(m4 + u, m_end - 1);
+            gv[u] = gp[(size_t)mc * gplane];
+            ov[u] = op[(size_t)mc * plane];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int m = m4 + u;
+            if (m < m_end) {
+                const float g = valid ? gv[u] : 0.0f;
+#pragma unroll
+                for (int j = 0; j < GX_KT; ++j) {
+                    const float of = (k0 + j < a.K) ? off[(size_t)m * a.K + j] : 0.0f;
+                    acc[j] += mex_term(xk[j] + of, ov[u], g, a.c1, a.c0, finite);
+                }
+            }
         }
     }
     if (!valid)
@@ -166,7 +182,7 @@ constexpr int GM_TM = kGradPackTm;   // (32) instances per packed group = contra
 // about 4e-8 * range in the factor - two to four times the error of the reference's own fp32 arithmetic on the same
 // data.  Measured against the fp64 oracle the gradients stay within the 1e-4 bar up to ranges of about 50 (at most 7e-5
 // at 48, 1.15e-4 at 64, 1.2e-4 at 77 on the tests' data; the reference's fp32 arithmetic: 1.5 ... 3e-5); the forward
-// pass's 90 is a bound against overflow, not this one.  Beyond it a region goes term by term (about 14 times slower).
+// pass's 90 is a bound against overflow, not this one.  Beyond it a region goes term by term (about 12 times slower).
 constexpr float kGradProductRange = 48.0f;
 constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) up to which a few instances give the bound
 constexpr int GM_KT = 64;
@@ -582,11 +598,18 @@ __device__ __forceinline__ void mex_grad_offsets_wave(const MexGradArgs &ga, int
         const size_t gplane = pooled_g_plane(ga, plane);
         const float *gp = ga.g + (size_t)px.b * a.M * gplane + (valid ? pooled_g_offset(ga, px.out_off) : 0);
         const float *op = ga.out + (size_t)px.b * a.M * plane + (valid ? px.out_off : 0);
+        float gv[GO_MT], ov[GO_MT];
+#pragma unroll
+        for (int i = 0; i < GO_MT; ++i) {   // (all requests first, on clamped rows)
+            const int mc = min(m0 + i, a.M - 1);
+            gv[i] = gp[(size_t)mc * gplane];
+            ov[i] = op[(size_t)mc * plane];
+        }
 #pragma unroll
         for (int i = 0; i < GO_MT; ++i) {
             const bool mok = valid && m0 + i < a.M;
-            const float g = mok ? gp[(size_t)(m0 + i) * gplane] : 0.0f;
-            const float o = mok ? op[(size_t)(m0 + i) * plane] : 0.0f;
+            const float g = mok ? gv[i] : 0.0f;
+            const float o = mok ? ov[i] : 0.0f;
 #pragma unroll
             for (int j = 0; j < GO_KT; ++j) {
                 const float e = mex_term(xk[j] + of[i][j], o, g, a.c1, a.c0, finite);
