@@ -112,8 +112,42 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
     bool prod = false;
     if (a.finite_eps) {
         const float *rng = a.orng + ((size_t)r * a.n_mgroups + mgroup) * TM;
-        const int wide = tid < TM ? !(rng[tid] <= kProductRange) : 0;
-        prod = !__syncthreads_or(wide);
+        const float rg = tid < TM ? rng[tid] : 0.0f;
+        prod = !__syncthreads_or(!(rg <= kProductRange));
+        if (!prod && !(KGATHER && a.kgather)) {
+            // Rows too wide on their own but finite: the product form still holds where every pixel's patch spans at
+            // most kProductRange (see there).  One extra sweep over the patches, only in such workgroups: thread
+            // (pixel sp, phase sk) takes the elements sk, sk + KSTEP, ... of its pixel.
+            const int any_unbounded = __syncthreads_or(!(rg < INFINITY));
+            float hi = -INFINITY, lo = INFINITY;
+            for (int k = sk_u; k < a.K; k += KSTEP) {
+                const int4 ke = a.ktab[k];
+                bool ok = true;
+                if (CHECK) {
+                    const int ci = gp.ci0 + ke.y, hi_ = gp.hi0 + ke.z, wi = gp.wi0 + ke.w;
+                    ok = ci >= 0 && ci < a.C && hi_ >= 0 && hi_ < a.H && wi >= 0 && wi < a.W;
+                }
+                const float raw = *(ok ? gp.base + ke.x : a.in);   // (always a valid address)
+                const float v = (ok ? raw : a.oob) * a.scale;
+                hi = fmaxf(hi, v);
+                lo = fminf(lo, v);
+            }
+            pmx[sk * TP + sp] = hi;
+            __syncthreads();
+            float chi = hi;
+#pragma unroll
+            for (int j = 0; j < KSTEP; ++j)
+                chi = fmaxf(chi, pmx[j * TP + sp]);
+            __syncthreads();
+            pmx[sk * TP + sp] = lo;
+            __syncthreads();
+            float clo = lo;
+#pragma unroll
+            for (int j = 0; j < KSTEP; ++j)
+                clo = fminf(clo, pmx[j * TP + sp]);
+            // (a pixel with an infinite value, or nothing finite, is not narrow; the barrier frees the array again)
+            prod = !__syncthreads_or(!(chi - clo <= kProductRange)) && !any_unbounded;
+        }
     }
     const float *offp = (prod ? a.offe : a.offp) + ((size_t)r * a.n_mgroups + mgroup) * a.K * TM;
     float m_run = -INFINITY;  // running maximum of this thread's staging pixel (product form)

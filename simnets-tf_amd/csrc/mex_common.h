@@ -43,10 +43,10 @@ struct MexKernelArgs {
 // The forward kernels' product form sum_k exp2(x_k - max x) * exp2(o_k - max o): its largest term is at least
 // exp2(-range of the row's scaled offsets) (take k where the patch peaks) and at least exp2(-range of the pixel's scaled
 // patch) (take k where the offsets peak).  While one of the two ranges is at most this many exponents of two the sum
-// stays far inside the normal range and the terms that underflow lie below its last bit.  The kernels that hold a
-// pixel's whole patch when they decide (the panel kernel, the wave-per-pixel kernel, the fused kernel on patches of
-// a single chunk) accept wide finite offsets rows on narrow pixels; the tiled kernel and the fused kernel on longer
-// patches, which would know the pixel's range only after a sweep over K, decide on the offsets' ranges alone.
+// stays far inside the normal range and the terms that underflow lie below its last bit.  Every forward kernel
+// decides on the offsets' ranges first (known from the pack) and, in a workgroup that has a wide but finite row, on
+// its pixels' patch ranges: the panel and the wave-per-pixel kernel hold the whole patch anyway, the fused and the
+// tiled kernel sweep the patches once more for it (not the tiled kernel's k-oriented gather, which keeps the first rule).
 constexpr float kProductRange = 90.0f;
 
 struct PixelRef {

@@ -303,7 +303,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
     // Product form or term by term: decided from the packed row ranges, after the first chunk's loads have been
     // issued (those assume the product form; a workgroup that turns out wide loads again).  Rows whose range is too
     // wide on its own but finite keep the product form when the patch of every pixel column spans at most
-    // kProductRange (see there) - known here when the patch is a single chunk, which the registers then hold.
+    // kProductRange (see there): the first chunk is in the registers, the others take a sweep of their own.
     auto decide = [&]() {
         int wide = 0, unbounded = 0;
         if (tid < TM) {
@@ -316,8 +316,6 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
         }
         if (!__syncthreads_or(wide))
             return true;
-        if (a.K > KC)
-            return false;
         const int any_unbounded = __syncthreads_or(unbounded);
         float hi = -INFINITY, lo = INFINITY;
 #pragma unroll
@@ -327,6 +325,18 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_kernel(const MexKernelArgs 
                 hi = fmaxf(hi, v);
                 lo = fminf(lo, v);
             }
+        // (longer patches: one extra sweep over the remaining chunks, only in workgroups with such a row)
+        for (int k0 = KC; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            float v[U];
+            gather(k0, kc, v);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (sk + u * KSTEP < kc) {
+                    hi = fmaxf(hi, v[u] * a.scale);
+                    lo = fminf(lo, v[u] * a.scale);
+                }
+        }
         pmx[sk * XP + col] = hi;
         xs[sk * XP + col] = lo;   // (the tile is filled later)
         __syncthreads();

@@ -416,25 +416,31 @@ def test_mex_offset_ranges_product_and_two_sweep_forms(pkg, geom, spread, eps):
     assert mex_err(got, x, off, n, **kw) <= MEX_TOL
 
 
-@pytest.mark.parametrize("im,n", [((9, 32, 16, 16), 64), ((21, 128, 4, 4), 70), ((45, 256, 2, 2), 40)])
+@pytest.mark.parametrize("im,n,blocks", [
+    ((9, 32, 16, 16), 64, None), ((21, 128, 4, 4), 70, None), ((45, 256, 2, 2), 40, None),   # panel and fused kernels
+    ((7, 100, 4, 4), 70, None),                   # fused kernel, several chunks; tiled kernel with K split over the waves
+    ((4, 8, 20, 20), 33, [8, 3, 3]),              # tiled kernel, spatial blocks with padding
+    ((3, 40, 12, 12), 20, None),                  # tiled kernel, two chunks
+])
 @pytest.mark.parametrize("eps", [1.0, -2.0])
 @pytest.mark.parametrize("span", [80.0, 100.0])
-def test_mex_wide_offsets_with_patch_and_offsets_against_each_other(pkg, im, n, eps, span):
-    """Panel form, offsets rows spanning far more than the product form's range.  The workgroup still takes the product
-    form when every pixel's patch spans at most that range (span 80: below it, in units of the scaled exponent; 100:
-    above it, the max-tracked log-sum-exp).  The case that stresses the bound: patch values and offsets run against
-    each other, so the largest term is neither where the patch nor where the offsets peak, and the offsets of most
-    terms lie hundreds of units below their row's maximum."""
+def test_mex_wide_offsets_with_patch_and_offsets_against_each_other(pkg, im, n, blocks, eps, span):
+    """Offsets rows spanning far more than the product form's range.  The workgroup still takes the product form when
+    every pixel's patch spans at most that range (span 80: below it, in units of the scaled exponent; 100: above it,
+    the max-tracked log-sum-exp).  The case that stresses the bound: patch values and offsets run against each other,
+    so the largest term is neither where the patch nor where the offsets peak, and the offsets of most terms lie
+    hundreds of units below their row's maximum."""
     g = np.random.default_rng(61)
     Cc = im[1]
-    kw = dict(softmax_mode=True, blocks=[Cc, 1, 1], strides=[Cc, 1, 1], epsilon=eps, use_unshared_regions=True,
-              unshared_offset_region=[1, 2, 2])
+    blocks = blocks or [Cc, 1, 1]
+    kw = dict(softmax_mode=True, blocks=blocks, strides=[Cc, 1, 1], padding=[0, blocks[1] // 2, blocks[2] // 2], epsilon=eps,
+              use_unshared_regions=True, unshared_offset_region=[1, 2, 2], blocks_out_of_bounds_value=0.0)
     c1 = abs(eps) * math.log2(math.e)
     ramp = np.linspace(-0.5, 0.5, Cc, dtype=np.float32)
     x = (ramp[None, :, None, None] * (span / c1) * g.uniform(0.6, 0.97, size=(im[0], 1, im[2], im[3]))
          + g.normal(size=im) * 0.01).astype(np.float32)
     off = (-ramp[None, None, :, None, None] * g.uniform(0.5, 8.0, size=(4, n, 1, 1, 1)) * (span / c1)
-           + g.normal(size=(4, n, Cc, 1, 1)) * 0.3).astype(np.float32)
+           + g.normal(size=(4, n) + tuple(blocks)) * 0.3).astype(np.float32)
     got = run_mex(pkg, x, off, n, **kw)
     assert np.isfinite(got).all()
     assert mex_err(got, x, off, n, **kw) <= MEX_TOL
