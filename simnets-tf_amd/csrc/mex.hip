@@ -645,19 +645,21 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
         each([&](int k, float x) { dst[(size_t)k * tm] = mex_scaled_offset(x, lse, scale); });
         return;
     }
-    float hi = -INFINITY, lo = INFINITY;
+    // the row's extreme elements (scaling is monotone: they give the largest and the smallest scaled value)
+    float xmx = -INFINITY, xmn = INFINITY;
     each([&](int, float x) {
-        const float v = mex_scaled_offset(x, lse, scale);
-        hi = fmaxf(hi, v);
-        lo = fminf(lo, v);
+        xmx = fmaxf(xmx, x);
+        xmn = fminf(xmn, x);
     });
     for (int d = 32; d > 0; d >>= 1) {
-        hi = fmaxf(hi, __shfl_xor(hi, d, 64));
-        lo = fminf(lo, __shfl_xor(lo, d, 64));
+        xmx = fmaxf(xmx, __shfl_xor(xmx, d, 64));
+        xmn = fminf(xmn, __shfl_xor(xmn, d, 64));
     }
+    const float xh = scale >= 0.0f ? xmx : xmn;
+    const float hi = mex_scaled_offset(xh, lse, scale), lo = mex_scaled_offset(scale >= 0.0f ? xmn : xmx, lse, scale);
     each([&](int k, float x) {
         const float v = mex_scaled_offset(x, lse, scale);
-        const float e = __builtin_amdgcn_exp2f(v - hi);
+        const float e = __builtin_amdgcn_exp2f(mex_offset_exponent(x, xh, lse, scale));
         dst[(size_t)k * tm] = v;
         dste[(size_t)k * tm] = e;
         if (dste2 != nullptr)

@@ -135,6 +135,15 @@ __device__ __forceinline__ float mex_scaled_offset(float x, float lse, float sca
     return (x - lse) * scale;
 }
 
+// The exponent of a packed offset's exponential, 2^(scaled offset - row maximum), from the offsets themselves: the
+// difference to the row's extreme element first, then the scale - one rounding at the size of the difference instead of
+// two at the size of the offsets (xh: the element whose scaled value is the row maximum).
+__device__ __forceinline__ float mex_offset_exponent(float x, float xh, float lse, float scale)
+{
+#pragma clang fp contract(off)
+    return ((x - lse) - (xh - lse)) * scale;
+}
+
 // exp(d) for d <= 0 and the row's logsumexp from the sum of such terms, as the packing paths compute them for
 // normalize_offsets: one v_exp_f32 / v_log_f32 each (results within about an ulp of the library functions', at a
 // tenth of their instructions: a workgroup that packs for itself evaluates 32 of them per thread), in one place so

@@ -177,13 +177,21 @@ __global__ __launch_bounds__(256) void mex_grad_input_kernel(const MexGradArgs g
 // workgroup falls back to the term-by-term waves.
 // grid.x: (region, pixel chunk of 64 slots); grid.y: tile of GM_KT patch elements (16 per wave)
 constexpr int GM_TM = kGradPackTm;   // (32) instances per packed group = contraction chunk
-// Widest offsets range (an exponent of two) the gradients' product form takes.  Its factors 2^(xs - a), 2^(os - mo) and W
-// carry exponents of up to the range, each rounded once: an error of ulp(range) in an exponent is a relative error of
-// about 4e-8 * range in the factor - two to four times the error of the reference's own fp32 arithmetic on the same
-// data.  Measured against the fp64 oracle the gradients stay within the 1e-4 bar up to ranges of about 50 (at most 7e-5
-// at 48, 1.15e-4 at 64, 1.2e-4 at 77 on the tests' data; the reference's fp32 arithmetic: 1.5 ... 3e-5); the forward
-// pass's 90 is a bound against overflow, not this one.  Beyond it a region goes term by term (about 12 times slower).
+// Widest offsets range (an exponent of two) the gradients' product form takes on the loose bound a (below).  Its factors
+// 2^(xs - a), 2^(os - mo) and W then carry exponents of up to the range, each rounded once: an error of ulp(range) in an
+// exponent is a relative error of about 4e-8 * range in the factor - two to four times the error of the reference's own
+// fp32 arithmetic on the same data.  Measured against the fp64 oracle the gradients stay within the 1e-4 bar up to
+// ranges of about 50 (at most 8e-5 at 48, 1.15e-4 at 64, 1.2e-4 at 77 on the tests' data; the reference's fp32 arithmetic:
+// 1.5 ... 3e-5); the forward pass's 90 is a bound against overflow, not this one.  Beyond it the gathering kernels take
+// a region term by term (about 12 times slower); the row-wise kernels switch to a tight bound (kGradRowsRange).
 constexpr float kGradProductRange = 48.0f;
+// Row-wise kernels: widest patch range of a pixel (exponents of two) for which a region with large offsets ranges
+// keeps the product form on the pixel's own maximum as the bound (the factors' exponents stay within this range)
+constexpr float kGradPixelRange = 64.0f;
+// ... and the widest offsets range such a region may have: with the tight bound the factors' errors follow the size of the
+// offsets themselves, as the reference's own do, at 1.5 to 2.4 times its error: within 1e-4 up to ranges of about 70 on the
+// tests' data (4e-5 ... 7e-5 at 77, 1.5e-4 at 88 on one seeded layer, 9e-5 ... 1.3e-4 at 110)
+constexpr float kGradRowsRange = 64.0f;
 constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) up to which a few instances give the bound
 constexpr int GM_KT = 64;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -921,15 +929,16 @@ __device__ __forceinline__ void rows_quad_g(const MexGradArgs &ga, const float4 
     gg[3] = ga.gpool ? v.y : v.w;
 }
 
-// per region: does some instance's offsets range exceed the product form's (flags[r]); flags[4]: does some range
-// exceed kLooseBoundRange.  All threads of the workgroup call it; the flags are in place behind its last barrier.
+// per region: is some instance's offsets range beyond kGradRowsRange or not finite (flags[r]: term by term); flags[4]:
+// does some range exceed kLooseBoundRange; flags[5]: does some range exceed kGradProductRange.  All threads of the
+// workgroup call it; the flags (six) are in place behind its last barrier.
 // (All loads go out before the first is looked at.)
 __device__ __forceinline__ void rows_ranges(const MexKernelArgs &a, int tid, int *flags)
 {
-    if (tid < 5)
+    if (tid < 6)
         flags[tid] = 0;
     const int per = a.n_mgroups * GM_TM;
-    int big = 0, wide[4] = {0, 0, 0, 0};
+    int big = 0, mid = 0, wide[4] = {0, 0, 0, 0};
     for (int mb = 0; mb < a.M; mb += 1024) {
         float v[4][4];
 #pragma unroll
@@ -943,7 +952,8 @@ __device__ __forceinline__ void rows_ranges(const MexKernelArgs &a, int tid, int
             for (int r = 0; r < 4; ++r)
                 if (mb + 256 * u + tid < a.M) {
                     big |= !(v[u][r] <= kLooseBoundRange);
-                    wide[r] |= !(v[u][r] <= kGradProductRange);
+                    mid |= !(v[u][r] <= kGradProductRange);
+                    wide[r] |= !(v[u][r] <= kGradRowsRange);
                 }
     }
     __syncthreads();
@@ -952,6 +962,8 @@ __device__ __forceinline__ void rows_ranges(const MexKernelArgs &a, int tid, int
     for (int r = 0; r < 4; ++r)
         if (__any(wide[r]) && first)
             flags[r] = 1;   // (every writer writes the same value)
+    if (__any(mid) && first)
+        flags[5] = 1;
     if (__any(big) && first)
         flags[4] = 1;
     __syncthreads();
@@ -974,7 +986,7 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
     __shared__ __attribute__((aligned(16))) float smem[kTile];
     __shared__ float ap[256];          // per column: the pixel's bound (0 for an empty slot)
     __shared__ float tab[2][128];      // per (region, instance of the group): omax + c0, for this group and the next
-    __shared__ int wide_sh[5];         // per region: wide offsets range; [4]: some range beyond the loose bound's
+    __shared__ int wide_sh[6];         // per region: term by term; [4]: some range beyond the loose bound's
     float *wt = smem, *eo = smem + kWt, *ot = smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1037,13 +1049,47 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
     request_bound(0, min(a.M, 4));
     rows_ranges(a, tid, wide_sh);
     const int roomy = wide_sh[4];
-    const bool my_wide = wide_sh[wave] != 0;
-    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
-    const int m_scan = roomy ? a.M : min(a.M, 4);
-    float amin = INFINITY;             // of column tid
+    const bool slot_ok = chunk * 64 + (tid & 63) < a.slots;
+    // Large offsets ranges: the bound from `out` and the offsets' minima is loose by up to the range, which costs the
+    // factors their precision (and, beyond kGradProductRange, the product form).  The pixel's own maximum over all of
+    // K - one sweep over the rows of the input - is tight: the exponents then stay within the pixel's patch range, and
+    // a region keeps the product form while those ranges are at most kGradPixelRange and its offsets span at most
+    // kGradRowsRange.
+    float amin = INFINITY;             // the bound of column tid
+    if (roomy) {
+        float amax = -INFINITY, alo = INFINITY;
+        for (int kb = 0; kb < a.K; kb += 32) {
+            float4 xr[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                xr[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + min(kb + pl0 + 4 * j, a.K - 1)) * HW + q.pix0);
+            __syncthreads();           // the previous block's readers are done with the tile
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int pl = pl0 + 4 * j;
+                const bool use = q.img_ok && kb + pl < a.K;
+                const float v[4] = {xr[j].x, xr[j].y, xr[j].z, xr[j].w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    wt[pl * WP + q.col[e]] = use ? v[e] * a.c1 : __builtin_nanf("");   // (fmax / fmin skip NaN)
+            }
+            __syncthreads();
+#pragma unroll 8
+            for (int pl = 0; pl < 32; ++pl) {
+                const float t = wt[pl * WP + tid];
+                amax = fmaxf(amax, t);
+                alo = fminf(alo, t);
+            }
+        }
+        // a pixel with an infinite value, nothing finite, or a patch range beyond the bound sends its region term by term
+        const bool px_ok = !slot_ok || (fabsf(amax) < INFINITY && amax - alo <= kGradPixelRange);
+        const int bad = __any(!px_ok) ? 1 : 0;
+        if (lane == 0)
+            wide_sh[wave] |= bad;      // (columns of wave w belong to region w)
+        amin = amax;
+    }
+    const int m_scan = roomy ? 0 : min(a.M, 4);
     for (int mb = 0; mb < m_scan; mb += 32) {
-        if (roomy)
-            request_bound(mb, m_scan);
         if (tid < 128)
             tab[0][tid] = lo_n;
         __syncthreads();               // tab in place; the previous block's readers are done with the tile
@@ -1062,10 +1108,12 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
         for (int pl = 0; pl < 32; ++pl)
             amin = fminf(amin, wt[pl * WP + tid]);
     }
-    ap[tid] = chunk * 64 + (tid & 63) < a.slots ? amin : 0.0f;
+    ap[tid] = slot_ok ? amin : 0.0f;
     if (tid < 128 && mg_begin < mg_end)   // (the loop above is done with the table: its last readers passed the
         tab[mg_begin & 1][tid] = a.omax[(tid >> 5) * per + mg_begin * GM_TM + (tid & 31)] + a.c0;   // barrier in front of the reduction)
     __syncthreads();
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
     float bound[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e)
@@ -1091,7 +1139,8 @@ __global__ __launch_bounds__(256, KSUB == 1 ? 3 : KSUB == 2 ? 2 : 1) void mex_gr
             rows_quad_g(ga, gv[j], gg);
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                // (a - outs) first: a small, once-rounded difference; the instance constant is added to that
+                // (a - outs) first: a small, once-rounded difference; the instance constant is added to that (forming
+                // a + mo first, about the size of outs, was tried for the tight bound: worse on half of the data)
                 const float ex = __builtin_fmaf(-o[e], a.c1, bound[e]) + tb[(q.rbase + (e & 1)) * 32 + pl];
                 wt[pl * WP + q.col[e]] = use ? gg[e] * __builtin_amdgcn_exp2f(ex) : 0.0f;
             }
@@ -1189,7 +1238,7 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
     __shared__ float wt[32 * TP];      // [instance][column]
     __shared__ float ex[32 * TP];      // [patch element][column]
     __shared__ float pm[4 * 256];      // per column: the four waves' minima
-    __shared__ int wide_sh[5];
+    __shared__ int wide_sh[6];
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lr = lane & 15, lq = lane >> 4;
@@ -1240,8 +1289,13 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
     if (n_steps > 0)
         request(0);
     rows_ranges(a, tid, wide_sh);      // (behind the requests above: one wait for everything)
-    const bool my_wide = wide_sh[wave] != 0;
-    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
+    // Some range beyond kGradProductRange: the bound of every pixel is its own maximum over all of K (a sweep over the
+    // rows of the input per chunk, see mex_grad_input_rows_kernel); a region then keeps the product form unless a range
+    // of its offsets is beyond kGradRowsRange (or not finite) or one of its pixels spans more than kGradPixelRange
+    // (found while sweeping: `bad`, which discards the region's sums at the end).
+    const bool sweep = wide_sh[5] != 0;
+    const bool unbounded = wide_sh[wave] != 0;   // (or beyond kGradRowsRange: term by term whatever the pixels)
+    int bad = unbounded ? 1 : 0;
     // the offset exponentials of the epilogue: requested in front of the last matrix steps
     float eov[2][2][4];
     for (int s = 0; s < n_steps; ++s) {
@@ -1256,16 +1310,53 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
             for (int e = 0; e < 4; ++e)
                 cand[e] = fminf(cand[e], __builtin_fmaf(o[e], a.c1, -lo[j][e & 1]));
         }
-        __syncthreads();               // the previous chunk's matrix steps are done with wt / ex, its readers with pm
-#pragma unroll
-        for (int e = 0; e < 4; ++e)
-            pm[pl0 * 256 + q0.col[e]] = cand[e];
-        __syncthreads();
         float bound[4];
+        if (sweep) {
+            const RowsQuad q = rows_quad(a, g, bx * ga.pxl + s, lane);
+            const size_t img = q.img_ok ? q.img : 0;
+            float amax = -INFINITY, alo = INFINITY;
+            for (int kb = 0; kb < a.K; kb += 32) {
+                float4 xr[8];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int c = q0.col[e];
-            bound[e] = cur_ok ? fminf(fminf(pm[c], pm[256 + c]), fminf(pm[512 + c], pm[768 + c])) : 0.0f;
+                for (int j = 0; j < 8; ++j)
+                    xr[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + min(kb + pl0 + 4 * j, a.K - 1)) * HW + q.pix0);
+                __syncthreads();       // the previous matrix steps / the previous block's readers are done with the tile
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    const int pl = pl0 + 4 * j;
+                    const bool use = q.img_ok && kb + pl < a.K;
+                    const float v[4] = {xr[j].x, xr[j].y, xr[j].z, xr[j].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        wt[pl * TP + q0.col[e]] = use ? v[e] * a.c1 : __builtin_nanf("");   // (fmax / fmin skip NaN)
+                }
+                __syncthreads();
+#pragma unroll 8
+                for (int pl = 0; pl < 32; ++pl) {
+                    const float t = wt[pl * TP + tid];
+                    amax = fmaxf(amax, t);
+                    alo = fminf(alo, t);
+                }
+            }
+            const bool slot_ok = (bx * ga.pxl + s) * 64 + (tid & 63) < a.slots;
+            const bool px_ok = !slot_ok || (fabsf(amax) < INFINITY && amax - alo <= kGradPixelRange);
+            bad |= __any(!px_ok) ? 1 : 0;          // (columns of wave w belong to region w)
+            pm[tid] = slot_ok ? amax : 0.0f;
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                bound[e] = cur_ok ? pm[q0.col[e]] : 0.0f;
+        } else {
+            __syncthreads();           // the previous chunk's matrix steps are done with wt / ex, its readers with pm
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                pm[pl0 * 256 + q0.col[e]] = cand[e];
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int c = q0.col[e];
+                bound[e] = cur_ok ? fminf(fminf(pm[c], pm[256 + c]), fminf(pm[512 + c], pm[768 + c])) : 0.0f;
+            }
         }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -1297,7 +1388,7 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
                 }
         }
         __syncthreads();
-        if (!my_wide) {
+        if (!unbounded) {
 #pragma unroll 4
             for (int ps = 0; ps < 64; ps += 4) {
                 float wa[2], xb[2];
@@ -1315,6 +1406,14 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
         }
     }
     // ---- partial sums of this chunk group: acc * 2^(os_mk - mo_m) ----
+    if (sweep) {
+        __syncthreads();               // (everyone has read the flags)
+        if (lane == 0)
+            wide_sh[wave] = bad;
+        __syncthreads();
+    }
+    const bool my_wide = wide_sh[wave] != 0;
+    const bool any_wide = (wide_sh[0] | wide_sh[1] | wide_sh[2] | wide_sh[3]) != 0;
     if (!my_wide) {
         float *dst = ga.partial + ((size_t)bx * a.R + wave) * a.M * a.K;
 #pragma unroll

@@ -557,7 +557,7 @@ struct PanelArgs {
 // the lanes of that kernel hold one element each and add their exponentials in a butterfly (partner lane ^ 32, 16, 8,
 // 4, 2, 1; the upper half of the wave holds zeros for a row of 32), which is the tree below.
 __device__ __forceinline__ void pack_row32(const float (&x)[32], int normalize, float scale, float &lse, float &hi,
-                                           float &lo)
+                                           float &lo, float &xh)
 {
     lse = 0.0f;
     if (normalize) {
@@ -578,14 +578,15 @@ __device__ __forceinline__ void pack_row32(const float (&x)[32], int normalize, 
                 e[k] = e[k] + e[k + d];
         lse = mex_lse_of(e[0], mxv);
     }
-    hi = -INFINITY;
-    lo = INFINITY;
+    float xmx = -INFINITY, xmn = INFINITY;
 #pragma unroll
     for (int k = 0; k < 32; ++k) {
-        const float v = mex_scaled_offset(x[k], lse, scale);
-        hi = fmaxf(hi, v);
-        lo = fminf(lo, v);
+        xmx = fmaxf(xmx, x[k]);
+        xmn = fminf(xmn, x[k]);
     }
+    xh = scale >= 0.0f ? xmx : xmn;
+    hi = mex_scaled_offset(xh, lse, scale);
+    lo = mex_scaled_offset(scale >= 0.0f ? xmn : xmx, lse, scale);
 }
 
 // POOL = false: the same tiling without the pooling, every MEX value stored (the plain MEX call on such a layer).
@@ -714,14 +715,14 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         reinterpret_cast<float4 *>(pmx)[kslot * (XP / 4) + cg] = pm;
     }
     float rx[SELFPACK ? KC : 1];   // SELFPACK: the row, its logsumexp (0 without normalisation) and its scaled maximum
-    float row_lse = 0.0f, row_hi = 0.0f;
+    float row_lse = 0.0f, row_hi = 0.0f, row_xh = 0.0f;
     if constexpr (SELFPACK) {
 #pragma unroll
         for (int i = 0; i < KC / 4; ++i) {
             rx[4 * i] = rw[i].x; rx[4 * i + 1] = rw[i].y; rx[4 * i + 2] = rw[i].z; rx[4 * i + 3] = rw[i].w;
         }
         float lo;
-        pack_row32(rx, g.normalize, a.scale, row_lse, row_hi, lo);
+        pack_row32(rx, g.normalize, a.scale, row_lse, row_hi, lo, row_xh);
         if (row_valid) {
             wide = !(row_hi - lo <= kProductRange);
             unbounded = !(row_hi - lo < INFINITY);    // NaN or inf (infinite entries) sends the workgroup to the VALU form
@@ -800,7 +801,7 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
 #pragma unroll
                 for (int k = 0; k < KC; ++k)
                     orow[k * TM + (mi ^ ((k & 3) << 4))] =
-                        row_valid ? __builtin_amdgcn_exp2f(mex_scaled_offset(rx[k], row_lse, a.scale) - row_hi) : 0.0f;
+                        row_valid ? __builtin_amdgcn_exp2f(mex_offset_exponent(rx[k], row_xh, row_lse, a.scale)) : 0.0f;
             } else {
                 float4 *dst = reinterpret_cast<float4 *>(os) + ((tid & ~15) | ((tid & 15) ^ (((tid >> 4) & 3) << 2)));
 #define SIMNETS_PANEL_PUT(i) dst[((i) / NO) * TILE4 + ((i) % NO) * kThreads] = on##i;
