@@ -1316,19 +1316,24 @@ __global__ __launch_bounds__(256, 2) void mex_grad_offsets_rows_kernel(const Mex
             const size_t img = q.img_ok ? q.img : 0;
             float amax = -INFINITY, alo = INFINITY;
             for (int kb = 0; kb < a.K; kb += 32) {
-                float4 xr[8];
-#pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    xr[j] = *reinterpret_cast<const float4 *>(a.in + (img * a.K + min(kb + pl0 + 4 * j, a.K - 1)) * HW + q.pix0);
                 __syncthreads();       // the previous matrix steps / the previous block's readers are done with the tile
+                // (two rows at a time: the chunk's own operands stay in their registers meanwhile)
 #pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    const int pl = pl0 + 4 * j;
-                    const bool use = q.img_ok && kb + pl < a.K;
-                    const float v[4] = {xr[j].x, xr[j].y, xr[j].z, xr[j].w};
+                for (int h = 0; h < 4; ++h) {
+                    float4 xr[2];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        wt[pl * TP + q0.col[e]] = use ? v[e] * a.c1 : __builtin_nanf("");   // (fmax / fmin skip NaN)
+                    for (int j = 0; j < 2; ++j)
+                        xr[j] = *reinterpret_cast<const float4 *>(
+                            a.in + (img * a.K + min(kb + pl0 + 4 * (2 * h + j), a.K - 1)) * HW + q.pix0);
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const int pl = pl0 + 4 * (2 * h + j);
+                        const bool use = q.img_ok && kb + pl < a.K;
+                        const float v[4] = {xr[j].x, xr[j].y, xr[j].z, xr[j].w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            wt[pl * TP + q0.col[e]] = use ? v[e] * a.c1 : __builtin_nanf("");   // (fmax / fmin skip NaN)
+                    }
                 }
                 __syncthreads();
 #pragma unroll 8
