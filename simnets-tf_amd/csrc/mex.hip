@@ -57,9 +57,11 @@ constexpr int cmax(int a, int b) { return a > b ? a : b; }
 
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
-template <int PX, int KS, int KC, bool NEG, bool CHECK>
+// EPS: 0 = finite epsilon, +1 / -1 = epsilon +inf / -inf (plain maximum / minimum of patch + offset).
+template <int PX, int KS, int KC, int EPS, bool CHECK>
 __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const MexKernelArgs a)
 {
+    constexpr bool NEG = EPS < 0, INF = EPS != 0;
     constexpr int WM = 4 / KS;            // instance waves per workgroup
     constexpr int TM = WM * MX;           // instances per workgroup
     constexpr int TP = 64 * PX;           // pixels per workgroup
@@ -110,7 +112,7 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
     // of all instances of the workgroup are small enough for that to stay far inside the normal range; otherwise
     // the workgroup runs the two sweeps.
     bool prod = false;
-    if (a.finite_eps) {
+    if constexpr (!INF) {
         const float *rng = a.orng + ((size_t)r * a.n_mgroups + mgroup) * TM;
         const float rg = tid < TM ? rng[tid] : 0.0f;
         prod = !__syncthreads_or(!(rg <= kProductRange));
@@ -380,6 +382,56 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
     //      at chunk granularity, one exponential per term and one per output and chunk; the patch elements and the
     //      offsets are fetched once.  Patch values and offsets are already multiplied by eps*log2(e), so a term is
     //      exp2 of a plain difference.  Infinite epsilon stops after the maximum. ----
+    if constexpr (INF) {
+        // The extreme value alone: two k per step, a term is an add whose offset operand comes from another lane of
+        // the quad and half a three-operand maximum.  Lane q of a quad fetches instances 4q .. 4q + 3 of the wave's
+        // 16 (one 16-byte read per lane and k instead of four: the reads of a step are what the LDS return path
+        // carries, whether or not the lanes ask for the same address).
+        auto quad = [](float v, auto q) {
+            return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
+                                                                         decltype(q)::value * 0x55, 0xF, 0xF, true));
+        };
+        auto best3 = [](float m, float p, float q) {
+            return NEG ? __builtin_fminf(__builtin_fminf(m, p), q) : __builtin_fmaxf(__builtin_fmaxf(m, p), q);
+        };
+        const float *oq = ol + 4 * (lane & 3);
+        for (int k0 = 0; k0 < a.K; k0 += KC) {
+            const int kc = min(KC, a.K - k0);
+            __syncthreads();
+            stage(k0, kc);
+            __syncthreads();
+            if (!wave_active)
+                continue;
+            const int kend = min(kc, (wk + 1) * KW);
+#pragma unroll 2
+            for (int kk = wk * KW; kk < kend; kk += 2) {
+                const int k1 = min(kk + 1, kend - 1);   // (an odd count takes its last k twice)
+                float x0[PX], x1[PX];
+#pragma unroll
+                for (int p = 0; p < PX; ++p) {
+                    x0[p] = xl[kk * XP + p * 64];
+                    x1[p] = xl[k1 * XP + p * 64];
+                }
+                const float4 f0 = *reinterpret_cast<const float4 *>(oq + kk * TM);
+                const float4 f1 = *reinterpret_cast<const float4 *>(oq + k1 * TM);
+                const float o0[4] = {f0.x, f0.y, f0.z, f0.w}, o1[4] = {f1.x, f1.y, f1.z, f1.w};
+#pragma unroll
+                for (int p = 0; p < PX; ++p)
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        using std::integral_constant;
+                        mx[p][j] = best3(mx[p][j], x0[p] + quad(o0[j], integral_constant<int, 0>{}),
+                                         x1[p] + quad(o1[j], integral_constant<int, 0>{}));
+                        mx[p][4 + j] = best3(mx[p][4 + j], x0[p] + quad(o0[j], integral_constant<int, 1>{}),
+                                             x1[p] + quad(o1[j], integral_constant<int, 1>{}));
+                        mx[p][8 + j] = best3(mx[p][8 + j], x0[p] + quad(o0[j], integral_constant<int, 2>{}),
+                                             x1[p] + quad(o1[j], integral_constant<int, 2>{}));
+                        mx[p][12 + j] = best3(mx[p][12 + j], x0[p] + quad(o0[j], integral_constant<int, 3>{}),
+                                              x1[p] + quad(o1[j], integral_constant<int, 3>{}));
+                    }
+            }
+        }
+    } else {
     for (int k0 = 0; k0 < a.K; k0 += KC) {
         const int kc = min(KC, a.K - k0);
         __syncthreads();
@@ -400,7 +452,7 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
             float cm[HM];
 #pragma unroll
             for (int m = 0; m < HM; ++m)
-                cm[m] = NEG ? INFINITY : -INFINITY;
+                cm[m] = -INFINITY;
 #pragma nounroll
             for (int kk = wk * KW; kk < kend; ++kk) {
                 const float x = xp[kk * XP];
@@ -413,14 +465,8 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int m = 0; m < HM; ++m)
-                    cm[m] = NEG ? __builtin_fminf(cm[m], v[m]) : __builtin_fmaxf(cm[m], v[m]);
+                    cm[m] = __builtin_fmaxf(cm[m], v[m]);
                 __builtin_amdgcn_sched_barrier(0);
-            }
-            if (!a.finite_eps) {
-#pragma unroll
-                for (int m = 0; m < HM; ++m)
-                    mx[p][h0 + m] = NEG ? __builtin_fminf(mx[p][h0 + m], cm[m]) : __builtin_fmaxf(mx[p][h0 + m], cm[m]);
-                continue;
             }
             // new running maximum; sums so far rescaled to it (a maximum that did not move: factor 1, which also keeps
             // -inf - -inf out of the exponent while nothing finite has been seen)
@@ -455,6 +501,7 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
             }
         }
     }
+    }
 
     if (KS > 1) {
         // ---- merge the (max, sum) pairs of the K-split waves into wave wk == 0 ----
@@ -467,7 +514,8 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
 #pragma unroll
                 for (int m = 0; m < MX; ++m) {
                     mg[((p * MX + m) * 2) * 64] = mx[p][m];
-                    mg[((p * MX + m) * 2 + 1) * 64] = s[p][m];
+                    if constexpr (!INF)
+                        mg[((p * MX + m) * 2 + 1) * 64] = s[p][m];
                 }
         }
         __syncthreads();
@@ -480,15 +528,18 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
                 for (int p = 0; p < PX; ++p)
 #pragma unroll
                     for (int m = 0; m < MX; ++m) {
-                        const float m2 = src[((p * MX + m) * 2) * 64], s2 = src[((p * MX + m) * 2 + 1) * 64];
+                        const float m2 = src[((p * MX + m) * 2) * 64];
                         const float m1 = mx[p][m];
                         const float mm = NEG ? __builtin_fminf(m1, m2) : __builtin_fmaxf(m1, m2);
+                        mx[p][m] = mm;
+                        if constexpr (INF)
+                            continue;
+                        const float s2 = src[((p * MX + m) * 2 + 1) * 64];
                         // a side that saw no finite term keeps sum 0; skip the rescale when its
                         // max equals the merged one (also avoids inf - inf)
                         const float f1 = (m1 == mm) ? 1.0f : __builtin_amdgcn_exp2f(m1 - mm);
                         const float f2 = (m2 == mm) ? 1.0f : __builtin_amdgcn_exp2f(m2 - mm);
                         s[p][m] = s[p][m] * f1 + s2 * f2;
-                        mx[p][m] = mm;
                     }
             }
         }
@@ -507,8 +558,7 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
 #pragma unroll
         for (int m = 0; m < MX; ++m) {
             // (max + ey*log2(e) + log2(sum)) * log(2)/eps in the scaled domain; the plain max for infinite eps
-            const float res = a.finite_eps ? (__builtin_amdgcn_logf(s[p][m]) + (mx[p][m] + a.c0)) * a.ln2_over_eps
-                                           : mx[p][m];
+            const float res = INF ? mx[p][m] : (__builtin_amdgcn_logf(s[p][m]) + (mx[p][m] + a.c0)) * a.ln2_over_eps;
             if (m0 + m < a.M)
                 o[(size_t)(m0 + m) * plane] = res;
         }
@@ -676,28 +726,32 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
 }
 
 template <int PX, int KS, int KC>
-hipError_t launch_variant(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, hipStream_t s)
+hipError_t launch_variant(const MexKernelArgs &a, dim3 grid, int eps, bool inside, hipStream_t s)
 {
-    if (neg && inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, true, false>), grid, dim3(256), 0, s, a);
-    else if (neg)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, true, true>), grid, dim3(256), 0, s, a);
+    if (eps < 0 && inside)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, -1, false>), grid, dim3(256), 0, s, a);
+    else if (eps < 0)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, -1, true>), grid, dim3(256), 0, s, a);
+    else if (eps > 0 && inside)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, 1, false>), grid, dim3(256), 0, s, a);
+    else if (eps > 0)
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, 1, true>), grid, dim3(256), 0, s, a);
     else if (inside)
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, false, false>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, 0, false>), grid, dim3(256), 0, s, a);
     else
-        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, false, true>), grid, dim3(256), 0, s, a);
+        hipLaunchKernelGGL((mex_fwd_kernel<PX, KS, KC, 0, true>), grid, dim3(256), 0, s, a);
     return hipGetLastError();
 }
 
 // one pixel per lane: the LDS chunk grows with K (fewer gather/barrier phases; K <= chunk needs one gather only)
 template <int KS>
-hipError_t launch_px1(const MexKernelArgs &a, dim3 grid, bool neg, bool inside, int kc, hipStream_t s)
+hipError_t launch_px1(const MexKernelArgs &a, dim3 grid, int eps, bool inside, int kc, hipStream_t s)
 {
     if (kc == 128)
-        return launch_variant<1, KS, 128>(a, grid, neg, inside, s);
+        return launch_variant<1, KS, 128>(a, grid, eps, inside, s);
     if (kc == 64)
-        return launch_variant<1, KS, 64>(a, grid, neg, inside, s);
-    return launch_variant<1, KS, kChunkMin>(a, grid, neg, inside, s);
+        return launch_variant<1, KS, 64>(a, grid, eps, inside, s);
+    return launch_variant<1, KS, kChunkMin>(a, grid, eps, inside, s);
 }
 
 // Few pixels, long K (the classifier head of a network: a handful of instances over hundreds of channels at 1x1
@@ -1140,16 +1194,16 @@ int mex_launch(const MexPlan &p, const float *input, const float *offsets, float
         return SIMNETS_ERR_TOO_LARGE;
     dim3 grid((unsigned)gx, (unsigned)t.n_mgroups);
     // finite eps: values are pre-multiplied by eps*log2(e), so the shift is always the maximum
-    const bool neg = !a.finite_eps && p.epsilon < 0;
+    const int eps = a.finite_eps ? 0 : p.epsilon < 0 ? -1 : 1;
     hipError_t e;
     if (t.px == 2)
-        e = launch_variant<2, 1, kChunkMin>(a, grid, neg, inside, s);
+        e = launch_variant<2, 1, kChunkMin>(a, grid, eps, inside, s);
     else if (t.ks == 1)
-        e = launch_px1<1>(a, grid, neg, inside, t.kc, s);
+        e = launch_px1<1>(a, grid, eps, inside, t.kc, s);
     else if (t.ks == 2)
-        e = launch_px1<2>(a, grid, neg, inside, t.kc, s);
+        e = launch_px1<2>(a, grid, eps, inside, t.kc, s);
     else
-        e = launch_px1<4>(a, grid, neg, inside, t.kc, s);
+        e = launch_px1<4>(a, grid, eps, inside, t.kc, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 

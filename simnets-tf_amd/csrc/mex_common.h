@@ -36,6 +36,7 @@ struct MexKernelArgs {
     float c0;           // (softmax ? 0 : -log K) * log2(e)
     float ln2_over_eps; // log(2) / eps
     int finite_eps;
+    float inf_sign;     // infinite eps: +1 (maximum) or -1 (minimum), else 0
     int kgather;        // tiled kernel: gather patch elements with lanes along k (pixels of a chunk lie an image apart)
     float oob;
 };
@@ -116,6 +117,7 @@ inline MexKernelArgs mex_kernel_args(const MexPlan &p)
     a.M = d.M; a.K = d.K; a.n_mgroups = 0;
     const double log2e = 1.4426950408889634;
     a.finite_eps = std::isfinite(p.epsilon);
+    a.inf_sign = a.finite_eps ? 0.0f : (p.epsilon < 0 ? -1.0f : 1.0f);
     a.c1 = a.finite_eps ? (float)((double)p.epsilon * log2e) : 0.0f;
     a.scale = a.finite_eps ? a.c1 : 1.0f;
     a.ln2_over_eps = a.finite_eps ? (float)(0.6931471805599453 / (double)p.epsilon) : 0.0f;

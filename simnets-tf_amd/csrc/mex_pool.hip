@@ -99,6 +99,62 @@ __device__ __forceinline__ void lse_chunk(float (&best)[4][4], float (&sum)[4][4
     }
 }
 
+// Infinite epsilon on the panel kernel's tiles: the maximum of patch + offset alone (the caller stages negated values
+// for the minimum).  Same lane layout as above.  The 16 offsets the 16 lanes of a row need per k - instances
+// 4*lq + v of the four regions - are fetched one per lane (lane lr: region lr / 4, v = lr % 4) and reach the others
+// through the add's row broadcast, so a k costs five 4-byte LDS reads per lane; two k per step, a term is an add and
+// half a three-operand maximum.  os: [region][k][position], position = ((instance ^ (k & 3) << 4) + 16 * region) % 64
+// (the rotation by the region keeps the four regions' reads of one instruction in different banks).
+template <int XP>
+__device__ __forceinline__ void max_chunk(float (&best)[4][4], const float *xs, const float *os, int colbase, int wm,
+                                          int lr, int lq)
+{
+    auto bcast = [](float v, auto n) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v),
+                                                                     0x150 + decltype(n)::value, 0xF, 0xF, true));
+    };
+    const int ot = lr >> 2;
+    const float *op = os + ot * KC * TM;
+    const int oi = wm * MX + 4 * lq + (lr & 3);
+    // the operands of two k: x[h][tile], o[h]
+    auto fetch = [&](int kk, float (&x)[2][4], float (&o)[2]) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int k = kk + h;
+            const int sx = ((k & 3) << 4) | (((k >> 2) & 3) << 2);
+            o[h] = op[k * TM + (((oi ^ ((k & 3) << 4)) + 16 * ot) & 63)];
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+                x[h][t] = xs[k * XP + ((colbase + t * 16 + lr) ^ sx)];
+        }
+    };
+#define SIMNETS_MAX_TERM(x, o, t, v)                                                                            \
+    best[t][v] = __builtin_fmaxf(                                                                               \
+        __builtin_fmaxf(best[t][v], x[0][t] + bcast(o[0], std::integral_constant<int, 4 * (t) + (v)>{})),      \
+        x[1][t] + bcast(o[1], std::integral_constant<int, 4 * (t) + (v)>{}));
+#define SIMNETS_MAX_TILE(x, o, t) \
+    SIMNETS_MAX_TERM(x, o, t, 0) SIMNETS_MAX_TERM(x, o, t, 1) SIMNETS_MAX_TERM(x, o, t, 2) SIMNETS_MAX_TERM(x, o, t, 3)
+#define SIMNETS_MAX_STEP(x, o) \
+    SIMNETS_MAX_TILE(x, o, 0) SIMNETS_MAX_TILE(x, o, 1) SIMNETS_MAX_TILE(x, o, 2) SIMNETS_MAX_TILE(x, o, 3)
+    // two register sets: the reads of the next step are on their way while a step's 48 instructions issue
+    float xa[2][4], oa[2], xb[2][4], ob[2];
+    fetch(0, xa, oa);
+#pragma nounroll
+    for (int kk = 0; kk < KC; kk += 4) {
+        fetch(kk + 2, xb, ob);
+        __builtin_amdgcn_sched_barrier(0);
+        SIMNETS_MAX_STEP(xa, oa)
+        __builtin_amdgcn_sched_barrier(0);
+        fetch(kk + 4 < KC ? kk + 4 : 0, xa, oa);   // (the last round reads the first step again, unused)
+        __builtin_amdgcn_sched_barrier(0);
+        SIMNETS_MAX_STEP(xb, ob)
+        __builtin_amdgcn_sched_barrier(0);
+    }
+#undef SIMNETS_MAX_STEP
+#undef SIMNETS_MAX_TILE
+#undef SIMNETS_MAX_TERM
+}
+
 // NH = column halves of a workgroup (64 pixel columns = 4 tiles of 16 each), 4 instance waves per half: two halves
 // share the offsets tiles and double the waves per SIMD the LDS budget allows, which is what hides the latencies of
 // the short dependent phases; one half only when there are no slots for a second one.
@@ -593,11 +649,14 @@ __device__ __forceinline__ void pack_row32(const float (&x)[32], int normalize, 
 // SELFPACK (one column half, one chunk, no pooling): no packed offsets exist; thread (region tid / 64, instance
 // tid % 64) packs its row of the caller's offsets into the LDS tile itself (pack_row32), so that a self-packing call of
 // a small layer is this one launch.
-template <int NH, int NCH, bool POOL, bool SELFPACK = false>
+// INF (plain call only): infinite epsilon - the extreme value of patch + offset through max_chunk, from the panel and
+// the scaled offsets; nothing of the product form (column maxima, packed exponentials, row ranges) is touched.
+template <int NH, int NCH, bool POOL, bool SELFPACK = false, bool INF = false>
 __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKernelArgs a, const PoolArgs q,
                                                                   const PanelArgs g)
 {
     static_assert(!SELFPACK || (NH == 1 && NCH == 1 && !POOL), "in-kernel packing: one row per thread, one chunk");
+    static_assert(!INF || (!SELFPACK && !POOL), "infinite epsilon: the plain call on packed offsets");
     constexpr int R = 4;
     constexpr int XP = 64 * NH;
     constexpr int kThreads = 256 * NH;
@@ -662,13 +721,13 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
 #pragma unroll
         for (int i = 0; i < KC / 4; ++i)
             rw[i] = src[i];
-    } else {
+    } else if constexpr (!INF) {
         SIMNETS_PANEL_ISSUE(0)
     }
 
     // wide: an offsets row whose range is beyond the product form's on its own; unbounded: ... and not even finite
     int wide = 0, unbounded = 0;
-    if (!SELFPACK && tid < TM) {
+    if (!SELFPACK && !INF && tid < TM) {
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             const float rg = a.orng[((size_t)r * a.n_mgroups + mgroup) * TM + tid];
@@ -700,6 +759,68 @@ __global__ __launch_bounds__(256 * NH) void mex_pool_panel_kernel(const MexKerne
         const int h = pix >> g.lgW, w = pix & ((1 << g.lgW) - 1);
         const int sl = pb * g.RS + (h >> 1) * g.Ws + (w >> 1) - chunk * (16 * NH);
         colx[e] = pvalid ? (sl >> 4) * 64 + ((h & 1) * 2 + (w & 1)) * 16 + (sl & 15) : 0;
+    }
+
+    if constexpr (INF) {
+        // ---- infinite epsilon: chunk by chunk, values times the sign of epsilon (the minimum is a negated maximum) ----
+        const int lr = lane & 15, lq = lane >> 4;
+        const float sg = a.inf_sign;
+        float best[4][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                best[t][v] = -INFINITY;
+        const int sw = ((kslot & 3) << 4) | (((kslot >> 2) & 3) << 2);
+        const float4 *psrc = reinterpret_cast<const float4 *>(a.offp + (size_t)mgroup * a.K * TM) + tid;
+        const int dst_row = tid & ~15, dst_col = (tid & 15) ^ (((tid >> 4) & 3) << 2);
+        float4 ov[R * NO];   // the scaled offsets of the next chunk: float4 i of region i / NO, round i % NO
+#pragma unroll
+        for (int i = 0; i < R * NO; ++i)
+            ov[i] = psrc[(size_t)(i / NO) * ostep + (i % NO) * kThreads];
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            if (c > 0)
+                __syncthreads();  // everyone is done with the previous chunk's tiles
+#pragma unroll
+            for (int i = 0; i < R * NO; ++i) {
+                float4 *dst = reinterpret_cast<float4 *>(os) + (dst_row | ((dst_col + 4 * (i / NO)) & 15));
+                dst[(i / NO) * TILE4 + (i % NO) * kThreads] =
+                    make_float4(ov[i].x * sg, ov[i].y * sg, ov[i].z * sg, ov[i].w * sg);
+            }
+            if (pvalid) {
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 v = pv[2 * c + h];
+                    float *row = xs + (kslot + 16 * h) * XP;
+                    row[colx[0] ^ sw] = v.x * sg;
+                    row[colx[1] ^ sw] = v.y * sg;
+                    row[colx[2] ^ sw] = v.z * sg;
+                    row[colx[3] ^ sw] = v.w * sg;
+                }
+            }
+            __syncthreads();
+            if (c + 1 < NCH) {
+#pragma unroll
+                for (int i = 0; i < R * NO; ++i)
+                    ov[i] = psrc[(size_t)(i / NO) * ostep + (i % NO) * kThreads + (size_t)((c + 1) * KC) * (TM / 4)];
+            }
+            max_chunk<XP>(best, xs, os, wh * 64, wm, lr, lq);
+        }
+        if (!wave_active)
+            return;
+        const long long pos = ppos[wh * 16 + lr];  // written before the first barrier
+        if (pos < 0)
+            return;
+        float res[4][4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int v = 0; v < 4; ++v)
+                res[t][v] = best[t][v] * sg;
+        store_window(q.pooled + pos + (size_t)(m0 + 4 * lq) * g.HW, g.HW, g.lgW, q.out_pairs, res,
+                     m0 + MX <= a.M ? 4 : a.M - (m0 + 4 * lq));
+        return;
     }
 
     // ---- column maxima over all of K ----
@@ -1020,6 +1141,18 @@ hipError_t launch_panel(const MexKernelArgs &a, const PoolArgs &q, const PanelAr
     return hipGetLastError();
 }
 
+template <int NH>
+hipError_t launch_panel_inf(const MexKernelArgs &a, const PoolArgs &q, const PanelArgs &g, dim3 grid, hipStream_t s)
+{
+    switch (a.K / KC) {
+    case 1: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 1, false, false, true>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    case 2: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 2, false, false, true>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    case 4: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 4, false, false, true>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    default: hipLaunchKernelGGL((mex_pool_panel_kernel<NH, 8, false, false, true>), grid, dim3(256 * NH), 0, s, a, q, g); break;
+    }
+    return hipGetLastError();
+}
+
 // Workgroup shape of the panel form for this layer (column halves), 0 when the layer does not have its geometry.
 int panel_halves(const MexPlan &p, int ph, int pw, const float *input, int slots, int n_mgroups, PanelArgs *g,
                  bool pool)
@@ -1054,12 +1187,12 @@ hipError_t launch_pool(const MexKernelArgs &a, const PoolArgs &q, dim3 grid, boo
 }
 
 // The fused kernel applies when a pooling window is exactly one pixel of every offsets region.
-bool fusable(const MexPlan &p, int ph, int pw)
+bool fusable(const MexPlan &p, int ph, int pw, bool any_epsilon = false)
 {
     const simnets_mex_dims &d = p.d;
     const int r = ph * pw;
-    return p.use_unshared && std::isfinite(p.epsilon) && d.offsets_c == 1 && d.offsets_h == ph && d.offsets_w == pw &&
-           (r == 2 || r == 4) && d.num_regions == r;
+    return p.use_unshared && (any_epsilon || std::isfinite(p.epsilon)) && d.offsets_c == 1 && d.offsets_h == ph &&
+           d.offsets_w == pw && (r == 2 || r == 4) && d.num_regions == r;
 }
 
 // ... and the Similarity layer in front can be evaluated inside the staging when its channels are exactly the MEX
@@ -1143,7 +1276,8 @@ bool mex_panel_geometry(const MexPlan &p)
 {
     PanelArgs g;
     const long long slots = (long long)p.B * p.d.region_size;
-    if (!fusable(p, 2, 2) || slots > 0x7fffffffLL)
+    // (the plain call's panel kernel also takes an infinite epsilon)
+    if (!fusable(p, 2, 2, true) || slots > 0x7fffffffLL)
         return false;
     // (the pointer is checked by the launch; any 16-byte aligned one stands in here)
     return panel_halves(p, 2, 2, reinterpret_cast<const float *>(uintptr_t(16)), (int)slots, (p.d.M + TM - 1) / TM,
@@ -1172,7 +1306,11 @@ int mex_panel_launch(const MexPlan &p, const MexKernelArgs &a, const float *inpu
     b.in = input;
     dim3 grid((unsigned)gx, (unsigned)a.n_mgroups);
     hipStream_t s = reinterpret_cast<hipStream_t>(stream);
-    const hipError_t e = nh == 1 ? launch_panel<1, false>(b, q, g, grid, s) : launch_panel<2, false>(b, q, g, grid, s);
+    hipError_t e;
+    if (!b.finite_eps)
+        e = nh == 1 ? launch_panel_inf<1>(b, q, g, grid, s) : launch_panel_inf<2>(b, q, g, grid, s);
+    else
+        e = nh == 1 ? launch_panel<1, false>(b, q, g, grid, s) : launch_panel<2, false>(b, q, g, grid, s);
     return e == hipSuccess ? SIMNETS_OK : SIMNETS_ERR_HIP;
 }
 
@@ -1180,7 +1318,7 @@ int mex_panel_launch_selfpack(const MexPlan &p, const MexKernelArgs &a, const fl
                               float *output, void *stream)
 {
     PanelArgs g;
-    if (p.d.K != KC || reinterpret_cast<uintptr_t>(offsets) % 16 != 0)
+    if (p.d.K != KC || reinterpret_cast<uintptr_t>(offsets) % 16 != 0 || !std::isfinite(p.epsilon))
         return SIMNETS_PANEL_NOT_TAKEN;
     if (panel_halves(p, 2, 2, input, a.slots, a.n_mgroups, &g, false) != 1)
         return SIMNETS_PANEL_NOT_TAKEN;

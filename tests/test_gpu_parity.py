@@ -556,6 +556,37 @@ def test_mex_panel_form_of_the_plain_call(pkg, im, n, spread, eps):
     assert mex_err(other, x, off, n, **kw) <= MEX_TOL
 
 
+@pytest.mark.parametrize("im,n", [
+    ((37, 64, 8, 8), 70), ((21, 128, 4, 4), 64), ((45, 256, 2, 2), 130), ((5, 64, 16, 16), 64), ((3, 64, 24, 16), 16),
+    ((2, 64, 4, 64), 16), ((64, 64, 16, 16), 256), ((9, 32, 16, 16), 64), ((3, 32, 4, 8), 20), ((300, 128, 4, 4), 200),
+])
+@pytest.mark.parametrize("eps", [math.inf, -math.inf])
+@pytest.mark.parametrize("softmax", [True, False])
+def test_mex_panel_form_with_infinite_epsilon(pkg, im, n, eps, softmax):
+    # the same layers with epsilon = +-inf: the panel kernel takes the largest (smallest) patch + offset from its
+    # tiles, an input that is not 16-byte aligned the tiled kernel; a term is one fp32 addition, so both give the
+    # oracle's values bit for bit, pixels without a finite channel included
+    g = np.random.default_rng(47)
+    kw = dict(softmax_mode=softmax, blocks=[im[1], 1, 1], strides=[im[1], 1, 1], epsilon=eps, use_unshared_regions=True,
+              unshared_offset_region=[1, 2, 2])
+    x = (g.normal(size=im) * 5).astype(np.float32)
+    lo = -math.inf if eps > 0 else math.inf
+    x[g.random(size=im) < 0.05] = lo
+    x[0, :, 0, 0] = lo
+    off = g.normal(size=(4, n, im[1], 1, 1)).astype(np.float32)
+    want = orc.mex_fwd(x, off, n, **kw)
+    assert want[0, 0, 0, 0] == lo and np.isfinite(want).sum() > want.size // 2
+    got = run_mex(pkg, x, off, n, **kw)
+    assert np.array_equal(got, want)
+    flat = torch.empty(x.size + 1, device="cuda")
+    shifted = flat[1:].view(*im)
+    shifted.copy_(dev(x))
+    assert shifted.data_ptr() % 16 == 4
+    assert np.array_equal(pkg.mex(shifted, dev(off), n, **kw).cpu().numpy(), want)
+    two = pkg.mex_sum_pool(dev(x), dev(off), n, (2, 2), **kw).cpu().numpy()
+    assert np.array_equal(two, pkg.sum_pooling(dev(got), (2, 2)).cpu().numpy())
+
+
 @pytest.mark.parametrize("im,n", [((19, 64, 8, 8), 40), ((40, 256, 2, 2), 64), ((6, 128, 16, 16), 64)])
 @pytest.mark.parametrize("eps", [1.0, -0.5])
 def test_mex_sum_pool_panel_form_with_infinite_and_missing_inputs(pkg, im, n, eps):
