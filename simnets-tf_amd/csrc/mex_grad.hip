@@ -188,10 +188,12 @@ constexpr float kGradProductRange = 48.0f;
 // Row-wise kernels: widest patch range of a pixel (exponents of two) for which a region with large offsets ranges
 // keeps the product form on the pixel's own maximum as the bound (the factors' exponents stay within this range)
 constexpr float kGradPixelRange = 64.0f;
-// ... and the widest offsets range such a region may have: with the tight bound the factors' errors follow the size of the
-// offsets themselves, as the reference's own do, at 1.5 to 2.4 times its error: within 1e-4 up to ranges of about 70 on the
-// tests' data (4e-5 ... 7e-5 at 77, 1.5e-4 at 88 on one seeded layer, 9e-5 ... 1.3e-4 at 110)
-constexpr float kGradRowsRange = 64.0f;
+// ... and the widest offsets range such a region may have.  With the tight bound the factors' errors follow the size of
+// the offsets themselves, as the reference's own do, at 1.5 to 4 times its error; what an element of the gradient sees
+// of it depends on how far its terms cancel: 4e-5 ... 7e-5 at 77 and 1.5e-4 at 88 on the tests' seeded layers, but
+// 1.1e-4 at a range of 55 on another (a sum of 4.8 in absolute terms that cancels to 0.08; error 2e-6 of the terms).  The
+// same limit as the gathering kernels' keeps such elements rare; beyond it a region goes term by term.
+constexpr float kGradRowsRange = 48.0f;
 constexpr float kLooseBoundRange = 24.0f;  // offsets ranges (exponents of two) up to which a few instances give the bound
 constexpr int GM_KT = 64;
 typedef float floatx4 __attribute__((ext_vector_type(4)));
@@ -800,8 +802,10 @@ __global__ __launch_bounds__(256) void mex_grad_offsets_mfma_kernel(const MexGra
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             const int m = ms0 + i;
+            // (an empty slot holds the values of another region's pixel: its exponent can be anything, and zero times
+            // an overflowed factor would put NaN into the sums)
             float w = 0.0f;
-            if (m < a.M)
+            if (cur.valid && m < a.M)
                 w = cur.gv[i] * __builtin_amdgcn_exp2f(__builtin_fmaf(-cur.ov[i], a.c1, a_p) + (omax_r[m] + a.c0));
             wt[lane * 65 + wave * 16 + i] = w;
         }
