@@ -577,7 +577,8 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
                                                               float *__restrict__ offe, float *__restrict__ omax,
                                                               float *__restrict__ orng, int4 *__restrict__ ktab, int H,
                                                               int W, int bh, int bw, int row_blocks, SimPackJob job,
-                                                              float *__restrict__ normalized_out, MexPackTwin tw)
+                                                              float *__restrict__ normalized_out, MexPackTwin tw,
+                                                              int for_gradients)
 {
     if ((int)blockIdx.x >= row_blocks) {
         // extra workgroups: the parameters of a Similarity layer evaluated inside the MEX staging
@@ -716,11 +717,13 @@ __global__ __launch_bounds__(256) void mex_pack_offsets_kernel(const float *__re
             dste2[(size_t)k * tm2] = e;
     });
     if (lane == 0) {
+        // the gradient kernels' copy: a row far from zero counts as too wide for their product form (kGradOffsetsSize)
+        const float grng = fabsf(hi) > kGradOffsetsSize || fabsf(lo) > kGradOffsetsSize ? INFINITY : hi - lo;
         omax[row] = hi;
-        orng[row] = hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
+        orng[row] = for_gradients ? grng : hi - lo;  // NaN or inf (infinite entries) sends the workgroup to the two sweeps
         if (dste2 != nullptr) {
             tw.omax[row2] = hi;
-            tw.orng[row2] = hi - lo;
+            tw.orng[row2] = grng;
         }
     }
 }
@@ -1068,7 +1071,7 @@ void mex_grad_pack_layout(const MexPlan &p, void *buffer, MexPackTwin *tw, float
 }
 
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
-                     void *stream, const SimPackJob *job, bool launch, float *normalized_out)
+                     void *stream, const SimPackJob *job, bool launch, float *normalized_out, bool for_gradients)
 {
     const simnets_mex_dims &d = p.d;
     const long long rows = (long long)d.num_regions * n_mgroups * tm;
@@ -1106,7 +1109,7 @@ int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgrou
 #define SIMNETS_PACK_LAUNCH(KL)                                                                                        \
     hipLaunchKernelGGL(mex_pack_offsets_kernel<KL>, grid, dim3(256), 0, hs, offsets, d.num_regions, d.M, d.K, n_mgroups, \
                        tm, p.normalize_offsets, a->scale, a->finite_eps, offp, offe, omax, orng, ktab, p.H, p.W,         \
-                       d.block_h, d.block_w, row_blocks, pj, normalized_out, tw)
+                       d.block_h, d.block_w, row_blocks, pj, normalized_out, tw, for_gradients ? 1 : 0)
     if (d.K <= 64)
         SIMNETS_PACK_LAUNCH(1);
     else if (d.K <= 256)

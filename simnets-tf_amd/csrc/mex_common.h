@@ -180,6 +180,13 @@ size_t mex_packed_bytes(const MexPlan &p, int tm, int n_mgroups);
 // follows it.  A plan whose grad_pack is set makes the forward's pack launch write it (and say so in `written`; a
 // forward that packs inside its own kernel does not).
 constexpr int kGradPackTm = 32;
+// The gradient kernels' product form builds its exponents from the scaled offsets, `out` and the bound, i.e. from values
+// of the size of the offsets: a term's relative error is about the last bit of such a value, 4e-6 at 64 exponents of two
+// and 1.5e-5 from 128 on - an order above the reference's, which subtracts `out` from patch + offset (exactly, for the
+// terms that matter) before it scales.  A row with a scaled offset beyond this size therefore gets an infinite range in
+// the arrays those kernels read, which sends its region to their term-by-term form (the reference's arithmetic).
+// Normalised offsets (log-probabilities) get there through their range first.
+constexpr float kGradOffsetsSize = 64.0f;
 struct MexPackTwin {
     float *offp, *offe, *omax, *orng;
     int4 *ktab;
@@ -189,9 +196,10 @@ void mex_grad_pack_layout(const MexPlan &p, void *buffer, MexPackTwin *tw, float
 // launch = false: the arrays were packed by an earlier call with the same arguments; only the pointers are set.
 // normalized_out: if not null, the launch also writes the offsets minus their rows' logsumexp there, [region][M][K]
 // (what the gradient kernels' term-by-term path and the chain rule through the normalisation read).
+// for_gradients: the ranges written are the gradient kernels' (kGradOffsetsSize), as in the layout a forward call keeps.
 int mex_pack_offsets(const MexPlan &p, const float *offsets, int tm, int n_mgroups, void *workspace, MexKernelArgs *a,
                      void *stream, const SimPackJob *job = nullptr, bool launch = true,
-                     float *normalized_out = nullptr);
+                     float *normalized_out = nullptr, bool for_gradients = false);
 
 
 // Panel form of the tiled forward kernel (csrc/mex_pool.hip) for layers with 2x2 unshared offsets over whole-channel

@@ -2052,7 +2052,7 @@ int mex_grad_pack_launch(const MexPlan &p, const float *offsets, void *buffer, v
         return prepare_offsets(q, offsets, norm, reinterpret_cast<hipStream_t>(stream), &used);
     }
     MexKernelArgs a = mex_kernel_args(q);
-    return mex_pack_offsets(q, offsets, GM_TM, tw.n_mgroups, buffer, &a, stream, nullptr, true, norm);
+    return mex_pack_offsets(q, offsets, GM_TM, tw.n_mgroups, buffer, &a, stream, nullptr, true, norm, true);
 }
 
 int mex_grads(const MexPlan &p, const float *input, const float *offsets, const float *output,
@@ -2171,7 +2171,7 @@ int mex_grads(const MexPlan &p, const float *input, const float *offsets, const 
                           (!want_input || aligned16(input_grad));
     if (t.mfma) {
         rc = mex_pack_offsets(p, offsets, GM_TM, (d.M + GM_TM - 1) / GM_TM, packed_at, &ga.k, stream, nullptr,
-                              !packed_already, pack_normalizes ? norm_at : nullptr);
+                              !packed_already, pack_normalizes ? norm_at : nullptr, true);
         if (rc)
             return rc;
         if (w.use_factors && !use_rows) {

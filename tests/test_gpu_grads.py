@@ -812,9 +812,9 @@ def test_similarity_input_grad_forms_agree_at_network_sizes(pkg, case):
 def test_mex_grads_regions_with_offsets_far_from_each_other(pkg, im, n, blocks, eps):
     # one region per pixel, a handful of pixel slots per region, the regions' offsets 300 apart: the empty slots of a
     # region's last group of 64 stand on a pixel of another region, whose output lies far from this region's offsets;
-    # they must not reach the sums (zero times an overflowed exponential would be NaN).  The exponents are formed from
-    # scaled values of size 150 |eps| log2(e), each known to its last bit (1.5e-5 ... 3e-5) only: terms carry relative
-    # errors of that order, which the 1 % floor of the metric magnifies where the terms of an element cancel
+    # they must not reach the sums (zero times an overflowed exponential would be NaN).  Offsets this far from zero also
+    # take the kernels' term-by-term form (exponents built from scaled values of size 150 |eps| log2(e) would carry
+    # their last bit, 1.5e-5 ... 3e-5, into every term): the reference's arithmetic, to the usual bar
     g = np.random.default_rng(91)
     kw = dict(blocks=blocks, strides=blocks, padding=[0, 0, 0], epsilon=eps, softmax_mode=True,
               use_unshared_regions=False, shared_offset_region=[2, 1, 1])
@@ -822,16 +822,23 @@ def test_mex_grads_regions_with_offsets_far_from_each_other(pkg, im, n, blocks, 
     x = g.normal(size=im).astype(np.float32)
     off = g.normal(size=(d.num_regions, n) + tuple(blocks)).astype(np.float32)
     off += (150.0 * np.where(np.arange(d.num_regions) % 2 == 0, -1.0, 1.0)).astype(np.float32)[:, None, None, None, None]
-    out = orc.mex_fwd(x, off, n, **kw)
-    gy = g.normal(size=out.shape).astype(np.float32)
-    X, O, Y, G = dev(x), dev(off), dev(out), dev(gy)
-    dx = pkg.mex_input_grad(X, O, Y, G, n, **kw).cpu().numpy()
-    doff = pkg.mex_offsets_grad(X, O, Y, G, n, **kw).cpu().numpy()
-    assert np.isfinite(dx).all() and np.isfinite(doff).all()
-    x64, off64, g64 = f64(x, off, gy)
-    out64 = orc.mex_fwd(x64, off64, n, **kw)
-    assert grad_err(dx, orc.mex_input_grad(x64, off64, out64, g64, n, **kw)) <= 2e-3
-    assert grad_err(doff, orc.mex_offsets_grad(x64, off64, out64, g64, n, **kw)) <= 2e-3
+    # (with more than one patch element the reference's own x + o - out is rounded at this size: 2e-4 against fp64)
+    check_mex_grads(pkg, x, off, n, strict=False, **kw)
+
+
+@pytest.mark.parametrize("size,eps", [(30.0, 1.0), (50.0, 1.0), (30.0, -2.0)])
+def test_mex_grads_single_element_patches_with_offsets_far_from_zero(pkg, size, eps):
+    # K = 1: out = x + o, every term of the gradients is g exactly in the reference's arithmetic (it subtracts out from
+    # x + o before scaling).  Offsets of a size whose scaled values reach 64 exponents of two are taken term by term for
+    # that reason; just below, the product form's exponents carry the last bit of values of that size (4e-6)
+    g = np.random.default_rng(92)
+    im, n = (12, 1, 3, 8), 69
+    kw = dict(blocks=[1, 1, 1], strides=[1, 1, 1], padding=[0, 0, 0], epsilon=eps, softmax_mode=True,
+              use_unshared_regions=False, shared_offset_region=[1, 2, 2])
+    d = orc.mex_dims(orc.mex_args(im, n, **kw))
+    x = g.normal(size=im).astype(np.float32)
+    off = (g.uniform(-1.0, 1.0, size=(d.num_regions, n, 1, 1, 1)) * size).astype(np.float32)
+    check_mex_grads(pkg, x, off, n, **kw)
 
 
 # ---- seeded sweeps over random layers -----------------------------------------------------------------------------
