@@ -619,6 +619,16 @@ def main():
                       args.warmup)
         others["config5_mex_offsets_grad"] = entry(ms, 33554432, 2097152 + 2 * 4194304 + 2 * 32768, "hbm", flop=5,
                                                    mex=True)
+        # ... and as a training step asks for them: both gradients from one call, without and with the offsets layout
+        # that the forward call of the step kept (then nothing is packed)
+        _, ms = timed(lambda: pkg.mex_grads(X2, O2, Y2, G2, n2, normalize_offsets=True, **kw2), args.steps, args.warmup)
+        others["config5_mex_both_grads_one_call"] = entry(ms, 2 * 33554432, 2 * 2097152 + 2 * 4194304 + 2 * 32768, "hbm",
+                                                          flop=5, mex=True)
+        Y2s, saved2 = pkg.mex_saving(X2, O2, n2, normalize_offsets=True, **kw2)
+        _, ms = timed(lambda: pkg.mex_grads(X2, O2, Y2s, G2, n2, normalize_offsets=True, saved=saved2, **kw2),
+                      args.steps, args.warmup)
+        others["config5_mex_both_grads_one_call_kept_offsets"] = entry(
+            ms, 2 * 33554432, 2 * 2097152 + 2 * 4194304 + 2 * 32768, "hbm", flop=5, mex=True)
 
         def cpu5():
             """Achieved gradient errors against the fp64 oracle, beside the fp32 oracle's own: the error of an element
