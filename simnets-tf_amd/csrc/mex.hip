@@ -558,7 +558,9 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
 #pragma unroll
         for (int m = 0; m < MX; ++m) {
             // (max + ey*log2(e) + log2(sum)) * log(2)/eps in the scaled domain; the plain max for infinite eps
-            const float res = INF ? mx[p][m] : (__builtin_amdgcn_logf(s[p][m]) + (mx[p][m] + a.c0)) * a.ln2_over_eps;
+            // (an infinite extreme value makes the finite-epsilon result NaN, as the reference's exp(inf - inf) does)
+            const float b = mx[p][m];
+            const float res = INF ? b : (__builtin_amdgcn_logf(s[p][m]) + ((b - b) + b + a.c0)) * a.ln2_over_eps;
             if (m0 + m < a.M)
                 o[(size_t)(m0 + m) * plane] = res;
         }
@@ -955,7 +957,9 @@ __global__ __launch_bounds__(256) void mex_small_kernel(const MexKernelArgs a)
 #pragma unroll
             for (int g = 0; g < MG; ++g)
                 if ((wide4 >> g) & 1u)
-                    res[g] = a.finite_eps ? (__builtin_amdgcn_logf(sum[g]) + (best[g] + a.c0)) * a.ln2_over_eps : best[g];
+                    // (an infinite extreme value makes the finite-epsilon result NaN, as the reference's exp(inf - inf) does)
+                    res[g] = a.finite_eps ? (__builtin_amdgcn_logf(sum[g]) + ((best[g] - best[g]) + best[g] + a.c0)) * a.ln2_over_eps
+                                          : best[g];
         }
         if (lane == 0) {
 #pragma unroll

@@ -615,6 +615,42 @@ def test_mex_sum_pool_panel_form_with_infinite_and_missing_inputs(pkg, im, n, ep
     assert np.abs(got[fin] - want[fin]).max() <= MEX_TOL * max(1.0, np.abs(want[fin]).max())
 
 
+@pytest.mark.parametrize("im,n,kw", [
+    ((6, 4, 7, 5), 55, dict(blocks=[1, 1, 2], strides=[1, 1, 1], use_unshared_regions=False, shared_offset_region=[1, 2, 2])),
+    ((3, 2, 3, 4), 63, dict(blocks=[1, 2, 1], strides=[1, 1, 1], unshared_offset_region=[1, 3, 1])),
+    ((40, 6, 2, 2), 130, dict(blocks=[6, 1, 1], strides=[6, 1, 1], unshared_offset_region=[2])),        # K-split waves
+    ((20, 64, 1, 1), 10, dict(blocks=[64, 1, 1], strides=[64, 1, 1], shared_offset_region=[1])),        # wave per pixel
+    ((7, 100, 2, 3), 5, dict(blocks=[100, 1, 1], strides=[100, 1, 1], unshared_offset_region=[2])),
+])
+@pytest.mark.parametrize("eps", [1.0, -2.0])
+@pytest.mark.parametrize("offsets", ["wide", "switched_off"])
+def test_mex_patches_without_a_finite_element_on_the_log_sum_exp_paths(pkg, im, n, kw, eps, offsets):
+    # The reference's exp(eps (x + o - max)) is exp(inf - inf) = NaN when nothing of a patch is finite (inputs of -inf,
+    # +inf for a negative epsilon: missing data), and so is its output; the product form reproduces that through its
+    # pixel bound, the max-tracked log-sum-exp of the tiled and the wave-per-pixel kernels (offsets rows too wide for
+    # the product form, or with entries that switch an element off) must as well - not -inf
+    g = np.random.default_rng(48)
+    kw = dict(kw, epsilon=eps, softmax_mode=True)
+    d = orc.mex_dims(orc.mex_args(im, n, **kw))
+    lo = -math.inf if eps > 0 else math.inf
+    x = g.normal(size=im).astype(np.float32)
+    x[g.random(size=im) < 0.3] = lo
+    x[0] = lo                                   # nothing finite in the first image at all
+    off = g.normal(size=(d.num_regions, n) + tuple(kw["blocks"])).astype(np.float32)
+    if offsets == "wide":
+        off *= 300.0
+    else:
+        off[g.random(size=off.shape) < 0.1] = lo
+    with np.errstate(invalid="ignore", over="ignore"):
+        want = orc.mex_fwd(x, off, n, **kw)
+    got = run_mex(pkg, x, off, n, **kw)
+    assert np.isnan(want[0]).all() and np.isfinite(want).any()
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    fin = np.isfinite(want)
+    assert np.array_equal(got[~fin & ~np.isnan(want)], want[~fin & ~np.isnan(want)])
+    assert np.abs(got[fin] - want[fin]).max() <= MEX_TOL * max(1.0, np.abs(want[fin]).max())
+
+
 @pytest.mark.parametrize("kw,pool", [
     (dict(use_unshared_regions=True, unshared_offset_region=[1, 2, 2], epsilon=math.inf), (2, 2)),   # max: no product form
     (dict(use_unshared_regions=True, unshared_offset_region=[1, 2, 2]), (4, 4)),                     # window != regions
