@@ -98,6 +98,10 @@ int so_mex_calc_dims(const so_mex_args *a, so_mex_dims *d)
     d->height_out = so_dimension_out_size(a->height, d->pad_h, d->block_h, d->stride_h, a->blocks_round_down);
     d->width_out = so_dimension_out_size(a->width, d->pad_w, d->block_w, d->stride_w, a->blocks_round_down);
     d->channels_out = so_dimension_out_size(a->channels, d->pad_c, d->block_c, d->stride_c, a->blocks_round_down);
+    /* A block larger than the padded image leaves an output extent of zero or less; the reference goes on and divides
+     * by the region extent it derives from it (an integer division by zero).  The checker reports it instead. */
+    if (d->height_out <= 0 || d->width_out <= 0 || d->channels_out <= 0)
+        return -9;
 
     if (!a->use_unshared_regions) {
         int sc, sh, sw;
@@ -113,6 +117,8 @@ int so_mex_calc_dims(const so_mex_args *a, so_mex_dims *d)
         sw = so_min(sw, d->width_out);
         if (sc < 0) sc = d->channels_out;
         sc = so_min(sc, d->channels_out);
+        if (sc == 0 || sh == 0 || sw == 0)
+            return -9; /* (a region extent of zero: the same division) */
         d->shared_region_c = sc; d->shared_region_h = sh; d->shared_region_w = sw;
         d->offsets_h = so_ceiled_div(d->height_out, sh);
         d->offsets_w = so_ceiled_div(d->width_out, sw);
@@ -131,6 +137,8 @@ int so_mex_calc_dims(const so_mex_args *a, so_mex_dims *d)
         uw = so_min(uw, d->width_out);
         if (uc < 0) uc = d->channels_out;
         uc = so_min(uc, d->channels_out);
+        if (uc == 0 || uh == 0 || uw == 0)
+            return -9;
         d->offsets_h = uh; d->offsets_w = uw; d->offsets_c = uc;
         d->shared_region_h = so_ceiled_div(d->height_out, uh);
         d->shared_region_w = so_ceiled_div(d->width_out, uw);

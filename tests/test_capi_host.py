@@ -152,6 +152,13 @@ def test_mex_validation_mirrors_the_reference(pkg):
     assert code(strides=[1, 0, 1]) == -10
     assert code(padding=[0, 0]) == 0              # two entries: -1 (the channel count) is prepended
     assert "block depth must be smaller than input depth" in pkg._lib.strerror(-14)
+    # a block larger than the padded image, a region extent of zero: the reference divides by zero in
+    # CalculateDimensions (src/kernels/mex_kernel_common.cpp:86-139); the library and the oracle report it
+    for bad in (dict(blocks=[1, 1, 9]), dict(blocks=[1, 9, 1], padding=[0, 0, 0]), dict(unshared_offset_region=[0]),
+                dict(use_unshared_regions=False, shared_offset_region=[1, 0, 2])):
+        assert code(**bad) < 0
+        with pytest.raises(ValueError):
+            orc.mex_dims(orc.mex_args((1, 3, 8, 8), 2, **bad))
 
 
 def test_compute_entry_points_reject_bad_arguments_without_touching_the_device(pkg):
