@@ -1243,8 +1243,16 @@ int pool_launch(const MexPlan &p, int ph, int pw, const float *input, const floa
     // ... and four halves (16 waves) when there are many slots and the patches are short: the offsets tiles are
     // then copied once per 256 pixel columns
     int nh = a.slots > 64 / (ph * pw) ? 2 : 1;
-    if (ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
+    // ... only with the Similarity inside (its patch taps and parameters are then fetched once per 256 columns:
+    // 512 images of the first layer 24.2 -> 18.3 us); without it two halves are as fast or faster (15.6 against
+    // 16.0 us, 104.7 against 111.0 us at 4096 images)
+    if (sp && ph * pw == 4 && d.K <= 2 * KC && a.slots >= 64 * 128)
         nh = 4;
+    // a single chunk on a grid that two halves would leave below one workgroup per compute unit: one half (64 images
+    // of 32 x 16 x 16: 6.7 -> 6.1 us)
+    const int spw2 = 2 * 64 / (ph * pw);   // slots of a workgroup of two halves
+    if (nh == 2 && d.K <= KC && ((long long)a.slots + spw2 - 1) / spw2 * n_mgroups < kPanelWorkgroups)
+        nh = 1;
     PanelArgs pg;
     const int panel = sp ? 0 : panel_halves(p, ph, pw, input, a.slots, n_mgroups, &pg, true);
     if (panel)
