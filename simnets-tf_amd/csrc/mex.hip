@@ -403,7 +403,6 @@ __global__ __launch_bounds__(256, PX == 2 ? 4 : 1) void mex_fwd_kernel(const Mex
             if (!wave_active)
                 continue;
             const int kend = min(kc, (wk + 1) * KW);
-#pragma unroll 2
             for (int kk = wk * KW; kk < kend; kk += 2) {
                 const int k1 = min(kk + 1, kend - 1);   // (an odd count takes its last k twice)
                 float x0[PX], x1[PX];
