@@ -105,12 +105,22 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
                 // reads (d, d, acc), (w, |d|, acc) or (q, d, acc): d of pixel p goes to a register of the opposite
                 // parity of acc[m][p] - pixels 2j+1, 2j as the (even, odd) halves of a 64-bit pair; the
                 // accumulators are held as such pairs in pixel order by the caller (sim_pin_pairs).  (Not for L1: the
-                // pairs cost it registers it does not have.)
+                // pairs cost it registers it does not have; see the copy of its weight below.)
 #pragma unroll
                 for (int j = 0; j < PT / 2; ++j) {
                     float2_t dd = {d[0][2 * j + 1], d[0][2 * j]};
                     asm volatile("" : : "v"(dd));
                 }
+            }
+            // L1 on parameters from 16-byte loads: the weight of a pair (t, w) sits in an odd register, t in an even one
+            // that is free once the differences are formed.  A copy of the weight goes there (one instruction per
+            // template and step), and the accumulate step of pixel p takes the copy of the parity opposite to
+            // acc[m][p]'s (a row of accumulators is handed out as consecutive registers from an even one): its three
+            // sources then never share a parity, wherever the allocator put the difference.
+            float nwe[MG];
+            if constexpr (MODE == SIM_MODE_L1 && VP && MG == 1 && PT % 2 == 0) {
+                nwe[0] = t[0];
+                asm volatile("v_mov_b32 %0, %1" : "+v"(nwe[0]) : "v"(nw[0]));
             }
             __builtin_amdgcn_sched_barrier(0);
             if (MODE == SIM_MODE_L2 || MODE == SIM_MODE_L2_NORM) {
@@ -132,6 +142,8 @@ __device__ __forceinline__ void sim_step(float (&acc)[MT][PT], const float (&x)[
                         // negation (8 bytes) - and negated by the caller at the end: every partial sum is the exact
                         // negative of the other form's.
                         acc[m][p] = __builtin_fmaf(d[g][p], d[g][p], acc[m][p]);
+                    else if (MODE == SIM_MODE_L1 && VP && MG == 1 && PT % 2 == 0)
+                        acc[m][p] = __builtin_fmaf((p & 1) ? nwe[g] : nw[g], __builtin_fabsf(d[g][p]), acc[m][p]);
                     else if (MODE == SIM_MODE_L1)
                         acc[m][p] = __builtin_fmaf(nw[g], __builtin_fabsf(d[g][p]), acc[m][p]);
                     else if (MODE == SIM_MODE_L2)
